@@ -1,0 +1,37 @@
+"""CPU oracle for the ODM-KV compression-and-decode path.
+
+TEST INFRASTRUCTURE ONLY.  This package restates, on the CPU, the arithmetic of
+the reference implementation (yiiwang118/ODM-KV) for the hot path
+
+    score -> Lagrangian bit allocation -> Lloyd-Max quantize/pack -> decode attention
+
+so that the HIP kernels can be compared against it.  Only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
+import it.  Nothing under ``odm-kv_amd/`` imports it, and the product raises if
+its HIP library is missing rather than falling back to this code.
+
+Every function cites the reference file:line it follows.
+
+Pin status (what independent evidence fixes each function):
+
+* ``codebook.lloyd_max_codebook``     pinned: textbook Gaussian Lloyd-Max levels
+  (Max 1960), symmetry, Panter-Dite bound, scipy's ``norm.pdf``; exact fp64
+  bits against the golden table in ``tests/golden`` when that fixture exists.
+* ``quantizer.pack_codes / unpack_codes``   pinned: byte layouts worked out by
+  hand from the reference text, round trips for every width.
+* ``quantizer.nearest_centroid``      pinned against brute-force argmin; the
+  reference's own routine (``kvquant.tq_triton.mse_nearest_centroid``) is not
+  shipped, so its behaviour exactly on a midpoint is **parity unpinned**.
+* ``quantizer.quantize / dequantize`` pinned: algebraic identities (identity
+  rotation, 2-entry codebook = sign quantisation), relative MSE against the
+  Lloyd-Max distortion table.
+* ``scorer.*``                        pinned: fp64 brute force on tiny inputs,
+  closed forms (uniform attention, G=1), scaling invariants.
+* ``allocator.optimal_scores_to_bits``  pinned: exhaustive Lagrangian argmin on
+  tiny inputs, budget invariants, trivial-case clamps; token choice *inside* a
+  group of equal scores at the repair cut-off is implementation-defined in the
+  reference (unstable argsort) and therefore **parity unpinned** there.
+* ``kvstate.*``                       pinned: partition/round-trip invariants.
+* ``attention.decode_attention``      pinned: equals torch SDPA on an all-exact
+  cache, single-token and permutation special cases.
+"""

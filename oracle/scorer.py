@@ -1,0 +1,168 @@
+"""Oracle: the ODM risk score  s = (p + eps)^2 * (|v|^2 + |k|^2/d * |v - o|^2).
+
+Follows /root/reference/kvquant/scorer.py
+  ExpectedAttentionScorer._query_statistics   :184-202
+  _expected_core_internals                    :285-318
+  _pad_sinks_and_normalize                    :321-325  (grain "global" = identity, :118-119)
+  RiskScorer.score_prefill                    :385-404
+  RiskScorer.score_with_attn                  :406-416
+  _NormFallback.score_prefill                 :145-147
+and /root/reference/kvquant/attention_utils.py
+  _repeat_kv :19-26, _get_query_states :29-54, _apply_avg_rope :57-115.
+
+Like the reference the code is dtype-generic: whatever dtype the caller passes is
+the dtype the attention estimate is computed in.  Parity tests pass fp32 tensors.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+
+def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """[b, Hkv, t, d] -> [b, Hkv*n_rep, t, d]; q-head q reads kv-head q // n_rep."""
+    if n_rep == 1:
+        return x
+    b, h, t, d = x.shape
+    return x[:, :, None].expand(b, h, n_rep, t, d).reshape(b, h * n_rep, t, d)
+
+
+def _num_heads(module) -> Optional[int]:
+    n = getattr(module, "num_heads", None)
+    cfg = getattr(module, "config", None)
+    if n is None and cfg is not None:
+        n = getattr(cfg, "num_attention_heads", None)
+    return n
+
+
+def query_states(module, hidden: torch.Tensor) -> torch.Tensor:
+    """Pre-RoPE queries [b, Hq, T, d] of an HF attention module (attention_utils.py:29-54)."""
+    b, t, _ = hidden.shape
+    n_heads = _num_heads(module)
+    if n_heads is None:
+        raise AttributeError("cannot determine num_heads")
+    cfg = getattr(module, "config", None)
+    head_dim = getattr(module, "head_dim", None)
+    if head_dim is None and cfg is not None:
+        head_dim = getattr(cfg, "head_dim", None)
+    if head_dim is None:
+        head_dim = hidden.shape[-1] // n_heads
+    if hasattr(module, "qkv_proj"):
+        q = module.qkv_proj(hidden)[..., : n_heads * head_dim]
+    elif hasattr(module, "q_proj"):
+        q = module.q_proj(hidden)
+    else:
+        raise NotImplementedError(type(module).__name__)
+    q = q.view(b, t, n_heads, head_dim).transpose(1, 2)
+    if hasattr(module, "q_norm"):
+        q = module.q_norm(q)
+    return q
+
+
+def avg_rope(module, mu: torch.Tensor, q_len: int, n_future: int) -> torch.Tensor:
+    """mu -> R_avg mu with R_avg the mean RoPE matrix over positions [q_len, q_len+n_future)
+    (attention_utils.py:57-115).  Identity without ``rotary_emb`` or with n_future <= 0."""
+    rotary = getattr(module, "rotary_emb", None)
+    if rotary is None or n_future <= 0:
+        return mu
+    pos = torch.arange(q_len, q_len + n_future, device=mu.device).unsqueeze(0)
+    cos, sin = rotary(mu, pos)
+    cos = cos.to(device=mu.device, dtype=mu.dtype)[0]
+    sin = sin.to(device=mu.device, dtype=mu.dtype)[0]
+    d = mu.shape[-1]
+    half = d // 2
+    eye = torch.eye(d, dtype=mu.dtype, device=mu.device)
+    perm = torch.zeros(d, d, dtype=mu.dtype, device=mu.device)
+    perm[half:, :half] = torch.eye(half, dtype=mu.dtype, device=mu.device)
+    perm[:half, half:] = -torch.eye(half, dtype=mu.dtype, device=mu.device)
+    r_avg = (cos.unsqueeze(-1) * eye + sin.unsqueeze(-1) * perm).mean(dim=0)
+    return torch.matmul(mu, r_avg.T)
+
+
+def mean_query(module, hidden: torch.Tensor, n_sink: int, n_future: int) -> torch.Tensor:
+    """[1, Hq, d]: mean over positions >= n_sink of the pre-RoPE queries, then averaged RoPE
+    (scorer.py:184-202 with use_covariance=False)."""
+    if hidden.dim() == 2:
+        hidden = hidden.unsqueeze(0)
+    q_len = hidden.shape[1]
+    if q_len <= n_sink:
+        raise ValueError("not enough tokens to estimate expected attention")
+    q = query_states(module, hidden[:, n_sink:])
+    return avg_rope(module, q.mean(dim=2), q_len, n_future)
+
+
+def expected_attention(keys: torch.Tensor, mu: torch.Tensor, n_sink: int,
+                       n_q_heads: int) -> torch.Tensor:
+    """p [1, Hkv, T - n_sink]: softmax over core tokens of mu . k / sqrt(d) per q-head,
+    then the mean over each GQA group (scorer.py:296-315)."""
+    core = keys[:, n_sink:]
+    h_kv, t_core, d = core.shape
+    groups = n_q_heads // h_kv
+    kt = repeat_kv(core.unsqueeze(0), groups).transpose(2, 3)          # [1, Hq, d, Tc]
+    logits = torch.matmul(mu.unsqueeze(2), kt).squeeze(2) / math.sqrt(d)
+    a = torch.softmax(logits, dim=-1)
+    return a.reshape(1, h_kv, groups, t_core).mean(dim=2)
+
+
+def risk_from_attention(p_raw: torch.Tensor, keys_core: torch.Tensor, values_core: torch.Tensor,
+                        epsilon: float) -> torch.Tensor:
+    """scorer.py:394-403: p_raw [1, H, Tc] in its own dtype, keys/values [H, Tc, d] -> [1, H, Tc]."""
+    d = keys_core.shape[-1]
+    p = p_raw[0].float()
+    p_hat = p / p.sum(dim=-1, keepdim=True).clamp(min=1e-8)
+    o_bar = torch.einsum("ht,htd->hd", p_hat, values_core.float())
+    irrep = (values_core.float() - o_bar.unsqueeze(1)).pow(2).sum(dim=-1)
+    kn2 = keys_core.unsqueeze(0).float().pow(2).sum(dim=-1)
+    vn2 = values_core.unsqueeze(0).float().pow(2).sum(dim=-1)
+    return (p_raw + epsilon).pow(2) * (vn2 + (kn2 / float(d)) * irrep.unsqueeze(0))
+
+
+def pad_sinks(core_scores: torch.Tensor, n_sink: int) -> torch.Tensor:
+    """Left-pad n_sink columns with the global maximum (scorer.py:321-325) -> [H, T]."""
+    top = float(core_scores.max().item()) if core_scores.numel() else 1.0
+    return torch.nn.functional.pad(core_scores, (n_sink, 0), value=top).squeeze(0)
+
+
+def norm_fallback(keys: torch.Tensor, values: torch.Tensor) -> torch.Tensor:
+    """|k| + |v| (scorer.py:145-147; grain "global" leaves it as is)."""
+    return keys.norm(dim=-1) + values.norm(dim=-1)
+
+
+def risk_score_from_mu(keys: torch.Tensor, values: torch.Tensor, mu: torch.Tensor,
+                       n_q_heads: int, *, n_sink: int = 4, epsilon: float = 1e-2) -> torch.Tensor:
+    """Scores [Hkv, T] given the (already RoPE-averaged) mean query mu [1, Hq, d]."""
+    if keys.shape[1] <= n_sink:
+        return torch.ones(keys.shape[:2], dtype=keys.dtype)
+    p = expected_attention(keys, mu, n_sink, n_q_heads)
+    s = risk_from_attention(p, keys[:, n_sink:], values[:, n_sink:], epsilon)
+    return pad_sinks(s, n_sink)
+
+
+def risk_score_prefill(keys: torch.Tensor, values: torch.Tensor, *, module=None,
+                       hidden_states: Optional[torch.Tensor] = None, n_sink: int = 4,
+                       epsilon: float = 1e-2, n_future: int = 512) -> torch.Tensor:
+    """RiskScorer.score_prefill (scorer.py:385-404), keys/values [Hkv, T, d] -> [Hkv, T]."""
+    if module is None or hidden_states is None:
+        return norm_fallback(keys, values)
+    if keys.shape[1] <= n_sink:
+        return torch.ones(keys.shape[:2], dtype=keys.dtype)
+    try:
+        mu = mean_query(module, hidden_states, n_sink, n_future)
+    except (AttributeError, NotImplementedError, ValueError):
+        return norm_fallback(keys, values)
+    n_q = _num_heads(module) or keys.shape[0]
+    return risk_score_from_mu(keys, values, mu, n_q, n_sink=n_sink, epsilon=epsilon)
+
+
+def risk_score_with_attn(keys: torch.Tensor, values: torch.Tensor, attn: torch.Tensor,
+                         epsilon: float = 1e-2) -> torch.Tensor:
+    """RiskScorer.score_with_attn (scorer.py:406-416): keys/values [H, T, d], attn [H, T]."""
+    p = attn.float()
+    p_hat = p / p.sum(dim=-1, keepdim=True).clamp(min=1e-8)
+    o_bar = torch.einsum("ht,htd->hd", p_hat, values.float())
+    irrep = (values.float() - o_bar.unsqueeze(1)).pow(2).sum(dim=-1)
+    kn2 = keys.float().pow(2).sum(dim=-1)
+    vn2 = values.float().pow(2).sum(dim=-1)
+    return (p + epsilon).pow(2) * (vn2 + (kn2 / float(keys.shape[-1])) * irrep)

@@ -1,0 +1,125 @@
+"""Pins for the oracle's ODM risk score: reference vectors, fp64 brute force, closed forms."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import scorer as sc
+
+
+class Stub(torch.nn.Module):
+    def __init__(self, w, b, n_heads, head_dim):
+        super().__init__()
+        self.q_proj = torch.nn.Linear(w.shape[1], w.shape[0], bias=True)
+        with torch.no_grad():
+            self.q_proj.weight.copy_(torch.as_tensor(w))
+            self.q_proj.bias.copy_(torch.as_tensor(b))
+        self.config = types.SimpleNamespace(num_attention_heads=n_heads, head_dim=head_dim)
+        self.head_dim = head_dim
+
+
+def _stub(golden, name, hq, d, dtype=torch.float32, rotary_cfg=None):
+    mod = Stub(golden[f"score_{name}_w"], golden[f"score_{name}_b"], hq, d)
+    if rotary_cfg is not None:
+        from transformers import LlamaConfig
+        from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+        mod.rotary_emb = LlamaRotaryEmbedding(LlamaConfig(**rotary_cfg))
+    return mod.to(dtype)
+
+
+@pytest.mark.parametrize("name,hq,d,nf", [("f32", 4, 16, 512), ("f32_g1", 3, 16, 512), ("f32_d128", 8, 128, 512)])
+def test_fp32_matches_reference(golden, name, hq, d, nf):
+    k, v, h = (torch.from_numpy(golden[f"score_{name}_{x}"]) for x in "kvh")
+    mod = _stub(golden, name, hq, d)
+    with torch.no_grad():
+        mu = sc.mean_query(mod, h, 4, nf)
+        got = sc.risk_score_prefill(k, v, module=mod, hidden_states=h, n_future=nf)
+    np.testing.assert_allclose(mu.numpy(), golden[f"score_{name}_mu"], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(got.numpy(), golden[f"score_{name}_out"], rtol=2e-5)
+
+
+def test_rope_average_matches_reference(golden):
+    cfg = dict(hidden_size=8 * 32, num_attention_heads=8, num_key_value_heads=2, head_dim=32,
+               rope_theta=10000.0, max_position_embeddings=4096)
+    k, v, h = (torch.from_numpy(golden[f"score_f32_rope_{x}"]) for x in "kvh")
+    mod = _stub(golden, "f32_rope", 8, 32, rotary_cfg=cfg)
+    with torch.no_grad():
+        mu = sc.mean_query(mod, h, 4, 64)
+        got = sc.risk_score_prefill(k, v, module=mod, hidden_states=h, n_future=64)
+        # closed form: mean cos * mu + mean sin * rotate_half(mu)
+        raw = sc.query_states(mod, h[:, 4:]).mean(dim=2)
+        cos, sin = mod.rotary_emb(raw, torch.arange(64, 128).unsqueeze(0))
+        half = torch.cat([-raw[..., 16:], raw[..., :16]], dim=-1)
+        closed = cos[0].mean(0) * raw + sin[0].mean(0) * half
+    np.testing.assert_allclose(mu.numpy(), golden["score_f32_rope_mu"], rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(mu.numpy(), closed.numpy(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(got.numpy(), golden["score_f32_rope_out"], rtol=2e-5)
+
+
+def test_fp16_model_dtype_matches_reference(golden):
+    k, v, h = (torch.from_numpy(golden[f"score_f16_{x}"]).half() for x in "kvh")
+    mod = _stub(golden, "f16", 4, 16, dtype=torch.float16)
+    with torch.no_grad():
+        got = sc.risk_score_prefill(k, v, module=mod, hidden_states=h)
+    np.testing.assert_allclose(got.float().numpy(), golden["score_f16_out"], rtol=5e-3)
+
+
+def test_with_attn_and_fallback_match_reference(golden):
+    k, v, a = (torch.from_numpy(golden[f"swa_{x}"]) for x in "kva")
+    np.testing.assert_allclose(sc.risk_score_with_attn(k, v, a).numpy(), golden["swa_out"], rtol=1e-5)
+    np.testing.assert_allclose(sc.risk_score_prefill(k, v).numpy(), golden["fallback_out"], rtol=1e-6)
+
+
+def _brute(k, v, mu, g, n_sink=4, eps=1e-2):
+    """fp64 loops straight from the formula."""
+    k, v, mu = k.double().numpy(), v.double().numpy(), mu.double().numpy()
+    h, t, d = k.shape
+    out = np.zeros((h, t))
+    for hh in range(h):
+        p = np.zeros(t - n_sink)
+        for gg in range(g):
+            logit = np.array([mu[hh * g + gg] @ k[hh, j] / np.sqrt(d) for j in range(n_sink, t)])
+            e = np.exp(logit - logit.max())
+            p += e / e.sum() / g
+        o = sum(p[j] / p.sum() * v[hh, n_sink + j] for j in range(t - n_sink))
+        for j in range(t - n_sink):
+            vv, kk = v[hh, n_sink + j], k[hh, n_sink + j]
+            out[hh, n_sink + j] = (p[j] + eps) ** 2 * (vv @ vv + (kk @ kk) / d * ((vv - o) @ (vv - o)))
+    out[:, :n_sink] = out[:, n_sink:].max()
+    return out
+
+
+def test_brute_force_fp64():
+    g = torch.Generator().manual_seed(9)
+    k = torch.randn(2, 16, 8, generator=g)
+    v = torch.randn(2, 16, 8, generator=g)
+    mu = torch.randn(4, 8, generator=g)
+    got = sc.risk_score_from_mu(k, v, mu.unsqueeze(0), 4)
+    np.testing.assert_allclose(got.numpy(), _brute(k, v, mu, 2), rtol=1e-5)
+
+
+def test_closed_forms_and_invariants():
+    g = torch.Generator().manual_seed(10)
+    k = torch.randn(2, 40, 8, generator=g)
+    v = torch.randn(2, 40, 8, generator=g)
+    mu = torch.randn(1, 4, 8, generator=g)
+    # attention sums to one over the core tokens
+    p = sc.expected_attention(k, mu, 4, 4)
+    np.testing.assert_allclose(p.sum(-1).numpy(), 1.0, rtol=1e-6)
+    # zero mean query: uniform attention, o-bar is the plain mean of the core values
+    s0 = sc.risk_score_from_mu(k, v, torch.zeros(1, 4, 8), 4, epsilon=0.0)
+    kc, vc = k[:, 4:], v[:, 4:]
+    var = (vc - vc.mean(1, keepdim=True)).pow(2).sum(-1)
+    expect = (1 / 36) ** 2 * (vc.pow(2).sum(-1) + kc.pow(2).sum(-1) / 8 * var)
+    np.testing.assert_allclose(s0[:, 4:].numpy(), expect.numpy(), rtol=1e-5)
+    assert torch.all(s0[:, :4] == s0[:, 4:].max())
+    # scaling V by c scales every score by c^2
+    s1 = sc.risk_score_from_mu(k, v, mu, 4)
+    s3 = sc.risk_score_from_mu(k, 3 * v, mu, 4)
+    np.testing.assert_allclose(s3.numpy(), 9 * s1.numpy(), rtol=1e-5)
+    # with_attn on the same p (no sinks) reproduces the prefill core
+    core = sc.risk_score_with_attn(k[:, 4:], v[:, 4:], p[0])
+    np.testing.assert_allclose(core.numpy(), s1[:, 4:].numpy(), rtol=1e-5)
+    # short inputs
+    assert torch.all(sc.risk_score_from_mu(k[:, :4], v[:, :4], mu, 4) == 1)
