@@ -6,7 +6,7 @@ Follows /root/reference/kvquant/scorer.py
   _pad_sinks_and_normalize                    :321-325  (grain "global" = identity, :118-119)
   RiskScorer.score_prefill                    :385-404
   RiskScorer.score_with_attn                  :406-416
-  _NormFallback.score_prefill                 :145-147
+  _NormFallback.score_prefill                 :145-147 (+ _normalize_scores "layer" :130-134)
 and /root/reference/kvquant/attention_utils.py
   _repeat_kv :19-26, _get_query_states :29-54, _apply_avg_rope :57-115.
 
@@ -126,8 +126,18 @@ def pad_sinks(core_scores: torch.Tensor, n_sink: int) -> torch.Tensor:
 
 
 def norm_fallback(keys: torch.Tensor, values: torch.Tensor) -> torch.Tensor:
-    """|k| + |v| (scorer.py:145-147; grain "global" leaves it as is)."""
-    return keys.norm(dim=-1) + values.norm(dim=-1)
+    """|k| + |v|, min-max normalised over the layer (scorer.py:145-147 with :130-134).
+
+    The fallback scorer is its own object (scorer.py:176) and keeps the class default
+    ``normalize_grain = "layer"``; the factory sets "global" on the risk scorer only
+    (press_factory.py:59), so this path does normalise."""
+    raw = keys.norm(dim=-1) + values.norm(dim=-1)
+    if raw.numel() == 0:
+        return raw
+    lo, hi = raw.min(), raw.max()
+    if (hi - lo) < 1e-8:
+        return torch.full_like(raw, 0.5)
+    return (raw - lo) / (hi - lo)
 
 
 def risk_score_from_mu(keys: torch.Tensor, values: torch.Tensor, mu: torch.Tensor,
