@@ -1,0 +1,197 @@
+/* odmkv.h - C ABI of libodmkv.so: ODM-KV compression-and-decode kernels for AMD MI355X (gfx950).
+ *
+ * Every pointer named "device" is HIP device memory owned by the caller (the Python host
+ * side hands over torch tensors' data pointers).  The library allocates nothing that outlives
+ * a call; scratch space is passed in as a workspace whose size the matching *_workspace_bytes
+ * function returns.  All kernels are enqueued on the caller's stream (a hipStream_t passed as
+ * void*); no entry point synchronises the device.  Every entry point returns 0 on success or
+ * a negative ODMKV_E* code, and odmkv_last_error() then holds a message (thread local).
+ *
+ * Citations name the reference code (yiiwang118/ODM-KV) that each entry point stands in for.
+ */
+#ifndef ODMKV_H
+#define ODMKV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ODMKV_VERSION 1
+
+#define ODMKV_EINVAL   (-1)   /* bad argument: shape, level set, null pointer, unsupported head_dim */
+#define ODMKV_ENOSPACE (-2)   /* workspace too small */
+#define ODMKV_EHIP     (-3)   /* a HIP runtime call failed */
+
+/* element types of K/V/Q tensors */
+#define ODMKV_F16  0
+#define ODMKV_BF16 1
+#define ODMKV_F32  2
+
+#define ODMKV_HEAD_DIM   128  /* the only head_dim the kernels are written for */
+#define ODMKV_TILE       64   /* tokens per packed tile = one wavefront */
+#define ODMKV_NQ         4    /* quantised widths, in this order: 2, 3, 4, 8 bits */
+#define ODMKV_MAX_LEVELS 8    /* candidate bit levels of the allocator */
+#define ODMKV_MAX_GROUP  8    /* query heads per KV head (GQA group) */
+
+int odmkv_version(void);
+const char* odmkv_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Scorer.  Replaces RiskScorer.score_prefill after the mean query is known
+ * (kvquant/scorer.py:285-325, 385-404) and RiskScorer.score_with_attn (kvquant/scorer.py:406-416).
+ *
+ *   p[h,t]  = mean over the G query heads of kv-head h of softmax_t( mu[q] . K[h,t] / sqrt(d) ),  t >= n_sink
+ *   obar[h] = sum_t p[h,t] V[h,t] / max(sum_t p[h,t], 1e-8)
+ *   s[h,t]  = (p[h,t] + eps)^2 * ( |V[h,t]|^2 + |K[h,t]|^2 / d * |V[h,t] - obar[h]|^2 )
+ *   s[h, 0..n_sink) = max over all (h, t >= n_sink) of s
+ *
+ * K, V: [Hkv, T, 128] of `dtype`, element strides (stride_h, stride_t), innermost contiguous.
+ * mu: device fp32 [Hq, 128] (the RoPE-averaged mean query; Hq = G * Hkv).
+ * attn: NULL, or device fp32 [Hkv, T] attention weights to use instead of computing p from mu
+ *       (then n_sink must be 0 and no sink padding happens: score_with_attn).
+ * scores: device fp32 [Hkv, T] out.
+ */
+size_t odmkv_score_workspace_bytes(int Hkv, int Hq, int T);
+int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int T,
+                int64_t stride_h, int64_t stride_t,
+                const float* mu, int Hq, const float* attn, int n_sink, float eps,
+                float* scores, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Allocator.  Replaces optimal_scores_to_bits (kvquant/allocator.py:459-663) for a batch of
+ * independent rows (one row = one (layer, sequence): the flattened [Hkv, T] scores).
+ *
+ * scores: device fp32 [rows, n].  sink_mask: device uint8 [rows, n] (non-zero = sink, gets
+ * sink_bits and is left out of the budget) or NULL, in which case token i of a row is a sink
+ * iff (i % period) < n_sink.  levels: n_levels ascending bit widths (host).  eps: host fp64
+ * table, eps[k] for levels[k], already multiplied by eviction_cost / blended for
+ * above_target_alpha as the reference does on the host (allocator.py:549-569).
+ * target: device fp64 [rows], one budget per row (clamped into the level range on the device).
+ * bits_out: device int32 [rows, n].
+ * level_counts: device int32 [rows, n_levels] count of non-sink tokens per level, or NULL.
+ * lambda_out: device fp64 [rows] the multiplier found, or NULL.
+ */
+size_t odmkv_allocate_workspace_bytes(int rows, int n);
+int odmkv_allocate(const float* scores, int rows, int n,
+                   const uint8_t* sink_mask, int period, int n_sink, int sink_bits,
+                   const int32_t* levels, int n_levels, const double* eps,
+                   const double* target,
+                   int32_t* bits_out, int32_t* level_counts, double* lambda_out,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Packed mixed-width KV store.  Replaces the banks of TurboQuantAdaptiveKVCacheState
+ * (kvquant/tq_adaptive_backend.py:74-243, 346-374) with TurboQuantMSE.quantize / _pack_indices
+ * (kvquant/tq_backend.py:185-197, 103-125) as the quantiser.
+ *
+ * Tokens of one (sequence b, kv-head h) stored at one bit level form a segment; a segment is a
+ * whole number of 64-token tiles, tokens in ascending position, the tail of the last tile
+ * padded (pos = -1, norm = 0).  Level index li = 0..3 means 2, 3, 4, 8 bits; "exact" tokens
+ * (16 bits) are fp16/bf16 rows.  Within a tile of width w:
+ *   K codes, token-major:  the 16*w bytes of token l are w chunks of 16 bytes; chunk c of token
+ *            l sits at byte (c*64 + l)*16 of the tile.  The token's code stream is little
+ *            endian: code i occupies bits [i*w, i*w + w).
+ *   V codes, dim-major:    the 8*w bytes of dim j hold the codes of the 64 tokens, token t at
+ *            bits [t*w, t*w + w); they are split into units of U bytes (U = 16 for w = 2, 4, 8
+ *            and U = 8 for w = 3), unit u of dim j at byte (u*128 + j)*U of the tile.
+ *   norms fp32 [64], pos int32 [64] per tile.
+ *   exact K, token-major:  chunk c (16 bytes = 8 elements) of token l at byte (c*64 + l)*16.
+ *   exact V, dim-major in groups of 4 tokens: element (t, j) at 2-byte index
+ *            ((t/4)*128 + j)*4 + t%4 of the tile.
+ */
+typedef struct odmkv_packed {
+    int32_t B, Hkv;                      /* segments are indexed bh = b*Hkv + h */
+    int32_t exact_dtype;                 /* ODMKV_F16 or ODMKV_BF16 */
+    int32_t n_tiles[ODMKV_NQ + 1];       /* tiles allocated per level; index 4 = exact */
+    uint8_t* kcodes[ODMKV_NQ];           /* device, n_tiles[li] * 1024*w bytes */
+    uint8_t* vcodes[ODMKV_NQ];           /* device, n_tiles[li] * 1024*w bytes */
+    float*   knorm[ODMKV_NQ];            /* device, n_tiles[li] * 64 */
+    float*   vnorm[ODMKV_NQ];
+    int32_t* pos[ODMKV_NQ + 1];          /* device, n_tiles * 64 token positions, -1 = padding */
+    int32_t* seg_tile[ODMKV_NQ + 1];     /* device [B*Hkv + 1] first tile of each segment */
+    int32_t* seg_count[ODMKV_NQ + 1];    /* device [B*Hkv] tokens stored in each segment */
+    uint16_t* kexact;                    /* device, n_tiles[4] * 64*128 elements */
+    uint16_t* vexact;
+} odmkv_packed_t;
+
+/* Count tokens per (b, h, level): bits is device int32 [B, Hkv, T] with values in
+ * {0, 2, 3, 4, 8, 16}; counts is device int32 [B*Hkv, 6] in the order 0, 2, 3, 4, 8, 16.
+ * (The per-level mask / nonzero of tq_adaptive_backend.py:355-361.) */
+int odmkv_level_counts(const int32_t* bits, int B, int Hkv, int T, int32_t* counts, void* stream);
+
+/* Quantise and pack T new tokens per (b, h) into a store whose seg_tile tables are filled in
+ * and whose seg_count hold the tokens already present (0 after a reset); new tokens are
+ * appended behind them and seg_count is advanced.  K, V: [B, Hkv, T, 128] of `dtype` with
+ * element strides (stride_b, stride_h, stride_t).  bits: device int32 [B, Hkv, T].
+ * pos_offset is added to the token index to form the stored position.
+ * pi_k, pi_v: device fp32 [128,128] row-major rotations; codebooks: device fp32, the 4+8+16+256
+ * centroids of widths 2, 3, 4, 8 back to back.
+ * The arithmetic per token is, in this order and in fp32:
+ *   ss = fma(x_j, x_j, ss) j=0..127; norm = sqrt(ss); u_j = x_j / (norm + 1e-10);
+ *   y_i = fma(u_j, Pi[i][j], y_i) j=0..127; code_i = nearer of the two centroids bracketing y_i
+ *   (lower index on a tie). */
+size_t odmkv_pack_workspace_bytes(int B, int Hkv, int T);
+int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, int Hkv, int T,
+                     int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                     const int32_t* bits, int pos_offset,
+                     const float* pi_k, const float* pi_v, const float* codebooks,
+                     const odmkv_packed_t* store, void* workspace, size_t workspace_bytes,
+                     void* stream);
+
+/* Row-wise quantiser without the packed store: x [N, 128] of `dtype` with element stride
+ * `stride_n` -> codes uint8 [N, 128] (one code per byte) and norms fp32 [N], same arithmetic as
+ * odmkv_quant_pack.  `bits` is 2, 3, 4 or 8; cb the 2^bits centroids (device).  This is
+ * TurboQuantMSE.quantize before _pack_indices (kvquant/tq_backend.py:185-196). */
+int odmkv_quantize_rows(const void* x, int dtype, int64_t N, int64_t stride_n, int bits,
+                        const float* pi, const float* cb, uint8_t* codes, float* norms, void* stream);
+
+/* out[n] = (cb[codes[n]] @ Pi) * norms[n], fp32 [N, 128] (TurboQuantMSE.dequantize,
+ * kvquant/tq_backend.py:199-203). */
+int odmkv_dequantize_rows(const uint8_t* codes, const float* norms, int64_t N, int bits,
+                          const float* pi, const float* cb, float* out, void* stream);
+
+/* Dequantise the store into dense [B, Hkv, T, 128] tensors of `dtype` (strides as above):
+ * x_hat = (centroids[code] @ Pi) * norm, cast to dtype, written at the stored positions
+ * (TurboQuantMSE.dequantize, kvquant/tq_backend.py:199-203, and the scatter of
+ * QuantizedBank.materialize_into, kvquant/tq_adaptive_backend.py:205-242).
+ * include_exact != 0 also writes the exact tokens (ExactBank.materialize_into, :66-70);
+ * positions not stored are left untouched. */
+int odmkv_dequant(const odmkv_packed_t* store, void* K, void* V, int dtype, int T,
+                  int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                  const float* pi_k, const float* pi_v, const float* codebooks,
+                  int include_exact, void* stream);
+
+/* Append one fp16/bf16 token per (b, h) to the exact segments (append_all_exact,
+ * kvquant/tq_adaptive_backend.py:380-425, for one decode step).  k, v: [B, Hkv, 128] of the
+ * store's exact dtype, contiguous.  Fails with ODMKV_ENOSPACE semantics on the device side by
+ * leaving seg_count untouched when a segment is full; the caller sizes segments. */
+int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v, int pos,
+                       void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Fused LUT decode attention over the packed store: one query token per sequence.
+ * Stands where the reference runs the HF attention function over the re-materialised fp16
+ * cache (kvquant/attention_patch.py:30-55 on the tensors of tq_adaptive_backend.py:439-464):
+ *   out[b,q] = sum_t softmax_t( scaling * q[b,q] . Khat[b,q/G,t] ) Vhat[b,q/G,t]
+ * over the stored (non-evicted) tokens.  Evicted tokens are simply absent.
+ *
+ * q: device fp32 [B, Hq, 128].  items: device int32 [n_items, 4] work list
+ * (bh, level index 0..4, first tile, tile count), sorted by bh; item_range: device int32
+ * [B*Hkv + 1] first item of each bh.  out: device fp32 [B, Hq, 128]; lse: device fp32 [B, Hq]
+ * or NULL (log-sum-exp of the scaled logits).
+ */
+size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);
+int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
+                      const odmkv_packed_t* store,
+                      const int32_t* items, int n_items, const int32_t* item_range,
+                      const float* pi_k, const float* pi_v, const float* codebooks,
+                      float* out, float* lse, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ODMKV_H */

@@ -1,0 +1,342 @@
+// ODM risk score  s = (p + eps)^2 * (|v|^2 + |k|^2/d * |v - obar|^2)  for one layer of one sequence.
+//
+// K and V are each streamed from HBM once for the sums that need them (V a second time for
+// |v - obar|^2, which is computed directly rather than expanded, to avoid cancellation).
+// A row of 128 elements is handled by 16 lanes x 8 elements, so a wavefront reads four rows
+// (1 KB contiguous for a dense cache) per load instruction.  All reductions run in a fixed
+// order (shuffle butterflies, then ordered sums over chunk partials): results do not depend
+// on scheduling.
+#include "common.h"
+
+#define ROWS_PER_WG 256     // rows of one kv-head handled by a 256-thread workgroup
+#define LANES_PER_ROW 16
+
+struct ScoreArgs {
+    const void* K;
+    const void* V;
+    int64_t sH, sT;
+    int Hkv, Hq, G, Gl, T, Tc, n_sink, nchunks;   // Gl: heads the logits pass covers (0 when p is given)
+    float eps;
+    const float* mu;      // [Hq, 128]
+    const float* attn;    // [Hkv, T] or null
+    float* scores;        // [Hkv, T]
+    float* logits;        // [Hq, Tc]
+    float* kn2;           // [Hkv, Tc]
+    float* p;             // [Hkv, Tc]
+    float* stats;         // [Hq, nchunks, 2]
+    float* mz;            // [Hq, 2]
+    float* opart;         // [Hkv, nchunks, 128]
+    float* psum;          // [Hkv, nchunks]
+    float* obar;          // [Hkv, 128]
+    unsigned int* gmax;   // bit pattern of the running maximum score (scores are >= 0)
+};
+
+template <int DT>
+__device__ static inline void load8(const void* base, size_t elem_off, float* x) {
+    if constexpr (DT == ODMKV_F32) {
+        const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + elem_off);
+        const float4 a = p[0], b = p[1];
+        x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+    } else {
+        const uint4 v = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + elem_off);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            x[2 * e] = Elem<DT>::to_f32((uint16_t)(w[e] & 0xffffu));
+            x[2 * e + 1] = Elem<DT>::to_f32((uint16_t)(w[e] >> 16));
+        }
+    }
+}
+
+__device__ static inline float group16_sum(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+
+// merge two online-softmax states
+__device__ static inline void ms_merge(float& m, float& s, float m2, float s2) {
+    const float mn = fmaxf(m, m2);
+    if (mn == -INFINITY) { m = mn; s = 0.0f; return; }
+    s = s * __expf(m - mn) + s2 * __expf(m2 - mn);
+    m = mn;
+}
+
+// ---- pass 1 over K: logits of every query head, |k|^2, per-chunk softmax statistics ----
+template <int DT, int GMAX>
+__global__ __launch_bounds__(256) void score_logits_kernel(ScoreArgs a) {
+    __shared__ float mu_s[GMAX * HD];
+    __shared__ float red_m[4][GMAX], red_s[4][GMAX];
+    const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, part = lane & 15, rsub = lane >> 4;
+    for (int e = tid; e < a.Gl * HD; e += 256) mu_s[e] = a.mu[(size_t)h * a.G * HD + e];
+    __syncthreads();
+    float mu_r[GMAX][8];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mu_r[g][e] = g < a.Gl ? mu_s[g * HD + part * 8 + e] : 0.0f;
+    float m[GMAX], s[GMAX];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) { m[g] = -INFINITY; s[g] = 0.0f; }
+    const float inv_div = 11.313708498984761f;        // sqrt(128)
+    const int t0 = chunk * ROWS_PER_WG;
+    for (int it = 0; it < ROWS_PER_WG / 16; ++it) {
+        const int t = t0 + it * 16 + wave * 4 + rsub;
+        const bool ok = t < a.Tc;
+        float x[8];
+        if (ok) load8<DT>(a.K, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, x);
+        else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = 0.0f;
+        }
+        float kn = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) kn = __fmaf_rn(x[e], x[e], kn);
+        kn = group16_sum(kn);
+        if (ok && part == 0) a.kn2[(size_t)h * a.Tc + t] = kn;
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g) {
+            if (g < a.Gl) {
+                float d = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) d = __fmaf_rn(x[e], mu_r[g][e], d);
+                d = group16_sum(d) / inv_div;
+                if (ok && part == 0) {
+                    a.logits[((size_t)h * a.G + g) * a.Tc + t] = d;
+                    ms_merge(m[g], s[g], d, 1.0f);
+                }
+            }
+        }
+    }
+    // only lanes with part == 0 hold statistics; butterfly over the wave, then over the 4 waves
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+        if (g < a.Gl) {
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float m2 = __shfl_xor(m[g], o, WAVE), s2 = __shfl_xor(s[g], o, WAVE);
+                ms_merge(m[g], s[g], m2, s2);
+            }
+            if (lane == 0) { red_m[wave][g] = m[g]; red_s[wave][g] = s[g]; }
+        }
+    }
+    __syncthreads();
+    if (tid < a.Gl) {
+        float mm = red_m[0][tid], ss = red_s[0][tid];
+        for (int w = 1; w < 4; ++w) ms_merge(mm, ss, red_m[w][tid], red_s[w][tid]);
+        float* st = a.stats + (((size_t)h * a.G + tid) * a.nchunks + chunk) * 2;
+        st[0] = mm; st[1] = ss;
+    }
+}
+
+// ---- merge chunk statistics into (max, sum) per query head; also clears the running maximum ----
+__global__ __launch_bounds__(64) void score_stats_kernel(ScoreArgs a) {
+    const int hq = blockIdx.x, lane = threadIdx.x;
+    if (hq == 0 && lane == 0) *a.gmax = 0u;
+    if (a.Gl == 0) return;                    // attention weights were supplied: nothing to merge
+    float m = -INFINITY, s = 0.0f;
+    for (int c = lane; c < a.nchunks; c += WAVE) {
+        const float* st = a.stats + ((size_t)hq * a.nchunks + c) * 2;
+        ms_merge(m, s, st[0], st[1]);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float m2 = __shfl_xor(m, o, WAVE), s2 = __shfl_xor(s, o, WAVE);
+        ms_merge(m, s, m2, s2);
+    }
+    if (lane == 0) { a.mz[2 * hq] = m; a.mz[2 * hq + 1] = s; }
+}
+
+// ---- pass 1 over V: p, sum p, partial sums of p * v ----
+template <int DT, int GMAX>
+__global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
+    __shared__ float osum[16][HD];
+    __shared__ float psum_s[16];
+    const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, part = lane & 15, rsub = lane >> 4;
+    float Mg[GMAX], Zg[GMAX];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+        Mg[g] = (a.attn == nullptr && g < a.G) ? a.mz[2 * (h * a.G + g)] : 0.0f;
+        Zg[g] = (a.attn == nullptr && g < a.G) ? a.mz[2 * (h * a.G + g) + 1] : 1.0f;
+    }
+    float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    float ps = 0.0f;
+    const int t0 = chunk * ROWS_PER_WG;
+    for (int it = 0; it < ROWS_PER_WG / 16; ++it) {
+        const int t = t0 + it * 16 + wave * 4 + rsub;
+        if (t < a.Tc) {
+            float pt;
+            if (a.attn != nullptr) {
+                pt = a.attn[(size_t)h * a.T + a.n_sink + t];
+            } else {
+                float acc = 0.0f;
+#pragma unroll
+                for (int g = 0; g < GMAX; ++g)
+                    if (g < a.G) acc += __expf(a.logits[((size_t)h * a.G + g) * a.Tc + t] - Mg[g]) / Zg[g];
+                pt = acc / (float)a.G;
+            }
+            if (part == 0) { a.p[(size_t)h * a.Tc + t] = pt; ps += pt; }
+            float x[8];
+            load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, x);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = __fmaf_rn(pt, x[e], o[e]);
+        }
+    }
+    const int grp = wave * 4 + rsub;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) osum[grp][part * 8 + e] = o[e];
+    if (part == 0) psum_s[grp] = ps;
+    __syncthreads();
+    if (tid < HD) {
+        float acc = 0.0f;
+        for (int g = 0; g < 16; ++g) acc += osum[g][tid];
+        a.opart[((size_t)h * a.nchunks + chunk) * HD + tid] = acc;
+    }
+    if (tid == 0) {
+        float acc = 0.0f;
+        for (int g = 0; g < 16; ++g) acc += psum_s[g];
+        a.psum[(size_t)h * a.nchunks + chunk] = acc;
+    }
+}
+
+__global__ __launch_bounds__(128) void score_obar_kernel(ScoreArgs a) {
+    const int h = blockIdx.x, j = threadIdx.x;
+    float acc = 0.0f, P = 0.0f;
+    for (int c = 0; c < a.nchunks; ++c) {
+        acc += a.opart[((size_t)h * a.nchunks + c) * HD + j];
+        P += a.psum[(size_t)h * a.nchunks + c];
+    }
+    a.obar[h * HD + j] = acc / fmaxf(P, 1e-8f);
+}
+
+// ---- pass 2 over V: |v|^2, |v - obar|^2, the score, and its global maximum ----
+template <int DT>
+__global__ __launch_bounds__(256) void score_final_kernel(ScoreArgs a) {
+    __shared__ unsigned int wmax[4];
+    const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, part = lane & 15, rsub = lane >> 4;
+    float ob[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ob[e] = a.obar[h * HD + part * 8 + e];
+    float best = 0.0f;
+    const int t0 = chunk * ROWS_PER_WG;
+    for (int it = 0; it < ROWS_PER_WG / 16; ++it) {
+        const int t = t0 + it * 16 + wave * 4 + rsub;
+        const bool ok = t < a.Tc;
+        float x[8];
+        if (ok) load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, x);
+        else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = 0.0f;
+        }
+        float vn = 0.0f, ir = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            vn = __fmaf_rn(x[e], x[e], vn);
+            const float dlt = x[e] - ob[e];
+            ir = __fmaf_rn(dlt, dlt, ir);
+        }
+        vn = group16_sum(vn);
+        ir = group16_sum(ir);
+        if (ok && part == 0) {
+            const float pe = a.p[(size_t)h * a.Tc + t] + a.eps;
+            const float kterm = (a.kn2[(size_t)h * a.Tc + t] / (float)HD) * ir;
+            const float sc = (pe * pe) * (vn + kterm);
+            a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
+            best = fmaxf(best, sc);
+        }
+    }
+    best = wave_max(best);
+    if (lane == 0) wmax[wave] = __float_as_uint(best);
+    __syncthreads();
+    if (tid == 0) {
+        unsigned int mx = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
+        atomicMax(a.gmax, mx);        // non-negative floats order like their bit patterns
+    }
+}
+
+__global__ void score_pad_kernel(ScoreArgs a) {
+    const int h = blockIdx.x, i = threadIdx.x;
+    if (i < a.n_sink) a.scores[(size_t)h * a.T + i] = __uint_as_float(*a.gmax);
+}
+
+static inline int n_chunks(int Tc) { return (Tc + ROWS_PER_WG - 1) / ROWS_PER_WG; }
+
+struct ScoreLayout { size_t logits, kn2, p, stats, mz, opart, psum, obar, gmax, total; };
+static ScoreLayout score_layout(int Hkv, int Hq, int T) {
+    ScoreLayout L;
+    const size_t Tc = T, nc = n_chunks(T);
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes, 256); return o; };
+    L.logits = take((size_t)Hq * Tc * 4);
+    L.kn2 = take((size_t)Hkv * Tc * 4);
+    L.p = take((size_t)Hkv * Tc * 4);
+    L.stats = take((size_t)Hq * nc * 8);
+    L.mz = take((size_t)Hq * 8);
+    L.opart = take((size_t)Hkv * nc * HD * 4);
+    L.psum = take((size_t)Hkv * nc * 4);
+    L.obar = take((size_t)Hkv * HD * 4);
+    L.gmax = take(4);
+    L.total = off;
+    return L;
+}
+
+extern "C" size_t odmkv_score_workspace_bytes(int Hkv, int Hq, int T) {
+    if (Hkv <= 0 || Hq <= 0 || T <= 0) return 0;
+    return score_layout(Hkv, Hq, T).total;
+}
+
+template <int DT>
+static int run_score(ScoreArgs& a, hipStream_t st) {
+    dim3 grid(a.nchunks, a.Hkv), block(256);
+    if (a.G <= 4) hipLaunchKernelGGL((score_logits_kernel<DT, 4>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((score_logits_kernel<DT, 8>), grid, block, 0, st, a);
+    ODMKV_CHECK_LAUNCH("score_logits_kernel");
+    hipLaunchKernelGGL(score_stats_kernel, dim3(a.attn ? 1 : a.Hq), dim3(64), 0, st, a);
+    ODMKV_CHECK_LAUNCH("score_stats_kernel");
+    if (a.G <= 4) hipLaunchKernelGGL((score_pv_kernel<DT, 4>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((score_pv_kernel<DT, 8>), grid, block, 0, st, a);
+    ODMKV_CHECK_LAUNCH("score_pv_kernel");
+    hipLaunchKernelGGL(score_obar_kernel, dim3(a.Hkv), dim3(128), 0, st, a);
+    ODMKV_CHECK_LAUNCH("score_obar_kernel");
+    hipLaunchKernelGGL((score_final_kernel<DT>), grid, block, 0, st, a);
+    ODMKV_CHECK_LAUNCH("score_final_kernel");
+    if (a.n_sink > 0) {
+        hipLaunchKernelGGL(score_pad_kernel, dim3(a.Hkv), dim3(64), 0, st, a);
+        ODMKV_CHECK_LAUNCH("score_pad_kernel");
+    }
+    return 0;
+}
+
+extern "C" int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int T,
+                           int64_t stride_h, int64_t stride_t,
+                           const float* mu, int Hq, const float* attn, int n_sink, float eps,
+                           float* scores, void* workspace, size_t workspace_bytes, void* stream) {
+    ODMKV_CHECK_ARG(K && V && scores && workspace, "score: null pointer");
+    ODMKV_CHECK_ARG(mu || attn, "score: need the mean query or attention weights");
+    ODMKV_CHECK_ARG(dtype == ODMKV_F16 || dtype == ODMKV_BF16 || dtype == ODMKV_F32, "score: bad dtype %d", dtype);
+    ODMKV_CHECK_ARG(Hkv > 0 && Hq > 0 && Hq % Hkv == 0 && Hq / Hkv <= ODMKV_MAX_GROUP,
+                    "score: bad head counts Hkv=%d Hq=%d", Hkv, Hq);
+    ODMKV_CHECK_ARG(n_sink >= 0 && n_sink <= 64 && T > n_sink, "score: need T > n_sink (T=%d, n_sink=%d)", T, n_sink);
+    ODMKV_CHECK_ARG(!(attn && n_sink != 0), "score: attention-weight mode takes n_sink = 0");
+    const int align = dtype == ODMKV_F32 ? 4 : 8;
+    ODMKV_CHECK_ARG(stride_h % align == 0 && stride_t % align == 0 && stride_t >= HD,
+                    "score: strides must keep rows 16-byte aligned");
+    ODMKV_CHECK_ARG(((uintptr_t)K & 15) == 0 && ((uintptr_t)V & 15) == 0, "score: K/V must be 16-byte aligned");
+    ODMKV_CHECK_ARG(workspace_bytes >= odmkv_score_workspace_bytes(Hkv, Hq, T), "score: workspace too small");
+    const ScoreLayout L = score_layout(Hkv, Hq, T);
+    char* ws = (char*)workspace;
+    ScoreArgs a;
+    a.K = K; a.V = V; a.sH = stride_h; a.sT = stride_t;
+    a.Hkv = Hkv; a.Hq = Hq; a.G = Hq / Hkv; a.Gl = attn ? 0 : Hq / Hkv; a.T = T; a.Tc = T - n_sink; a.n_sink = n_sink;
+    a.nchunks = n_chunks(a.Tc); a.eps = eps; a.mu = mu; a.attn = attn; a.scores = scores;
+    a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
+    a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
+    a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == ODMKV_F16) return run_score<ODMKV_F16>(a, st);
+    if (dtype == ODMKV_BF16) return run_score<ODMKV_BF16>(a, st);
+    return run_score<ODMKV_F32>(a, st);
+}

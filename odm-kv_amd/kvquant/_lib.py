@@ -1,0 +1,122 @@
+"""ctypes binding of libodmkv.so, the C ABI declared in include/odmkv.h.
+
+The HIP library is the only compute path: importing this module fails if the library
+has not been built (``python odm-kv_amd/build.py``), and nothing falls back to PyTorch.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libodmkv.so")
+
+F16, BF16, F32 = 0, 1, 2
+HEAD_DIM = 128
+TILE = 64
+WIDTHS = (2, 3, 4, 8)                 # level index 0..3
+LEVEL_ORDER = (0, 2, 3, 4, 8, 16)     # order of odmkv_level_counts columns
+CODEBOOK_OFFSETS = (0, 4, 12, 28)
+CODEBOOK_FLOATS = 284
+
+_DT = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
+
+
+class Packed(C.Structure):
+    """struct odmkv_packed of include/odmkv.h."""
+    _fields_ = [
+        ("B", C.c_int32), ("Hkv", C.c_int32), ("exact_dtype", C.c_int32),
+        ("n_tiles", C.c_int32 * 5),
+        ("kcodes", C.c_void_p * 4), ("vcodes", C.c_void_p * 4),
+        ("knorm", C.c_void_p * 4), ("vnorm", C.c_void_p * 4),
+        ("pos", C.c_void_p * 5), ("seg_tile", C.c_void_p * 5), ("seg_count", C.c_void_p * 5),
+        ("kexact", C.c_void_p), ("vexact", C.c_void_p),
+    ]
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build the HIP kernels first (python odm-kv_amd/build.py). "
+            "There is no PyTorch fallback for the ODM-KV kernels.")
+    lib = C.CDLL(LIB_PATH)
+    i32, i64, vp, f32, sz = C.c_int, C.c_int64, C.c_void_p, C.c_float, C.c_size_t
+    sig = {
+        "odmkv_version": (C.c_int, []),
+        "odmkv_last_error": (C.c_char_p, []),
+        "odmkv_score_workspace_bytes": (sz, [i32, i32, i32]),
+        "odmkv_score": (C.c_int, [vp, vp, i32, i32, i32, i64, i64, vp, i32, vp, i32, f32, vp, vp, sz, vp]),
+        "odmkv_allocate_workspace_bytes": (sz, [i32, i32]),
+        "odmkv_allocate": (C.c_int, [vp, i32, i32, vp, i32, i32, i32, C.POINTER(C.c_int32), i32,
+                                     C.POINTER(C.c_double), vp, vp, vp, vp, vp, sz, vp]),
+        "odmkv_level_counts": (C.c_int, [vp, i32, i32, i32, vp, vp]),
+        "odmkv_pack_workspace_bytes": (sz, [i32, i32, i32]),
+        "odmkv_quant_pack": (C.c_int, [vp, vp, i32, i32, i32, i32, i64, i64, i64, vp, i32, vp, vp, vp,
+                                       C.POINTER(Packed), vp, sz, vp]),
+        "odmkv_quantize_rows": (C.c_int, [vp, i32, i64, i64, i32, vp, vp, vp, vp, vp]),
+        "odmkv_dequantize_rows": (C.c_int, [vp, vp, i64, i32, vp, vp, vp, vp]),
+        "odmkv_dequant": (C.c_int, [C.POINTER(Packed), vp, vp, i32, i32, i64, i64, i64, vp, vp, vp, i32, vp]),
+        "odmkv_append_exact": (C.c_int, [C.POINTER(Packed), vp, vp, i32, vp]),
+        "odmkv_decode_workspace_bytes": (sz, [i32, i32, i32]),
+        "odmkv_decode_attn": (C.c_int, [vp, i32, i32, f32, C.POINTER(Packed), vp, i32, vp, vp, vp, vp,
+                                        vp, vp, vp, sz, vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+EXPORTS = ("odmkv_version", "odmkv_last_error", "odmkv_score_workspace_bytes", "odmkv_score",
+           "odmkv_allocate_workspace_bytes", "odmkv_allocate", "odmkv_level_counts",
+           "odmkv_pack_workspace_bytes", "odmkv_quant_pack", "odmkv_quantize_rows",
+           "odmkv_dequantize_rows", "odmkv_dequant", "odmkv_append_exact",
+           "odmkv_decode_workspace_bytes", "odmkv_decode_attn")
+
+
+def check(rc: int) -> None:
+    """0 -> ok; EINVAL / ENOSPACE -> ValueError (as the reference raises on bad shapes and levels);
+    anything else -> RuntimeError."""
+    if rc == 0:
+        return
+    msg = lib.odmkv_last_error().decode("utf-8", "replace")
+    if rc in (-1, -2):
+        raise ValueError(f"odmkv: {msg}")
+    raise RuntimeError(f"odmkv: {msg} (code {rc})")
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {t.dtype}; expected float16, bfloat16 or float32") from None
+
+
+def require_gpu(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{what} must live on the GPU: the ODM-KV kernels have no CPU path")
+
+
+def stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+_ws_cache: dict[tuple, torch.Tensor] = {}
+
+
+def workspace(device, nbytes: int, tag: str = "") -> torch.Tensor:
+    """A reusable scratch buffer per (device, stream, tag); grown, never shrunk."""
+    key = (str(device), torch.cuda.current_stream(device).cuda_stream, tag)
+    buf = _ws_cache.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        _ws_cache[key] = buf
+    return buf

@@ -1,0 +1,164 @@
+"""KV-unit scoring: the ODM risk score on the GPU.
+
+Class names, constructor arguments and method signatures follow the reference's
+kvquant/scorer.py (BaseScorer :29-97, ExpectedAttentionScorer :154-202, RiskScorer :363-416);
+the per-token arithmetic runs in libodmkv:
+
+    s_j = (p_j + eps)^2 * ( |v_j|^2 + |k_j|^2 / d * |v_j - o_bar|^2 )
+
+with p the expected attention of the mean (RoPE-averaged) query, averaged over the GQA group.
+"""
+from __future__ import annotations
+
+from abc import ABC, abstractmethod
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import _lib
+from ._lib import lib
+from .attention_utils import (  # noqa: F401  (re-exported under the names callers import from here)
+    _aligned_rotary_outputs,
+    _apply_avg_rope,
+    _apply_rotary_pos_emb_q,
+    _get_query_states,
+    _mean_query_states,
+    _repeat_kv,
+    _rotate_half,
+)
+
+
+def _normalize_scores(raw: torch.Tensor, *, grain: str = "layer") -> torch.Tensor:
+    """Min-max normalisation: "layer" over the whole tensor, "head" per row, "global" none."""
+    if raw.numel() == 0 or grain == "global":
+        return raw
+    if grain == "head" and raw.dim() >= 2:
+        lo = raw.amin(dim=-1, keepdim=True)
+        hi = raw.amax(dim=-1, keepdim=True)
+        span = hi - lo
+        out = (raw - lo) / torch.where(span < 1e-8, torch.ones_like(span), span)
+        dead = span.squeeze(-1) < 1e-8
+        if dead.any():
+            out[dead] = 0.5
+        return out
+    lo, hi = raw.min(), raw.max()
+    if (hi - lo) < 1e-8:
+        return torch.full_like(raw, 0.5)
+    return (raw - lo) / (hi - lo)
+
+
+class BaseScorer(ABC):
+    """Interface every scorer implements."""
+
+    normalize_grain: str = "layer"
+
+    def _maybe_normalize(self, raw: torch.Tensor) -> torch.Tensor:
+        return _normalize_scores(raw, grain=self.normalize_grain)
+
+    @abstractmethod
+    def score_prefill(self, keys: torch.Tensor, values: torch.Tensor, layer_idx: int, *,
+                      module: nn.Module | None = None,
+                      hidden_states: torch.Tensor | None = None) -> torch.Tensor:
+        """keys/values [H, T, d] -> scores [H, T]."""
+
+    def score_decode(self, key: torch.Tensor, value: torch.Tensor, layer_idx: int, *,
+                     module: nn.Module | None = None,
+                     hidden_states: torch.Tensor | None = None) -> torch.Tensor:
+        return torch.ones(key.shape[0], device=key.device)
+
+    def score_with_attn(self, keys: torch.Tensor, values: torch.Tensor, attn_weights: torch.Tensor, *,
+                        module: nn.Module | None = None) -> torch.Tensor:
+        eps = float(getattr(self, "epsilon", 0.0) or 0.0)
+        return (attn_weights + eps).pow(2) * values.float().pow(2).sum(dim=-1)
+
+
+class _NormFallback(BaseScorer):
+    """|k| + |v|, used when the query statistics cannot be formed."""
+
+    def score_prefill(self, keys, values, layer_idx, *, module=None, hidden_states=None):
+        return self._maybe_normalize(keys.norm(dim=-1) + values.norm(dim=-1))
+
+    def score_decode(self, key, value, layer_idx, *, module=None, hidden_states=None):
+        return self._maybe_normalize(key.norm(dim=-1) + value.norm(dim=-1))
+
+
+class ExpectedAttentionScorer(BaseScorer):
+    """Holds the query statistics shared with ``RiskScorer``: the mean pre-RoPE query over the
+    prefill positions after the sinks, passed through the averaged future RoPE."""
+
+    def __init__(self, *, n_future_positions: int = 512, n_sink: int = 4, use_covariance: bool = True,
+                 use_vnorm: bool = True, epsilon: float = 0.0):
+        self.n_future_positions = n_future_positions
+        self.n_sink = n_sink
+        self.use_covariance = use_covariance
+        self.use_vnorm = use_vnorm
+        self.epsilon = epsilon
+        self._fallback = _NormFallback()
+
+    def _query_statistics(self, module: nn.Module, hidden_states: torch.Tensor):
+        q_len = hidden_states.shape[1]
+        if q_len <= self.n_sink:
+            raise ValueError("not enough tokens to estimate expected attention")
+        if self.use_covariance:
+            raise NotImplementedError("the covariance term is not part of the risk score and is not built")
+        mu = _mean_query_states(module, hidden_states[:, self.n_sink:])
+        return _apply_avg_rope(module, mu, None, q_len, self.n_future_positions)
+
+    def score_prefill(self, keys, values, layer_idx, *, module=None, hidden_states=None):
+        raise NotImplementedError("only the risk score (RiskScorer) runs on the GPU kernels")
+
+    def score_decode(self, key, value, layer_idx, *, module=None, hidden_states=None):
+        return self._fallback.score_decode(key, value, layer_idx, module=module, hidden_states=hidden_states)
+
+
+def _launch_score(keys: torch.Tensor, values: torch.Tensor, mu: Optional[torch.Tensor],
+                  attn: Optional[torch.Tensor], n_q_heads: int, n_sink: int, eps: float) -> torch.Tensor:
+    _lib.require_gpu(keys, "keys")
+    H, T, D = keys.shape
+    if D != _lib.HEAD_DIM:
+        raise ValueError(f"the HIP kernels are written for head_dim {_lib.HEAD_DIM}, got {D}")
+    align = 4 if keys.dtype == torch.float32 else 8
+    def ok(t):
+        return t.stride(-1) == 1 and t.stride(0) % align == 0 and t.stride(1) % align == 0 and t.data_ptr() % 16 == 0
+    if not ok(keys) or not ok(values) or keys.stride() != values.stride():
+        keys, values = keys.contiguous(), values.contiguous()
+    dev = keys.device
+    scores = torch.empty(H, T, dtype=torch.float32, device=dev)
+    ws_bytes = lib.odmkv_score_workspace_bytes(H, n_q_heads, T)
+    ws = _lib.workspace(dev, ws_bytes, "score")
+    mu32 = None if mu is None else mu.reshape(n_q_heads, D).float().contiguous()
+    a32 = None if attn is None else attn.float().contiguous()
+    _lib.check(lib.odmkv_score(
+        keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys), H, T, keys.stride(0), keys.stride(1),
+        _lib.ptr(mu32), n_q_heads, _lib.ptr(a32), n_sink, float(eps), scores.data_ptr(),
+        ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
+    return scores
+
+
+class RiskScorer(ExpectedAttentionScorer):
+    """s = (p + eps)^2 * [ |v|^2 + (|k|^2 / d) * |v - o|^2 ]: first-order joint error of the
+    attention output under independent key and value quantisation noise."""
+
+    def __init__(self, **kw):
+        kw["use_covariance"] = False
+        super().__init__(**kw)
+
+    def score_prefill(self, keys, values, layer_idx, *, module=None, hidden_states=None):
+        if module is None or hidden_states is None:
+            return self._fallback.score_prefill(keys, values, layer_idx)
+        if keys.shape[1] <= self.n_sink:
+            return torch.ones(keys.shape[:2], device=keys.device, dtype=keys.dtype)
+        if hidden_states.dim() == 2:
+            hidden_states = hidden_states.unsqueeze(0)
+        try:
+            mu, _ = self._query_statistics(module, hidden_states)
+        except (AttributeError, NotImplementedError, ValueError):
+            return self._fallback.score_prefill(keys, values, layer_idx)
+        n_q = mu.shape[1]
+        scores = _launch_score(keys, values, mu[0], None, n_q, self.n_sink, self.epsilon)
+        return self._maybe_normalize(scores)
+
+    def score_with_attn(self, keys, values, attn_weights, *, module=None):
+        H = keys.shape[0]
+        return _launch_score(keys, values, None, attn_weights, H, 0, self.epsilon)

@@ -1,0 +1,439 @@
+"""Mixed-precision KV store on the GPU: bit-packed tiles instead of per-level banks.
+
+``TurboQuantAdaptiveKVCacheState`` keeps the constructor and the method set of the reference's
+class of the same name (kvquant/tq_adaptive_backend.py:245-541): ``prefill``, ``append``,
+``append_all_exact``, ``truncate``, ``materialize``, ``materialize_quantized_into``,
+``get_buffer_tokens``, ``flush_buffer``, ``masked_key_indices`` - and adds what a packed store
+makes possible: ``decode_attention`` (fused LUT attention straight from the packed bytes) and
+``packed_bytes``.
+
+Layout (see include/odmkv.h): per bit level, tokens of one (sequence, kv-head) form a segment of
+64-token tiles in ascending position; keys are stored token-major, values dim-major, norms fp32.
+Evicted (0-bit) tokens are not stored at all.  The host keeps a mirror of every segment's length,
+so that after the one synchronisation an ``append`` needs (to size the buffers from the level
+counts) no later call has to read anything back.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from typing import Optional
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import lib, Packed, TILE, HEAD_DIM, WIDTHS
+from .tq_backend import (cached_rotation, codebook_table, normalize_key_quantizer,
+                         normalize_value_quantizer)
+
+_LEVEL_INDEX = {2: 0, 3: 1, 4: 2, 8: 3, 16: 4}
+_TILE_BYTES = [TILE * 16 * w + 2 * TILE * 4 for w in WIDTHS] + [2 * TILE * HEAD_DIM * 2]
+
+
+def _empty_positions(device) -> torch.Tensor:
+    return torch.empty((0, 3), dtype=torch.long, device=device)
+
+
+class TurboQuantAdaptiveKVCacheState:
+    def __init__(self, head_dim: int, bit_levels, value_group_size: int = 32, device=None,
+                 dtype: torch.dtype = torch.float16, key_quantizer: str = "prod",
+                 value_quantizer: str = "minmax", seed: int = 42, outlier_indices=None,
+                 regular_indices=None, outlier_min_bits: int = 4, exact_slack: int = 256):
+        levels = tuple(sorted(set(int(b) for b in bit_levels)))
+        self.key_quantizer = normalize_key_quantizer(key_quantizer)
+        self.value_quantizer = normalize_value_quantizer(value_quantizer)
+        min_bits = 2 if self.key_quantizer == "prod" else 1
+        invalid = [b for b in levels if b not in (0, 16) and b < min_bits]
+        if invalid:
+            raise ValueError(
+                f"Adaptive TurboQuant backend requires key bits >= {min_bits} "
+                f"for key_quantizer={self.key_quantizer!r}; unsupported levels: {invalid}")
+        if self.key_quantizer != "mse" or self.value_quantizer != "mse":
+            raise NotImplementedError(
+                "the packed GPU store implements key_quantizer='mse' and value_quantizer='mse' "
+                "(the paper configuration); QJL keys and min-max values are not built")
+        if outlier_indices is not None or regular_indices is not None:
+            raise NotImplementedError("outlier-channel separation is not built (n_outlier_channels must be 0)")
+        unsupported = [b for b in levels if b not in (0, 2, 3, 4, 8, 16)]
+        if unsupported:
+            raise ValueError(f"bit levels must come from (0, 2, 3, 4, 8, 16); got {unsupported}")
+        if head_dim != HEAD_DIM:
+            raise ValueError(f"the HIP kernels are written for head_dim {HEAD_DIM}, got {head_dim}")
+        self.head_dim = head_dim
+        self.bit_levels = levels
+        group = min(value_group_size, head_dim)
+        if head_dim % group != 0:
+            group = math.gcd(head_dim, group)
+        self.value_group_size = max(1, group)
+        self.device = torch.device(device) if device is not None else torch.device("cuda")
+        self.dtype = dtype
+        self.seed = seed
+        self.outlier_min_bits = outlier_min_bits
+        self.exact_slack = int(exact_slack)
+        if self.device.type != "cuda":
+            raise RuntimeError("the packed KV store lives on the GPU; there is no CPU path")
+        self.pi_k = cached_rotation(head_dim, self.device, seed)
+        self.pi_v = cached_rotation(head_dim, self.device, seed + 2000)
+        self.codebooks = codebook_table(head_dim, self.device)
+        self._exact_torch_dtype = torch.bfloat16 if dtype == torch.bfloat16 else torch.float16
+        self._reset()
+
+    # ------------------------------------------------------------------ storage
+    def _reset(self) -> None:
+        self.batch_size = 0
+        self.num_heads = 0
+        self.seq_len = 0
+        self._nseg = 0
+        self._counts = None           # np.int64 [5, nseg]   tokens stored per level and segment
+        self._seg_tile = None         # np.int64 [5, nseg+1] first tile of each segment
+        self._bufs = None
+        self._level_map = None        # uint8 [B, H, seq_len]: bit level of every position
+        self._items = None
+        self._packed = None
+
+    def _alloc(self, seg_tile: np.ndarray) -> dict:
+        dev = self.device
+        n_tiles = seg_tile[:, -1]
+        bufs = {"seg_tile": [], "seg_count": [], "pos": [], "kcodes": [], "vcodes": [], "knorm": [], "vnorm": []}
+        for li in range(5):
+            nt = int(n_tiles[li])
+            bufs["seg_tile"].append(torch.from_numpy(seg_tile[li].astype(np.int32)).to(dev))
+            bufs["seg_count"].append(torch.zeros(self._nseg, dtype=torch.int32, device=dev))
+            bufs["pos"].append(torch.full((max(nt, 1) * TILE,), -1, dtype=torch.int32, device=dev))
+            if li < 4:
+                w = WIDTHS[li]
+                bufs["kcodes"].append(torch.zeros(max(nt, 1) * TILE * 16 * w, dtype=torch.uint8, device=dev))
+                bufs["vcodes"].append(torch.zeros(max(nt, 1) * HEAD_DIM * 8 * w, dtype=torch.uint8, device=dev))
+                bufs["knorm"].append(torch.zeros(max(nt, 1) * TILE, dtype=torch.float32, device=dev))
+                bufs["vnorm"].append(torch.zeros(max(nt, 1) * TILE, dtype=torch.float32, device=dev))
+        nt = int(n_tiles[4])
+        bufs["kexact"] = torch.zeros(max(nt, 1) * TILE * HEAD_DIM, dtype=self._exact_torch_dtype, device=dev)
+        bufs["vexact"] = torch.zeros(max(nt, 1) * TILE * HEAD_DIM, dtype=self._exact_torch_dtype, device=dev)
+        return bufs
+
+    def _make_struct(self) -> None:
+        p = Packed()
+        p.B, p.Hkv = self.batch_size, self.num_heads
+        p.exact_dtype = _lib.BF16 if self._exact_torch_dtype == torch.bfloat16 else _lib.F16
+        b = self._bufs
+        for li in range(5):
+            p.n_tiles[li] = int(self._seg_tile[li, -1])
+            p.pos[li] = b["pos"][li].data_ptr()
+            p.seg_tile[li] = b["seg_tile"][li].data_ptr()
+            p.seg_count[li] = b["seg_count"][li].data_ptr()
+            if li < 4:
+                p.kcodes[li] = b["kcodes"][li].data_ptr()
+                p.vcodes[li] = b["vcodes"][li].data_ptr()
+                p.knorm[li] = b["knorm"][li].data_ptr()
+                p.vnorm[li] = b["vnorm"][li].data_ptr()
+        p.kexact = b["kexact"].data_ptr()
+        p.vexact = b["vexact"].data_ptr()
+        self._packed = p
+
+    def _capacity_tiles(self, counts: np.ndarray) -> np.ndarray:
+        """Tiles per (level, segment) for `counts` tokens; exact segments get room to grow."""
+        cap = (counts + TILE - 1) // TILE
+        cap[4] = (counts[4] + self.exact_slack + TILE - 1) // TILE
+        return cap
+
+    def _ensure_capacity(self, new_counts: np.ndarray) -> None:
+        """Make every segment large enough for `new_counts`, moving stored tiles if it must grow."""
+        if self._bufs is not None:
+            have = np.diff(self._seg_tile, axis=1)
+            if np.all((new_counts + TILE - 1) // TILE <= have):
+                return
+        cap = self._capacity_tiles(new_counts)
+        if self._bufs is not None:
+            cap = np.maximum(cap, np.diff(self._seg_tile, axis=1))
+        seg_tile = np.zeros((5, self._nseg + 1), np.int64)
+        seg_tile[:, 1:] = np.cumsum(cap, axis=1)
+        new = self._alloc(seg_tile)
+        if self._bufs is not None:
+            old, old_tile = self._bufs, self._seg_tile
+            for li in range(5):
+                used = (self._counts[li] + TILE - 1) // TILE
+                if used.sum() == 0:
+                    continue
+                src = np.concatenate([np.arange(old_tile[li, s], old_tile[li, s] + used[s]) for s in range(self._nseg)])
+                dst = np.concatenate([np.arange(seg_tile[li, s], seg_tile[li, s] + used[s]) for s in range(self._nseg)])
+                src_t = torch.from_numpy(src).to(self.device)
+                dst_t = torch.from_numpy(dst).to(self.device)
+                names = ["pos"] + (["kcodes", "vcodes", "knorm", "vnorm"] if li < 4 else [])
+                for name in names:
+                    o, n = old[name][li], new[name][li]
+                    per = o.numel() // max(int(old_tile[li, -1]), 1)
+                    n.view(-1, per)[dst_t] = o.view(-1, per)[src_t]
+                if li == 4:
+                    for name in ("kexact", "vexact"):
+                        new[name].view(-1, TILE * HEAD_DIM)[dst_t] = old[name].view(-1, TILE * HEAD_DIM)[src_t]
+                new["seg_count"][li].copy_(old["seg_count"][li])
+        self._bufs = new
+        self._seg_tile = seg_tile
+        self._make_struct()
+
+    # ------------------------------------------------------------------ validation
+    def _validate_shapes(self, keys: torch.Tensor, values: torch.Tensor, bits: Optional[torch.Tensor]) -> None:
+        if keys.shape != values.shape:
+            raise ValueError(f"Mismatched key/value shapes: {keys.shape} vs {values.shape}")
+        if keys.dim() != 4:
+            raise ValueError(f"Expected keys/values with shape [B, H, T, D], got {keys.shape}")
+        if bits is not None and tuple(bits.shape) != tuple(keys.shape[:3]):
+            raise ValueError(f"Expected bits shape {tuple(keys.shape[:3])}, got {tuple(bits.shape)}")
+        if keys.shape[-1] != self.head_dim:
+            raise ValueError(f"Expected head_dim {self.head_dim}, got {keys.shape[-1]}")
+        _lib.require_gpu(keys, "keys")
+        _lib.require_gpu(values, "values")
+        if self.batch_size == 0:
+            self.batch_size = int(keys.shape[0])
+            self.num_heads = int(keys.shape[1])
+            self._nseg = self.batch_size * self.num_heads
+            self._counts = np.zeros((5, self._nseg), np.int64)
+        elif self.batch_size != int(keys.shape[0]) or self.num_heads != int(keys.shape[1]):
+            raise ValueError(
+                f"Adaptive backend state shape changed from (B={self.batch_size}, H={self.num_heads}) "
+                f"to (B={keys.shape[0]}, H={keys.shape[1]})")
+
+    @staticmethod
+    def _rows_ok(t: torch.Tensor) -> bool:
+        align = 4 if t.dtype == torch.float32 else 8
+        return (t.stride(-1) == 1 and all(s % align == 0 for s in t.stride()[:-1])
+                and t.stride(2) >= t.shape[-1] and t.data_ptr() % 16 == 0)
+
+    # ------------------------------------------------------------------ writes
+    def prefill(self, keys: torch.Tensor, values: torch.Tensor, bits: torch.Tensor) -> None:
+        self._reset()
+        self.append(keys, values, bits)
+
+    def append(self, keys: torch.Tensor, values: torch.Tensor, bits: torch.Tensor,
+               _pos_offset: Optional[int] = None) -> None:
+        self._validate_shapes(keys, values, bits)
+        B, H, T, D = keys.shape
+        if T == 0:
+            return
+        dev = self.device
+        bits = bits.to(device=dev, dtype=torch.int32).contiguous()
+        if not self._rows_ok(keys):
+            keys = keys.contiguous()
+        if not self._rows_ok(values) or values.stride() != keys.stride():
+            values = values.contiguous()
+            keys = keys.contiguous()
+        st = _lib.stream_ptr(dev)
+        counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
+        _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
+        counts = counts_dev.cpu().numpy().astype(np.int64)            # the one synchronisation
+        if int(counts.sum()) != self._nseg * T:
+            raise ValueError("bits must take values in (0, 2, 3, 4, 8, 16)")
+        present = {lvl for lvl, c in zip(_lib.LEVEL_ORDER, counts.sum(axis=0)) if c > 0}
+        if not present <= set(self.bit_levels):
+            raise ValueError(f"bits use levels {sorted(present - set(self.bit_levels))} outside bit_levels={self.bit_levels}")
+        new_counts = self._counts + counts[:, 1:].T
+        self._ensure_capacity(new_counts)
+        pos_offset = self.seq_len if _pos_offset is None else int(_pos_offset)
+        ws_bytes = lib.odmkv_pack_workspace_bytes(B, H, T)
+        ws = _lib.workspace(dev, ws_bytes, "pack")
+        _lib.check(lib.odmkv_quant_pack(
+            keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys), B, H, T,
+            keys.stride(0), keys.stride(1), keys.stride(2), bits.data_ptr(), pos_offset,
+            self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
+            C.byref(self._packed), ws.data_ptr(), ws_bytes, st))
+        self._counts = new_counts
+        lm = bits.to(torch.uint8)
+        if _pos_offset is None:
+            self._level_map = lm if self._level_map is None else torch.cat([self._level_map, lm], dim=2)
+            self.seq_len += T
+        else:
+            self._level_map[:, :, pos_offset:pos_offset + T] = lm
+        self._items = None
+
+    def append_all_exact(self, keys: torch.Tensor, values: torch.Tensor) -> None:
+        """Every new token goes to the exact (16-bit) segments."""
+        self._validate_shapes(keys, values, None)
+        B, H, T, D = keys.shape
+        if T == 0:
+            return
+        if T > 1 or self._bufs is None or keys.dtype != self._exact_torch_dtype:
+            bits = torch.full((B, H, T), 16, dtype=torch.int32, device=self.device)
+            self.append(keys, values, bits)
+            return
+        new_counts = self._counts.copy()
+        new_counts[4] += 1
+        had = self._seg_tile
+        self._ensure_capacity(new_counts)
+        k = keys.reshape(B, H, D).contiguous()
+        v = values.reshape(B, H, D).contiguous()
+        _lib.check(lib.odmkv_append_exact(C.byref(self._packed), k.data_ptr(), v.data_ptr(), self.seq_len,
+                                          _lib.stream_ptr(self.device)))
+        self._counts = new_counts
+        fresh = torch.full((B, H, 1), 16, dtype=torch.uint8, device=self.device)
+        self._level_map = torch.cat([self._level_map, fresh], dim=2)
+        self.seq_len += 1
+        if had is not self._seg_tile:
+            self._items = None
+
+    def truncate(self, seq_len: int) -> None:
+        seq_len = int(seq_len)
+        if seq_len >= self.seq_len:
+            return
+        self.seq_len = seq_len
+        self._level_map = self._level_map[:, :, :seq_len].contiguous()
+        # positions ascend inside a segment, so the survivors are a prefix of it
+        for li in range(5):
+            if self._counts[li].sum() == 0:
+                continue
+            pos = self._bufs["pos"][li].cpu().numpy()
+            for s in range(self._nseg):
+                c = int(self._counts[li, s])
+                if c:
+                    first = int(self._seg_tile[li, s]) * TILE
+                    self._counts[li, s] = int(np.searchsorted(pos[first:first + c], seq_len, side="left"))
+            self._bufs["seg_count"][li].copy_(torch.from_numpy(self._counts[li].astype(np.int32)))
+        self._items = None
+
+    # ------------------------------------------------------------------ reads
+    def _dequant_into(self, keys: torch.Tensor, values: torch.Tensor, include_exact: bool) -> None:
+        if self._bufs is None:
+            return
+        if not (self._rows_ok(keys) and self._rows_ok(values) and keys.stride() == values.stride()):
+            raise ValueError("materialisation targets must be row-contiguous [B, H, T, D] tensors with equal strides")
+        _lib.check(lib.odmkv_dequant(
+            C.byref(self._packed), keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys),
+            int(keys.shape[2]), keys.stride(0), keys.stride(1), keys.stride(2),
+            self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
+            1 if include_exact else 0, _lib.stream_ptr(self.device)))
+
+    def materialize(self) -> tuple[torch.Tensor, torch.Tensor]:
+        keys = torch.zeros(self.batch_size, self.num_heads, self.seq_len, self.head_dim,
+                           device=self.device, dtype=self.dtype)
+        values = torch.zeros_like(keys)
+        self._dequant_into(keys, values, True)
+        return keys, values
+
+    def materialize_quantized_into(self, keys: torch.Tensor, values: torch.Tensor) -> None:
+        """Overwrite the quantised positions of existing dense tensors; exact and evicted
+        positions are left as they are."""
+        self._dequant_into(keys, values, False)
+
+    def masked_key_indices(self):
+        if self._level_map is None:
+            return None
+        idx = (self._level_map == 0).nonzero(as_tuple=True)
+        if idx[0].numel() == 0:
+            return None
+        return idx
+
+    def visible_mask(self) -> torch.Tensor:
+        return self._level_map != 0
+
+    def level_counts(self) -> dict[int, int]:
+        out = {b: int(self._counts[_LEVEL_INDEX[b]].sum()) for b in (2, 3, 4, 8, 16)}
+        out[0] = self.batch_size * self.num_heads * self.seq_len - sum(out.values())
+        return out
+
+    def packed_bytes(self) -> int:
+        """Bytes the fused decode kernel has to read: codes + norms of the quantised tokens and the
+        fp16 rows of the exact ones (positions and segment tables are not read by it)."""
+        total = int(self._counts[4].sum()) * 2 * HEAD_DIM * 2
+        for li, w in enumerate(WIDTHS):
+            total += int(self._counts[li].sum()) * (2 * w * HEAD_DIM // 8 + 8)
+        return total
+
+    # ------------------------------------------------------------------ decode buffer
+    def _exact_rows(self, start: int):
+        """(positions [N,3] long, keys [N,D], values [N,D]) of exact tokens at positions >= start,
+        ordered by (batch, head, position)."""
+        if self._bufs is None or self._counts[4].sum() == 0:
+            return None
+        pos = self._bufs["pos"][4]
+        slots, bh = [], []
+        pos_host = pos.cpu().numpy()
+        for s in range(self._nseg):
+            c = int(self._counts[4, s])
+            first = int(self._seg_tile[4, s]) * TILE
+            k = int(np.searchsorted(pos_host[first:first + c], start, side="left"))
+            slots.append(np.arange(first + k, first + c))
+            bh.append(np.full(c - k, s))
+        slots = np.concatenate(slots)
+        if slots.size == 0:
+            return None
+        bh = np.concatenate(bh)
+        st = torch.from_numpy(slots).to(self.device)
+        nt = self._bufs["kexact"].numel() // (TILE * HEAD_DIM)
+        krows = self._bufs["kexact"].view(nt, 16, TILE, 8).permute(0, 2, 1, 3).reshape(nt * TILE, HEAD_DIM)[st]
+        vrows = self._bufs["vexact"].view(nt, 16, HEAD_DIM, 4).permute(0, 1, 3, 2).reshape(nt * TILE, HEAD_DIM)[st]
+        p3 = np.stack([bh // self.num_heads, bh % self.num_heads, pos_host[slots]], axis=-1).astype(np.int64)
+        return torch.from_numpy(p3).to(self.device), krows, vrows
+
+    def get_buffer_tokens(self, buffer_start_seq: int):
+        got = self._exact_rows(int(buffer_start_seq))
+        if got is None:
+            empty = torch.empty(0, self.head_dim, device=self.device, dtype=self.dtype)
+            return _empty_positions(self.device), empty, empty.clone()
+        return got
+
+    def flush_buffer(self, buffer_start_seq: int, new_bits: torch.Tensor) -> None:
+        """Re-quantise the exact tokens at positions >= buffer_start_seq to `new_bits` (one entry
+        per token, in the order `get_buffer_tokens` returns them)."""
+        start = int(buffer_start_seq)
+        got = self._exact_rows(start)
+        if got is None:
+            return
+        pos3, krows, vrows = got
+        n_buf = self.seq_len - start
+        if pos3.shape[0] != self._nseg * n_buf:
+            raise ValueError("flush_buffer expects every position >= buffer_start_seq to be exact in every head")
+        B, H = self.batch_size, self.num_heads
+        k = krows.reshape(B, H, n_buf, self.head_dim).contiguous()
+        v = vrows.reshape(B, H, n_buf, self.head_dim).contiguous()
+        bits = new_bits.to(device=self.device, dtype=torch.int32).reshape(B, H, n_buf)
+        # drop the buffered tokens from the exact segments, then append them at their new levels
+        self._counts[4] -= n_buf
+        self._bufs["seg_count"][4].copy_(torch.from_numpy(self._counts[4].astype(np.int32)))
+        self.append(k, v, bits, _pos_offset=start)
+
+    # ------------------------------------------------------------------ fused attention
+    def _build_items(self, target_items: int = 1024, min_item_bytes: int = 16384) -> None:
+        used = (self._counts + TILE - 1) // TILE
+        used[4] = np.diff(self._seg_tile[4])              # exact segments grow between rebuilds
+        total = sum(int(used[li].sum()) * _TILE_BYTES[li] for li in range(5))
+        per_item = max(total // max(target_items, 1), min_item_bytes)
+        items, ranges = [], [0]
+        for s in range(self._nseg):
+            for li in range(5):
+                nt = int(used[li, s])
+                if nt == 0:
+                    continue
+                step = max(1, int(round(per_item / _TILE_BYTES[li])))
+                t0 = int(self._seg_tile[li, s])
+                for a in range(0, nt, step):
+                    items.append((s, li, t0 + a, min(step, nt - a)))
+            ranges.append(len(items))
+        arr = np.asarray(items, np.int32).reshape(-1, 4)
+        self._items = (torch.from_numpy(arr).to(self.device),
+                       torch.from_numpy(np.asarray(ranges, np.int32)).to(self.device), len(items))
+
+    def decode_attention(self, query: torch.Tensor, scaling: Optional[float] = None,
+                         return_lse: bool = False):
+        """softmax(scaling * q K^T) V over the stored tokens, for one query token per sequence.
+
+        query: [B, Hq, D] or [B, Hq, 1, D] on the GPU; returns fp32 [B, Hq, D] (and lse [B, Hq])."""
+        _lib.require_gpu(query, "query")
+        if self._bufs is None:
+            raise ValueError("the store is empty")
+        q = query.reshape(query.shape[0], query.shape[1], self.head_dim).float().contiguous()
+        B, Hq, D = q.shape
+        if B != self.batch_size or Hq % self.num_heads != 0:
+            raise ValueError(f"query heads {tuple(q.shape)} do not match the store (B={self.batch_size}, Hkv={self.num_heads})")
+        if self._items is None:
+            self._build_items()
+        items, ranges, n_items = self._items
+        scale = 1.0 / math.sqrt(D) if scaling is None else float(scaling)
+        out = torch.empty(B, Hq, D, dtype=torch.float32, device=self.device)
+        lse = torch.empty(B, Hq, dtype=torch.float32, device=self.device) if return_lse else None
+        ws_bytes = lib.odmkv_decode_workspace_bytes(B, Hq, n_items)
+        ws = _lib.workspace(self.device, ws_bytes, "decode")
+        _lib.check(lib.odmkv_decode_attn(
+            q.data_ptr(), B, Hq, scale, C.byref(self._packed), items.data_ptr(), n_items,
+            ranges.data_ptr(), self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
+            out.data_ptr(), _lib.ptr(lse), ws.data_ptr(), ws_bytes, _lib.stream_ptr(self.device)))
+        return (out, lse) if return_lse else out

@@ -1,0 +1,94 @@
+"""CPU-only checks of the C ABI: the library loads, exports every declared symbol, and rejects
+bad arguments with an error code and a message before touching a GPU."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "odm-kv_amd", "lib", "libodmkv.so")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(LIB):
+        pytest.fail("libodmkv.so is not built: run python odm-kv_amd/build.py")
+    return C.CDLL(LIB)
+
+
+def test_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "odmkv.h")).read()
+    declared = set(re.findall(r"\b(odmkv_[a-z_]+)\s*\(", header))
+    assert len(declared) >= 15
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in odmkv.h but not exported"
+    from kvquant import _lib
+    assert set(_lib.EXPORTS) == declared
+
+
+def test_version_and_error_slot(lib):
+    assert lib.odmkv_version() == 1
+    lib.odmkv_last_error.restype = C.c_char_p
+    lib.odmkv_score.restype = C.c_int
+    rc = lib.odmkv_score(None, None, 0, 8, 100, C.c_int64(0), C.c_int64(0), None, 32, None, 4,
+                         C.c_float(0.01), None, None, C.c_size_t(0), None)
+    assert rc == -1 and b"null" in lib.odmkv_last_error()
+
+
+def test_argument_checks_without_a_gpu(lib):
+    lib.odmkv_last_error.restype = C.c_char_p
+    buf = C.create_string_buffer(4096)
+    p = C.cast(buf, C.c_void_p)
+    # head counts that do not divide
+    rc = lib.odmkv_score(p, p, 0, 3, 100, C.c_int64(128 * 100), C.c_int64(128), p, 8, None, 4,
+                         C.c_float(0.01), p, p, C.c_size_t(1 << 30), None)
+    assert rc == -1 and b"head counts" in lib.odmkv_last_error()
+    # T <= n_sink
+    rc = lib.odmkv_score(p, p, 0, 2, 4, C.c_int64(512), C.c_int64(128), p, 4, None, 4,
+                         C.c_float(0.01), p, p, C.c_size_t(1 << 30), None)
+    assert rc == -1 and b"n_sink" in lib.odmkv_last_error()
+    # workspace too small
+    lib.odmkv_score_workspace_bytes.restype = C.c_size_t
+    assert lib.odmkv_score_workspace_bytes(8, 32, 4096) > 0
+    # descending levels
+    levels = (C.c_int32 * 3)(4, 2, 8)
+    eps = (C.c_double * 3)(0.1, 0.2, 0.3)
+    rc = lib.odmkv_allocate(p, 1, 64, None, 64, 4, 16, levels, 3, eps, p, p, None, None, p, C.c_size_t(1 << 30), None)
+    assert rc == -1 and b"ascending" in lib.odmkv_last_error()
+    # unsupported width
+    rc = lib.odmkv_quantize_rows(p, 0, C.c_int64(4), C.c_int64(128), 5, p, p, p, p, None)
+    assert rc == -1 and b"width" in lib.odmkv_last_error()
+    rc = lib.odmkv_decode_attn(None, 1, 8, C.c_float(1.0), None, None, 0, None, None, None, None, None, None, None,
+                               C.c_size_t(0), None)
+    assert rc == -1
+
+
+def test_host_modules_import_and_validate():
+    import torch
+    from kvquant import RiskScorer, effective_bits, ratio_scores_to_bits, scores_to_bits
+    from kvquant.tq_backend import _pack_indices, _unpack_indices, random_rotation
+    assert effective_bits(2, 8, 128, 4) == 2 + 8 * 2 / 128
+    codes = torch.randint(0, 8, (3, 128))
+    assert torch.equal(_unpack_indices(_pack_indices(codes, 3), 3, 128), codes)
+    pi = random_rotation(128, "cpu", torch.float32, seed=42)
+    assert torch.allclose(pi @ pi.T, torch.eye(128), atol=1e-5)
+    s = torch.rand(2, 40)
+    assert set(scores_to_bits(s, (2, 4, 8)).unique().tolist()) <= {2, 4, 8}
+    assert ratio_scores_to_bits(s, (2, 4), (0.5, 0.5)).shape == s.shape
+    sc = RiskScorer(n_future_positions=512, n_sink=4, epsilon=1e-2)
+    # CPU tensors have no kernel path: asking for it is an error, not a silent fallback
+    with pytest.raises(RuntimeError):
+        sc.score_with_attn(torch.zeros(1, 8, 128), torch.zeros(1, 8, 128), torch.ones(1, 8) / 8)
+
+
+def test_host_ratio_and_container_match_reference(golden):
+    import torch
+    from kvquant.allocator import ratio_scores_to_bits, scores_to_bits
+    from kvquant.tq_backend import _pack_indices
+    sr = torch.from_numpy(golden["ratio_scores"])
+    assert (ratio_scores_to_bits(sr, (2, 3, 4, 8, 16), (0.5, 0.2, 0.15, 0.1, 0.05)).numpy() == golden["ratio_bits"]).all()
+    assert (scores_to_bits(sr, (2, 3, 4, 8, 16)).numpy() == golden["uniform_bits"]).all()
+    for b in (1, 2, 3, 4, 8):
+        codes = torch.from_numpy(golden[f"pack_b{b}_codes"])
+        assert (_pack_indices(codes, b).numpy() == golden[f"pack_b{b}_bytes"]).all()

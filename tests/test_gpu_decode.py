@@ -1,0 +1,136 @@
+"""GPU parity: fused LUT decode attention over the packed store vs the oracle
+(fp64 softmax attention over the oracle's materialised cache), <= 1e-3 relative."""
+import numpy as np
+import pytest
+import torch
+
+from oracle.attention import decode_attention, decode_attention_state
+from oracle.kvstate import KVState
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+ATTN_RTOL = 1e-3       # the tolerance the north star states for attention outputs
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    """Worst per-head relative L2 error."""
+    num = (got.double() - want.double()).norm(dim=-1)
+    return float((num / want.double().norm(dim=-1).clamp_min(1e-30)).max())
+
+
+def _rand_bits(g, shape, probs):
+    levels = torch.tensor((0, 2, 3, 4, 8, 16), dtype=torch.int32)
+    return levels[torch.multinomial(torch.tensor(probs), int(np.prod(shape)), replacement=True, generator=g)].reshape(shape)
+
+
+def _pair(k, v, bits, dtype=torch.float16, seed=42):
+    from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+    st = TurboQuantAdaptiveKVCacheState(128, (0, 2, 3, 4, 8, 16), device=DEV, dtype=dtype,
+                                        key_quantizer="mse", value_quantizer="mse", seed=seed)
+    st.prefill(k.to(DEV), v.to(DEV), bits.to(DEV))
+    ref = KVState(128, (0, 2, 3, 4, 8, 16), dtype=dtype, seed=seed, order="canonical")
+    ref.prefill(k, v, bits)
+    return st, ref
+
+
+@pytest.mark.parametrize("B,Hkv,G,T,probs", [
+    (1, 2, 4, 700, (0.25, 0.4, 0.12, 0.1, 0.08, 0.05)),
+    (2, 2, 7, 333, (0.3, 0.3, 0.1, 0.1, 0.1, 0.1)),
+    (1, 8, 4, 4096, (0.3, 0.55, 0.07, 0.05, 0.02, 0.01)),
+    (3, 1, 1, 130, (0.0, 1.0, 0.0, 0.0, 0.0, 0.0)),
+    (1, 2, 8, 257, (0.0, 0.0, 0.0, 0.0, 1.0, 0.0)),
+    (1, 2, 2, 200, (0.0, 0.0, 1.0, 0.0, 0.0, 0.0)),
+])
+def test_decode_matches_oracle(B, Hkv, G, T, probs):
+    g = torch.Generator().manual_seed(T + G)
+    k = torch.randn(B, Hkv, T, 128, generator=g)
+    v = torch.randn(B, Hkv, T, 128, generator=g)
+    k[:, :, :4] *= 8; v[:, :, :4] *= 8
+    k, v = k.half(), v.half()
+    bits = _rand_bits(g, (B, Hkv, T), probs)
+    bits[..., :4] = 16
+    bits[..., -16:] = 16
+    q = torch.randn(B, Hkv * G, 128, generator=g)
+    st, ref = _pair(k, v, bits)
+    got, lse = st.decode_attention(q.to(DEV), return_lse=True)
+    want = decode_attention_state(q, ref)
+    assert got.shape == (B, Hkv * G, 128) and got.dtype == torch.float32
+    assert rel_err(got.cpu(), want) < ATTN_RTOL
+    # the log-sum-exp of the scaled logits
+    kk, vv = ref.materialize()
+    logits = torch.einsum("bhd,bhtd->bht", q.double(), kk.double().repeat_interleave(G, dim=1)) / 128 ** 0.5
+    logits = logits.masked_fill(~ref.visible_mask().repeat_interleave(G, dim=1), float("-inf"))
+    np.testing.assert_allclose(lse.cpu().numpy(), torch.logsumexp(logits, -1).numpy(), rtol=1e-3, atol=1e-3)
+
+
+def test_decode_special_cases():
+    g = torch.Generator().manual_seed(1)
+    k = torch.randn(1, 2, 300, 128, generator=g).half(); v = torch.randn(1, 2, 300, 128, generator=g).half()
+    q = torch.randn(1, 8, 128, generator=g)
+    # every token exact: equals SDPA on the fp16 cache
+    st, _ = _pair(k, v, torch.full((1, 2, 300), 16, dtype=torch.int32))
+    sdpa = torch.nn.functional.scaled_dot_product_attention(
+        q[:, :, None].double(), k.double().repeat_interleave(4, dim=1), v.double().repeat_interleave(4, dim=1))[:, :, 0]
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), sdpa) < 1e-5
+    # a single visible token: the output is that token's (dequantised) value
+    bits = torch.zeros(1, 2, 300, dtype=torch.int32); bits[:, :, 17] = 4
+    st, ref = _pair(k, v, bits)
+    _, vm = ref.materialize()
+    want = vm[:, :, 17].double().repeat_interleave(4, dim=1)
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
+    # a custom scaling and the [B, Hq, 1, D] query shape
+    bits = _rand_bits(g, (1, 2, 300), (0.2, 0.4, 0.1, 0.1, 0.1, 0.1))
+    st, ref = _pair(k, v, bits)
+    got = st.decode_attention(q[:, :, None].to(DEV), scaling=0.05)
+    assert rel_err(got.cpu(), decode_attention_state(q, ref, scaling=0.05)) < ATTN_RTOL
+    # bf16 cache
+    st, ref = _pair(k.bfloat16(), v.bfloat16(), bits, dtype=torch.bfloat16)
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
+
+
+def test_decode_after_appends_and_flush():
+    g = torch.Generator().manual_seed(8)
+    B, H, G = 1, 4, 4
+    k = torch.randn(B, H, 500, 128, generator=g).half(); v = torch.randn(B, H, 500, 128, generator=g).half()
+    bits = _rand_bits(g, (B, H, 500), (0.3, 0.4, 0.1, 0.1, 0.05, 0.05)); bits[..., -32:] = 16
+    st, ref = _pair(k, v, bits)
+    for step in range(70):
+        kn = torch.randn(B, H, 1, 128, generator=g).half(); vn = torch.randn(B, H, 1, 128, generator=g).half()
+        st.append_all_exact(kn.to(DEV), vn.to(DEV)); ref.append_all_exact(kn, vn)
+        if step % 23 == 0 or step == 69:
+            q = torch.randn(B, H * G, 128, generator=g)
+            assert rel_err(st.decode_attention(q.to(DEV)).cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
+    pos, _, _ = st.get_buffer_tokens(500)
+    rpos, _, _ = ref.get_buffer_tokens(500)
+    nb = _rand_bits(g, (pos.shape[0],), (0.0, 0.5, 0.2, 0.15, 0.1, 0.05))
+    key_ours = (pos[:, 1] * 10 ** 6 + pos[:, 2]).cpu().numpy()
+    lookup = {kk: i for i, kk in enumerate(key_ours)}
+    perm = np.asarray([lookup[kk] for kk in (rpos[:, 1] * 10 ** 6 + rpos[:, 2])])
+    st.flush_buffer(500, nb.to(DEV)); ref.flush_buffer(500, nb[perm])
+    q = torch.randn(B, H * G, 128, generator=g)
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
+
+
+def test_config1_end_to_end():
+    """Benchmark config 1: score -> allocate (2.0 bits) -> pack -> one-token decode, all on the GPU,
+    each stage compared with the oracle fed the previous stage's GPU output."""
+    import synthetic
+    from kvquant.allocator import calibrate_epsilon, optimal_scores_to_bits
+    from kvquant.scorer import _launch_score
+    from oracle import allocator as oal, scorer as osc
+    L = synthetic.config("c1")
+    Hkv, T, _ = L.keys.shape
+    scores = _launch_score(L.keys.to(DEV), L.values.to(DEV), L.mu.to(DEV), None, L.n_q_heads, 4, 1e-2)
+    want_scores = osc.risk_score_from_mu(L.keys.float(), L.values.float(), L.mu.unsqueeze(0), L.n_q_heads)
+    np.testing.assert_allclose(scores.cpu().numpy(), want_scores.numpy(), rtol=1e-3)
+    eps = calibrate_epsilon(128, synthetic.LEVELS, device=DEV, value_quantizer="mse")
+    sink = torch.zeros(Hkv, T, dtype=torch.bool); sink[:, :4] = True
+    bits = optimal_scores_to_bits(scores, synthetic.LEVELS, 2.0, eps, sink.to(DEV), eviction_cost=0.5)
+    want_bits = oal.optimal_scores_to_bits(scores.cpu(), synthetic.LEVELS, 2.0, eps, sink, eviction_cost=0.5)
+    np.testing.assert_array_equal(bits.cpu().numpy(), want_bits.numpy())
+    core = bits[:, 4:].float()
+    assert abs(core.mean().item() - 2.0) < 1e-3
+    bits = bits.clone(); bits[:, -128:] = 16
+    st, ref = _pair(L.keys[None], L.values[None], bits[None].cpu())
+    got = st.decode_attention(L.query[None].to(DEV))
+    assert rel_err(got.cpu(), decode_attention_state(L.query[None], ref)) < ATTN_RTOL

@@ -1,0 +1,210 @@
+"""GPU parity: TurboQuant-MSE quantiser, packed store, dequantise (through the C ABI)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import quantizer as oq
+from oracle.codebook import codebook_f32
+from oracle.kvstate import KVState
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _rand_bits(g, shape, levels=(0, 2, 3, 4, 8, 16), probs=(0.25, 0.4, 0.12, 0.1, 0.08, 0.05)):
+    idx = torch.multinomial(torch.tensor(probs), int(np.prod(shape)), replacement=True, generator=g)
+    return torch.tensor(levels, dtype=torch.int32)[idx].reshape(shape)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_quantize_rows_bit_exact(bits, dtype):
+    from kvquant.tq_backend import TurboQuantMSE
+    g = torch.Generator().manual_seed(100 + bits)
+    x = (torch.randn(1000, 128, generator=g) * torch.exp(torch.randn(1000, 1, generator=g))).to(dtype)
+    x[5] = 0                                                   # a zero row must not blow up
+    q = TurboQuantMSE(128, bits, device=DEV, dtype=dtype, seed=42)
+    np.testing.assert_array_equal(q.centroids.cpu().numpy(), codebook_f32(bits, 128))
+    codes, norms = q.quantize_codes(x.to(DEV))
+    ref = oq.quantize(x, q.pi.cpu(), bits, order="canonical")
+    np.testing.assert_array_equal(norms.cpu().numpy(), ref.norms)          # same fp32 bits
+    np.testing.assert_array_equal(codes.cpu().numpy(), ref.codes)          # every code identical
+    # against the library-ordered (BLAS) statement: only coordinates on a cell boundary may move
+    blas = oq.quantize(x, q.pi.cpu(), bits, order="blas")
+    diff = blas.codes != codes.cpu().numpy()
+    assert diff.mean() < 2e-3
+    assert np.all(np.abs(blas.codes[diff].astype(int) - codes.cpu().numpy()[diff].astype(int)) == 1)
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+def test_container_roundtrip_and_dequantize(bits):
+    from kvquant.tq_backend import TurboQuantMSE, _unpack_indices
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(300, 128, generator=g).half()
+    q = TurboQuantMSE(128, bits, device=DEV, dtype=torch.float16, seed=7)
+    mq = q.quantize(x.to(DEV))
+    codes, _ = q.quantize_codes(x.to(DEV))
+    np.testing.assert_array_equal(mq.indices.cpu().numpy(), oq.pack_codes(codes.cpu().numpy(), bits))
+    assert torch.equal(_unpack_indices(mq.indices, bits, 128), codes.long())
+    rec = q.dequantize(mq).cpu()
+    ref = oq.dequantize(oq.Quantized(codes.cpu().numpy(), mq.norms.cpu().numpy(), bits), q.pi.cpu())
+    # fp32 with a different summation order: 1e-5 relative to the row norm
+    err = (rec - ref).norm(dim=-1) / ref.norm(dim=-1)
+    assert err.max() < 1e-5
+    rel = ((x.float() - rec) ** 2).sum() / (x.float() ** 2).sum()
+    assert rel < {2: 0.13, 3: 0.04, 4: 0.011, 8: 1e-4}[bits]
+
+
+def _state(levels=(0, 2, 3, 4, 8, 16), dtype=torch.float16, seed=42):
+    from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+    return TurboQuantAdaptiveKVCacheState(128, levels, device=DEV, dtype=dtype, key_quantizer="mse",
+                                          value_quantizer="mse", seed=seed)
+
+
+def _check_store_against_oracle(state, ref: KVState):
+    from packed_layout import decode_exact, decode_level
+    H = state.num_heads
+    for li, w in enumerate((2, 3, 4, 8)):
+        bank = ref.banks.get(w)
+        got = decode_level(state, li)
+        n_ref = 0 if bank is None else bank.size
+        assert len(got["pos"]) == n_ref, f"level {w}: {len(got['pos'])} stored, oracle {n_ref}"
+        if n_ref == 0:
+            continue
+        # oracle banks are in (b, h, t) order within an append; sort both by (bh, pos)
+        key_ref = bank.pos[:, 0] * H * 10 ** 7 + bank.pos[:, 1] * 10 ** 7 + bank.pos[:, 2]
+        key_got = got["bh"].astype(np.int64) * 10 ** 7 + got["pos"]
+        o_ref, o_got = np.argsort(key_ref, kind="stable"), np.argsort(key_got, kind="stable")
+        np.testing.assert_array_equal(key_got[o_got], key_ref[o_ref])
+        np.testing.assert_array_equal(got["kcodes"][o_got], bank.kc[o_ref])
+        np.testing.assert_array_equal(got["vcodes"][o_got], bank.vc[o_ref])
+        np.testing.assert_array_equal(got["knorm"][o_got], bank.kn[o_ref])
+        np.testing.assert_array_equal(got["vnorm"][o_got], bank.vn[o_ref])
+        # ascending positions inside every segment
+        for s in np.unique(got["bh"]):
+            assert np.all(np.diff(got["pos"][got["bh"] == s]) > 0)
+    ex = decode_exact(state)
+    assert len(ex["pos"]) == ref.exact.size
+    if ref.exact.size:
+        key_ref = ref.exact.pos[:, 0] * H * 10 ** 7 + ref.exact.pos[:, 1] * 10 ** 7 + ref.exact.pos[:, 2]
+        key_got = ex["bh"].astype(np.int64) * 10 ** 7 + ex["pos"]
+        o_ref, o_got = np.argsort(key_ref, kind="stable"), np.argsort(key_got, kind="stable")
+        np.testing.assert_array_equal(key_got[o_got], key_ref[o_ref])
+        np.testing.assert_array_equal(ex["k"][o_got], ref.exact.k.view(torch.int16).numpy()[o_ref])
+        np.testing.assert_array_equal(ex["v"][o_got], ref.exact.v.view(torch.int16).numpy()[o_ref])
+
+
+def _ulp_close_fp16(a: torch.Tensor, b: torch.Tensor, max_ulp=1, max_frac=0.02):
+    ai, bi = a.view(torch.int16).int(), b.view(torch.int16).int()
+    ai = torch.where(ai < 0, -32768 - ai, ai)          # map sign-magnitude to a monotone scale
+    bi = torch.where(bi < 0, -32768 - bi, bi)
+    d = (ai - bi).abs()
+    assert int(d.max()) <= max_ulp, f"max fp16 ulp distance {int(d.max())}"
+    assert float((d > 0).float().mean()) <= max_frac
+
+
+@pytest.mark.parametrize("B,H,T", [(1, 2, 300), (2, 3, 129), (1, 8, 1000)])
+def test_prefill_codes_positions_and_materialize(B, H, T):
+    g = torch.Generator().manual_seed(B * 1000 + T)
+    k = torch.randn(B, H, T, 128, generator=g).half()
+    v = (torch.randn(B, H, T, 128, generator=g) * 2).half()
+    bits = _rand_bits(g, (B, H, T))
+    bits[..., -5:] = 16
+    state = _state()
+    state.prefill(k.to(DEV), v.to(DEV), bits.to(DEV))
+    ref = KVState(128, (0, 2, 3, 4, 8, 16), seed=42, order="canonical")
+    ref.prefill(k, v, bits)
+    assert state.seq_len == T and state.batch_size == B and state.num_heads == H
+    _check_store_against_oracle(state, ref)
+    assert state.packed_bytes() == ref.packed_bytes()
+    # dense read-back
+    km, vm = state.materialize()
+    kr, vr = ref.materialize()
+    _ulp_close_fp16(km.cpu(), kr)
+    _ulp_close_fp16(vm.cpu(), vr)
+    evicted = torch.from_numpy(ref.level_map() == 0)
+    assert torch.all(km.cpu()[evicted] == 0) and torch.all(vm.cpu()[evicted] == 0)
+    exact = torch.from_numpy(ref.level_map() == 16)
+    assert torch.equal(km.cpu()[exact], k[exact]) and torch.equal(vm.cpu()[exact], v[exact])
+    # in-place variant leaves exact and evicted positions untouched
+    k2, v2 = k.clone().to(DEV), v.clone().to(DEV)
+    state.materialize_quantized_into(k2, v2)
+    untouched = evicted | exact
+    assert torch.equal(k2.cpu()[untouched], k[untouched])
+    assert torch.equal(k2.cpu()[~untouched], km.cpu()[~untouched])
+    # evicted index lists agree
+    mi, ri = state.masked_key_indices(), ref.masked_key_indices()
+    assert (mi is None) == (ri is None)
+    if mi is not None:
+        for a, b in zip(mi, ri):
+            assert torch.equal(a.cpu(), b)
+
+
+def test_append_truncate_and_flush_follow_the_oracle():
+    g = torch.Generator().manual_seed(77)
+    B, H, D = 1, 4, 128
+    k0 = torch.randn(B, H, 200, D, generator=g).half(); v0 = torch.randn(B, H, 200, D, generator=g).half()
+    bits0 = _rand_bits(g, (B, H, 200)); bits0[..., -16:] = 16
+    state, ref = _state(), KVState(128, (0, 2, 3, 4, 8, 16), seed=42, order="canonical")
+    state.prefill(k0.to(DEV), v0.to(DEV), bits0.to(DEV)); ref.prefill(k0, v0, bits0)
+    # a second block with its own bits (tail tiles are partially filled: read-modify-write on V)
+    k1 = torch.randn(B, H, 70, D, generator=g).half(); v1 = torch.randn(B, H, 70, D, generator=g).half()
+    bits1 = _rand_bits(g, (B, H, 70))
+    state.append(k1.to(DEV), v1.to(DEV), bits1.to(DEV)); ref.append(k1, v1, bits1)
+    _check_store_against_oracle(state, ref)
+    # 40 single-token decode steps into the exact segments
+    for _ in range(40):
+        kn = torch.randn(B, H, 1, D, generator=g).half(); vn = torch.randn(B, H, 1, D, generator=g).half()
+        state.append_all_exact(kn.to(DEV), vn.to(DEV)); ref.append_all_exact(kn, vn)
+    assert state.seq_len == ref.seq_len == 310
+    _check_store_against_oracle(state, ref)
+    # flush the 40 buffered tokens to new levels
+    pos, bk, bv = state.get_buffer_tokens(270)
+    rpos, rk, rv = ref.get_buffer_tokens(270)
+    assert pos.shape[0] == rpos.shape[0] == H * 40
+    new_bits = _rand_bits(g, (H * 40,), probs=(0.0, 0.5, 0.2, 0.15, 0.1, 0.05))
+    # the oracle's buffer order is step-major; ours is (b, h, t): map one onto the other
+    key_ours = (pos[:, 1] * 10 ** 6 + pos[:, 2]).cpu().numpy()
+    key_ref = rpos[:, 1] * 10 ** 6 + rpos[:, 2]
+    lookup = {kk: i for i, kk in enumerate(key_ours)}
+    perm = np.asarray([lookup[kk] for kk in key_ref])
+    assert torch.equal(bk.cpu()[perm], rk) and torch.equal(bv.cpu()[perm], rv)
+    state.flush_buffer(270, new_bits.to(DEV)); ref.flush_buffer(270, new_bits[perm])
+    _check_store_against_oracle(state, ref)
+    km, vm = state.materialize(); kr, vr = ref.materialize()
+    _ulp_close_fp16(km.cpu(), kr); _ulp_close_fp16(vm.cpu(), vr)
+    # rewind
+    state.truncate(150); ref.truncate(150)
+    assert state.seq_len == 150
+    _check_store_against_oracle(state, ref)
+    km, vm = state.materialize(); kr, vr = ref.materialize()
+    assert km.shape == kr.shape
+    _ulp_close_fp16(km.cpu(), kr)
+
+
+def test_edge_cases_and_errors():
+    from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn(1, 2, 64, 128, generator=g).half().to(DEV)
+    # everything evicted / everything exact / a single level
+    for fill in (0, 16, 4):
+        st = _state()
+        st.prefill(k, k, torch.full((1, 2, 64), fill, dtype=torch.int32, device=DEV))
+        km, _ = st.materialize()
+        if fill == 0:
+            assert torch.all(km == 0) and st.packed_bytes() == 0
+        if fill == 16:
+            assert torch.equal(km, k)
+    st = _state()
+    with pytest.raises(ValueError):
+        st.prefill(k, k[:, :1], torch.zeros(1, 2, 64, dtype=torch.int32, device=DEV))
+    with pytest.raises(ValueError):
+        st.prefill(k, k, torch.zeros(1, 2, 63, dtype=torch.int32, device=DEV))
+    with pytest.raises(ValueError):
+        st.prefill(k, k, torch.full((1, 2, 64), 5, dtype=torch.int32, device=DEV))
+    with pytest.raises(ValueError):
+        TurboQuantAdaptiveKVCacheState(128, (0, 1, 4), device=DEV, key_quantizer="prod", value_quantizer="mse")
+    with pytest.raises(NotImplementedError):
+        TurboQuantAdaptiveKVCacheState(128, (0, 2, 4), device=DEV)      # defaults are prod / minmax
+    with pytest.raises(ValueError):
+        TurboQuantAdaptiveKVCacheState(64, (0, 2, 4), device=DEV, key_quantizer="mse", value_quantizer="mse")

@@ -1,0 +1,160 @@
+"""GPU parity: risk scorer (<= 1e-3 relative, fp32 accumulate) and Lagrangian allocator (bit exact)."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import allocator as oal
+from oracle import scorer as osc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+LEVELS = (0, 2, 3, 4, 8, 16)
+EPS = {0: 1.0, 2: 0.12022445693985273, 3: 0.037507650590957564, 4: 0.012159048378616812,
+       8: 0.0011957171333694236, 16: 0.0}
+SCORE_RTOL = 1e-3      # the tolerance the north star states for scores
+
+
+def _sink(h, t, n=4):
+    m = torch.zeros(h, t, dtype=torch.bool)
+    m[:, :n] = True
+    return m
+
+
+class Stub(torch.nn.Module):
+    def __init__(self, hidden, n_heads, head_dim, seed, rotary=False, n_kv=None):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.q_proj = torch.nn.Linear(hidden, n_heads * head_dim, bias=True)
+        with torch.no_grad():
+            self.q_proj.weight.copy_(torch.randn(n_heads * head_dim, hidden, generator=g) / hidden ** 0.5)
+            self.q_proj.bias.copy_(torch.randn(n_heads * head_dim, generator=g) * 0.1)
+        self.config = types.SimpleNamespace(num_attention_heads=n_heads, head_dim=head_dim)
+        self.head_dim = head_dim
+        if rotary:
+            from transformers import LlamaConfig
+            from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+            self.rotary_emb = LlamaRotaryEmbedding(LlamaConfig(
+                hidden_size=n_heads * head_dim, num_attention_heads=n_heads, num_key_value_heads=n_kv or n_heads,
+                head_dim=head_dim, rope_theta=500000.0, max_position_embeddings=8192))
+
+
+@pytest.mark.parametrize("hkv,hq,T,dtype,rotary", [
+    (2, 8, 700, torch.float32, False), (8, 32, 4096, torch.float16, False), (4, 28, 1500, torch.bfloat16, False),
+    (2, 4, 300, torch.float32, True), (3, 3, 261, torch.float16, False), (1, 1, 5, torch.float32, False)])
+def test_score_prefill_matches_oracle(hkv, hq, T, dtype, rotary):
+    from kvquant.scorer import RiskScorer
+    g = torch.Generator().manual_seed(T)
+    k = torch.randn(hkv, T, 128, generator=g); v = torch.randn(hkv, T, 128, generator=g)
+    k[:, :4] *= 8; v[:, :4] *= 8
+    k, v = k.to(dtype), v.to(dtype)
+    h = torch.randn(1, T, 96, generator=g)
+    mod = Stub(96, hq, 128, T + 1, rotary=rotary, n_kv=hkv)
+    sc = RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
+    sc.normalize_grain = "global"
+    with torch.no_grad():
+        # the oracle runs the reference arithmetic on fp32 copies of the same K/V values
+        want = osc.risk_score_prefill(k.float(), v.float(), module=mod, hidden_states=h)
+        got = sc.score_prefill(k.to(DEV), v.to(DEV), 0, module=mod.to(DEV), hidden_states=h.to(DEV))
+    assert got.shape == (hkv, T) and got.dtype == torch.float32
+    np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=SCORE_RTOL)
+    assert torch.all(got[:, :4] == got[:, 4:].max())
+
+
+def test_score_special_cases():
+    from kvquant.scorer import RiskScorer
+    sc = RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
+    sc.normalize_grain = "global"
+    g = torch.Generator().manual_seed(3)
+    k = torch.randn(2, 50, 128, generator=g).half(); v = torch.randn(2, 50, 128, generator=g).half()
+    a = torch.softmax(torch.randn(2, 50, generator=g), dim=-1)
+    got = sc.score_with_attn(k.to(DEV), v.to(DEV), a.to(DEV))
+    np.testing.assert_allclose(got.cpu().numpy(), osc.risk_score_with_attn(k, v, a).numpy(), rtol=SCORE_RTOL)
+    # no module: the norm fallback (layer min-max)
+    fb = sc.score_prefill(k.to(DEV), v.to(DEV), 0)
+    np.testing.assert_allclose(fb.float().cpu().numpy(), osc.risk_score_prefill(k, v).float().numpy(), rtol=2e-3, atol=1e-3)
+    # not longer than the sinks: ones
+    assert torch.all(sc.score_prefill(k[:, :4].to(DEV), v[:, :4].to(DEV), 0, module=Stub(8, 2, 128, 1),
+                                      hidden_states=torch.zeros(1, 4, 8)) == 1)
+
+
+def _check_alloc(scores, target, sink=None, levels=LEVELS, **kw):
+    from kvquant.allocator import optimal_scores_to_bits
+    kw.setdefault("eviction_cost", 0.5)
+    got = optimal_scores_to_bits(scores.to(DEV), levels, target, EPS, None if sink is None else sink.to(DEV), **kw)
+    want = oal.optimal_scores_to_bits(scores, levels, target, EPS, sink, **kw)
+    assert got.dtype == torch.int32 and got.shape == scores.shape
+    np.testing.assert_array_equal(got.cpu().numpy(), want.numpy())
+    return got
+
+
+@pytest.mark.parametrize("target", [1.5, 2.0, 3.0, 6.5])
+def test_allocator_bit_exact_random(target):
+    g = torch.Generator().manual_seed(int(target * 10))
+    s = torch.exp(2.0 * torch.randn(8, 4096, generator=g))
+    s[:, :4] = s.max()
+    _check_alloc(s, target, _sink(8, 4096))
+
+
+def test_allocator_bit_exact_edge_cases():
+    g = torch.Generator().manual_seed(9)
+    vals = torch.exp(torch.linspace(-3, 6, 12))
+    ties = vals[torch.randint(0, 12, (4, 900), generator=g)]
+    _check_alloc(ties, 2.0, _sink(4, 900))                     # repair inside groups of equal scores
+    _check_alloc(ties, 3.0, _sink(4, 900))
+    _check_alloc(torch.full((2, 640), 3.0), 2.0)               # all equal
+    bad = torch.exp(torch.randn(2, 500, generator=g))
+    bad[0, 10] = float("inf"); bad[1, 20] = float("nan"); bad[0, 30] = -5.0; bad[1, 40] = float("-inf")
+    _check_alloc(bad, 2.0, _sink(2, 500))
+    _check_alloc(torch.full((1, 64), float("nan")), 2.0)
+    s = torch.exp(torch.randn(2, 333, generator=g))
+    _check_alloc(s, 40.0)                                       # target above the top level
+    _check_alloc(s, 0.5, levels=(2, 4, 8), eviction_cost=5.0)   # below the lowest
+    _check_alloc(s, 2.0, _sink(2, 333), levels=(4,))            # a single level
+    _check_alloc(s, 2.5, levels=(0, 2, 4, 8), eviction_cost=5.0)
+    _check_alloc(s, 2.0, _sink(2, 333), above_target_alpha=0.5)
+    _check_alloc(s, 2.0, torch.ones(2, 333, dtype=torch.bool))  # nothing but sinks
+    for n in (1, 2, 5):
+        _check_alloc(torch.exp(torch.randn(1, n, generator=g)), 2.0)
+    # an arbitrary (not prefix-shaped) sink mask
+    m = torch.rand(2, 333, generator=g) < 0.1
+    _check_alloc(s, 2.0, m)
+
+
+def test_allocator_matches_reference_vectors(golden):
+    from kvquant.allocator import optimal_scores_to_bits
+    eps = {int(k): float(v) for k, v in zip(golden["alloc_eps_levels"], golden["alloc_eps_values"])}
+    for name, kw in {"paper2": dict(target_avg_bits=2.0), "paper15": dict(target_avg_bits=1.5),
+                     "paper3": dict(target_avg_bits=3.0), "nonfinite": dict(target_avg_bits=2.0)}.items():
+        s = torch.from_numpy(golden[f"alloc_{name}_scores"])
+        sink = torch.from_numpy(golden[f"alloc_{name}_sink"])
+        got = optimal_scores_to_bits(s.to(DEV), LEVELS, kw["target_avg_bits"], eps, sink.to(DEV), eviction_cost=0.5)
+        np.testing.assert_array_equal(got.cpu().numpy(), golden[f"alloc_{name}_bits"])
+
+
+def test_allocator_batched_rows_with_mixed_budgets():
+    from kvquant.allocator import optimal_scores_to_bits_batched
+    g = torch.Generator().manual_seed(33)
+    H, T = 8, 1024
+    s = torch.exp(1.5 * torch.randn(6, H * T, generator=g))
+    targets = [1.5, 2.0, 3.0, 1.5, 2.0, 3.0]
+    bits, counts, lam = optimal_scores_to_bits_batched(s.to(DEV), LEVELS, targets, EPS, n_sink=4, period=T,
+                                                       eviction_cost=0.5, return_stats=True)
+    for r in range(6):
+        info = {}
+        want = oal.optimal_scores_to_bits(s[r].reshape(H, T), LEVELS, targets[r], EPS, _sink(H, T),
+                                          eviction_cost=0.5, info=info)
+        np.testing.assert_array_equal(bits[r].reshape(H, T).cpu().numpy(), want.numpy())
+        assert lam[r].item() == info["lam"]
+        hist = [(want[:, 4:] == b).sum().item() for b in LEVELS]
+        assert counts[r].cpu().tolist() == hist
+
+
+def test_calibrate_epsilon_matches_oracle():
+    from kvquant.allocator import calibrate_epsilon
+    got = calibrate_epsilon(128, LEVELS, device=DEV, value_quantizer="mse")
+    want = oal.calibrate_epsilon(128, LEVELS, order="canonical")
+    assert set(got) == set(want)
+    for b in LEVELS:
+        assert abs(got[b] - want[b]) <= 1e-6 * max(want[b], 1e-9) + 1e-12
