@@ -191,6 +191,16 @@ int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
                       float* out, float* lse, void* workspace, size_t workspace_bytes,
                       void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Measurement hooks (no counterpart in the reference).  While enabled, every odmkv_decode_attn
+ * call records a pair of HIP events around its main (streaming) kernel on the caller's stream;
+ * odmkv_profile_collect waits for them and returns the kernel durations in milliseconds.
+ * The event pool is created by odmkv_profile_enable and destroyed by odmkv_profile_disable.
+ */
+int odmkv_profile_enable(int max_records);
+int odmkv_profile_collect(float* ms, int capacity, int* n_out);
+int odmkv_profile_disable(void);
+
 #ifdef __cplusplus
 }
 #endif

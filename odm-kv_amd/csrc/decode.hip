@@ -279,6 +279,42 @@ __global__ __launch_bounds__(128) void decode_merge_kernel(DecodeArgs a) {
 
 static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
 
+// ---- measurement hooks: event pairs around the main kernel ----
+#include <vector>
+static std::vector<hipEvent_t> g_prof_events;   // 2 per record
+static int g_prof_used = 0;
+static bool g_prof_on = false;
+
+extern "C" int odmkv_profile_enable(int max_records) {
+    ODMKV_CHECK_ARG(max_records > 0 && max_records <= (1 << 20), "profile_enable: bad record count %d", max_records);
+    if (g_prof_on) odmkv_profile_disable();
+    g_prof_events.resize((size_t)2 * max_records);
+    for (auto& e : g_prof_events) ODMKV_CHECK_HIP(hipEventCreate(&e));
+    g_prof_used = 0;
+    g_prof_on = true;
+    return 0;
+}
+
+extern "C" int odmkv_profile_collect(float* ms, int capacity, int* n_out) {
+    ODMKV_CHECK_ARG(ms && n_out && capacity >= 0, "profile_collect: bad arguments");
+    int n = 0;
+    for (int r = 0; r < g_prof_used && n < capacity; ++r, ++n) {
+        ODMKV_CHECK_HIP(hipEventSynchronize(g_prof_events[2 * r + 1]));
+        ODMKV_CHECK_HIP(hipEventElapsedTime(&ms[n], g_prof_events[2 * r], g_prof_events[2 * r + 1]));
+    }
+    *n_out = n;
+    g_prof_used = 0;
+    return 0;
+}
+
+extern "C" int odmkv_profile_disable(void) {
+    for (auto& e : g_prof_events) hipEventDestroy(e);
+    g_prof_events.clear();
+    g_prof_used = 0;
+    g_prof_on = false;
+    return 0;
+}
+
 extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     size_t q = align_up((size_t)B * Hq * HD * sizeof(float), 256);
     return 2 * q + align_up((size_t)n_items * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
@@ -312,9 +348,15 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     ODMKV_CHECK_LAUNCH("decode_prep_kernel");
     const int GP = group_pad(G);
     if (n_items > 0) {
+        const bool rec = g_prof_on && (size_t)(2 * g_prof_used + 1) < g_prof_events.size();
+        if (rec) ODMKV_CHECK_HIP(hipEventRecord(g_prof_events[2 * g_prof_used], st));
         if (GP == 4) hipLaunchKernelGGL((decode_main_kernel<4>), dim3(n_items), dim3(256), 0, st, a);
         else hipLaunchKernelGGL((decode_main_kernel<8>), dim3(n_items), dim3(256), 0, st, a);
         ODMKV_CHECK_LAUNCH("decode_main_kernel");
+        if (rec) {
+            ODMKV_CHECK_HIP(hipEventRecord(g_prof_events[2 * g_prof_used + 1], st));
+            ++g_prof_used;
+        }
     }
     if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq), dim3(128), 0, st, a);
     else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq), dim3(128), 0, st, a);

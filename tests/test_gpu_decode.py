@@ -83,8 +83,17 @@ def test_decode_special_cases():
     st, ref = _pair(k, v, bits)
     got = st.decode_attention(q[:, :, None].to(DEV), scaling=0.05)
     assert rel_err(got.cpu(), decode_attention_state(q, ref, scaling=0.05)) < ATTN_RTOL
-    # bf16 cache
-    st, ref = _pair(k.bfloat16(), v.bfloat16(), bits, dtype=torch.bfloat16)
+    # bf16 cache.  The reference rounds the dequantised rows to the cache dtype before attention;
+    # for bf16 that rounding alone is 2^-9 per element, above the 1e-3 bar, and the fused kernel
+    # does not reproduce it (it keeps the dequantised values in fp32).  So the oracle state here
+    # holds the same bf16 inputs but materialises in fp32.
+    from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+    kb, vb = k.bfloat16(), v.bfloat16()
+    st = TurboQuantAdaptiveKVCacheState(128, (0, 2, 3, 4, 8, 16), device=DEV, dtype=torch.bfloat16,
+                                        key_quantizer="mse", value_quantizer="mse", seed=42)
+    st.prefill(kb.to(DEV), vb.to(DEV), bits.to(DEV))
+    ref = KVState(128, (0, 2, 3, 4, 8, 16), dtype=torch.float32, seed=42, order="canonical")
+    ref.prefill(kb.float(), vb.float(), bits)
     assert rel_err(st.decode_attention(q.to(DEV)).cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
 
 

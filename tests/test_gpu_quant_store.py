@@ -39,7 +39,7 @@ def test_quantize_rows_bit_exact(bits, dtype):
 @pytest.mark.parametrize("bits", [2, 3, 4, 8])
 def test_container_roundtrip_and_dequantize(bits):
     from kvquant.tq_backend import TurboQuantMSE, _unpack_indices
-    g = torch.Generator().manual_seed(7)
+    g = torch.Generator().manual_seed(1007)      # not the rotation's seed: see calibrate_epsilon's quirk
     x = torch.randn(300, 128, generator=g).half()
     q = TurboQuantMSE(128, bits, device=DEV, dtype=torch.float16, seed=7)
     mq = q.quantize(x.to(DEV))
