@@ -47,7 +47,7 @@ def make_layer(seed, n_kv, n_q, T, dev):
     k[:, :4] *= 8
     v[:, :4] *= 8
     mu = torch.randn(n_q, 64, 128, generator=g, device=dev).mean(dim=1)
-    q = torch.randn(1, n_q, 128, generator=g, device=dev)
+    q = torch.randn(1, n_q, 128, generator=g, device=dev).half().float()
     return k.half(), v.half(), mu, q
 
 

@@ -1,185 +1,408 @@
-// Fused LUT decode attention over the packed mixed-width KV store.
+// Fused LUT decode attention over the packed mixed-width KV store (one query token per sequence).
 //
 // Three launches per call:
-//   1. prep:   q' = scaling * Pi_k q (queries in the rotated basis of the quantised keys) and
-//              qs = scaling * q (for the exact fp16 tokens)
-//   2. main:   one workgroup per work item (a run of tiles of one (sequence, kv-head, level));
-//              each wavefront streams tiles: lane = token for the key side (codes -> centroid
-//              lookup -> dot with the G query heads sharing this kv-head), an online softmax
-//              per query head, then lane = dim for the value side, accumulating
-//              sum_t p_t |v_t| centroid[code] in the rotated basis.  Partial (acc, m, l) per
-//              item go to the workspace.
-//   3. merge:  log-sum-exp merge of a kv-head's items per query head, rotate the quantised
-//              part back (acc . Pi_v), add the exact part, normalise.
-// Packed bytes are read exactly once; evicted tokens do not exist in the store.
+//   1. prep:   q16 = the query rounded to fp16 (what a model in fp16/bf16 hands over anyway);
+//              q' = Pi_k q16 in fp32 (queries in the rotated basis of the quantised keys)
+//   2. main:   one workgroup per work item = a run of 64-token tiles of one (sequence, kv-head,
+//              level).  The packed bytes are read once from HBM; nothing else is.
+//   3. merge:  log-sum-exp merge of a kv-head's items per query head, rotation of the quantised
+//              part back to the model basis (acc . Pi_v), addition of the exact part, normalise.
+//
+// Main kernel, per wavefront and tile (MFMA 4x4x4 f16, 16 blocks of 4 lanes):
+//   keys    lane = token.  Four consecutive codes of the token index an LDS table that returns
+//           their four centroids as fp16; that is operand A (row = token of the quad) of
+//             D[i][j] = sum_k A[lane 4b+i][k] * B[lane 4b+j][k]
+//           and operand B is the query of head j = lane % 4.  After 32 steps over the 128 dims,
+//           lane (quad b, j) holds the logits of tokens 4b..4b+3 for head j.
+//   softmax one head per lane: scale by |k|, running max over the 16 lanes that share the head,
+//           p = exp2(logit - m), times |v|, rounded to fp16: already laid out as operand A
+//           (row = head, k = token of the quad) of the value product.
+//   values  lane = dim.  Values are stored dim-major, so four consecutive codes are four tokens
+//           of this lane's dim: the same LDS table gives operand B, and the A operand of step s
+//           is broadcast from quad s (cbsz/abid).  16 steps accumulate sum_t p_t |v_t| c[code]
+//           for four heads x 128 dims in the rotated basis.
+// The LDS table is replicated over 32 slots (slot = lane % 32) so that lanes never share a bank.
+// All softmax state is kept in base-2 logarithms.
 #include "quant.h"
+
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
 
 #define PSTRIDE 132          // floats per (item, head) partial: 128 acc + m + l + 2 pad
 #define NWAVES 4
+#define LUT_BYTES 65536
+#define LOG2E 1.4426950408889634f
+#define LN2 0.6931471805599453f
 
 struct DecodeArgs {
     odmkv_packed_t s;
     const float* q;
-    int Hq, G;
+    int Hq, G, B;
     float scaling;
     const int32_t* items;
     const int32_t* item_range;
     const float* pi_k;
     const float* pi_v;
     const float* cb;
-    float* qrot;      // [B*Hq, 128]
-    float* qs;        // [B*Hq, 128]
+    float* qrot;      // [B*Hq, 128] Pi_k q16
+    float* qs;        // [B*Hq, 128] q16
+    float inv_s[4];   // 1 / table scale per width
     float* partial;   // [n_items, GP, PSTRIDE]
     float* out;
     float* lse;
 };
 
-__global__ __launch_bounds__(128) void decode_prep_kernel(DecodeArgs a) {
-    __shared__ float qsh[HD];
-    const int bq = blockIdx.x, i = threadIdx.x;
-    const float qi = a.q[(size_t)bq * HD + i];
-    qsh[i] = qi;
-    __syncthreads();
-    const float* row = a.pi_k + (size_t)i * HD;
-    float acc = 0.0f;
-#pragma unroll 8
-    for (int j = 0; j < HD; ++j) acc = __fmaf_rn(row[j], qsh[j], acc);
-    a.qrot[(size_t)bq * HD + i] = acc * a.scaling;
-    a.qs[(size_t)bq * HD + i] = qi * a.scaling;
-}
-
-// online-softmax update shared by both tile kinds: logits -> p (this lane's token), rescale
-template <int GP>
-__device__ static inline void softmax_step(const float (&logit)[GP], float (&m)[GP], float (&l)[GP],
-                                           float (&acc)[GP][2], float (&p)[GP]) {
-#pragma unroll
-    for (int g = 0; g < GP; ++g) {
-        const float mt = wave_max(logit[g]);
-        const float mn = fmaxf(m[g], mt);
-        const float alpha = __expf(m[g] - mn);        // m = -inf on the first tile -> 0
-        p[g] = __expf(logit[g] - mn);                 // padded lanes carry -inf -> 0
-        l[g] = __fmaf_rn(l[g], alpha, p[g]);
-        acc[g][0] *= alpha;
-        acc[g][1] *= alpha;
-        m[g] = mn;
+// ------------------------------------------------------------------------------------------------
+// prep: rotate and scale the queries
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void decode_prep_kernel(DecodeArgs a) {
+    const int bq = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    // the query is consumed at fp16 precision, like the attention it replaces (model dtype)
+    const float q0 = __half2float(__float2half_rn(a.q[(size_t)bq * HD + lane]));
+    const float q1 = __half2float(__float2half_rn(a.q[(size_t)bq * HD + lane + 64]));
+    if (wave == 0) {
+        a.qs[(size_t)bq * HD + lane] = q0;
+        a.qs[(size_t)bq * HD + lane + 64] = q1;
+    }
+#pragma unroll 4
+    for (int i = wave; i < HD; i += 4) {
+        const float* row = a.pi_k + (size_t)i * HD;
+        float v = __fmaf_rn(row[lane], q0, row[lane + 64] * q1);
+        v = wave_sum(v);
+        if (lane == 0) a.qrot[(size_t)bq * HD + i] = v;
     }
 }
 
-template <int W, int GP>
-__device__ static inline void tile_quant(const DecodeArgs& a, int li, int tile, int nvalid, int lane,
-                                         const float* qT, const float* cb, float* pw,
-                                         float (&m)[GP], float (&l)[GP], float (&acc)[GP][2]) {
-    const size_t slot = (size_t)tile * TILE + lane;
-    // ---- keys: lane = token ----
+// ------------------------------------------------------------------------------------------------
+// small helpers
+// ------------------------------------------------------------------------------------------------
+__device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
+
+__device__ static inline h4 as_h4(uint32_t lo, uint32_t hi) {
+    union { uint32_t u[2]; h4 h; } x;
+    x.u[0] = lo; x.u[1] = hi;
+    return x.h;
+}
+
+// two bf16 in a dword -> two fp16 in a dword
+__device__ static inline uint32_t bf16x2_to_f16x2(uint32_t w) {
+    const float lo = __uint_as_float(w << 16), hi = __uint_as_float(w & 0xffff0000u);
+    return half_bits(lo) | (half_bits(hi) << 16);
+}
+
+template <int CTRL>
+__device__ static inline float dpp(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+#define DPP_ROR4 0x124
+#define DPP_ROR8 0x128
+#define DPP_QUAD(i) ((i) | ((i) << 2) | ((i) << 4) | ((i) << 6))
+
+// reduce over the 16 lanes that share lane % 4
+__device__ static inline float head_max(float v) {
+    v = fmaxf(v, dpp<DPP_ROR4>(v));
+    v = fmaxf(v, dpp<DPP_ROR8>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, WAVE));
+    v = fmaxf(v, __shfl_xor(v, 32, WAVE));
+    return v;
+}
+__device__ static inline float head_sum(float v) {
+    v += dpp<DPP_ROR4>(v);
+    v += dpp<DPP_ROR8>(v);
+    v += __shfl_xor(v, 16, WAVE);
+    v += __shfl_xor(v, 32, WAVE);
+    return v;
+}
+
+#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_4x4x4f16((a), (b), (c), 0, 0, 0)
+#define MFMA_BCAST(a, b, c, s) __builtin_amdgcn_mfma_f32_4x4x4f16((a), (b), (c), 4, (s), 0)
+
+// ------------------------------------------------------------------------------------------------
+// LDS tables: code group -> fp16 centroids, replicated over 32 slots
+//   W = 2: index = byte (4 codes) -> 4 halfs (8 bytes),  row = 256 bytes
+//   W = 3: index = 6 bits (2 codes) -> 2 halfs (4 bytes), row = 128 bytes
+//   W = 4: index = byte (2 codes) -> 2 halfs,             row = 128 bytes
+//   W = 8: index = byte (1 code)  -> the half in both halves of a dword, row = 128 bytes
+// ------------------------------------------------------------------------------------------------
+template <int W>
+__device__ static inline void build_lut(uint8_t* lut, const float* __restrict__ cb, int tid) {
+    if constexpr (W == 2) {
+        uint32_t h[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) h[k] = half_bits(cb[(tid >> (2 * k)) & 3]);
+        const uint4 v = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+        uint4* dst = reinterpret_cast<uint4*>(lut + tid * 256);
+#pragma unroll
+        for (int s = 0; s < 16; ++s) dst[s] = v;
+    } else {
+        uint32_t v;
+        bool on = true;
+        if constexpr (W == 3) { on = tid < 64; v = half_bits(cb[tid & 7]) | (half_bits(cb[(tid >> 3) & 7]) << 16); }
+        else if constexpr (W == 4) { v = half_bits(cb[tid & 15]) | (half_bits(cb[tid >> 4]) << 16); }
+        else { v = half_bits(cb[tid]) * 0x10001u; }
+        if (on) {
+            uint4* dst = reinterpret_cast<uint4*>(lut + tid * 128);
+#pragma unroll
+            for (int s = 0; s < 8; ++s) dst[s] = make_uint4(v, v, v, v);
+        }
+    }
+}
+
+// centroids of code group s (codes 4s..4s+3 of the stream held in w), as four halfs
+template <int W>
+__device__ static inline h4 lut4(const uint32_t* w, int s, const uint8_t* lut, uint32_t slot4) {
+    if constexpr (W == 2) {
+        const int bit = 8 * s;
+        const uint32_t idx = (w[bit >> 5] >> (bit & 31)) & 0xffu;
+        const uint2 v = *reinterpret_cast<const uint2*>(lut + (idx << 8) + 2 * slot4);
+        return as_h4(v.x, v.y);
+    } else if constexpr (W == 4) {
+        const int bit = 16 * s;
+        const uint32_t x = w[bit >> 5] >> (bit & 31);
+        const uint32_t lo = *reinterpret_cast<const uint32_t*>(lut + ((x & 0xffu) << 7) + slot4);
+        const uint32_t hi = *reinterpret_cast<const uint32_t*>(lut + (((x >> 8) & 0xffu) << 7) + slot4);
+        return as_h4(lo, hi);
+    } else if constexpr (W == 8) {
+        const uint32_t x = w[s];
+        const uint32_t t0 = *reinterpret_cast<const uint32_t*>(lut + ((x & 0xffu) << 7) + slot4);
+        const uint32_t t1 = *reinterpret_cast<const uint32_t*>(lut + (((x >> 8) & 0xffu) << 7) + slot4);
+        const uint32_t t2 = *reinterpret_cast<const uint32_t*>(lut + (((x >> 16) & 0xffu) << 7) + slot4);
+        const uint32_t t3 = *reinterpret_cast<const uint32_t*>(lut + ((x >> 24) << 7) + slot4);
+        return as_h4((t0 & 0xffffu) | (t1 & 0xffff0000u), (t2 & 0xffffu) | (t3 & 0xffff0000u));
+    } else {
+        const int bit = 12 * s, k = bit >> 5, sh = bit & 31;
+        uint32_t x = w[k] >> sh;
+        if (sh + 12 > 32) x |= w[k + 1] << (32 - sh);
+        const uint32_t lo = *reinterpret_cast<const uint32_t*>(lut + ((x & 63u) << 7) + slot4);
+        const uint32_t hi = *reinterpret_cast<const uint32_t*>(lut + (((x >> 6) & 63u) << 7) + slot4);
+        return as_h4(lo, hi);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// per-wavefront running state: one softmax head per lane and pass, four heads x two dims per lane
+// ------------------------------------------------------------------------------------------------
+template <int NP>
+struct WaveState {
+    float m[NP], l[NP];
+    f4 acc[NP][2];
+};
+
+// logits of this lane's head for the quad's four tokens -> p (fp16, times |v|), state update
+template <int NP>
+__device__ static inline h4 softmax_step(WaveState<NP>& st, int p, const f4& logit, const f4& vn) {
+    float mx = fmaxf(fmaxf(logit[0], logit[1]), fmaxf(logit[2], logit[3]));
+    mx = head_max(mx);
+    const float mn = fmaxf(st.m[p], mx);
+    const float alpha = __builtin_amdgcn_exp2f(st.m[p] - mn);     // first tile: exp2(-inf) = 0
+    float pr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pr[i] = __builtin_amdgcn_exp2f(logit[i] - mn);   // padded tokens: -inf -> 0
+    st.l[p] = __fmaf_rn(st.l[p], alpha, (pr[0] + pr[1]) + (pr[2] + pr[3]));
+    st.m[p] = mn;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {         // the maximum moved for some head
+        const float a0 = dpp<DPP_QUAD(0)>(alpha), a1 = dpp<DPP_QUAD(1)>(alpha);
+        const float a2 = dpp<DPP_QUAD(2)>(alpha), a3 = dpp<DPP_QUAD(3)>(alpha);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            st.acc[p][h][0] *= a0; st.acc[p][h][1] *= a1; st.acc[p][h][2] *= a2; st.acc[p][h][3] *= a3;
+        }
+    }
+    h4 pa;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pa[i] = (_Float16)(pr[i] * vn[i]);
+    return pa;
+}
+
+// ---- quantised tiles -----------------------------------------------------------------------------
+template <int W>
+struct TileData {
     uint32_t kw[4 * W];
+    uint32_t vw[2][2 * W];
+    f4 kn, vn;
+};
+
+template <int W>
+__device__ static inline void load_tile(TileData<W>& t, const DecodeArgs& a, int li, int tile, int lane) {
     const uint8_t* ksrc = a.s.kcodes[li] + (size_t)tile * (TILE * 16 * W);
 #pragma unroll
     for (int c = 0; c < W; ++c) {
         const uint4 v = *reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 16);
-        kw[4 * c] = v.x; kw[4 * c + 1] = v.y; kw[4 * c + 2] = v.z; kw[4 * c + 3] = v.w;
+        t.kw[4 * c] = v.x; t.kw[4 * c + 1] = v.y; t.kw[4 * c + 2] = v.z; t.kw[4 * c + 3] = v.w;
     }
-    const float kn = a.s.knorm[li][slot];
-    const float vn = a.s.vnorm[li][slot];
-    // ---- values: lane = dim (lane, lane + 64), issued early so the loads overlap the key math ----
-    uint32_t vw[2][2 * W];
     const uint8_t* vsrc = a.s.vcodes[li] + (size_t)tile * (HD * 8 * W);
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int h = 0; h < 2; ++h) {
+        const int j = lane + 64 * h;
+        if constexpr (W == 3) {
 #pragma unroll
-        for (int k = 0; k < 2 * W; ++k)
-            vw[h][k] = *reinterpret_cast<const uint32_t*>(vsrc + v_word_offset<W>(k, lane + 64 * h));
-
-    float dot[GP];
+            for (int u = 0; u < 3; ++u) {
+                const uint2 v = *reinterpret_cast<const uint2*>(vsrc + ((size_t)u * HD + j) * 8);
+                t.vw[h][2 * u] = v.x; t.vw[h][2 * u + 1] = v.y;
+            }
+        } else {
 #pragma unroll
-    for (int g = 0; g < GP; ++g) dot[g] = 0.0f;
-#pragma unroll
-    for (int i = 0; i < HD; ++i) {
-        const float val = cb[get_code<W>(kw, i)];
-#pragma unroll
-        for (int g = 0; g < GP; ++g) dot[g] = __fmaf_rn(val, qT[i * GP + g], dot[g]);
-    }
-    float logit[GP], p[GP];
-#pragma unroll
-    for (int g = 0; g < GP; ++g) logit[g] = lane < nvalid ? dot[g] * kn : -INFINITY;
-    softmax_step<GP>(logit, m, l, acc, p);
-#pragma unroll
-    for (int g = 0; g < GP; ++g) pw[lane * GP + g] = lane < nvalid ? p[g] * vn : 0.0f;
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int t = 0; t < TILE; ++t) {
-        const float v0 = cb[get_code<W>(vw[0], t)];
-        const float v1 = cb[get_code<W>(vw[1], t)];
-#pragma unroll
-        for (int g = 0; g < GP; ++g) {
-            const float pg = pw[t * GP + g];
-            acc[g][0] = __fmaf_rn(pg, v0, acc[g][0]);
-            acc[g][1] = __fmaf_rn(pg, v1, acc[g][1]);
-        }
-    }
-    __builtin_amdgcn_wave_barrier();
-}
-
-__device__ static inline float half_bits_to_f32(uint16_t v, int bf16) {
-    return bf16 ? __uint_as_float(((uint32_t)v) << 16) : __half2float(__ushort_as_half(v));
-}
-
-template <int GP>
-__device__ static inline void tile_exact(const DecodeArgs& a, int tile, int nvalid, int lane,
-                                         const float* qT, float* pw,
-                                         float (&m)[GP], float (&l)[GP], float (&acc)[GP][2]) {
-    const int bf = a.s.exact_dtype == ODMKV_BF16;
-    const uint16_t* ksrc = a.s.kexact + (size_t)tile * TILE * HD;
-    const uint16_t* vsrc = a.s.vexact + (size_t)tile * TILE * HD;
-    float dot[GP];
-#pragma unroll
-    for (int g = 0; g < GP; ++g) dot[g] = 0.0f;
-#pragma unroll
-    for (int c = 0; c < 16; ++c) {
-        const uint4 v = *reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 8);
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float val = half_bits_to_f32((uint16_t)((w[e >> 1] >> (16 * (e & 1))) & 0xffffu), bf);
-#pragma unroll
-            for (int g = 0; g < GP; ++g) dot[g] = __fmaf_rn(val, qT[(8 * c + e) * GP + g], dot[g]);
-        }
-    }
-    float logit[GP], p[GP];
-#pragma unroll
-    for (int g = 0; g < GP; ++g) logit[g] = lane < nvalid ? dot[g] : -INFINITY;
-    softmax_step<GP>(logit, m, l, acc, p);
-#pragma unroll
-    for (int g = 0; g < GP; ++g) pw[lane * GP + g] = lane < nvalid ? p[g] : 0.0f;
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll 4
-    for (int tg = 0; tg < TILE / 4; ++tg) {
-        const uint2 r0 = *reinterpret_cast<const uint2*>(vsrc + ((size_t)tg * HD + lane) * 4);
-        const uint2 r1 = *reinterpret_cast<const uint2*>(vsrc + ((size_t)tg * HD + lane + 64) * 4);
-        const uint32_t w0[2] = {r0.x, r0.y}, w1[2] = {r1.x, r1.y};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            // padded tokens hold stale bytes: their p is 0, but 0 * inf would poison the sum
-            const bool live = 4 * tg + e < nvalid;
-            const float v0 = live ? half_bits_to_f32((uint16_t)((w0[e >> 1] >> (16 * (e & 1))) & 0xffffu), bf) : 0.0f;
-            const float v1 = live ? half_bits_to_f32((uint16_t)((w1[e >> 1] >> (16 * (e & 1))) & 0xffffu), bf) : 0.0f;
-#pragma unroll
-            for (int g = 0; g < GP; ++g) {
-                const float pg = pw[(4 * tg + e) * GP + g];
-                acc[g][0] = __fmaf_rn(pg, v0, acc[g][0]);
-                acc[g][1] = __fmaf_rn(pg, v1, acc[g][1]);
+            for (int u = 0; u < W / 2; ++u) {
+                const uint4 v = *reinterpret_cast<const uint4*>(vsrc + ((size_t)u * HD + j) * 16);
+                t.vw[h][4 * u] = v.x; t.vw[h][4 * u + 1] = v.y; t.vw[h][4 * u + 2] = v.z; t.vw[h][4 * u + 3] = v.w;
             }
         }
     }
-    __builtin_amdgcn_wave_barrier();
+    const size_t quad = (size_t)tile * TILE + (lane & ~3);
+    t.kn = *reinterpret_cast<const f4*>(a.s.knorm[li] + quad);
+    t.vn = *reinterpret_cast<const f4*>(a.s.vnorm[li] + quad);
 }
 
-template <int GP>
-__global__ __launch_bounds__(256) void decode_main_kernel(DecodeArgs a) {
-    __shared__ float qT[HD * GP];                 // [dim][head]
-    __shared__ float cb[256];
-    __shared__ float pw_all[NWAVES][TILE * GP];   // per-wave p * |v|
-    __shared__ float wm[NWAVES][GP], wl[NWAVES][GP];
-    __shared__ float wacc[NWAVES][GP][HD];
+#define PV_STEP(s)                                                                              \
+    {                                                                                           \
+        const h4 b0 = lut4<W>(t.vw[0], (s), lut, slot4), b1 = lut4<W>(t.vw[1], (s), lut, slot4); \
+        _Pragma("unroll") for (int p = 0; p < NP; ++p) {                                        \
+            st.acc[p][0] = MFMA_BCAST(pa[p], b0, st.acc[p][0], (s));                            \
+            st.acc[p][1] = MFMA_BCAST(pa[p], b1, st.acc[p][1], (s));                            \
+        }                                                                                       \
+    }
+
+template <int W, int NP>
+__device__ static inline void compute_tile(const TileData<W>& t, int nvalid, int lane, const uint8_t* lut,
+                                           uint32_t slot4, const h4* qr, const h4* ql, float ksc, float vsc,
+                                           WaveState<NP>& st) {
+    // ---- keys ----
+    f4 dk[NP][4];
+#pragma unroll
+    for (int p = 0; p < NP; ++p)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) dk[p][c] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 32; ++s) {
+        const h4 kv = lut4<W>(t.kw, s, lut, slot4);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            dk[p][s & 3] = MFMA(kv, qr[p * 32 + s], dk[p][s & 3]);
+            dk[p][(s + 2) & 3] = MFMA(kv, ql[p * 32 + s], dk[p][(s + 2) & 3]);    // low half of the query
+        }
+    }
+    const int tok0 = lane & ~3;
+    h4 pa[NP];
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const f4 d = (dk[p][0] + dk[p][1]) + (dk[p][2] + dk[p][3]);
+        f4 logit;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) logit[i] = tok0 + i < nvalid ? d[i] * (t.kn[i] * ksc) : -INFINITY;
+        f4 vn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vn[i] = tok0 + i < nvalid ? t.vn[i] * vsc : 0.0f;
+        pa[p] = softmax_step<NP>(st, p, logit, vn);
+    }
+    // ---- values ----
+    PV_STEP(0) PV_STEP(1) PV_STEP(2) PV_STEP(3) PV_STEP(4) PV_STEP(5) PV_STEP(6) PV_STEP(7)
+    PV_STEP(8) PV_STEP(9) PV_STEP(10) PV_STEP(11) PV_STEP(12) PV_STEP(13) PV_STEP(14) PV_STEP(15)
+}
+
+template <int W, int NP>
+__device__ static inline void run_quant_level(const DecodeArgs& a, int li, int tile0, int ntiles, int seg_first,
+                                              int count, int wave, int lane, const uint8_t* lut, const h4* qr,
+                                              const h4* ql, WaveState<NP>& st) {
+    const uint32_t slot4 = (lane & 31) * 4;
+    const float vsc = a.inv_s[li], ksc = a.inv_s[li] * a.scaling * LOG2E;
+    if constexpr (W == 8) {
+        // wide rows: no double buffering, the registers go to the query
+        TileData<W> cur;
+        for (int tt = wave; tt < ntiles; tt += NWAVES) {
+            const int nvalid = min(count - (tile0 + tt - seg_first) * TILE, TILE);
+            if (nvalid <= 0) break;
+            load_tile<W>(cur, a, li, tile0 + tt, lane);
+            compute_tile<W, NP>(cur, nvalid, lane, lut, slot4, qr, ql, ksc, vsc, st);
+        }
+        return;
+    }
+    TileData<W> cur, nxt;
+    int tt = wave;
+    if (tt >= ntiles) return;
+    int nvalid = min(count - (tile0 + tt - seg_first) * TILE, TILE);
+    if (nvalid <= 0) return;
+    load_tile<W>(cur, a, li, tile0 + tt, lane);
+    while (true) {
+        const int tn = tt + NWAVES;
+        const int nvalid_n = tn < ntiles ? min(count - (tile0 + tn - seg_first) * TILE, TILE) : 0;
+        if (nvalid_n > 0) load_tile<W>(nxt, a, li, tile0 + tn, lane);     // in flight while this tile is computed
+        compute_tile<W, NP>(cur, nvalid, lane, lut, slot4, qr, ql, ksc, vsc, st);
+        if (nvalid_n <= 0) break;
+        cur = nxt;
+        tt = tn;
+        nvalid = nvalid_n;
+    }
+}
+
+// ---- exact (fp16 / bf16) tiles ---------------------------------------------------------------------
+#define PV_EXACT_STEP(s)                                                                         \
+    {                                                                                            \
+        uint2 r0 = *reinterpret_cast<const uint2*>(vsrc + ((size_t)(s) * HD + lane) * 4);        \
+        uint2 r1 = *reinterpret_cast<const uint2*>(vsrc + ((size_t)(s) * HD + lane + 64) * 4);   \
+        if (bf) { r0.x = bf16x2_to_f16x2(r0.x); r0.y = bf16x2_to_f16x2(r0.y);                    \
+                  r1.x = bf16x2_to_f16x2(r1.x); r1.y = bf16x2_to_f16x2(r1.y); }                  \
+        const h4 b0 = as_h4(r0.x, r0.y), b1 = as_h4(r1.x, r1.y);                                 \
+        _Pragma("unroll") for (int p = 0; p < NP; ++p) {                                         \
+            st.acc[p][0] = MFMA_BCAST(pa[p], b0, st.acc[p][0], (s));                             \
+            st.acc[p][1] = MFMA_BCAST(pa[p], b1, st.acc[p][1], (s));                             \
+        }                                                                                        \
+    }
+
+template <int NP>
+__device__ static inline void run_exact_level(const DecodeArgs& a, int tile0, int ntiles, int seg_first, int count,
+                                              int wave, int lane, const h4* qr, WaveState<NP>& st) {
+    const bool bf = a.s.exact_dtype == ODMKV_BF16;
+    const float esc = a.scaling * LOG2E;
+    for (int tt = wave; tt < ntiles; tt += NWAVES) {
+        const int tile = tile0 + tt;
+        const int nvalid = min(count - (tile - seg_first) * TILE, TILE);
+        if (nvalid <= 0) break;
+        const uint16_t* ksrc = a.s.kexact + (size_t)tile * TILE * HD;
+        const uint16_t* vsrc = a.s.vexact + (size_t)tile * TILE * HD;
+        f4 dk[NP][4];
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) dk[p][c] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            uint4 v = *reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 8);
+            if (bf) { v.x = bf16x2_to_f16x2(v.x); v.y = bf16x2_to_f16x2(v.y); v.z = bf16x2_to_f16x2(v.z); v.w = bf16x2_to_f16x2(v.w); }
+            const h4 k0 = as_h4(v.x, v.y), k1 = as_h4(v.z, v.w);
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+                dk[p][(2 * c) & 3] = MFMA(k0, qr[p * 32 + 2 * c], dk[p][(2 * c) & 3]);
+                dk[p][(2 * c + 1) & 3] = MFMA(k1, qr[p * 32 + 2 * c + 1], dk[p][(2 * c + 1) & 3]);
+            }
+        }
+        const int tok0 = lane & ~3;
+        h4 pa[NP];
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const f4 d = (dk[p][0] + dk[p][1]) + (dk[p][2] + dk[p][3]);
+            f4 logit, vn;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                logit[i] = tok0 + i < nvalid ? d[i] * esc : -INFINITY;
+                vn[i] = tok0 + i < nvalid ? 1.0f : 0.0f;
+            }
+            pa[p] = softmax_step<NP>(st, p, logit, vn);
+        }
+        PV_EXACT_STEP(0) PV_EXACT_STEP(1) PV_EXACT_STEP(2) PV_EXACT_STEP(3)
+        PV_EXACT_STEP(4) PV_EXACT_STEP(5) PV_EXACT_STEP(6) PV_EXACT_STEP(7)
+        PV_EXACT_STEP(8) PV_EXACT_STEP(9) PV_EXACT_STEP(10) PV_EXACT_STEP(11)
+        PV_EXACT_STEP(12) PV_EXACT_STEP(13) PV_EXACT_STEP(14) PV_EXACT_STEP(15)
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// main kernel: NP passes of four query heads (GQA groups up to 4 * NP)
+// ------------------------------------------------------------------------------------------------
+template <int NP>
+__global__ __launch_bounds__(256, 2) void decode_main_kernel(DecodeArgs a) {
+    __shared__ __align__(16) uint8_t lut[LUT_BYTES];     // centroid table; reused to combine the wavefronts
+    __shared__ float wm[NWAVES][4 * NP], wl[NWAVES][4 * NP];
+    __shared__ __align__(16) float qsh[4 * NP * HD];
 
     const int item = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int bh = a.items[4 * item + 0];
@@ -188,45 +411,61 @@ __global__ __launch_bounds__(256) void decode_main_kernel(DecodeArgs a) {
     const int ntiles = a.items[4 * item + 3];
     const int b = bh / a.s.Hkv, hkv = bh % a.s.Hkv;
 
-    // queries of this kv-head's group, transposed to [dim][head]; unused heads are zero
+    // the group's queries go through LDS (one coalesced read), then every lane keeps its own
+    // head (lane % 4 per pass) in registers as fp16 high and low halves; heads beyond the group are 0
     const float* qsrc = (li == 4 ? a.qs : a.qrot) + ((size_t)b * a.Hq + (size_t)hkv * a.G) * HD;
-    for (int e = tid; e < HD * GP; e += 256) {
-        const int i = e / GP, g = e % GP;
-        qT[e] = g < a.G ? qsrc[(size_t)g * HD + i] : 0.0f;
-    }
-    if (li < 4) {
-        const int n = 1 << width_of(li);
-        for (int e = tid; e < n; e += 256) cb[e] = a.cb[codebook_offset(li) + e];
+    for (int e = tid; e < 4 * NP * HD; e += 256) qsh[e] = (e >> 7) < a.G ? qsrc[e] : 0.0f;
+    switch (li) {
+        case 0: build_lut<2>(lut, a.cb + codebook_offset(0), tid); break;
+        case 1: build_lut<3>(lut, a.cb + codebook_offset(1), tid); break;
+        case 2: build_lut<4>(lut, a.cb + codebook_offset(2), tid); break;
+        case 3: build_lut<8>(lut, a.cb + codebook_offset(3), tid); break;
+        default: break;
     }
     __syncthreads();
-
-    float m[GP], l[GP], acc[GP][2];
+    h4 qr[NP * 32], ql[NP * 32];
 #pragma unroll
-    for (int g = 0; g < GP; ++g) { m[g] = -INFINITY; l[g] = 0.0f; acc[g][0] = 0.0f; acc[g][1] = 0.0f; }
-
-    const int seg_first = a.s.seg_tile[li][bh];
-    const int count = a.s.seg_count[li][bh];
-    float* pw = pw_all[wave];
-    for (int tt = wave; tt < ntiles; tt += NWAVES) {
-        const int tile = tile0 + tt;
-        const int nvalid = min(count - (tile - seg_first) * TILE, TILE);
-        if (nvalid <= 0) break;                                  // tiles are filled front to back
-        switch (li) {
-            case 0: tile_quant<2, GP>(a, 0, tile, nvalid, lane, qT, cb, pw, m, l, acc); break;
-            case 1: tile_quant<3, GP>(a, 1, tile, nvalid, lane, qT, cb, pw, m, l, acc); break;
-            case 2: tile_quant<4, GP>(a, 2, tile, nvalid, lane, qT, cb, pw, m, l, acc); break;
-            case 3: tile_quant<8, GP>(a, 3, tile, nvalid, lane, qT, cb, pw, m, l, acc); break;
-            default: tile_exact<GP>(a, tile, nvalid, lane, qT, pw, m, l, acc); break;
+    for (int p = 0; p < NP; ++p) {
+        const f4* src = reinterpret_cast<const f4*>(qsh + (4 * p + (lane & 3)) * HD);
+#pragma unroll
+        for (int s = 0; s < 32; ++s) {
+            const f4 v = src[s];
+            const h4 hi = (h4){(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+            qr[p * 32 + s] = hi;
+            ql[p * 32 + s] = (h4){(_Float16)(v[0] - (float)hi[0]), (_Float16)(v[1] - (float)hi[1]),
+                                  (_Float16)(v[2] - (float)hi[2]), (_Float16)(v[3] - (float)hi[3])};
         }
     }
 
-    // ---- combine the four wavefronts ----
+    WaveState<NP> st;
 #pragma unroll
-    for (int g = 0; g < GP; ++g) {
-        const float ls = wave_sum(l[g]);
-        if (lane == 0) { wm[wave][g] = m[g]; wl[wave][g] = ls; }
-        wacc[wave][g][lane] = acc[g][0];
-        wacc[wave][g][lane + 64] = acc[g][1];
+    for (int p = 0; p < NP; ++p) {
+        st.m[p] = -INFINITY; st.l[p] = 0.0f;
+        st.acc[p][0] = (f4){0.f, 0.f, 0.f, 0.f}; st.acc[p][1] = (f4){0.f, 0.f, 0.f, 0.f};
+    }
+    const int seg_first = a.s.seg_tile[li][bh];
+    const int count = a.s.seg_count[li][bh];
+    switch (li) {
+        case 0: run_quant_level<2, NP>(a, 0, tile0, ntiles, seg_first, count, wave, lane, lut, qr, ql, st); break;
+        case 1: run_quant_level<3, NP>(a, 1, tile0, ntiles, seg_first, count, wave, lane, lut, qr, ql, st); break;
+        case 2: run_quant_level<4, NP>(a, 2, tile0, ntiles, seg_first, count, wave, lane, lut, qr, ql, st); break;
+        case 3: run_quant_level<8, NP>(a, 3, tile0, ntiles, seg_first, count, wave, lane, lut, qr, ql, st); break;
+        default: run_exact_level<NP>(a, tile0, ntiles, seg_first, count, wave, lane, qr, st); break;
+    }
+
+    // ---- combine the four wavefronts (the table is no longer needed) ----
+    __syncthreads();
+    float* wacc = reinterpret_cast<float*>(lut);          // [NWAVES][4*NP][128]
+    constexpr int GP = 4 * NP;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const float ls = head_sum(st.l[p]);
+        if (lane < 4) { wm[wave][4 * p + lane] = st.m[p]; wl[wave][4 * p + lane] = ls; }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            wacc[((wave * GP) + 4 * p + i) * HD + lane] = st.acc[p][0][i];
+            wacc[((wave * GP) + 4 * p + i) * HD + lane + 64] = st.acc[p][1][i];
+        }
     }
     __syncthreads();
     float* dst = a.partial + (size_t)item * GP * PSTRIDE;
@@ -239,8 +478,8 @@ __global__ __launch_bounds__(256) void decode_main_kernel(DecodeArgs a) {
         if (M > -INFINITY) {
 #pragma unroll
             for (int w = 0; w < NWAVES; ++w) {
-                const float f = __expf(wm[w][g] - M);
-                s = __fmaf_rn(wacc[w][g][j], f, s);
+                const float f = __builtin_amdgcn_exp2f(wm[w][g] - M);
+                s = __fmaf_rn(wacc[((w * GP) + g) * HD + j], f, s);
                 L = __fmaf_rn(wl[w][g], f, L);
             }
         }
@@ -249,41 +488,99 @@ __global__ __launch_bounds__(256) void decode_main_kernel(DecodeArgs a) {
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// merge: one workgroup per query head
+// ------------------------------------------------------------------------------------------------
+#define MERGE_THREADS 512
+#define MERGE_SLICES (MERGE_THREADS / HD)
+#define MERGE_MAX_ITEMS 1024
+
 template <int GP>
-__global__ __launch_bounds__(128) void decode_merge_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs a) {
+    __shared__ float wts[MERGE_MAX_ITEMS];           // exp2(m_item - M); the sign bit marks exact items
+    __shared__ float red[MERGE_THREADS / 64];
+    __shared__ float part[2][MERGE_SLICES][HD];      // [rotated | exact][slice][dim]
     __shared__ float rot[HD];
-    const int bq = blockIdx.x, j = threadIdx.x;
+    __shared__ float Lsh;
+    const int bq = blockIdx.x, tid = threadIdx.x, j = tid & (HD - 1), slice = tid >> 7;
     const int b = bq / a.Hq, hq = bq % a.Hq;
     const int bh = b * a.s.Hkv + hq / a.G, g = hq % a.G;
-    const int i0 = a.item_range[bh], i1 = a.item_range[bh + 1];
-    float M = -INFINITY;
-    for (int it = i0; it < i1; ++it) M = fmaxf(M, a.partial[((size_t)it * GP + g) * PSTRIDE + HD]);
-    float L = 0.0f, arot = 0.0f, aex = 0.0f;
-    if (M > -INFINITY) {
-        for (int it = i0; it < i1; ++it) {
-            const float* p = a.partial + ((size_t)it * GP + g) * PSTRIDE;
-            const float f = __expf(p[HD] - M);
-            L = __fmaf_rn(p[HD + 1], f, L);
-            if (a.items[4 * it + 1] == 4) aex = __fmaf_rn(p[j], f, aex);
-            else arot = __fmaf_rn(p[j], f, arot);
-        }
-    }
-    rot[j] = arot;
+    const int i0 = a.item_range[bh], n = min(a.item_range[bh + 1] - i0, MERGE_MAX_ITEMS);
+    // maximum over the items
+    float mx = -INFINITY;
+    for (int it = tid; it < n; it += MERGE_THREADS)
+        mx = fmaxf(mx, a.partial[((size_t)(i0 + it) * GP + g) * PSTRIDE + HD]);
+    mx = wave_max(mx);
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
     __syncthreads();
-    float o = aex;
-#pragma unroll 8
-    for (int i = 0; i < HD; ++i) o = __fmaf_rn(rot[i], a.pi_v[(size_t)i * HD + j], o);
-    a.out[(size_t)bq * HD + j] = L > 0.0f ? o / L : 0.0f;
-    if (a.lse && j == 0) a.lse[bq] = L > 0.0f ? M + __logf(L) : -INFINITY;
+    float M = red[0];
+#pragma unroll
+    for (int w = 1; w < MERGE_THREADS / 64; ++w) M = fmaxf(M, red[w]);
+    __syncthreads();
+    // weights and the normaliser
+    float lpart = 0.0f;
+    for (int it = tid; it < n; it += MERGE_THREADS) {
+        const float* p = a.partial + ((size_t)(i0 + it) * GP + g) * PSTRIDE;
+        const float f = M > -INFINITY ? __builtin_amdgcn_exp2f(p[HD] - M) : 0.0f;
+        lpart = __fmaf_rn(p[HD + 1], f, lpart);
+        wts[it] = a.items[4 * (i0 + it) + 1] == 4 ? -f : f;
+    }
+    lpart = wave_sum(lpart);
+    if ((tid & 63) == 0) red[tid >> 6] = lpart;
+    __syncthreads();
+    if (tid == 0) {
+        float L = 0.0f;
+        for (int w = 0; w < MERGE_THREADS / 64; ++w) L += red[w];
+        Lsh = L;
+    }
+    float arot = 0.0f, aex = 0.0f;
+#pragma unroll 4
+    for (int it = slice; it < n; it += MERGE_SLICES) {
+        const float w = wts[it];
+        const float v = a.partial[((size_t)(i0 + it) * GP + g) * PSTRIDE + j];
+        if (__float_as_uint(w) >> 31) aex = __fmaf_rn(v, -w, aex);
+        else arot = __fmaf_rn(v, w, arot);
+    }
+    part[0][slice][j] = arot;
+    part[1][slice][j] = aex;
+    __syncthreads();
+    if (tid < HD) {
+        float r = 0.0f;
+#pragma unroll
+        for (int s = 0; s < MERGE_SLICES; ++s) r += part[0][s][tid];
+        rot[tid] = r;
+    }
+    __syncthreads();
+    // rotate the quantised part back: out_j = sum_i rot_i Pi_v[i][j]; the slices split the i range
+    float o = 0.0f;
+    for (int i = slice * (HD / MERGE_SLICES); i < (slice + 1) * (HD / MERGE_SLICES); ++i)
+        o = __fmaf_rn(rot[i], a.pi_v[(size_t)i * HD + j], o);
+    __syncthreads();
+    part[0][slice][j] = o;
+    __syncthreads();
+    if (tid < HD) {
+        float tot = 0.0f;
+#pragma unroll
+        for (int s = 0; s < MERGE_SLICES; ++s) tot += part[0][s][tid] + part[1][s][tid];
+        const float L = Lsh;
+        a.out[(size_t)bq * HD + tid] = L > 0.0f ? tot / L : 0.0f;
+        if (a.lse && tid == 0) a.lse[bq] = L > 0.0f ? (M + __log2f(L)) * LN2 : -INFINITY;
+    }
 }
-
-static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
 
 // ---- measurement hooks: event pairs around the main kernel ----
 #include <vector>
 static std::vector<hipEvent_t> g_prof_events;   // 2 per record
 static int g_prof_used = 0;
 static bool g_prof_on = false;
+
+extern "C" int odmkv_profile_disable(void) {
+    for (auto& e : g_prof_events) (void)hipEventDestroy(e);
+    g_prof_events.clear();
+    g_prof_used = 0;
+    g_prof_on = false;
+    return 0;
+}
 
 extern "C" int odmkv_profile_enable(int max_records) {
     ODMKV_CHECK_ARG(max_records > 0 && max_records <= (1 << 20), "profile_enable: bad record count %d", max_records);
@@ -307,13 +604,7 @@ extern "C" int odmkv_profile_collect(float* ms, int capacity, int* n_out) {
     return 0;
 }
 
-extern "C" int odmkv_profile_disable(void) {
-    for (auto& e : g_prof_events) hipEventDestroy(e);
-    g_prof_events.clear();
-    g_prof_used = 0;
-    g_prof_on = false;
-    return 0;
-}
+static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
 
 extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     size_t q = align_up((size_t)B * Hq * HD * sizeof(float), 256);
@@ -324,8 +615,10 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
                                  const odmkv_packed_t* store,
                                  const int32_t* items, int n_items, const int32_t* item_range,
                                  const float* pi_k, const float* pi_v, const float* codebooks,
+                                 const float* inv_scales,
                                  float* out, float* lse, void* workspace, size_t workspace_bytes,
                                  void* stream) {
+    ODMKV_CHECK_ARG(inv_scales != nullptr, "decode_attn: null table scales");
     ODMKV_CHECK_ARG(q && store && item_range && pi_k && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
     ODMKV_CHECK_ARG(n_items == 0 || items, "decode_attn: null work list");
     ODMKV_CHECK_ARG(B > 0 && Hq > 0 && store->B == B && store->Hkv > 0 && Hq % store->Hkv == 0,
@@ -336,30 +629,31 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     ODMKV_CHECK_ARG(workspace_bytes >= odmkv_decode_workspace_bytes(B, Hq, n_items), "decode_attn: workspace too small");
     hipStream_t st = (hipStream_t)stream;
     DecodeArgs a;
-    a.s = *store; a.q = q; a.Hq = Hq; a.G = G; a.scaling = scaling;
+    a.s = *store; a.q = q; a.Hq = Hq; a.G = G; a.B = B; a.scaling = scaling;
     a.items = items; a.item_range = item_range;
     a.pi_k = pi_k; a.pi_v = pi_v; a.cb = codebooks;
+    for (int w = 0; w < 4; ++w) a.inv_s[w] = inv_scales[w];
     const size_t qbytes = align_up((size_t)B * Hq * HD * sizeof(float), 256);
     a.qrot = (float*)workspace;
     a.qs = (float*)((char*)workspace + qbytes);
     a.partial = (float*)((char*)workspace + 2 * qbytes);
     a.out = out; a.lse = lse;
-    hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(128), 0, st, a);
+    hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(256), 0, st, a);
     ODMKV_CHECK_LAUNCH("decode_prep_kernel");
     const int GP = group_pad(G);
     if (n_items > 0) {
         const bool rec = g_prof_on && (size_t)(2 * g_prof_used + 1) < g_prof_events.size();
         if (rec) ODMKV_CHECK_HIP(hipEventRecord(g_prof_events[2 * g_prof_used], st));
-        if (GP == 4) hipLaunchKernelGGL((decode_main_kernel<4>), dim3(n_items), dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((decode_main_kernel<8>), dim3(n_items), dim3(256), 0, st, a);
+        if (GP == 4) hipLaunchKernelGGL((decode_main_kernel<1>), dim3(n_items), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((decode_main_kernel<2>), dim3(n_items), dim3(256), 0, st, a);
         ODMKV_CHECK_LAUNCH("decode_main_kernel");
         if (rec) {
             ODMKV_CHECK_HIP(hipEventRecord(g_prof_events[2 * g_prof_used + 1], st));
             ++g_prof_used;
         }
     }
-    if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq), dim3(128), 0, st, a);
-    else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq), dim3(128), 0, st, a);
+    if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);
+    else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);
     ODMKV_CHECK_LAUNCH("decode_merge_kernel");
     return 0;
 }

@@ -24,7 +24,7 @@ import torch
 
 from . import _lib
 from ._lib import lib, Packed, TILE, HEAD_DIM, WIDTHS
-from .tq_backend import (cached_rotation, codebook_table, normalize_key_quantizer,
+from .tq_backend import (cached_rotation, codebook_table, decode_tables, normalize_key_quantizer,
                          normalize_value_quantizer)
 
 _LEVEL_INDEX = {2: 0, 3: 1, 4: 2, 8: 3, 16: 4}
@@ -76,6 +76,8 @@ class TurboQuantAdaptiveKVCacheState:
         self.pi_k = cached_rotation(head_dim, self.device, seed)
         self.pi_v = cached_rotation(head_dim, self.device, seed + 2000)
         self.codebooks = codebook_table(head_dim, self.device)
+        self._decode_cb, inv = decode_tables(head_dim, self.device)
+        self._decode_inv = (C.c_float * 4)(*inv)
         self._exact_torch_dtype = torch.bfloat16 if dtype == torch.bfloat16 else torch.float16
         self._reset()
 
@@ -392,7 +394,10 @@ class TurboQuantAdaptiveKVCacheState:
         self.append(k, v, bits, _pos_offset=start)
 
     # ------------------------------------------------------------------ fused attention
-    def _build_items(self, target_items: int = 1024, min_item_bytes: int = 16384) -> None:
+    def _build_items(self, target_items: Optional[int] = None, min_item_bytes: Optional[int] = None) -> None:
+        import os
+        target_items = int(os.environ.get("ODMKV_DECODE_ITEMS", 1024)) if target_items is None else target_items
+        min_item_bytes = int(os.environ.get("ODMKV_DECODE_MIN_ITEM_BYTES", 16384)) if min_item_bytes is None else min_item_bytes
         used = (self._counts + TILE - 1) // TILE
         used[4] = np.diff(self._seg_tile[4])              # exact segments grow between rebuilds
         total = sum(int(used[li].sum()) * _TILE_BYTES[li] for li in range(5))
@@ -434,6 +439,6 @@ class TurboQuantAdaptiveKVCacheState:
         ws = _lib.workspace(self.device, ws_bytes, "decode")
         _lib.check(lib.odmkv_decode_attn(
             q.data_ptr(), B, Hq, scale, C.byref(self._packed), items.data_ptr(), n_items,
-            ranges.data_ptr(), self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
-            out.data_ptr(), _lib.ptr(lse), ws.data_ptr(), ws_bytes, _lib.stream_ptr(self.device)))
+            ranges.data_ptr(), self.pi_k.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
+            self._decode_inv, out.data_ptr(), _lib.ptr(lse), ws.data_ptr(), ws_bytes, _lib.stream_ptr(self.device)))
         return (out, lse) if return_lse else out

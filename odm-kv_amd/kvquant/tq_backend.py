@@ -74,6 +74,41 @@ def codebook_table(dim: int, device) -> torch.Tensor:
     return tab
 
 
+_DECODE_TABLE_CACHE: dict[tuple[int, str], tuple[torch.Tensor, list[float]]] = {}
+
+
+def _fp16_friendly_scale(c: np.ndarray, n_candidates: int = 100_000) -> float:
+    """A scale S in [1, 2) for which every S * c_k is as close as possible to an fp16 number.
+
+    The decode kernel keeps centroid tables in fp16.  Rounding c_k itself costs up to 2^-11
+    relative per entry; rounding S * c_k for a well chosen S costs far less when the table has
+    few distinct magnitudes (2 for the 2-bit table, 4 for the 3-bit one), and the common factor
+    S is divided out of the per-token norm in fp32."""
+    mags = np.unique(np.abs(c.astype(np.float64)))
+    mags = mags[mags > 0]
+    cand = np.exp2(np.linspace(0.0, 1.0, n_candidates, endpoint=False))
+    prod = cand[:, None] * mags[None, :]
+    err = np.abs(prod.astype(np.float16).astype(np.float64) - prod) / prod
+    return float(cand[int(np.argmin(err.max(axis=1)))])
+
+
+def decode_tables(dim: int, device) -> tuple[torch.Tensor, list[float]]:
+    """(scaled centroid tables [284] on `device`, reciprocal scales per width) for the fused
+    decode kernel."""
+    key = (dim, str(device))
+    got = _DECODE_TABLE_CACHE.get(key)
+    if got is None:
+        parts, inv = [], []
+        for b in SUPPORTED_WIDTHS:
+            c = _load_or_compute_codebook(b, dim, "cpu", torch.float32).numpy()
+            s = _fp16_friendly_scale(c)
+            parts.append(torch.from_numpy((c.astype(np.float64) * s).astype(np.float32)))
+            inv.append(float(np.float32(1.0 / s)))
+        got = (torch.cat(parts).to(device).contiguous(), inv)
+        _DECODE_TABLE_CACHE[key] = got
+    return got
+
+
 class MSEQuantized(NamedTuple):
     indices: torch.Tensor     # container bytes as the reference packs them
     norms: torch.Tensor

@@ -37,7 +37,7 @@ def gaussian_layer(seed: int, n_kv: int, n_q: int, T: int, d: int = 128, dtype=t
     k[:, :N_SINK] *= sink_scale
     v[:, :N_SINK] *= sink_scale
     qwin = torch.randn(n_q, window_queries, d, generator=g)
-    q = torch.randn(n_q, d, generator=g)
+    q = torch.randn(n_q, d, generator=g).half().float()      # queries arrive in the model dtype
     return Layer(k.to(dtype), v.to(dtype), qwin.mean(dim=1), q, n_q)
 
 
@@ -55,7 +55,7 @@ def heavy_tail_layer(seed: int, n_kv: int = 4, n_q: int = 28, T: int = 32768, d:
     k[:, :N_SINK] *= 8.0
     v[:, :N_SINK] *= 8.0
     qwin = torch.randn(n_q, 64, d, generator=g)
-    q = torch.randn(n_q, d, generator=g)
+    q = torch.randn(n_q, d, generator=g).half().float()      # queries arrive in the model dtype
     return Layer(k.to(dtype), v.to(dtype), qwin.mean(dim=1), q, n_q)
 
 
@@ -73,7 +73,7 @@ def lognormal_norm_layer(seed: int, n_kv: int = 8, n_q: int = 32, T: int = 13107
     k[:, :N_SINK] *= 8.0
     v[:, :N_SINK] *= 8.0
     qwin = torch.randn(n_q, 64, d, generator=g)
-    q = torch.randn(n_q, d, generator=g)
+    q = torch.randn(n_q, d, generator=g).half().float()      # queries arrive in the model dtype
     return Layer(k.to(dtype), v.to(dtype), qwin.mean(dim=1), q, n_q)
 
 

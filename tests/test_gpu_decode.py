@@ -50,7 +50,7 @@ def test_decode_matches_oracle(B, Hkv, G, T, probs):
     bits = _rand_bits(g, (B, Hkv, T), probs)
     bits[..., :4] = 16
     bits[..., -16:] = 16
-    q = torch.randn(B, Hkv * G, 128, generator=g)
+    q = torch.randn(B, Hkv * G, 128, generator=g).half().float()     # a model hands over fp16 queries
     st, ref = _pair(k, v, bits)
     got, lse = st.decode_attention(q.to(DEV), return_lse=True)
     want = decode_attention_state(q, ref)
@@ -66,12 +66,14 @@ def test_decode_matches_oracle(B, Hkv, G, T, probs):
 def test_decode_special_cases():
     g = torch.Generator().manual_seed(1)
     k = torch.randn(1, 2, 300, 128, generator=g).half(); v = torch.randn(1, 2, 300, 128, generator=g).half()
-    q = torch.randn(1, 8, 128, generator=g)
+    q = torch.randn(1, 8, 128, generator=g).half().float()
     # every token exact: equals SDPA on the fp16 cache
     st, _ = _pair(k, v, torch.full((1, 2, 300), 16, dtype=torch.int32))
     sdpa = torch.nn.functional.scaled_dot_product_attention(
         q[:, :, None].double(), k.double().repeat_interleave(4, dim=1), v.double().repeat_interleave(4, dim=1))[:, :, 0]
-    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), sdpa) < 1e-5
+    # exact keys and values, fp16 query: what is left is the fp16 rounding of the softmax weights
+    # that feed the matrix cores (2^-11 per weight)
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), sdpa) < 5e-4
     # a single visible token: the output is that token's (dequantised) value
     bits = torch.zeros(1, 2, 300, dtype=torch.int32); bits[:, :, 17] = 4
     st, ref = _pair(k, v, bits)
@@ -107,7 +109,7 @@ def test_decode_after_appends_and_flush():
         kn = torch.randn(B, H, 1, 128, generator=g).half(); vn = torch.randn(B, H, 1, 128, generator=g).half()
         st.append_all_exact(kn.to(DEV), vn.to(DEV)); ref.append_all_exact(kn, vn)
         if step % 23 == 0 or step == 69:
-            q = torch.randn(B, H * G, 128, generator=g)
+            q = torch.randn(B, H * G, 128, generator=g).half().float()
             assert rel_err(st.decode_attention(q.to(DEV)).cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
     pos, _, _ = st.get_buffer_tokens(500)
     rpos, _, _ = ref.get_buffer_tokens(500)
@@ -116,7 +118,7 @@ def test_decode_after_appends_and_flush():
     lookup = {kk: i for i, kk in enumerate(key_ours)}
     perm = np.asarray([lookup[kk] for kk in (rpos[:, 1] * 10 ** 6 + rpos[:, 2])])
     st.flush_buffer(500, nb.to(DEV)); ref.flush_buffer(500, nb[perm])
-    q = torch.randn(B, H * G, 128, generator=g)
+    q = torch.randn(B, H * G, 128, generator=g).half().float()
     assert rel_err(st.decode_attention(q.to(DEV)).cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
 
 
