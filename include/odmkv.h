@@ -178,14 +178,17 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  *   out[b,q] = sum_t softmax_t( scaling * q[b,q] . Khat[b,q/G,t] ) Vhat[b,q/G,t]
  * over the stored (non-evicted) tokens.  Evicted tokens are simply absent.
  *
- * q: device fp32 [B, Hq, 128].  items: device int32 [n_items, 4] work list
- * (bh, level index 0..4, first tile, tile count), sorted by bh; item_range: device int32
+ * q: device fp32 [B, Hq, 128].  items: device int32 [n_items, 8] work list, sorted by bh:
+ * (bh, level index 0..4, first tile, tile count, tokens held by those tiles, first tile of the
+ * segment, 0, 0); for the exact level (index 4) the token count is read from seg_count instead,
+ * so that tokens appended since the list was built are seen.  item_range: device int32
  * [B*Hkv + 1] first item of each bh.  out: device fp32 [B, Hq, 128]; lse: device fp32 [B, Hq]
  * or NULL (log-sum-exp of the scaled logits).
  * The query is rounded to fp16 on entry (the attention being replaced receives it in the model's
  * fp16/bf16).  The centroid tables live in LDS as fp16; to keep their rounding out of the result,
  * `codebooks` here holds the centroids of each width times a per-width scale chosen on the host
- * so that the scaled values are (nearly) exact in fp16, and inv_scales (host, 4 floats) the
+ * so that the scaled values are (nearly) exact in fp16, codebooks_host a host copy of the same 284
+ * floats (the small tables travel as kernel arguments), and inv_scales (host, 4 floats) the
  * reciprocals of those scales.
  */
 size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);
@@ -193,7 +196,7 @@ int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
                       const odmkv_packed_t* store,
                       const int32_t* items, int n_items, const int32_t* item_range,
                       const float* pi_k, const float* pi_v, const float* codebooks,
-                      const float* inv_scales,
+                      const float* codebooks_host, const float* inv_scales,
                       float* out, float* lse, void* workspace, size_t workspace_bytes,
                       void* stream);
 

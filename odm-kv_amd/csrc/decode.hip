@@ -24,6 +24,7 @@
 // The LDS table is replicated over 32 slots (slot = lane % 32) so that lanes never share a bank.
 // All softmax state is kept in base-2 logarithms.
 #include "quant.h"
+#include <hip/hip_ext.h>
 
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef float f4 __attribute__((ext_vector_type(4)));
@@ -33,6 +34,17 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 #define LUT_BYTES 65536
 #define LOG2E 1.4426950408889634f
 #define LN2 0.6931471805599453f
+
+// optional per-workgroup timestamps for tuning (compiled out of the shipped library)
+#ifdef ODMKV_TRACE
+__device__ unsigned long long g_trace[8192 * 8];
+#define TRACE(k) if (tid == 0 && blockIdx.x < 8192) g_trace[blockIdx.x * 8 + (k)] = wall_clock64();
+extern "C" int odmkv_debug_read_trace(unsigned long long* host, int n) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace), sizeof(unsigned long long) * n);
+}
+#else
+#define TRACE(k)
+#endif
 
 struct DecodeArgs {
     odmkv_packed_t s;
@@ -44,9 +56,10 @@ struct DecodeArgs {
     const float* pi_k;
     const float* pi_v;
     const float* cb;
-    float* qrot;      // [B*Hq, 128] Pi_k q16
-    float* qs;        // [B*Hq, 128] q16
+    uint4* qrot;      // [B*Hq, 32] per 4-dim step: fp16 high halves (8 bytes) and low halves (8 bytes) of Pi_k q16
+    uint4* qs;        // [B*Hq, 32] the same for q16 itself (low halves are zero)
     float inv_s[4];   // 1 / table scale per width
+    float cbs[28];    // scaled centroids of widths 2, 3, 4 (kept in scalar registers; 8-bit ones stay in memory)
     float* partial;   // [n_items, GP, PSTRIDE]
     float* out;
     float* lse;
@@ -55,29 +68,39 @@ struct DecodeArgs {
 // ------------------------------------------------------------------------------------------------
 // prep: rotate and scale the queries
 // ------------------------------------------------------------------------------------------------
+__device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
+
 __global__ __launch_bounds__(256) void decode_prep_kernel(DecodeArgs a) {
     const int bq = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     // the query is consumed at fp16 precision, like the attention it replaces (model dtype)
     const float q0 = __half2float(__float2half_rn(a.q[(size_t)bq * HD + lane]));
     const float q1 = __half2float(__float2half_rn(a.q[(size_t)bq * HD + lane + 64]));
+    uint16_t* qs16 = reinterpret_cast<uint16_t*>(a.qs + (size_t)bq * 32);
+    uint16_t* qr16 = reinterpret_cast<uint16_t*>(a.qrot + (size_t)bq * 32);
     if (wave == 0) {
-        a.qs[(size_t)bq * HD + lane] = q0;
-        a.qs[(size_t)bq * HD + lane + 64] = q1;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int i = lane + 64 * h;
+            qs16[(i >> 2) * 8 + (i & 3)] = (uint16_t)half_bits(h ? q1 : q0);
+            qs16[(i >> 2) * 8 + 4 + (i & 3)] = 0;
+        }
     }
 #pragma unroll 4
     for (int i = wave; i < HD; i += 4) {
         const float* row = a.pi_k + (size_t)i * HD;
         float v = __fmaf_rn(row[lane], q0, row[lane + 64] * q1);
         v = wave_sum(v);
-        if (lane == 0) a.qrot[(size_t)bq * HD + i] = v;
+        if (lane == 0) {
+            const __half hi = __float2half_rn(v);
+            qr16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(hi);
+            qr16[(i >> 2) * 8 + 4 + (i & 3)] = (uint16_t)half_bits(v - __half2float(hi));
+        }
     }
 }
 
 // ------------------------------------------------------------------------------------------------
 // small helpers
 // ------------------------------------------------------------------------------------------------
-__device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
-
 __device__ static inline h4 as_h4(uint32_t lo, uint32_t hi) {
     union { uint32_t u[2]; h4 h; } x;
     x.u[0] = lo; x.u[1] = hi;
@@ -124,12 +147,22 @@ __device__ static inline float head_sum(float v) {
 //   W = 4: index = byte (2 codes) -> 2 halfs,             row = 128 bytes
 //   W = 8: index = byte (1 code)  -> the half in both halves of a dword, row = 128 bytes
 // ------------------------------------------------------------------------------------------------
+// pick table[idx] from a table that lives in scalar registers (no memory access: every workgroup
+// of a launch would otherwise hammer the same cache line)
+template <int N>
+__device__ static inline float pick(const float* t, uint32_t idx) {
+    float v = t[0];
+#pragma unroll
+    for (int k = 1; k < N; ++k) v = idx == (uint32_t)k ? t[k] : v;
+    return v;
+}
+
 template <int W>
-__device__ static inline void build_lut(uint8_t* lut, const float* __restrict__ cb, int tid) {
+__device__ static inline void build_lut(uint8_t* lut, const DecodeArgs& a, int tid) {
     if constexpr (W == 2) {
         uint32_t h[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) h[k] = half_bits(cb[(tid >> (2 * k)) & 3]);
+        for (int k = 0; k < 4; ++k) h[k] = half_bits(pick<4>(a.cbs, (tid >> (2 * k)) & 3));
         const uint4 v = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[0] | (h[1] << 16), h[2] | (h[3] << 16));
         uint4* dst = reinterpret_cast<uint4*>(lut + tid * 256);
 #pragma unroll
@@ -137,9 +170,9 @@ __device__ static inline void build_lut(uint8_t* lut, const float* __restrict__ 
     } else {
         uint32_t v;
         bool on = true;
-        if constexpr (W == 3) { on = tid < 64; v = half_bits(cb[tid & 7]) | (half_bits(cb[(tid >> 3) & 7]) << 16); }
-        else if constexpr (W == 4) { v = half_bits(cb[tid & 15]) | (half_bits(cb[tid >> 4]) << 16); }
-        else { v = half_bits(cb[tid]) * 0x10001u; }
+        if constexpr (W == 3) { on = tid < 64; v = half_bits(pick<8>(a.cbs + 4, tid & 7)) | (half_bits(pick<8>(a.cbs + 4, (tid >> 3) & 7)) << 16); }
+        else if constexpr (W == 4) { v = half_bits(pick<16>(a.cbs + 12, tid & 15)) | (half_bits(pick<16>(a.cbs + 12, tid >> 4)) << 16); }
+        else { v = half_bits(a.cb[codebook_offset(3) + tid]) * 0x10001u; }
         if (on) {
             uint4* dst = reinterpret_cast<uint4*>(lut + tid * 128);
 #pragma unroll
@@ -152,9 +185,11 @@ __device__ static inline void build_lut(uint8_t* lut, const float* __restrict__ 
 template <int W>
 __device__ static inline h4 lut4(const uint32_t* w, int s, const uint8_t* lut, uint32_t slot4) {
     if constexpr (W == 2) {
-        const int bit = 8 * s;
-        const uint32_t idx = (w[bit >> 5] >> (bit & 31)) & 0xffu;
-        const uint2 v = *reinterpret_cast<const uint2*>(lut + (idx << 8) + 2 * slot4);
+        // address = (byte s of the stream) * 256 + slot * 8, formed by one byte permute:
+        // byte 0 <- slot * 8 (< 256), byte 1 <- the code byte, bytes 2, 3 <- 0
+        const uint32_t sel = 0x0c0c0000u | ((4u + (uint32_t)(s & 3)) << 8);
+        const uint32_t addr = __builtin_amdgcn_perm(w[s >> 2], 2 * slot4, sel);
+        const uint2 v = *reinterpret_cast<const uint2*>(lut + addr);
         return as_h4(v.x, v.y);
     } else if constexpr (W == 4) {
         const int bit = 16 * s;
@@ -299,38 +334,72 @@ __device__ static inline void compute_tile(const TileData<W>& t, int nvalid, int
     PV_STEP(8) PV_STEP(9) PV_STEP(10) PV_STEP(11) PV_STEP(12) PV_STEP(13) PV_STEP(14) PV_STEP(15)
 }
 
+// stage the group's queries (fp16 high/low halves per 4-dim step) in LDS; heads beyond the group are 0
+template <int NP>
+__device__ static inline void stage_queries(const DecodeArgs& a, const uint4* src, uint4* qsh, int tid) {
+    if (tid < 4 * NP * 32) qsh[tid] = (tid >> 5) < a.G ? src[tid] : make_uint4(0u, 0u, 0u, 0u);
+}
+template <int NP>
+__device__ static inline void fetch_queries(const uint4* qsh, int lane, h4* qr, h4* ql) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p)
+#pragma unroll
+        for (int s = 0; s < 32; ++s) {
+            const uint4 v = qsh[(4 * p + (lane & 3)) * 32 + s];
+            qr[p * 32 + s] = as_h4(v.x, v.y);
+            ql[p * 32 + s] = as_h4(v.z, v.w);
+        }
+}
+
+// One work item of a quantised level.  The first tile's loads are issued before the table is built
+// and the queries are staged, so that HBM latency overlaps the set-up.
 template <int W, int NP>
-__device__ static inline void run_quant_level(const DecodeArgs& a, int li, int tile0, int ntiles, int seg_first,
-                                              int count, int wave, int lane, const uint8_t* lut, const h4* qr,
-                                              const h4* ql, WaveState<NP>& st) {
+__device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq0, int tile0, int ntiles, int ntok,
+                                              int tid, uint8_t* lut, uint4* qsh, WaveState<NP>& st) {
+    const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
     const float vsc = a.inv_s[li], ksc = a.inv_s[li] * a.scaling * LOG2E;
+    TileData<W> cur;
+    int tt = wave;
+    int nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
+    if (nvalid > 0) load_tile<W>(cur, a, li, tile0 + tt, lane);
+    // second buffer (not for the widest rows: the registers go to the query there).  Both tiles are
+    // requested before the set-up waits on anything: a wavefront rarely owns more than a few tiles,
+    // so the second tile's HBM latency must not start after the first tile is done.
+    TileData<W> nxt;
+    int nv1 = 0;
+    if constexpr (W != 8) {
+        nv1 = tt + NWAVES < ntiles ? min(ntok - (tt + NWAVES) * TILE, TILE) : 0;
+        if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + NWAVES, lane);
+    }
+    stage_queries<NP>(a, a.qrot + (size_t)bq0 * 32, qsh, tid);
+    build_lut<W>(lut, a, tid);
+    __syncthreads();
+    TRACE(1)
+    h4 qr[NP * 32], ql[NP * 32];
+    fetch_queries<NP>(qsh, lane, qr, ql);
+    if (nvalid <= 0) return;
+    TRACE(2)
     if constexpr (W == 8) {
-        // wide rows: no double buffering, the registers go to the query
-        TileData<W> cur;
-        for (int tt = wave; tt < ntiles; tt += NWAVES) {
-            const int nvalid = min(count - (tile0 + tt - seg_first) * TILE, TILE);
+        while (true) {
+            compute_tile<W, NP>(cur, nvalid, lane, lut, slot4, qr, ql, ksc, vsc, st);
+            tt += NWAVES;
+            nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
             if (nvalid <= 0) break;
             load_tile<W>(cur, a, li, tile0 + tt, lane);
-            compute_tile<W, NP>(cur, nvalid, lane, lut, slot4, qr, ql, ksc, vsc, st);
         }
-        return;
-    }
-    TileData<W> cur, nxt;
-    int tt = wave;
-    if (tt >= ntiles) return;
-    int nvalid = min(count - (tile0 + tt - seg_first) * TILE, TILE);
-    if (nvalid <= 0) return;
-    load_tile<W>(cur, a, li, tile0 + tt, lane);
-    while (true) {
-        const int tn = tt + NWAVES;
-        const int nvalid_n = tn < ntiles ? min(count - (tile0 + tn - seg_first) * TILE, TILE) : 0;
-        if (nvalid_n > 0) load_tile<W>(nxt, a, li, tile0 + tn, lane);     // in flight while this tile is computed
-        compute_tile<W, NP>(cur, nvalid, lane, lut, slot4, qr, ql, ksc, vsc, st);
-        if (nvalid_n <= 0) break;
-        cur = nxt;
-        tt = tn;
-        nvalid = nvalid_n;
+    } else {
+        while (true) {
+            compute_tile<W, NP>(cur, nvalid, lane, lut, slot4, qr, ql, ksc, vsc, st);
+            if (nv1 <= 0) break;
+            tt += 2 * NWAVES;
+            nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
+            if (nvalid > 0) load_tile<W>(cur, a, li, tile0 + tt, lane);
+            compute_tile<W, NP>(nxt, nv1, lane, lut, slot4, qr, ql, ksc, vsc, st);
+            if (nvalid <= 0) break;
+            nv1 = tt + NWAVES < ntiles ? min(ntok - (tt + NWAVES) * TILE, TILE) : 0;
+            if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + NWAVES, lane);
+        }
     }
 }
 
@@ -349,10 +418,16 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int t
     }
 
 template <int NP>
-__device__ static inline void run_exact_level(const DecodeArgs& a, int tile0, int ntiles, int seg_first, int count,
-                                              int wave, int lane, const h4* qr, WaveState<NP>& st) {
+__device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int bq0, int tile0, int ntiles, int seg_first,
+                                              int tid, uint4* qsh, WaveState<NP>& st) {
+    const int wave = tid >> 6, lane = tid & 63;
     const bool bf = a.s.exact_dtype == ODMKV_BF16;
     const float esc = a.scaling * LOG2E;
+    const int count = a.s.seg_count[4][bh];          // exact segments grow between work-list rebuilds
+    stage_queries<NP>(a, a.qs + (size_t)bq0 * 32, qsh, tid);
+    __syncthreads();
+    h4 qr[NP * 32], ql[NP * 32];
+    fetch_queries<NP>(qsh, lane, qr, ql);
     for (int tt = wave; tt < ntiles; tt += NWAVES) {
         const int tile = tile0 + tt;
         const int nvalid = min(count - (tile - seg_first) * TILE, TILE);
@@ -402,40 +477,14 @@ template <int NP>
 __global__ __launch_bounds__(256, 2) void decode_main_kernel(DecodeArgs a) {
     __shared__ __align__(16) uint8_t lut[LUT_BYTES];     // centroid table; reused to combine the wavefronts
     __shared__ float wm[NWAVES][4 * NP], wl[NWAVES][4 * NP];
-    __shared__ __align__(16) float qsh[4 * NP * HD];
+    __shared__ uint4 qsh[4 * NP * 32];
 
     const int item = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int bh = a.items[4 * item + 0];
-    const int li = a.items[4 * item + 1];
-    const int tile0 = a.items[4 * item + 2];
-    const int ntiles = a.items[4 * item + 3];
-    const int b = bh / a.s.Hkv, hkv = bh % a.s.Hkv;
-
-    // the group's queries go through LDS (one coalesced read), then every lane keeps its own
-    // head (lane % 4 per pass) in registers as fp16 high and low halves; heads beyond the group are 0
-    const float* qsrc = (li == 4 ? a.qs : a.qrot) + ((size_t)b * a.Hq + (size_t)hkv * a.G) * HD;
-    for (int e = tid; e < 4 * NP * HD; e += 256) qsh[e] = (e >> 7) < a.G ? qsrc[e] : 0.0f;
-    switch (li) {
-        case 0: build_lut<2>(lut, a.cb + codebook_offset(0), tid); break;
-        case 1: build_lut<3>(lut, a.cb + codebook_offset(1), tid); break;
-        case 2: build_lut<4>(lut, a.cb + codebook_offset(2), tid); break;
-        case 3: build_lut<8>(lut, a.cb + codebook_offset(3), tid); break;
-        default: break;
-    }
-    __syncthreads();
-    h4 qr[NP * 32], ql[NP * 32];
-#pragma unroll
-    for (int p = 0; p < NP; ++p) {
-        const f4* src = reinterpret_cast<const f4*>(qsh + (4 * p + (lane & 3)) * HD);
-#pragma unroll
-        for (int s = 0; s < 32; ++s) {
-            const f4 v = src[s];
-            const h4 hi = (h4){(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-            qr[p * 32 + s] = hi;
-            ql[p * 32 + s] = (h4){(_Float16)(v[0] - (float)hi[0]), (_Float16)(v[1] - (float)hi[1]),
-                                  (_Float16)(v[2] - (float)hi[2]), (_Float16)(v[3] - (float)hi[3])};
-        }
-    }
+    TRACE(0)
+    const int4 d0 = reinterpret_cast<const int4*>(a.items)[2 * item];       // bh, level, first tile, tiles
+    const int4 d1 = reinterpret_cast<const int4*>(a.items)[2 * item + 1];   // tokens, first tile of the segment
+    const int bh = d0.x, li = d0.y, tile0 = d0.z, ntiles = d0.w;
+    const int bq0 = (bh / a.s.Hkv) * a.Hq + (bh % a.s.Hkv) * a.G;            // first query head of the group
 
     WaveState<NP> st;
 #pragma unroll
@@ -443,18 +492,18 @@ __global__ __launch_bounds__(256, 2) void decode_main_kernel(DecodeArgs a) {
         st.m[p] = -INFINITY; st.l[p] = 0.0f;
         st.acc[p][0] = (f4){0.f, 0.f, 0.f, 0.f}; st.acc[p][1] = (f4){0.f, 0.f, 0.f, 0.f};
     }
-    const int seg_first = a.s.seg_tile[li][bh];
-    const int count = a.s.seg_count[li][bh];
     switch (li) {
-        case 0: run_quant_level<2, NP>(a, 0, tile0, ntiles, seg_first, count, wave, lane, lut, qr, ql, st); break;
-        case 1: run_quant_level<3, NP>(a, 1, tile0, ntiles, seg_first, count, wave, lane, lut, qr, ql, st); break;
-        case 2: run_quant_level<4, NP>(a, 2, tile0, ntiles, seg_first, count, wave, lane, lut, qr, ql, st); break;
-        case 3: run_quant_level<8, NP>(a, 3, tile0, ntiles, seg_first, count, wave, lane, lut, qr, ql, st); break;
-        default: run_exact_level<NP>(a, tile0, ntiles, seg_first, count, wave, lane, qr, st); break;
+        case 0: run_quant_level<2, NP>(a, 0, bq0, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        case 1: run_quant_level<3, NP>(a, 1, bq0, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        case 2: run_quant_level<4, NP>(a, 2, bq0, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        case 3: run_quant_level<8, NP>(a, 3, bq0, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        default: run_exact_level<NP>(a, bh, bq0, tile0, ntiles, d1.y, tid, qsh, st); break;
     }
 
     // ---- combine the four wavefronts (the table is no longer needed) ----
+    TRACE(3)
     __syncthreads();
+    TRACE(4)
     float* wacc = reinterpret_cast<float*>(lut);          // [NWAVES][4*NP][128]
     constexpr int GP = 4 * NP;
 #pragma unroll
@@ -486,6 +535,7 @@ __global__ __launch_bounds__(256, 2) void decode_main_kernel(DecodeArgs a) {
         dst[g * PSTRIDE + j] = s;
         if (j == 0) { dst[g * PSTRIDE + HD] = M; dst[g * PSTRIDE + HD + 1] = L; }
     }
+    TRACE(5)
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -523,7 +573,7 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
         const float* p = a.partial + ((size_t)(i0 + it) * GP + g) * PSTRIDE;
         const float f = M > -INFINITY ? __builtin_amdgcn_exp2f(p[HD] - M) : 0.0f;
         lpart = __fmaf_rn(p[HD + 1], f, lpart);
-        wts[it] = a.items[4 * (i0 + it) + 1] == 4 ? -f : f;
+        wts[it] = a.items[8 * (i0 + it) + 1] == 4 ? -f : f;
     }
     lpart = wave_sum(lpart);
     if ((tid & 63) == 0) red[tid >> 6] = lpart;
@@ -607,7 +657,7 @@ extern "C" int odmkv_profile_collect(float* ms, int capacity, int* n_out) {
 static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
 
 extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
-    size_t q = align_up((size_t)B * Hq * HD * sizeof(float), 256);
+    size_t q = align_up((size_t)B * Hq * 32 * sizeof(uint4), 256);
     return 2 * q + align_up((size_t)n_items * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
 }
 
@@ -615,9 +665,10 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
                                  const odmkv_packed_t* store,
                                  const int32_t* items, int n_items, const int32_t* item_range,
                                  const float* pi_k, const float* pi_v, const float* codebooks,
-                                 const float* inv_scales,
+                                 const float* codebooks_host, const float* inv_scales,
                                  float* out, float* lse, void* workspace, size_t workspace_bytes,
                                  void* stream) {
+    ODMKV_CHECK_ARG(codebooks_host != nullptr, "decode_attn: null host copy of the centroid tables");
     ODMKV_CHECK_ARG(inv_scales != nullptr, "decode_attn: null table scales");
     ODMKV_CHECK_ARG(q && store && item_range && pi_k && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
     ODMKV_CHECK_ARG(n_items == 0 || items, "decode_attn: null work list");
@@ -633,9 +684,10 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     a.items = items; a.item_range = item_range;
     a.pi_k = pi_k; a.pi_v = pi_v; a.cb = codebooks;
     for (int w = 0; w < 4; ++w) a.inv_s[w] = inv_scales[w];
-    const size_t qbytes = align_up((size_t)B * Hq * HD * sizeof(float), 256);
-    a.qrot = (float*)workspace;
-    a.qs = (float*)((char*)workspace + qbytes);
+    for (int k = 0; k < 28; ++k) a.cbs[k] = codebooks_host[k];
+    const size_t qbytes = align_up((size_t)B * Hq * 32 * sizeof(uint4), 256);
+    a.qrot = (uint4*)workspace;
+    a.qs = (uint4*)((char*)workspace + qbytes);
     a.partial = (float*)((char*)workspace + 2 * qbytes);
     a.out = out; a.lse = lse;
     hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(256), 0, st, a);
@@ -643,14 +695,14 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     const int GP = group_pad(G);
     if (n_items > 0) {
         const bool rec = g_prof_on && (size_t)(2 * g_prof_used + 1) < g_prof_events.size();
-        if (rec) ODMKV_CHECK_HIP(hipEventRecord(g_prof_events[2 * g_prof_used], st));
-        if (GP == 4) hipLaunchKernelGGL((decode_main_kernel<1>), dim3(n_items), dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((decode_main_kernel<2>), dim3(n_items), dim3(256), 0, st, a);
+        // when measuring, the events are attached to the dispatch itself: they carry the kernel's own
+        // start and end timestamps, not those of separate marker packets
+        hipEvent_t e0 = rec ? g_prof_events[2 * g_prof_used] : nullptr;
+        hipEvent_t e1 = rec ? g_prof_events[2 * g_prof_used + 1] : nullptr;
+        if (GP == 4) hipExtLaunchKernelGGL((decode_main_kernel<1>), dim3(n_items), dim3(256), 0, st, e0, e1, 0, a);
+        else hipExtLaunchKernelGGL((decode_main_kernel<2>), dim3(n_items), dim3(256), 0, st, e0, e1, 0, a);
         ODMKV_CHECK_LAUNCH("decode_main_kernel");
-        if (rec) {
-            ODMKV_CHECK_HIP(hipEventRecord(g_prof_events[2 * g_prof_used + 1], st));
-            ++g_prof_used;
-        }
+        if (rec) ++g_prof_used;
     }
     if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);
     else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);

@@ -11,7 +11,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libodmkv.so")
+LIB_PATH = os.environ.get("ODMKV_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libodmkv.so")
 
 F16, BF16, F32 = 0, 1, 2
 HEAD_DIM = 128
@@ -61,7 +61,7 @@ def _load() -> C.CDLL:
         "odmkv_append_exact": (C.c_int, [C.POINTER(Packed), vp, vp, i32, vp]),
         "odmkv_decode_workspace_bytes": (sz, [i32, i32, i32]),
         "odmkv_decode_attn": (C.c_int, [vp, i32, i32, f32, C.POINTER(Packed), vp, i32, vp, vp, vp, vp,
-                                        C.POINTER(C.c_float), vp, vp, vp, sz, vp]),
+                                        C.POINTER(C.c_float), C.POINTER(C.c_float), vp, vp, vp, sz, vp]),
         "odmkv_profile_enable": (C.c_int, [i32]),
         "odmkv_profile_collect": (C.c_int, [C.POINTER(C.c_float), i32, C.POINTER(C.c_int)]),
         "odmkv_profile_disable": (C.c_int, []),

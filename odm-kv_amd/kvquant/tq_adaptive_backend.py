@@ -78,6 +78,7 @@ class TurboQuantAdaptiveKVCacheState:
         self.codebooks = codebook_table(head_dim, self.device)
         self._decode_cb, inv = decode_tables(head_dim, self.device)
         self._decode_inv = (C.c_float * 4)(*inv)
+        self._decode_cb_host = (C.c_float * 284)(*self._decode_cb.cpu().tolist())
         self._exact_torch_dtype = torch.bfloat16 if dtype == torch.bfloat16 else torch.float16
         self._reset()
 
@@ -410,10 +411,13 @@ class TurboQuantAdaptiveKVCacheState:
                     continue
                 step = max(1, int(round(per_item / _TILE_BYTES[li])))
                 t0 = int(self._seg_tile[li, s])
+                cnt = int(self._counts[li, s])
                 for a in range(0, nt, step):
-                    items.append((s, li, t0 + a, min(step, nt - a)))
+                    # (segment, level, first tile, tiles, tokens in those tiles, segment's first tile, -, -)
+                    n = min(step, nt - a)
+                    items.append((s, li, t0 + a, n, min(cnt - a * TILE, n * TILE), t0, 0, 0))
             ranges.append(len(items))
-        arr = np.asarray(items, np.int32).reshape(-1, 4)
+        arr = np.asarray(items, np.int32).reshape(-1, 8)
         self._items = (torch.from_numpy(arr).to(self.device),
                        torch.from_numpy(np.asarray(ranges, np.int32)).to(self.device), len(items))
 
@@ -440,5 +444,5 @@ class TurboQuantAdaptiveKVCacheState:
         _lib.check(lib.odmkv_decode_attn(
             q.data_ptr(), B, Hq, scale, C.byref(self._packed), items.data_ptr(), n_items,
             ranges.data_ptr(), self.pi_k.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
-            self._decode_inv, out.data_ptr(), _lib.ptr(lse), ws.data_ptr(), ws_bytes, _lib.stream_ptr(self.device)))
+            self._decode_cb_host, self._decode_inv, out.data_ptr(), _lib.ptr(lse), ws.data_ptr(), ws_bytes, _lib.stream_ptr(self.device)))
         return (out, lse) if return_lse else out
