@@ -53,7 +53,7 @@ struct DecodeArgs {
     float scaling;
     const int32_t* items;
     const int32_t* item_range;
-    const float* pi_k;
+    const float* pi_k_t;   // Pi_k transposed
     const float* pi_v;
     const float* cb;
     uint4* qrot;      // [B*Hq, 32] per 4-dim step: fp16 high halves (8 bytes) and low halves (8 bytes) of Pi_k q16
@@ -70,32 +70,24 @@ struct DecodeArgs {
 // ------------------------------------------------------------------------------------------------
 __device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
 
-__global__ __launch_bounds__(256) void decode_prep_kernel(DecodeArgs a) {
-    const int bq = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+__global__ __launch_bounds__(128) void decode_prep_kernel(DecodeArgs a) {
+    __shared__ float qsh[HD];
+    const int bq = blockIdx.x, i = threadIdx.x;
     // the query is consumed at fp16 precision, like the attention it replaces (model dtype)
-    const float q0 = __half2float(__float2half_rn(a.q[(size_t)bq * HD + lane]));
-    const float q1 = __half2float(__float2half_rn(a.q[(size_t)bq * HD + lane + 64]));
+    const __half q16 = __float2half_rn(a.q[(size_t)bq * HD + i]);
+    qsh[i] = __half2float(q16);
     uint16_t* qs16 = reinterpret_cast<uint16_t*>(a.qs + (size_t)bq * 32);
     uint16_t* qr16 = reinterpret_cast<uint16_t*>(a.qrot + (size_t)bq * 32);
-    if (wave == 0) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int i = lane + 64 * h;
-            qs16[(i >> 2) * 8 + (i & 3)] = (uint16_t)half_bits(h ? q1 : q0);
-            qs16[(i >> 2) * 8 + 4 + (i & 3)] = 0;
-        }
-    }
-#pragma unroll 4
-    for (int i = wave; i < HD; i += 4) {
-        const float* row = a.pi_k + (size_t)i * HD;
-        float v = __fmaf_rn(row[lane], q0, row[lane + 64] * q1);
-        v = wave_sum(v);
-        if (lane == 0) {
-            const __half hi = __float2half_rn(v);
-            qr16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(hi);
-            qr16[(i >> 2) * 8 + 4 + (i & 3)] = (uint16_t)half_bits(v - __half2float(hi));
-        }
-    }
+    qs16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(q16);
+    qs16[(i >> 2) * 8 + 4 + (i & 3)] = 0;
+    __syncthreads();
+    // q'_i = sum_j Pi_k[i][j] q_j, read from the transposed matrix so that threads read side by side
+    float acc = 0.0f;
+#pragma unroll 16
+    for (int j = 0; j < HD; ++j) acc = __fmaf_rn(a.pi_k_t[(size_t)j * HD + i], qsh[j], acc);
+    const __half hi = __float2half_rn(acc);
+    qr16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(hi);
+    qr16[(i >> 2) * 8 + 4 + (i & 3)] = (uint16_t)half_bits(acc - __half2float(hi));
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -664,13 +656,13 @@ extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
 extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
                                  const odmkv_packed_t* store,
                                  const int32_t* items, int n_items, const int32_t* item_range,
-                                 const float* pi_k, const float* pi_v, const float* codebooks,
+                                 const float* pi_k_t, const float* pi_v, const float* codebooks,
                                  const float* codebooks_host, const float* inv_scales,
                                  float* out, float* lse, void* workspace, size_t workspace_bytes,
                                  void* stream) {
     ODMKV_CHECK_ARG(codebooks_host != nullptr, "decode_attn: null host copy of the centroid tables");
     ODMKV_CHECK_ARG(inv_scales != nullptr, "decode_attn: null table scales");
-    ODMKV_CHECK_ARG(q && store && item_range && pi_k && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
+    ODMKV_CHECK_ARG(q && store && item_range && pi_k_t && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
     ODMKV_CHECK_ARG(n_items == 0 || items, "decode_attn: null work list");
     ODMKV_CHECK_ARG(B > 0 && Hq > 0 && store->B == B && store->Hkv > 0 && Hq % store->Hkv == 0,
                     "decode_attn: bad head counts B=%d Hq=%d store(B=%d,Hkv=%d)", B, Hq, store->B, store->Hkv);
@@ -682,7 +674,7 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     DecodeArgs a;
     a.s = *store; a.q = q; a.Hq = Hq; a.G = G; a.B = B; a.scaling = scaling;
     a.items = items; a.item_range = item_range;
-    a.pi_k = pi_k; a.pi_v = pi_v; a.cb = codebooks;
+    a.pi_k_t = pi_k_t; a.pi_v = pi_v; a.cb = codebooks;
     for (int w = 0; w < 4; ++w) a.inv_s[w] = inv_scales[w];
     for (int k = 0; k < 28; ++k) a.cbs[k] = codebooks_host[k];
     const size_t qbytes = align_up((size_t)B * Hq * 32 * sizeof(uint4), 256);
@@ -690,7 +682,7 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     a.qs = (uint4*)((char*)workspace + qbytes);
     a.partial = (float*)((char*)workspace + 2 * qbytes);
     a.out = out; a.lse = lse;
-    hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(128), 0, st, a);
     ODMKV_CHECK_LAUNCH("decode_prep_kernel");
     const int GP = group_pad(G);
     if (n_items > 0) {

@@ -75,6 +75,7 @@ class TurboQuantAdaptiveKVCacheState:
             raise RuntimeError("the packed KV store lives on the GPU; there is no CPU path")
         self.pi_k = cached_rotation(head_dim, self.device, seed)
         self.pi_v = cached_rotation(head_dim, self.device, seed + 2000)
+        self._pi_k_t = self.pi_k.t().contiguous()
         self.codebooks = codebook_table(head_dim, self.device)
         self._decode_cb, inv = decode_tables(head_dim, self.device)
         self._decode_inv = (C.c_float * 4)(*inv)
@@ -397,7 +398,7 @@ class TurboQuantAdaptiveKVCacheState:
     # ------------------------------------------------------------------ fused attention
     def _build_items(self, target_items: Optional[int] = None, min_item_bytes: Optional[int] = None) -> None:
         import os
-        target_items = int(os.environ.get("ODMKV_DECODE_ITEMS", 1024)) if target_items is None else target_items
+        target_items = int(os.environ.get("ODMKV_DECODE_ITEMS", 512)) if target_items is None else target_items
         min_item_bytes = int(os.environ.get("ODMKV_DECODE_MIN_ITEM_BYTES", 16384)) if min_item_bytes is None else min_item_bytes
         used = (self._counts + TILE - 1) // TILE
         used[4] = np.diff(self._seg_tile[4])              # exact segments grow between rebuilds
@@ -443,6 +444,6 @@ class TurboQuantAdaptiveKVCacheState:
         ws = _lib.workspace(self.device, ws_bytes, "decode")
         _lib.check(lib.odmkv_decode_attn(
             q.data_ptr(), B, Hq, scale, C.byref(self._packed), items.data_ptr(), n_items,
-            ranges.data_ptr(), self.pi_k.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
+            ranges.data_ptr(), self._pi_k_t.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
             self._decode_cb_host, self._decode_inv, out.data_ptr(), _lib.ptr(lse), ws.data_ptr(), ws_bytes, _lib.stream_ptr(self.device)))
         return (out, lse) if return_lse else out
