@@ -1,0 +1,306 @@
+"""TurboQuantPerTokenBackendPress: the ODM-KV press that keeps the packed mixed-precision cache.
+
+Host-side mirror of the reference class (kvquant/adaptive_backend_press.py:22-682): same
+constructor, hook protocol, prefill finalisation (:292-325), decode buffering (:383-458), flush
+(:464-595), flush attention (:601-665) and cached-ratio allocation (:198-290).  Differences that
+follow from running on the packed store:
+
+* decode attention is computed by the fused LUT kernel over the store (see attention_patch.py),
+  not by the HF attention function over a re-materialised cache; the HF cache tensors are still
+  kept in step (quantised positions overwritten in place) so the dense path remains usable;
+* layer-wise allocation of all layers runs as one batched allocator launch;
+* flush scoring handles all kv-heads of a sequence in one launch instead of a loop per head.
+"""
+from __future__ import annotations
+
+import contextlib
+import math
+from typing import Optional
+
+import torch
+from torch import nn
+
+from kvquant.allocator import optimal_scores_to_bits, ratio_scores_to_bits, scores_to_bits
+from kvquant.attention_utils import _aligned_rotary_outputs, _apply_rotary_pos_emb_q, _get_query_states
+from kvquant.press import TurboQuantPerTokenPress
+from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+
+
+class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
+    def __init__(self, *, value_group_size: int = 32, key_quantizer: str = "prod", value_quantizer: str = "minmax",
+                 scorer=None, bit_levels: tuple[int, ...] = (0, 2, 4, 8, 16), ratios: Optional[tuple[float, ...]] = None,
+                 target_avg_bits: Optional[float] = None, eviction_cost: float = 5.0, above_target_alpha: float = 1.0,
+                 n_outlier_channels: int = 0, outlier_min_bits: int = 4, seed: int = 42, decode_quant: bool = True,
+                 sink_tokens: int = 0, layerwise: bool = False, buffer_size: int = 128, initial_layers_fp16: int = 0,
+                 allow_decode_eviction: bool = False):
+        min_bits = 2 if key_quantizer in ("prod", "turboquant_prod", "turboquantprod") else 1
+        invalid = [b for b in bit_levels if b not in (0, 16) and b < min_bits]
+        if invalid:
+            raise ValueError(f"TurboQuantPerTokenBackendPress does not support key bit-levels below "
+                             f"{min_bits} with key_quantizer={key_quantizer!r}: {invalid}")
+        super().__init__(scorer=scorer, bit_levels=bit_levels, ratios=ratios, target_avg_bits=target_avg_bits,
+                         eviction_cost=eviction_cost, above_target_alpha=above_target_alpha,
+                         n_outlier_channels=n_outlier_channels, outlier_min_bits=outlier_min_bits, seed=seed,
+                         decode_quant=decode_quant, sink_tokens=sink_tokens, layerwise=layerwise,
+                         quantizer="turboquant", value_quantizer=value_quantizer,
+                         value_group_size=value_group_size, allow_decode_eviction=allow_decode_eviction)
+        self.key_quantizer = key_quantizer
+        self.buffer_size = buffer_size
+        self.initial_layers_fp16 = initial_layers_fp16
+        self._states: dict[int, TurboQuantAdaptiveKVCacheState] = {}
+        self._buffer_counts: dict[int, int] = {}
+        self._buffer_start_seqs: dict[int, int] = {}
+        # (layer, head) -> ((level, fraction), ...) observed in the prefill allocation
+        self._observed_ratios: dict[tuple[int, int], tuple[tuple[int, float], ...]] = {}
+
+    def _prewarm_quantizers(self, model) -> None:
+        return          # the state builds its rotations and tables when it is created
+
+    def _get_or_create_state(self, layer_idx: int, keys: torch.Tensor) -> TurboQuantAdaptiveKVCacheState:
+        state = self._states.get(layer_idx)
+        if state is not None:
+            return state
+        levels = self.bit_levels
+        if self.buffer_size > 0 and 16 not in levels:
+            levels = tuple(sorted(set(levels) | {16}))
+        state = TurboQuantAdaptiveKVCacheState(
+            head_dim=keys.shape[-1], bit_levels=levels, key_quantizer=self.key_quantizer,
+            value_quantizer=self.value_quantizer, value_group_size=self.value_group_size,
+            device=keys.device, dtype=keys.dtype, seed=self.seed + layer_idx * 7,
+            outlier_min_bits=self.outlier_min_bits)
+        state.exact_decode_append = self.buffer_size > 0 and self.decode_quant
+        self._states[layer_idx] = state
+        return state
+
+    def _attach(self, cache, layer_idx: int, module: nn.Module, state) -> None:
+        module.masked_key_indices = state.masked_key_indices()
+        module._odmkv_state = state
+        if hasattr(cache, "layers"):
+            cache.layers[layer_idx]._tq_backend_state = state
+
+    def _sync_cache_from_state(self, cache, layer_idx: int, module: nn.Module, state, *, prefill_fast: bool = False) -> None:
+        if prefill_fast:
+            keys, values = self._get_cache_tensors(cache, layer_idx)
+            state.materialize_quantized_into(keys, values)
+        else:
+            keys, values = state.materialize()
+            self._set_cache_tensors(cache, layer_idx, keys, values)
+        self._attach(cache, layer_idx, module, state)
+
+    # ------------------------------------------------------------------ cached ratios
+    def _record_observed_ratios(self, layer_idx: int, bits: torch.Tensor) -> None:
+        """Level fractions per kv-head over the bulk of the prefill (sinks and the protected tail
+        left out), taken before the window override."""
+        if bits.dim() != 3 or bits.shape[-1] == 0:
+            return
+        B, H, T = bits.shape
+        start = min(int(self.sink_tokens), T) if self.sink_tokens > 0 else 0
+        end = T - min(int(self.buffer_size), T) if self.buffer_size > 0 else T
+        if end <= start:
+            start, end = 0, T
+        bulk = bits[..., start:end].reshape(B * H, end - start)
+        levels = sorted(set(int(b) for b in self.bit_levels) | {16})
+        lv = torch.tensor(levels, device=bits.device, dtype=bits.dtype)
+        counts = (bulk.unsqueeze(-1) == lv).sum(dim=1).cpu()                 # [B*H, K], one transfer
+        for row in range(B * H):
+            c = counts[row]
+            total = int(c.sum())
+            if total == 0:
+                continue
+            fracs = (c.float() / total).tolist()
+            self._observed_ratios[(layer_idx, row % H)] = tuple(
+                (b, f) for b, f, n in zip(levels, fracs, c.tolist()) if n > 0)
+
+    def _allocate_bits_via_cached_ratios(self, scores, positions, num_heads, layer_idx, allowed_levels):
+        if not all((layer_idx, h) in self._observed_ratios for h in range(num_heads)):
+            return None
+        bits = torch.empty_like(scores, dtype=torch.int32)
+        head_indices = positions[:, 1]
+        for h in range(num_heads):
+            kept = [(b, r) for b, r in self._observed_ratios[(layer_idx, h)] if b in allowed_levels and r > 0]
+            if not kept:
+                return None
+            total = sum(r for _, r in kept)
+            levels, ratios = zip(*[(b, r / total) for b, r in kept])
+            mask = head_indices == h
+            if not mask.any():
+                continue
+            bits[mask] = ratio_scores_to_bits(scores[mask], tuple(levels), tuple(ratios)).to(torch.int32)
+        return bits
+
+    # ------------------------------------------------------------------ prefill
+    def _finalize_prefill(self, cache) -> None:
+        if self.n_outlier_channels > 0:
+            raise NotImplementedError("outlier-channel separation is not built (n_outlier_channels must be 0)")
+        for layer_idx, bits in self._allocate_bits_for_prefill().items():
+            keys, values = self._get_cache_tensors(cache, layer_idx)
+            self._record_observed_ratios(layer_idx, bits)
+            if layer_idx < self.initial_layers_fp16:
+                bits = torch.full_like(bits, 16)
+            elif self.buffer_size > 0:
+                bits = bits.clone()
+                bits[..., -min(self.buffer_size, bits.shape[-1]):] = 16
+            state = self._get_or_create_state(layer_idx, keys)
+            state.prefill(keys, values, bits.to(dtype=torch.int32, device=keys.device))
+            module = self._layer_modules.get(layer_idx)
+            if module is not None:
+                self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True)
+            if self.buffer_size > 0:
+                self._buffer_start_seqs[layer_idx] = int(keys.shape[2])
+                self._buffer_counts[layer_idx] = 0
+        self._reset_prefill_state()
+
+    # ------------------------------------------------------------------ hook
+    def _forward_hook(self, module: nn.Module, args, kwargs, output):
+        cache, hidden_states = self._hook_inputs(module, args, kwargs)
+        if cache is None or hidden_states is None:
+            return output
+        layer_idx = int(module.layer_idx)
+        self._layer_modules[layer_idx] = module
+        keys, values = self._get_cache_tensors(cache, layer_idx)
+        if self._head_dim is None:
+            self._head_dim = keys.shape[-1]
+        q_len, cache_len = hidden_states.shape[1], keys.shape[2]
+        if cache_len == q_len:
+            self._prefill_hook(module, cache, hidden_states, layer_idx, keys, values)
+            return output
+        if not self.decode_quant or layer_idx < self.initial_layers_fp16:
+            return output
+
+        state = self._get_or_create_state(layer_idx, keys)
+        if self.buffer_size > 0:
+            buf_start = self._buffer_start_seqs.get(layer_idx)
+            if buf_start is not None and buf_start > state.seq_len:        # the cache was trimmed
+                self._buffer_start_seqs[layer_idx] = state.seq_len
+                self._buffer_counts[layer_idx] = 0
+
+        already_stored = state.seq_len == cache_len       # the fused attention path stored the token
+        new_k = keys[:, :, -q_len:, :]
+        new_v = values[:, :, -q_len:, :]
+        if self.buffer_size > 0:
+            if not already_stored:
+                state.append_all_exact(new_k, new_v)
+            if q_len > 1:
+                # a multi-token call after the prefill is prompt text (e.g. the question): it stays
+                # exact and out of reach of the flush
+                self._buffer_start_seqs[layer_idx] = state.seq_len
+                self._attach(cache, layer_idx, module, state)
+                return output
+            self._buffer_counts[layer_idx] = self._buffer_counts.get(layer_idx, 0) + q_len
+            if self._buffer_counts[layer_idx] >= self.buffer_size:
+                self._flush_decode_buffer(state, layer_idx, cache, module, hidden_states)
+                return output
+            self._attach(cache, layer_idx, module, state)
+            return output
+
+        batch_bits = []
+        for b in range(keys.shape[0]):
+            h_batch = hidden_states[b:b + 1]
+            if q_len == 1:
+                scores = self._score_decode(new_k[b, :, 0, :], new_v[b, :, 0, :], layer_idx, module=module,
+                                            hidden_states=h_batch).unsqueeze(-1)
+            else:
+                scores = self._score_prefill(new_k[b], new_v[b], layer_idx, module=module, hidden_states=h_batch)
+            batch_bits.append(scores_to_bits(scores, self._decode_bit_levels))
+        bits = torch.stack(batch_bits, dim=0).to(dtype=torch.int32, device=keys.device)
+        state.append(new_k, new_v, bits)
+        self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True)
+        return output
+
+    # ------------------------------------------------------------------ flush
+    def _flush_decode_buffer(self, state, layer_idx: int, cache, module: nn.Module,
+                             hidden_states: Optional[torch.Tensor] = None) -> None:
+        """Score the buffered (exact) decode tokens with the current query and re-store them at the
+        levels the budget gives them."""
+        buffer_start = self._buffer_start_seqs.get(layer_idx)
+        if buffer_start is None:
+            self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True)
+            return
+        positions, buf_keys, buf_values = state.get_buffer_tokens(buffer_start)
+        if positions.shape[0] == 0:
+            self._buffer_start_seqs[layer_idx] = state.seq_len
+            self._buffer_counts[layer_idx] = 0
+            self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True)
+            return
+
+        attn = self._flush_attention(module, hidden_states, buf_keys, positions, state)
+        if attn is not None and self.scorer is not None:
+            # tokens are ordered (batch, head, position) with the same count in every (batch, head)
+            B, H = state.batch_size, state.num_heads
+            n_buf = positions.shape[0] // (B * H)
+            scores = torch.empty_like(attn, dtype=torch.float32)
+            kb = buf_keys.reshape(B, H, n_buf, -1)
+            vb = buf_values.reshape(B, H, n_buf, -1)
+            ab = attn.reshape(B, H, n_buf)
+            for b in range(B):
+                scores.view(B, H, n_buf)[b] = self.scorer.score_with_attn(kb[b], vb[b], ab[b], module=module).float()
+        elif attn is not None:
+            scores = attn.pow(2) * buf_values.float().pow(2).sum(-1)
+        else:
+            scores = buf_keys.float().pow(2).sum(-1) + buf_values.float().pow(2).sum(-1)
+
+        lo, hi = scores.min(), scores.max()
+        if hi - lo > 1e-8:
+            scores = (scores - lo) / (hi - lo)
+        else:
+            scores = torch.full_like(scores, 0.5)
+
+        levels = self._decode_bit_levels
+        allowed = set(levels)
+        bits = None
+        if self.ratios is not None:
+            pairs = [(b, r) for b, r in zip(self.bit_levels, self.ratios) if b in allowed]
+            if pairs:
+                flush_levels, flush_ratios = zip(*pairs)
+                bits = ratio_scores_to_bits(scores, tuple(flush_levels), tuple(flush_ratios))
+        elif self.target_avg_bits is not None:
+            bits = self._allocate_bits_via_cached_ratios(scores, positions, state.num_heads, layer_idx, allowed)
+            if bits is None:
+                eps = self._ensure_epsilon(scores.device)
+                bits = optimal_scores_to_bits(
+                    scores, levels, self.target_avg_bits, {b: eps.get(b, 0.0) for b in levels},
+                    eviction_cost=self.eviction_cost, n_outlier=self.n_outlier_channels,
+                    head_dim=self._head_dim or 128, outlier_min_bits=self.outlier_min_bits,
+                    above_target_alpha=self.above_target_alpha)
+        if bits is None:
+            bits = scores_to_bits(scores, levels)
+
+        state.flush_buffer(buffer_start, bits)
+        self._buffer_start_seqs[layer_idx] = state.seq_len
+        self._buffer_counts[layer_idx] = 0
+        self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True)
+
+    @torch.no_grad()
+    def _flush_attention(self, module: nn.Module, hidden_states, buf_keys: torch.Tensor,
+                         positions: torch.Tensor, state) -> Optional[torch.Tensor]:
+        """Attention weights [N_buf] of the current query (GQA mean, RoPE at the last position) over
+        the buffered keys, softmax within each (batch, head); None if the query cannot be formed."""
+        if hidden_states is None or not hasattr(module, "layer_idx"):
+            return None
+        try:
+            q = _get_query_states(module, hidden_states)                    # [B, Hq, q, d]
+        except (AttributeError, NotImplementedError, ValueError):
+            return None
+        rotary_emb = getattr(module, "rotary_emb", None)
+        if rotary_emb is not None:
+            pos_ids = torch.arange(state.seq_len - 1, state.seq_len, device=q.device).unsqueeze(0)
+            cos, sin = _aligned_rotary_outputs(rotary_emb, q, pos_ids)
+            q = _apply_rotary_pos_emb_q(q, cos, sin)
+        B, Hq, _, d = q.shape
+        H = state.num_heads
+        q_kv = q[:, :, -1, :].reshape(B, H, Hq // H, d).mean(dim=2)          # [B, H, d]
+        n_buf = positions.shape[0] // (B * H)
+        if n_buf * B * H != positions.shape[0]:
+            return None
+        keys = buf_keys.reshape(B, H, n_buf, d)
+        logits = (q_kv.unsqueeze(2) * keys).sum(-1) / math.sqrt(d)           # [B, H, n_buf]
+        return torch.softmax(logits, dim=-1).reshape(-1)
+
+    @contextlib.contextmanager
+    def __call__(self, model):
+        self._states, self._buffer_counts, self._buffer_start_seqs = {}, {}, {}
+        try:
+            with super().__call__(model):
+                yield
+        finally:
+            self._states, self._buffer_counts, self._buffer_start_seqs = {}, {}, {}

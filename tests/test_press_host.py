@@ -1,0 +1,99 @@
+"""CPU: host logic of the press classes and the attention patch (no kernels run)."""
+import numpy as np
+import pytest
+import torch
+
+
+def _scorer():
+    from kvquant import RiskScorer
+    return RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
+
+
+def test_package_exports_reference_names():
+    import kvquant
+    for name in ("scores_to_bits", "ratio_scores_to_bits", "optimal_scores_to_bits", "calibrate_epsilon",
+                 "effective_bits", "DEFAULT_BIT_LEVELS", "BaseScorer", "ExpectedAttentionScorer", "RiskScorer",
+                 "TurboQuantBackendPress", "TurboQuantPerTokenPress", "TurboQuantPerTokenBackendPress"):
+        assert hasattr(kvquant, name), name
+
+
+def test_constructor_errors_follow_reference():
+    from kvquant import TurboQuantPerTokenBackendPress, TurboQuantPerTokenPress
+    with pytest.raises(ValueError, match="explicit scorer"):
+        TurboQuantPerTokenPress()
+    with pytest.raises(ValueError, match="below 2"):
+        TurboQuantPerTokenBackendPress(scorer=_scorer(), bit_levels=(0, 1, 2, 16), key_quantizer="prod")
+    p = TurboQuantPerTokenBackendPress(scorer=_scorer(), bit_levels=(0, 2, 3, 4, 8, 16), key_quantizer="mse",
+                                       value_quantizer="mse", target_avg_bits=2.0)
+    assert p._decode_bit_levels == (2, 3, 4, 8, 16) and p.decode_quant and p.buffer_size == 128
+    q = TurboQuantPerTokenBackendPress(scorer=_scorer(), bit_levels=(0, 2, 16), key_quantizer="mse",
+                                       value_quantizer="mse", allow_decode_eviction=True)
+    assert q._decode_bit_levels == (0, 2, 16)
+
+
+def test_sink_mask_and_uniform_partition():
+    from kvquant import TurboQuantPerTokenPress
+    p = TurboQuantPerTokenPress(scorer=_scorer(), bit_levels=(0, 2, 4, 16), sink_tokens=4, value_quantizer="mse")
+    m = p._build_sink_mask(3, 10, "cpu")
+    assert m.shape == (3, 10) and m[:, :4].all() and not m[:, 4:].any()
+    assert TurboQuantPerTokenPress(scorer=_scorer(), value_quantizer="mse")._build_sink_mask(2, 5, "cpu") is None
+    s = torch.tensor([[0.0, 0.1, 0.3, 0.6, 0.9, 1.0, 0.2, 0.4, 0.7, 0.99]]).repeat(3, 1)
+    bits = p._compute_bits(s, m)               # neither ratios nor target: uniform partition, sinks 16
+    assert bits[:, :4].eq(16).all()
+    assert bits[0, 4:].tolist() == [16, 16, 0, 2, 4, 16]
+
+
+def test_search_hyperplane_gives_negative_logits():
+    from kvquant.attention_patch import search_hyperplane
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(6, 12, 128, generator=g) + 0.5
+    y = search_hyperplane(x)
+    assert y.shape == (6, 128)
+    logits = torch.einsum("nmd,nd->nm", x, y)
+    assert (logits < -1e3).all()
+
+
+def test_group_and_scalar_value_quantisers():
+    from kvquant.press import _qd_scalar, _qd_values_group
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(5, 128, generator=g)
+    for b in (2, 4, 8):
+        y = _qd_values_group(x, b, 32)
+        xg = x.numpy().reshape(5, 4, 32)
+        lo, hi = xg.min(-1, keepdims=True), xg.max(-1, keepdims=True)
+        sc = np.maximum((hi - lo) / (2 ** b - 1), 1e-10)
+        want = (np.clip(np.round((xg - lo) / sc), 0, 2 ** b - 1) * sc + lo).reshape(5, 128)
+        assert np.allclose(y.numpy(), want, atol=1e-6)
+        assert (y - x).abs().max() <= (hi - lo).max() / (2 ** b - 1) * 0.5 + 1e-6
+        z = _qd_scalar(x, b)
+        assert (z - x).abs().max() <= (x.amax(-1) - x.amin(-1)).max() / (2 ** b - 1) * 0.5 + 1e-6
+    assert torch.equal(_qd_values_group(x[:, :100], 2, 32), _qd_scalar(x[:, :100], 2))   # d not divisible: per-vector
+
+
+def test_observed_ratios_and_cached_allocation():
+    from kvquant import TurboQuantPerTokenBackendPress
+    p = TurboQuantPerTokenBackendPress(scorer=_scorer(), bit_levels=(0, 2, 4, 16), key_quantizer="mse",
+                                       value_quantizer="mse", target_avg_bits=2.0, sink_tokens=4, buffer_size=8)
+    T = 4 + 40 + 8
+    bits = torch.full((1, 2, T), 16, dtype=torch.int32)
+    bits[0, 0, 4:44] = torch.tensor([0] * 10 + [2] * 20 + [4] * 10)
+    bits[0, 1, 4:44] = torch.tensor([2] * 30 + [4] * 10)
+    p._record_observed_ratios(3, bits)
+    assert p._observed_ratios[(3, 0)] == ((0, 0.25), (2, 0.5), (4, 0.25))
+    assert p._observed_ratios[(3, 1)] == ((2, 0.75), (4, 0.25))
+    # flush allocation from the cached ratios, eviction not allowed at decode: level 0 dropped, rest renormalised
+    n = 12
+    pos = torch.stack([torch.zeros(2 * n, dtype=torch.long), torch.arange(2).repeat_interleave(n),
+                       torch.arange(n).repeat(2)], dim=-1)
+    scores = torch.linspace(0, 1, 2 * n)
+    out = p._allocate_bits_via_cached_ratios(scores, pos, 2, 3, {2, 4, 16})
+    assert out[:n].tolist() == [2] * 8 + [4] * 4          # 2/3 and 1/3 of 12
+    assert out[n:].tolist() == [2] * 9 + [4] * 3
+    assert p._allocate_bits_via_cached_ratios(scores, pos, 2, 5, {2, 4, 16}) is None     # layer without a record
+
+
+def test_backend_press_rejects_unbuilt_quantisers():
+    from kvquant import TurboQuantBackendPress
+    with pytest.raises(NotImplementedError):
+        TurboQuantBackendPress()                       # min-max values by default
+    TurboQuantBackendPress(key_quantizer="mse", value_quantizer="mse")
