@@ -2,12 +2,19 @@
 // with lambda found by bisection so that the mean of the chosen widths meets the row's budget,
 // then close the remaining gap by moving the lowest- (or highest-) scored tokens one level.
 //
-// The search is a fixed sequence of 74 evaluations (1 at lambda = 1, up to 8 widenings of the
-// bracket, 64 halvings, 1 final), each a launch that histograms the chosen levels of all rows.
-// The workgroup that finishes an evaluation last turns the histogram into the average and
-// advances that row's bracket for the next launch; nothing ever waits on another workgroup
-// and the host is never consulted.  All counts are integers, so the result does not depend
-// on the order in which workgroups run.
+// The search is the fixed sequence the host formulation runs: lambda = 1, up to 8 widenings of the
+// bracket (x10 each), 64 halvings, one final assignment.  It is evaluated in 18 launches:
+//   launch 0      all nine widening candidates 1, 10, .. 1e8 at once;
+//   launch 1..16  four halvings each: the 15 midpoints the next four steps can reach form a binary
+//                 tree that is known in advance, so one pass over the scores evaluates them all;
+//   launch 17     the final lambda, which also records the chosen level of every token.
+// Every workgroup writes its partial bit sums; the workgroup that finishes last (found by an
+// atomic ticket) adds them up, walks the bracket and prepares the next launch's candidates.
+// Nothing ever waits on another workgroup and the host is never consulted.  All sums are
+// integers, so the result does not depend on the order in which workgroups run.
+// The partial sums travel as device-scope atomic stores and loads (they go to the memory side of
+// the per-XCD L2s), ordered before the ticket by waiting for the stores to complete; a device-scope
+// fence instead would write back the whole L2 from every workgroup.
 //
 // Arithmetic is kept exactly as the host formulation it replaces: fp32 products rounded
 // separately and then added (no fused multiply-add), lambda rounded to fp32 before use, the
@@ -15,16 +22,22 @@
 #include "common.h"
 
 #define NLV ODMKV_MAX_LEVELS
-#define ITERS 74
-#define IT_FINAL 73
-#define HIST_TPT 8                       // tokens per thread in an evaluation
-#define HIST_TOKENS (256 * HIST_TPT)
+#define STEPS 4                               // halvings per launch
+#define NCAND ((1 << STEPS) - 1)              // 15 tree nodes, numbered 1..15
+#define N_WIDEN 9
+#define N_HALVE_LAUNCH (64 / STEPS)
+#define N_LAUNCH (1 + N_HALVE_LAUNCH + 1)
+#define L_FINAL (N_LAUNCH - 1)
+#define SLOTS 16                              // partial sums per workgroup
+#define EV_THREADS 512
+#ifndef EV_TPT
+#define EV_TPT 4                              // tokens per thread in an evaluation
+#endif
+#define EV_TOKENS (EV_THREADS * EV_TPT)
+#define CAND_MAX 16                           // repair moves of at most this many tokens take the short path
 
 struct RowState {
     double lo, hi, target, gap, lam;
-    double avg_hi;
-    float lam32;
-    int skip_until;          // evaluations with index < skip_until do nothing
     int n_active;
     unsigned int max_finite; // bit pattern
     int has_finite, has_nonfinite;
@@ -34,16 +47,16 @@ struct RowState {
 struct AllocArgs {
     const float* scores;
     const uint8_t* sink_mask;
-    int rows, n, period, n_sink, sink_bits, K;
+    int rows, n, period, n_sink, sink_bits, K, n_chunks;
     float eps[NLV];
     float bitsf[NLV];
     int nominal[NLV];
-    const double* target;    // device, [rows]
-    float* s_clean;          // [rows, n]
-    uint8_t* chosen;         // [rows, n]
-    unsigned int* hist;      // [rows, ITERS, NLV]
-    unsigned int* tickets;   // [rows, ITERS]
-    RowState* state;         // [rows]
+    const double* target;          // device, [rows]
+    uint8_t* chosen;               // [rows, n]
+    unsigned int* partial;         // [rows, n_chunks, SLOTS]
+    unsigned int* tickets;         // [rows, N_LAUNCH]
+    unsigned long long* cand;      // [rows, n_chunks, CAND_MAX]
+    RowState* state;               // [rows]
     int32_t* bits_out;
     int32_t* level_counts;
     double* lambda_out;
@@ -54,26 +67,49 @@ __device__ static inline bool is_sink(const AllocArgs& a, int row, int i) {
     return a.n_sink > 0 && (i % a.period) < a.n_sink;
 }
 
+// torch's clamp(min=0) / non-finite patch / nan_to_num, in that order
+__device__ static inline float clean_score(float v, bool patch, float top) {
+    if (!(v != v)) v = fmaxf(v, 0.0f);                // clamp(min=0) keeps NaN
+    if (patch && !isfinite(v)) v = top;
+    if (v != v) v = 0.0f;
+    else if (v == INFINITY) v = 3.4028234663852886e38f;
+    return v;
+}
+
+struct Cleaner {
+    bool patch;
+    float top;
+    __device__ inline Cleaner(const RowState& st) : patch(st.has_finite && st.has_nonfinite), top(__uint_as_float(st.max_finite)) {}
+    __device__ inline float operator()(float v) const { return clean_score(v, patch, top); }
+};
+
+__device__ static inline int wave_sum_int(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+
 // ---- clear counters, set up the bracket ----
 __global__ void alloc_init_kernel(AllocArgs a) {
     const int row = blockIdx.x;
-    for (int e = threadIdx.x; e < ITERS * NLV; e += blockDim.x) a.hist[(size_t)row * ITERS * NLV + e] = 0u;
-    for (int e = threadIdx.x; e < ITERS; e += blockDim.x) a.tickets[(size_t)row * ITERS + e] = 0u;
+    for (int e = threadIdx.x; e < N_LAUNCH; e += blockDim.x) a.tickets[(size_t)row * N_LAUNCH + e] = 0u;
     if (a.level_counts && threadIdx.x < a.K) a.level_counts[row * a.K + threadIdx.x] = 0;
     if (threadIdx.x == 0) {
         RowState& st = a.state[row];
         double t = a.target[row];                    // clamp the budget into the level range
         t = fmin(t, (double)a.nominal[a.K - 1]);
         t = fmax(t, (double)a.nominal[0]);
-        st.lo = 0.0; st.hi = 1.0; st.target = t; st.gap = 0.0; st.lam = 1.0; st.avg_hi = 0.0;
-        st.lam32 = 1.0f; st.skip_until = 0; st.n_active = 0; st.max_finite = 0u;
-        st.has_finite = 0; st.has_nonfinite = 0;
+        st.lo = 0.0; st.hi = 1.0; st.target = t; st.gap = 0.0; st.lam = 1.0;
+        st.n_active = 0; st.max_finite = 0u; st.has_finite = 0; st.has_nonfinite = 0;
         for (int k = 0; k < NLV; ++k) st.final_hist[k] = 0;
     }
 }
 
 // ---- what the sanitiser needs to know about a row ----
-__global__ __launch_bounds__(256) void alloc_scan_kernel(AllocArgs a) {
+#define SC_THREADS 1024
+#define SC_TPT 8
+#define SC_TOKENS (SC_THREADS * SC_TPT)
+__global__ __launch_bounds__(SC_THREADS) void alloc_scan_kernel(AllocArgs a) {
     __shared__ unsigned int smax;
     __shared__ int sfin, snon, sact;
     const int row = blockIdx.y;
@@ -81,13 +117,13 @@ __global__ __launch_bounds__(256) void alloc_scan_kernel(AllocArgs a) {
     __syncthreads();
     unsigned int mx = 0u;
     int fin = 0, non = 0, act = 0;
-    const int base = blockIdx.x * HIST_TOKENS;
-    for (int e = 0; e < HIST_TPT; ++e) {
-        const int i = base + e * 256 + threadIdx.x;
+    const int base = blockIdx.x * SC_TOKENS;
+    for (int e = 0; e < SC_TPT; ++e) {
+        const int i = base + e * SC_THREADS + threadIdx.x;
         if (i < a.n && !is_sink(a, row, i)) {
             ++act;
             float v = a.scores[(size_t)row * a.n + i];
-            if (!(v != v)) v = fmaxf(v, 0.0f);          // clamp(min=0) keeps NaN
+            if (!(v != v)) v = fmaxf(v, 0.0f);
             if (isfinite(v)) { fin = 1; mx = max(mx, __float_as_uint(v)); }
             else non = 1;
         }
@@ -106,123 +142,290 @@ __global__ __launch_bounds__(256) void alloc_scan_kernel(AllocArgs a) {
     }
 }
 
-__global__ __launch_bounds__(256) void alloc_clean_kernel(AllocArgs a) {
-    const int row = blockIdx.y;
-    const RowState& st = a.state[row];
-    const bool patch = st.has_finite && st.has_nonfinite;
-    const float top = __uint_as_float(st.max_finite);
-    const int base = blockIdx.x * HIST_TOKENS;
-    for (int e = 0; e < HIST_TPT; ++e) {
-        const int i = base + e * 256 + threadIdx.x;
-        if (i < a.n) {
-            float v = a.scores[(size_t)row * a.n + i];
-            if (!(v != v)) v = fmaxf(v, 0.0f);
-            if (patch && !isfinite(v)) v = top;
-            if (v != v) v = 0.0f;                         // nan_to_num
-            else if (v == INFINITY) v = 3.4028234663852886e38f;
-            a.s_clean[(size_t)row * a.n + i] = v;
-        }
+// lambda candidates of the four halvings that follow bracket (lo, hi): node 1 is the midpoint;
+// from node m the search moves to 2m when the average is within budget (hi = mid), else to 2m + 1
+__device__ static inline float tree_candidate(double lo, double hi, int node) {
+    int depth = 31 - __clz(node);
+    for (int d = depth - 1; d >= 0; --d) {
+        const double mid = (lo + hi) * 0.5;
+        if ((node >> d) & 1) lo = mid; else hi = mid;
     }
+    return (float)((lo + hi) * 0.5);
 }
 
-__device__ static inline int pick_level(const AllocArgs& a, float s, float lam32) {
-    int best = 0;
-    float bc = __fadd_rn(__fmul_rn(s, a.eps[0]), __fmul_rn(lam32, a.bitsf[0]));
-#pragma unroll
-    for (int k = 1; k < NLV; ++k) {
-        if (k < a.K) {
-            const float c = __fadd_rn(__fmul_rn(s, a.eps[k]), __fmul_rn(lam32, a.bitsf[k]));
-            if (c < bc) { bc = c; best = k; }
-        }
-    }
-    return best;
-}
-
-// the last workgroup of evaluation `it` advances the row's search state
-__device__ static void advance(const AllocArgs& a, int row, int it) {
+// the last workgroup of launch L: sums[] holds the row's totals; advance the search
+__device__ static void advance(const AllocArgs& a, int row, int L, const unsigned int* sums) {
     RowState& st = a.state[row];
-    unsigned long long S = 0ull;
-    unsigned int h[NLV];
-    for (int k = 0; k < a.K; ++k) {
-        h[k] = atomicAdd(&a.hist[((size_t)row * ITERS + it) * NLV + k], 0u);
-        S += (unsigned long long)h[k] * (unsigned long long)a.nominal[k];
-    }
-    const float avg32 = (float)S / (float)st.n_active;
-    const double avg = (double)avg32;
-    if (it <= 8) {                      // bracket widening: lambda = hi
-        st.avg_hi = avg;
-        if (avg > st.target && st.hi < 1e8 && it < 8) {
-            st.hi *= 10.0;
-            st.lam = st.hi;
-            st.lam32 = (float)st.hi;
-            st.skip_until = it + 1;
-        } else {
-            st.lam = (st.lo + st.hi) * 0.5;
-            st.lam32 = (float)st.lam;
-            st.skip_until = 9;
+    const float nf = (float)st.n_active;
+    if (L == 0) {
+        double hi = 1.0;
+        int j = 0;
+        double avg_hi = (double)((float)sums[0] / nf);
+        while (avg_hi > st.target && hi < 1e8) {
+            hi *= 10.0;
+            ++j;
+            avg_hi = (double)((float)sums[j] / nf);
         }
-    } else if (it < IT_FINAL) {         // halving
-        if (avg > st.target) st.lo = st.lam; else st.hi = st.lam;
-        st.lam = (st.lo + st.hi) * 0.5;
-        st.lam32 = (float)st.lam;
-        st.skip_until = it + 1;
-    } else {                            // final assignment done
+        st.lo = 0.0; st.hi = hi;
+    } else if (L < L_FINAL) {
+        double lo = st.lo, hi = st.hi;
+        int node = 1;
+        for (int s = 0; s < STEPS; ++s) {
+            const double mid = (lo + hi) * 0.5;
+            const double avg = (double)((float)sums[node] / nf);
+            if (avg > st.target) { lo = mid; node = 2 * node + 1; } else { hi = mid; node = 2 * node; }
+        }
+        st.lo = lo; st.hi = hi;
+    } else {
+        unsigned long long S = 0ull;
+        for (int k = 0; k < a.K; ++k) {
+            S += (unsigned long long)sums[k] * (unsigned long long)a.nominal[k];
+            st.final_hist[k] = (int)sums[k];
+        }
+        const double avg = (double)((float)S / nf);
         st.gap = (avg - st.target) * (double)st.n_active;
-        for (int k = 0; k < a.K; ++k) st.final_hist[k] = (int)h[k];
         if (a.lambda_out) a.lambda_out[row] = st.lam;
+        return;
     }
+    if (L + 1 == L_FINAL) st.lam = (st.lo + st.hi) * 0.5;
 }
 
-__global__ __launch_bounds__(256) void alloc_eval_kernel(AllocArgs a, int it) {
-    __shared__ unsigned int lh[NLV];
-    __shared__ int is_last;
-    const int row = blockIdx.y;
-    const RowState& st = a.state[row];
-    if (it < st.skip_until || st.n_active == 0) return;
-    if (threadIdx.x < NLV) lh[threadIdx.x] = 0u;
-    __syncthreads();
-    const float lam32 = st.lam32;
-    unsigned int cnt[NLV];
+// the lambda that slot c of launch L evaluates (slots a launch does not use evaluate lambda = 0 and are ignored)
+__device__ static inline float candidate(const RowState& st, int L, int c) {
+    if (L == 0) {
+        double h = 1.0;
+        for (int j = 0; j < c; ++j) h *= 10.0;
+        return c < N_WIDEN ? (float)h : 0.0f;
+    }
+    if (L == L_FINAL) return (float)((st.lo + st.hi) * 0.5);
+    return c >= 1 ? tree_candidate(st.lo, st.hi, c) : 0.0f;
+}
+
+// sums of 16-bit fields over the wave: on return, lanes with (lane & 7) == 0 hold packed pair
+// number (lane >> 3) in v[0]
+__device__ static inline void reduce_scatter8(unsigned int (&v)[8], int lane) {
 #pragma unroll
-    for (int k = 0; k < NLV; ++k) cnt[k] = 0u;
-    const int base = blockIdx.x * HIST_TOKENS;
-    for (int e = 0; e < HIST_TPT; ++e) {
-        const int i = base + e * 256 + threadIdx.x;
-        if (i < a.n && !is_sink(a, row, i)) {
-            const int k = pick_level(a, a.s_clean[(size_t)row * a.n + i], lam32);
+    for (int half = 4; half >= 1; half >>= 1) {
+        const int o = half * 8;                 // 32, 16, 8
+        const bool upper = (lane & o) != 0;
 #pragma unroll
-            for (int j = 0; j < NLV; ++j) cnt[j] += (k == j);
-            if (it == IT_FINAL) a.chosen[(size_t)row * a.n + i] = (uint8_t)k;
+        for (int i = 0; i < half; ++i) {
+            const unsigned int send = upper ? v[i] : v[i + half];
+            const unsigned int keep = upper ? v[i + half] : v[i];
+            v[i] = keep + (unsigned int)__shfl_xor((int)send, o, WAVE);
         }
     }
 #pragma unroll
-    for (int k = 0; k < NLV; ++k)
-        if (cnt[k]) atomicAdd(&lh[k], cnt[k]);
+    for (int o = 4; o > 0; o >>= 1) v[0] += (unsigned int)__shfl_xor((int)v[0], o, WAVE);
+}
+
+template <int K>
+__global__ __launch_bounds__(EV_THREADS) void alloc_eval_kernel(AllocArgs a, int L) {
+    __shared__ __align__(16) float lamb[SLOTS][NLV];     // fl32(lambda_c * b_k)
+    __shared__ int lsum[SLOTS];
+    __shared__ unsigned int tot[SLOTS];
+    __shared__ int is_last;
+    const int row = blockIdx.y, tid = threadIdx.x;
+    const RowState& st = a.state[row];
+    if (st.n_active == 0) return;
+    if (tid < SLOTS * NLV) {
+        const int c = tid / NLV, k = tid % NLV;
+        lamb[c][k] = __fmul_rn(candidate(st, L, c), a.bitsf[k]);
+    }
+    if (tid < SLOTS) lsum[tid] = 0;
     __syncthreads();
-    if (threadIdx.x < a.K && lh[threadIdx.x])
-        atomicAdd(&a.hist[((size_t)row * ITERS + it) * NLV + threadIdx.x], lh[threadIdx.x]);
-    __threadfence();
+
+    const Cleaner clean(st);
+    float se[EV_TPT][K];
+    bool active[EV_TPT];
+    const int base = blockIdx.x * EV_TOKENS;
+#pragma unroll
+    for (int e = 0; e < EV_TPT; ++e) {
+        const int i = base + e * EV_THREADS + tid;
+        active[e] = i < a.n && !is_sink(a, row, i);
+        const float s = active[e] ? clean(a.scores[(size_t)row * a.n + i]) : 0.0f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) se[e][k] = __fmul_rn(s, a.eps[k]);
+    }
+
+    if (L != L_FINAL) {
+        unsigned int acc[8];
+#pragma unroll
+        for (int p = 0; p < 8; ++p) acc[p] = 0u;
+#pragma unroll
+        for (int c = 0; c < SLOTS; ++c) {
+            const float4 l0 = *reinterpret_cast<const float4*>(&lamb[c][0]);
+            const float4 l1 = *reinterpret_cast<const float4*>(&lamb[c][4]);
+            const float lb[NLV] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
+            unsigned int sum = 0u;
+#pragma unroll
+            for (int e = 0; e < EV_TPT; ++e) {
+                float bc = __fadd_rn(se[e][0], lb[0]);
+                int bn = a.nominal[0];
+#pragma unroll
+                for (int k = 1; k < K; ++k) {
+                    const float cst = __fadd_rn(se[e][k], lb[k]);
+                    if (cst < bc) { bc = cst; bn = a.nominal[k]; }
+                }
+                sum += active[e] ? (unsigned int)bn : 0u;
+            }
+            acc[c >> 1] += sum << (16 * (c & 1));           // at most 64 lanes * EV_TPT * 16 per field
+        }
+        reduce_scatter8(acc, tid & 63);
+        if ((tid & 7) == 0) {
+            const int p = (tid & 63) >> 3;
+            if (acc[0] & 0xffffu) atomicAdd(&lsum[2 * p], (int)(acc[0] & 0xffffu));
+            if (acc[0] >> 16) atomicAdd(&lsum[2 * p + 1], (int)(acc[0] >> 16));
+        }
+    } else {
+        int cnt[NLV];
+#pragma unroll
+        for (int k = 0; k < NLV; ++k) cnt[k] = 0;
+#pragma unroll
+        for (int e = 0; e < EV_TPT; ++e) {
+            float bc = __fadd_rn(se[e][0], lamb[0][0]);
+            int best = 0;
+#pragma unroll
+            for (int k = 1; k < K; ++k) {
+                const float cst = __fadd_rn(se[e][k], lamb[0][k]);
+                if (cst < bc) { bc = cst; best = k; }
+            }
+            if (active[e]) {
+                a.chosen[(size_t)row * a.n + base + e * EV_THREADS + tid] = (uint8_t)best;
+#pragma unroll
+                for (int k = 0; k < NLV; ++k) cnt[k] += (best == k);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < NLV; ++k) {
+            const int s = wave_sum_int(cnt[k]);
+            if ((tid & 63) == 0 && s) atomicAdd(&lsum[k], s);
+        }
+    }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        const unsigned int t = atomicAdd(&a.tickets[(size_t)row * ITERS + it], 1u);
+    unsigned int* mine = a.partial + ((size_t)row * a.n_chunks + blockIdx.x) * SLOTS;
+    if (tid < SLOTS) {
+        __hip_atomic_store(mine + tid, (unsigned int)lsum[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0);            // the stores have reached the memory side
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned int t = __hip_atomic_fetch_add(&a.tickets[(size_t)row * N_LAUNCH + L], 1u, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT);
         is_last = (t == gridDim.x - 1);
     }
     __syncthreads();
-    if (is_last && threadIdx.x == 0) {
-        __threadfence();
-        advance(a, row, it);
+    if (!is_last) return;
+    if (tid < SLOTS) tot[tid] = 0u;
+    __syncthreads();
+    {
+        // 16 threads per slot walk the chunks
+        const int slot = tid & (SLOTS - 1), part = tid / SLOTS;
+        unsigned int s = 0u;
+        const unsigned int* p = a.partial + (size_t)row * a.n_chunks * SLOTS;
+        for (int w = part; w < a.n_chunks; w += EV_THREADS / SLOTS)
+            s += __hip_atomic_load(p + (size_t)w * SLOTS + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (s) atomicAdd(&tot[slot], s);
+    }
+    __syncthreads();
+    if (tid == 0) advance(a, row, L, tot);
+}
+
+// ---- budget repair -------------------------------------------------------------------------------
+// The host formulation sorts the row by score (stable) and, walking the level pairs, moves the
+// n lowest-scored tokens of the upper level down (over budget) or the n highest-scored tokens of the
+// lower level up (under budget).  Equivalent without a sort: among the tokens at level `from`,
+// take the n smallest (largest) 64-bit keys (score bits, index).
+struct Move { int from, to, want, i; bool lowest; double delta; };
+
+// the first level pair, at or after pair index i in walking order, that moves tokens
+__device__ static inline bool next_move(const AllocArgs& a, const int* hist, double gap_abs, bool over, int i, Move& m) {
+    for (; over ? i < a.K - 1 : i >= 0; i += over ? 1 : -1) {
+        const double delta = (double)a.bitsf[i + 1] - (double)a.bitsf[i];
+        if (delta <= 0) continue;
+        const int have = over ? hist[i + 1] : hist[i];
+        const int n = min(have, (int)(gap_abs / delta + 0.5));
+        if (n <= 0) continue;
+        m.from = over ? i + 1 : i; m.to = over ? i : i + 1; m.want = n; m.i = i; m.lowest = over; m.delta = delta;
+        return true;
+    }
+    return false;
+}
+
+__device__ static inline unsigned long long token_key(float s, int i, bool lowest) {
+    // + 1 keeps both k and ~k away from the "no key" value
+    const unsigned long long k = (((unsigned long long)__float_as_uint(s) << 32) | (unsigned int)i) + 1ull;
+    return lowest ? k : ~k;            // always select minima
+}
+__device__ static inline unsigned int key_index(unsigned long long g, bool lowest) {
+    return (unsigned int)(((lowest ? g : ~g) - 1ull) & 0xffffffffull);
+}
+
+__device__ static inline unsigned long long wave_min_u64(unsigned long long v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(v, o, WAVE);
+        v = other < v ? other : v;
+    }
+    return v;
+}
+
+#define KEY_NONE 0xffffffffffffffffull
+
+// `want` rounds of a workgroup-wide minimum over the keys held in registers; every selected key is
+// handed to `emit(round, key)` by thread 0 and struck from its owner's registers
+template <int NK, int NWAVES, typename F>
+__device__ static inline void select_smallest(unsigned long long (&keys)[NK], int want, unsigned long long* wbest, F emit) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    for (int r = 0; r < want; ++r) {
+        unsigned long long best = KEY_NONE;
+#pragma unroll
+        for (int e = 0; e < NK; ++e) best = keys[e] < best ? keys[e] : best;
+        const unsigned long long wb = wave_min_u64(best);
+        if (lane == 0) wbest[wave] = wb;
+        __syncthreads();
+        unsigned long long g = KEY_NONE;
+        for (int w = 0; w < NWAVES; ++w) g = wbest[w] < g ? wbest[w] : g;
+        if (g != KEY_NONE) {
+#pragma unroll
+            for (int e = 0; e < NK; ++e) keys[e] = keys[e] == g ? KEY_NONE : keys[e];
+        }
+        if (tid == 0) emit(r, g);
+        __syncthreads();
     }
 }
 
-// ---- budget repair: one workgroup per row, ordered passes over the row ----
+// per chunk: the candidates for the first move when it is small
+__global__ __launch_bounds__(EV_THREADS) void alloc_cand_kernel(AllocArgs a) {
+    __shared__ unsigned long long wbest[EV_THREADS / 64];
+    const int row = blockIdx.y, tid = threadIdx.x;
+    const RowState& st = a.state[row];
+    if (st.n_active == 0 || fabs(st.gap) <= 0.5) return;
+    const bool over = st.gap > 0;
+    Move m;
+    if (!next_move(a, st.final_hist, fabs(st.gap), over, over ? 0 : a.K - 2, m) || m.want > CAND_MAX) return;
+    const Cleaner clean(st);
+    unsigned long long keys[EV_TPT];
+    const int base = blockIdx.x * EV_TOKENS;
+#pragma unroll
+    for (int e = 0; e < EV_TPT; ++e) {
+        const int i = base + e * EV_THREADS + tid;
+        keys[e] = KEY_NONE;
+        if (i < a.n && !is_sink(a, row, i) && a.chosen[(size_t)row * a.n + i] == m.from)
+            keys[e] = token_key(clean(a.scores[(size_t)row * a.n + i]), i, m.lowest);
+    }
+    unsigned long long* out = a.cand + ((size_t)row * a.n_chunks + blockIdx.x) * CAND_MAX;
+    select_smallest<EV_TPT, EV_THREADS / 64>(keys, m.want, wbest, [&](int r, unsigned long long g) { out[r] = g; });
+}
+
 #define RB 1024
 
 // Moves `want` tokens currently at level `from` to level `to`: those with the smallest
 // (score, index) if lowest, else those with the largest.  Scores are non-negative and finite,
 // so their bit patterns order like the values.
-__device__ static void move_tokens(const AllocArgs& a, int row, int from, int to, int want, bool lowest,
-                                   unsigned int* hist256, int* scratch) {
-    const float* s = a.s_clean + (size_t)row * a.n;
+__device__ static void move_tokens(const AllocArgs& a, int row, const Cleaner& clean, int from, int to, int want,
+                                   bool lowest, unsigned int* hist256, int* scratch) {
+    const float* s = a.scores + (size_t)row * a.n;
     uint8_t* ch = a.chosen + (size_t)row * a.n;
     const int tid = threadIdx.x;
     // radix select, most significant byte first: find the key of the want-th token
@@ -234,7 +437,7 @@ __device__ static void move_tokens(const AllocArgs& a, int row, int from, int to
         __syncthreads();
         for (int i = tid; i < a.n; i += RB) {
             if (ch[i] == from && !is_sink(a, row, i)) {
-                const unsigned int key = __float_as_uint(s[i]);
+                const unsigned int key = __float_as_uint(clean(s[i]));
                 if ((key & pmask) == prefix) atomicAdd(&hist256[(key >> shift) & 0xffu], 1u);
             }
         }
@@ -265,7 +468,7 @@ __device__ static void move_tokens(const AllocArgs& a, int row, int from, int to
         __syncthreads();
         int local = 0;
         for (int i = tid; i < a.n; i += RB)
-            if (ch[i] == from && !is_sink(a, row, i) && __float_as_uint(s[i]) == prefix) ++local;
+            if (ch[i] == from && !is_sink(a, row, i) && __float_as_uint(clean(s[i])) == prefix) ++local;
         if (local) atomicAdd(&scratch[3], local);
         __syncthreads();
     }
@@ -279,7 +482,7 @@ __device__ static void move_tokens(const AllocArgs& a, int row, int from, int to
         bool member = false, tie = false, strict = false;
         if (i < a.n && ch[i] == from && !is_sink(a, row, i)) {
             member = true;
-            const unsigned int key = __float_as_uint(s[i]);
+            const unsigned int key = __float_as_uint(clean(s[i]));
             tie = key == prefix;
             strict = lowest ? key < prefix : key > prefix;
         }
@@ -299,46 +502,60 @@ __device__ static void move_tokens(const AllocArgs& a, int row, int from, int to
     }
 }
 
+// one workgroup per row: apply the first move from the chunk candidates when it is small, any other
+// move by a radix select over the row
 __global__ __launch_bounds__(RB) void alloc_repair_kernel(AllocArgs a) {
     __shared__ unsigned int hist256[256];
     __shared__ int scratch[32];
-    const int row = blockIdx.x;
+    __shared__ unsigned long long wbest[RB / 64];
+    const int row = blockIdx.x, tid = threadIdx.x;
     const RowState& st = a.state[row];
     if (st.n_active == 0) return;
     double gap = st.gap;
     if (fabs(gap) <= 0.5) return;
-    if (gap > 0) {
-        for (int i = 0; i < a.K - 1; ++i) {
-            const double delta = (double)a.bitsf[i + 1] - (double)a.bitsf[i];
-            if (delta <= 0) continue;
-            const int n_dem = min(st.final_hist[i + 1], (int)(gap / delta + 0.5));
-            if (n_dem <= 0) continue;
-            move_tokens(a, row, i + 1, i, n_dem, true, hist256, scratch);
-            gap -= n_dem * delta;
-            if (gap <= 0.5) break;
+    const bool over = gap > 0;
+    gap = fabs(gap);
+    const Cleaner clean(st);
+    int i = over ? 0 : a.K - 2;
+    Move m;
+    bool first = true;
+    while (next_move(a, st.final_hist, gap, over, i, m)) {
+        if (first && m.want <= CAND_MAX) {
+            uint8_t* ch = a.chosen + (size_t)row * a.n;
+            const unsigned long long* cand = a.cand + (size_t)row * a.n_chunks * CAND_MAX;
+            const int total = a.n_chunks * m.want;
+            if (total <= 4 * RB) {
+                unsigned long long keys[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int idx = e * RB + tid;
+                    keys[e] = idx < total ? cand[(size_t)(idx / m.want) * CAND_MAX + idx % m.want] : KEY_NONE;
+                }
+                select_smallest<4, RB / 64>(keys, m.want, wbest, [&](int, unsigned long long g) {
+                    if (g != KEY_NONE) ch[key_index(g, m.lowest)] = (uint8_t)m.to;
+                });
+            } else {
+                move_tokens(a, row, clean, m.from, m.to, m.want, m.lowest, hist256, scratch);
+            }
+        } else {
+            __syncthreads();
+            move_tokens(a, row, clean, m.from, m.to, m.want, m.lowest, hist256, scratch);
         }
-    } else {
-        gap = -gap;
-        for (int i = a.K - 2; i >= 0; --i) {
-            const double delta = (double)a.bitsf[i + 1] - (double)a.bitsf[i];
-            if (delta <= 0) continue;
-            const int n_pro = min(st.final_hist[i], (int)(gap / delta + 0.5));
-            if (n_pro <= 0) continue;
-            move_tokens(a, row, i, i + 1, n_pro, false, hist256, scratch);
-            gap -= n_pro * delta;
-            if (gap <= 0.5) break;
-        }
+        first = false;
+        gap -= m.want * m.delta;
+        if (gap <= 0.5) break;
+        i = m.i + (over ? 1 : -1);
     }
 }
 
-__global__ __launch_bounds__(256) void alloc_write_kernel(AllocArgs a, int single_level) {
+__global__ __launch_bounds__(EV_THREADS) void alloc_write_kernel(AllocArgs a, int single_level) {
     __shared__ int lh[NLV];
     const int row = blockIdx.y;
     if (threadIdx.x < NLV) lh[threadIdx.x] = 0;
     __syncthreads();
-    const int base = blockIdx.x * HIST_TOKENS;
-    for (int e = 0; e < HIST_TPT; ++e) {
-        const int i = base + e * 256 + threadIdx.x;
+    const int base = blockIdx.x * EV_TOKENS;
+    for (int e = 0; e < EV_TPT; ++e) {
+        const int i = base + e * EV_THREADS + threadIdx.x;
         if (i < a.n) {
             int out;
             if (is_sink(a, row, i)) out = a.sink_bits;
@@ -355,15 +572,16 @@ __global__ __launch_bounds__(256) void alloc_write_kernel(AllocArgs a, int singl
         atomicAdd(&a.level_counts[row * a.K + threadIdx.x], lh[threadIdx.x]);
 }
 
-struct AllocLayout { size_t s_clean, chosen, hist, tickets, state, total; };
+struct AllocLayout { size_t chosen, partial, tickets, cand, state, total; };
 static AllocLayout alloc_layout(int rows, int n) {
     AllocLayout L;
+    const size_t chunks = ((size_t)n + EV_TOKENS - 1) / EV_TOKENS;
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes, 256); return o; };
-    L.s_clean = take((size_t)rows * n * sizeof(float));
     L.chosen = take((size_t)rows * n);
-    L.hist = take((size_t)rows * ITERS * NLV * sizeof(unsigned int));
-    L.tickets = take((size_t)rows * ITERS * sizeof(unsigned int));
+    L.partial = take((size_t)rows * chunks * SLOTS * sizeof(unsigned int));
+    L.tickets = take((size_t)rows * N_LAUNCH * sizeof(unsigned int));
+    L.cand = take((size_t)rows * chunks * CAND_MAX * sizeof(unsigned long long));
     L.state = take((size_t)rows * sizeof(RowState));
     L.total = off;
     return L;
@@ -390,6 +608,7 @@ extern "C" int odmkv_allocate(const float* scores, int rows, int n,
     ODMKV_CHECK_ARG(sink_mask || n_sink == 0 || (period > 0 && n % period == 0 && n_sink <= period),
                     "allocate: bad sink pattern period=%d n_sink=%d n=%d", period, n_sink, n);
     ODMKV_CHECK_ARG((double)n * 16.0 < 16777216.0, "allocate: rows longer than 1,048,575 tokens lose exactness of the fp32 mean");
+    ODMKV_CHECK_ARG(rows <= 65535, "allocate: at most 65535 rows per call");
     ODMKV_CHECK_ARG(workspace_bytes >= odmkv_allocate_workspace_bytes(rows, n), "allocate: workspace too small");
     hipStream_t st = (hipStream_t)stream;
     const AllocLayout L = alloc_layout(rows, n);
@@ -397,28 +616,38 @@ extern "C" int odmkv_allocate(const float* scores, int rows, int n,
     AllocArgs a;
     a.scores = scores; a.sink_mask = sink_mask; a.rows = rows; a.n = n;
     a.period = period > 0 ? period : n; a.n_sink = sink_mask ? 0 : n_sink; a.sink_bits = sink_bits; a.K = n_levels;
+    a.n_chunks = (n + EV_TOKENS - 1) / EV_TOKENS;
     for (int k = 0; k < NLV; ++k) {
         a.eps[k] = k < n_levels ? (float)eps[k] : 0.0f;
         a.bitsf[k] = k < n_levels ? (float)levels[k] : 0.0f;
         a.nominal[k] = k < n_levels ? levels[k] : 0;
     }
     a.target = target;
-    a.s_clean = (float*)(ws + L.s_clean); a.chosen = (uint8_t*)(ws + L.chosen);
-    a.hist = (unsigned int*)(ws + L.hist); a.tickets = (unsigned int*)(ws + L.tickets);
+    a.chosen = (uint8_t*)(ws + L.chosen);
+    a.partial = (unsigned int*)(ws + L.partial); a.tickets = (unsigned int*)(ws + L.tickets);
+    a.cand = (unsigned long long*)(ws + L.cand);
     a.state = (RowState*)(ws + L.state);
     a.bits_out = bits_out; a.level_counts = level_counts; a.lambda_out = lambda_out;
-    const dim3 grid((n + HIST_TOKENS - 1) / HIST_TOKENS, rows), block(256);
-    hipLaunchKernelGGL(alloc_init_kernel, dim3(rows), dim3(256), 0, st, a);
+    const dim3 grid(a.n_chunks, rows), block(EV_THREADS);
+    hipLaunchKernelGGL(alloc_init_kernel, dim3(rows), dim3(64), 0, st, a);
     ODMKV_CHECK_LAUNCH("alloc_init_kernel");
     if (n_levels > 1) {
-        hipLaunchKernelGGL(alloc_scan_kernel, grid, block, 0, st, a);
+        hipLaunchKernelGGL(alloc_scan_kernel, dim3((n + SC_TOKENS - 1) / SC_TOKENS, rows), dim3(SC_THREADS), 0, st, a);
         ODMKV_CHECK_LAUNCH("alloc_scan_kernel");
-        hipLaunchKernelGGL(alloc_clean_kernel, grid, block, 0, st, a);
-        ODMKV_CHECK_LAUNCH("alloc_clean_kernel");
-        for (int it = 0; it < ITERS; ++it) {
-            hipLaunchKernelGGL(alloc_eval_kernel, grid, block, 0, st, a, it);
+        for (int l = 0; l < N_LAUNCH; ++l) {
+            switch (n_levels) {
+                case 2: hipLaunchKernelGGL(alloc_eval_kernel<2>, grid, block, 0, st, a, l); break;
+                case 3: hipLaunchKernelGGL(alloc_eval_kernel<3>, grid, block, 0, st, a, l); break;
+                case 4: hipLaunchKernelGGL(alloc_eval_kernel<4>, grid, block, 0, st, a, l); break;
+                case 5: hipLaunchKernelGGL(alloc_eval_kernel<5>, grid, block, 0, st, a, l); break;
+                case 6: hipLaunchKernelGGL(alloc_eval_kernel<6>, grid, block, 0, st, a, l); break;
+                case 7: hipLaunchKernelGGL(alloc_eval_kernel<7>, grid, block, 0, st, a, l); break;
+                default: hipLaunchKernelGGL(alloc_eval_kernel<8>, grid, block, 0, st, a, l); break;
+            }
             ODMKV_CHECK_LAUNCH("alloc_eval_kernel");
         }
+        hipLaunchKernelGGL(alloc_cand_kernel, grid, block, 0, st, a);
+        ODMKV_CHECK_LAUNCH("alloc_cand_kernel");
         hipLaunchKernelGGL(alloc_repair_kernel, dim3(rows), dim3(RB), 0, st, a);
         ODMKV_CHECK_LAUNCH("alloc_repair_kernel");
     }

@@ -1,93 +1,189 @@
 // Packed mixed-width KV store: level counts, position compaction, TurboQuant-MSE quantise + pack,
 // exact-row gather, decode-time append, and dequantise-to-dense.
 //
-// One wavefront owns one 64-token tile.  During quantisation and dequantisation a lane owns one
-// token: it keeps the 128 coordinates in registers and walks the rotation matrix through
-// scalar (wave-uniform) loads, so the 128x128 rotation needs no LDS traffic and its fp32
-// summation order is exactly the sequential one the CPU oracle uses.
+// One wavefront owns one 64-token tile.  The quantiser runs the rotation on the fp32 matrix cores
+// one k at a time; the dequantiser keeps a token per lane and walks the rotation matrix through
+// scalar (wave-uniform) loads.  Both keep the sequential fp32 summation order of the definition.
+#include <algorithm>
 #include "quant.h"
 
 // ------------------------------------------------------------------------------------------------
 // level counts
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void level_counts_kernel(const int32_t* __restrict__ bits, int T,
-                                                           int32_t* __restrict__ counts) {
+#define LC_THREADS 1024
+
+__device__ static inline int wave_sum_i32(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+
+__global__ __launch_bounds__(LC_THREADS) void level_counts_kernel(const int32_t* __restrict__ bits, int T,
+                                                                  int32_t* __restrict__ counts) {
     __shared__ int c[6];
-    const int bh = blockIdx.x;
-    if (threadIdx.x < 6) c[threadIdx.x] = 0;
+    const int bh = blockIdx.x, tid = threadIdx.x;
+    if (tid < 6) c[tid] = 0;
     __syncthreads();
     int local[6] = {0, 0, 0, 0, 0, 0};
-    for (int t = threadIdx.x; t < T; t += blockDim.x) {
-        const int s = level_slot(bits[(size_t)bh * T + t]);
+    const int32_t* row = bits + (size_t)bh * T;
+    const bool vec = (T % 4 == 0) && ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
+    if (vec) {
+        const int4* row4 = reinterpret_cast<const int4*>(row);
+        for (int q = tid; q < T / 4; q += LC_THREADS) {
+            const int4 v = row4[q];
+            const int s4[4] = {level_slot(v.x), level_slot(v.y), level_slot(v.z), level_slot(v.w)};
 #pragma unroll
-        for (int k = 0; k < 6; ++k) local[k] += (s == k);
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int k = 0; k < 6; ++k) local[k] += (s4[e] == k);
+        }
+    } else {
+        for (int t = tid; t < T; t += LC_THREADS) {
+            const int sl = level_slot(row[t]);
+#pragma unroll
+            for (int k = 0; k < 6; ++k) local[k] += (sl == k);
+        }
     }
 #pragma unroll
-    for (int k = 0; k < 6; ++k)
-        if (local[k]) atomicAdd(&c[k], local[k]);
+    for (int k = 0; k < 6; ++k) {
+        const int w = wave_sum_i32(local[k]);
+        if ((tid & 63) == 0 && w) atomicAdd(&c[k], w);
+    }
     __syncthreads();
-    if (threadIdx.x < 6) counts[bh * 6 + threadIdx.x] = c[threadIdx.x];
+    if (tid < 6) counts[bh * 6 + tid] = c[tid];
 }
 
 extern "C" int odmkv_level_counts(const int32_t* bits, int B, int Hkv, int T, int32_t* counts,
                                   void* stream) {
     ODMKV_CHECK_ARG(bits && counts, "level_counts: null pointer");
     ODMKV_CHECK_ARG(B > 0 && Hkv > 0 && T >= 0, "level_counts: bad shape B=%d Hkv=%d T=%d", B, Hkv, T);
-    hipLaunchKernelGGL(level_counts_kernel, dim3(B * Hkv), dim3(256), 0, (hipStream_t)stream, bits, T, counts);
+    hipLaunchKernelGGL(level_counts_kernel, dim3(B * Hkv), dim3(LC_THREADS), 0, (hipStream_t)stream, bits, T, counts);
     ODMKV_CHECK_LAUNCH("level_counts_kernel");
     return 0;
 }
 
 // ------------------------------------------------------------------------------------------------
-// compaction: ascending token positions per (bh, level), appended behind what is stored
+// compaction: ascending token positions per (bh, level), appended behind what is stored.
+// Two launches over chunks of 2048 tokens: count per (bh, chunk, level), then every chunk places
+// its tokens behind the chunks before it.
 // ------------------------------------------------------------------------------------------------
+#define CP_THREADS 256
+#define CP_TPT 8
+#define CP_TOKENS (CP_THREADS * CP_TPT)
+
 struct CompactArgs {
     const int32_t* bits;
-    int T, pos_offset, nseg;
+    int T, pos_offset, nseg, n_chunks;
     int32_t* pos[5];
     const int32_t* seg_tile[5];
     int32_t* seg_count[5];
-    int32_t* old_count;   // [5][nseg]
+    int32_t* old_count;     // [5][nseg]
+    int32_t* chunk_count;   // [nseg][n_chunks][5]
 };
 
-__global__ __launch_bounds__(256) void compact_kernel(CompactArgs a) {
-    __shared__ int wave_tot[5][4];
-    __shared__ int base[5];
-    __shared__ int cap[5];
-    const int bh = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    if (tid < 5) {
-        const int b0 = a.seg_count[tid][bh];
-        base[tid] = b0;
-        a.old_count[tid * a.nseg + bh] = b0;
-        cap[tid] = (a.seg_tile[tid][bh + 1] - a.seg_tile[tid][bh]) * TILE;
+// levels (1..5, 0 = evicted, -1 = past the end) of the 8 consecutive tokens this thread owns
+__device__ static inline void load_slots(const CompactArgs& a, int bh, int t0, int* sl) {
+    const int32_t* row = a.bits + (size_t)bh * a.T;
+    if (t0 + CP_TPT <= a.T && ((reinterpret_cast<uintptr_t>(row + t0) & 15) == 0)) {
+        const int4 v0 = *reinterpret_cast<const int4*>(row + t0);
+        const int4 v1 = *reinterpret_cast<const int4*>(row + t0 + 4);
+        const int b[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int e = 0; e < CP_TPT; ++e) sl[e] = level_slot(b[e]);
+    } else {
+#pragma unroll
+        for (int e = 0; e < CP_TPT; ++e) sl[e] = (t0 + e < a.T) ? level_slot(row[t0 + e]) : -1;
+    }
+}
+
+__global__ __launch_bounds__(CP_THREADS) void chunk_count_kernel(CompactArgs a) {
+    __shared__ int c[5];
+    const int bh = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+    if (tid < 5) c[tid] = 0;
+    if (chunk == 0 && tid < 5) a.old_count[tid * a.nseg + bh] = a.seg_count[tid][bh];
+    __syncthreads();
+    int sl[CP_TPT];
+    load_slots(a, bh, chunk * CP_TOKENS + tid * CP_TPT, sl);
+#pragma unroll
+    for (int L = 0; L < 5; ++L) {
+        int n = 0;
+#pragma unroll
+        for (int e = 0; e < CP_TPT; ++e) n += (sl[e] == L + 1);
+        n = wave_sum_i32(n);
+        if ((tid & 63) == 0 && n) atomicAdd(&c[L], n);
     }
     __syncthreads();
-    for (int c = 0; c < a.T; c += 256) {
-        const int t = c + tid;
-        const int s = (t < a.T) ? level_slot(a.bits[(size_t)bh * a.T + t]) : -1;
-        int rank = 0;
-#pragma unroll
-        for (int L = 0; L < 5; ++L) {
-            const unsigned long long m = __ballot(s == L + 1);
-            if (lane == 0) wave_tot[L][wave] = __popcll(m);
-            if (s == L + 1) rank = __popcll(m & ((1ull << lane) - 1ull));
+    if (tid < 5) a.chunk_count[((size_t)bh * a.n_chunks + chunk) * 5 + tid] = c[tid];
+}
+
+__global__ __launch_bounds__(CP_THREADS) void compact_kernel(CompactArgs a) {
+    __shared__ int base[5];
+    __shared__ int cap[5];
+    __shared__ int wave_tot[5][CP_THREADS / 64];
+    const int bh = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    if (tid < 5) {
+        const int32_t* cc = a.chunk_count + (size_t)bh * a.n_chunks * 5 + tid;
+        int before = 0, total = 0;
+        for (int c = 0; c < a.n_chunks; ++c) {
+            const int v = cc[(size_t)c * 5];
+            total += v;
+            before += (c < chunk) ? v : 0;
         }
-        __syncthreads();
-        if (s >= 1) {
-            const int L = s - 1;
-            int off = base[L] + rank;
-            for (int w = 0; w < wave; ++w) off += wave_tot[L][w];
-            if (off < cap[L]) a.pos[L][(size_t)a.seg_tile[L][bh] * TILE + off] = t + a.pos_offset;
-        }
-        __syncthreads();
-        if (tid < 5) base[tid] += wave_tot[tid][0] + wave_tot[tid][1] + wave_tot[tid][2] + wave_tot[tid][3];
-        __syncthreads();
+        const int old = a.old_count[tid * a.nseg + bh];
+        const int room = (a.seg_tile[tid][bh + 1] - a.seg_tile[tid][bh]) * TILE;
+        base[tid] = old + before;
+        cap[tid] = room;
+        if (chunk == 0) a.seg_count[tid][bh] = min(old + total, room);
     }
-    if (tid < 5) a.seg_count[tid][bh] = min(base[tid], cap[tid]);
+    int sl[CP_TPT];
+    const int t0 = chunk * CP_TOKENS + tid * CP_TPT;
+    load_slots(a, bh, t0, sl);
+    int mine[5], incl[5];
+#pragma unroll
+    for (int L = 0; L < 5; ++L) {
+        int n = 0;
+#pragma unroll
+        for (int e = 0; e < CP_TPT; ++e) n += (sl[e] == L + 1);
+        mine[L] = n;
+        int x = n;                                         // inclusive scan over the wave
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int y = __shfl_up(x, o, WAVE);
+            x += (lane >= o) ? y : 0;
+        }
+        incl[L] = x;
+        if (lane == 63) wave_tot[L][wave] = x;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int L = 0; L < 5; ++L) {
+        int off = base[L] + incl[L] - mine[L];
+        for (int w = 0; w < wave; ++w) off += wave_tot[L][w];
+        if (mine[L]) {
+            int32_t* dst = a.pos[L] + (size_t)a.seg_tile[L][bh] * TILE;
+#pragma unroll
+            for (int e = 0; e < CP_TPT; ++e) {
+                if (sl[e] == L + 1) {
+                    if (off < cap[L]) dst[off] = t0 + e + a.pos_offset;
+                    ++off;
+                }
+            }
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
-// quantise + pack one tile (blockIdx.y: 0 = keys, 1 = values)
+// quantise + pack
+//
+// The 128x128 rotation runs on the fp32 matrix cores with K = 1 per instruction
+// (v_mfma_f32_32x32x1_2b_f32): one instruction adds u[token][j] * Pi[out][j] to a 64-token x
+// 32-output block, so chaining j = 0..127 reproduces the sequential fp32 fma order of the scalar
+// definition bit for bit, at twice the rate of the vector ALU and with the vector ALU free for
+// the division, the centroid search and the packing.  Lane = token for the A operand; the B
+// operand (Pi^T[j][4c..4c+3] for lane c of either half) is one ds_read_b128 from LDS.
+//
+// Workgroups are persistent: even ones take keys, odd ones values; each keeps its rotation in LDS
+// and its waves walk the tiles of all quantised levels.
 // ------------------------------------------------------------------------------------------------
 struct QuantArgs {
     const void* K;
@@ -96,18 +192,19 @@ struct QuantArgs {
     int Hkv, nseg, pos_offset;
     const float* pi_k;
     const float* pi_v;
-    const float* cb;             // this width's centroids
-    const int32_t* pos;          // this level
-    const int32_t* seg_tile;
-    const int32_t* seg_count;
-    const int32_t* old_count;
-    uint8_t* kcodes;
-    uint8_t* vcodes;
-    float* knorm;
-    float* vnorm;
+    const float* cb;             // centroids of widths 2, 3, 4, 8 back to back
+    const int32_t* old_count;    // [5][nseg]
+    int tile_base[ODMKV_NQ + 1]; // running sum of the levels' tile counts
+    odmkv_packed_t s;
 };
 
-#define CODE_ROW 144   // LDS bytes per token row of codes (128 + padding, multiple of 16)
+typedef float f32x32 __attribute__((ext_vector_type(32)));
+
+#define CODE_ROW 144      // K staging: LDS bytes per token row of codes (128 + padding, multiple of 16)
+#define CODE_ROW_T 72     // V staging: LDS bytes per dim row of 64 token codes (64 + padding, multiple of 8)
+#define QP_STAGE (TILE * CODE_ROW)
+#define QP_PI_BYTES (HD * HD * 4)
+#define QP_CB_FLOATS 284
 
 // which segment owns `tile`: the largest bh with seg_tile[bh] <= tile
 __device__ static inline int find_segment(const int32_t* seg_tile, int nseg, int tile) {
@@ -119,114 +216,230 @@ __device__ static inline int find_segment(const int32_t* seg_tile, int nseg, int
     return lo;
 }
 
-template <int W, int DT>
-__global__ __launch_bounds__(64) void quant_pack_kernel(QuantArgs a) {
-    __shared__ __align__(16) uint8_t codes[TILE * CODE_ROW];
-    __shared__ float cb[1 << W];
-    const int lane = threadIdx.x;
-    const int tile = blockIdx.x;
-    const bool is_v = blockIdx.y != 0;
+// token (0..63) that accumulator register vv of lane `lane` belongs to
+__device__ static inline int mfma_token(int vv, int lane) {
+    return (vv >> 4) * 32 + ((vv & 15) >> 2) * 8 + (lane >> 5) * 4 + (vv & 3);
+}
 
-    const int bh = find_segment(a.seg_tile, a.nseg, tile);
-    const int ts = (tile - a.seg_tile[bh]) * TILE;
-    const int lo = max(a.old_count[bh] - ts, 0);
-    const int hi = min(a.seg_count[bh] - ts, TILE);
-    if (lo >= hi) return;                                   // nothing new in this tile (wave-uniform)
-
-    for (int i = lane; i < (1 << W); i += WAVE) cb[i] = a.cb[i];
-    const bool valid = lane >= lo && lane < hi;
-    const size_t slot = (size_t)tile * TILE + lane;
-
-    float x[HD];
-    if (valid) {
-        const int t = a.pos[slot] - a.pos_offset;
-        const size_t off = (size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH + (size_t)t * a.sT;
-        load_row<DT>(is_v ? a.V : a.K, off, x);
-    } else {
+template <int W>
+__device__ static inline void stage_codes_k(const f32x32& a0, const f32x32& a1, const f32x32& a2, const f32x32& a3,
+                                            const float* cb, uint8_t* stage, int lane) {
+    const int c = lane & 31;
 #pragma unroll
-        for (int j = 0; j < HD; ++j) x[j] = 0.0f;
+    for (int vv = 0; vv < 32; ++vv) {
+        const uint32_t w = nearest_code<W>(a0[vv], cb) | (nearest_code<W>(a1[vv], cb) << 8) |
+                           (nearest_code<W>(a2[vv], cb) << 16) | (nearest_code<W>(a3[vv], cb) << 24);
+        *reinterpret_cast<uint32_t*>(stage + mfma_token(vv, lane) * CODE_ROW + 4 * c) = w;
     }
-    float ss = 0.0f;
-#pragma unroll
-    for (int j = 0; j < HD; ++j) ss = __fmaf_rn(x[j], x[j], ss);
-    const float norm = sqrtf(ss);
-    const float den = norm + 1e-10f;
-#pragma unroll
-    for (int j = 0; j < HD; ++j) x[j] = x[j] / den;
-    __syncthreads();                                        // codebook visible
+}
 
-    const float* __restrict__ pi = is_v ? a.pi_v : a.pi_k;
-#pragma unroll 1
-    for (int i0 = 0; i0 < HD; i0 += 8) {
-        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        const float* __restrict__ rows = pi + (size_t)i0 * HD;
+template <int W>
+__device__ static inline void stage_codes_v(const f32x32& acc, int g, const float* cb, uint8_t* stage, int lane) {
+    const int c = lane & 31;
 #pragma unroll
-        for (int j = 0; j < HD; ++j) {
-#pragma unroll
-            for (int b = 0; b < 8; ++b) acc[b] = __fmaf_rn(x[j], rows[b * HD + j], acc[b]);
-        }
-        uint32_t w0 = 0, w1 = 0;
-#pragma unroll
-        for (int b = 0; b < 4; ++b) w0 |= nearest_code<W>(acc[b], cb) << (8 * b);
-#pragma unroll
-        for (int b = 0; b < 4; ++b) w1 |= nearest_code<W>(acc[4 + b], cb) << (8 * b);
-        *reinterpret_cast<uint2*>(&codes[lane * CODE_ROW + i0]) = make_uint2(w0, w1);
+    for (int q = 0; q < 8; ++q) {
+        const uint32_t w = nearest_code<W>(acc[4 * q], cb) | (nearest_code<W>(acc[4 * q + 1], cb) << 8) |
+                           (nearest_code<W>(acc[4 * q + 2], cb) << 16) | (nearest_code<W>(acc[4 * q + 3], cb) << 24);
+        *reinterpret_cast<uint32_t*>(stage + (g * 32 + c) * CODE_ROW_T + mfma_token(4 * q, lane)) = w;
     }
-    __syncthreads();
+}
 
-    if (!is_v) {
-        // token-major: this lane packs its own 128 codes
-        if (valid) {
-            uint32_t words[4 * W];
+template <int W>
+__device__ static inline void pack_store_k(const uint8_t* stage, uint8_t* kcodes, int tile, int lane) {
+    uint32_t words[4 * W];
 #pragma unroll
-            for (int k = 0; k < 4 * W; ++k) words[k] = 0;
+    for (int k = 0; k < 4 * W; ++k) words[k] = 0;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                const uint4 v = *reinterpret_cast<const uint4*>(&codes[lane * CODE_ROW + 16 * c]);
-                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    for (int c = 0; c < 8; ++c) {
+        const uint4 v = *reinterpret_cast<const uint4*>(stage + lane * CODE_ROW + 16 * c);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                for (int e = 0; e < 16; ++e) put_code<W>(words, 16 * c + e, (w[e >> 2] >> (8 * (e & 3))) & 0xffu);
-            }
-            uint8_t* dst = a.kcodes + (size_t)tile * (TILE * 16 * W);
+        for (int e = 0; e < 16; ++e) put_code<W>(words, 16 * c + e, (w[e >> 2] >> (8 * (e & 3))) & 0xffu);
+    }
+    uint8_t* dst = kcodes + (size_t)tile * (TILE * 16 * W);
 #pragma unroll
-            for (int c = 0; c < W; ++c)
-                *reinterpret_cast<uint4*>(dst + ((size_t)c * TILE + lane) * 16) =
-                    make_uint4(words[4 * c], words[4 * c + 1], words[4 * c + 2], words[4 * c + 3]);
-            a.knorm[slot] = norm;
-        }
-    } else {
-        // dim-major: this lane packs the 64 tokens' codes of dims `lane` and `lane + 64`
-        uint8_t* dst = a.vcodes + (size_t)tile * (HD * 8 * W);
+    for (int c = 0; c < W; ++c)
+        *reinterpret_cast<uint4*>(dst + ((size_t)c * TILE + lane) * 16) =
+            make_uint4(words[4 * c], words[4 * c + 1], words[4 * c + 2], words[4 * c + 3]);
+}
+
+template <int W>
+__device__ static inline void pack_store_v(const uint8_t* stage, uint8_t* vcodes, int tile, int lane, int lo, int hi) {
+    uint8_t* dst = vcodes + (size_t)tile * (HD * 8 * W);
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int j = lane + 64 * half;
-            uint32_t words[2 * W];
+    for (int half = 0; half < 2; ++half) {
+        const int j = lane + 64 * half;
+        uint32_t words[2 * W];
 #pragma unroll
-            for (int k = 0; k < 2 * W; ++k) words[k] = 0;
+        for (int k = 0; k < 2 * W; ++k) words[k] = 0;
 #pragma unroll
-            for (int t = 0; t < TILE; ++t) {
-                uint32_t c = codes[t * CODE_ROW + j];
+        for (int t8 = 0; t8 < 8; ++t8) {
+            const uint2 v = *reinterpret_cast<const uint2*>(stage + j * CODE_ROW_T + 8 * t8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int t = 8 * t8 + e;
+                uint32_t c = ((e < 4 ? v.x : v.y) >> (8 * (e & 3))) & 0xffu;
                 c = (t >= lo && t < hi) ? c : 0u;
                 put_code<W>(words, t, c);
             }
-            if (lo > 0) {
-                // tokens below `lo` were packed earlier: keep their bits
-                const int keep_bits = lo * W;
+        }
+        if (lo > 0) {
+            // tokens below `lo` were packed earlier: keep their bits
+            const int keep_bits = lo * W;
 #pragma unroll
-                for (int k = 0; k < 2 * W; ++k) {
-                    const int nb = keep_bits - 32 * k;
-                    if (nb > 0) {
-                        const uint32_t old = *reinterpret_cast<const uint32_t*>(dst + v_word_offset<W>(k, j));
-                        const uint32_t mask = nb >= 32 ? 0xffffffffu : ((1u << nb) - 1u);
-                        words[k] = (old & mask) | (words[k] & ~mask);
-                    }
+            for (int k = 0; k < 2 * W; ++k) {
+                const int nb = keep_bits - 32 * k;
+                if (nb > 0) {
+                    const uint32_t old = *reinterpret_cast<const uint32_t*>(dst + v_word_offset<W>(k, j));
+                    const uint32_t mask = nb >= 32 ? 0xffffffffu : ((1u << nb) - 1u);
+                    words[k] = (old & mask) | (words[k] & ~mask);
                 }
             }
-#pragma unroll
-            for (int k = 0; k < 2 * W; ++k)
-                *reinterpret_cast<uint32_t*>(dst + v_word_offset<W>(k, j)) = words[k];
         }
-        if (valid) a.vnorm[slot] = norm;
+#pragma unroll
+        for (int k = 0; k < 2 * W; ++k)
+            *reinterpret_cast<uint32_t*>(dst + v_word_offset<W>(k, j)) = words[k];
+    }
+}
+
+// LDS writes of this wave visible to its own later reads (no other wave touches its staging area)
+__device__ static inline void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// a row of 128 elements kept as loaded: fp32 as 128 floats, 16-bit types as 64 packed words
+template <int DT> struct RowRegs {
+    static constexpr int N = (DT == ODMKV_F32) ? HD : HD / 2;
+    uint32_t w[N];
+    __device__ inline void zero() {
+#pragma unroll
+        for (int i = 0; i < N; ++i) w[i] = 0;
+    }
+    __device__ inline void load(const void* base, size_t elem_off) {
+        if constexpr (DT == ODMKV_F32) {
+            const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(base) + elem_off);
+#pragma unroll
+            for (int c = 0; c < 32; ++c) { const uint4 v = p[c]; w[4 * c] = v.x; w[4 * c + 1] = v.y; w[4 * c + 2] = v.z; w[4 * c + 3] = v.w; }
+        } else {
+            const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + elem_off);
+#pragma unroll
+            for (int c = 0; c < 16; ++c) { const uint4 v = p[c]; w[4 * c] = v.x; w[4 * c + 1] = v.y; w[4 * c + 2] = v.z; w[4 * c + 3] = v.w; }
+        }
+    }
+    __device__ inline float get(int j) const {
+        if constexpr (DT == ODMKV_F32) return __uint_as_float(w[j]);
+        else return Elem<DT>::to_f32((uint16_t)((j & 1) ? (w[j >> 1] >> 16) : (w[j >> 1] & 0xffffu)));
+    }
+};
+
+template <int DT, int NW>
+__global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    float* piT = reinterpret_cast<float*>(smem);                                   // [j][slot]
+    float* cbs = reinterpret_cast<float*>(smem + QP_PI_BYTES + NW * QP_STAGE);     // all widths
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint8_t* stage = smem + QP_PI_BYTES + wave * QP_STAGE;
+    const bool is_v = (blockIdx.x & 1) != 0;
+
+    // rotation -> LDS, transposed.  Keys: slot = output index.  Values: slot 4c+g holds output
+    // g*32+c, so that a lane's four accumulators are 32 outputs apart and its registers hold four
+    // consecutive tokens of one output (the dim-major order the V codes are stored in).
+    {
+        const float* __restrict__ pi = is_v ? a.pi_v : a.pi_k;
+        for (int idx = tid; idx < HD * HD; idx += NW * 64) {
+            const int i = idx >> 7, j = idx & 127;
+            const int slot = is_v ? ((i & 31) * 4 + (i >> 5)) : i;
+            piT[j * HD + slot] = pi[idx];
+        }
+        for (int i = tid; i < QP_CB_FLOATS; i += NW * 64) cbs[i] = a.cb[i];
+    }
+    __syncthreads();
+
+    const int total_tiles = a.tile_base[ODMKV_NQ];
+    const int wg = blockIdx.x >> 1, n_wg = gridDim.x >> 1;
+    for (int gt = wg * NW + wave; gt < total_tiles; gt += n_wg * NW) {
+        int li = 0;
+#pragma unroll
+        for (int k = 1; k < ODMKV_NQ; ++k) li += (gt >= a.tile_base[k]);
+        const int tile = gt - a.tile_base[li];
+        const int32_t* seg_tile = a.s.seg_tile[li];
+        const int bh = find_segment(seg_tile, a.nseg, tile);
+        const int ts = (tile - seg_tile[bh]) * TILE;
+        const int lo = max(a.old_count[li * a.nseg + bh] - ts, 0);
+        const int hi = min(a.s.seg_count[li][bh] - ts, TILE);
+        if (lo >= hi) continue;                                 // nothing new in this tile (wave-uniform)
+
+        const bool valid = lane >= lo && lane < hi;
+        const size_t slot = (size_t)tile * TILE + lane;
+        RowRegs<DT> x;
+        if (valid) {
+            const int t = a.s.pos[li][slot] - a.pos_offset;
+            const size_t off = (size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH + (size_t)t * a.sT;
+            x.load(is_v ? a.V : a.K, off);
+        } else {
+            x.zero();
+        }
+        float ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < HD; ++j) { const float xj = x.get(j); ss = __fmaf_rn(xj, xj, ss); }
+        const float norm = sqrtf(ss);
+        const float den = norm + 1e-10f;
+
+        f32x32 acc0, acc1, acc2, acc3;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; acc2[i] = 0.0f; acc3[i] = 0.0f; }
+        const float4* __restrict__ brow = reinterpret_cast<const float4*>(piT) + (lane & 31);
+#pragma unroll
+        for (int j = 0; j < HD; ++j) {
+            const float u = x.get(j) / den;
+            const float4 b = brow[j * (HD / 4)];
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.x, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.y, acc1, 0, 0, 0);
+            acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.z, acc2, 0, 0, 0);
+            acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.w, acc3, 0, 0, 0);
+        }
+
+        const float* cb = cbs + codebook_offset(li);
+        if (!is_v) {
+            switch (li) {
+                case 0: stage_codes_k<2>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                case 1: stage_codes_k<3>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                case 2: stage_codes_k<4>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                default: stage_codes_k<8>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+            }
+            wave_lds_fence();
+            if (valid) {
+                switch (li) {
+                    case 0: pack_store_k<2>(stage, a.s.kcodes[0], tile, lane); break;
+                    case 1: pack_store_k<3>(stage, a.s.kcodes[1], tile, lane); break;
+                    case 2: pack_store_k<4>(stage, a.s.kcodes[2], tile, lane); break;
+                    default: pack_store_k<8>(stage, a.s.kcodes[3], tile, lane); break;
+                }
+                a.s.knorm[li][slot] = norm;
+            }
+        } else {
+            switch (li) {
+                case 0: stage_codes_v<2>(acc0, 0, cb, stage, lane); stage_codes_v<2>(acc1, 1, cb, stage, lane);
+                        stage_codes_v<2>(acc2, 2, cb, stage, lane); stage_codes_v<2>(acc3, 3, cb, stage, lane); break;
+                case 1: stage_codes_v<3>(acc0, 0, cb, stage, lane); stage_codes_v<3>(acc1, 1, cb, stage, lane);
+                        stage_codes_v<3>(acc2, 2, cb, stage, lane); stage_codes_v<3>(acc3, 3, cb, stage, lane); break;
+                case 2: stage_codes_v<4>(acc0, 0, cb, stage, lane); stage_codes_v<4>(acc1, 1, cb, stage, lane);
+                        stage_codes_v<4>(acc2, 2, cb, stage, lane); stage_codes_v<4>(acc3, 3, cb, stage, lane); break;
+                default: stage_codes_v<8>(acc0, 0, cb, stage, lane); stage_codes_v<8>(acc1, 1, cb, stage, lane);
+                         stage_codes_v<8>(acc2, 2, cb, stage, lane); stage_codes_v<8>(acc3, 3, cb, stage, lane); break;
+            }
+            wave_lds_fence();
+            switch (li) {
+                case 0: pack_store_v<2>(stage, a.s.vcodes[0], tile, lane, lo, hi); break;
+                case 1: pack_store_v<3>(stage, a.s.vcodes[1], tile, lane, lo, hi); break;
+                case 2: pack_store_v<4>(stage, a.s.vcodes[2], tile, lane, lo, hi); break;
+                default: pack_store_v<8>(stage, a.s.vcodes[3], tile, lane, lo, hi); break;
+            }
+            if (valid) a.s.vnorm[li][slot] = norm;
+        }
+        wave_lds_fence();                                       // staging area free for the next tile
     }
 }
 
@@ -334,20 +547,33 @@ static int check_store(const odmkv_packed_t* s, const char* who) {
     return 0;
 }
 
+static inline int compact_chunks(int T) { return (T + CP_TOKENS - 1) / CP_TOKENS; }
+
 extern "C" size_t odmkv_pack_workspace_bytes(int B, int Hkv, int T) {
-    (void)T;
-    return align_up((size_t)5 * B * Hkv * sizeof(int32_t), 256);
+    if (B <= 0 || Hkv <= 0 || T <= 0) return 0;
+    return align_up((size_t)5 * B * Hkv * sizeof(int32_t), 256) +
+           align_up((size_t)5 * B * Hkv * compact_chunks(T) * sizeof(int32_t), 256);
 }
 
 template <int DT>
-static int launch_quant(const QuantArgs& qa, int li, int n_tiles, hipStream_t st) {
-    dim3 grid(n_tiles, 2), block(64);
-    switch (li) {
-        case 0: hipLaunchKernelGGL((quant_pack_kernel<2, DT>), grid, block, 0, st, qa); break;
-        case 1: hipLaunchKernelGGL((quant_pack_kernel<3, DT>), grid, block, 0, st, qa); break;
-        case 2: hipLaunchKernelGGL((quant_pack_kernel<4, DT>), grid, block, 0, st, qa); break;
-        default: hipLaunchKernelGGL((quant_pack_kernel<8, DT>), grid, block, 0, st, qa); break;
+static int launch_quant(const QuantArgs& qa, hipStream_t st) {
+    // fp32 rows take 128 registers on top of the 128 accumulators: one wave per SIMD then
+    constexpr int NW = (DT == ODMKV_F32) ? 4 : 8;
+    const size_t lds = QP_PI_BYTES + (size_t)NW * QP_STAGE + QP_CB_FLOATS * sizeof(float);
+    static bool attr_set = false;
+    if (!attr_set) {
+        ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&quant_pack_kernel<DT, NW>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
     }
+    const int total = qa.tile_base[ODMKV_NQ];
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+    }
+    const int per_tensor = std::max(1, std::min((total + NW - 1) / NW, std::max(cus / 2, 1)));
+    hipLaunchKernelGGL((quant_pack_kernel<DT, NW>), dim3(2 * per_tensor), dim3(NW * 64), lds, st, qa);
     ODMKV_CHECK_LAUNCH("quant_pack_kernel");
     return 0;
 }
@@ -385,24 +611,29 @@ extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, 
 
     CompactArgs ca;
     ca.bits = bits; ca.T = T; ca.pos_offset = pos_offset; ca.nseg = nseg; ca.old_count = old_count;
+    ca.n_chunks = compact_chunks(T);
+    ca.chunk_count = (int32_t*)((char*)workspace + align_up((size_t)5 * nseg * sizeof(int32_t), 256));
     for (int li = 0; li < 5; ++li) { ca.pos[li] = store->pos[li]; ca.seg_tile[li] = store->seg_tile[li]; ca.seg_count[li] = store->seg_count[li]; }
-    hipLaunchKernelGGL(compact_kernel, dim3(nseg), dim3(256), 0, st, ca);
+    ODMKV_CHECK_ARG(nseg <= 65535, "quant_pack: at most 65535 (sequence, head) pairs per call");
+    hipLaunchKernelGGL(chunk_count_kernel, dim3(ca.n_chunks, nseg), dim3(CP_THREADS), 0, st, ca);
+    ODMKV_CHECK_LAUNCH("chunk_count_kernel");
+    hipLaunchKernelGGL(compact_kernel, dim3(ca.n_chunks, nseg), dim3(CP_THREADS), 0, st, ca);
     ODMKV_CHECK_LAUNCH("compact_kernel");
 
-    for (int li = 0; li < ODMKV_NQ; ++li) {
-        if (store->n_tiles[li] == 0) continue;
+    {
         QuantArgs qa;
         qa.K = K; qa.V = V; qa.sB = stride_b; qa.sH = stride_h; qa.sT = stride_t;
         qa.Hkv = Hkv; qa.nseg = nseg; qa.pos_offset = pos_offset;
-        qa.pi_k = pi_k; qa.pi_v = pi_v; qa.cb = codebooks + codebook_offset(li);
-        qa.pos = store->pos[li]; qa.seg_tile = store->seg_tile[li]; qa.seg_count = store->seg_count[li];
-        qa.old_count = old_count + (size_t)li * nseg;
-        qa.kcodes = store->kcodes[li]; qa.vcodes = store->vcodes[li];
-        qa.knorm = store->knorm[li]; qa.vnorm = store->vnorm[li];
-        int rc = dtype == ODMKV_F16 ? launch_quant<ODMKV_F16>(qa, li, store->n_tiles[li], st)
-               : dtype == ODMKV_BF16 ? launch_quant<ODMKV_BF16>(qa, li, store->n_tiles[li], st)
-                                     : launch_quant<ODMKV_F32>(qa, li, store->n_tiles[li], st);
-        if (rc) return rc;
+        qa.pi_k = pi_k; qa.pi_v = pi_v; qa.cb = codebooks; qa.old_count = old_count;
+        qa.s = *store;
+        qa.tile_base[0] = 0;
+        for (int li = 0; li < ODMKV_NQ; ++li) qa.tile_base[li + 1] = qa.tile_base[li] + store->n_tiles[li];
+        if (qa.tile_base[ODMKV_NQ] > 0) {
+            int rc = dtype == ODMKV_F16 ? launch_quant<ODMKV_F16>(qa, st)
+                   : dtype == ODMKV_BF16 ? launch_quant<ODMKV_BF16>(qa, st)
+                                         : launch_quant<ODMKV_F32>(qa, st);
+            if (rc) return rc;
+        }
     }
     if (store->n_tiles[4] > 0) {
         ExactArgs ea;

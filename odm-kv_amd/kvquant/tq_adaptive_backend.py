@@ -97,23 +97,63 @@ class TurboQuantAdaptiveKVCacheState:
         self._packed = None
 
     def _alloc(self, seg_tile: np.ndarray) -> dict:
+        """All buffers of the store as views into one allocation: the segment tables (one upload),
+        the counters, norms and exact rows (zeroed), the positions (-1), then the codes (left as they
+        come: every code the kernels read is written first or is a padding lane masked by count)."""
         dev = self.device
-        n_tiles = seg_tile[:, -1]
-        bufs = {"seg_tile": [], "seg_count": [], "pos": [], "kcodes": [], "vcodes": [], "knorm": [], "vnorm": []}
+        n_tiles = [max(int(t), 1) for t in seg_tile[:, -1]]
+        exact_bytes = 2
+        plan, off = [], 0
+
+        def take(name, li, nbytes, dtype):
+            nonlocal off
+            plan.append((name, li, off, nbytes, dtype))
+            off += (nbytes + 255) // 256 * 256
+
         for li in range(5):
-            nt = int(n_tiles[li])
-            bufs["seg_tile"].append(torch.from_numpy(seg_tile[li].astype(np.int32)).to(dev))
-            bufs["seg_count"].append(torch.zeros(self._nseg, dtype=torch.int32, device=dev))
-            bufs["pos"].append(torch.full((max(nt, 1) * TILE,), -1, dtype=torch.int32, device=dev))
-            if li < 4:
-                w = WIDTHS[li]
-                bufs["kcodes"].append(torch.zeros(max(nt, 1) * TILE * 16 * w, dtype=torch.uint8, device=dev))
-                bufs["vcodes"].append(torch.zeros(max(nt, 1) * HEAD_DIM * 8 * w, dtype=torch.uint8, device=dev))
-                bufs["knorm"].append(torch.zeros(max(nt, 1) * TILE, dtype=torch.float32, device=dev))
-                bufs["vnorm"].append(torch.zeros(max(nt, 1) * TILE, dtype=torch.float32, device=dev))
-        nt = int(n_tiles[4])
-        bufs["kexact"] = torch.zeros(max(nt, 1) * TILE * HEAD_DIM, dtype=self._exact_torch_dtype, device=dev)
-        bufs["vexact"] = torch.zeros(max(nt, 1) * TILE * HEAD_DIM, dtype=self._exact_torch_dtype, device=dev)
+            take("seg_tile", li, (self._nseg + 1) * 4, torch.int32)
+        for li in range(5):
+            take("seg_count", li, self._nseg * 4, torch.int32)
+        for li in range(4):
+            take("knorm", li, n_tiles[li] * TILE * 4, torch.float32)
+            take("vnorm", li, n_tiles[li] * TILE * 4, torch.float32)
+        # exact rows take part in the products as they are (a zero weight does not silence a NaN)
+        take("kexact", None, n_tiles[4] * TILE * HEAD_DIM * exact_bytes, self._exact_torch_dtype)
+        take("vexact", None, n_tiles[4] * TILE * HEAD_DIM * exact_bytes, self._exact_torch_dtype)
+        zero_end = off
+        for li in range(5):
+            take("pos", li, n_tiles[li] * TILE * 4, torch.int32)
+        pos_end = off
+        for li in range(4):
+            w = WIDTHS[li]
+            take("kcodes", li, n_tiles[li] * TILE * 16 * w, torch.uint8)
+            take("vcodes", li, n_tiles[li] * HEAD_DIM * 8 * w, torch.uint8)
+
+        arena = getattr(self, "_arena", None)
+        if arena is None or arena.numel() < off or arena.device != dev:
+            arena = torch.empty(off + off // 8, dtype=torch.uint8, device=dev)
+            self._arena_spare = None
+        elif self._bufs is not None:
+            # the live store is in this arena: build the new one elsewhere, keep the old as the spare
+            spare = getattr(self, "_arena_spare", None)
+            if spare is None or spare.numel() < off:
+                spare = torch.empty(off + off // 8, dtype=torch.uint8, device=dev)
+            arena, self._arena_spare = spare, arena
+        self._arena = arena
+        tables_end = plan[5][2]
+        table = np.zeros(tables_end // 4, np.int32)
+        for name, li, o, nbytes, _ in plan[:5]:
+            table[o // 4:o // 4 + self._nseg + 1] = seg_tile[li]
+        arena[:tables_end].view(torch.int32).copy_(torch.from_numpy(table))
+        arena[tables_end:zero_end].zero_()
+        arena[zero_end:pos_end].view(torch.int32).fill_(-1)
+        bufs = {"seg_tile": [], "seg_count": [], "pos": [], "kcodes": [], "vcodes": [], "knorm": [], "vnorm": []}
+        for name, li, o, nbytes, dtype in plan:
+            view = arena[o:o + nbytes].view(dtype)
+            if li is None:
+                bufs[name] = view
+            else:
+                bufs[name].append(view)
         return bufs
 
     def _make_struct(self) -> None:
