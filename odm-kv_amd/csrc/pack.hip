@@ -204,7 +204,6 @@ typedef float f32x32 __attribute__((ext_vector_type(32)));
 #define CODE_ROW_T 72     // V staging: LDS bytes per dim row of 64 token codes (64 + padding, multiple of 8)
 #define QP_STAGE (TILE * CODE_ROW)
 #define QP_PI_BYTES (HD * HD * 4)
-#define QP_CB_FLOATS 284
 
 // which segment owns `tile`: the largest bh with seg_tile[bh] <= tile
 __device__ static inline int find_segment(const int32_t* seg_tile, int nseg, int tile) {
@@ -221,31 +220,87 @@ __device__ static inline int mfma_token(int vv, int lane) {
     return (vv >> 4) * 32 + ((vv & 15) >> 2) * 8 + (lane >> 5) * 4 + (vv & 3);
 }
 
+// ---- nearest centroid through decision thresholds -------------------------------------------------
+// The rule (quant.h: nearest_code) compares the distances to the two centroids that bracket y.  Both
+// rounded distances are monotone in y between two neighbouring centroids, so for every boundary k
+// there is one smallest float thr[k] from which on centroid k+1 wins, and
+// code(y) = #{k : y >= thr[k]} reproduces the rule bit for bit.  The thresholds are found once per
+// workgroup by bisection over the float bit patterns with the rule's own comparison.
+__device__ static inline int float_key(float f) {            // monotone map float -> int
+    const int b = __float_as_int(f);
+    return b ^ ((b >> 31) & 0x7fffffff);
+}
+__device__ static inline float key_float(int k) { return __int_as_float(k ^ ((k >> 31) & 0x7fffffff)); }
+
+__device__ static inline float decision_threshold(float c_lo, float c_hi) {
+    int lo = float_key(c_lo), hi = float_key(c_hi);          // rule false at c_lo, true at c_hi
+    while (hi - lo > 1) {
+        const int mid = lo + ((hi - lo) >> 1);
+        const float y = key_float(mid);
+        if (fabsf(y - c_hi) < fabsf(y - c_lo)) hi = mid; else lo = mid;
+    }
+    return key_float(hi);
+}
+
+// thresholds of width index li start at thr_offset(li): 3 + 7 + 15 + 255 floats
+__device__ static inline int thr_offset(int li) { return li == 0 ? 0 : li == 1 ? 3 : li == 2 ? 10 : 25; }
+#define QP_THR_FLOATS 280
+#ifndef QP_STAGGER_TICKS
+#define QP_STAGGER_TICKS 1700            // 17 us
+#endif
+
+template <int W> struct Coder {
+    static constexpr int K = 1 << W;
+    float t[(W <= 3) ? K - 1 : 1];
+    const float* thr;
+    __device__ inline Coder(const float* thr_li) : thr(thr_li) {
+        if constexpr (W <= 3) {
+#pragma unroll
+            for (int k = 0; k < K - 1; ++k) t[k] = thr_li[k];
+        }
+    }
+    __device__ inline uint32_t operator()(float y) const {
+        if constexpr (W <= 3) {
+            uint32_t c = 0;
+#pragma unroll
+            for (int k = 0; k < K - 1; ++k) c += (y >= t[k]) ? 1u : 0u;
+            return c;
+        } else {
+            int pos = 0;                                     // #thresholds <= y, by binary search
+#pragma unroll
+            for (int s = K / 2; s >= 1; s >>= 1)
+                if (y >= thr[pos + s - 1]) pos += s;
+            return (uint32_t)pos;
+        }
+    }
+};
+
 template <int W>
-__device__ static inline void stage_codes_k(const f32x32& a0, const f32x32& a1, const f32x32& a2, const f32x32& a3,
-                                            const float* cb, uint8_t* stage, int lane) {
+__device__ static __forceinline__ void stage_codes_k(const f32x32& a0, const f32x32& a1, const f32x32& a2, const f32x32& a3,
+                                            const float* thr, uint8_t* stage, int lane) {
+    const Coder<W> code(thr);
     const int c = lane & 31;
 #pragma unroll
     for (int vv = 0; vv < 32; ++vv) {
-        const uint32_t w = nearest_code<W>(a0[vv], cb) | (nearest_code<W>(a1[vv], cb) << 8) |
-                           (nearest_code<W>(a2[vv], cb) << 16) | (nearest_code<W>(a3[vv], cb) << 24);
+        const uint32_t w = code(a0[vv]) | (code(a1[vv]) << 8) | (code(a2[vv]) << 16) | (code(a3[vv]) << 24);
         *reinterpret_cast<uint32_t*>(stage + mfma_token(vv, lane) * CODE_ROW + 4 * c) = w;
     }
 }
 
 template <int W>
-__device__ static inline void stage_codes_v(const f32x32& acc, int g, const float* cb, uint8_t* stage, int lane) {
+__device__ static __forceinline__ void stage_codes_v(const f32x32& acc, int g, const float* thr, uint8_t* stage, int lane) {
+    const Coder<W> code(thr);
     const int c = lane & 31;
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-        const uint32_t w = nearest_code<W>(acc[4 * q], cb) | (nearest_code<W>(acc[4 * q + 1], cb) << 8) |
-                           (nearest_code<W>(acc[4 * q + 2], cb) << 16) | (nearest_code<W>(acc[4 * q + 3], cb) << 24);
+        const uint32_t w = code(acc[4 * q]) | (code(acc[4 * q + 1]) << 8) | (code(acc[4 * q + 2]) << 16) |
+                           (code(acc[4 * q + 3]) << 24);
         *reinterpret_cast<uint32_t*>(stage + (g * 32 + c) * CODE_ROW_T + mfma_token(4 * q, lane)) = w;
     }
 }
 
 template <int W>
-__device__ static inline void pack_store_k(const uint8_t* stage, uint8_t* kcodes, int tile, int lane) {
+__device__ static __forceinline__ void pack_store_k(const uint8_t* stage, uint8_t* kcodes, int tile, int lane) {
     uint32_t words[4 * W];
 #pragma unroll
     for (int k = 0; k < 4 * W; ++k) words[k] = 0;
@@ -264,7 +319,7 @@ __device__ static inline void pack_store_k(const uint8_t* stage, uint8_t* kcodes
 }
 
 template <int W>
-__device__ static inline void pack_store_v(const uint8_t* stage, uint8_t* vcodes, int tile, int lane, int lo, int hi) {
+__device__ static __forceinline__ void pack_store_v(const uint8_t* stage, uint8_t* vcodes, int tile, int lane, int lo, int hi) {
     uint8_t* dst = vcodes + (size_t)tile * (HD * 8 * W);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
@@ -338,8 +393,9 @@ template <int DT, int NW>
 __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     float* piT = reinterpret_cast<float*>(smem);                                   // [j][slot]
-    float* cbs = reinterpret_cast<float*>(smem + QP_PI_BYTES + NW * QP_STAGE);     // all widths
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float* thrs = reinterpret_cast<float*>(smem + QP_PI_BYTES + NW * QP_STAGE);    // all widths
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);          // wave-uniform: keep it in a scalar register
     uint8_t* stage = smem + QP_PI_BYTES + wave * QP_STAGE;
     const bool is_v = (blockIdx.x & 1) != 0;
 
@@ -353,12 +409,23 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
             const int slot = is_v ? ((i & 31) * 4 + (i >> 5)) : i;
             piT[j * HD + slot] = pi[idx];
         }
-        for (int i = tid; i < QP_CB_FLOATS; i += NW * 64) cbs[i] = a.cb[i];
+        for (int i = tid; i < QP_THR_FLOATS; i += NW * 64) {
+            const int li = i < 3 ? 0 : i < 10 ? 1 : i < 25 ? 2 : 3;
+            const int k = i - thr_offset(li);
+            thrs[i] = decision_threshold(a.cb[codebook_offset(li) + k], a.cb[codebook_offset(li) + k + 1]);
+        }
     }
     __syncthreads();
 
     const int total_tiles = a.tile_base[ODMKV_NQ];
     const int wg = blockIdx.x >> 1, n_wg = gridDim.x >> 1;
+    // Two waves share a SIMD and its matrix pipe.  Started together they would both load, then both
+    // queue for the pipe; the second one starts half a tile late so that one computes while the
+    // other loads, quantises and packs.  (A fixed wait on the 100 MHz wall clock; nothing is awaited.)
+    if (NW == 8 && wave >= 4 && wg * NW + wave + n_wg * NW < total_tiles) {
+        const long long until = wall_clock64() + QP_STAGGER_TICKS;
+        while (wall_clock64() < until) __builtin_amdgcn_s_sleep(32);
+    }
     for (int gt = wg * NW + wave; gt < total_tiles; gt += n_wg * NW) {
         int li = 0;
 #pragma unroll
@@ -381,9 +448,14 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
         } else {
             x.zero();
         }
-        float ss = 0.0f;
+        float ss = 0.0f, amin = INFINITY;                      // amin: smallest non-zero magnitude of the row
 #pragma unroll
-        for (int j = 0; j < HD; ++j) { const float xj = x.get(j); ss = __fmaf_rn(xj, xj, ss); }
+        for (int j = 0; j < HD; ++j) {
+            const float xj = x.get(j);
+            ss = __fmaf_rn(xj, xj, ss);
+            const float ax = fabsf(xj);
+            amin = fminf(amin, ax == 0.0f ? INFINITY : ax);
+        }
         const float norm = sqrtf(ss);
         const float den = norm + 1e-10f;
 
@@ -391,17 +463,64 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
 #pragma unroll
         for (int i = 0; i < 32; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; acc2[i] = 0.0f; acc3[i] = 0.0f; }
         const float4* __restrict__ brow = reinterpret_cast<const float4*>(piT) + (lane & 31);
+        // u_j = x_j / den, correctly rounded.  With den in [2^-40, 2^60] and every non-zero |x_j| at
+        // least den * 2^-60 the hardware division sequence never rescales its operands, so the part
+        // of it that depends on den alone (reciprocal estimate and its refinement) is computed once
+        // per row and five multiply-adds per element remain; the results are the same bits.  Rows
+        // outside that range (any lane of the wave) take the plain division.
+        const bool row_plain = !(den >= 9.094947017729282e-13f && den <= 1.152921504606847e18f &&
+                                 amin >= den * 8.673617379884035e-19f);
+        if (!__any(row_plain)) {
+            const float r0 = __builtin_amdgcn_rcpf(den);
+            const float rr = __fmaf_rn(__fmaf_rn(-den, r0, 1.0f), r0, r0);
+            const float nden = -den;
+            // Issue order is pinned: every matrix instruction is followed by a slice of the next
+            // step's operand preparation (LDS read, conversion, division), so the matrix pipe is
+            // handed its next instruction the moment it frees up.
+            float4 b = brow[0];
+            float u;
+            {
+                const float n0 = x.get(0);
+                const float q0 = __fmul_rn(n0, rr);
+                const float q1 = __fmaf_rn(__fmaf_rn(nden, q0, n0), rr, q0);
+                u = __fmaf_rn(__fmaf_rn(nden, q1, n0), rr, q1);
+            }
 #pragma unroll
-        for (int j = 0; j < HD; ++j) {
-            const float u = x.get(j) / den;
-            const float4 b = brow[j * (HD / 4)];
-            acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.x, acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.y, acc1, 0, 0, 0);
-            acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.z, acc2, 0, 0, 0);
-            acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.w, acc3, 0, 0, 0);
+            for (int j = 0; j < HD; ++j) {
+                float4 bn = b;
+                float un = u;
+                const int jn = j + 1 < HD ? j + 1 : j;
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.x, acc0, 0, 0, 0);
+                bn = brow[jn * (HD / 4)];
+                const float nn = x.get(jn);
+                const float q0 = __fmul_rn(nn, rr);
+                __builtin_amdgcn_sched_barrier(0);
+                acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.y, acc1, 0, 0, 0);
+                const float e2 = __fmaf_rn(nden, q0, nn);
+                const float q1 = __fmaf_rn(e2, rr, q0);
+                __builtin_amdgcn_sched_barrier(0);
+                acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.z, acc2, 0, 0, 0);
+                const float e3 = __fmaf_rn(nden, q1, nn);
+                un = __fmaf_rn(e3, rr, q1);
+                __builtin_amdgcn_sched_barrier(0);
+                acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.w, acc3, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                b = bn;
+                u = un;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < HD; ++j) {
+                const float u = x.get(j) / den;
+                const float4 b = brow[j * (HD / 4)];
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.x, acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.y, acc1, 0, 0, 0);
+                acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.z, acc2, 0, 0, 0);
+                acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.w, acc3, 0, 0, 0);
+            }
         }
 
-        const float* cb = cbs + codebook_offset(li);
+        const float* cb = thrs + thr_offset(li);
         if (!is_v) {
             switch (li) {
                 case 0: stage_codes_k<2>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
@@ -559,7 +678,7 @@ template <int DT>
 static int launch_quant(const QuantArgs& qa, hipStream_t st) {
     // fp32 rows take 128 registers on top of the 128 accumulators: one wave per SIMD then
     constexpr int NW = (DT == ODMKV_F32) ? 4 : 8;
-    const size_t lds = QP_PI_BYTES + (size_t)NW * QP_STAGE + QP_CB_FLOATS * sizeof(float);
+    const size_t lds = QP_PI_BYTES + (size_t)NW * QP_STAGE + QP_THR_FLOATS * sizeof(float);
     static bool attr_set = false;
     if (!attr_set) {
         ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&quant_pack_kernel<DT, NW>),

@@ -31,6 +31,28 @@ _LEVEL_INDEX = {2: 0, 3: 1, 4: 2, 8: 3, 16: 4}
 _TILE_BYTES = [TILE * 16 * w + 2 * TILE * 4 for w in WIDTHS] + [2 * TILE * HEAD_DIM * 2]
 
 
+class _Buffers:
+    """The store's buffers inside one allocation; tensor views are made when somebody asks."""
+
+    def __init__(self, arena: torch.Tensor, plan: dict):
+        self.arena = arena
+        self.plan = plan
+        self._base = arena.data_ptr()
+
+    def ptr(self, name: str, li) -> int:
+        return self._base + self.plan[(name, li)][0]
+
+    def view(self, name: str, li=None) -> torch.Tensor:
+        off, nbytes, dtype = self.plan[(name, li)]
+        return self.arena[off:off + nbytes].view(dtype)
+
+    def __getitem__(self, name: str):
+        if (name, None) in self.plan:
+            return self.view(name)
+        n = 5 if name in ("pos", "seg_tile", "seg_count") else 4
+        return [self.view(name, li) for li in range(n)]
+
+
 def _empty_positions(device) -> torch.Tensor:
     return torch.empty((0, 3), dtype=torch.long, device=device)
 
@@ -96,30 +118,31 @@ class TurboQuantAdaptiveKVCacheState:
         self._items = None
         self._packed = None
 
-    def _alloc(self, seg_tile: np.ndarray) -> dict:
+    def _alloc(self, seg_tile: np.ndarray) -> "_Buffers":
         """All buffers of the store as views into one allocation: the segment tables (one upload),
         the counters, norms and exact rows (zeroed), the positions (-1), then the codes (left as they
         come: every code the kernels read is written first or is a padding lane masked by count)."""
         dev = self.device
+        nseg = self._nseg
         n_tiles = [max(int(t), 1) for t in seg_tile[:, -1]]
-        exact_bytes = 2
-        plan, off = [], 0
+        plan, off = {}, 0
 
         def take(name, li, nbytes, dtype):
             nonlocal off
-            plan.append((name, li, off, nbytes, dtype))
+            plan[(name, li)] = (off, nbytes, dtype)
             off += (nbytes + 255) // 256 * 256
 
         for li in range(5):
-            take("seg_tile", li, (self._nseg + 1) * 4, torch.int32)
+            take("seg_tile", li, (nseg + 1) * 4, torch.int32)
+        tables_end = off
         for li in range(5):
-            take("seg_count", li, self._nseg * 4, torch.int32)
+            take("seg_count", li, nseg * 4, torch.int32)
         for li in range(4):
             take("knorm", li, n_tiles[li] * TILE * 4, torch.float32)
             take("vnorm", li, n_tiles[li] * TILE * 4, torch.float32)
         # exact rows take part in the products as they are (a zero weight does not silence a NaN)
-        take("kexact", None, n_tiles[4] * TILE * HEAD_DIM * exact_bytes, self._exact_torch_dtype)
-        take("vexact", None, n_tiles[4] * TILE * HEAD_DIM * exact_bytes, self._exact_torch_dtype)
+        take("kexact", None, n_tiles[4] * TILE * HEAD_DIM * 2, self._exact_torch_dtype)
+        take("vexact", None, n_tiles[4] * TILE * HEAD_DIM * 2, self._exact_torch_dtype)
         zero_end = off
         for li in range(5):
             take("pos", li, n_tiles[li] * TILE * 4, torch.int32)
@@ -140,21 +163,14 @@ class TurboQuantAdaptiveKVCacheState:
                 spare = torch.empty(off + off // 8, dtype=torch.uint8, device=dev)
             arena, self._arena_spare = spare, arena
         self._arena = arena
-        tables_end = plan[5][2]
         table = np.zeros(tables_end // 4, np.int32)
-        for name, li, o, nbytes, _ in plan[:5]:
-            table[o // 4:o // 4 + self._nseg + 1] = seg_tile[li]
+        for li in range(5):
+            o = plan[("seg_tile", li)][0] // 4
+            table[o:o + nseg + 1] = seg_tile[li]
         arena[:tables_end].view(torch.int32).copy_(torch.from_numpy(table))
         arena[tables_end:zero_end].zero_()
         arena[zero_end:pos_end].view(torch.int32).fill_(-1)
-        bufs = {"seg_tile": [], "seg_count": [], "pos": [], "kcodes": [], "vcodes": [], "knorm": [], "vnorm": []}
-        for name, li, o, nbytes, dtype in plan:
-            view = arena[o:o + nbytes].view(dtype)
-            if li is None:
-                bufs[name] = view
-            else:
-                bufs[name].append(view)
-        return bufs
+        return _Buffers(arena, plan)
 
     def _make_struct(self) -> None:
         p = Packed()
@@ -163,16 +179,16 @@ class TurboQuantAdaptiveKVCacheState:
         b = self._bufs
         for li in range(5):
             p.n_tiles[li] = int(self._seg_tile[li, -1])
-            p.pos[li] = b["pos"][li].data_ptr()
-            p.seg_tile[li] = b["seg_tile"][li].data_ptr()
-            p.seg_count[li] = b["seg_count"][li].data_ptr()
+            p.pos[li] = b.ptr("pos", li)
+            p.seg_tile[li] = b.ptr("seg_tile", li)
+            p.seg_count[li] = b.ptr("seg_count", li)
             if li < 4:
-                p.kcodes[li] = b["kcodes"][li].data_ptr()
-                p.vcodes[li] = b["vcodes"][li].data_ptr()
-                p.knorm[li] = b["knorm"][li].data_ptr()
-                p.vnorm[li] = b["vnorm"][li].data_ptr()
-        p.kexact = b["kexact"].data_ptr()
-        p.vexact = b["vexact"].data_ptr()
+                p.kcodes[li] = b.ptr("kcodes", li)
+                p.vcodes[li] = b.ptr("vcodes", li)
+                p.knorm[li] = b.ptr("knorm", li)
+                p.vnorm[li] = b.ptr("vnorm", li)
+        p.kexact = b.ptr("kexact", None)
+        p.vexact = b.ptr("vexact", None)
         self._packed = p
 
     def _capacity_tiles(self, counts: np.ndarray) -> np.ndarray:
