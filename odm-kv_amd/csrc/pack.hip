@@ -245,9 +245,6 @@ __device__ static inline float decision_threshold(float c_lo, float c_hi) {
 // thresholds of width index li start at thr_offset(li): 3 + 7 + 15 + 255 floats
 __device__ static inline int thr_offset(int li) { return li == 0 ? 0 : li == 1 ? 3 : li == 2 ? 10 : 25; }
 #define QP_THR_FLOATS 280
-#ifndef QP_STAGGER_TICKS
-#define QP_STAGGER_TICKS 1700            // 17 us
-#endif
 
 template <int W> struct Coder {
     static constexpr int K = 1 << W;
@@ -419,13 +416,6 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
 
     const int total_tiles = a.tile_base[ODMKV_NQ];
     const int wg = blockIdx.x >> 1, n_wg = gridDim.x >> 1;
-    // Two waves share a SIMD and its matrix pipe.  Started together they would both load, then both
-    // queue for the pipe; the second one starts half a tile late so that one computes while the
-    // other loads, quantises and packs.  (A fixed wait on the 100 MHz wall clock; nothing is awaited.)
-    if (NW == 8 && wave >= 4 && wg * NW + wave + n_wg * NW < total_tiles) {
-        const long long until = wall_clock64() + QP_STAGGER_TICKS;
-        while (wall_clock64() < until) __builtin_amdgcn_s_sleep(32);
-    }
     for (int gt = wg * NW + wave; gt < total_tiles; gt += n_wg * NW) {
         int li = 0;
 #pragma unroll
@@ -595,23 +585,23 @@ __global__ __launch_bounds__(64) void exact_gather_kernel(ExactArgs a) {
     const size_t slot = (size_t)tile * TILE + lane;
     const int t = a.pos[slot] - a.pos_offset;
     const size_t off = (size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH + (size_t)t * a.sT;
-    const typename Elem<DT>::raw* kr = reinterpret_cast<const typename Elem<DT>::raw*>(a.K) + off;
-    const typename Elem<DT>::raw* vr = reinterpret_cast<const typename Elem<DT>::raw*>(a.V) + off;
     uint16_t* kd = a.kexact + (size_t)tile * TILE * HD;
     uint16_t* vd = a.vexact + (size_t)tile * TILE * HD;
-    for (int c = 0; c < 16; ++c) {
-        uint16_t tmp[8];
+    float x[HD];
+    load_row<DT>(a.K, off, x);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) tmp[e] = to_store16<DT, ODT>(kr[8 * c + e]);
+    for (int c = 0; c < 16; ++c) {
         uint4 pk;
-        pk.x = tmp[0] | ((uint32_t)tmp[1] << 16);
-        pk.y = tmp[2] | ((uint32_t)tmp[3] << 16);
-        pk.z = tmp[4] | ((uint32_t)tmp[5] << 16);
-        pk.w = tmp[6] | ((uint32_t)tmp[7] << 16);
+        pk.x = Elem<ODT>::from_f32(x[8 * c]) | ((uint32_t)Elem<ODT>::from_f32(x[8 * c + 1]) << 16);
+        pk.y = Elem<ODT>::from_f32(x[8 * c + 2]) | ((uint32_t)Elem<ODT>::from_f32(x[8 * c + 3]) << 16);
+        pk.z = Elem<ODT>::from_f32(x[8 * c + 4]) | ((uint32_t)Elem<ODT>::from_f32(x[8 * c + 5]) << 16);
+        pk.w = Elem<ODT>::from_f32(x[8 * c + 6]) | ((uint32_t)Elem<ODT>::from_f32(x[8 * c + 7]) << 16);
         *reinterpret_cast<uint4*>(kd + ((size_t)c * TILE + lane) * 8) = pk;
     }
+    load_row<DT>(a.V, off, x);
+#pragma unroll
     for (int j = 0; j < HD; ++j)
-        vd[((size_t)(lane >> 2) * HD + j) * 4 + (lane & 3)] = to_store16<DT, ODT>(vr[j]);
+        vd[((size_t)(lane >> 2) * HD + j) * 4 + (lane & 3)] = Elem<ODT>::from_f32(x[j]);
 }
 
 // one new token per (b, h) behind the stored exact tokens

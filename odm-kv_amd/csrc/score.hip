@@ -201,14 +201,25 @@ __global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
     }
 }
 
-__global__ __launch_bounds__(128) void score_obar_kernel(ScoreArgs a) {
-    const int h = blockIdx.x, j = threadIdx.x;
+__global__ __launch_bounds__(1024) void score_obar_kernel(ScoreArgs a) {
+    // 8 groups of 128 threads take every eighth chunk, then the groups are added in order
+    __shared__ float part_o[8][HD];
+    __shared__ float part_p[8];
+    const int h = blockIdx.x, j = threadIdx.x & (HD - 1), grp = threadIdx.x >> 7;
     float acc = 0.0f, P = 0.0f;
-    for (int c = 0; c < a.nchunks; ++c) {
+    for (int c = grp; c < a.nchunks; c += 8) {
         acc += a.opart[((size_t)h * a.nchunks + c) * HD + j];
         P += a.psum[(size_t)h * a.nchunks + c];
     }
-    a.obar[h * HD + j] = acc / fmaxf(P, 1e-8f);
+    part_o[grp][j] = acc;
+    if (j == 0) part_p[grp] = P;
+    __syncthreads();
+    if (grp == 0) {
+        float o = 0.0f, p = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) { o += part_o[g][j]; p += part_p[g]; }
+        a.obar[h * HD + j] = o / fmaxf(p, 1e-8f);
+    }
 }
 
 // ---- pass 2 over V: |v|^2, |v - obar|^2, the score, and its global maximum ----
@@ -299,7 +310,7 @@ static int run_score(ScoreArgs& a, hipStream_t st) {
     if (a.G <= 4) hipLaunchKernelGGL((score_pv_kernel<DT, 4>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((score_pv_kernel<DT, 8>), grid, block, 0, st, a);
     ODMKV_CHECK_LAUNCH("score_pv_kernel");
-    hipLaunchKernelGGL(score_obar_kernel, dim3(a.Hkv), dim3(128), 0, st, a);
+    hipLaunchKernelGGL(score_obar_kernel, dim3(a.Hkv), dim3(1024), 0, st, a);
     ODMKV_CHECK_LAUNCH("score_obar_kernel");
     hipLaunchKernelGGL((score_final_kernel<DT>), grid, block, 0, st, a);
     ODMKV_CHECK_LAUNCH("score_final_kernel");
