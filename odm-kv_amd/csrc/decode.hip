@@ -129,6 +129,10 @@ __device__ static inline float head_sum(float v) {
     return v;
 }
 
+// workgroup barrier that orders LDS traffic only: global loads issued before it stay in flight
+// (__syncthreads would first wait for every outstanding load of the wavefront)
+__device__ static inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 #define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_4x4x4f16((a), (b), (c), 0, 0, 0)
 #define MFMA_BCAST(a, b, c, s) __builtin_amdgcn_mfma_f32_4x4x4f16((a), (b), (c), 4, (s), 0)
 
@@ -328,8 +332,12 @@ __device__ static inline void compute_tile(const TileData<W>& t, int nvalid, int
 
 // stage the group's queries (fp16 high/low halves per 4-dim step) in LDS; heads beyond the group are 0
 template <int NP>
-__device__ static inline void stage_queries(const DecodeArgs& a, const uint4* src, uint4* qsh, int tid) {
-    if (tid < 4 * NP * 32) qsh[tid] = (tid >> 5) < a.G ? src[tid] : make_uint4(0u, 0u, 0u, 0u);
+__device__ static inline uint4 load_query_slice(const DecodeArgs& a, const uint4* src, int tid) {
+    return (tid < 4 * NP * 32 && (tid >> 5) < a.G) ? src[tid] : make_uint4(0u, 0u, 0u, 0u);
+}
+template <int NP>
+__device__ static inline void stage_queries(uint4 v, uint4* qsh, int tid) {
+    if (tid < 4 * NP * 32) qsh[tid] = v;
 }
 template <int NP>
 __device__ static inline void fetch_queries(const uint4* qsh, int lane, h4* qr, h4* ql) {
@@ -351,6 +359,9 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
     const float vsc = a.inv_s[li], ksc = a.inv_s[li] * a.scaling * LOG2E;
+    // loads return in issue order: the (small) query slice goes first so that staging it does not
+    // have to wait for the tiles
+    const uint4 qslice = load_query_slice<NP>(a, a.qrot + (size_t)bq0 * 32, tid);
     TileData<W> cur;
     int tt = wave;
     int nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
@@ -364,9 +375,9 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
         nv1 = tt + NWAVES < ntiles ? min(ntok - (tt + NWAVES) * TILE, TILE) : 0;
         if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + NWAVES, lane);
     }
-    stage_queries<NP>(a, a.qrot + (size_t)bq0 * 32, qsh, tid);
+    stage_queries<NP>(qslice, qsh, tid);
     build_lut<W>(lut, a, tid);
-    __syncthreads();
+    lds_barrier();
     TRACE(1)
     h4 qr[NP * 32], ql[NP * 32];
     fetch_queries<NP>(qsh, lane, qr, ql);
@@ -416,7 +427,7 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
     const bool bf = a.s.exact_dtype == ODMKV_BF16;
     const float esc = a.scaling * LOG2E;
     const int count = a.s.seg_count[4][bh];          // exact segments grow between work-list rebuilds
-    stage_queries<NP>(a, a.qs + (size_t)bq0 * 32, qsh, tid);
+    stage_queries<NP>(load_query_slice<NP>(a, a.qs + (size_t)bq0 * 32, tid), qsh, tid);
     __syncthreads();
     h4 qr[NP * 32], ql[NP * 32];
     fetch_queries<NP>(qsh, lane, qr, ql);
