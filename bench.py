@@ -11,7 +11,8 @@ over all layers' packed caches, launched layer after layer on one stream.  The p
 
 Prints ONE JSON line:
   value          whole-job GB/s = packed bytes of all layers / mean step time (prep + main + merge
-                 kernels and launch gaps included; inputs resident in HBM)
+                 kernels and launch gaps included; inputs resident in HBM; the step is replayed as
+                 one HIP graph unless --no-graph)
   roofline       the main streaming kernel alone: packed bytes per launch / its mean duration from
                  HIP events recorded around it on its own stream, against 8 TB/s
   cpu_baseline   the oracle's restatement of the reference's CPU decode step (SDPA over the
@@ -34,6 +35,10 @@ for p in (ROOT, os.path.join(ROOT, "odm-kv_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the main decode kernel on the default workload, from the L2 counters
+# (FETCH_SIZE and WRITE_SIZE, one rocprofv3 --pmc run each, scaled by a 256 MiB copy of known size):
+# 20.41 MB fetched + 1.10 MB written.  Applies to --layers 32 --ctx 32768 --target 2.0 only.
+MEASURED_TRAFFIC_BYTES = 21.51e6
 LEVELS = (0, 2, 3, 4, 8, 16)
 
 
@@ -132,13 +137,17 @@ def cpu_baseline(sample_T, n_kv, n_q, eps, threads):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-graph", action="store_true", help="launch every step from Python instead of replaying a HIP graph")
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--target", type=float, default=2.0)
     ap.add_argument("--cpu-sample-ctx", type=int, default=8192)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="for counter runs under rocprofv3 --pmc: a few eager decode steps and one plain 256 MiB "
+                         "device copy (the calibration kernel), nothing else timed")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the path: every box in this build has one GPU and "
@@ -208,20 +217,70 @@ def main() -> int:
         for st, q in zip(states, qs):
             st.decode_attention(q)
 
+    def collect_kernel_ms(n_launches, fn):
+        """Durations of the main streaming kernel from the library's HIP events (launch stream)."""
+        _lib.check(_lib.lib.odmkv_profile_enable(n_launches + 8))
+        fn()
+        torch.cuda.synchronize()
+        buf = (C.c_float * (n_launches + 8))()
+        n = C.c_int(0)
+        _lib.check(_lib.lib.odmkv_profile_collect(buf, len(buf), C.byref(n)))
+        _lib.check(_lib.lib.odmkv_profile_disable())
+        return sorted(buf[i] for i in range(n.value))
+
+    if args.traffic_probe:
+        for _ in range(3):
+            step()
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"traffic_probe": True, "packed_bytes_per_layer": int(packed_bytes / NL), "copy_bytes": 256 << 20}))
+        return 0
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    _lib.check(_lib.lib.odmkv_profile_enable(args.steps * NL + 8))
+
+    # the timed region replays one captured step (96 kernels) so that the host's per-call work does
+    # not sit between the kernels; falls back to launching from Python if capture is not possible
+    graph, launch_mode = None, "python"
+    if not args.no_graph:
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                step()
+            g.replay()
+            torch.cuda.synchronize()
+            graph, launch_mode = g, "hip graph"
+        except Exception as exc:                                   # noqa: BLE001
+            print(f"graph capture not available ({exc}); timing eager launches", file=sys.stderr)
+            torch.cuda.synchronize()
+    run = graph.replay if graph is not None else step
+    for _ in range(3):
+        run()
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        run()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    buf = (C.c_float * (args.steps * NL + 8))()
-    n = C.c_int(0)
-    _lib.check(_lib.lib.odmkv_profile_collect(buf, len(buf), C.byref(n)))
-    _lib.check(_lib.lib.odmkv_profile_disable())
-    kernel_ms = [buf[i] for i in range(n.value)]
+
+    # kernel durations: an eager pass over the same rotating 32 buffers, then one buffer alone (cache-resident)
+    prof_steps = min(args.steps, 20)
+    kernel_ms = collect_kernel_ms(prof_steps * NL, lambda: [step() for _ in range(prof_steps)])
+    hot_ms = collect_kernel_ms(200, lambda: [states[0].decode_attention(qs[0]) for _ in range(200)])
+
+    def pct(v, p):
+        return v[min(len(v) - 1, int(p / 100.0 * len(v)))]
+
     ms_per_step = elapsed / args.steps * 1e3
     value = packed_bytes / (elapsed / args.steps) / 1e9
     bytes_per_launch = packed_bytes / NL
@@ -232,10 +291,10 @@ def main() -> int:
         "metric": "LUT decode-attn achieved GB/s (% HBM peak); ms to score+pack a 32k-token layer",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "u8 codes, f32 accumulate", "data": "synthetic",
+        "dtype": "f16 products, f32 accumulate (2/3/4/8-bit codes)", "data": "synthetic",
         "config": {"workload": f"c2 kernel-only: {NL} layers x [Hkv 8, T {T}, d 128] fp16, Hq 32, {args.target} avg bits, "
                                "1 decode token per step over all layers' packed caches",
-                   "levels": list(LEVELS), "n_sink": 4, "window": 128},
+                   "levels": list(LEVELS), "n_sink": 4, "window": 128, "launch": launch_mode},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "packed_bytes_per_layer": int(bytes_per_launch),
         "level_counts": counts,
@@ -243,9 +302,12 @@ def main() -> int:
         "stage_ms": {k: round(statistics.median(v) * 1e3, 3) for k, v in t_stage.items()},
         "parity": {"gate_attn_rel_err": gate_err, "full_size_fused_vs_dense_rel_err": full_err},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES if (NL, T, args.target) == (32, 32768, 2.0) else None,
                      "kernel": "decode_main_kernel", "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
-                     "launches": len(kernel_ms)},
+                     "kernel_median_us": round(pct(kernel_ms, 50) * 1e3, 2), "kernel_p10_us": round(pct(kernel_ms, 10) * 1e3, 2),
+                     "kernel_p90_us": round(pct(kernel_ms, 90) * 1e3, 2), "launches": len(kernel_ms),
+                     "single_buffer_cache_resident_median_us": round(pct(hot_ms, 50) * 1e3, 2)},
     }
     if not args.no_cpu:
         threads = os.cpu_count() or 1
