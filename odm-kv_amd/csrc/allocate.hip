@@ -607,7 +607,8 @@ extern "C" int odmkv_allocate(const float* scores, int rows, int n,
     }
     ODMKV_CHECK_ARG(sink_mask || n_sink == 0 || (period > 0 && n % period == 0 && n_sink <= period),
                     "allocate: bad sink pattern period=%d n_sink=%d n=%d", period, n_sink, n);
-    ODMKV_CHECK_ARG((double)n * 16.0 < 16777216.0, "allocate: rows longer than 1,048,575 tokens lose exactness of the fp32 mean");
+    // bit sums up to 2^24 are exact in fp32, which the fp32 mean of the host formulation relies on
+    ODMKV_CHECK_ARG((double)n * 16.0 <= 16777216.0, "allocate: rows longer than 1,048,576 tokens lose exactness of the fp32 mean");
     ODMKV_CHECK_ARG(rows <= 65535, "allocate: at most 65535 rows per call");
     ODMKV_CHECK_ARG(workspace_bytes >= odmkv_allocate_workspace_bytes(rows, n), "allocate: workspace too small");
     hipStream_t st = (hipStream_t)stream;

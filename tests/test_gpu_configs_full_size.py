@@ -1,0 +1,141 @@
+"""GPU: the benchmark configurations at their full sizes, through properties that do not need the
+CPU oracle to run at that size (it would take minutes): the allocation against the oracle allocator on
+the GPU's own scores (bit exact; the oracle allocator is fast), budget and sink/window invariants,
+the partition of every position over the levels, and the fused decode attention against dense
+attention over the store's own dequantised tensors (<= 1e-3 relative, the stated tolerance).
+"""
+import numpy as np
+import pytest
+import torch
+
+import synthetic
+from oracle import allocator as oal
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+LEVELS = (0, 2, 3, 4, 8, 16)
+EPS = {0: 1.0, 2: 0.12022445693985273, 3: 0.037507650590957564, 4: 0.012159048378616812,
+       8: 0.0011957171333694236, 16: 0.0}
+ATTN_RTOL = 1e-3
+
+
+def _compress(layers, targets, window=128):
+    """layers: list of synthetic.Layer (one per sequence).  Returns (state, bits [B,H,T], scores [B,H,T])."""
+    from kvquant.allocator import optimal_scores_to_bits_batched
+    from kvquant.scorer import _launch_score
+    from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+    H, T, _ = layers[0].keys.shape
+    k = torch.stack([L.keys for L in layers]).to(DEV)
+    v = torch.stack([L.values for L in layers]).to(DEV)
+    scores = torch.stack([_launch_score(k[b], v[b], layers[b].mu.to(DEV), None, layers[b].n_q_heads, 4, 1e-2)
+                          for b in range(len(layers))])
+    bits = optimal_scores_to_bits_batched(scores.reshape(len(layers), -1), LEVELS, list(targets), EPS, n_sink=4,
+                                          period=T, eviction_cost=0.5).reshape(len(layers), H, T)
+    stored = bits.clone()
+    stored[..., -window:] = 16
+    st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=DEV, dtype=torch.float16, key_quantizer="mse",
+                                        value_quantizer="mse", seed=42)
+    st.prefill(k, v, stored)
+    return st, bits, stored, scores
+
+
+def _dense_attention(st, q, G):
+    # dequantised in fp32: the fp16 cast of materialize() would put its own 2^-11 rounding on every
+    # key, which large-norm keys (c5 scales four key channels by 20) turn into visible logit errors
+    kd = torch.zeros(st.batch_size, st.num_heads, st.seq_len, 128, dtype=torch.float32, device=DEV)
+    vd = torch.zeros_like(kd)
+    st._dequant_into(kd, vd, True)
+    vis = st.visible_mask()
+    out = torch.empty(q.shape, dtype=torch.float32, device=DEV)
+    for b in range(q.shape[0]):                       # one sequence at a time keeps the temporaries small
+        kb = kd[b].float().repeat_interleave(G, dim=0)
+        vb = vd[b].float().repeat_interleave(G, dim=0)
+        logits = torch.einsum("hd,htd->ht", q[b].float(), kb) / 128 ** 0.5
+        logits = logits.masked_fill(~vis[b].repeat_interleave(G, dim=0), float("-inf"))
+        out[b] = torch.einsum("ht,htd->hd", torch.softmax(logits, -1), vb)
+    return out
+
+
+def _check_attention(st, layers, G):
+    q = torch.stack([L.query for L in layers]).to(DEV)
+    fused = st.decode_attention(q)
+    dense = _dense_attention(st, q, G)
+    err = ((fused - dense).norm(dim=-1) / dense.norm(dim=-1)).max().item()
+    assert err < ATTN_RTOL, err
+    return err
+
+
+def _check_levels(st, stored):
+    lm = st._level_map
+    assert torch.equal(lm.to(torch.int32), stored)
+    counts = st.level_counts()
+    assert sum(counts.values()) == stored.numel()
+    for b in LEVELS:
+        assert counts[b] == int((stored == b).sum())
+
+
+def test_c3_sixteen_sequences_with_cycling_budgets():
+    layers = [synthetic.config("c3", seq=s) for s in range(16)]
+    targets = [synthetic.C3_TARGETS[s % 3] for s in range(16)]
+    st, bits, stored, scores = _compress(layers, targets)
+    H, T = 8, 8192
+    sink = torch.zeros(H, T, dtype=torch.bool)
+    sink[:, :4] = True
+    for s in (0, 1, 2, 7, 15):                         # the oracle allocator on the same scores: bit exact
+        want = oal.optimal_scores_to_bits(scores[s].cpu(), LEVELS, targets[s], EPS, sink, eviction_cost=0.5)
+        assert torch.equal(bits[s].cpu(), want), f"sequence {s}"
+    n_active = H * (T - 4)
+    for s in range(16):
+        got = bits[s, :, 4:].sum().item() / n_active
+        assert abs(got - targets[s]) * n_active <= 8, (s, got)
+        assert (bits[s, :, :4] == 16).all()
+    _check_levels(st, stored)
+    _check_attention(st, layers, 4)
+
+
+def test_c4_long_context_heavy_eviction():
+    L = synthetic.config("c4")
+    st, bits, stored, scores = _compress([L], [2.0])
+    evicted = (bits == 0).float().mean().item()
+    assert 0.30 <= evicted <= 0.50, evicted              # the configuration is built to evict about 40 %
+    n_active = 8 * (131072 - 4)
+    assert abs(bits[0, :, 4:].sum().item() - 2.0 * n_active) <= 8
+    sink = torch.zeros(8, 131072, dtype=torch.bool)
+    sink[:, :4] = True
+    want = oal.optimal_scores_to_bits(scores[0].cpu(), LEVELS, 2.0, EPS, sink, eviction_cost=0.5)
+    assert torch.equal(bits[0].cpu(), want)
+    _check_levels(st, stored)
+    masked = st.masked_key_indices()
+    assert masked[0].numel() == int((stored == 0).sum())
+    _check_attention(st, [L], 4)
+    # 128 decode steps keep new tokens exact and visible
+    g = torch.Generator().manual_seed(9)
+    for step in range(3):
+        kn = torch.randn(1, 8, 1, 128, generator=g).half().to(DEV)
+        st.append_all_exact(kn, torch.randn(1, 8, 1, 128, generator=g).half().to(DEV))
+    assert st.seq_len == 131072 + 3
+    _check_attention(st, [L], 4)
+
+
+def test_c5_group_of_seven_heavy_tailed_values():
+    L = synthetic.config("c5")
+    st, bits, stored, scores = _compress([L], [3.0])
+    n_active = 4 * (32768 - 4)
+    assert abs(bits[0, :, 4:].sum().item() - 3.0 * n_active) <= 8
+    sink = torch.zeros(4, 32768, dtype=torch.bool)
+    sink[:, :4] = True
+    want = oal.optimal_scores_to_bits(scores[0].cpu(), LEVELS, 3.0, EPS, sink, eviction_cost=0.5)
+    assert torch.equal(bits[0].cpu(), want)
+    used = {b for b in LEVELS if (stored == b).any()}
+    assert len(used) >= 4, used                          # a 3-bit budget on heavy tails spreads over the levels
+    _check_levels(st, stored)
+    _check_attention(st, [L], 7)
+
+
+def test_c2_one_layer_score_matches_oracle_at_full_size():
+    from oracle import scorer as osc
+    L = synthetic.config("c2", layer=3)
+    from kvquant.scorer import _launch_score
+    got = _launch_score(L.keys.to(DEV), L.values.to(DEV), L.mu.to(DEV), None, 32, 4, 1e-2).cpu()
+    want = osc.risk_score_from_mu(L.keys.float(), L.values.float(), L.mu.unsqueeze(0), 32)
+    np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=1e-3, atol=0)
