@@ -153,26 +153,36 @@ __device__ static inline float pick(const float* t, uint32_t idx) {
     return v;
 }
 
+// Thread tid computes table entry tid; the entry is then replicated over its row.  A thread writing
+// its own row would put all lanes of a wavefront on the same banks (rows are 256 or 128 bytes
+// apart), so the wavefront writes row after row instead: the lanes of one store instruction cover
+// consecutive 16-byte pieces of four (eight) rows, and fetch the row's entry from its owner by a
+// cross-lane read.
 template <int W>
 __device__ static inline void build_lut(uint8_t* lut, const DecodeArgs& a, int tid) {
+    const int lane = tid & 63, wave = tid >> 6;
     if constexpr (W == 2) {
         uint32_t h[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) h[k] = half_bits(pick<4>(a.cbs, (tid >> (2 * k)) & 3));
-        const uint4 v = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-        uint4* dst = reinterpret_cast<uint4*>(lut + tid * 256);
+        const uint32_t lo = h[0] | (h[1] << 16), hi = h[2] | (h[3] << 16);
 #pragma unroll
-        for (int s = 0; s < 16; ++s) dst[s] = v;
+        for (int i = 0; i < 16; ++i) {
+            const int src = i * 4 + (lane >> 4);
+            const uint32_t x = __shfl(lo, src, WAVE), y = __shfl(hi, src, WAVE);
+            *reinterpret_cast<uint4*>(lut + (wave * 64 + src) * 256 + (lane & 15) * 16) = make_uint4(x, y, x, y);
+        }
     } else {
         uint32_t v;
-        bool on = true;
-        if constexpr (W == 3) { on = tid < 64; v = half_bits(pick<8>(a.cbs + 4, tid & 7)) | (half_bits(pick<8>(a.cbs + 4, (tid >> 3) & 7)) << 16); }
+        if constexpr (W == 3) { v = half_bits(pick<8>(a.cbs + 4, tid & 7)) | (half_bits(pick<8>(a.cbs + 4, (tid >> 3) & 7)) << 16); }
         else if constexpr (W == 4) { v = half_bits(pick<16>(a.cbs + 12, tid & 15)) | (half_bits(pick<16>(a.cbs + 12, tid >> 4)) << 16); }
         else { v = half_bits(a.cb[codebook_offset(3) + tid]) * 0x10001u; }
-        if (on) {
-            uint4* dst = reinterpret_cast<uint4*>(lut + tid * 128);
+        const bool on = W != 3 || wave == 0;              // the 3-bit table has 64 entries
 #pragma unroll
-            for (int s = 0; s < 8; ++s) dst[s] = make_uint4(v, v, v, v);
+        for (int i = 0; i < 8; ++i) {
+            const int src = i * 8 + (lane >> 3);
+            const uint32_t x = __shfl(v, src, WAVE);
+            if (on) *reinterpret_cast<uint4*>(lut + (wave * 64 + src) * 128 + (lane & 7) * 16) = make_uint4(x, x, x, x);
         }
     }
 }
@@ -375,8 +385,8 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
         nv1 = tt + NWAVES < ntiles ? min(ntok - (tt + NWAVES) * TILE, TILE) : 0;
         if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + NWAVES, lane);
     }
+    build_lut<W>(lut, a, tid);                 // needs nothing from memory: runs while the query slice is on its way
     stage_queries<NP>(qslice, qsh, tid);
-    build_lut<W>(lut, a, tid);
     lds_barrier();
     TRACE(1)
     h4 qr[NP * 32], ql[NP * 32];
@@ -407,69 +417,106 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
 }
 
 // ---- exact (fp16 / bf16) tiles ---------------------------------------------------------------------
-#define PV_EXACT_STEP(s)                                                                         \
-    {                                                                                            \
-        uint2 r0 = *reinterpret_cast<const uint2*>(vsrc + ((size_t)(s) * HD + lane) * 4);        \
-        uint2 r1 = *reinterpret_cast<const uint2*>(vsrc + ((size_t)(s) * HD + lane + 64) * 4);   \
-        if (bf) { r0.x = bf16x2_to_f16x2(r0.x); r0.y = bf16x2_to_f16x2(r0.y);                    \
-                  r1.x = bf16x2_to_f16x2(r1.x); r1.y = bf16x2_to_f16x2(r1.y); }                  \
-        const h4 b0 = as_h4(r0.x, r0.y), b1 = as_h4(r1.x, r1.y);                                 \
-        _Pragma("unroll") for (int p = 0; p < NP; ++p) {                                         \
-            st.acc[p][0] = MFMA_BCAST(pa[p], b0, st.acc[p][0], (s));                             \
-            st.acc[p][1] = MFMA_BCAST(pa[p], b1, st.acc[p][1], (s));                             \
-        }                                                                                        \
-    }
+// One exact tile in registers: 64 tokens x 128 dims of keys (token-major chunks) and of values
+// (dim-major groups of four tokens).  Everything is requested at once; the products then run
+// without touching memory again.
+struct ExactTile {
+    uint4 k[16];
+    uint2 v[16][2];
+};
 
+__device__ static inline void load_exact_tile(ExactTile& t, const DecodeArgs& a, int tile, int lane) {
+    const uint16_t* ksrc = a.s.kexact + (size_t)tile * TILE * HD;
+    const uint16_t* vsrc = a.s.vexact + (size_t)tile * TILE * HD;
+#pragma unroll
+    for (int c = 0; c < 16; ++c) t.k[c] = *reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 8);
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        t.v[s][0] = *reinterpret_cast<const uint2*>(vsrc + ((size_t)s * HD + lane) * 4);
+        t.v[s][1] = *reinterpret_cast<const uint2*>(vsrc + ((size_t)s * HD + lane + 64) * 4);
+    }
+}
+
+template <int NP>
+__device__ static inline void compute_exact_tile(const ExactTile& t, bool bf, int nvalid, int lane, float esc,
+                                                 const h4* qr, WaveState<NP>& st) {
+    f4 dk[NP][4];
+#pragma unroll
+    for (int p = 0; p < NP; ++p)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) dk[p][c] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+        uint4 v = t.k[c];
+        if (bf) { v.x = bf16x2_to_f16x2(v.x); v.y = bf16x2_to_f16x2(v.y); v.z = bf16x2_to_f16x2(v.z); v.w = bf16x2_to_f16x2(v.w); }
+        const h4 k0 = as_h4(v.x, v.y), k1 = as_h4(v.z, v.w);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            dk[p][(2 * c) & 3] = MFMA(k0, qr[p * 32 + 2 * c], dk[p][(2 * c) & 3]);
+            dk[p][(2 * c + 1) & 3] = MFMA(k1, qr[p * 32 + 2 * c + 1], dk[p][(2 * c + 1) & 3]);
+        }
+    }
+    const int tok0 = lane & ~3;
+    h4 pa[NP];
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const f4 d = (dk[p][0] + dk[p][1]) + (dk[p][2] + dk[p][3]);
+        f4 logit, vn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            logit[i] = tok0 + i < nvalid ? d[i] * esc : -INFINITY;
+            vn[i] = tok0 + i < nvalid ? 1.0f : 0.0f;
+        }
+        pa[p] = softmax_step<NP>(st, p, logit, vn);
+    }
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+        uint2 r0 = t.v[s][0], r1 = t.v[s][1];
+        if (bf) { r0.x = bf16x2_to_f16x2(r0.x); r0.y = bf16x2_to_f16x2(r0.y);
+                  r1.x = bf16x2_to_f16x2(r1.x); r1.y = bf16x2_to_f16x2(r1.y); }
+        const h4 b0 = as_h4(r0.x, r0.y), b1 = as_h4(r1.x, r1.y);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            // the A operand of step s comes from quad s; the broadcast selector must be a constant
+            switch (s) {
+#define ODMKV_CASE(S) case S: st.acc[p][0] = MFMA_BCAST(pa[p], b0, st.acc[p][0], S); st.acc[p][1] = MFMA_BCAST(pa[p], b1, st.acc[p][1], S); break;
+                ODMKV_CASE(0) ODMKV_CASE(1) ODMKV_CASE(2) ODMKV_CASE(3) ODMKV_CASE(4) ODMKV_CASE(5) ODMKV_CASE(6) ODMKV_CASE(7)
+                ODMKV_CASE(8) ODMKV_CASE(9) ODMKV_CASE(10) ODMKV_CASE(11) ODMKV_CASE(12) ODMKV_CASE(13) ODMKV_CASE(14) ODMKV_CASE(15)
+#undef ODMKV_CASE
+            }
+        }
+    }
+}
+
+// Exact (16-bit) tokens: the query is the fp16-rounded one itself (its low halves are zero), so only
+// the high halves are fetched.  The first tile's loads are issued before anything is waited for.
 template <int NP>
 __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int bq0, int tile0, int ntiles, int seg_first,
                                               int tid, uint4* qsh, WaveState<NP>& st) {
     const int wave = tid >> 6, lane = tid & 63;
     const bool bf = a.s.exact_dtype == ODMKV_BF16;
     const float esc = a.scaling * LOG2E;
+    const uint4 qslice = load_query_slice<NP>(a, a.qs + (size_t)bq0 * 32, tid);
     const int count = a.s.seg_count[4][bh];          // exact segments grow between work-list rebuilds
-    stage_queries<NP>(load_query_slice<NP>(a, a.qs + (size_t)bq0 * 32, tid), qsh, tid);
-    __syncthreads();
-    h4 qr[NP * 32], ql[NP * 32];
-    fetch_queries<NP>(qsh, lane, qr, ql);
-    for (int tt = wave; tt < ntiles; tt += NWAVES) {
-        const int tile = tile0 + tt;
-        const int nvalid = min(count - (tile - seg_first) * TILE, TILE);
-        if (nvalid <= 0) break;
-        const uint16_t* ksrc = a.s.kexact + (size_t)tile * TILE * HD;
-        const uint16_t* vsrc = a.s.vexact + (size_t)tile * TILE * HD;
-        f4 dk[NP][4];
+    ExactTile cur;
+    int tt = wave;
+    int nvalid = tt < ntiles ? min(count - (tile0 + tt - seg_first) * TILE, TILE) : 0;
+    if (nvalid > 0) load_exact_tile(cur, a, tile0 + tt, lane);
+    stage_queries<NP>(qslice, qsh, tid);
+    lds_barrier();
+    h4 qr[NP * 32];
 #pragma unroll
-        for (int p = 0; p < NP; ++p)
+    for (int p = 0; p < NP; ++p)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) dk[p][c] = (f4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int c = 0; c < 16; ++c) {
-            uint4 v = *reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 8);
-            if (bf) { v.x = bf16x2_to_f16x2(v.x); v.y = bf16x2_to_f16x2(v.y); v.z = bf16x2_to_f16x2(v.z); v.w = bf16x2_to_f16x2(v.w); }
-            const h4 k0 = as_h4(v.x, v.y), k1 = as_h4(v.z, v.w);
-#pragma unroll
-            for (int p = 0; p < NP; ++p) {
-                dk[p][(2 * c) & 3] = MFMA(k0, qr[p * 32 + 2 * c], dk[p][(2 * c) & 3]);
-                dk[p][(2 * c + 1) & 3] = MFMA(k1, qr[p * 32 + 2 * c + 1], dk[p][(2 * c + 1) & 3]);
-            }
+        for (int s = 0; s < 32; ++s) {
+            const uint2 v = *reinterpret_cast<const uint2*>(&qsh[(4 * p + (lane & 3)) * 32 + s]);
+            qr[p * 32 + s] = as_h4(v.x, v.y);
         }
-        const int tok0 = lane & ~3;
-        h4 pa[NP];
-#pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            const f4 d = (dk[p][0] + dk[p][1]) + (dk[p][2] + dk[p][3]);
-            f4 logit, vn;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                logit[i] = tok0 + i < nvalid ? d[i] * esc : -INFINITY;
-                vn[i] = tok0 + i < nvalid ? 1.0f : 0.0f;
-            }
-            pa[p] = softmax_step<NP>(st, p, logit, vn);
-        }
-        PV_EXACT_STEP(0) PV_EXACT_STEP(1) PV_EXACT_STEP(2) PV_EXACT_STEP(3)
-        PV_EXACT_STEP(4) PV_EXACT_STEP(5) PV_EXACT_STEP(6) PV_EXACT_STEP(7)
-        PV_EXACT_STEP(8) PV_EXACT_STEP(9) PV_EXACT_STEP(10) PV_EXACT_STEP(11)
-        PV_EXACT_STEP(12) PV_EXACT_STEP(13) PV_EXACT_STEP(14) PV_EXACT_STEP(15)
+    while (nvalid > 0) {
+        compute_exact_tile<NP>(cur, bf, nvalid, lane, esc, qr, st);
+        tt += NWAVES;
+        nvalid = tt < ntiles ? min(count - (tile0 + tt - seg_first) * TILE, TILE) : 0;
+        if (nvalid > 0) load_exact_tile(cur, a, tile0 + tt, lane);
     }
 }
 
