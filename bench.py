@@ -145,6 +145,8 @@ def main() -> int:
     ap.add_argument("--target", type=float, default=2.0)
     ap.add_argument("--cpu-sample-ctx", type=int, default=8192)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--read-ceiling", action="store_true",
+                    help="time a plain streaming read kernel at the decode kernel's launch sizes (cold buffers) and exit")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for counter runs under rocprofv3 --pmc: a few eager decode steps and one plain 256 MiB "
                          "device copy (the calibration kernel), nothing else timed")
@@ -165,6 +167,31 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     n_kv, n_q, T, NL = 8, 32, args.ctx, args.layers
+
+    if args.read_ceiling:
+        # what can ONE launch of a given size reach?  buffers rotate through 2 GiB so every launch reads HBM
+        pool = torch.ones(2 << 30, dtype=torch.uint8, device=dev)
+        sink = torch.zeros(64, dtype=torch.int32, device=dev)
+        st_ptr = _lib.stream_ptr(dev)
+        rows = []
+        for nbytes in (19336677, 80740000, 536870912):
+            stride = (nbytes + (2 << 20)) & ~((2 << 20) - 1)
+            nbuf = min((2 << 30) // stride, 64)
+            for grid in (1024, 2048, 4096):
+                ms = []
+                for it in range(3 * nbuf):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    _lib.check(_lib.lib.odmkv_probe_read(pool.data_ptr() + (it % nbuf) * stride, nbytes, grid, sink.data_ptr(), st_ptr))
+                    e1.record()
+                    e1.synchronize()
+                    if it >= nbuf:
+                        ms.append(e0.elapsed_time(e1))
+                med = statistics.median(ms)
+                rows.append({"bytes": nbytes, "grid": grid, "median_us": round(med * 1e3, 2),
+                             "GBps": round(nbytes / (med * 1e-3) / 1e9), "pct_of_8TBps": round(100 * nbytes / (med * 1e-3) / 8e12, 1)})
+        print(json.dumps({"read_ceiling": rows}))
+        return 0
 
     eps, gate_err = parity_gate(dev)
 

@@ -211,6 +211,12 @@ int odmkv_profile_enable(int max_records);
 int odmkv_profile_collect(float* ms, int capacity, int* n_out);
 int odmkv_profile_disable(void);
 
+/* Yardstick for the roofline (no counterpart in the reference): a plain streaming read of `bytes`
+ * bytes at `buf` (device, 16-byte aligned) by `grid` workgroups of 256 threads; `sink` is a device
+ * word that is practically never written.  Timing it over buffers that rotate through more than
+ * the last-level cache shows what one launch of that size can reach on the machine. */
+int odmkv_probe_read(const void* buf, size_t bytes, int grid, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -704,6 +704,25 @@ extern "C" int odmkv_profile_collect(float* ms, int capacity, int* n_out) {
     return 0;
 }
 
+// plain streaming read of a buffer (grid-stride 16-byte loads folded into one word per thread):
+// the yardstick for what a single launch of a given size can reach on the machine
+__global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ p, size_t n16, unsigned int* sink) {
+    unsigned int acc = 0u;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) {
+        const uint4 v = p[i];
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9e3779b9u) sink[0] = acc;       // practically never taken: keeps the loads alive
+}
+
+extern "C" int odmkv_probe_read(const void* buf, size_t bytes, int grid, void* sink, void* stream) {
+    ODMKV_CHECK_ARG(buf && sink && grid > 0 && ((uintptr_t)buf & 15) == 0, "probe_read: bad arguments");
+    hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<const uint4*>(buf), bytes / 16, reinterpret_cast<unsigned int*>(sink));
+    ODMKV_CHECK_LAUNCH("probe_read_kernel");
+    return 0;
+}
+
 static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
 
 extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
