@@ -70,24 +70,40 @@ struct DecodeArgs {
 // ------------------------------------------------------------------------------------------------
 __device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
 
-__global__ __launch_bounds__(128) void decode_prep_kernel(DecodeArgs a) {
+#define PREP_SLICES 4
+__global__ __launch_bounds__(128 * PREP_SLICES) void decode_prep_kernel(DecodeArgs a) {
     __shared__ float qsh[HD];
-    const int bq = blockIdx.x, i = threadIdx.x;
-    // the query is consumed at fp16 precision, like the attention it replaces (model dtype)
-    const __half q16 = __float2half_rn(a.q[(size_t)bq * HD + i]);
-    qsh[i] = __half2float(q16);
-    uint16_t* qs16 = reinterpret_cast<uint16_t*>(a.qs + (size_t)bq * 32);
-    uint16_t* qr16 = reinterpret_cast<uint16_t*>(a.qrot + (size_t)bq * 32);
-    qs16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(q16);
-    qs16[(i >> 2) * 8 + 4 + (i & 3)] = 0;
+    __shared__ float part[PREP_SLICES][HD];
+    const int bq = blockIdx.x, i = threadIdx.x & (HD - 1), slice = threadIdx.x >> 7;
+    // this thread's 32 elements of column i of Pi_k (rows of the transposed matrix): all requested at once
+    constexpr int JN = HD / PREP_SLICES;
+    float pk[JN];
+#pragma unroll
+    for (int jj = 0; jj < JN; ++jj) pk[jj] = a.pi_k_t[(size_t)(slice * JN + jj) * HD + i];
+    if (slice == 0) {
+        // the query is consumed at fp16 precision, like the attention it replaces (model dtype)
+        const __half q16 = __float2half_rn(a.q[(size_t)bq * HD + i]);
+        qsh[i] = __half2float(q16);
+        uint16_t* qs16 = reinterpret_cast<uint16_t*>(a.qs + (size_t)bq * 32);
+        qs16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(q16);
+        qs16[(i >> 2) * 8 + 4 + (i & 3)] = 0;
+    }
     __syncthreads();
-    // q'_i = sum_j Pi_k[i][j] q_j, read from the transposed matrix so that threads read side by side
+    // q'_i = sum_j Pi_k[i][j] q_j: every slice sums its quarter of j in order, the quarters are added in order
     float acc = 0.0f;
-#pragma unroll 16
-    for (int j = 0; j < HD; ++j) acc = __fmaf_rn(a.pi_k_t[(size_t)j * HD + i], qsh[j], acc);
-    const __half hi = __float2half_rn(acc);
-    qr16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(hi);
-    qr16[(i >> 2) * 8 + 4 + (i & 3)] = (uint16_t)half_bits(acc - __half2float(hi));
+#pragma unroll
+    for (int jj = 0; jj < JN; ++jj) acc = __fmaf_rn(pk[jj], qsh[slice * JN + jj], acc);
+    part[slice][i] = acc;
+    __syncthreads();
+    if (slice == 0) {
+        float tot = part[0][i];
+#pragma unroll
+        for (int sl = 1; sl < PREP_SLICES; ++sl) tot += part[sl][i];
+        uint16_t* qr16 = reinterpret_cast<uint16_t*>(a.qrot + (size_t)bq * 32);
+        const __half hi = __float2half_rn(tot);
+        qr16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(hi);
+        qr16[(i >> 2) * 8 + 4 + (i & 3)] = (uint16_t)half_bits(tot - __half2float(hi));
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -606,9 +622,29 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
     const int b = bq / a.Hq, hq = bq % a.Hq;
     const int bh = b * a.s.Hkv + hq / a.G, g = hq % a.G;
     const int i0 = a.item_range[bh], n = min(a.item_range[bh + 1] - i0, MERGE_MAX_ITEMS);
+    // Everything that does not depend on the weights is requested now, in one round trip: this thread's
+    // share of the value rotation, the first MERGE_PRE accumulator values of its slice, its item's (m, l, level)
+    constexpr int IN = HD / MERGE_SLICES;
+    float pv[IN];
+#pragma unroll
+    for (int ii = 0; ii < IN; ++ii) pv[ii] = a.pi_v[(size_t)(slice * IN + ii) * HD + j];
+    constexpr int MERGE_PRE = 16;
+    float pre[MERGE_PRE];
+#pragma unroll
+    for (int k = 0; k < MERGE_PRE; ++k) {
+        const int it = slice + k * MERGE_SLICES;
+        pre[k] = it < n ? a.partial[((size_t)(i0 + it) * GP + g) * PSTRIDE + j] : 0.0f;
+    }
+    float my_m = -INFINITY, my_l = 0.0f;
+    int my_level = 0;
+    if (tid < n) {
+        const float* p = a.partial + ((size_t)(i0 + tid) * GP + g) * PSTRIDE;
+        my_m = p[HD]; my_l = p[HD + 1];
+        my_level = a.items[8 * (i0 + tid) + 1];
+    }
     // maximum over the items
-    float mx = -INFINITY;
-    for (int it = tid; it < n; it += MERGE_THREADS)
+    float mx = my_m;
+    for (int it = tid + MERGE_THREADS; it < n; it += MERGE_THREADS)
         mx = fmaxf(mx, a.partial[((size_t)(i0 + it) * GP + g) * PSTRIDE + HD]);
     mx = wave_max(mx);
     if ((tid & 63) == 0) red[tid >> 6] = mx;
@@ -619,7 +655,12 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
     __syncthreads();
     // weights and the normaliser
     float lpart = 0.0f;
-    for (int it = tid; it < n; it += MERGE_THREADS) {
+    if (tid < n) {
+        const float f = M > -INFINITY ? __builtin_amdgcn_exp2f(my_m - M) : 0.0f;
+        lpart = my_l * f;
+        wts[tid] = my_level == 4 ? -f : f;
+    }
+    for (int it = tid + MERGE_THREADS; it < n; it += MERGE_THREADS) {
         const float* p = a.partial + ((size_t)(i0 + it) * GP + g) * PSTRIDE;
         const float f = M > -INFINITY ? __builtin_amdgcn_exp2f(p[HD] - M) : 0.0f;
         lpart = __fmaf_rn(p[HD + 1], f, lpart);
@@ -634,8 +675,18 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
         Lsh = L;
     }
     float arot = 0.0f, aex = 0.0f;
+    __syncthreads();                                   // weights written
+#pragma unroll
+    for (int k = 0; k < MERGE_PRE; ++k) {
+        const int it = slice + k * MERGE_SLICES;
+        if (it < n) {
+            const float w = wts[it];
+            if (__float_as_uint(w) >> 31) aex = __fmaf_rn(pre[k], -w, aex);
+            else arot = __fmaf_rn(pre[k], w, arot);
+        }
+    }
 #pragma unroll 4
-    for (int it = slice; it < n; it += MERGE_SLICES) {
+    for (int it = slice + MERGE_PRE * MERGE_SLICES; it < n; it += MERGE_SLICES) {
         const float w = wts[it];
         const float v = a.partial[((size_t)(i0 + it) * GP + g) * PSTRIDE + j];
         if (__float_as_uint(w) >> 31) aex = __fmaf_rn(v, -w, aex);
@@ -653,8 +704,8 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
     __syncthreads();
     // rotate the quantised part back: out_j = sum_i rot_i Pi_v[i][j]; the slices split the i range
     float o = 0.0f;
-    for (int i = slice * (HD / MERGE_SLICES); i < (slice + 1) * (HD / MERGE_SLICES); ++i)
-        o = __fmaf_rn(rot[i], a.pi_v[(size_t)i * HD + j], o);
+#pragma unroll
+    for (int ii = 0; ii < IN; ++ii) o = __fmaf_rn(rot[slice * IN + ii], pv[ii], o);
     __syncthreads();
     part[0][slice][j] = o;
     __syncthreads();
@@ -759,7 +810,7 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     a.qs = (uint4*)((char*)workspace + qbytes);
     a.partial = (float*)((char*)workspace + 2 * qbytes);
     a.out = out; a.lse = lse;
-    hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(128), 0, st, a);
+    hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(128 * PREP_SLICES), 0, st, a);
     ODMKV_CHECK_LAUNCH("decode_prep_kernel");
     const int GP = group_pad(G);
     if (n_items > 0) {
