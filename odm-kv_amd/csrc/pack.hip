@@ -382,7 +382,13 @@ template <int DT> struct RowRegs {
     }
     __device__ inline float get(int j) const {
         if constexpr (DT == ODMKV_F32) return __uint_as_float(w[j]);
-        else return Elem<DT>::to_f32((uint16_t)((j & 1) ? (w[j >> 1] >> 16) : (w[j >> 1] & 0xffffu)));
+        else {
+            // the conversion is one instruction; converting all 128 elements ahead of time and keeping
+            // them (what the optimiser would do) costs 64 more registers than the packed words
+            uint32_t word = w[j >> 1];
+            asm volatile("" : "+v"(word));
+            return Elem<DT>::to_f32((uint16_t)((j & 1) ? (word >> 16) : (word & 0xffffu)));
+        }
     }
 };
 
