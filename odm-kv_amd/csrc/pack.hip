@@ -245,6 +245,7 @@ __device__ static inline float decision_threshold(float c_lo, float c_hi) {
 // thresholds of width index li start at thr_offset(li): 3 + 7 + 15 + 255 floats
 __device__ static inline int thr_offset(int li) { return li == 0 ? 0 : li == 1 ? 3 : li == 2 ? 10 : 25; }
 #define QP_THR_FLOATS 280
+#define QP_GROUP 2           // rotation steps whose matrix instructions are issued back to back
 
 template <int W> struct Coder {
     static constexpr int K = 1 << W;
@@ -256,20 +257,31 @@ template <int W> struct Coder {
             for (int k = 0; k < K - 1; ++k) t[k] = thr_li[k];
         }
     }
-    __device__ inline uint32_t operator()(float y) const {
-        if constexpr (W <= 3) {
-            uint32_t c = 0;
-#pragma unroll
-            for (int k = 0; k < K - 1; ++k) c += (y >= t[k]) ? 1u : 0u;
-            return c;
+    // r * 2^W + code(y): the code's bits are decided top down (each comparison picks the threshold of
+    // the next one) and shifted into r one at a time, which the hardware does as r + r + carry
+    __device__ __forceinline__ uint32_t push(uint32_t r, float y) const {
+        if constexpr (W == 2) {
+            const bool b1 = y >= t[1];
+            r = r + r + (b1 ? 1u : 0u);
+            const bool b0 = y >= (b1 ? t[2] : t[0]);
+            return r + r + (b0 ? 1u : 0u);
+        } else if constexpr (W == 3) {
+            const bool b2 = y >= t[3];
+            r = r + r + (b2 ? 1u : 0u);
+            const bool b1 = y >= (b2 ? t[5] : t[1]);
+            r = r + r + (b1 ? 1u : 0u);
+            const float lo_pair = b1 ? t[2] : t[0], hi_pair = b1 ? t[6] : t[4];
+            const bool b0 = y >= (b2 ? hi_pair : lo_pair);
+            return r + r + (b0 ? 1u : 0u);
         } else {
             int pos = 0;                                     // #thresholds <= y, by binary search
 #pragma unroll
             for (int s = K / 2; s >= 1; s >>= 1)
                 if (y >= thr[pos + s - 1]) pos += s;
-            return (uint32_t)pos;
+            return (r << W) | (uint32_t)pos;
         }
     }
+    __device__ __forceinline__ uint32_t operator()(float y) const { return push(0u, y); }
 };
 
 template <int W>
@@ -293,6 +305,70 @@ __device__ static __forceinline__ void stage_codes_v(const f32x32& acc, int g, c
         const uint32_t w = code(acc[4 * q]) | (code(acc[4 * q + 1]) << 8) | (code(acc[4 * q + 2]) << 16) |
                            (code(acc[4 * q + 3]) << 24);
         *reinterpret_cast<uint32_t*>(stage + (g * 32 + c) * CODE_ROW_T + mfma_token(4 * q, lane)) = w;
+    }
+}
+
+// ---- direct packing (widths 2, 4, 8; tiles that start empty) -----------------------------------------
+// The four outputs a lane holds for a token are neighbours in the token's code stream, and the four
+// tokens it holds for a value dim are neighbours in the dim's stream: 4*W bits that go to the staging
+// area already in their final bit order.  The second pass then only moves 16-byte pieces.
+template <int W> struct Direct {
+    static constexpr int GROUP_BYTES = W / 2;            // 4 codes
+    static constexpr int ROW_K = 16 * W + 16;            // staging bytes per token (multiple of 16)
+    static constexpr int ROW_V = 8 * W + 8;              // staging bytes per dim (multiple of 8)
+};
+
+template <int W>
+__device__ static __forceinline__ void put_group(uint8_t* p, uint32_t bits) {
+    if constexpr (W == 2) *p = (uint8_t)bits;
+    else if constexpr (W == 4) *reinterpret_cast<uint16_t*>(p) = (uint16_t)bits;
+    else *reinterpret_cast<uint32_t*>(p) = bits;
+}
+
+template <int W>
+__device__ static __forceinline__ void stage_direct_k(const f32x32& a0, const f32x32& a1, const f32x32& a2, const f32x32& a3,
+                                                      const float* thr, uint8_t* stage, int lane) {
+    const Coder<W> code(thr);
+    const int c = lane & 31;
+#pragma unroll
+    for (int vv = 0; vv < 32; ++vv) {
+        const uint32_t bits = code.push(code.push(code.push(code.push(0u, a3[vv]), a2[vv]), a1[vv]), a0[vv]);
+        put_group<W>(stage + mfma_token(vv, lane) * Direct<W>::ROW_K + c * Direct<W>::GROUP_BYTES, bits);
+    }
+}
+
+template <int W>
+__device__ static __forceinline__ void store_direct_k(const uint8_t* stage, uint8_t* kcodes, int tile, int lane) {
+    uint8_t* dst = kcodes + (size_t)tile * (TILE * 16 * W);
+#pragma unroll
+    for (int ch = 0; ch < W; ++ch)
+        *reinterpret_cast<uint4*>(dst + ((size_t)ch * TILE + lane) * 16) =
+            *reinterpret_cast<const uint4*>(stage + lane * Direct<W>::ROW_K + 16 * ch);
+}
+
+template <int W>
+__device__ static __forceinline__ void stage_direct_v(const f32x32& acc, int g, const float* thr, uint8_t* stage, int lane) {
+    const Coder<W> code(thr);
+    const int c = lane & 31;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+        const uint32_t bits = code.push(code.push(code.push(code.push(0u, acc[4 * q + 3]), acc[4 * q + 2]), acc[4 * q + 1]), acc[4 * q]);
+        put_group<W>(stage + (g * 32 + c) * Direct<W>::ROW_V + (mfma_token(4 * q, lane) >> 2) * Direct<W>::GROUP_BYTES, bits);
+    }
+}
+
+template <int W>
+__device__ static __forceinline__ void store_direct_v(const uint8_t* stage, uint8_t* vcodes, int tile, int lane) {
+    uint8_t* dst = vcodes + (size_t)tile * (HD * 8 * W);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int j = lane + 64 * half;
+#pragma unroll
+        for (int u = 0; u < W / 2; ++u) {                                  // 16-byte units of the dim's stream
+            const uint2 x = *reinterpret_cast<const uint2*>(stage + j * Direct<W>::ROW_V + 16 * u);
+            const uint2 y = *reinterpret_cast<const uint2*>(stage + j * Direct<W>::ROW_V + 16 * u + 8);
+            *reinterpret_cast<uint4*>(dst + ((size_t)u * HD + j) * 16) = make_uint4(x.x, x.y, y.x, y.y);
+        }
     }
 }
 
@@ -449,8 +525,10 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
         for (int j = 0; j < HD; ++j) {
             const float xj = x.get(j);
             ss = __fmaf_rn(xj, xj, ss);
-            const float ax = fabsf(xj);
-            amin = fminf(amin, ax == 0.0f ? INFINITY : ax);
+            if constexpr (DT != ODMKV_F16) {                   // fp16 inputs cannot get that small against their norm
+                const float ax = fabsf(xj);
+                amin = fminf(amin, ax == 0.0f ? INFINITY : ax);
+            }
         }
         const float norm = sqrtf(ss);
         const float den = norm + 1e-10f;
@@ -470,39 +548,36 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
             const float r0 = __builtin_amdgcn_rcpf(den);
             const float rr = __fmaf_rn(__fmaf_rn(-den, r0, 1.0f), r0, r0);
             const float nden = -den;
-            // Issue order is pinned: every matrix instruction is followed by a slice of the next
-            // step's operand preparation (LDS read, conversion, division), so the matrix pipe is
-            // handed its next instruction the moment it frees up.
-            float4 b = brow[0];
-            float u;
-            {
-                const float n0 = x.get(0);
-                const float q0 = __fmul_rn(n0, rr);
-                const float q1 = __fmaf_rn(__fmaf_rn(nden, q0, n0), rr, q0);
-                u = __fmaf_rn(__fmaf_rn(nden, q1, n0), rr, q1);
-            }
+            // Issue order is pinned.  A vector instruction between two matrix instructions of one
+            // wave costs the matrix pipe about 13 idle clocks (a later one 4 more each), and never
+            // runs in its shadow; so the matrix instructions of QP_GROUP steps go back to back and the
+            // operand preparation of the next group (LDS reads, conversions, divisions) follows in
+            // one block.
+            const auto quotient = [&](int j) {
+                const float n = x.get(j);
+                const float q0 = __fmul_rn(n, rr);
+                const float q1 = __fmaf_rn(__fmaf_rn(nden, q0, n), rr, q0);
+                return __fmaf_rn(__fmaf_rn(nden, q1, n), rr, q1);
+            };
+            float4 b[QP_GROUP];
+            float u[QP_GROUP];
 #pragma unroll
-            for (int j = 0; j < HD; ++j) {
-                float4 bn = b;
-                float un = u;
-                const int jn = j + 1 < HD ? j + 1 : j;
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.x, acc0, 0, 0, 0);
-                bn = brow[jn * (HD / 4)];
-                const float nn = x.get(jn);
-                const float q0 = __fmul_rn(nn, rr);
+            for (int g = 0; g < QP_GROUP; ++g) { b[g] = brow[g * (HD / 4)]; u[g] = quotient(g); }
+#pragma unroll
+            for (int j = 0; j < HD; j += QP_GROUP) {
+#pragma unroll
+                for (int g = 0; g < QP_GROUP; ++g) {
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b[g].x, acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b[g].y, acc1, 0, 0, 0);
+                    acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b[g].z, acc2, 0, 0, 0);
+                    acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b[g].w, acc3, 0, 0, 0);
+                }
                 __builtin_amdgcn_sched_barrier(0);
-                acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.y, acc1, 0, 0, 0);
-                const float e2 = __fmaf_rn(nden, q0, nn);
-                const float q1 = __fmaf_rn(e2, rr, q0);
+                if (j + QP_GROUP < HD) {
+#pragma unroll
+                    for (int g = 0; g < QP_GROUP; ++g) { b[g] = brow[(j + QP_GROUP + g) * (HD / 4)]; u[g] = quotient(j + QP_GROUP + g); }
+                }
                 __builtin_amdgcn_sched_barrier(0);
-                acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.z, acc2, 0, 0, 0);
-                const float e3 = __fmaf_rn(nden, q1, nn);
-                un = __fmaf_rn(e3, rr, q1);
-                __builtin_amdgcn_sched_barrier(0);
-                acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(u, b.w, acc3, 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                b = bn;
-                u = un;
             }
         } else {
 #pragma unroll
@@ -517,40 +592,75 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
         }
 
         const float* cb = thrs + thr_offset(li);
+        // widths 2, 4, 8; keys into a tile that starts empty, values into a tile this call fills whole
+        const bool direct = li != 1 && lo == 0 && (!is_v || hi == TILE);
         if (!is_v) {
-            switch (li) {
-                case 0: stage_codes_k<2>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
-                case 1: stage_codes_k<3>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
-                case 2: stage_codes_k<4>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
-                default: stage_codes_k<8>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+            if (direct) {
+                switch (li) {
+                    case 0: stage_direct_k<2>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                    case 2: stage_direct_k<4>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                    default: stage_direct_k<8>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                }
+            } else {
+                switch (li) {
+                    case 0: stage_codes_k<2>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                    case 1: stage_codes_k<3>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                    case 2: stage_codes_k<4>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                    default: stage_codes_k<8>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                }
             }
             wave_lds_fence();
             if (valid) {
-                switch (li) {
-                    case 0: pack_store_k<2>(stage, a.s.kcodes[0], tile, lane); break;
-                    case 1: pack_store_k<3>(stage, a.s.kcodes[1], tile, lane); break;
-                    case 2: pack_store_k<4>(stage, a.s.kcodes[2], tile, lane); break;
-                    default: pack_store_k<8>(stage, a.s.kcodes[3], tile, lane); break;
+                if (direct) {
+                    switch (li) {
+                        case 0: store_direct_k<2>(stage, a.s.kcodes[0], tile, lane); break;
+                        case 2: store_direct_k<4>(stage, a.s.kcodes[2], tile, lane); break;
+                        default: store_direct_k<8>(stage, a.s.kcodes[3], tile, lane); break;
+                    }
+                } else {
+                    switch (li) {
+                        case 0: pack_store_k<2>(stage, a.s.kcodes[0], tile, lane); break;
+                        case 1: pack_store_k<3>(stage, a.s.kcodes[1], tile, lane); break;
+                        case 2: pack_store_k<4>(stage, a.s.kcodes[2], tile, lane); break;
+                        default: pack_store_k<8>(stage, a.s.kcodes[3], tile, lane); break;
+                    }
                 }
                 a.s.knorm[li][slot] = norm;
             }
         } else {
-            switch (li) {
-                case 0: stage_codes_v<2>(acc0, 0, cb, stage, lane); stage_codes_v<2>(acc1, 1, cb, stage, lane);
-                        stage_codes_v<2>(acc2, 2, cb, stage, lane); stage_codes_v<2>(acc3, 3, cb, stage, lane); break;
-                case 1: stage_codes_v<3>(acc0, 0, cb, stage, lane); stage_codes_v<3>(acc1, 1, cb, stage, lane);
-                        stage_codes_v<3>(acc2, 2, cb, stage, lane); stage_codes_v<3>(acc3, 3, cb, stage, lane); break;
-                case 2: stage_codes_v<4>(acc0, 0, cb, stage, lane); stage_codes_v<4>(acc1, 1, cb, stage, lane);
-                        stage_codes_v<4>(acc2, 2, cb, stage, lane); stage_codes_v<4>(acc3, 3, cb, stage, lane); break;
-                default: stage_codes_v<8>(acc0, 0, cb, stage, lane); stage_codes_v<8>(acc1, 1, cb, stage, lane);
-                         stage_codes_v<8>(acc2, 2, cb, stage, lane); stage_codes_v<8>(acc3, 3, cb, stage, lane); break;
-            }
-            wave_lds_fence();
-            switch (li) {
-                case 0: pack_store_v<2>(stage, a.s.vcodes[0], tile, lane, lo, hi); break;
-                case 1: pack_store_v<3>(stage, a.s.vcodes[1], tile, lane, lo, hi); break;
-                case 2: pack_store_v<4>(stage, a.s.vcodes[2], tile, lane, lo, hi); break;
-                default: pack_store_v<8>(stage, a.s.vcodes[3], tile, lane, lo, hi); break;
+            if (direct) {
+                switch (li) {
+                    case 0: stage_direct_v<2>(acc0, 0, cb, stage, lane); stage_direct_v<2>(acc1, 1, cb, stage, lane);
+                            stage_direct_v<2>(acc2, 2, cb, stage, lane); stage_direct_v<2>(acc3, 3, cb, stage, lane); break;
+                    case 2: stage_direct_v<4>(acc0, 0, cb, stage, lane); stage_direct_v<4>(acc1, 1, cb, stage, lane);
+                            stage_direct_v<4>(acc2, 2, cb, stage, lane); stage_direct_v<4>(acc3, 3, cb, stage, lane); break;
+                    default: stage_direct_v<8>(acc0, 0, cb, stage, lane); stage_direct_v<8>(acc1, 1, cb, stage, lane);
+                             stage_direct_v<8>(acc2, 2, cb, stage, lane); stage_direct_v<8>(acc3, 3, cb, stage, lane); break;
+                }
+                wave_lds_fence();
+                switch (li) {
+                    case 0: store_direct_v<2>(stage, a.s.vcodes[0], tile, lane); break;
+                    case 2: store_direct_v<4>(stage, a.s.vcodes[2], tile, lane); break;
+                    default: store_direct_v<8>(stage, a.s.vcodes[3], tile, lane); break;
+                }
+            } else {
+                switch (li) {
+                    case 0: stage_codes_v<2>(acc0, 0, cb, stage, lane); stage_codes_v<2>(acc1, 1, cb, stage, lane);
+                            stage_codes_v<2>(acc2, 2, cb, stage, lane); stage_codes_v<2>(acc3, 3, cb, stage, lane); break;
+                    case 1: stage_codes_v<3>(acc0, 0, cb, stage, lane); stage_codes_v<3>(acc1, 1, cb, stage, lane);
+                            stage_codes_v<3>(acc2, 2, cb, stage, lane); stage_codes_v<3>(acc3, 3, cb, stage, lane); break;
+                    case 2: stage_codes_v<4>(acc0, 0, cb, stage, lane); stage_codes_v<4>(acc1, 1, cb, stage, lane);
+                            stage_codes_v<4>(acc2, 2, cb, stage, lane); stage_codes_v<4>(acc3, 3, cb, stage, lane); break;
+                    default: stage_codes_v<8>(acc0, 0, cb, stage, lane); stage_codes_v<8>(acc1, 1, cb, stage, lane);
+                             stage_codes_v<8>(acc2, 2, cb, stage, lane); stage_codes_v<8>(acc3, 3, cb, stage, lane); break;
+                }
+                wave_lds_fence();
+                switch (li) {
+                    case 0: pack_store_v<2>(stage, a.s.vcodes[0], tile, lane, lo, hi); break;
+                    case 1: pack_store_v<3>(stage, a.s.vcodes[1], tile, lane, lo, hi); break;
+                    case 2: pack_store_v<4>(stage, a.s.vcodes[2], tile, lane, lo, hi); break;
+                    default: pack_store_v<8>(stage, a.s.vcodes[3], tile, lane, lo, hi); break;
+                }
             }
             if (valid) a.s.vnorm[li][slot] = norm;
         }
