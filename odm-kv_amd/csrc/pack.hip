@@ -245,7 +245,7 @@ __device__ static inline float decision_threshold(float c_lo, float c_hi) {
 // thresholds of width index li start at thr_offset(li): 3 + 7 + 15 + 255 floats
 __device__ static inline int thr_offset(int li) { return li == 0 ? 0 : li == 1 ? 3 : li == 2 ? 10 : 25; }
 #define QP_THR_FLOATS 280
-#define QP_GROUP 2           // rotation steps whose matrix instructions are issued back to back
+#define QP_GROUP 32           // rotation steps whose matrix instructions are issued back to back
 
 template <int W> struct Coder {
     static constexpr int K = 1 << W;
@@ -536,6 +536,7 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
         f32x32 acc0, acc1, acc2, acc3;
 #pragma unroll
         for (int i = 0; i < 32; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; acc2[i] = 0.0f; acc3[i] = 0.0f; }
+        __builtin_amdgcn_s_setprio(0);
         const float4* __restrict__ brow = reinterpret_cast<const float4*>(piT) + (lane & 31);
         // u_j = x_j / den, correctly rounded.  With den in [2^-40, 2^60] and every non-zero |x_j| at
         // least den * 2^-60 the hardware division sequence never rescales its operands, so the part
@@ -549,35 +550,33 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
             const float rr = __fmaf_rn(__fmaf_rn(-den, r0, 1.0f), r0, r0);
             const float nden = -den;
             // Issue order is pinned.  A vector instruction between two matrix instructions of one
-            // wave costs the matrix pipe about 13 idle clocks (a later one 4 more each), and never
-            // runs in its shadow; so the matrix instructions of QP_GROUP steps go back to back and the
-            // operand preparation of the next group (LDS reads, conversions, divisions) follows in
-            // one block.
+            // wave costs the matrix pipe about 13 idle clocks (a later one 4 more each) and never
+            // runs in its shadow, while an LDS read costs about one; so the quotients of QP_GROUP
+            // steps are computed in one block, and the matrix instructions of those steps then go
+            // back to back with only the LDS reads of the rotation between them.
             const auto quotient = [&](int j) {
                 const float n = x.get(j);
                 const float q0 = __fmul_rn(n, rr);
                 const float q1 = __fmaf_rn(__fmaf_rn(nden, q0, n), rr, q0);
                 return __fmaf_rn(__fmaf_rn(nden, q1, n), rr, q1);
             };
-            float4 b[QP_GROUP];
-            float u[QP_GROUP];
+            float4 b = brow[0];
 #pragma unroll
-            for (int g = 0; g < QP_GROUP; ++g) { b[g] = brow[g * (HD / 4)]; u[g] = quotient(g); }
+            for (int j0 = 0; j0 < HD; j0 += QP_GROUP) {
+                float u[QP_GROUP];
 #pragma unroll
-            for (int j = 0; j < HD; j += QP_GROUP) {
+                for (int g = 0; g < QP_GROUP; ++g) u[g] = quotient(j0 + g);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int g = 0; g < QP_GROUP; ++g) {
-                    acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b[g].x, acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b[g].y, acc1, 0, 0, 0);
-                    acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b[g].z, acc2, 0, 0, 0);
-                    acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b[g].w, acc3, 0, 0, 0);
+                    const int jn = j0 + g + 1 < HD ? j0 + g + 1 : j0 + g;
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b.x, acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b.y, acc1, 0, 0, 0);
+                    acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b.z, acc2, 0, 0, 0);
+                    acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(u[g], b.w, acc3, 0, 0, 0);
+                    b = brow[jn * (HD / 4)];
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                __builtin_amdgcn_sched_barrier(0);
-                if (j + QP_GROUP < HD) {
-#pragma unroll
-                    for (int g = 0; g < QP_GROUP; ++g) { b[g] = brow[(j + QP_GROUP + g) * (HD / 4)]; u[g] = quotient(j + QP_GROUP + g); }
-                }
-                __builtin_amdgcn_sched_barrier(0);
             }
         } else {
 #pragma unroll
@@ -592,37 +591,44 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
         }
 
         const float* cb = thrs + thr_offset(li);
+        // the lane index as the coding phase sees it: opaque to the compiler, so that the staging and
+        // store addresses are computed here and not carried (spilled) across the rotation loop
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        // while one wave of a SIMD streams matrix instructions (it needs one issue slot in 64 clocks),
+        // the other's vector and memory instructions are the ones that must not wait
+        __builtin_amdgcn_s_setprio(3);
         // widths 2, 4, 8; keys into a tile that starts empty, values into a tile this call fills whole
         const bool direct = li != 1 && lo == 0 && (!is_v || hi == TILE);
         if (!is_v) {
             if (direct) {
                 switch (li) {
-                    case 0: stage_direct_k<2>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
-                    case 2: stage_direct_k<4>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
-                    default: stage_direct_k<8>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                    case 0: stage_direct_k<2>(acc0, acc1, acc2, acc3, cb, stage, ln); break;
+                    case 2: stage_direct_k<4>(acc0, acc1, acc2, acc3, cb, stage, ln); break;
+                    default: stage_direct_k<8>(acc0, acc1, acc2, acc3, cb, stage, ln); break;
                 }
             } else {
                 switch (li) {
-                    case 0: stage_codes_k<2>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
-                    case 1: stage_codes_k<3>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
-                    case 2: stage_codes_k<4>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
-                    default: stage_codes_k<8>(acc0, acc1, acc2, acc3, cb, stage, lane); break;
+                    case 0: stage_codes_k<2>(acc0, acc1, acc2, acc3, cb, stage, ln); break;
+                    case 1: stage_codes_k<3>(acc0, acc1, acc2, acc3, cb, stage, ln); break;
+                    case 2: stage_codes_k<4>(acc0, acc1, acc2, acc3, cb, stage, ln); break;
+                    default: stage_codes_k<8>(acc0, acc1, acc2, acc3, cb, stage, ln); break;
                 }
             }
             wave_lds_fence();
             if (valid) {
                 if (direct) {
                     switch (li) {
-                        case 0: store_direct_k<2>(stage, a.s.kcodes[0], tile, lane); break;
-                        case 2: store_direct_k<4>(stage, a.s.kcodes[2], tile, lane); break;
-                        default: store_direct_k<8>(stage, a.s.kcodes[3], tile, lane); break;
+                        case 0: store_direct_k<2>(stage, a.s.kcodes[0], tile, ln); break;
+                        case 2: store_direct_k<4>(stage, a.s.kcodes[2], tile, ln); break;
+                        default: store_direct_k<8>(stage, a.s.kcodes[3], tile, ln); break;
                     }
                 } else {
                     switch (li) {
-                        case 0: pack_store_k<2>(stage, a.s.kcodes[0], tile, lane); break;
-                        case 1: pack_store_k<3>(stage, a.s.kcodes[1], tile, lane); break;
-                        case 2: pack_store_k<4>(stage, a.s.kcodes[2], tile, lane); break;
-                        default: pack_store_k<8>(stage, a.s.kcodes[3], tile, lane); break;
+                        case 0: pack_store_k<2>(stage, a.s.kcodes[0], tile, ln); break;
+                        case 1: pack_store_k<3>(stage, a.s.kcodes[1], tile, ln); break;
+                        case 2: pack_store_k<4>(stage, a.s.kcodes[2], tile, ln); break;
+                        default: pack_store_k<8>(stage, a.s.kcodes[3], tile, ln); break;
                     }
                 }
                 a.s.knorm[li][slot] = norm;
@@ -630,36 +636,36 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
         } else {
             if (direct) {
                 switch (li) {
-                    case 0: stage_direct_v<2>(acc0, 0, cb, stage, lane); stage_direct_v<2>(acc1, 1, cb, stage, lane);
-                            stage_direct_v<2>(acc2, 2, cb, stage, lane); stage_direct_v<2>(acc3, 3, cb, stage, lane); break;
-                    case 2: stage_direct_v<4>(acc0, 0, cb, stage, lane); stage_direct_v<4>(acc1, 1, cb, stage, lane);
-                            stage_direct_v<4>(acc2, 2, cb, stage, lane); stage_direct_v<4>(acc3, 3, cb, stage, lane); break;
-                    default: stage_direct_v<8>(acc0, 0, cb, stage, lane); stage_direct_v<8>(acc1, 1, cb, stage, lane);
-                             stage_direct_v<8>(acc2, 2, cb, stage, lane); stage_direct_v<8>(acc3, 3, cb, stage, lane); break;
+                    case 0: stage_direct_v<2>(acc0, 0, cb, stage, ln); stage_direct_v<2>(acc1, 1, cb, stage, ln);
+                            stage_direct_v<2>(acc2, 2, cb, stage, ln); stage_direct_v<2>(acc3, 3, cb, stage, ln); break;
+                    case 2: stage_direct_v<4>(acc0, 0, cb, stage, ln); stage_direct_v<4>(acc1, 1, cb, stage, ln);
+                            stage_direct_v<4>(acc2, 2, cb, stage, ln); stage_direct_v<4>(acc3, 3, cb, stage, ln); break;
+                    default: stage_direct_v<8>(acc0, 0, cb, stage, ln); stage_direct_v<8>(acc1, 1, cb, stage, ln);
+                             stage_direct_v<8>(acc2, 2, cb, stage, ln); stage_direct_v<8>(acc3, 3, cb, stage, ln); break;
                 }
                 wave_lds_fence();
                 switch (li) {
-                    case 0: store_direct_v<2>(stage, a.s.vcodes[0], tile, lane); break;
-                    case 2: store_direct_v<4>(stage, a.s.vcodes[2], tile, lane); break;
-                    default: store_direct_v<8>(stage, a.s.vcodes[3], tile, lane); break;
+                    case 0: store_direct_v<2>(stage, a.s.vcodes[0], tile, ln); break;
+                    case 2: store_direct_v<4>(stage, a.s.vcodes[2], tile, ln); break;
+                    default: store_direct_v<8>(stage, a.s.vcodes[3], tile, ln); break;
                 }
             } else {
                 switch (li) {
-                    case 0: stage_codes_v<2>(acc0, 0, cb, stage, lane); stage_codes_v<2>(acc1, 1, cb, stage, lane);
-                            stage_codes_v<2>(acc2, 2, cb, stage, lane); stage_codes_v<2>(acc3, 3, cb, stage, lane); break;
-                    case 1: stage_codes_v<3>(acc0, 0, cb, stage, lane); stage_codes_v<3>(acc1, 1, cb, stage, lane);
-                            stage_codes_v<3>(acc2, 2, cb, stage, lane); stage_codes_v<3>(acc3, 3, cb, stage, lane); break;
-                    case 2: stage_codes_v<4>(acc0, 0, cb, stage, lane); stage_codes_v<4>(acc1, 1, cb, stage, lane);
-                            stage_codes_v<4>(acc2, 2, cb, stage, lane); stage_codes_v<4>(acc3, 3, cb, stage, lane); break;
-                    default: stage_codes_v<8>(acc0, 0, cb, stage, lane); stage_codes_v<8>(acc1, 1, cb, stage, lane);
-                             stage_codes_v<8>(acc2, 2, cb, stage, lane); stage_codes_v<8>(acc3, 3, cb, stage, lane); break;
+                    case 0: stage_codes_v<2>(acc0, 0, cb, stage, ln); stage_codes_v<2>(acc1, 1, cb, stage, ln);
+                            stage_codes_v<2>(acc2, 2, cb, stage, ln); stage_codes_v<2>(acc3, 3, cb, stage, ln); break;
+                    case 1: stage_codes_v<3>(acc0, 0, cb, stage, ln); stage_codes_v<3>(acc1, 1, cb, stage, ln);
+                            stage_codes_v<3>(acc2, 2, cb, stage, ln); stage_codes_v<3>(acc3, 3, cb, stage, ln); break;
+                    case 2: stage_codes_v<4>(acc0, 0, cb, stage, ln); stage_codes_v<4>(acc1, 1, cb, stage, ln);
+                            stage_codes_v<4>(acc2, 2, cb, stage, ln); stage_codes_v<4>(acc3, 3, cb, stage, ln); break;
+                    default: stage_codes_v<8>(acc0, 0, cb, stage, ln); stage_codes_v<8>(acc1, 1, cb, stage, ln);
+                             stage_codes_v<8>(acc2, 2, cb, stage, ln); stage_codes_v<8>(acc3, 3, cb, stage, ln); break;
                 }
                 wave_lds_fence();
                 switch (li) {
-                    case 0: pack_store_v<2>(stage, a.s.vcodes[0], tile, lane, lo, hi); break;
-                    case 1: pack_store_v<3>(stage, a.s.vcodes[1], tile, lane, lo, hi); break;
-                    case 2: pack_store_v<4>(stage, a.s.vcodes[2], tile, lane, lo, hi); break;
-                    default: pack_store_v<8>(stage, a.s.vcodes[3], tile, lane, lo, hi); break;
+                    case 0: pack_store_v<2>(stage, a.s.vcodes[0], tile, ln, lo, hi); break;
+                    case 1: pack_store_v<3>(stage, a.s.vcodes[1], tile, ln, lo, hi); break;
+                    case 2: pack_store_v<4>(stage, a.s.vcodes[2], tile, ln, lo, hi); break;
+                    default: pack_store_v<8>(stage, a.s.vcodes[3], tile, ln, lo, hi); break;
                 }
             }
             if (valid) a.s.vnorm[li][slot] = norm;
