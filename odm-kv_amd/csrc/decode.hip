@@ -178,15 +178,18 @@ template <int W>
 __device__ static inline void build_lut(uint8_t* lut, const DecodeArgs& a, int tid) {
     const int lane = tid & 63, wave = tid >> 6;
     if constexpr (W == 2) {
+        // row = code byte = wave * 64 + i * 4 + (lane >> 4): its codes are lane >> 4, i & 3, i >> 2 and
+        // wave, so the row's eight bytes are put together from the four centroids without any
+        // cross-lane traffic; the lanes of one store cover consecutive 16-byte pieces of four rows
         uint32_t h[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) h[k] = half_bits(pick<4>(a.cbs, (tid >> (2 * k)) & 3));
-        const uint32_t lo = h[0] | (h[1] << 16), hi = h[2] | (h[3] << 16);
+        for (int k = 0; k < 4; ++k) h[k] = half_bits(a.cbs[k]);
+        const auto sel = [&](int k) { return k == 0 ? h[0] : k == 1 ? h[1] : k == 2 ? h[2] : h[3]; };
+        const uint32_t own = sel(lane >> 4), top = sel(wave) << 16;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const int src = i * 4 + (lane >> 4);
-            const uint32_t x = __shfl(lo, src, WAVE), y = __shfl(hi, src, WAVE);
-            *reinterpret_cast<uint4*>(lut + (wave * 64 + src) * 256 + (lane & 15) * 16) = make_uint4(x, y, x, y);
+            const uint32_t x = own | (h[i & 3] << 16), y = h[i >> 2] | top;
+            *reinterpret_cast<uint4*>(lut + (wave * 64 + i * 4 + (lane >> 4)) * 256 + (lane & 15) * 16) = make_uint4(x, y, x, y);
         }
     } else {
         uint32_t v;
@@ -377,34 +380,34 @@ __device__ static inline void fetch_queries(const uint4* qsh, int lane, h4* qr, 
         }
 }
 
-// One work item of a quantised level.  The first tile's loads are issued before the table is built
-// and the queries are staged, so that HBM latency overlaps the set-up.
+// One work item of a quantised level.
 template <int W, int NP>
 __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq0, int tile0, int ntiles, int ntok,
                                               int tid, uint8_t* lut, uint4* qsh, WaveState<NP>& st) {
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
     const float vsc = a.inv_s[li], ksc = a.inv_s[li] * a.scaling * LOG2E;
-    // loads return in issue order: the (small) query slice goes first so that staging it does not
-    // have to wait for the tiles
+    // The table needs nothing from memory and is built first: behind a wavefront's tile requests its
+    // LDS traffic would wait for the memory pipeline to accept them (every wavefront of the chip asks
+    // for its tiles at the same moment).  Loads return in issue order: the (small) query slice goes
+    // first so that staging it does not have to wait for the tile.
+    build_lut<W>(lut, a, tid);
     const uint4 qslice = load_query_slice<NP>(a, a.qrot + (size_t)bq0 * 32, tid);
     TileData<W> cur;
     int tt = wave;
     int nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
     if (nvalid > 0) load_tile<W>(cur, a, li, tile0 + tt, lane);
-    // second buffer (not for the widest rows: the registers go to the query there).  Both tiles are
-    // requested before the set-up waits on anything: a wavefront rarely owns more than a few tiles,
-    // so the second tile's HBM latency must not start after the first tile is done.
+    stage_queries<NP>(qslice, qsh, tid);
+    lds_barrier();
+    TRACE(1)
+    // second buffer (not for the widest rows: the registers go to the query there), requested before
+    // the queries are fetched into registers
     TileData<W> nxt;
     int nv1 = 0;
     if constexpr (W != 8) {
         nv1 = tt + NWAVES < ntiles ? min(ntok - (tt + NWAVES) * TILE, TILE) : 0;
         if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + NWAVES, lane);
     }
-    build_lut<W>(lut, a, tid);                 // needs nothing from memory: runs while the query slice is on its way
-    stage_queries<NP>(qslice, qsh, tid);
-    lds_barrier();
-    TRACE(1)
     h4 qr[NP * 32], ql[NP * 32];
     fetch_queries<NP>(qsh, lane, qr, ql);
     if (nvalid <= 0) return;
