@@ -30,7 +30,9 @@ typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 
 #define PSTRIDE 132          // floats per (item, head) partial: 128 acc + m + l + 2 pad
-#define NWAVES 4
+#ifndef NWAVES
+#define NWAVES 8        // wavefronts of a workgroup of the main kernel: two per SIMD, one workgroup per CU
+#endif
 #define LUT_BYTES 65536
 #define LOG2E 1.4426950408889634f
 #define LN2 0.6931471805599453f
@@ -178,25 +180,27 @@ template <int W>
 __device__ static inline void build_lut(uint8_t* lut, const DecodeArgs& a, int tid) {
     const int lane = tid & 63, wave = tid >> 6;
     if constexpr (W == 2) {
-        // row = code byte = wave * 64 + i * 4 + (lane >> 4): its codes are lane >> 4, i & 3, i >> 2 and
-        // wave, so the row's eight bytes are put together from the four centroids without any
+        // row = code byte: its lowest code is lane >> 4 and the other three are the same for the whole
+        // wavefront, so the row's eight bytes are put together from the four centroids without any
         // cross-lane traffic; the lanes of one store cover consecutive 16-byte pieces of four rows
         uint32_t h[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) h[k] = half_bits(a.cbs[k]);
         const auto sel = [&](int k) { return k == 0 ? h[0] : k == 1 ? h[1] : k == 2 ? h[2] : h[3]; };
-        const uint32_t own = sel(lane >> 4), top = sel(wave) << 16;
+        const uint32_t own = sel(lane >> 4);
+        constexpr int ROWS = 256 / NWAVES;                   // rows of this wavefront
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t x = own | (h[i & 3] << 16), y = h[i >> 2] | top;
-            *reinterpret_cast<uint4*>(lut + (wave * 64 + i * 4 + (lane >> 4)) * 256 + (lane & 15) * 16) = make_uint4(x, y, x, y);
+        for (int i = 0; i < ROWS / 4; ++i) {
+            const int base = wave * ROWS + i * 4;            // wave-uniform; the row is base + (lane >> 4)
+            const uint32_t x = own | (sel((base >> 2) & 3) << 16), y = sel((base >> 4) & 3) | (sel(base >> 6) << 16);
+            *reinterpret_cast<uint4*>(lut + (base + (lane >> 4)) * 256 + (lane & 15) * 16) = make_uint4(x, y, x, y);
         }
     } else {
         uint32_t v;
         if constexpr (W == 3) { v = half_bits(pick<8>(a.cbs + 4, tid & 7)) | (half_bits(pick<8>(a.cbs + 4, (tid >> 3) & 7)) << 16); }
-        else if constexpr (W == 4) { v = half_bits(pick<16>(a.cbs + 12, tid & 15)) | (half_bits(pick<16>(a.cbs + 12, tid >> 4)) << 16); }
-        else { v = half_bits(a.cb[codebook_offset(3) + tid]) * 0x10001u; }
-        const bool on = W != 3 || wave == 0;              // the 3-bit table has 64 entries
+        else if constexpr (W == 4) { v = half_bits(pick<16>(a.cbs + 12, tid & 15)) | (half_bits(pick<16>(a.cbs + 12, (tid >> 4) & 15)) << 16); }
+        else { v = half_bits(a.cb[codebook_offset(3) + (tid & 255)]) * 0x10001u; }
+        const bool on = wave < 4 && (W != 3 || wave == 0);  // 256 entries (64 for the 3-bit table): four wavefronts' worth
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int src = i * 8 + (lane >> 3);
@@ -543,7 +547,7 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
 // main kernel: NP passes of four query heads (GQA groups up to 4 * NP)
 // ------------------------------------------------------------------------------------------------
 template <int NP>
-__global__ __launch_bounds__(256, 2) void decode_main_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs a) {
     __shared__ __align__(16) uint8_t lut[LUT_BYTES];     // centroid table; reused to combine the wavefronts
     __shared__ float wm[NWAVES][4 * NP], wl[NWAVES][4 * NP];
     __shared__ uint4 qsh[4 * NP * 32];
@@ -587,7 +591,7 @@ __global__ __launch_bounds__(256, 2) void decode_main_kernel(DecodeArgs a) {
     }
     __syncthreads();
     float* dst = a.partial + (size_t)item * GP * PSTRIDE;
-    for (int e = tid; e < GP * HD; e += 256) {
+    for (int e = tid; e < GP * HD; e += NWAVES * 64) {
         const int g = e / HD, j = e % HD;
         float M = wm[0][g];
 #pragma unroll
@@ -822,8 +826,8 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
         // start and end timestamps, not those of separate marker packets
         hipEvent_t e0 = rec ? g_prof_events[2 * g_prof_used] : nullptr;
         hipEvent_t e1 = rec ? g_prof_events[2 * g_prof_used + 1] : nullptr;
-        if (GP == 4) hipExtLaunchKernelGGL((decode_main_kernel<1>), dim3(n_items), dim3(256), 0, st, e0, e1, 0, a);
-        else hipExtLaunchKernelGGL((decode_main_kernel<2>), dim3(n_items), dim3(256), 0, st, e0, e1, 0, a);
+        if (GP == 4) hipExtLaunchKernelGGL((decode_main_kernel<1>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
+        else hipExtLaunchKernelGGL((decode_main_kernel<2>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
         ODMKV_CHECK_LAUNCH("decode_main_kernel");
         if (rec) ++g_prof_used;
     }

@@ -454,12 +454,26 @@ class TurboQuantAdaptiveKVCacheState:
     # ------------------------------------------------------------------ fused attention
     def _build_items(self, target_items: Optional[int] = None, min_item_bytes: Optional[int] = None) -> None:
         import os
-        target_items = int(os.environ.get("ODMKV_DECODE_ITEMS", 512)) if target_items is None else target_items
+        if target_items is None:
+            # one workgroup per item, one (eight-wavefront) workgroup per compute unit: all resident at once
+            target_items = int(os.environ.get("ODMKV_DECODE_ITEMS", 0)) or \
+                torch.cuda.get_device_properties(self.device).multi_processor_count
         min_item_bytes = int(os.environ.get("ODMKV_DECODE_MIN_ITEM_BYTES", 16384)) if min_item_bytes is None else min_item_bytes
         used = (self._counts + TILE - 1) // TILE
         used[4] = np.diff(self._seg_tile[4])              # exact segments grow between rebuilds
         total = sum(int(used[li].sum()) * _TILE_BYTES[li] for li in range(5))
+        # the largest number of items that does not exceed the target: every (segment, level) run of
+        # tiles is cut into pieces of about per_item bytes, and a run's last piece may be short, so
+        # per_item grows until the pieces fit (one workgroup per item, all resident at once)
+        runs = [int(used[li, s]) * _TILE_BYTES[li] for s in range(self._nseg) for li in range(5) if used[li, s] > 0]
+        tile_b = [_TILE_BYTES[li] for s in range(self._nseg) for li in range(5) if used[li, s] > 0]
+
+        def n_pieces(per_item: int) -> int:
+            return sum(-(-(r // b) // max(1, int(round(per_item / b)))) for r, b in zip(runs, tile_b))
+
         per_item = max(total // max(target_items, 1), min_item_bytes)
+        while n_pieces(per_item) > target_items and per_item < total:
+            per_item += max(per_item // 64, 1)
         items, ranges = [], [0]
         for s in range(self._nseg):
             for li in range(5):
