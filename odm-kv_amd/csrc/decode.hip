@@ -391,12 +391,12 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
     const float vsc = a.inv_s[li], ksc = a.inv_s[li] * a.scaling * LOG2E;
-    // The table needs nothing from memory and is built first: behind a wavefront's tile requests its
-    // LDS traffic would wait for the memory pipeline to accept them (every wavefront of the chip asks
-    // for its tiles at the same moment).  Loads return in issue order: the (small) query slice goes
-    // first so that staging it does not have to wait for the tile.
+    // The table needs nothing from memory and is built before the tiles are requested: behind a
+    // wavefront's tile requests its LDS traffic would wait for the memory pipeline to accept them
+    // (every wavefront of the chip asks for its tiles at the same moment).  Loads return in issue
+    // order: the (small) query slice goes first so that staging it does not have to wait for the tile.
+    const uint4 qslice = load_query_slice<NP>(a, a.qrot + (size_t)bq0 * 32, tid);   // one request: lands while the table is built
     build_lut<W>(lut, a, tid);
-    const uint4 qslice = load_query_slice<NP>(a, a.qrot + (size_t)bq0 * 32, tid);
     TileData<W> cur;
     int tt = wave;
     int nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
