@@ -211,6 +211,12 @@ int odmkv_profile_enable(int max_records);
 int odmkv_profile_collect(float* ms, int capacity, int* n_out);
 int odmkv_profile_disable(void);
 
+/* Which of the three kernels of odmkv_decode_attn later calls launch: bit 0 the query preparation,
+ * bit 1 the main (streaming) kernel, bit 2 the merge.  7 (the default) is the product behaviour; any
+ * other value is for timing one kernel in isolation over buffers that a full call has filled
+ * (e.g. 2: the main kernel alone, back to back, between two events).  Returns the previous mask. */
+int odmkv_decode_stage_mask(int mask);
+
 /* Yardstick for the roofline (no counterpart in the reference): a plain streaming read of `bytes`
  * bytes at `buf` (device, 16-byte aligned) by `grid` workgroups of 256 threads; `sink` is a device
  * word that is practically never written.  Timing it over buffers that rotate through more than

@@ -781,6 +781,13 @@ extern "C" int odmkv_probe_read(const void* buf, size_t bytes, int grid, void* s
     return 0;
 }
 
+static int g_stage_mask = 7;
+extern "C" int odmkv_decode_stage_mask(int mask) {
+    const int old = g_stage_mask;
+    g_stage_mask = mask & 7;
+    return old;
+}
+
 static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
 
 extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
@@ -817,10 +824,12 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     a.qs = (uint4*)((char*)workspace + qbytes);
     a.partial = (float*)((char*)workspace + 2 * qbytes);
     a.out = out; a.lse = lse;
-    hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(128 * PREP_SLICES), 0, st, a);
-    ODMKV_CHECK_LAUNCH("decode_prep_kernel");
+    if (g_stage_mask & 1) {
+        hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(128 * PREP_SLICES), 0, st, a);
+        ODMKV_CHECK_LAUNCH("decode_prep_kernel");
+    }
     const int GP = group_pad(G);
-    if (n_items > 0) {
+    if (n_items > 0 && (g_stage_mask & 2)) {
         const bool rec = g_prof_on && (size_t)(2 * g_prof_used + 1) < g_prof_events.size();
         // when measuring, the events are attached to the dispatch itself: they carry the kernel's own
         // start and end timestamps, not those of separate marker packets
@@ -831,8 +840,10 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
         ODMKV_CHECK_LAUNCH("decode_main_kernel");
         if (rec) ++g_prof_used;
     }
-    if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);
-    else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);
-    ODMKV_CHECK_LAUNCH("decode_merge_kernel");
+    if (g_stage_mask & 4) {
+        if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);
+        else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);
+        ODMKV_CHECK_LAUNCH("decode_merge_kernel");
+    }
     return 0;
 }

@@ -65,6 +65,7 @@ def _load() -> C.CDLL:
         "odmkv_profile_enable": (C.c_int, [i32]),
         "odmkv_profile_collect": (C.c_int, [C.POINTER(C.c_float), i32, C.POINTER(C.c_int)]),
         "odmkv_profile_disable": (C.c_int, []),
+        "odmkv_decode_stage_mask": (C.c_int, [i32]),
         "odmkv_probe_read": (C.c_int, [vp, sz, i32, vp, vp]),
     }
     for name, (res, args) in sig.items():
@@ -80,7 +81,7 @@ EXPORTS = ("odmkv_version", "odmkv_last_error", "odmkv_score_workspace_bytes", "
            "odmkv_pack_workspace_bytes", "odmkv_quant_pack", "odmkv_quantize_rows",
            "odmkv_dequantize_rows", "odmkv_dequant", "odmkv_append_exact",
            "odmkv_decode_workspace_bytes", "odmkv_decode_attn",
-           "odmkv_profile_enable", "odmkv_profile_collect", "odmkv_profile_disable", "odmkv_probe_read")
+           "odmkv_profile_enable", "odmkv_profile_collect", "odmkv_profile_disable", "odmkv_decode_stage_mask", "odmkv_probe_read")
 
 
 def check(rc: int) -> None:
