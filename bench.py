@@ -37,8 +37,8 @@ for p in (ROOT, os.path.join(ROOT, "odm-kv_amd")):
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the main decode kernel on the default workload, from the L2 counters
 # (FETCH_SIZE and WRITE_SIZE, one rocprofv3 --pmc run each, scaled by a 256 MiB copy of known size):
-# 20.41 MB fetched + 1.10 MB written.  Applies to --layers 32 --ctx 32768 --target 2.0 only.
-MEASURED_TRAFFIC_BYTES = 21.51e6
+# 20.16 MB fetched + 0.54 MB written.  Applies to --layers 32 --ctx 32768 --target 2.0 only.
+MEASURED_TRAFFIC_BYTES = 20.70e6
 LEVELS = (0, 2, 3, 4, 8, 16)
 
 
