@@ -8,6 +8,9 @@
 //   launch 1..16  four halvings each: the 15 midpoints the next four steps can reach form a binary
 //                 tree that is known in advance, so one pass over the scores evaluates them all;
 //   launch 17     the final lambda, which also records the chosen level of every token.
+// The costs use lambda rounded to fp32, so once the bracket's ends are neighbouring fp32 numbers
+// (after about 32 halvings on typical scores) the rest of the search is decided by rounding alone:
+// it is walked on the spot and the remaining halving launches return immediately.
 // Every workgroup writes its partial bit sums; the workgroup that finishes last (found by an
 // atomic ticket) adds them up, walks the bracket and prepares the next launch's candidates.
 // Nothing ever waits on another workgroup and the host is never consulted.  All sums are
@@ -41,6 +44,8 @@ struct RowState {
     int n_active;
     unsigned int max_finite; // bit pattern
     int has_finite, has_nonfinite;
+    int lo_moved, hi_within;       // the bracket ends' averages are known (lo: above budget, hi: within)
+    int collapsed;                 // the remaining halvings were resolved without evaluations
     int final_hist[NLV];
 };
 
@@ -101,6 +106,7 @@ __global__ void alloc_init_kernel(AllocArgs a) {
         t = fmax(t, (double)a.nominal[0]);
         st.lo = 0.0; st.hi = 1.0; st.target = t; st.gap = 0.0; st.lam = 1.0;
         st.n_active = 0; st.max_finite = 0u; st.has_finite = 0; st.has_nonfinite = 0;
+        st.lo_moved = 0; st.hi_within = 0; st.collapsed = 0;
         for (int k = 0; k < NLV; ++k) st.final_hist[k] = 0;
     }
 }
@@ -167,13 +173,27 @@ __device__ static void advance(const AllocArgs& a, int row, int L, const unsigne
             avg_hi = (double)((float)sums[j] / nf);
         }
         st.lo = 0.0; st.hi = hi;
+        st.hi_within = !(avg_hi > st.target);
     } else if (L < L_FINAL) {
         double lo = st.lo, hi = st.hi;
         int node = 1;
         for (int s = 0; s < STEPS; ++s) {
             const double mid = (lo + hi) * 0.5;
             const double avg = (double)((float)sums[node] / nf);
-            if (avg > st.target) { lo = mid; node = 2 * node + 1; } else { hi = mid; node = 2 * node; }
+            if (avg > st.target) { lo = mid; node = 2 * node + 1; st.lo_moved = 1; } else { hi = mid; node = 2 * node; st.hi_within = 1; }
+        }
+        // The costs see lambda rounded to fp32.  Once fp32(lo) and fp32(hi) are neighbouring floats,
+        // every later midpoint rounds to one of the two, whose averages are known (lo was evaluated
+        // above the budget, hi within it): the remaining halvings need no pass over the scores and
+        // are walked here; the launches that would have evaluated them return at once.
+        const float fl = (float)lo, fh = (float)hi;
+        if (st.lo_moved && st.hi_within && fl < fh && nextafterf(fl, INFINITY) == fh) {
+            for (int s = L * STEPS; s < N_HALVE_LAUNCH * STEPS; ++s) {
+                const double mid = (lo + hi) * 0.5;
+                if ((float)mid == fl) lo = mid; else hi = mid;
+            }
+            st.collapsed = 1;
+            st.lam = (lo + hi) * 0.5;
         }
         st.lo = lo; st.hi = hi;
     } else {
@@ -228,6 +248,7 @@ __global__ __launch_bounds__(EV_THREADS) void alloc_eval_kernel(AllocArgs a, int
     const int row = blockIdx.y, tid = threadIdx.x;
     const RowState& st = a.state[row];
     if (st.n_active == 0) return;
+    if (L > 0 && L < L_FINAL && st.collapsed) return;       // this launch's halvings are already decided
     if (tid < SLOTS * NLV) {
         const int c = tid / NLV, k = tid % NLV;
         lamb[c][k] = __fmul_rn(candidate(st, L, c), a.bitsf[k]);
