@@ -97,6 +97,18 @@ def test_allocator_bit_exact_random(target):
     _check_alloc(s, target, _sink(8, 4096))
 
 
+@pytest.mark.parametrize("scale,target", [(1e-9, 2.0), (1e-20, 3.0), (1e6, 8.0), (1e12, 2.0), (1.0, 15.9), (1e-30, 2.0)])
+def test_allocator_bit_exact_across_score_scales(scale, target):
+    """The multiplier bracket reaches neighbouring fp32 numbers after a number of halvings that depends
+    on the scale of the scores (24 for large ones, all 64 for tiny ones, never when the bracket was
+    widened to its limit): from there the search is resolved without evaluations, and must still land
+    on the lambda, and the bits, of the evaluated search."""
+    g = torch.Generator().manual_seed(41)
+    s = torch.exp(1.5 * torch.randn(4, 3000, generator=g)) * scale
+    s[:, :4] = s.max()
+    _check_alloc(s, target, _sink(4, 3000))
+
+
 def test_allocator_bit_exact_edge_cases():
     g = torch.Generator().manual_seed(9)
     vals = torch.exp(torch.linspace(-3, 6, 12))
