@@ -172,24 +172,38 @@ def main() -> int:
         # what can ONE launch of a given size reach?  buffers rotate through 2 GiB so every launch reads HBM
         pool = torch.ones(2 << 30, dtype=torch.uint8, device=dev)
         sink = torch.zeros(64, dtype=torch.int32, device=dev)
-        st_ptr = _lib.stream_ptr(dev)
         rows = []
         for nbytes in (19336677, 80740000, 536870912):
             stride = (nbytes + (2 << 20)) & ~((2 << 20) - 1)
             nbuf = min((2 << 30) // stride, 64)
             for grid in (1024, 2048, 4096):
-                ms = []
-                for it in range(3 * nbuf):
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e0.record()
-                    _lib.check(_lib.lib.odmkv_probe_read(pool.data_ptr() + (it % nbuf) * stride, nbytes, grid, sink.data_ptr(), st_ptr))
-                    e1.record()
-                    e1.synchronize()
-                    if it >= nbuf:
-                        ms.append(e0.elapsed_time(e1))
-                med = statistics.median(ms)
-                rows.append({"bytes": nbytes, "grid": grid, "median_us": round(med * 1e3, 2),
-                             "GBps": round(nbytes / (med * 1e-3) / 1e9), "pct_of_8TBps": round(100 * nbytes / (med * 1e-3) / 8e12, 1)})
+                def sweep():
+                    for it in range(nbuf):
+                        _lib.check(_lib.lib.odmkv_probe_read(pool.data_ptr() + it * stride, nbytes, grid, sink.data_ptr(),
+                                                             _lib.stream_ptr(dev)))
+                # the launches of one sweep over the buffers go back to back (one graph), timed between two
+                # events: event pairs around single launches would add about 2 us to each
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    sweep()
+                torch.cuda.current_stream().wait_stream(side)
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    sweep()
+                g.replay()
+                reps = 5
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                e0.record()
+                for _ in range(reps):
+                    g.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                avg = e0.elapsed_time(e1) / (reps * nbuf)
+                rows.append({"bytes": nbytes, "grid": grid, "buffers": nbuf, "avg_us": round(avg * 1e3, 2),
+                             "GBps": round(nbytes / (avg * 1e-3) / 1e9), "pct_of_8TBps": round(100 * nbytes / (avg * 1e-3) / 8e12, 1)})
         print(json.dumps({"read_ceiling": rows}))
         return 0
 
