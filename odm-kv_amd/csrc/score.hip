@@ -48,11 +48,22 @@ __device__ static inline void load8(const void* base, size_t elem_off, float* x)
     }
 }
 
+// sum over the 16 lanes that share a row, by data-parallel-primitive moves (no LDS traffic): inside the
+// quad, then the neighbouring quad, then the other half of the 16-lane row.  Every lane ends with the
+// total; the order of the additions is fixed per lane (only lane 0 of the row is used).
+template <int CTRL>
+__device__ static inline float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
 __device__ static inline float group16_sum(float v) {
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    v += dpp_move<0xB1>(v);     // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);     // quad_perm [2,3,0,1]
+    v += dpp_move<0x124>(v);    // row_ror 4
+    v += dpp_move<0x128>(v);    // row_ror 8
     return v;
 }
+#define SC_UNROLL 4            // rows in flight per lane group: their loads are issued before any is used
+#define SC_UNROLL_V 4          // the same for the two passes over V
 
 // merge two online-softmax states
 __device__ static inline void ms_merge(float& m, float& s, float m2, float s2) {
@@ -81,35 +92,58 @@ __global__ __launch_bounds__(256) void score_logits_kernel(ScoreArgs a) {
     for (int g = 0; g < GMAX; ++g) { m[g] = -INFINITY; s[g] = 0.0f; }
     const float inv_div = 11.313708498984761f;        // sqrt(128)
     const int t0 = chunk * ROWS_PER_WG;
-    for (int it = 0; it < ROWS_PER_WG / 16; ++it) {
-        const int t = t0 + it * 16 + wave * 4 + rsub;
-        const bool ok = t < a.Tc;
-        float x[8];
-        if (ok) load8<DT>(a.K, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, x);
-        else {
+    // A group of 16 lanes takes four consecutive rows per trip (all four requested before any is
+    // used).  The row sums leave the reduction in every lane of the group, so lane u < 4 of the group
+    // owns row u: it stores the row's results (the 16 owners of a wave write 16 consecutive floats)
+    // and keeps the running softmax statistics of its rows.
+    static_assert(SC_UNROLL == 4, "four rows per lane group and trip");
+    const bool owner = part < SC_UNROLL;
+    for (int it0 = 0; it0 < ROWS_PER_WG / 16; it0 += SC_UNROLL) {
+        const int tb = t0 + it0 * 16 + (wave * 4 + rsub) * SC_UNROLL;
+        float xs[SC_UNROLL][8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = 0.0f;
+        for (int u = 0; u < SC_UNROLL; ++u) {
+            if (tb + u < a.Tc) load8<DT>(a.K, (size_t)h * a.sH + (size_t)(a.n_sink + tb + u) * a.sT + part * 8, xs[u]);
+            else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) xs[u][e] = 0.0f;
+            }
         }
-        float kn = 0.0f;
+        float kn_own = 0.0f, d_own[GMAX];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) kn = __fmaf_rn(x[e], x[e], kn);
-        kn = group16_sum(kn);
-        if (ok && part == 0) a.kn2[(size_t)h * a.Tc + t] = kn;
+        for (int g = 0; g < GMAX; ++g) d_own[g] = 0.0f;
 #pragma unroll
-        for (int g = 0; g < GMAX; ++g) {
-            if (g < a.Gl) {
-                float d = 0.0f;
+        for (int u = 0; u < SC_UNROLL; ++u) {
+            const float* x = xs[u];
+            float kn = 0.0f;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) d = __fmaf_rn(x[e], mu_r[g][e], d);
-                d = group16_sum(d) / inv_div;
-                if (ok && part == 0) {
-                    a.logits[((size_t)h * a.G + g) * a.Tc + t] = d;
-                    ms_merge(m[g], s[g], d, 1.0f);
+            for (int e = 0; e < 8; ++e) kn = __fmaf_rn(x[e], x[e], kn);
+            kn = group16_sum(kn);
+            kn_own = part == u ? kn : kn_own;
+#pragma unroll
+            for (int g = 0; g < GMAX; ++g) {
+                if (g < a.Gl) {
+                    float d = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) d = __fmaf_rn(x[e], mu_r[g][e], d);
+                    d = group16_sum(d) / inv_div;
+                    d_own[g] = part == u ? d : d_own[g];
+                }
+            }
+        }
+        const int t = tb + part;
+        if (owner && t < a.Tc) {
+            a.kn2[(size_t)h * a.Tc + t] = kn_own;
+#pragma unroll
+            for (int g = 0; g < GMAX; ++g) {
+                if (g < a.Gl) {
+                    a.logits[((size_t)h * a.G + g) * a.Tc + t] = d_own[g];
+                    ms_merge(m[g], s[g], d_own[g], 1.0f);
                 }
             }
         }
     }
-    // only lanes with part == 0 hold statistics; butterfly over the wave, then over the 4 waves
+    // only the owner lanes hold statistics; butterfly over the wave, then over the 4 waves
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) {
         if (g < a.Gl) {
@@ -164,24 +198,39 @@ __global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     float ps = 0.0f;
     const int t0 = chunk * ROWS_PER_WG;
-    for (int it = 0; it < ROWS_PER_WG / 16; ++it) {
-        const int t = t0 + it * 16 + wave * 4 + rsub;
-        if (t < a.Tc) {
-            float pt;
-            if (a.attn != nullptr) {
-                pt = a.attn[(size_t)h * a.T + a.n_sink + t];
-            } else {
-                float acc = 0.0f;
+    for (int it0 = 0; it0 < ROWS_PER_WG / 16; it0 += SC_UNROLL_V) {
+        float xs[SC_UNROLL_V][8], lg[SC_UNROLL_V][GMAX];
 #pragma unroll
-                for (int g = 0; g < GMAX; ++g)
-                    if (g < a.G) acc += __expf(a.logits[((size_t)h * a.G + g) * a.Tc + t] - Mg[g]) / Zg[g];
-                pt = acc / (float)a.G;
+        for (int u = 0; u < SC_UNROLL_V; ++u) {
+            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
+            if (t < a.Tc) {
+                load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, xs[u]);
+                if (a.attn != nullptr) lg[u][0] = a.attn[(size_t)h * a.T + a.n_sink + t];
+                else {
+#pragma unroll
+                    for (int g = 0; g < GMAX; ++g)
+                        if (g < a.G) lg[u][g] = a.logits[((size_t)h * a.G + g) * a.Tc + t];
+                }
             }
-            if (part == 0) { a.p[(size_t)h * a.Tc + t] = pt; ps += pt; }
-            float x[8];
-            load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, x);
+        }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = __fmaf_rn(pt, x[e], o[e]);
+        for (int u = 0; u < SC_UNROLL_V; ++u) {
+            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
+            if (t < a.Tc) {
+                float pt;
+                if (a.attn != nullptr) {
+                    pt = lg[u][0];
+                } else {
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int g = 0; g < GMAX; ++g)
+                        if (g < a.G) acc += __expf(lg[u][g] - Mg[g]) / Zg[g];
+                    pt = acc / (float)a.G;
+                }
+                if (part == 0) { a.p[(size_t)h * a.Tc + t] = pt; ps += pt; }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = __fmaf_rn(pt, xs[u][e], o[e]);
+            }
         }
     }
     const int grp = wave * 4 + rsub;
@@ -233,30 +282,40 @@ __global__ __launch_bounds__(256) void score_final_kernel(ScoreArgs a) {
     for (int e = 0; e < 8; ++e) ob[e] = a.obar[h * HD + part * 8 + e];
     float best = 0.0f;
     const int t0 = chunk * ROWS_PER_WG;
-    for (int it = 0; it < ROWS_PER_WG / 16; ++it) {
-        const int t = t0 + it * 16 + wave * 4 + rsub;
-        const bool ok = t < a.Tc;
-        float x[8];
-        if (ok) load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, x);
-        else {
+    for (int it0 = 0; it0 < ROWS_PER_WG / 16; it0 += SC_UNROLL_V) {
+        float xs[SC_UNROLL_V][8], pin[SC_UNROLL_V], knin[SC_UNROLL_V];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = 0.0f;
-        }
-        float vn = 0.0f, ir = 0.0f;
+        for (int u = 0; u < SC_UNROLL_V; ++u) {
+            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
+            pin[u] = 0.0f; knin[u] = 0.0f;
+            if (t < a.Tc) {
+                load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, xs[u]);
+                if (part == 0) { pin[u] = a.p[(size_t)h * a.Tc + t]; knin[u] = a.kn2[(size_t)h * a.Tc + t]; }
+            } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            vn = __fmaf_rn(x[e], x[e], vn);
-            const float dlt = x[e] - ob[e];
-            ir = __fmaf_rn(dlt, dlt, ir);
+                for (int e = 0; e < 8; ++e) xs[u][e] = 0.0f;
+            }
         }
-        vn = group16_sum(vn);
-        ir = group16_sum(ir);
-        if (ok && part == 0) {
-            const float pe = a.p[(size_t)h * a.Tc + t] + a.eps;
-            const float kterm = (a.kn2[(size_t)h * a.Tc + t] / (float)HD) * ir;
-            const float sc = (pe * pe) * (vn + kterm);
-            a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
-            best = fmaxf(best, sc);
+#pragma unroll
+        for (int u = 0; u < SC_UNROLL_V; ++u) {
+            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
+            const bool ok = t < a.Tc;
+            float vn = 0.0f, ir = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                vn = __fmaf_rn(xs[u][e], xs[u][e], vn);
+                const float dlt = xs[u][e] - ob[e];
+                ir = __fmaf_rn(dlt, dlt, ir);
+            }
+            vn = group16_sum(vn);
+            ir = group16_sum(ir);
+            if (ok && part == 0) {
+                const float pe = pin[u] + a.eps;
+                const float kterm = (knin[u] / (float)HD) * ir;
+                const float sc = (pe * pe) * (vn + kterm);
+                a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
+                best = fmaxf(best, sc);
+            }
         }
     }
     best = wave_max(best);
