@@ -182,8 +182,9 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  * (bh, level index 0..4, first tile, tile count, tokens held by those tiles, first tile of the
  * segment, 0, 0); for the exact level (index 4) the token count is read from seg_count instead,
  * so that tokens appended since the list was built are seen.  item_range: device int32
- * [B*Hkv + 1] first item of each bh.  out: device fp32 [B, Hq, 128]; lse: device fp32 [B, Hq]
- * or NULL (log-sum-exp of the scaled logits).
+ * [B*Hkv + 1] first item of each bh; a bh may have at most ODMKV_MAX_ITEMS_PER_SEGMENT items (the
+ * caller builds the list and keeps to it; one item per compute unit is what performs best).
+ * out: device fp32 [B, Hq, 128]; lse: device fp32 [B, Hq] or NULL (log-sum-exp of the scaled logits).
  * pi_k_t is the key rotation TRANSPOSED (row-major [128,128] of Pi_k^T), pi_v the value rotation as is.
  * The query is rounded to fp16 on entry (the attention being replaced receives it in the model's
  * fp16/bf16).  The centroid tables live in LDS as fp16; to keep their rounding out of the result,
@@ -192,6 +193,7 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  * floats (the small tables travel as kernel arguments), and inv_scales (host, 4 floats) the
  * reciprocals of those scales.
  */
+#define ODMKV_MAX_ITEMS_PER_SEGMENT 1024
 size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);
 int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
                       const odmkv_packed_t* store,

@@ -616,7 +616,7 @@ __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs 
 // ------------------------------------------------------------------------------------------------
 #define MERGE_THREADS 512
 #define MERGE_SLICES (MERGE_THREADS / HD)
-#define MERGE_MAX_ITEMS 1024
+#define MERGE_MAX_ITEMS ODMKV_MAX_ITEMS_PER_SEGMENT
 
 template <int GP>
 __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs a) {
@@ -811,6 +811,8 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     const int G = Hq / store->Hkv;
     ODMKV_CHECK_ARG(G <= ODMKV_MAX_GROUP, "decode_attn: GQA group %d exceeds %d", G, ODMKV_MAX_GROUP);
     ODMKV_CHECK_ARG(n_items >= 0, "decode_attn: negative item count");
+    ODMKV_CHECK_ARG((long)n_items <= (long)ODMKV_MAX_ITEMS_PER_SEGMENT * B * store->Hkv,
+                    "decode_attn: %d items exceed %d per (sequence, kv-head)", n_items, ODMKV_MAX_ITEMS_PER_SEGMENT);
     ODMKV_CHECK_ARG(workspace_bytes >= odmkv_decode_workspace_bytes(B, Hq, n_items), "decode_attn: workspace too small");
     hipStream_t st = (hipStream_t)stream;
     DecodeArgs a;

@@ -28,6 +28,7 @@ from .tq_backend import (cached_rotation, codebook_table, decode_tables, normali
                          normalize_value_quantizer)
 
 _LEVEL_INDEX = {2: 0, 3: 1, 4: 2, 8: 3, 16: 4}
+_MAX_ITEMS_PER_SEGMENT = 1024        # ODMKV_MAX_ITEMS_PER_SEGMENT of include/odmkv.h
 _TILE_BYTES = [TILE * 16 * w + 2 * TILE * 4 for w in WIDTHS] + [2 * TILE * HEAD_DIM * 2]
 
 
@@ -471,8 +472,13 @@ class TurboQuantAdaptiveKVCacheState:
         def n_pieces(per_item: int) -> int:
             return sum(-(-(r // b) // max(1, int(round(per_item / b)))) for r, b in zip(runs, tile_b))
 
+        def most_per_segment(per_item: int) -> int:
+            return max(sum(-(-int(used[li, s]) // max(1, int(round(per_item / _TILE_BYTES[li])))) for li in range(5))
+                       for s in range(self._nseg))
+
         per_item = max(total // max(target_items, 1), min_item_bytes)
-        while n_pieces(per_item) > target_items and per_item < total:
+        # (the merge kernel takes at most _MAX_ITEMS_PER_SEGMENT items of one (sequence, kv-head))
+        while (n_pieces(per_item) > target_items or most_per_segment(per_item) > _MAX_ITEMS_PER_SEGMENT) and per_item < total:
             per_item += max(per_item // 64, 1)
         items, ranges = [], [0]
         for s in range(self._nseg):

@@ -99,6 +99,26 @@ def test_decode_special_cases():
     assert rel_err(st.decode_attention(q.to(DEV)).cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
 
 
+def test_work_list_respects_the_per_segment_item_limit():
+    """One long (sequence, kv-head) cut into one-tile items would exceed the number of items the merge
+    kernel takes per segment; the work-list builder must cut coarser, and the result must not change."""
+    g = torch.Generator().manual_seed(5)
+    T = 70000
+    k = torch.randn(1, 1, T, 128, generator=g).half(); v = torch.randn(1, 1, T, 128, generator=g).half()
+    bits = torch.full((1, 1, T), 2, dtype=torch.int32); bits[..., :4] = 16; bits[..., -64:] = 16
+    st, ref = _pair(k, v, bits)
+    q = torch.randn(1, 4, 128, generator=g).half().float()
+    want = decode_attention_state(q, ref)
+    st._build_items(1 << 20, 1)                       # as many, as small items as the builder will give
+    items, ranges, n_items = st._items
+    per_segment = np.diff(ranges.cpu().numpy())
+    assert per_segment.max() <= 1024 and n_items >= 512
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
+    st._build_items(8, 1 << 30)                       # and a handful of huge ones
+    assert st._items[2] <= 8
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
+
+
 def test_decode_after_appends_and_flush():
     g = torch.Generator().manual_seed(8)
     B, H, G = 1, 4, 4
