@@ -90,6 +90,57 @@ def parity_gate(dev):
     return eps, err
 
 
+def press_e2e(dev, T, target, n_new):
+    """The press end to end on a model of Llama-3-8B's attention shape (2 layers, random weights):
+    prefill T tokens under the press, then n_new greedy decode steps, once over the packed cache
+    with the fused kernel and once over the dense re-materialised cache with the model's own
+    attention function (what the reference executes).  Wall time per decode step, device-synchronised."""
+    import torch
+    from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM
+    from kvquant import RiskScorer, TurboQuantPerTokenBackendPress, attention_patch
+    torch.manual_seed(0)
+    cfg = LlamaConfig(hidden_size=4096, num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                      intermediate_size=14336, vocab_size=32000, max_position_embeddings=max(T + n_new + 8, 8192),
+                      rope_theta=500000.0, attn_implementation="sdpa")
+    model = LlamaForCausalLM(cfg).to(device=dev, dtype=torch.float16).eval()
+    ids = torch.randint(0, 32000, (1, T), generator=torch.Generator().manual_seed(1)).to(dev)
+    out = {"model": "2 x Llama-3-8B-shaped layer, random init, fp16", "prefill_tokens": T, "decode_tokens": n_new,
+           "target_avg_bits": target}
+    for mode in ("fused", "dense"):
+        os.environ["ODMKV_FUSED_DECODE"] = "1" if mode == "fused" else "0"
+        scorer = RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
+        scorer.normalize_grain = "global"
+        press = TurboQuantPerTokenBackendPress(
+            scorer=scorer, bit_levels=LEVELS, target_avg_bits=target, eviction_cost=0.5, seed=42, decode_quant=True,
+            sink_tokens=4, layerwise=True, key_quantizer="mse", value_quantizer="mse", buffer_size=128)
+        before = dict(attention_patch.call_counts)
+        cache = DynamicCache()
+        with torch.inference_mode(), press(model):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            h = model.model(input_ids=ids, past_key_values=cache).last_hidden_state[:, -1:, :]
+            tok = model.lm_head(h)[0, -1].argmax().view(1, 1)
+            torch.cuda.synchronize()
+            t_prefill = time.perf_counter() - t0
+            steps = []
+            for step in range(n_new):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                logits = model(input_ids=tok, past_key_values=cache,
+                               position_ids=torch.tensor([[T + step]], device=dev)).logits
+                tok = logits[0, -1].argmax().view(1, 1)
+                torch.cuda.synchronize()
+                steps.append(time.perf_counter() - t0)
+        took = {k: attention_patch.call_counts[k] - before[k] for k in before}
+        out[mode] = {"prefill_s": round(t_prefill, 3), "decode_step_ms_median": round(statistics.median(steps[4:]) * 1e3, 3),
+                     "decode_step_ms_min": round(min(steps[4:]) * 1e3, 3), "attention_calls": took}
+        del cache, press
+        torch.cuda.empty_cache()
+    os.environ.pop("ODMKV_FUSED_DECODE", None)
+    out["dense_over_fused"] = round(out["dense"]["decode_step_ms_median"] / out["fused"]["decode_step_ms_median"], 2)
+    return out
+
+
 def cpu_baseline(sample_T, n_kv, n_q, eps, threads):
     """The reference's CPU path, restated by the oracle, on a bounded sample (one layer of
     `sample_T` tokens): compress it, then time what a decode step costs the reference - SDPA over
@@ -150,6 +201,11 @@ def main() -> int:
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for counter runs under rocprofv3 --pmc: a few eager decode steps and one plain 256 MiB "
                          "device copy (the calibration kernel), nothing else timed")
+    ap.add_argument("--press-e2e", action="store_true",
+                    help="instead of the kernel benchmark: a 2-layer random-init Llama-3-8B-shaped model under the "
+                         "press, prefill of --ctx tokens, then greedy decode with the fused kernel and with the dense "
+                         "re-materialised cache (the reference's path); prints per-token times")
+    ap.add_argument("--e2e-tokens", type=int, default=48)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the path: every box in this build has one GPU and "
@@ -167,6 +223,10 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     n_kv, n_q, T, NL = 8, 32, args.ctx, args.layers
+
+    if args.press_e2e:
+        print(json.dumps({"press_e2e": press_e2e(dev, T, args.target, args.e2e_tokens)}))
+        return 0
 
     if args.read_ceiling:
         # what can ONE launch of a given size reach?  buffers rotate through 2 GiB so every launch reads HBM
