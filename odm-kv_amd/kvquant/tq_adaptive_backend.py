@@ -115,9 +115,27 @@ class TurboQuantAdaptiveKVCacheState:
         self._counts = None           # np.int64 [5, nseg]   tokens stored per level and segment
         self._seg_tile = None         # np.int64 [5, nseg+1] first tile of each segment
         self._bufs = None
-        self._level_map = None        # uint8 [B, H, seq_len]: bit level of every position
+        self._level_store = None      # uint8 [B, H, capacity]: bit level of every position (grown by doubling)
+        self._masked = None           # cached (indices of evicted positions,) or None when stale
         self._items = None
         self._packed = None
+
+    @property
+    def _level_map(self):
+        """uint8 [B, H, seq_len]: bit level of every position (a view of the growing store)."""
+        return None if self._level_store is None else self._level_store[:, :, :self.seq_len]
+
+    def _extend_levels(self, lm: torch.Tensor) -> None:
+        """Write the levels of T new positions behind the current ones (before seq_len is advanced)."""
+        B, H, T = lm.shape
+        need = self.seq_len + T
+        if self._level_store is None or self._level_store.shape[2] < need:
+            cap = max(need, 2 * (0 if self._level_store is None else self._level_store.shape[2]), 256)
+            grown = torch.empty(B, H, cap, dtype=torch.uint8, device=self.device)
+            if self._level_store is not None and self.seq_len:
+                grown[:, :, :self.seq_len] = self._level_store[:, :, :self.seq_len]
+            self._level_store = grown
+        self._level_store[:, :, self.seq_len:need] = lm
 
     def _alloc(self, seg_tile: np.ndarray) -> "_Buffers":
         """All buffers of the store as views into one allocation: the segment tables (one upload),
@@ -301,10 +319,11 @@ class TurboQuantAdaptiveKVCacheState:
         self._counts = new_counts
         lm = bits.to(torch.uint8)
         if _pos_offset is None:
-            self._level_map = lm if self._level_map is None else torch.cat([self._level_map, lm], dim=2)
+            self._extend_levels(lm)
             self.seq_len += T
         else:
-            self._level_map[:, :, pos_offset:pos_offset + T] = lm
+            self._level_store[:, :, pos_offset:pos_offset + T] = lm
+        self._masked = None
         self._items = None
 
     def append_all_exact(self, keys: torch.Tensor, values: torch.Tensor) -> None:
@@ -326,8 +345,11 @@ class TurboQuantAdaptiveKVCacheState:
         _lib.check(lib.odmkv_append_exact(C.byref(self._packed), k.data_ptr(), v.data_ptr(), self.seq_len,
                                           _lib.stream_ptr(self.device)))
         self._counts = new_counts
-        fresh = torch.full((B, H, 1), 16, dtype=torch.uint8, device=self.device)
-        self._level_map = torch.cat([self._level_map, fresh], dim=2)
+        need = self.seq_len + 1
+        if self._level_store.shape[2] < need:
+            self._extend_levels(torch.full((B, H, 1), 16, dtype=torch.uint8, device=self.device))
+        else:
+            self._level_store[:, :, self.seq_len:need].fill_(16)       # an exact token: the evicted set does not change
         self.seq_len += 1
         if had is not self._seg_tile:
             self._items = None
@@ -337,7 +359,7 @@ class TurboQuantAdaptiveKVCacheState:
         if seq_len >= self.seq_len:
             return
         self.seq_len = seq_len
-        self._level_map = self._level_map[:, :, :seq_len].contiguous()
+        self._masked = None
         # positions ascend inside a segment, so the survivors are a prefix of it
         for li in range(5):
             if self._counts[li].sum() == 0:
@@ -376,12 +398,14 @@ class TurboQuantAdaptiveKVCacheState:
         self._dequant_into(keys, values, False)
 
     def masked_key_indices(self):
-        if self._level_map is None:
+        """Indices (b, h, t) of the evicted positions, or None when there are none.  The answer is
+        kept until positions are stored with levels again (exact appends cannot evict)."""
+        if self._level_store is None:
             return None
-        idx = (self._level_map == 0).nonzero(as_tuple=True)
-        if idx[0].numel() == 0:
-            return None
-        return idx
+        if self._masked is None:
+            idx = (self._level_map == 0).nonzero(as_tuple=True)
+            self._masked = (idx if idx[0].numel() else None,)
+        return self._masked[0]
 
     def visible_mask(self) -> torch.Tensor:
         return self._level_map != 0
