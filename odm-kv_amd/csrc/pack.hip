@@ -901,69 +901,116 @@ struct DequantArgs {
     const float* vnorm;
 };
 
+// x_hat[token][j] = |x| * sum_i c[code_i] * Pi[i][j] on the fp32 matrix cores, like the rotation of the
+// quantiser: operand A = the centroid of the token's code i (lane = token), operand B = row i of Pi
+// from LDS (four outputs per lane), 128 steps of K = 1.  Persistent workgroups of DQ_NW waves keep Pi in
+// LDS (even workgroups keys, odd ones values) and walk the level's tiles, a wave per tile.  A lane
+// ends up with outputs 4c..4c+3 of 32 tokens: 8 (16) bytes of a row per store, the 32 lanes of a half
+// wave covering the row.
+#define DQ_NW 8
+#define DQ_GROUP 16                       // centroid lookups are done in blocks, ahead of their matrix instructions
 template <int W, int DT>
-__global__ __launch_bounds__(64) void dequant_kernel(DequantArgs a) {
-    __shared__ __align__(16) uint8_t codes[TILE * CODE_ROW];
-    __shared__ float cb[1 << W];
-    const int lane = threadIdx.x, tile = blockIdx.x;
-    const bool is_v = blockIdx.y != 0;
-    const int bh = find_segment(a.seg_tile, a.nseg, tile);
-    const int ts = (tile - a.seg_tile[bh]) * TILE;
-    const int hi = min(a.seg_count[bh] - ts, TILE);
-    if (hi <= 0) return;
-    for (int i = lane; i < (1 << W); i += WAVE) cb[i] = a.cb[i];
-    const size_t slot = (size_t)tile * TILE + lane;
-    const bool valid = lane < hi;
-
-    float y[HD];
-    if (!is_v) {
-        uint32_t words[4 * W];
-        const uint8_t* src = a.kcodes + (size_t)tile * (TILE * 16 * W);
-#pragma unroll
-        for (int c = 0; c < W; ++c) {
-            const uint4 v = *reinterpret_cast<const uint4*>(src + ((size_t)c * TILE + lane) * 16);
-            words[4 * c] = v.x; words[4 * c + 1] = v.y; words[4 * c + 2] = v.z; words[4 * c + 3] = v.w;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < HD; ++i) y[i] = cb[get_code<W>(words, i)];
-    } else {
-        const uint8_t* src = a.vcodes + (size_t)tile * (HD * 8 * W);
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int j = lane + 64 * half;
-            uint32_t words[2 * W];
-#pragma unroll
-            for (int k = 0; k < 2 * W; ++k) words[k] = *reinterpret_cast<const uint32_t*>(src + v_word_offset<W>(k, j));
-#pragma unroll
-            for (int t = 0; t < TILE; ++t) codes[t * CODE_ROW + j] = (uint8_t)get_code<W>(words, t);
-        }
-        __syncthreads();
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            const uint4 v = *reinterpret_cast<const uint4*>(&codes[lane * CODE_ROW + 16 * c]);
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int e = 0; e < 16; ++e) y[16 * c + e] = cb[(w[e >> 2] >> (8 * (e & 3))) & 0xffu];
-        }
+__global__ __launch_bounds__(DQ_NW * 64) void dequant_kernel(DequantArgs a, int n_tiles) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    float* pis = reinterpret_cast<float*>(smem);                                  // Pi [i][j], as stored
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint8_t* codes = smem + QP_PI_BYTES + wave * QP_STAGE;                         // this wave's [token][dim] codes (values)
+    float* cb = reinterpret_cast<float*>(smem + QP_PI_BYTES + DQ_NW * QP_STAGE);   // [256] centroids
+    float* norms = cb + 256 + wave * TILE;                                         // [DQ_NW][64] norm of the wave's tokens
+    long long* offs = reinterpret_cast<long long*>(cb + 256 + DQ_NW * TILE) + wave * TILE;   // element offset of the row, -1: none
+    const bool is_v = (blockIdx.x & 1) != 0;
+    {
+        const float4* __restrict__ src = reinterpret_cast<const float4*>(is_v ? a.pi_v : a.pi_k);
+        for (int i = tid; i < HD * HD / 4; i += DQ_NW * 64) reinterpret_cast<float4*>(pis)[i] = src[i];
+        for (int i = tid; i < (1 << W); i += DQ_NW * 64) cb[i] = a.cb[i];
     }
-    const float norm = valid ? (is_v ? a.vnorm[slot] : a.knorm[slot]) : 0.0f;
-    const int t = valid ? a.pos[slot] : -1;
-    const bool write = valid && t >= 0 && t < a.T;
-    const size_t off = write ? (size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH + (size_t)t * a.sT : 0;
+    __syncthreads();
     void* out = is_v ? a.V : a.K;
-    const float* __restrict__ pi = is_v ? a.pi_v : a.pi_k;
-#pragma unroll 1
-    for (int j0 = 0; j0 < HD; j0 += 8) {
-        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int i = 0; i < HD; ++i) {
-#pragma unroll
-            for (int b = 0; b < 8; ++b) acc[b] = __fmaf_rn(y[i], pi[i * HD + j0 + b], acc[b]);
+    const int wg = blockIdx.x >> 1, n_wg = gridDim.x >> 1;
+    const float4* __restrict__ brow = reinterpret_cast<const float4*>(pis) + (lane & 31);
+    for (int tile = wg * DQ_NW + wave; tile < n_tiles; tile += n_wg * DQ_NW) {
+        const int bh = find_segment(a.seg_tile, a.nseg, tile);
+        const int ts = (tile - a.seg_tile[bh]) * TILE;
+        const int hi = min(a.seg_count[bh] - ts, TILE);
+        if (hi <= 0) continue;                                       // wave-uniform
+        const size_t slot = (size_t)tile * TILE + lane;
+        const bool valid = lane < hi;
+        {
+            const int t = valid ? a.pos[slot] : -1;
+            const bool write = valid && t >= 0 && t < a.T;
+            offs[lane] = write ? (long long)((size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH + (size_t)t * a.sT) : -1ll;
+            norms[lane] = valid ? (is_v ? a.vnorm[slot] : a.knorm[slot]) : 0.0f;
         }
+        uint32_t words[4 * W];                                       // keys: the token's code words
+        if (!is_v) {
+            const uint8_t* src = a.kcodes + (size_t)tile * (TILE * 16 * W);
 #pragma unroll
-        for (int b = 0; b < 8; ++b) acc[b] = acc[b] * norm;
-        if (write) store8<DT>(out, off + j0, acc);
+            for (int c = 0; c < W; ++c) {
+                const uint4 v = *reinterpret_cast<const uint4*>(src + ((size_t)c * TILE + lane) * 16);
+                words[4 * c] = v.x; words[4 * c + 1] = v.y; words[4 * c + 2] = v.z; words[4 * c + 3] = v.w;
+            }
+        } else {                                                     // values are stored dim-major: transpose through LDS
+            const uint8_t* src = a.vcodes + (size_t)tile * (HD * 8 * W);
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int j = lane + 64 * half;
+                uint32_t vw[2 * W];
+#pragma unroll
+                for (int k = 0; k < 2 * W; ++k) vw[k] = *reinterpret_cast<const uint32_t*>(src + v_word_offset<W>(k, j));
+#pragma unroll
+                for (int t = 0; t < TILE; ++t) codes[t * CODE_ROW + j] = (uint8_t)get_code<W>(vw, t);
+            }
+        }
+        wave_lds_fence();
+        f32x32 acc0, acc1, acc2, acc3;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; acc2[i] = 0.0f; acc3[i] = 0.0f; }
+        float4 b = brow[0];
+#pragma unroll
+        for (int i0 = 0; i0 < HD; i0 += DQ_GROUP) {
+            float y[DQ_GROUP];
+            if (!is_v) {
+#pragma unroll
+                for (int g = 0; g < DQ_GROUP; ++g) y[g] = cb[get_code<W>(words, i0 + g)];
+            } else {
+                const uint4 v = *reinterpret_cast<const uint4*>(&codes[lane * CODE_ROW + i0]);
+                const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int g = 0; g < DQ_GROUP; ++g) y[g] = cb[(w4[g >> 2] >> (8 * (g & 3))) & 0xffu];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < DQ_GROUP; ++g) {
+                const int in = i0 + g + 1 < HD ? i0 + g + 1 : i0 + g;
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(y[g], b.x, acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(y[g], b.y, acc1, 0, 0, 0);
+                acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(y[g], b.z, acc2, 0, 0, 0);
+                acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(y[g], b.w, acc3, 0, 0, 0);
+                b = brow[in * (HD / 4)];
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        int ln = lane;
+        asm volatile("" : "+v"(ln));                                 // keeps the store addresses out of the loop above
+        const int c4 = (ln & 31) * 4;
+#pragma unroll
+        for (int vv = 0; vv < 32; ++vv) {
+            const int token = mfma_token(vv, ln);
+            const long long off = offs[token];
+            const float n = norms[token];
+            if (off >= 0) {
+                const float r[4] = {acc0[vv] * n, acc1[vv] * n, acc2[vv] * n, acc3[vv] * n};
+                if constexpr (DT == ODMKV_F32) {
+                    *reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + off + c4) = make_float4(r[0], r[1], r[2], r[3]);
+                } else {
+                    const uint32_t lo = (uint32_t)Elem<DT>::from_f32(r[0]) | ((uint32_t)Elem<DT>::from_f32(r[1]) << 16);
+                    const uint32_t hi2 = (uint32_t)Elem<DT>::from_f32(r[2]) | ((uint32_t)Elem<DT>::from_f32(r[3]) << 16);
+                    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(out) + off + c4) = make_uint2(lo, hi2);
+                }
+            }
+        }
+        wave_lds_fence();                                            // offs / norms / codes free for the next tile
     }
 }
 
@@ -992,17 +1039,37 @@ __global__ __launch_bounds__(64) void exact_scatter_kernel(odmkv_packed_t s, voi
     }
 }
 
-template <int DT>
-static int launch_dequant(const DequantArgs& da, int li, int n_tiles, hipStream_t st) {
-    dim3 grid(n_tiles, 2), block(64);
-    switch (li) {
-        case 0: hipLaunchKernelGGL((dequant_kernel<2, DT>), grid, block, 0, st, da); break;
-        case 1: hipLaunchKernelGGL((dequant_kernel<3, DT>), grid, block, 0, st, da); break;
-        case 2: hipLaunchKernelGGL((dequant_kernel<4, DT>), grid, block, 0, st, da); break;
-        default: hipLaunchKernelGGL((dequant_kernel<8, DT>), grid, block, 0, st, da); break;
+template <int W, int DT>
+static int launch_dequant_w(const DequantArgs& da, int n_tiles, hipStream_t st) {
+    const size_t lds = QP_PI_BYTES + (size_t)DQ_NW * QP_STAGE + 256 * sizeof(float) + DQ_NW * TILE * (sizeof(float) + sizeof(long long));
+    static bool attr_set = false;
+    if (!attr_set) {
+        ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(dequant_kernel<W, DT>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
     }
+    int dev = 0, cus = 256;
+    ODMKV_CHECK_HIP(hipGetDevice(&dev));
+    ODMKV_CHECK_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    // one persistent workgroup per compute unit, keys on the even and values on the odd ones; never
+    // more workgroups than there are tiles for their waves
+    int pairs = cus / 2;
+    const int need = (n_tiles + DQ_NW - 1) / DQ_NW;
+    if (pairs > need) pairs = need;
+    if (pairs < 1) pairs = 1;
+    hipLaunchKernelGGL((dequant_kernel<W, DT>), dim3(2 * pairs), dim3(DQ_NW * 64), lds, st, da, n_tiles);
     ODMKV_CHECK_LAUNCH("dequant_kernel");
     return 0;
+}
+
+template <int DT>
+static int launch_dequant(const DequantArgs& da, int li, int n_tiles, hipStream_t st) {
+    switch (li) {
+        case 0: return launch_dequant_w<2, DT>(da, n_tiles, st);
+        case 1: return launch_dequant_w<3, DT>(da, n_tiles, st);
+        case 2: return launch_dequant_w<4, DT>(da, n_tiles, st);
+        default: return launch_dequant_w<8, DT>(da, n_tiles, st);
+    }
 }
 
 extern "C" int odmkv_dequant(const odmkv_packed_t* store, void* K, void* V, int dtype, int T,
