@@ -62,7 +62,8 @@ struct DecodeArgs {
     uint4* qs;        // [B*Hq, 32] the same for q16 itself (low halves are zero)
     float inv_s[4];   // 1 / table scale per width
     float cbs[28];    // scaled centroids of widths 2, 3, 4 (kept in scalar registers; 8-bit ones stay in memory)
-    float* partial;   // [n_items, GP, PSTRIDE]
+    int gp;           // head slots per item in `partial`: 4 or 8
+    float* partial;   // [n_items, gp, PSTRIDE]
     float* out;
     float* lse;
 };
@@ -365,8 +366,8 @@ __device__ static inline void compute_tile(const TileData<W>& t, int nvalid, int
 
 // stage the group's queries (fp16 high/low halves per 4-dim step) in LDS; heads beyond the group are 0
 template <int NP>
-__device__ static inline uint4 load_query_slice(const DecodeArgs& a, const uint4* src, int tid) {
-    return (tid < 4 * NP * 32 && (tid >> 5) < a.G) ? src[tid] : make_uint4(0u, 0u, 0u, 0u);
+__device__ static inline uint4 load_query_slice(const DecodeArgs& a, const uint4* src, int tid, int nheads) {
+    return (tid < 4 * NP * 32 && (tid >> 5) < nheads) ? src[tid] : make_uint4(0u, 0u, 0u, 0u);
 }
 template <int NP>
 __device__ static inline void stage_queries(uint4 v, uint4* qsh, int tid) {
@@ -386,7 +387,7 @@ __device__ static inline void fetch_queries(const uint4* qsh, int lane, h4* qr, 
 
 // One work item of a quantised level.
 template <int W, int NP>
-__device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq0, int tile0, int ntiles, int ntok,
+__device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq0, int nheads, int tile0, int ntiles, int ntok,
                                               int tid, uint8_t* lut, uint4* qsh, WaveState<NP>& st) {
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
@@ -395,7 +396,7 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     // wavefront's tile requests its LDS traffic would wait for the memory pipeline to accept them
     // (every wavefront of the chip asks for its tiles at the same moment).  Loads return in issue
     // order: the (small) query slice goes first so that staging it does not have to wait for the tile.
-    const uint4 qslice = load_query_slice<NP>(a, a.qrot + (size_t)bq0 * 32, tid);   // one request: lands while the table is built
+    const uint4 qslice = load_query_slice<NP>(a, a.qrot + (size_t)bq0 * 32, tid, nheads);   // one request: lands while the table is built
     build_lut<W>(lut, a, tid);
     TileData<W> cur;
     int tt = wave;
@@ -514,12 +515,12 @@ __device__ static inline void compute_exact_tile(const ExactTile& t, bool bf, in
 // Exact (16-bit) tokens: the query is the fp16-rounded one itself (its low halves are zero), so only
 // the high halves are fetched.  The first tile's loads are issued before anything is waited for.
 template <int NP>
-__device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int bq0, int tile0, int ntiles, int seg_first,
+__device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int bq0, int nheads, int tile0, int ntiles, int seg_first,
                                               int tid, uint4* qsh, WaveState<NP>& st) {
     const int wave = tid >> 6, lane = tid & 63;
     const bool bf = a.s.exact_dtype == ODMKV_BF16;
     const float esc = a.scaling * LOG2E;
-    const uint4 qslice = load_query_slice<NP>(a, a.qs + (size_t)bq0 * 32, tid);
+    const uint4 qslice = load_query_slice<NP>(a, a.qs + (size_t)bq0 * 32, tid, nheads);
     const int count = a.s.seg_count[4][bh];          // exact segments grow between work-list rebuilds
     ExactTile cur;
     int tt = wave;
@@ -544,20 +545,24 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
 }
 
 // ------------------------------------------------------------------------------------------------
-// main kernel: NP passes of four query heads (GQA groups up to 4 * NP)
+// main kernel: four query heads per workgroup (NP = 1); larger GQA groups take one workgroup pass per four heads
 // ------------------------------------------------------------------------------------------------
-template <int NP>
+template <int NP, bool MULTI>
 __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs a) {
     __shared__ __align__(16) uint8_t lut[LUT_BYTES];     // centroid table; reused to combine the wavefronts
     __shared__ float wm[NWAVES][4 * NP], wl[NWAVES][4 * NP];
     __shared__ uint4 qsh[4 * NP * 32];
 
-    const int item = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    // A GQA group of more than four query heads is served four heads at a time by separate workgroups
+    // of the same item (the item's codes are read once per pass; the second read mostly hits the caches).
+    const int item = blockIdx.x, pass = MULTI ? (int)blockIdx.y : 0;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     TRACE(0)
     const int4 d0 = reinterpret_cast<const int4*>(a.items)[2 * item];       // bh, level, first tile, tiles
     const int4 d1 = reinterpret_cast<const int4*>(a.items)[2 * item + 1];   // tokens, first tile of the segment
     const int bh = d0.x, li = d0.y, tile0 = d0.z, ntiles = d0.w;
-    const int bq0 = (bh / a.s.Hkv) * a.Hq + (bh % a.s.Hkv) * a.G;            // first query head of the group
+    const int bq0 = (bh / a.s.Hkv) * a.Hq + (bh % a.s.Hkv) * a.G + 4 * NP * pass;   // first query head of this pass
+    const int nheads = MULTI ? min(a.G - 4 * NP * pass, 4 * NP) : a.G;
 
     WaveState<NP> st;
 #pragma unroll
@@ -566,11 +571,11 @@ __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs 
         st.acc[p][0] = (f4){0.f, 0.f, 0.f, 0.f}; st.acc[p][1] = (f4){0.f, 0.f, 0.f, 0.f};
     }
     switch (li) {
-        case 0: run_quant_level<2, NP>(a, 0, bq0, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
-        case 1: run_quant_level<3, NP>(a, 1, bq0, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
-        case 2: run_quant_level<4, NP>(a, 2, bq0, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
-        case 3: run_quant_level<8, NP>(a, 3, bq0, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
-        default: run_exact_level<NP>(a, bh, bq0, tile0, ntiles, d1.y, tid, qsh, st); break;
+        case 0: run_quant_level<2, NP>(a, 0, bq0, nheads, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        case 1: run_quant_level<3, NP>(a, 1, bq0, nheads, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        case 2: run_quant_level<4, NP>(a, 2, bq0, nheads, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        case 3: run_quant_level<8, NP>(a, 3, bq0, nheads, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        default: run_exact_level<NP>(a, bh, bq0, nheads, tile0, ntiles, d1.y, tid, qsh, st); break;
     }
 
     // ---- combine the four wavefronts (the table is no longer needed) ----
@@ -590,7 +595,7 @@ __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs 
         }
     }
     __syncthreads();
-    float* dst = a.partial + (size_t)item * GP * PSTRIDE;
+    float* dst = a.partial + (MULTI ? ((size_t)item * a.gp + GP * pass) : (size_t)item * GP) * PSTRIDE;
     for (int e = tid; e < GP * HD; e += NWAVES * 64) {
         const int g = e / HD, j = e % HD;
         float M = wm[0][g];
@@ -831,14 +836,15 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
         ODMKV_CHECK_LAUNCH("decode_prep_kernel");
     }
     const int GP = group_pad(G);
+    a.gp = GP;
     if (n_items > 0 && (g_stage_mask & 2)) {
         const bool rec = g_prof_on && (size_t)(2 * g_prof_used + 1) < g_prof_events.size();
         // when measuring, the events are attached to the dispatch itself: they carry the kernel's own
         // start and end timestamps, not those of separate marker packets
         hipEvent_t e0 = rec ? g_prof_events[2 * g_prof_used] : nullptr;
         hipEvent_t e1 = rec ? g_prof_events[2 * g_prof_used + 1] : nullptr;
-        if (GP == 4) hipExtLaunchKernelGGL((decode_main_kernel<1>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
-        else hipExtLaunchKernelGGL((decode_main_kernel<2>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
+        if (GP == 4) hipExtLaunchKernelGGL((decode_main_kernel<1, false>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
+        else hipExtLaunchKernelGGL((decode_main_kernel<1, true>), dim3(n_items, GP / 4), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
         ODMKV_CHECK_LAUNCH("decode_main_kernel");
         if (rec) ++g_prof_used;
     }
