@@ -119,6 +119,36 @@ def test_work_list_respects_the_per_segment_item_limit():
     assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
 
 
+def test_decode_replayed_from_a_graph_matches_eager():
+    """The three launches of a decode call captured in a HIP graph and replayed with new queries in the
+    captured buffer, with eager work and synchronisations between the replays: every replay must give
+    what an eager call gives for the same query."""
+    g = torch.Generator().manual_seed(21)
+    k = torch.randn(1, 4, 900, 128, generator=g).half(); v = torch.randn(1, 4, 900, 128, generator=g).half()
+    bits = _rand_bits(g, (1, 4, 900), (0.2, 0.5, 0.1, 0.1, 0.05, 0.05)); bits[..., -16:] = 16
+    st, ref = _pair(k, v, bits)
+    q_static = torch.randn(1, 16, 128, generator=g).half().float().to(DEV)
+    st.decode_attention(q_static)                       # builds the work list and the workspaces outside the capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        st.decode_attention(q_static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static = st.decode_attention(q_static)
+    for rep in range(4):
+        q = torch.randn(1, 16, 128, generator=g).half().float()
+        eager = st.decode_attention(q.to(DEV)).clone()  # eager work between the replays
+        torch.cuda.synchronize()
+        q_static.copy_(q.to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, eager), f"replay {rep}"
+        assert rel_err(out_static.cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
+
+
 def test_decode_after_appends_and_flush():
     g = torch.Generator().manual_seed(8)
     B, H, G = 1, 4, 4
