@@ -184,6 +184,9 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  * so that tokens appended since the list was built are seen.  item_range: device int32
  * [B*Hkv + 1] first item of each bh; a bh may have at most ODMKV_MAX_ITEMS_PER_SEGMENT items (the
  * caller builds the list and keeps to it; one item per compute unit is what performs best).
+ * dispatch_order: device int32 [n_items], a permutation of the items in the order the workgroups
+ * should take them (longest first, when there are more items than compute units), or NULL for the
+ * list's own order.
  * out: device fp32 [B, Hq, 128]; lse: device fp32 [B, Hq] or NULL (log-sum-exp of the scaled logits).
  * pi_k_t is the key rotation TRANSPOSED (row-major [128,128] of Pi_k^T), pi_v the value rotation as is.
  * The query is rounded to fp16 on entry (the attention being replaced receives it in the model's
@@ -198,6 +201,7 @@ size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);
 int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
                       const odmkv_packed_t* store,
                       const int32_t* items, int n_items, const int32_t* item_range,
+                      const int32_t* dispatch_order,
                       const float* pi_k_t, const float* pi_v, const float* codebooks,
                       const float* codebooks_host, const float* inv_scales,
                       float* out, float* lse, void* workspace, size_t workspace_bytes,

@@ -55,6 +55,7 @@ struct DecodeArgs {
     float scaling;
     const int32_t* items;
     const int32_t* item_range;
+    const int32_t* order;      // order[k] = item that workgroup k takes (long items first), or null: item k
     const float* pi_k_t;   // Pi_k transposed
     const float* pi_v;
     const float* cb;
@@ -547,7 +548,7 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
 // ------------------------------------------------------------------------------------------------
 // main kernel: four query heads per workgroup (NP = 1); larger GQA groups take one workgroup pass per four heads
 // ------------------------------------------------------------------------------------------------
-template <int NP, bool MULTI>
+template <int NP, bool MULTI, bool ORDERED>
 __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs a) {
     __shared__ __align__(16) uint8_t lut[LUT_BYTES];     // centroid table; reused to combine the wavefronts
     __shared__ float wm[NWAVES][4 * NP], wl[NWAVES][4 * NP];
@@ -555,7 +556,7 @@ __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs 
 
     // A GQA group of more than four query heads is served four heads at a time by separate workgroups
     // of the same item (the item's codes are read once per pass; the second read mostly hits the caches).
-    const int item = blockIdx.x, pass = MULTI ? (int)blockIdx.y : 0;
+    const int item = ORDERED ? a.order[blockIdx.x] : (int)blockIdx.x, pass = MULTI ? (int)blockIdx.y : 0;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     TRACE(0)
     const int4 d0 = reinterpret_cast<const int4*>(a.items)[2 * item];       // bh, level, first tile, tiles
@@ -803,6 +804,7 @@ extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
 extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
                                  const odmkv_packed_t* store,
                                  const int32_t* items, int n_items, const int32_t* item_range,
+                                 const int32_t* dispatch_order,
                                  const float* pi_k_t, const float* pi_v, const float* codebooks,
                                  const float* codebooks_host, const float* inv_scales,
                                  float* out, float* lse, void* workspace, size_t workspace_bytes,
@@ -822,7 +824,7 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     hipStream_t st = (hipStream_t)stream;
     DecodeArgs a;
     a.s = *store; a.q = q; a.Hq = Hq; a.G = G; a.B = B; a.scaling = scaling;
-    a.items = items; a.item_range = item_range;
+    a.items = items; a.item_range = item_range; a.order = dispatch_order;
     a.pi_k_t = pi_k_t; a.pi_v = pi_v; a.cb = codebooks;
     for (int w = 0; w < 4; ++w) a.inv_s[w] = inv_scales[w];
     for (int k = 0; k < 28; ++k) a.cbs[k] = codebooks_host[k];
@@ -843,8 +845,11 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
         // start and end timestamps, not those of separate marker packets
         hipEvent_t e0 = rec ? g_prof_events[2 * g_prof_used] : nullptr;
         hipEvent_t e1 = rec ? g_prof_events[2 * g_prof_used + 1] : nullptr;
-        if (GP == 4) hipExtLaunchKernelGGL((decode_main_kernel<1, false>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
-        else hipExtLaunchKernelGGL((decode_main_kernel<1, true>), dim3(n_items, GP / 4), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
+        // (the plain case keeps its own instantiation: a branch on either option at the kernel's start costs it 0.25 us)
+        if (GP == 4 && !a.order) hipExtLaunchKernelGGL((decode_main_kernel<1, false, false>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
+        else if (GP == 4) hipExtLaunchKernelGGL((decode_main_kernel<1, false, true>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
+        else if (!a.order) hipExtLaunchKernelGGL((decode_main_kernel<1, true, false>), dim3(n_items, GP / 4), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
+        else hipExtLaunchKernelGGL((decode_main_kernel<1, true, true>), dim3(n_items, GP / 4), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
         ODMKV_CHECK_LAUNCH("decode_main_kernel");
         if (rec) ++g_prof_used;
     }

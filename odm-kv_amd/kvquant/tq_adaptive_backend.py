@@ -118,6 +118,7 @@ class TurboQuantAdaptiveKVCacheState:
         self._level_store = None      # uint8 [B, H, capacity]: bit level of every position (grown by doubling)
         self._masked = None           # cached (indices of evicted positions,) or None when stale
         self._items = None
+        self._item_order = None
         self._packed = None
 
     @property
@@ -478,49 +479,87 @@ class TurboQuantAdaptiveKVCacheState:
 
     # ------------------------------------------------------------------ fused attention
     def _build_items(self, target_items: Optional[int] = None, min_item_bytes: Optional[int] = None) -> None:
+        """The decode work list: every (segment, level) run of tiles cut into items of about equal
+        bytes, one workgroup (one compute unit, eight wavefronts) per item.
+
+        With a target the cut is the coarsest one that does not exceed it.  Without one, a few cuts
+        are compared by the time a longest-first assignment of their items to the compute units
+        would take (a small cost model of the kernel: fixed set-up plus a round of eight tiles at a
+        time), and the best is kept; when it has more items than compute units, the order in which
+        the workgroups take the items (longest first) is handed to the kernel as well."""
         import os
-        if target_items is None:
-            # one workgroup per item, one (eight-wavefront) workgroup per compute unit: all resident at once
-            target_items = int(os.environ.get("ODMKV_DECODE_ITEMS", 0)) or \
-                torch.cuda.get_device_properties(self.device).multi_processor_count
+        n_cu = torch.cuda.get_device_properties(self.device).multi_processor_count
+        env_target = int(os.environ.get("ODMKV_DECODE_ITEMS", 0))
         min_item_bytes = int(os.environ.get("ODMKV_DECODE_MIN_ITEM_BYTES", 16384)) if min_item_bytes is None else min_item_bytes
         used = (self._counts + TILE - 1) // TILE
         used[4] = np.diff(self._seg_tile[4])              # exact segments grow between rebuilds
         total = sum(int(used[li].sum()) * _TILE_BYTES[li] for li in range(5))
-        # the largest number of items that does not exceed the target: every (segment, level) run of
-        # tiles is cut into pieces of about per_item bytes, and a run's last piece may be short, so
-        # per_item grows until the pieces fit (one workgroup per item, all resident at once)
-        runs = [int(used[li, s]) * _TILE_BYTES[li] for s in range(self._nseg) for li in range(5) if used[li, s] > 0]
-        tile_b = [_TILE_BYTES[li] for s in range(self._nseg) for li in range(5) if used[li, s] > 0]
+        runs = [(s, li, int(used[li, s])) for s in range(self._nseg) for li in range(5) if used[li, s] > 0]
+
+        def step_of(per_item: int, li: int) -> int:
+            return max(1, int(round(per_item / _TILE_BYTES[li])))
 
         def n_pieces(per_item: int) -> int:
-            return sum(-(-(r // b) // max(1, int(round(per_item / b)))) for r, b in zip(runs, tile_b))
+            return sum(-(-nt // step_of(per_item, li)) for _, li, nt in runs)
 
         def most_per_segment(per_item: int) -> int:
-            return max(sum(-(-int(used[li, s]) // max(1, int(round(per_item / _TILE_BYTES[li])))) for li in range(5))
-                       for s in range(self._nseg))
+            per = np.zeros(self._nseg, np.int64)
+            for s, li, nt in runs:
+                per[s] += -(-nt // step_of(per_item, li))
+            return int(per.max()) if len(runs) else 0
 
-        per_item = max(total // max(target_items, 1), min_item_bytes)
-        # (the merge kernel takes at most _MAX_ITEMS_PER_SEGMENT items of one (sequence, kv-head))
-        while (n_pieces(per_item) > target_items or most_per_segment(per_item) > _MAX_ITEMS_PER_SEGMENT) and per_item < total:
-            per_item += max(per_item // 64, 1)
-        items, ranges = [], [0]
-        for s in range(self._nseg):
-            for li in range(5):
-                nt = int(used[li, s])
-                if nt == 0:
-                    continue
-                step = max(1, int(round(per_item / _TILE_BYTES[li])))
-                t0 = int(self._seg_tile[li, s])
-                cnt = int(self._counts[li, s])
-                for a in range(0, nt, step):
+        def fit(target: int) -> int:
+            # the coarsest cut with at most `target` items (a run's last piece may be short) and no
+            # segment above the merge kernel's limit
+            per_item = max(total // max(target, 1), min_item_bytes)
+            while (n_pieces(per_item) > target or most_per_segment(per_item) > _MAX_ITEMS_PER_SEGMENT) and per_item < total:
+                per_item += max(per_item // 64, 1)
+            return per_item
+
+        def cut(per_item: int):
+            items = []
+            for s, li, nt in runs:
+                step = step_of(per_item, li)
+                t0, cnt = int(self._seg_tile[li, s]), int(self._counts[li, s])
+                for a0 in range(0, nt, step):
+                    n = min(step, nt - a0)
                     # (segment, level, first tile, tiles, tokens in those tiles, segment's first tile, -, -)
-                    n = min(step, nt - a)
-                    items.append((s, li, t0 + a, n, min(cnt - a * TILE, n * TILE), t0, 0, 0))
-            ranges.append(len(items))
+                    items.append((s, li, t0 + a0, n, min(cnt - a0 * TILE, n * TILE), t0, 0, 0))
+            return items
+
+        def cost(item) -> float:                     # microseconds of one workgroup, roughly
+            rounds = -(-item[3] // 8)
+            return (3.0 + 1.0 * rounds) if item[1] == 4 else (3.5 + 1.5 * rounds)
+
+        def makespan(items) -> float:
+            import heapq
+            free = [0.0] * n_cu
+            for c in sorted((cost(it) for it in items), reverse=True):
+                heapq.heappush(free, heapq.heappop(free) + c)
+            return max(free)
+
+        explicit = target_items if target_items is not None else (env_target or None)
+        if explicit is not None:
+            items = cut(fit(int(explicit)))
+        else:
+            best = None
+            for mult in (1.0, 1.5, 2.0, 3.0, 4.0):
+                cand = cut(fit(int(n_cu * mult)))
+                t = makespan(cand)
+                if best is None or t < best[0] - 1e-9:
+                    best = (t, cand)
+            items = best[1]
+        ranges = [0]
+        for s in range(self._nseg):
+            ranges.append(ranges[-1] + sum(1 for it in items if it[0] == s))
         arr = np.asarray(items, np.int32).reshape(-1, 8)
+        order = None
+        if len(items) > n_cu:
+            order = np.argsort(-np.asarray([cost(it) for it in items]), kind="stable").astype(np.int32)
+            order = torch.from_numpy(order).to(self.device)
         self._items = (torch.from_numpy(arr).to(self.device),
                        torch.from_numpy(np.asarray(ranges, np.int32)).to(self.device), len(items))
+        self._item_order = order
 
     def decode_attention(self, query: torch.Tensor, scaling: Optional[float] = None,
                          return_lse: bool = False):
@@ -544,6 +583,6 @@ class TurboQuantAdaptiveKVCacheState:
         ws = _lib.workspace(self.device, ws_bytes, "decode")
         _lib.check(lib.odmkv_decode_attn(
             q.data_ptr(), B, Hq, scale, C.byref(self._packed), items.data_ptr(), n_items,
-            ranges.data_ptr(), self._pi_k_t.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
+            ranges.data_ptr(), _lib.ptr(self._item_order), self._pi_k_t.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
             self._decode_cb_host, self._decode_inv, out.data_ptr(), _lib.ptr(lse), ws.data_ptr(), ws_bytes, _lib.stream_ptr(self.device)))
         return (out, lse) if return_lse else out

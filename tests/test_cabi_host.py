@@ -60,7 +60,7 @@ def test_argument_checks_without_a_gpu(lib):
     rc = lib.odmkv_quantize_rows(p, 0, C.c_int64(4), C.c_int64(128), 5, p, p, p, p, None)
     assert rc == -1 and b"width" in lib.odmkv_last_error()
     rc = lib.odmkv_decode_attn(None, 1, 8, C.c_float(1.0), None, None, 0, None, None, None, None, None, None, None,
-                               C.c_size_t(0), None)
+                               None, None, None, C.c_size_t(0), None)
     assert rc == -1
 
 
