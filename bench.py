@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers 32] [--ctx 32768]
 
-Workload (BASELINE.json config 2, kernel-only form): 32 independent Llama-3-8B-shaped layers
+Workload (the second benchmark configuration, kernel-only form): 32 independent Llama-3-8B-shaped layers
 (Hq 32, Hkv 8, d 128), 32k-token context each, K/V ~ N(0,1) with 8x sink tokens, compressed at a
 2.0 average-bit budget (score -> allocate -> window override -> quantise + pack), then decoded one
 token at a time over the packed caches.  One "step" = one decode token = the fused LUT attention
