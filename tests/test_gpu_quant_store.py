@@ -140,6 +140,33 @@ def test_prefill_codes_positions_and_materialize(B, H, T):
             assert torch.equal(a.cpu(), b)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_dequantise_into_other_cache_dtypes(out_dtype):
+    """The dense read-back into fp32 and bf16 tensors (the store itself holds fp16 exact rows):
+    quantised positions equal the oracle's fp32 dequantisation (to the output type's rounding),
+    exact positions are the stored fp16 rows converted, evicted ones are left alone."""
+    g = torch.Generator().manual_seed(31)
+    B, H, T = 2, 3, 257
+    k = torch.randn(B, H, T, 128, generator=g).half(); v = (torch.randn(B, H, T, 128, generator=g) * 3).half()
+    bits = _rand_bits(g, (B, H, T)); bits[..., :2] = 16
+    state = _state()
+    state.prefill(k.to(DEV), v.to(DEV), bits.to(DEV))
+    ref = KVState(128, (0, 2, 3, 4, 8, 16), dtype=torch.float32, seed=42, order="canonical")
+    ref.prefill(k.float(), v.float(), bits)
+    kr, vr = ref.materialize()
+    kd = torch.full((B, H, T, 128), 7.0, dtype=out_dtype, device=DEV); vd = torch.full_like(kd, 7.0)
+    state._dequant_into(kd, vd, True)
+    lm = torch.from_numpy(ref.level_map())
+    quant = (lm != 0) & (lm != 16)
+    tol = 2e-5 if out_dtype == torch.float32 else 2 ** -8
+    for got, want in ((kd, kr), (vd, vr)):
+        got = got.float().cpu()
+        err = (got[quant] - want[quant]).norm(dim=-1) / want[quant].norm(dim=-1)
+        assert err.max() < tol, float(err.max())
+        assert torch.equal(got[lm == 16], want[lm == 16].to(out_dtype).float())
+        assert torch.all(got[lm == 0] == 7.0)
+
+
 def test_append_truncate_and_flush_follow_the_oracle():
     g = torch.Generator().manual_seed(77)
     B, H, D = 1, 4, 128
