@@ -277,23 +277,24 @@ def main() -> int:
         for rep in range(2 if li == 0 else 1):               # the first pass also warms allocators
             st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=dev, dtype=torch.float16, key_quantizer="mse",
                                                 value_quantizer="mse", seed=42 + 7 * li)
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
             torch.cuda.synchronize()
-            t0 = time.perf_counter()
+            ev[0].record()
             s = _launch_score(k, v, mu, None, n_q, 4, 1e-2)
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
+            ev[1].record()
             bits = optimal_scores_to_bits_batched(s.reshape(1, -1), LEVELS, [args.target], eps, n_sink=4, period=T,
                                                   eviction_cost=0.5).reshape(n_kv, T)
             bits[:, -128:] = 16
-            torch.cuda.synchronize()
-            t2 = time.perf_counter()
+            ev[2].record()
             st.prefill(k[None], v[None], bits[None])
+            ev[3].record()
             torch.cuda.synchronize()
-            t3 = time.perf_counter()
-        t_stage["score"].append(t1 - t0)
-        t_stage["alloc"].append(t2 - t1)
-        t_stage["pack"].append(t3 - t2)
-        t_stage["total"].append(t3 - t0)
+        # device events on the launch stream, no host synchronisation between the stages (the pack
+        # stage's own read-back of the level counts is inside its interval)
+        t_stage["score"].append(ev[0].elapsed_time(ev[1]) * 1e-3)
+        t_stage["alloc"].append(ev[1].elapsed_time(ev[2]) * 1e-3)
+        t_stage["pack"].append(ev[2].elapsed_time(ev[3]) * 1e-3)
+        t_stage["total"].append(ev[0].elapsed_time(ev[3]) * 1e-3)
         states.append(st)
         qs.append(q)
         if li == 0:
