@@ -288,12 +288,26 @@ struct TileData {
     f4 kn, vn;
 };
 
+// the packed codes are read once per call and never again before the whole cache has streamed by:
+// loaded with the non-temporal hint, so that they do not push the small per-layer operands (rotations,
+// work lists, tables) out of the caches
+__device__ static inline uint4 stream_load(const uint4* p) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ static inline uint2 stream_load(const uint2* p) {
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+    return make_uint2(v.x, v.y);
+}
+
 template <int W>
 __device__ static inline void load_tile(TileData<W>& t, const DecodeArgs& a, int li, int tile, int lane) {
     const uint8_t* ksrc = a.s.kcodes[li] + (size_t)tile * (TILE * 16 * W);
 #pragma unroll
     for (int c = 0; c < W; ++c) {
-        const uint4 v = *reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 16);
+        const uint4 v = stream_load(reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 16));
         t.kw[4 * c] = v.x; t.kw[4 * c + 1] = v.y; t.kw[4 * c + 2] = v.z; t.kw[4 * c + 3] = v.w;
     }
     const uint8_t* vsrc = a.s.vcodes[li] + (size_t)tile * (HD * 8 * W);
@@ -303,20 +317,20 @@ __device__ static inline void load_tile(TileData<W>& t, const DecodeArgs& a, int
         if constexpr (W == 3) {
 #pragma unroll
             for (int u = 0; u < 3; ++u) {
-                const uint2 v = *reinterpret_cast<const uint2*>(vsrc + ((size_t)u * HD + j) * 8);
+                const uint2 v = stream_load(reinterpret_cast<const uint2*>(vsrc + ((size_t)u * HD + j) * 8));
                 t.vw[h][2 * u] = v.x; t.vw[h][2 * u + 1] = v.y;
             }
         } else {
 #pragma unroll
             for (int u = 0; u < W / 2; ++u) {
-                const uint4 v = *reinterpret_cast<const uint4*>(vsrc + ((size_t)u * HD + j) * 16);
+                const uint4 v = stream_load(reinterpret_cast<const uint4*>(vsrc + ((size_t)u * HD + j) * 16));
                 t.vw[h][4 * u] = v.x; t.vw[h][4 * u + 1] = v.y; t.vw[h][4 * u + 2] = v.z; t.vw[h][4 * u + 3] = v.w;
             }
         }
     }
     const size_t quad = (size_t)tile * TILE + (lane & ~3);
-    t.kn = *reinterpret_cast<const f4*>(a.s.knorm[li] + quad);
-    t.vn = *reinterpret_cast<const f4*>(a.s.vnorm[li] + quad);
+    t.kn = __builtin_nontemporal_load(reinterpret_cast<const f4*>(a.s.knorm[li] + quad));
+    t.vn = __builtin_nontemporal_load(reinterpret_cast<const f4*>(a.s.vnorm[li] + quad));
 }
 
 #define PV_STEP(s)                                                                              \
@@ -454,11 +468,11 @@ __device__ static inline void load_exact_tile(ExactTile& t, const DecodeArgs& a,
     const uint16_t* ksrc = a.s.kexact + (size_t)tile * TILE * HD;
     const uint16_t* vsrc = a.s.vexact + (size_t)tile * TILE * HD;
 #pragma unroll
-    for (int c = 0; c < 16; ++c) t.k[c] = *reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 8);
+    for (int c = 0; c < 16; ++c) t.k[c] = stream_load(reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 8));
 #pragma unroll
     for (int s = 0; s < 16; ++s) {
-        t.v[s][0] = *reinterpret_cast<const uint2*>(vsrc + ((size_t)s * HD + lane) * 4);
-        t.v[s][1] = *reinterpret_cast<const uint2*>(vsrc + ((size_t)s * HD + lane + 64) * 4);
+        t.v[s][0] = stream_load(reinterpret_cast<const uint2*>(vsrc + ((size_t)s * HD + lane) * 4));
+        t.v[s][1] = stream_load(reinterpret_cast<const uint2*>(vsrc + ((size_t)s * HD + lane + 64) * 4));
     }
 }
 
