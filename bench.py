@@ -463,10 +463,21 @@ def main() -> int:
                       "the re-materialised dense cache (what a reference decode step costs), packed bytes / time",
             "sdpa_ms": round(cb["t_sdpa"] * 1e3, 2), "materialize_ms": round(cb["t_materialize"] * 1e3, 1),
             "score_ms": round(cb["t_score"] * 1e3, 1), "alloc_ms": round(cb["t_alloc"] * 1e3, 1),
-            "pack_ms": round(cb["t_pack"] * 1e3, 1),
+            "pack_ms": round(cb["t_pack"] * 1e3, 1), "cpu_model": _cpu_model(),
         }
     print(json.dumps(out))
     return 0
+
+
+def _cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 if __name__ == "__main__":
