@@ -90,8 +90,8 @@ def parity_gate(dev):
     return eps, err
 
 
-def press_e2e(dev, T, target, n_new):
-    """The press end to end on a model of Llama-3-8B's attention shape (2 layers, random weights):
+def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
+    """The press end to end on a model of Llama-3-8B's shape (n_layers layers, random weights):
     prefill T tokens under the press, then n_new greedy decode steps, once over the packed cache
     with the fused kernel and once over the dense re-materialised cache with the model's own
     attention function (what the reference executes).  Wall time per decode step, device-synchronised."""
@@ -99,13 +99,22 @@ def press_e2e(dev, T, target, n_new):
     from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM
     from kvquant import RiskScorer, TurboQuantPerTokenBackendPress, attention_patch
     torch.manual_seed(0)
-    cfg = LlamaConfig(hidden_size=4096, num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
-                      intermediate_size=14336, vocab_size=32000, max_position_embeddings=max(T + n_new + 8, 8192),
-                      rope_theta=500000.0, attn_implementation="sdpa")
-    model = LlamaForCausalLM(cfg).to(device=dev, dtype=torch.float16).eval()
-    ids = torch.randint(0, 32000, (1, T), generator=torch.Generator().manual_seed(1)).to(dev)
-    out = {"model": "2 x Llama-3-8B-shaped layer, random init, fp16", "prefill_tokens": T, "decode_tokens": n_new,
-           "target_avg_bits": target}
+    cfg = LlamaConfig(hidden_size=4096, num_hidden_layers=n_layers, num_attention_heads=32, num_key_value_heads=8,
+                      head_dim=128, intermediate_size=14336, vocab_size=vocab,
+                      max_position_embeddings=max(T + n_new + 8, 8192), rope_theta=500000.0, attn_implementation="sdpa")
+    # weights are drawn on the device in fp16: a host-side fp32 initialisation of 8 B parameters takes minutes
+    default_dtype = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float16)
+    try:
+        with torch.device(dev):
+            model = LlamaForCausalLM(cfg).eval()
+    finally:
+        torch.set_default_dtype(default_dtype)
+    print(f"[press-e2e] model of {n_layers} layers built", file=sys.stderr, flush=True)
+    ids = torch.randint(0, vocab, (1, T), generator=torch.Generator().manual_seed(1)).to(dev)
+    out = {"model": f"{n_layers} x Llama-3-8B-shaped layer, vocabulary {vocab}, random init, fp16", "prefill_tokens": T,
+           "decode_tokens": n_new, "target_avg_bits": target}
+    tokens = {}
     for mode in ("fused", "dense"):
         os.environ["ODMKV_FUSED_DECODE"] = "1" if mode == "fused" else "0"
         scorer = RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
@@ -122,7 +131,8 @@ def press_e2e(dev, T, target, n_new):
             tok = model.lm_head(h)[0, -1].argmax().view(1, 1)
             torch.cuda.synchronize()
             t_prefill = time.perf_counter() - t0
-            steps = []
+            print(f"[press-e2e] {mode}: prefill of {T} tokens {t_prefill:.2f} s", file=sys.stderr, flush=True)
+            steps, emitted = [], [int(tok)]
             for step in range(n_new):
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
@@ -131,12 +141,23 @@ def press_e2e(dev, T, target, n_new):
                 tok = logits[0, -1].argmax().view(1, 1)
                 torch.cuda.synchronize()
                 steps.append(time.perf_counter() - t0)
+                emitted.append(int(tok))
+        tokens[mode] = emitted
+        print(f"[press-e2e] {mode}: {n_new} decode steps done", file=sys.stderr, flush=True)
         took = {k: attention_patch.call_counts[k] - before[k] for k in before}
         out[mode] = {"prefill_s": round(t_prefill, 3), "decode_step_ms_median": round(statistics.median(steps[4:]) * 1e3, 3),
-                     "decode_step_ms_min": round(min(steps[4:]) * 1e3, 3), "attention_calls": took}
+                     "decode_step_ms_min": round(min(steps[4:]) * 1e3, 3),
+                     "decode_step_ms_mean_with_flushes": round(statistics.fmean(steps[4:]) * 1e3, 3),
+                     "attention_calls": took}
         del cache, press
         torch.cuda.empty_cache()
     os.environ.pop("ODMKV_FUSED_DECODE", None)
+    same = 0
+    for x, y in zip(tokens["fused"], tokens["dense"]):      # greedy tokens agree until the first near-tie
+        if x != y:
+            break
+        same += 1
+    out["greedy_tokens_equal_prefix"] = same
     out["dense_over_fused"] = round(out["dense"]["decode_step_ms_median"] / out["fused"]["decode_step_ms_median"], 2)
     return out
 
@@ -202,10 +223,12 @@ def main() -> int:
                     help="for counter runs under rocprofv3 --pmc: a few eager decode steps and one plain 256 MiB "
                          "device copy (the calibration kernel), nothing else timed")
     ap.add_argument("--press-e2e", action="store_true",
-                    help="instead of the kernel benchmark: a 2-layer random-init Llama-3-8B-shaped model under the "
+                    help="instead of the kernel benchmark: a random-init Llama-3-8B-shaped model (--e2e-layers) under the "
                          "press, prefill of --ctx tokens, then greedy decode with the fused kernel and with the dense "
                          "re-materialised cache (the reference's path); prints per-token times")
     ap.add_argument("--e2e-tokens", type=int, default=48)
+    ap.add_argument("--e2e-layers", type=int, default=2, help="layers of the --press-e2e model (32 = Llama-3-8B)")
+    ap.add_argument("--e2e-vocab", type=int, default=32000, help="vocabulary of the --press-e2e model (Llama-3: 128256)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the path: every box in this build has one GPU and "
@@ -225,7 +248,8 @@ def main() -> int:
     n_kv, n_q, T, NL = 8, 32, args.ctx, args.layers
 
     if args.press_e2e:
-        print(json.dumps({"press_e2e": press_e2e(dev, T, args.target, args.e2e_tokens)}))
+        print(json.dumps({"press_e2e": press_e2e(dev, T, args.target, args.e2e_tokens, args.e2e_layers,
+                                                   args.e2e_vocab)}))
         return 0
 
     if args.read_ceiling:

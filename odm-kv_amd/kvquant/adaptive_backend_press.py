@@ -26,6 +26,22 @@ from kvquant.press import TurboQuantPerTokenPress
 from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
 
 
+def _levels_by_rank(levels, ratios, n: int):
+    """Level of the token of every rank 0..n-1 (ascending score) under `ratio_scores_to_bits`'
+    tier sizes: round(share * n) tokens per tier from the lowest level up, the last tier takes the rest."""
+    import numpy as np
+    share = torch.tensor(ratios, dtype=torch.float64)
+    share = (share / share.sum()).tolist()
+    tiers = sorted(zip(levels, share), key=lambda t: t[0])
+    out = np.empty(n, np.int32)
+    cursor = 0
+    for i, (b, frac) in enumerate(tiers):
+        count = n - cursor if i == len(tiers) - 1 else min(int(round(frac * n)), n - cursor)
+        out[cursor:cursor + count] = b
+        cursor += count
+    return out
+
+
 class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
     def __init__(self, *, value_group_size: int = 32, key_quantizer: str = "prod", value_quantizer: str = "minmax",
                  scorer=None, bit_levels: tuple[int, ...] = (0, 2, 4, 8, 16), ratios: Optional[tuple[float, ...]] = None,
@@ -111,17 +127,35 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
             self._observed_ratios[(layer_idx, row % H)] = tuple(
                 (b, f) for b, f, n in zip(levels, fracs, c.tolist()) if n > 0)
 
-    def _allocate_bits_via_cached_ratios(self, scores, positions, num_heads, layer_idx, allowed_levels):
+    def _allocate_bits_via_cached_ratios(self, scores, positions, num_heads, layer_idx, allowed_levels,
+                                         batch_size: Optional[int] = None):
+        """Rank tiers per kv-head with the level shares seen at prefill.  With `batch_size` the
+        caller states that the tokens come ordered (batch, head, position) with the same count in
+        every (batch, head): all heads are then ranked by one sort instead of a loop of sorts."""
         if not all((layer_idx, h) in self._observed_ratios for h in range(num_heads)):
             return None
-        bits = torch.empty_like(scores, dtype=torch.int32)
-        head_indices = positions[:, 1]
+        tiers = []
         for h in range(num_heads):
             kept = [(b, r) for b, r in self._observed_ratios[(layer_idx, h)] if b in allowed_levels and r > 0]
             if not kept:
                 return None
             total = sum(r for _, r in kept)
-            levels, ratios = zip(*[(b, r / total) for b, r in kept])
+            tiers.append(tuple(zip(*[(b, r / total) for b, r in kept])))
+        n_tok = scores.shape[0]
+        if batch_size is not None and n_tok > 0 and n_tok % (batch_size * num_heads) == 0:
+            B, H, n = int(batch_size), int(num_heads), n_tok // (batch_size * num_heads)
+            rows = scores.reshape(B, H, n).permute(1, 0, 2).reshape(H, B * n)       # one row per head
+            order = torch.argsort(rows, dim=1, stable=True)
+            by_rank = torch.empty(H, B * n, dtype=torch.int32)
+            for h, (levels, ratios) in enumerate(tiers):
+                by_rank[h] = torch.from_numpy(_levels_by_rank(levels, ratios, B * n))
+            out = torch.empty(H, B * n, dtype=torch.int32, device=scores.device)
+            out.scatter_(1, order, by_rank.to(scores.device, non_blocking=True))
+            return out.reshape(H, B, n).permute(1, 0, 2).reshape(-1)
+        bits = torch.empty_like(scores, dtype=torch.int32)
+        head_indices = positions[:, 1]
+        for h in range(num_heads):
+            levels, ratios = tiers[h]
             mask = head_indices == h
             if not mask.any():
                 continue
@@ -239,11 +273,9 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         else:
             scores = buf_keys.float().pow(2).sum(-1) + buf_values.float().pow(2).sum(-1)
 
-        lo, hi = scores.min(), scores.max()
-        if hi - lo > 1e-8:
-            scores = (scores - lo) / (hi - lo)
-        else:
-            scores = torch.full_like(scores, 0.5)
+        lo, hi = torch.aminmax(scores)
+        spread = hi - lo                                     # stays on the device: no wait for the scores here
+        scores = torch.where(spread > 1e-8, (scores - lo) / spread.clamp_min(1e-30), torch.full_like(scores, 0.5))
 
         levels = self._decode_bit_levels
         allowed = set(levels)
@@ -254,7 +286,8 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
                 flush_levels, flush_ratios = zip(*pairs)
                 bits = ratio_scores_to_bits(scores, tuple(flush_levels), tuple(flush_ratios))
         elif self.target_avg_bits is not None:
-            bits = self._allocate_bits_via_cached_ratios(scores, positions, state.num_heads, layer_idx, allowed)
+            bits = self._allocate_bits_via_cached_ratios(scores, positions, state.num_heads, layer_idx, allowed,
+                                                         batch_size=state.batch_size)
             if bits is None:
                 eps = self._ensure_epsilon(scores.device)
                 bits = optimal_scores_to_bits(

@@ -119,6 +119,7 @@ class TurboQuantAdaptiveKVCacheState:
         self._masked = None           # cached (indices of evicted positions,) or None when stale
         self._items = None
         self._item_order = None
+        self._items_choice = None     # (winning items-per-compute-unit multiple, packed bytes it was chosen at)
         self._packed = None
 
     @property
@@ -225,6 +226,9 @@ class TurboQuantAdaptiveKVCacheState:
                 return
         cap = self._capacity_tiles(new_counts)
         if self._bufs is not None:
+            # a store that grows once will grow again (every decode-time flush adds tokens to the
+            # quantised levels): leave a sixteenth of head-room so that the tiles move rarely
+            cap[:4] += np.maximum(cap[:4] // 16, 2)
             cap = np.maximum(cap, np.diff(self._seg_tile, axis=1))
         seg_tile = np.zeros((5, self._nseg + 1), np.int64)
         seg_tile[:, 1:] = np.cumsum(cap, axis=1)
@@ -542,23 +546,29 @@ class TurboQuantAdaptiveKVCacheState:
         if explicit is not None:
             items = cut(fit(int(explicit)))
         else:
-            best = None
-            for mult in (1.0, 1.5, 2.0, 3.0, 4.0):
-                cand = cut(fit(int(n_cu * mult)))
-                t = makespan(cand)
-                if best is None or t < best[0] - 1e-9:
-                    best = (t, cand)
-            items = best[1]
-        ranges = [0]
-        for s in range(self._nseg):
-            ranges.append(ranges[-1] + sum(1 for it in items if it[0] == s))
+            # the comparison is repeated only when the store has grown by more than 5 % since the
+            # last one (a decode-time flush adds a fraction of a percent): until then its winner is re-cut
+            chosen = self._items_choice
+            if chosen is not None and abs(total - chosen[1]) <= 0.05 * chosen[1]:
+                items = cut(fit(int(n_cu * chosen[0])))
+            else:
+                best = None
+                for mult in (1.0, 1.5, 2.0, 3.0, 4.0):
+                    cand = cut(fit(int(n_cu * mult)))
+                    t = makespan(cand)
+                    if best is None or t < best[0] - 1e-9:
+                        best = (t, cand, mult)
+                items = best[1]
+                self._items_choice = (best[2], total)
         arr = np.asarray(items, np.int32).reshape(-1, 8)
+        per_seg = np.bincount(arr[:, 0], minlength=self._nseg) if len(items) else np.zeros(self._nseg, np.int64)
+        ranges = np.concatenate([[0], np.cumsum(per_seg)])          # items are generated in segment order
         order = None
         if len(items) > n_cu:
             order = np.argsort(-np.asarray([cost(it) for it in items]), kind="stable").astype(np.int32)
             order = torch.from_numpy(order).to(self.device)
         self._items = (torch.from_numpy(arr).to(self.device),
-                       torch.from_numpy(np.asarray(ranges, np.int32)).to(self.device), len(items))
+                       torch.from_numpy(ranges.astype(np.int32)).to(self.device), len(items))
         self._item_order = order
 
     def decode_attention(self, query: torch.Tensor, scaling: Optional[float] = None,

@@ -90,6 +90,17 @@ def test_observed_ratios_and_cached_allocation():
     assert out[:n].tolist() == [2] * 8 + [4] * 4          # 2/3 and 1/3 of 12
     assert out[n:].tolist() == [2] * 9 + [4] * 3
     assert p._allocate_bits_via_cached_ratios(scores, pos, 2, 5, {2, 4, 16}) is None     # layer without a record
+    # the one-sort form taken when the caller vouches for the (batch, head, position) order: same levels
+    assert torch.equal(p._allocate_bits_via_cached_ratios(scores, pos, 2, 3, {2, 4, 16}, batch_size=1), out)
+    B, H, n = 3, 2, 37
+    g = torch.Generator().manual_seed(5)
+    scores = torch.rand(B * H * n, generator=g)
+    scores[7] = scores[9]                                  # a tie keeps index order in both forms
+    pos = torch.stack([torch.arange(B).repeat_interleave(H * n), torch.arange(H).repeat_interleave(n).repeat(B),
+                       torch.arange(n).repeat(B * H)], dim=-1)
+    for allowed in ({0, 2, 4, 16}, {2, 4}):
+        loop = p._allocate_bits_via_cached_ratios(scores, pos, H, 3, allowed)
+        assert torch.equal(p._allocate_bits_via_cached_ratios(scores, pos, H, 3, allowed, batch_size=B), loop)
 
 
 def test_backend_press_rejects_unbuilt_quantisers():
