@@ -152,6 +152,15 @@ def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
         del cache, press
         torch.cuda.empty_cache()
     os.environ.pop("ODMKV_FUSED_DECODE", None)
+    cache = DynamicCache()
+    with torch.inference_mode():                             # the same prefill with no press attached
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        h = model.model(input_ids=ids, past_key_values=cache).last_hidden_state[:, -1:, :]
+        model.lm_head(h)
+        torch.cuda.synchronize()
+        out["prefill_s_without_press"] = round(time.perf_counter() - t0, 3)
+    del cache
     same = 0
     for x, y in zip(tokens["fused"], tokens["dense"]):      # greedy tokens agree until the first near-tie
         if x != y:
