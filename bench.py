@@ -92,9 +92,10 @@ def parity_gate(dev):
 
 def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
     """The press end to end on a model of Llama-3-8B's shape (n_layers layers, random weights):
-    prefill T tokens under the press, then n_new greedy decode steps, once over the packed cache
-    with the fused kernel and once over the dense re-materialised cache with the model's own
-    attention function (what the reference executes).  Wall time per decode step, device-synchronised."""
+    prefill T tokens under the press, then n_new greedy decode steps: over the packed cache with the
+    fused kernel, the same with the model's dense cache copy released, and over the dense
+    re-materialised cache with the model's own attention function (what the reference executes).
+    Wall time per decode step, device-synchronised; device memory the caches hold after the prefill."""
     import torch
     from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM
     from kvquant import RiskScorer, TurboQuantPerTokenBackendPress, attention_patch
@@ -115,13 +116,16 @@ def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
     out = {"model": f"{n_layers} x Llama-3-8B-shaped layer, vocabulary {vocab}, random init, fp16", "prefill_tokens": T,
            "decode_tokens": n_new, "target_avg_bits": target}
     tokens = {}
-    for mode in ("fused", "dense"):
-        os.environ["ODMKV_FUSED_DECODE"] = "1" if mode == "fused" else "0"
+    for mode in ("fused", "fused_released", "dense"):
+        os.environ["ODMKV_FUSED_DECODE"] = "0" if mode == "dense" else "1"
+        torch.cuda.synchronize()
+        base_bytes = torch.cuda.memory_allocated()
         scorer = RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
         scorer.normalize_grain = "global"
         press = TurboQuantPerTokenBackendPress(
             scorer=scorer, bit_levels=LEVELS, target_avg_bits=target, eviction_cost=0.5, seed=42, decode_quant=True,
-            sink_tokens=4, layerwise=True, key_quantizer="mse", value_quantizer="mse", buffer_size=128)
+            sink_tokens=4, layerwise=True, key_quantizer="mse", value_quantizer="mse", buffer_size=128,
+            release_dense_cache=(mode == "fused_released"))
         before = dict(attention_patch.call_counts)
         cache = DynamicCache()
         with torch.inference_mode(), press(model):
@@ -131,6 +135,8 @@ def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
             tok = model.lm_head(h)[0, -1].argmax().view(1, 1)
             torch.cuda.synchronize()
             t_prefill = time.perf_counter() - t0
+            del h
+            cache_bytes = torch.cuda.memory_allocated() - base_bytes      # packed stores + what the HF cache holds
             print(f"[press-e2e] {mode}: prefill of {T} tokens {t_prefill:.2f} s", file=sys.stderr, flush=True)
             steps, emitted = [], [int(tok)]
             for step in range(n_new):
@@ -148,8 +154,11 @@ def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
         out[mode] = {"prefill_s": round(t_prefill, 3), "decode_step_ms_median": round(statistics.median(steps[4:]) * 1e3, 3),
                      "decode_step_ms_min": round(min(steps[4:]) * 1e3, 3),
                      "decode_step_ms_mean_with_flushes": round(statistics.fmean(steps[4:]) * 1e3, 3),
-                     "attention_calls": took}
+                     "attention_calls": took, "cache_bytes_after_prefill": int(cache_bytes)}
         del cache, press
+        for layer in model.model.layers:                     # the modules keep their last store attached
+            layer.self_attn._odmkv_state = None
+            layer.self_attn.masked_key_indices = None
         torch.cuda.empty_cache()
     os.environ.pop("ODMKV_FUSED_DECODE", None)
     cache = DynamicCache()
@@ -168,6 +177,8 @@ def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
         same += 1
     out["greedy_tokens_equal_prefix"] = same
     out["dense_over_fused"] = round(out["dense"]["decode_step_ms_median"] / out["fused"]["decode_step_ms_median"], 2)
+    out["dense_over_fused_released"] = round(
+        out["dense"]["decode_step_ms_median"] / out["fused_released"]["decode_step_ms_median"], 2)
     return out
 
 

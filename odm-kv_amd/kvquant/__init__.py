@@ -14,6 +14,7 @@ _LAZY = {
     "TurboQuantPerTokenBackendPress": "kvquant.adaptive_backend_press",
     "TurboQuantBackendPress": "kvquant.backend_press",
     "TurboQuantPerTokenPress": "kvquant.press",
+    "PackedCacheLayer": "kvquant.hf_cache",          # not in the reference: a cache layer without a dense copy
 }
 
 

@@ -21,7 +21,9 @@ import torch
 from torch import nn
 
 from kvquant.allocator import optimal_scores_to_bits, ratio_scores_to_bits, scores_to_bits
+from kvquant.attention_patch import fused_decode_enabled
 from kvquant.attention_utils import _aligned_rotary_outputs, _apply_rotary_pos_emb_q, _get_query_states
+from kvquant.hf_cache import PackedCacheLayer
 from kvquant.press import TurboQuantPerTokenPress
 from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
 
@@ -48,7 +50,7 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
                  target_avg_bits: Optional[float] = None, eviction_cost: float = 5.0, above_target_alpha: float = 1.0,
                  n_outlier_channels: int = 0, outlier_min_bits: int = 4, seed: int = 42, decode_quant: bool = True,
                  sink_tokens: int = 0, layerwise: bool = False, buffer_size: int = 128, initial_layers_fp16: int = 0,
-                 allow_decode_eviction: bool = False):
+                 allow_decode_eviction: bool = False, release_dense_cache: bool = False):
         min_bits = 2 if key_quantizer in ("prod", "turboquant_prod", "turboquantprod") else 1
         invalid = [b for b in bit_levels if b not in (0, 16) and b < min_bits]
         if invalid:
@@ -63,6 +65,11 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         self.key_quantizer = key_quantizer
         self.buffer_size = buffer_size
         self.initial_layers_fp16 = initial_layers_fp16
+        # not in the reference: once a layer's prefill is packed, swap its cache layer for one that
+        # keeps no dense copy (kvquant/hf_cache.py); decode then needs the fused attention path
+        if release_dense_cache and not decode_quant:
+            raise ValueError("release_dense_cache needs decode_quant=True: new tokens must reach the packed store")
+        self.release_dense_cache = bool(release_dense_cache)
         self._states: dict[int, TurboQuantAdaptiveKVCacheState] = {}
         self._buffer_counts: dict[int, int] = {}
         self._buffer_start_seqs: dict[int, int] = {}
@@ -88,6 +95,24 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         self._states[layer_idx] = state
         return state
 
+    @staticmethod
+    def _packed_layer(cache, layer_idx: int) -> Optional[PackedCacheLayer]:
+        layers = getattr(cache, "layers", None)
+        if layers is not None and layer_idx < len(layers) and isinstance(layers[layer_idx], PackedCacheLayer):
+            return layers[layer_idx]
+        return None
+
+    def _release_dense(self, cache, layer_idx: int, state) -> None:
+        """Swap the layer's dense tensors for aliased views of its last token."""
+        if not self.release_dense_cache or layer_idx < self.initial_layers_fp16:
+            return
+        if not hasattr(cache, "layers") or self._packed_layer(cache, layer_idx) is not None:
+            return
+        if not fused_decode_enabled():
+            raise RuntimeError("release_dense_cache needs the fused decode path (ODMKV_FUSED_DECODE=0 is set)")
+        keys, values = self._get_cache_tensors(cache, layer_idx)
+        cache.layers[layer_idx] = PackedCacheLayer(state, keys, values)
+
     def _attach(self, cache, layer_idx: int, module: nn.Module, state) -> None:
         module.masked_key_indices = state.masked_key_indices()
         module._odmkv_state = state
@@ -95,6 +120,9 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
             cache.layers[layer_idx]._tq_backend_state = state
 
     def _sync_cache_from_state(self, cache, layer_idx: int, module: nn.Module, state, *, prefill_fast: bool = False) -> None:
+        if self._packed_layer(cache, layer_idx) is not None:
+            self._attach(cache, layer_idx, module, state)            # no dense copy to bring up to date
+            return
         if prefill_fast:
             keys, values = self._get_cache_tensors(cache, layer_idx)
             state.materialize_quantized_into(keys, values)
@@ -178,6 +206,8 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
             state.prefill(keys, values, bits.to(dtype=torch.int32, device=keys.device))
             module = self._layer_modules.get(layer_idx)
             if module is not None:
+                if self.release_dense_cache and layer_idx >= self.initial_layers_fp16:
+                    self._release_dense(cache, layer_idx, state)
                 self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True)
             if self.buffer_size > 0:
                 self._buffer_start_seqs[layer_idx] = int(keys.shape[2])
@@ -209,8 +239,12 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
                 self._buffer_counts[layer_idx] = 0
 
         already_stored = state.seq_len == cache_len       # the fused attention path stored the token
-        new_k = keys[:, :, -q_len:, :]
-        new_v = values[:, :, -q_len:, :]
+        packed_layer = self._packed_layer(cache, layer_idx)
+        if packed_layer is not None:
+            new_k, new_v = packed_layer.recent            # the layer's tensors alias one token
+        else:
+            new_k = keys[:, :, -q_len:, :]
+            new_v = values[:, :, -q_len:, :]
         if self.buffer_size > 0:
             if not already_stored:
                 state.append_all_exact(new_k, new_v)

@@ -93,6 +93,11 @@ def _attention_patch(func):
             if fused is not None:
                 call_counts["fused"] += 1
                 return fused, None
+            if key.dim() == 4 and key.shape[2] > 1 and key.stride(2) == 0:
+                raise RuntimeError(
+                    "this layer's dense cache was released (release_dense_cache=True) and the call cannot take the "
+                    "fused decode path (padding mask, dropout, sliding window, soft cap or a batch the store was "
+                    "not built for): keep the dense cache for such calls")
             call_counts["dense"] += 1
             if getattr(module, "masked_key_indices", None) is not None:
                 bsz, num_heads, seq_len, head_dim = query.shape

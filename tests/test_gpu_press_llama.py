@@ -158,3 +158,90 @@ def test_free_running_greedy_tokens_agree():
     tok_d, _, _, _ = _generate(model, _press(), ids, 24, fused=False)
     tok_f, _, _, _ = _generate(model, _press(), ids, 24, fused=True)
     assert (tok_d == tok_f).float().mean().item() >= 0.9
+
+
+def _rewind(cache, length):
+    """Rewind the way the reference's runner does between questions (benchmark/core/pipeline.py:211-228):
+    truncate the store attached to each layer and slice the layer's tensors."""
+    for layer in cache.layers:
+        store = getattr(layer, "_tq_backend_state", None)
+        if store is not None:
+            store.truncate(length)
+        for name in ("keys", "values"):
+            t = getattr(layer, name)
+            if t.shape[2] > length:
+                setattr(layer, name, t[:, :, :length])
+
+
+@torch.inference_mode()
+def _session(model, press, ids, forced, question):
+    """Prefill, teacher-forced single-token steps, a multi-token step, a rewind by three tokens and
+    one more step; returns the logits of every call and the cache."""
+    from transformers import DynamicCache
+    cache = DynamicCache()
+    T = ids.shape[1]
+    logits = []
+    with press(model):
+        out = model.model(input_ids=ids, past_key_values=cache)
+        logits.append(model.lm_head(out.last_hidden_state[:, -1:, :])[0, -1].float())
+        pos = T
+        for tok in forced:
+            out = model(input_ids=tok.view(1, 1), past_key_values=cache, position_ids=torch.tensor([[pos]], device=DEV))
+            logits.append(out.logits[0, -1].float())
+            pos += 1
+        mid_layers = [type(layer).__name__ for layer in cache.layers]
+        mid_strides = [layer.keys.stride(2) for layer in cache.layers]
+        q = question.view(1, -1)
+        out = model(input_ids=q, past_key_values=cache,
+                    position_ids=torch.arange(pos, pos + q.shape[1], device=DEV).view(1, -1))
+        logits.append(out.logits[0, -1].float())
+        pos += q.shape[1]
+        assert cache.get_seq_length() == pos
+        pos -= 2
+        _rewind(cache, pos)
+        if mid_layers[0] == "PackedCacheLayer":
+            cache.crop(-1)                                 # the packed layer truncates its store itself
+        else:
+            _rewind(cache, pos - 1)
+        pos -= 1
+        assert cache.get_seq_length() == pos
+        assert all(st.seq_len == pos for st in press._states.values())
+        out = model(input_ids=forced[0].view(1, 1), past_key_values=cache, position_ids=torch.tensor([[pos]], device=DEV))
+        logits.append(out.logits[0, -1].float())
+    return torch.stack(logits), cache, mid_layers, mid_strides
+
+
+def test_released_dense_cache_decodes_identically():
+    """`release_dense_cache=True` keeps no dense copy of the packed layers (stride-0 views of the
+    newest token) and gives the logits of the press that keeps the copy: the same at single-token
+    steps (same kernel, same store), within fp16 rounding at the multi-token step (dense attention
+    over the dequantised store against dense attention over the kept copy), across a rewind."""
+    model = _model(4)
+    ids = _ids(600, 21)
+    g = torch.Generator().manual_seed(22)
+    forced = torch.randint(0, 1000, (140,), generator=g).to(DEV)          # crosses one buffer flush
+    question = torch.randint(0, 1000, (5,), generator=g).to(DEV)
+    keep, cache_k, layers_k, strides_k = _session(model, _press(), ids, forced, question)
+    rel, cache_r, layers_r, strides_r = _session(model, _press(release_dense_cache=True), ids, forced, question)
+    assert layers_k == ["DynamicLayer"] * 2 and all(s != 0 for s in strides_k)
+    assert layers_r == ["PackedCacheLayer"] * 2 and strides_r == [0, 0]
+    n_single = 1 + forced.shape[0]
+    assert torch.equal(rel[:n_single], keep[:n_single])
+    assert (rel[n_single:] - keep[n_single:]).abs().max().item() < LOGIT_ATOL
+    assert torch.isfinite(rel).all()
+
+
+def test_released_dense_cache_refuses_the_dense_path():
+    from transformers import DynamicCache
+    model = _model(5)
+    ids = _ids(300, 23)
+    press = _press(release_dense_cache=True)
+    cache = DynamicCache()
+    with torch.inference_mode(), press(model):
+        model.model(input_ids=ids, past_key_values=cache)
+        os.environ["ODMKV_FUSED_DECODE"] = "0"
+        try:
+            with pytest.raises(RuntimeError, match="dense cache was released"):
+                model(input_ids=ids[:, :1], past_key_values=cache, position_ids=torch.tensor([[300]], device=DEV))
+        finally:
+            os.environ.pop("ODMKV_FUSED_DECODE", None)

@@ -108,3 +108,69 @@ def test_backend_press_rejects_unbuilt_quantisers():
     with pytest.raises(NotImplementedError):
         TurboQuantBackendPress()                       # min-max values by default
     TurboQuantBackendPress(key_quantizer="mse", value_quantizer="mse")
+
+
+class _FakeStore:
+    """What PackedCacheLayer needs of a packed store: a length, dense rows on request, truncation."""
+    def __init__(self, keys, values):
+        self.k, self.v = keys.clone(), values.clone()
+
+    @property
+    def seq_len(self):
+        return self.k.shape[2]
+
+    def append(self, k, v):
+        self.k, self.v = torch.cat([self.k, k], 2), torch.cat([self.v, v], 2)
+
+    def materialize(self):
+        return self.k, self.v
+
+    def truncate(self, n):
+        self.k, self.v = self.k[:, :, :n], self.v[:, :, :n]
+
+
+def test_packed_cache_layer_aliases_the_newest_token():
+    from kvquant.hf_cache import PackedCacheLayer, is_aliased
+    g = torch.Generator().manual_seed(0)
+    k0, v0 = torch.randn(2, 3, 10, 8, generator=g), torch.randn(2, 3, 10, 8, generator=g)
+    store = _FakeStore(k0, v0)
+    layer = PackedCacheLayer(store, k0, v0)
+    assert layer.get_seq_length() == 10 and layer.get_mask_sizes(1) == (11, 0)
+    assert is_aliased(layer.keys) and layer.keys.untyped_storage().nbytes() == 2 * 3 * 8 * 4
+    # one token: shapes in step, every position aliases the new token, nothing is concatenated
+    k1, v1 = torch.randn(2, 3, 1, 8, generator=g), torch.randn(2, 3, 1, 8, generator=g)
+    keys, values = layer.update(k1, v1)
+    assert keys.shape == (2, 3, 11, 8) and is_aliased(keys) and torch.equal(keys[:, :, -1:], k1)
+    assert torch.equal(values[:, :, -1:], v1) and layer.recent[0] is k1
+    store.append(k1, v1)                                   # what the attention path does with the token
+    # several tokens: real dense tensors for this call (store rows + the new ones), views afterwards
+    k2, v2 = torch.randn(2, 3, 4, 8, generator=g), torch.randn(2, 3, 4, 8, generator=g)
+    keys, values = layer.update(k2, v2)
+    assert not is_aliased(keys) and torch.equal(keys, torch.cat([k0, k1, k2], 2))
+    assert torch.equal(values, torch.cat([v0, v1, v2], 2))
+    assert layer.get_seq_length() == 15 and is_aliased(layer.keys) and torch.equal(layer.recent[0], k2)
+    store.append(k2, v2)
+    # out of step: refused rather than answered from the wrong rows
+    store.truncate(14)
+    with pytest.raises(RuntimeError, match="in step"):
+        layer.update(k2, v2)
+    store.append(k2[:, :, -1:], v2[:, :, -1:])
+    # crop, both spellings
+    layer.crop(-2)
+    assert layer.get_seq_length() == 13 and store.seq_len == 13
+    layer.crop(12)
+    assert layer.get_seq_length() == 12 and store.seq_len == 12
+    layer.crop(40)
+    assert layer.get_seq_length() == 12
+    with pytest.raises(NotImplementedError):
+        layer.reorder_cache(torch.tensor([0, 1]))
+    with pytest.raises(ValueError, match="holds"):
+        PackedCacheLayer(store, k0, v0)
+
+
+def test_release_dense_cache_needs_decode_quant():
+    from kvquant import TurboQuantPerTokenBackendPress
+    with pytest.raises(ValueError, match="release_dense_cache"):
+        TurboQuantPerTokenBackendPress(scorer=_scorer(), bit_levels=(0, 2, 4, 16), key_quantizer="mse",
+                                       value_quantizer="mse", target_avg_bits=2.0, decode_quant=False,
+                                       release_dense_cache=True)
