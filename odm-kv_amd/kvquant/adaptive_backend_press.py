@@ -9,7 +9,10 @@ follow from running on the packed store:
   not by the HF attention function over a re-materialised cache; the HF cache tensors are still
   kept in step (quantised positions overwritten in place) so the dense path remains usable;
 * layer-wise allocation of all layers runs as one batched allocator launch;
-* flush scoring handles all kv-heads of a sequence in one launch instead of a loop per head.
+* flush scoring handles all kv-heads of a sequence in one launch instead of a loop per head, and
+  the cached-ratio allocation ranks all heads with one sort;
+* ``release_dense_cache=True`` (a constructor argument the reference does not have) swaps each
+  packed layer of the model's cache for one that keeps no dense copy (hf_cache.py).
 """
 from __future__ import annotations
 
