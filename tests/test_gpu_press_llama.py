@@ -245,3 +245,24 @@ def test_released_dense_cache_refuses_the_dense_path():
                 model(input_ids=ids[:, :1], past_key_values=cache, position_ids=torch.tensor([[300]], device=DEV))
         finally:
             os.environ.pop("ODMKV_FUSED_DECODE", None)
+
+
+@torch.inference_mode()
+def test_released_dense_cache_with_a_batch_of_two():
+    from transformers import DynamicCache
+    model = _model(6)
+    g = torch.Generator().manual_seed(31)
+    ids = torch.randint(0, 1000, (2, 400), generator=g).to(DEV)
+    forced = torch.randint(0, 1000, (12, 2), generator=g).to(DEV)
+    runs = []
+    for release in (False, True):
+        cache, logits = DynamicCache(), []
+        with _press(release_dense_cache=release)(model) as _:
+            model.model(input_ids=ids, past_key_values=cache)
+            for step in range(forced.shape[0]):
+                out = model(input_ids=forced[step].view(2, 1), past_key_values=cache,
+                            position_ids=torch.full((2, 1), 400 + step, device=DEV))
+                logits.append(out.logits[:, -1].float())
+        assert cache.get_seq_length() == 400 + forced.shape[0]
+        runs.append(torch.stack(logits))
+    assert torch.equal(runs[0], runs[1])
