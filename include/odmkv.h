@@ -166,10 +166,12 @@ int odmkv_dequant(const odmkv_packed_t* store, void* K, void* V, int dtype, int 
 
 /* Append one fp16/bf16 token per (b, h) to the exact segments (append_all_exact,
  * kvquant/tq_adaptive_backend.py:380-425, for one decode step).  k, v: [B, Hkv, 128] of the
- * store's exact dtype, contiguous.  Fails with ODMKV_ENOSPACE semantics on the device side by
- * leaving seg_count untouched when a segment is full; the caller sizes segments. */
-int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v, int pos,
-                       void* stream);
+ * store's exact dtype with batch and head strides in elements (the same for k and v; the 128
+ * values of a row are contiguous), so the newest token of a [B, Hkv, T, 128] cache is passed as
+ * it lies.  Fails with ODMKV_ENOSPACE semantics on the device side by leaving seg_count
+ * untouched when a segment is full; the caller sizes segments. */
+int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v, int64_t stride_b,
+                       int64_t stride_h, int pos, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Fused LUT decode attention over the packed store: one query token per sequence.

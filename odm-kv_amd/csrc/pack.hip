@@ -728,8 +728,10 @@ __global__ __launch_bounds__(64) void exact_gather_kernel(ExactArgs a) {
 
 // one new token per (b, h) behind the stored exact tokens
 __global__ __launch_bounds__(128) void append_exact_kernel(odmkv_packed_t s, const uint16_t* __restrict__ k,
-                                                           const uint16_t* __restrict__ v, int pos) {
+                                                           const uint16_t* __restrict__ v, int64_t stride_b,
+                                                           int64_t stride_h, int pos) {
     const int bh = blockIdx.x, j = threadIdx.x;
+    const size_t src = (size_t)(bh / s.Hkv) * stride_b + (size_t)(bh % s.Hkv) * stride_h + j;
     const int cnt = s.seg_count[4][bh];
     const int cap = (s.seg_tile[4][bh + 1] - s.seg_tile[4][bh]) * TILE;
     if (cnt >= cap) return;                                  // full: the host sized it too small
@@ -737,8 +739,8 @@ __global__ __launch_bounds__(128) void append_exact_kernel(odmkv_packed_t s, con
     const int l = cnt % TILE;
     uint16_t* kd = s.kexact + (size_t)tile * TILE * HD;
     uint16_t* vd = s.vexact + (size_t)tile * TILE * HD;
-    kd[((size_t)(j >> 3) * TILE + l) * 8 + (j & 7)] = k[(size_t)bh * HD + j];
-    vd[((size_t)(l >> 2) * HD + j) * 4 + (l & 3)] = v[(size_t)bh * HD + j];
+    kd[((size_t)(j >> 3) * TILE + l) * 8 + (j & 7)] = k[src];
+    vd[((size_t)(l >> 2) * HD + j) * 4 + (l & 3)] = v[src];
     __syncthreads();
     if (j == 0) {
         s.pos[4][(size_t)tile * TILE + l] = pos;
@@ -746,13 +748,15 @@ __global__ __launch_bounds__(128) void append_exact_kernel(odmkv_packed_t s, con
     }
 }
 
-extern "C" int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v, int pos,
-                                  void* stream) {
+extern "C" int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v, int64_t stride_b,
+                                  int64_t stride_h, int pos, void* stream) {
     ODMKV_CHECK_ARG(store && k && v, "append_exact: null pointer");
+    ODMKV_CHECK_ARG(stride_b >= 0 && stride_h >= 0, "append_exact: negative strides (%lld, %lld)", (long long)stride_b,
+                    (long long)stride_h);
     ODMKV_CHECK_ARG(store->kexact && store->vexact && store->seg_tile[4] && store->seg_count[4] && store->pos[4],
                     "append_exact: store has no exact segments");
     hipLaunchKernelGGL(append_exact_kernel, dim3(store->B * store->Hkv), dim3(128), 0, (hipStream_t)stream,
-                       *store, (const uint16_t*)k, (const uint16_t*)v, pos);
+                       *store, (const uint16_t*)k, (const uint16_t*)v, stride_b, stride_h, pos);
     ODMKV_CHECK_LAUNCH("append_exact_kernel");
     return 0;
 }

@@ -58,7 +58,7 @@ def _load() -> C.CDLL:
         "odmkv_quantize_rows": (C.c_int, [vp, i32, i64, i64, i32, vp, vp, vp, vp, vp]),
         "odmkv_dequantize_rows": (C.c_int, [vp, vp, i64, i32, vp, vp, vp, vp]),
         "odmkv_dequant": (C.c_int, [C.POINTER(Packed), vp, vp, i32, i32, i64, i64, i64, vp, vp, vp, i32, vp]),
-        "odmkv_append_exact": (C.c_int, [C.POINTER(Packed), vp, vp, i32, vp]),
+        "odmkv_append_exact": (C.c_int, [C.POINTER(Packed), vp, vp, i64, i64, i32, vp]),
         "odmkv_decode_workspace_bytes": (sz, [i32, i32, i32]),
         "odmkv_decode_attn": (C.c_int, [vp, i32, i32, f32, C.POINTER(Packed), vp, i32, vp, vp, vp, vp, vp,
                                         C.POINTER(C.c_float), C.POINTER(C.c_float), vp, vp, vp, sz, vp]),

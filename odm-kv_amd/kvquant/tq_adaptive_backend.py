@@ -133,7 +133,8 @@ class TurboQuantAdaptiveKVCacheState:
         need = self.seq_len + T
         if self._level_store is None or self._level_store.shape[2] < need:
             cap = max(need, 2 * (0 if self._level_store is None else self._level_store.shape[2]), 256)
-            grown = torch.empty(B, H, cap, dtype=torch.uint8, device=self.device)
+            # positions behind seq_len read 16, so that a single exact token needs no write
+            grown = torch.full((B, H, cap), 16, dtype=torch.uint8, device=self.device)
             if self._level_store is not None and self.seq_len:
                 grown[:, :, :self.seq_len] = self._level_store[:, :, :self.seq_len]
             self._level_store = grown
@@ -345,16 +346,17 @@ class TurboQuantAdaptiveKVCacheState:
         new_counts[4] += 1
         had = self._seg_tile
         self._ensure_capacity(new_counts)
-        k = keys.reshape(B, H, D).contiguous()
-        v = values.reshape(B, H, D).contiguous()
-        _lib.check(lib.odmkv_append_exact(C.byref(self._packed), k.data_ptr(), v.data_ptr(), self.seq_len,
-                                          _lib.stream_ptr(self.device)))
+        # the token is read where it lies (the newest row of the model's cache): no staging copies
+        k, v = keys[:, :, 0, :], values[:, :, 0, :]
+        if k.stride(2) != 1 or v.stride() != k.stride():
+            k, v = k.contiguous(), v.contiguous()
+        _lib.check(lib.odmkv_append_exact(C.byref(self._packed), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1),
+                                          self.seq_len, _lib.stream_ptr(self.device)))
         self._counts = new_counts
-        need = self.seq_len + 1
-        if self._level_store.shape[2] < need:
+        if self._level_store.shape[2] < self.seq_len + 1:
             self._extend_levels(torch.full((B, H, 1), 16, dtype=torch.uint8, device=self.device))
-        else:
-            self._level_store[:, :, self.seq_len:need].fill_(16)       # an exact token: the evicted set does not change
+        # otherwise nothing to write: the level store reads 16 behind seq_len (an exact token leaves
+        # the evicted set as it is)
         self.seq_len += 1
         if had is not self._seg_tile:
             self._items = None
@@ -363,6 +365,7 @@ class TurboQuantAdaptiveKVCacheState:
         seq_len = int(seq_len)
         if seq_len >= self.seq_len:
             return
+        self._level_store[:, :, seq_len:self.seq_len].fill_(16)       # the store reads 16 behind seq_len
         self.seq_len = seq_len
         self._masked = None
         # positions ascend inside a segment, so the survivors are a prefix of it
