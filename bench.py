@@ -170,6 +170,20 @@ def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
         torch.cuda.synchronize()
         out["prefill_s_without_press"] = round(time.perf_counter() - t0, 3)
     del cache
+    # what the model itself costs per decode step: no press, a 16-token context (attention is negligible)
+    cache = DynamicCache()
+    with torch.inference_mode():
+        tok = model(input_ids=ids[:, :16], past_key_values=cache).logits[0, -1].argmax().view(1, 1)
+        steps = []
+        for step in range(24):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            tok = model(input_ids=tok, past_key_values=cache,
+                        position_ids=torch.tensor([[16 + step]], device=dev)).logits[0, -1].argmax().view(1, 1)
+            torch.cuda.synchronize()
+            steps.append(time.perf_counter() - t0)
+        out["decode_step_ms_model_alone_short_context"] = round(statistics.median(steps[4:]) * 1e3, 3)
+    del cache
     same = 0
     for x, y in zip(tokens["fused"], tokens["dense"]):      # greedy tokens agree until the first near-tie
         if x != y:

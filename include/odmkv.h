@@ -180,7 +180,8 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  *   out[b,q] = sum_t softmax_t( scaling * q[b,q] . Khat[b,q/G,t] ) Vhat[b,q/G,t]
  * over the stored (non-evicted) tokens.  Evicted tokens are simply absent.
  *
- * q: device fp32 [B, Hq, 128].  items: device int32 [n_items, 8] work list, sorted by bh:
+ * q: device [B, Hq, 128] of q_dtype (ODMKV_F16 / ODMKV_BF16 / ODMKV_F32), contiguous: the model's
+ * query states are passed as they are.  items: device int32 [n_items, 8] work list, sorted by bh:
  * (bh, level index 0..4, first tile, tile count, tokens held by those tiles, first tile of the
  * segment, 0, 0); for the exact level (index 4) the token count is read from seg_count instead,
  * so that tokens appended since the list was built are seen.  item_range: device int32
@@ -189,7 +190,8 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  * dispatch_order: device int32 [n_items], a permutation of the items in the order the workgroups
  * should take them (longest first, when there are more items than compute units), or NULL for the
  * list's own order.
- * out: device fp32 [B, Hq, 128]; lse: device fp32 [B, Hq] or NULL (log-sum-exp of the scaled logits).
+ * out: device [B, Hq, 128] of out_dtype (accumulated in fp32, rounded once on the store);
+ * lse: device fp32 [B, Hq] or NULL (log-sum-exp of the scaled logits).
  * pi_k_t is the key rotation TRANSPOSED (row-major [128,128] of Pi_k^T), pi_v the value rotation as is.
  * The query is rounded to fp16 on entry (the attention being replaced receives it in the model's
  * fp16/bf16).  The centroid tables live in LDS as fp16; to keep their rounding out of the result,
@@ -200,13 +202,13 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  */
 #define ODMKV_MAX_ITEMS_PER_SEGMENT 1024
 size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);
-int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
+int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
                       const odmkv_packed_t* store,
                       const int32_t* items, int n_items, const int32_t* item_range,
                       const int32_t* dispatch_order,
                       const float* pi_k_t, const float* pi_v, const float* codebooks,
                       const float* codebooks_host, const float* inv_scales,
-                      float* out, float* lse, void* workspace, size_t workspace_bytes,
+                      void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                       void* stream);
 
 /* ---------------------------------------------------------------------------------------------

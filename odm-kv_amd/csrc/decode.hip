@@ -50,7 +50,8 @@ extern "C" int odmkv_debug_read_trace(unsigned long long* host, int n) {
 
 struct DecodeArgs {
     odmkv_packed_t s;
-    const float* q;
+    const void* q;
+    int q_dt, out_dt;   // element types of q and out (ODMKV_F16 / BF16 / F32)
     int Hq, G, B;
     float scaling;
     const int32_t* items;
@@ -65,7 +66,7 @@ struct DecodeArgs {
     float cbs[28];    // scaled centroids of widths 2, 3, 4 (kept in scalar registers; 8-bit ones stay in memory)
     int gp;           // head slots per item in `partial`: 4 or 8
     float* partial;   // [n_items, gp, PSTRIDE]
-    float* out;
+    void* out;
     float* lse;
 };
 
@@ -86,7 +87,11 @@ __global__ __launch_bounds__(128 * PREP_SLICES) void decode_prep_kernel(DecodeAr
     for (int jj = 0; jj < JN; ++jj) pk[jj] = a.pi_k_t[(size_t)(slice * JN + jj) * HD + i];
     if (slice == 0) {
         // the query is consumed at fp16 precision, like the attention it replaces (model dtype)
-        const __half q16 = __float2half_rn(a.q[(size_t)bq * HD + i]);
+        const size_t qi = (size_t)bq * HD + i;
+        const float qf = a.q_dt == ODMKV_F32 ? reinterpret_cast<const float*>(a.q)[qi]
+                       : a.q_dt == ODMKV_F16 ? Elem<ODMKV_F16>::to_f32(reinterpret_cast<const uint16_t*>(a.q)[qi])
+                                             : Elem<ODMKV_BF16>::to_f32(reinterpret_cast<const uint16_t*>(a.q)[qi]);
+        const __half q16 = __float2half_rn(qf);
         qsh[i] = __half2float(q16);
         uint16_t* qs16 = reinterpret_cast<uint16_t*>(a.qs + (size_t)bq * 32);
         qs16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(q16);
@@ -741,7 +746,11 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
 #pragma unroll
         for (int s = 0; s < MERGE_SLICES; ++s) tot += part[0][s][tid] + part[1][s][tid];
         const float L = Lsh;
-        a.out[(size_t)bq * HD + tid] = L > 0.0f ? tot / L : 0.0f;
+        const float o32 = L > 0.0f ? tot / L : 0.0f;
+        const size_t oi = (size_t)bq * HD + tid;
+        if (a.out_dt == ODMKV_F32) reinterpret_cast<float*>(a.out)[oi] = o32;
+        else if (a.out_dt == ODMKV_F16) reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_F16>::from_f32(o32);
+        else reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_BF16>::from_f32(o32);
         if (a.lse && tid == 0) a.lse[bq] = L > 0.0f ? (M + __log2f(L)) * LN2 : -INFINITY;
     }
 }
@@ -815,14 +824,16 @@ extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     return 2 * q + align_up((size_t)n_items * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
 }
 
-extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
+extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
                                  const odmkv_packed_t* store,
                                  const int32_t* items, int n_items, const int32_t* item_range,
                                  const int32_t* dispatch_order,
                                  const float* pi_k_t, const float* pi_v, const float* codebooks,
                                  const float* codebooks_host, const float* inv_scales,
-                                 float* out, float* lse, void* workspace, size_t workspace_bytes,
+                                 void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                                  void* stream) {
+    ODMKV_CHECK_ARG(q_dtype == ODMKV_F16 || q_dtype == ODMKV_BF16 || q_dtype == ODMKV_F32, "decode_attn: bad query dtype %d", q_dtype);
+    ODMKV_CHECK_ARG(out_dtype == ODMKV_F16 || out_dtype == ODMKV_BF16 || out_dtype == ODMKV_F32, "decode_attn: bad output dtype %d", out_dtype);
     ODMKV_CHECK_ARG(codebooks_host != nullptr, "decode_attn: null host copy of the centroid tables");
     ODMKV_CHECK_ARG(inv_scales != nullptr, "decode_attn: null table scales");
     ODMKV_CHECK_ARG(q && store && item_range && pi_k_t && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
@@ -837,7 +848,7 @@ extern "C" int odmkv_decode_attn(const float* q, int B, int Hq, float scaling,
     ODMKV_CHECK_ARG(workspace_bytes >= odmkv_decode_workspace_bytes(B, Hq, n_items), "decode_attn: workspace too small");
     hipStream_t st = (hipStream_t)stream;
     DecodeArgs a;
-    a.s = *store; a.q = q; a.Hq = Hq; a.G = G; a.B = B; a.scaling = scaling;
+    a.s = *store; a.q = q; a.q_dt = q_dtype; a.out_dt = out_dtype; a.Hq = Hq; a.G = G; a.B = B; a.scaling = scaling;
     a.items = items; a.item_range = item_range; a.order = dispatch_order;
     a.pi_k_t = pi_k_t; a.pi_v = pi_v; a.cb = codebooks;
     for (int w = 0; w < 4; ++w) a.inv_s[w] = inv_scales[w];

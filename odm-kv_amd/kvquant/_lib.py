@@ -60,8 +60,8 @@ def _load() -> C.CDLL:
         "odmkv_dequant": (C.c_int, [C.POINTER(Packed), vp, vp, i32, i32, i64, i64, i64, vp, vp, vp, i32, vp]),
         "odmkv_append_exact": (C.c_int, [C.POINTER(Packed), vp, vp, i64, i64, i32, vp]),
         "odmkv_decode_workspace_bytes": (sz, [i32, i32, i32]),
-        "odmkv_decode_attn": (C.c_int, [vp, i32, i32, f32, C.POINTER(Packed), vp, i32, vp, vp, vp, vp, vp,
-                                        C.POINTER(C.c_float), C.POINTER(C.c_float), vp, vp, vp, sz, vp]),
+        "odmkv_decode_attn": (C.c_int, [vp, i32, i32, i32, f32, C.POINTER(Packed), vp, i32, vp, vp, vp, vp, vp,
+                                        C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp, sz, vp]),
         "odmkv_profile_enable": (C.c_int, [i32]),
         "odmkv_profile_collect": (C.c_int, [C.POINTER(C.c_float), i32, C.POINTER(C.c_int)]),
         "odmkv_profile_disable": (C.c_int, []),

@@ -64,7 +64,7 @@ def _fused_decode(module, query, key, value, attention_mask, dropout, kwargs):
         # press's hook sees the store already in step and does not append it again
         state.append_all_exact(key[:, :, -1:, :], value[:, :, -1:, :])
     if state.seq_len == k_len:
-        out = state.decode_attention(query, scaling=scaling)
+        return state.decode_attention(query, scaling=scaling, out_dtype=query.dtype).view(B, 1, Hq, D)
     else:
         # merge the newest (still dense) token with the store's partial result by log-sum-exp
         out, lse = state.decode_attention(query, scaling=scaling, return_lse=True)

@@ -575,14 +575,18 @@ class TurboQuantAdaptiveKVCacheState:
         self._item_order = order
 
     def decode_attention(self, query: torch.Tensor, scaling: Optional[float] = None,
-                         return_lse: bool = False):
+                         return_lse: bool = False, out_dtype: torch.dtype = torch.float32):
         """softmax(scaling * q K^T) V over the stored tokens, for one query token per sequence.
 
-        query: [B, Hq, D] or [B, Hq, 1, D] on the GPU; returns fp32 [B, Hq, D] (and lse [B, Hq])."""
+        query: [B, Hq, D] or [B, Hq, 1, D] on the GPU, fp16 / bf16 / fp32 (read as it is); returns
+        [B, Hq, D] of `out_dtype` (accumulated in fp32, rounded once) and, on request, lse fp32 [B, Hq]."""
         _lib.require_gpu(query, "query")
         if self._bufs is None:
             raise ValueError("the store is empty")
-        q = query.reshape(query.shape[0], query.shape[1], self.head_dim).float().contiguous()
+        q = query.reshape(query.shape[0], query.shape[1], self.head_dim)
+        if q.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+            q = q.float()
+        q = q.contiguous()
         B, Hq, D = q.shape
         if B != self.batch_size or Hq % self.num_heads != 0:
             raise ValueError(f"query heads {tuple(q.shape)} do not match the store (B={self.batch_size}, Hkv={self.num_heads})")
@@ -590,12 +594,13 @@ class TurboQuantAdaptiveKVCacheState:
             self._build_items()
         items, ranges, n_items = self._items
         scale = 1.0 / math.sqrt(D) if scaling is None else float(scaling)
-        out = torch.empty(B, Hq, D, dtype=torch.float32, device=self.device)
+        out = torch.empty(B, Hq, D, dtype=out_dtype, device=self.device)
         lse = torch.empty(B, Hq, dtype=torch.float32, device=self.device) if return_lse else None
         ws_bytes = lib.odmkv_decode_workspace_bytes(B, Hq, n_items)
         ws = _lib.workspace(self.device, ws_bytes, "decode")
         _lib.check(lib.odmkv_decode_attn(
-            q.data_ptr(), B, Hq, scale, C.byref(self._packed), items.data_ptr(), n_items,
+            q.data_ptr(), _lib.dtype_code(q), B, Hq, scale, C.byref(self._packed), items.data_ptr(), n_items,
             ranges.data_ptr(), _lib.ptr(self._item_order), self._pi_k_t.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
-            self._decode_cb_host, self._decode_inv, out.data_ptr(), _lib.ptr(lse), ws.data_ptr(), ws_bytes, _lib.stream_ptr(self.device)))
+            self._decode_cb_host, self._decode_inv, out.data_ptr(), _lib.dtype_code(out), _lib.ptr(lse), ws.data_ptr(), ws_bytes,
+            _lib.stream_ptr(self.device)))
         return (out, lse) if return_lse else out

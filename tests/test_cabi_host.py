@@ -59,9 +59,12 @@ def test_argument_checks_without_a_gpu(lib):
     # unsupported width
     rc = lib.odmkv_quantize_rows(p, 0, C.c_int64(4), C.c_int64(128), 5, p, p, p, p, None)
     assert rc == -1 and b"width" in lib.odmkv_last_error()
-    rc = lib.odmkv_decode_attn(None, 1, 8, C.c_float(1.0), None, None, 0, None, None, None, None, None, None, None,
-                               None, None, None, C.c_size_t(0), None)
+    rc = lib.odmkv_decode_attn(None, 2, 1, 8, C.c_float(1.0), None, None, 0, None, None, None, None, None, None, None,
+                               None, 2, None, None, C.c_size_t(0), None)
     assert rc == -1
+    rc = lib.odmkv_decode_attn(p, 7, 1, 8, C.c_float(1.0), None, None, 0, None, None, None, None, None, None, None,
+                               p, 2, None, None, C.c_size_t(0), None)
+    assert rc == -1 and b"query dtype" in lib.odmkv_last_error()
 
 
 def test_host_modules_import_and_validate():

@@ -195,3 +195,23 @@ def test_config1_end_to_end():
     st, ref = _pair(L.keys[None], L.values[None], bits[None].cpu())
     got = st.decode_attention(L.query[None].to(DEV))
     assert rel_err(got.cpu(), decode_attention_state(L.query[None], ref)) < ATTN_RTOL
+
+
+def test_decode_reads_and_writes_the_model_dtype():
+    """The query is taken in fp16 / bf16 / fp32 as it is and the output rounded once to the requested
+    type: the same numbers as the fp32 call on the same query values."""
+    g = torch.Generator().manual_seed(77)
+    B, Hkv, G, T = 2, 2, 4, 500
+    k = torch.randn(B, Hkv, T, 128, generator=g).half()
+    v = torch.randn(B, Hkv, T, 128, generator=g).half()
+    bits = _rand_bits(g, (B, Hkv, T), (0.2, 0.4, 0.15, 0.1, 0.05, 0.1))
+    bits[..., :4] = 16
+    st, ref = _pair(k, v, bits)
+    q32 = torch.randn(B, Hkv * G, 128, generator=g)
+    for qdt in (torch.float16, torch.bfloat16):
+        q = q32.to(qdt).to(DEV)
+        base = st.decode_attention(q.float())                       # fp32 in, fp32 out
+        assert rel_err(base.cpu(), decode_attention_state(q.float().cpu(), ref)) < ATTN_RTOL
+        for odt in (torch.float32, torch.float16, torch.bfloat16):
+            got = st.decode_attention(q.view(B, Hkv * G, 1, 128), out_dtype=odt)
+            assert got.dtype == odt and torch.equal(got, base.to(odt)), (qdt, odt)
