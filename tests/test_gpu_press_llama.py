@@ -266,3 +266,29 @@ def test_released_dense_cache_with_a_batch_of_two():
         assert cache.get_seq_length() == 400 + forced.shape[0]
         runs.append(torch.stack(logits))
     assert torch.equal(runs[0], runs[1])
+
+
+@torch.inference_mode()
+def test_released_dense_cache_without_a_decode_buffer():
+    """buffer_size=0: every decoded token is scored and quantised in the hook; the attention call
+    merges the still-dense newest token with the store's partial result.  Same logits with and
+    without the dense copy."""
+    from transformers import DynamicCache
+    model = _model(7)
+    ids = _ids(350, 41)
+    forced = torch.randint(0, 1000, (10,), generator=torch.Generator().manual_seed(42)).to(DEV)
+    runs = []
+    for release in (False, True):
+        cache, logits = DynamicCache(), []
+        press = _press(buffer_size=0, release_dense_cache=release)
+        with press(model):
+            model.model(input_ids=ids, past_key_values=cache)
+            for step in range(forced.shape[0]):
+                out = model(input_ids=forced[step].view(1, 1), past_key_values=cache,
+                            position_ids=torch.tensor([[350 + step]], device=DEV))
+                logits.append(out.logits[0, -1].float())
+            assert all(st.seq_len == 350 + forced.shape[0] for st in press._states.values())
+            lm = press._states[0]._level_map[0].cpu()
+            assert (lm[:, 350:] != 16).any()                   # decoded tokens were quantised, not buffered
+        runs.append(torch.stack(logits))
+    assert torch.equal(runs[0], runs[1])
