@@ -292,3 +292,16 @@ def test_released_dense_cache_without_a_decode_buffer():
             assert (lm[:, 350:] != 16).any()                   # decoded tokens were quantised, not buffered
         runs.append(torch.stack(logits))
     assert torch.equal(runs[0], runs[1])
+
+
+def test_bf16_model_fused_matches_dense_path():
+    """The same comparison on a bf16 model (exact tokens are then stored as bf16): logits are O(1) and one
+    bf16 step near 2 is 0.016, so a few steps of difference between the two attention paths are expected."""
+    model = _model(8).to(torch.bfloat16)
+    ids = _ids(600, 51)
+    n_new = 140                                   # crosses one buffer flush
+    tok_d, log_d, _, _ = _generate(model, _press(), ids, n_new, fused=False)
+    tok_f, log_f, _, states = _generate(model, _press(), ids, n_new, forced=tok_d, fused=True)
+    assert states[0]._exact_torch_dtype == torch.bfloat16
+    assert (log_f - log_d).abs().max().item() < 0.06
+    assert (log_f.argmax(-1) == tok_d).float().mean().item() >= 0.95
