@@ -9,7 +9,7 @@ WIDTHS = (2, 3, 4, 8)
 def _bits_to_codes(byte_rows: np.ndarray, w: int) -> np.ndarray:
     """[..., nbytes] little-endian bit streams -> [..., nbytes*8/w] codes."""
     bits = np.unpackbits(byte_rows, axis=-1, bitorder="little")
-    bits = bits.reshape(bits.shape[:-1] + (-1, w)).astype(np.uint16)
+    bits = bits.reshape(bits.shape[:-1] + (bits.shape[-1] // w, w)).astype(np.uint16)     # also for zero rows
     return (bits << np.arange(w, dtype=np.uint16)).sum(axis=-1).astype(np.uint8)
 
 
