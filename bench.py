@@ -130,12 +130,14 @@ def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
         cache = DynamicCache()
         with torch.inference_mode(), press(model):
             torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
             t0 = time.perf_counter()
             h = model.model(input_ids=ids, past_key_values=cache).last_hidden_state[:, -1:, :]
             tok = model.lm_head(h)[0, -1].argmax().view(1, 1)
             torch.cuda.synchronize()
             t_prefill = time.perf_counter() - t0
             del h
+            peak_bytes = torch.cuda.max_memory_allocated() - base_bytes   # activations + caches at the prefill's peak
             cache_bytes = torch.cuda.memory_allocated() - base_bytes      # packed stores + what the HF cache holds
             print(f"[press-e2e] {mode}: prefill of {T} tokens {t_prefill:.2f} s", file=sys.stderr, flush=True)
             steps, emitted = [], [int(tok)]
@@ -154,7 +156,8 @@ def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
         out[mode] = {"prefill_s": round(t_prefill, 3), "decode_step_ms_median": round(statistics.median(steps[4:]) * 1e3, 3),
                      "decode_step_ms_min": round(min(steps[4:]) * 1e3, 3),
                      "decode_step_ms_mean_with_flushes": round(statistics.fmean(steps[4:]) * 1e3, 3),
-                     "attention_calls": took, "cache_bytes_after_prefill": int(cache_bytes)}
+                     "attention_calls": took, "cache_bytes_after_prefill": int(cache_bytes),
+                     "prefill_peak_bytes_over_model": int(peak_bytes)}
         del cache, press
         for layer in model.model.layers:                     # the modules keep their last store attached
             layer.self_attn._odmkv_state = None

@@ -194,6 +194,11 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         return bits
 
     # ------------------------------------------------------------------ prefill
+    def _finalize_each_layer(self) -> bool:
+        # with the dense copy released there is a reason not to wait for the last layer: each layer's
+        # fp16 keys and values are freed while the prefill of the layers above it is still running
+        return self.layerwise and self.release_dense_cache
+
     def _finalize_prefill(self, cache) -> None:
         if self.n_outlier_channels > 0:
             raise NotImplementedError("outlier-channel separation is not built (n_outlier_channels must be 0)")

@@ -302,8 +302,14 @@ class TurboQuantPerTokenPress:
             self._prefill_hooks_fired += 1
         self._prefill_scores[layer_idx] = torch.stack(layer_scores, dim=0)
         self._prefill_sink_masks[layer_idx] = self._build_sink_mask(keys.shape[1], keys.shape[2], keys.device)
-        if self._last_hooked_layer_idx is None or layer_idx == self._last_hooked_layer_idx:
+        if (self._last_hooked_layer_idx is None or layer_idx == self._last_hooked_layer_idx
+                or self._finalize_each_layer()):
             self._finalize_prefill(cache)
+
+    def _finalize_each_layer(self) -> bool:
+        """Whether a layer's prefill is allocated and stored as soon as its own hook has fired
+        (possible when layers have independent budgets) instead of after the last layer's."""
+        return False
 
     def _forward_hook(self, module: nn.Module, args, kwargs, output):
         cache, hidden_states = self._hook_inputs(module, args, kwargs)
