@@ -189,6 +189,7 @@ def _session(model, press, ids, forced, question):
             out = model(input_ids=tok.view(1, 1), past_key_values=cache, position_ids=torch.tensor([[pos]], device=DEV))
             logits.append(out.logits[0, -1].float())
             pos += 1
+        levels_after_decode = {l: st._level_map.clone() for l, st in press._states.items()}
         mid_layers = [type(layer).__name__ for layer in cache.layers]
         mid_strides = [layer.keys.stride(2) for layer in cache.layers]
         q = question.view(1, -1)
@@ -208,7 +209,7 @@ def _session(model, press, ids, forced, question):
         assert all(st.seq_len == pos for st in press._states.values())
         out = model(input_ids=forced[0].view(1, 1), past_key_values=cache, position_ids=torch.tensor([[pos]], device=DEV))
         logits.append(out.logits[0, -1].float())
-    return torch.stack(logits), cache, mid_layers, mid_strides
+    return torch.stack(logits), cache, mid_layers, mid_strides, levels_after_decode
 
 
 def test_released_dense_cache_decodes_identically():
@@ -221,8 +222,10 @@ def test_released_dense_cache_decodes_identically():
     g = torch.Generator().manual_seed(22)
     forced = torch.randint(0, 1000, (140,), generator=g).to(DEV)          # crosses one buffer flush
     question = torch.randint(0, 1000, (5,), generator=g).to(DEV)
-    keep, cache_k, layers_k, strides_k = _session(model, _press(), ids, forced, question)
-    rel, cache_r, layers_r, strides_r = _session(model, _press(release_dense_cache=True), ids, forced, question)
+    keep, cache_k, layers_k, strides_k, levels_k = _session(model, _press(), ids, forced, question)
+    rel, cache_r, layers_r, strides_r, levels_r = _session(model, _press(release_dense_cache=True), ids, forced, question)
+    # the released press stores each layer as its own hook fires, the other after the last layer: same levels
+    assert levels_k.keys() == levels_r.keys() and all(torch.equal(levels_k[l], levels_r[l]) for l in levels_k)
     assert layers_k == ["DynamicLayer"] * 2 and all(s != 0 for s in strides_k)
     assert layers_r == ["PackedCacheLayer"] * 2 and strides_r == [0, 0]
     n_single = 1 + forced.shape[0]
