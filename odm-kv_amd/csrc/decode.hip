@@ -641,6 +641,9 @@ __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs 
 // ------------------------------------------------------------------------------------------------
 #define MERGE_THREADS 512
 #define MERGE_SLICES (MERGE_THREADS / HD)
+#ifndef MERGE_SPLIT
+#define MERGE_SPLIT 4
+#endif
 #define MERGE_MAX_ITEMS ODMKV_MAX_ITEMS_PER_SEGMENT
 
 template <int GP>
@@ -650,16 +653,23 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
     __shared__ float part[2][MERGE_SLICES][HD];      // [rotated | exact][slice][dim]
     __shared__ float rot[HD];
     __shared__ float Lsh;
-    const int bq = blockIdx.x, tid = threadIdx.x, j = tid & (HD - 1), slice = tid >> 7;
+    // MERGE_SPLIT workgroups per query head: each merges the head's partial results in full (they are small and
+    // shared through the caches) and rotates back a quarter of the output dims, so that no workgroup has to pull
+    // the whole 64 KB rotation through one compute unit
+    const int bq = blockIdx.x / MERGE_SPLIT, quarter = blockIdx.x % MERGE_SPLIT;
+    const int tid = threadIdx.x, j = tid & (HD - 1), slice = tid >> 7;
     const int b = bq / a.Hq, hq = bq % a.Hq;
     const int bh = b * a.s.Hkv + hq / a.G, g = hq % a.G;
     const int i0 = a.item_range[bh], n = min(a.item_range[bh + 1] - i0, MERGE_MAX_ITEMS);
     // Everything that does not depend on the weights is requested now, in one round trip: this thread's
     // share of the value rotation, the first MERGE_PRE accumulator values of its slice, its item's (m, l, level)
-    constexpr int IN = HD / MERGE_SLICES;
+    constexpr int QD = HD / MERGE_SPLIT;                 // output dims of this workgroup
+    constexpr int RS = MERGE_THREADS / QD;                // row slices of the rotation
+    constexpr int IN = HD / RS;                           // rows per slice
+    const int jj = tid % QD, rs = tid / QD;
     float pv[IN];
 #pragma unroll
-    for (int ii = 0; ii < IN; ++ii) pv[ii] = a.pi_v[(size_t)(slice * IN + ii) * HD + j];
+    for (int ii = 0; ii < IN; ++ii) pv[ii] = a.pi_v[(size_t)(rs * IN + ii) * HD + quarter * QD + jj];
     constexpr int MERGE_PRE = 16;
     float pre[MERGE_PRE];
 #pragma unroll
@@ -734,24 +744,28 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
         rot[tid] = r;
     }
     __syncthreads();
-    // rotate the quantised part back: out_j = sum_i rot_i Pi_v[i][j]; the slices split the i range
+    // rotate the quantised part back: out_j = sum_i rot_i Pi_v[i][j] for this workgroup's dims; the slices split the i range
     float o = 0.0f;
 #pragma unroll
-    for (int ii = 0; ii < IN; ++ii) o = __fmaf_rn(rot[slice * IN + ii], pv[ii], o);
+    for (int ii = 0; ii < IN; ++ii) o = __fmaf_rn(rot[rs * IN + ii], pv[ii], o);
     __syncthreads();
-    part[0][slice][j] = o;
+    float* part2 = &part[0][0][0];                        // [RS][QD], the first half of `part` is free again
+    part2[rs * QD + jj] = o;
     __syncthreads();
-    if (tid < HD) {
+    if (tid < QD) {
+        const int dim = quarter * QD + tid;
         float tot = 0.0f;
 #pragma unroll
-        for (int s = 0; s < MERGE_SLICES; ++s) tot += part[0][s][tid] + part[1][s][tid];
+        for (int r = 0; r < RS; ++r) tot += part2[r * QD + tid];
+#pragma unroll
+        for (int s = 0; s < MERGE_SLICES; ++s) tot += part[1][s][dim];
         const float L = Lsh;
         const float o32 = L > 0.0f ? tot / L : 0.0f;
-        const size_t oi = (size_t)bq * HD + tid;
+        const size_t oi = (size_t)bq * HD + dim;
         if (a.out_dt == ODMKV_F32) reinterpret_cast<float*>(a.out)[oi] = o32;
         else if (a.out_dt == ODMKV_F16) reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_F16>::from_f32(o32);
         else reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_BF16>::from_f32(o32);
-        if (a.lse && tid == 0) a.lse[bq] = L > 0.0f ? (M + __log2f(L)) * LN2 : -INFINITY;
+        if (a.lse && tid == 0 && quarter == 0) a.lse[bq] = L > 0.0f ? (M + __log2f(L)) * LN2 : -INFINITY;
     }
 }
 
@@ -879,8 +893,8 @@ extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, floa
         if (rec) ++g_prof_used;
     }
     if (g_stage_mask & 4) {
-        if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);
-        else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq), dim3(MERGE_THREADS), 0, st, a);
+        if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq * MERGE_SPLIT), dim3(MERGE_THREADS), 0, st, a);
+        else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq * MERGE_SPLIT), dim3(MERGE_THREADS), 0, st, a);
         ODMKV_CHECK_LAUNCH("decode_merge_kernel");
     }
     return 0;
