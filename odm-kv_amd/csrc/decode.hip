@@ -75,39 +75,48 @@ struct DecodeArgs {
 // ------------------------------------------------------------------------------------------------
 __device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
 
-#define PREP_SLICES 4
-__global__ __launch_bounds__(128 * PREP_SLICES) void decode_prep_kernel(DecodeArgs a) {
+#ifndef PREP_SPLIT
+#define PREP_SPLIT 4                       // workgroups per query head, each producing HD / PREP_SPLIT rotated dims
+#endif
+#define PREP_THREADS 512
+__global__ __launch_bounds__(PREP_THREADS) void decode_prep_kernel(DecodeArgs a) {
+    constexpr int QD = HD / PREP_SPLIT;     // rotated dims of this workgroup
+    constexpr int JS = PREP_THREADS / QD;   // slices of the sum over j
+    constexpr int JN = HD / JS;             // terms per slice
     __shared__ float qsh[HD];
-    __shared__ float part[PREP_SLICES][HD];
-    const int bq = blockIdx.x, i = threadIdx.x & (HD - 1), slice = threadIdx.x >> 7;
-    // this thread's 32 elements of column i of Pi_k (rows of the transposed matrix): all requested at once
-    constexpr int JN = HD / PREP_SLICES;
+    __shared__ float part[JS][QD];
+    const int bq = blockIdx.x / PREP_SPLIT, quarter = blockIdx.x % PREP_SPLIT, tid = threadIdx.x;
+    const int ii = tid % QD, js = tid / QD, i = quarter * QD + ii;
+    // this thread's JN elements of column i of Pi_k (rows of the transposed matrix): all requested at once.
+    // No workgroup pulls the whole 64 KB matrix through one compute unit.
     float pk[JN];
 #pragma unroll
-    for (int jj = 0; jj < JN; ++jj) pk[jj] = a.pi_k_t[(size_t)(slice * JN + jj) * HD + i];
-    if (slice == 0) {
+    for (int jj = 0; jj < JN; ++jj) pk[jj] = a.pi_k_t[(size_t)(js * JN + jj) * HD + i];
+    if (tid < HD) {
         // the query is consumed at fp16 precision, like the attention it replaces (model dtype)
-        const size_t qi = (size_t)bq * HD + i;
+        const size_t qi = (size_t)bq * HD + tid;
         const float qf = a.q_dt == ODMKV_F32 ? reinterpret_cast<const float*>(a.q)[qi]
                        : a.q_dt == ODMKV_F16 ? Elem<ODMKV_F16>::to_f32(reinterpret_cast<const uint16_t*>(a.q)[qi])
                                              : Elem<ODMKV_BF16>::to_f32(reinterpret_cast<const uint16_t*>(a.q)[qi]);
         const __half q16 = __float2half_rn(qf);
-        qsh[i] = __half2float(q16);
-        uint16_t* qs16 = reinterpret_cast<uint16_t*>(a.qs + (size_t)bq * 32);
-        qs16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(q16);
-        qs16[(i >> 2) * 8 + 4 + (i & 3)] = 0;
+        qsh[tid] = __half2float(q16);
+        if (tid / QD == quarter) {           // the un-rotated copy (for exact tiles): every workgroup writes its own dims
+            uint16_t* qs16 = reinterpret_cast<uint16_t*>(a.qs + (size_t)bq * 32);
+            qs16[(tid >> 2) * 8 + (tid & 3)] = __half_as_ushort(q16);
+            qs16[(tid >> 2) * 8 + 4 + (tid & 3)] = 0;
+        }
     }
     __syncthreads();
-    // q'_i = sum_j Pi_k[i][j] q_j: every slice sums its quarter of j in order, the quarters are added in order
+    // q'_i = sum_j Pi_k[i][j] q_j: every slice sums its share of j in order, the slices are added in order
     float acc = 0.0f;
 #pragma unroll
-    for (int jj = 0; jj < JN; ++jj) acc = __fmaf_rn(pk[jj], qsh[slice * JN + jj], acc);
-    part[slice][i] = acc;
+    for (int jj = 0; jj < JN; ++jj) acc = __fmaf_rn(pk[jj], qsh[js * JN + jj], acc);
+    part[js][ii] = acc;
     __syncthreads();
-    if (slice == 0) {
-        float tot = part[0][i];
+    if (tid < QD) {
+        float tot = part[0][tid];
 #pragma unroll
-        for (int sl = 1; sl < PREP_SLICES; ++sl) tot += part[sl][i];
+        for (int sl = 1; sl < JS; ++sl) tot += part[sl][tid];
         uint16_t* qr16 = reinterpret_cast<uint16_t*>(a.qrot + (size_t)bq * 32);
         const __half hi = __float2half_rn(tot);
         qr16[(i >> 2) * 8 + (i & 3)] = __half_as_ushort(hi);
@@ -873,7 +882,7 @@ extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, floa
     a.partial = (float*)((char*)workspace + 2 * qbytes);
     a.out = out; a.lse = lse;
     if (g_stage_mask & 1) {
-        hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq), dim3(128 * PREP_SLICES), 0, st, a);
+        hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq * PREP_SPLIT), dim3(PREP_THREADS), 0, st, a);
         ODMKV_CHECK_LAUNCH("decode_prep_kernel");
     }
     const int GP = group_pad(G);
