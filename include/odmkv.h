@@ -60,6 +60,25 @@ int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int T,
                 const float* mu, int Hq, const float* attn, int n_sink, float eps,
                 float* scores, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Expected-attention score.  Replaces ExpectedAttentionScorer.score_prefill after the query
+ * statistics are known (kvquant/scorer.py:204-257):
+ *
+ *   logit[q,t] = mu[q] . K[h,t] / sqrt(d) + K[h,t]^T cov[q] K[h,t] / (2 d),   t >= n_sink, h = q / G
+ *   p[h,t]     = mean over the G query heads of softmax_t(logit[q,:])
+ *   s[h,t]     = use_vnorm ? (p[h,t] + eps) * |V[h,t]| : p[h,t]
+ *   s[h, 0..n_sink) = max over all (h, t >= n_sink) of s
+ *
+ * mu: device fp32 [Hq, 128]; cov: device fp32 [Hq, 128, 128] (the RoPE-averaged query covariance),
+ * or NULL for the mean-query term alone (use_covariance=False).  The quadratic form runs on the
+ * fp32 matrix cores.  K, V, strides, scores and the workspace (odmkv_score_workspace_bytes) are
+ * those of odmkv_score.
+ */
+int odmkv_score_expected(const void* K, const void* V, int dtype, int Hkv, int T,
+                         int64_t stride_h, int64_t stride_t,
+                         const float* mu, const float* cov, int Hq, int n_sink, float eps,
+                         int use_vnorm, float* scores, void* workspace, size_t workspace_bytes,
+                         void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Allocator.  Replaces optimal_scores_to_bits (kvquant/allocator.py:459-663) for a batch of
  * independent rows (one row = one (layer, sequence): the flattened [Hkv, T] scores).

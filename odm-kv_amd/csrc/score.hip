@@ -19,6 +19,8 @@ struct ScoreArgs {
     float eps;
     const float* mu;      // [Hq, 128]
     const float* attn;    // [Hkv, T] or null
+    const float* cov;     // [Hq, 128, 128] query covariance (expected-attention score only) or null
+    int use_vnorm;        // expected-attention score: multiply (p + eps) by |v|
     float* scores;        // [Hkv, T]
     float* logits;        // [Hq, Tc]
     float* kn2;           // [Hkv, Tc]
@@ -332,6 +334,188 @@ __global__ void score_pad_kernel(ScoreArgs a) {
     if (i < a.n_sink) a.scores[(size_t)h * a.T + i] = __uint_as_float(*a.gmax);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Expected-attention score (ExpectedAttentionScorer.score_prefill, kvquant/scorer.py:204-257):
+//
+//   logit[q,t] = mu[q] . k[t] / sqrt(d)  +  k[t]^T Cov[q] k[t] / (2 d)
+//   p[h,t]     = mean over the group of softmax_t(logit[q,:]);   s = (p + eps) * |v|   (or p alone)
+//
+// The quadratic form is a true dense contraction, [T,128] x [128,128] per query head, and runs on
+// the fp32 matrix cores (v_mfma_f32_32x32x2_f32): a wave takes 32 tokens, D = K . Cov/(2d) with the
+// accumulator preset to mu/sqrt(d) in every row, so that logit[t] = sum_c K[t][c] * D[t][c] holds
+// both terms.  Cov/(2d) stays in LDS (64 KB) for the workgroup's life; K is read from HBM by the
+// first head of a group and from the caches by the others.
+// ------------------------------------------------------------------------------------------------
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+#define EA_CHUNKS_PER_WG 2   // 256-token chunks a workgroup walks with one copy of the covariance
+
+// the 32 elements [32*blk, 32*blk+32) of a row, as raw registers; elem() picks one of them
+template <int DT> struct RowBlock;
+template <> struct RowBlock<ODMKV_F32> {
+    float4 r[8];
+    __device__ inline void load(const void* base, size_t off, int blk) {
+        const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + off + blk * 32);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = p[i];
+    }
+    // element 2*s + half of the block
+    __device__ inline float elem(int s, int half) const {
+        const float4 v = r[s >> 1];
+        const float lo = (s & 1) ? v.z : v.x, hi = (s & 1) ? v.w : v.y;
+        return half ? hi : lo;
+    }
+};
+template <int DT> struct RowBlock {
+    uint4 r[4];
+    __device__ inline void load(const void* base, size_t off, int blk) {
+        const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + off + blk * 32);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = p[i];
+    }
+    __device__ inline float elem(int s, int half) const {
+        const uint4 v = r[s >> 2];
+        const uint32_t w = (s & 3) == 0 ? v.x : (s & 3) == 1 ? v.y : (s & 3) == 2 ? v.z : v.w;
+        return Elem<DT>::to_f32((uint16_t)(half ? (w >> 16) : (w & 0xffffu)));
+    }
+};
+
+template <int DT>
+__device__ static inline float load_elem(const void* base, size_t off) {
+    if constexpr (DT == ODMKV_F32) return reinterpret_cast<const float*>(base)[off];
+    else return Elem<DT>::to_f32(reinterpret_cast<const uint16_t*>(base)[off]);
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void ea_logits_kernel(ScoreArgs a) {
+    extern __shared__ __align__(16) float cov_s[];      // [128][128], already divided by 2 d
+    __shared__ float red_m[4], red_s[4];
+    const int hq = blockIdx.y, h = hq / a.G, tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, col = lane & 31, half = lane >> 5;
+    {
+        const float4* src = reinterpret_cast<const float4*>(a.cov + (size_t)hq * HD * HD);
+        float4* dst = reinterpret_cast<float4*>(cov_s);
+        const float sc = 1.0f / (2.0f * HD);            // a power of two: exact
+        for (int e = tid; e < HD * HD / 4; e += 256) {
+            float4 v = src[e];
+            v.x *= sc; v.y *= sc; v.z *= sc; v.w *= sc;
+            dst[e] = v;
+        }
+    }
+    float mu_c[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) mu_c[cb] = a.mu[(size_t)hq * HD + cb * 32 + col] / 11.313708498984761f;
+    __syncthreads();
+    for (int cc = 0; cc < EA_CHUNKS_PER_WG; ++cc) {
+        const int chunk = blockIdx.x * EA_CHUNKS_PER_WG + cc;
+        if (chunk >= a.nchunks) break;                  // the same for every thread of the workgroup
+        float m = -INFINITY, s = 0.0f;
+        for (int sub = 0; sub < 2; ++sub) {
+            const int t0 = chunk * ROWS_PER_WG + (wave * 2 + sub) * 32;
+            if (t0 >= a.Tc) break;                      // wave-uniform
+            // operand A: lane = token t0 + col (rows past the end repeat the last row and are not stored)
+            const size_t arow = (size_t)h * a.sH + (size_t)(a.n_sink + min(t0 + col, a.Tc - 1)) * a.sT;
+            f32x16 acc[4];
+#pragma unroll
+            for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[cb][r] = mu_c[cb];
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk) {
+                RowBlock<DT> rb;
+                rb.load(a.K, arow, blk);
+#pragma unroll
+                for (int st = 0; st < 16; ++st) {
+                    const float av = rb.elem(st, half);
+                    const float* brow = cov_s + (blk * 32 + 2 * st + half) * HD + col;
+#pragma unroll
+                    for (int cb = 0; cb < 4; ++cb)
+                        acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, brow[cb * 32], acc[cb], 0, 0, 0);
+                }
+            }
+            // logit[row] = sum over columns of K[row][c] * D[row][c]; register r of a lane is row
+            // 8 (r / 4) + 4 half + r % 4, column 32 cb + col
+            float part[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = 8 * (r >> 2) + 4 * half + (r & 3);
+                const size_t off = (size_t)h * a.sH + (size_t)(a.n_sink + min(t0 + row, a.Tc - 1)) * a.sT + col;
+                float acc_r = 0.0f;
+#pragma unroll
+                for (int cb = 0; cb < 4; ++cb) acc_r = __fmaf_rn(load_elem<DT>(a.K, off + cb * 32), acc[cb][r], acc_r);
+                part[r] = acc_r;
+            }
+#pragma unroll
+            for (int o = 1; o < 32; o <<= 1)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) part[r] += __shfl_xor(part[r], o, WAVE);
+            // lanes col < 16 of either half own register r = col: 16 + 16 rows per wave
+            float mine = part[0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) mine = (col & 15) == r ? part[r] : mine;
+            const int rown = col & 15;
+            const int t = t0 + 8 * (rown >> 2) + 4 * half + (rown & 3);
+            if (col < 16 && t < a.Tc) {
+                a.logits[(size_t)hq * a.Tc + t] = mine;
+                ms_merge(m, s, mine, 1.0f);
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float m2 = __shfl_xor(m, o, WAVE), s2 = __shfl_xor(s, o, WAVE);
+            ms_merge(m, s, m2, s2);
+        }
+        if (lane == 0) { red_m[wave] = m; red_s[wave] = s; }
+        __syncthreads();
+        if (tid == 0) {
+            float mm = red_m[0], ss = red_s[0];
+            for (int w = 1; w < 4; ++w) ms_merge(mm, ss, red_m[w], red_s[w]);
+            float* st = a.stats + ((size_t)hq * a.nchunks + chunk) * 2;
+            st[0] = mm; st[1] = ss;
+        }
+        __syncthreads();
+    }
+}
+
+// p from the logits, then (p + eps) * |v| (or p alone), and the running maximum
+template <int DT, int GMAX>
+__global__ __launch_bounds__(256) void ea_final_kernel(ScoreArgs a) {
+    __shared__ unsigned int wmax[4];
+    const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, part = lane & 15, rsub = lane >> 4;
+    float Mg[GMAX], Zg[GMAX];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+        Mg[g] = g < a.G ? a.mz[2 * (h * a.G + g)] : 0.0f;
+        Zg[g] = g < a.G ? a.mz[2 * (h * a.G + g) + 1] : 1.0f;
+    }
+    float best = 0.0f;
+    const int t0 = chunk * ROWS_PER_WG;
+    for (int it = 0; it < ROWS_PER_WG / 16; ++it) {
+        const int t = t0 + it * 16 + wave * 4 + rsub;
+        const bool ok = t < a.Tc;
+        float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (ok && a.use_vnorm) load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, x);
+        float vn = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vn = __fmaf_rn(x[e], x[e], vn);
+        vn = group16_sum(vn);
+        if (ok && part == 0) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int g = 0; g < GMAX; ++g)
+                if (g < a.G) acc += __expf(a.logits[((size_t)h * a.G + g) * a.Tc + t] - Mg[g]) / Zg[g];
+            const float pt = acc / (float)a.G;
+            const float sc = a.use_vnorm ? (pt + a.eps) * sqrtf(vn) : pt;
+            a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
+            best = fmaxf(best, sc);
+        }
+    }
+    best = wave_max(best);
+    if (lane == 0) wmax[wave] = __float_as_uint(best);
+    __syncthreads();
+    if (tid == 0) atomicMax(a.gmax, max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
+}
+
 static inline int n_chunks(int Tc) { return (Tc + ROWS_PER_WG - 1) / ROWS_PER_WG; }
 
 struct ScoreLayout { size_t logits, kn2, p, stats, mz, opart, psum, obar, gmax, total; };
@@ -402,6 +586,7 @@ extern "C" int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int
     a.K = K; a.V = V; a.sH = stride_h; a.sT = stride_t;
     a.Hkv = Hkv; a.Hq = Hq; a.G = Hq / Hkv; a.Gl = attn ? 0 : Hq / Hkv; a.T = T; a.Tc = T - n_sink; a.n_sink = n_sink;
     a.nchunks = n_chunks(a.Tc); a.eps = eps; a.mu = mu; a.attn = attn; a.scores = scores;
+    a.cov = nullptr; a.use_vnorm = 0;
     a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
     a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
     a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);
@@ -409,4 +594,67 @@ extern "C" int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int
     if (dtype == ODMKV_F16) return run_score<ODMKV_F16>(a, st);
     if (dtype == ODMKV_BF16) return run_score<ODMKV_BF16>(a, st);
     return run_score<ODMKV_F32>(a, st);
+}
+
+template <int DT>
+static int run_expected(ScoreArgs& a, hipStream_t st) {
+    dim3 grid(a.nchunks, a.Hkv), block(256);
+    if (a.cov) {
+        static bool attr_set = false;
+        const int lds = HD * HD * (int)sizeof(float);
+        if (!attr_set) {
+            ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ea_logits_kernel<DT>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            attr_set = true;
+        }
+        dim3 g2((a.nchunks + EA_CHUNKS_PER_WG - 1) / EA_CHUNKS_PER_WG, a.Hq);
+        hipLaunchKernelGGL((ea_logits_kernel<DT>), g2, block, lds, st, a);
+        ODMKV_CHECK_LAUNCH("ea_logits_kernel");
+    } else {
+        if (a.G <= 4) hipLaunchKernelGGL((score_logits_kernel<DT, 4>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((score_logits_kernel<DT, 8>), grid, block, 0, st, a);
+        ODMKV_CHECK_LAUNCH("score_logits_kernel");
+    }
+    hipLaunchKernelGGL(score_stats_kernel, dim3(a.Hq), dim3(64), 0, st, a);
+    ODMKV_CHECK_LAUNCH("score_stats_kernel");
+    if (a.G <= 4) hipLaunchKernelGGL((ea_final_kernel<DT, 4>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((ea_final_kernel<DT, 8>), grid, block, 0, st, a);
+    ODMKV_CHECK_LAUNCH("ea_final_kernel");
+    if (a.n_sink > 0) {
+        hipLaunchKernelGGL(score_pad_kernel, dim3(a.Hkv), dim3(64), 0, st, a);
+        ODMKV_CHECK_LAUNCH("score_pad_kernel");
+    }
+    return 0;
+}
+
+extern "C" int odmkv_score_expected(const void* K, const void* V, int dtype, int Hkv, int T,
+                                    int64_t stride_h, int64_t stride_t,
+                                    const float* mu, const float* cov, int Hq, int n_sink, float eps,
+                                    int use_vnorm, float* scores, void* workspace, size_t workspace_bytes,
+                                    void* stream) {
+    ODMKV_CHECK_ARG(K && V && scores && workspace && mu, "score_expected: null pointer");
+    ODMKV_CHECK_ARG(dtype == ODMKV_F16 || dtype == ODMKV_BF16 || dtype == ODMKV_F32, "score_expected: bad dtype %d", dtype);
+    ODMKV_CHECK_ARG(Hkv > 0 && Hq > 0 && Hq % Hkv == 0 && Hq / Hkv <= ODMKV_MAX_GROUP,
+                    "score_expected: bad head counts Hkv=%d Hq=%d", Hkv, Hq);
+    ODMKV_CHECK_ARG(n_sink >= 0 && n_sink <= 64 && T > n_sink, "score_expected: need T > n_sink (T=%d, n_sink=%d)", T, n_sink);
+    const int align = dtype == ODMKV_F32 ? 4 : 8;
+    ODMKV_CHECK_ARG(stride_h % align == 0 && stride_t % align == 0 && stride_t >= HD,
+                    "score_expected: strides must keep rows 16-byte aligned");
+    ODMKV_CHECK_ARG(((uintptr_t)K & 15) == 0 && ((uintptr_t)V & 15) == 0, "score_expected: K/V must be 16-byte aligned");
+    ODMKV_CHECK_ARG(((uintptr_t)cov & 15) == 0, "score_expected: the covariance must be 16-byte aligned");
+    ODMKV_CHECK_ARG(workspace_bytes >= odmkv_score_workspace_bytes(Hkv, Hq, T), "score_expected: workspace too small");
+    const ScoreLayout L = score_layout(Hkv, Hq, T);
+    char* ws = (char*)workspace;
+    ScoreArgs a;
+    a.K = K; a.V = V; a.sH = stride_h; a.sT = stride_t;
+    a.Hkv = Hkv; a.Hq = Hq; a.G = Hq / Hkv; a.Gl = a.G; a.T = T; a.Tc = T - n_sink; a.n_sink = n_sink;
+    a.nchunks = n_chunks(a.Tc); a.eps = eps; a.mu = mu; a.attn = nullptr; a.scores = scores;
+    a.cov = cov; a.use_vnorm = use_vnorm ? 1 : 0;
+    a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
+    a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
+    a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == ODMKV_F16) return run_expected<ODMKV_F16>(a, st);
+    if (dtype == ODMKV_BF16) return run_expected<ODMKV_BF16>(a, st);
+    return run_expected<ODMKV_F32>(a, st);
 }

@@ -89,17 +89,25 @@ def _apply_rotary_pos_emb_q(q: torch.Tensor, cos: torch.Tensor, sin: torch.Tenso
 
 def _apply_avg_rope(module: nn.Module, mu: torch.Tensor, cov: Optional[torch.Tensor], q_len: int,
                     n_future_positions: int, n_samples: int = 8):
-    """mu -> R_avg mu, R_avg = mean RoPE matrix over positions [q_len, q_len + n_future).
+    """mu -> R_avg mu and cov -> R_avg cov R_avg^T, R_avg = mean RoPE matrix over positions
+    [q_len, q_len + n_future).
 
     Averaging the rotation matrices element-wise leaves diag(mean cos) + diag(mean sin) P with P
-    the half-rotation, i.e. mean(cos) * mu + mean(sin) * rotate_half(mu): high-frequency pairs
-    average towards zero (a low-pass on the query), low-frequency pairs survive."""
+    the half-rotation, i.e. R_avg x = mean(cos) * x + mean(sin) * rotate_half(x): high-frequency
+    pairs average towards zero (a low-pass on the query), low-frequency pairs survive.  The
+    covariance takes the same map on its rows and then on its columns."""
     rotary_emb = getattr(module, "rotary_emb", None)
     if rotary_emb is None or n_future_positions <= 0:
         return mu, cov
-    if cov is not None:
-        raise NotImplementedError("query covariance is not used by the risk scorer and is not built")
     pos = torch.arange(q_len, q_len + n_future_positions, device=mu.device).unsqueeze(0)
     cos, sin = _aligned_rotary_outputs(rotary_emb, mu, pos)
     c_bar, s_bar = cos[0].mean(dim=0), sin[0].mean(dim=0)
-    return c_bar * mu + s_bar * _rotate_half(mu), None
+
+    def r_avg(x):
+        return c_bar * x + s_bar * _rotate_half(x)
+
+    mu_out = r_avg(mu)
+    if cov is None:
+        return mu_out, None
+    half = r_avg(cov)                                     # cov R^T  (the map acts on the last axis)
+    return mu_out, r_avg(half.transpose(-1, -2)).transpose(-1, -2)

@@ -84,8 +84,13 @@ class _NormFallback(BaseScorer):
 
 
 class ExpectedAttentionScorer(BaseScorer):
-    """Holds the query statistics shared with ``RiskScorer``: the mean pre-RoPE query over the
-    prefill positions after the sinks, passed through the averaged future RoPE."""
+    """Expected attention of future queries (kvquant/scorer.py:154-282 of the reference):
+
+        softmax_t( E[q] . k_t / sqrt(d) + k_t^T Cov[q] k_t / (2 d) ) * |v_t|
+
+    with E[q], Cov[q] the mean and covariance of the pre-RoPE queries over the prefill positions
+    after the sinks, passed through the averaged future RoPE.  Also holds the query statistics
+    shared with ``RiskScorer`` (which switches the covariance off)."""
 
     def __init__(self, *, n_future_positions: int = 512, n_sink: int = 4, use_covariance: bool = True,
                  use_vnorm: bool = True, epsilon: float = 0.0):
@@ -100,29 +105,74 @@ class ExpectedAttentionScorer(BaseScorer):
         q_len = hidden_states.shape[1]
         if q_len <= self.n_sink:
             raise ValueError("not enough tokens to estimate expected attention")
-        if self.use_covariance:
-            raise NotImplementedError("the covariance term is not part of the risk score and is not built")
-        mu = _mean_query_states(module, hidden_states[:, self.n_sink:])
-        return _apply_avg_rope(module, mu, None, q_len, self.n_future_positions)
+        query_input = hidden_states[:, self.n_sink:]
+        if not self.use_covariance:
+            mu = _mean_query_states(module, query_input)
+            return _apply_avg_rope(module, mu, None, q_len, self.n_future_positions)
+        # the covariance is accumulated in fp32 whatever the model's dtype: a 16-bit result of a sum
+        # over tens of thousands of positions would overflow or lose the small eigen-directions
+        q = _get_query_states(module, query_input).float()            # [b, Hq, t, d]
+        mu = q.mean(dim=2)
+        centered = q - mu.unsqueeze(2)
+        cov = torch.matmul(centered.transpose(-1, -2), centered) / query_input.shape[1]
+        return _apply_avg_rope(module, mu, cov, q_len, self.n_future_positions)
 
     def score_prefill(self, keys, values, layer_idx, *, module=None, hidden_states=None):
-        raise NotImplementedError("only the risk score (RiskScorer) runs on the GPU kernels")
+        if module is None or hidden_states is None:
+            return self._fallback.score_prefill(keys, values, layer_idx)
+        if hidden_states.dim() == 2:
+            hidden_states = hidden_states.unsqueeze(0)
+        if hidden_states.shape[0] != 1:
+            raise ValueError("ExpectedAttentionScorer expects a single-sample hidden-state slice.")
+        if keys.shape[1] <= self.n_sink:
+            return torch.ones(keys.shape[:2], device=keys.device, dtype=keys.dtype)
+        try:
+            mu, cov = self._query_statistics(module, hidden_states)
+        except (AttributeError, NotImplementedError, ValueError):
+            return self._fallback.score_prefill(keys, values, layer_idx)
+        scores = _launch_score_expected(keys, values, mu[0], None if cov is None else cov[0],
+                                        mu.shape[1], self.n_sink, self.epsilon, self.use_vnorm)
+        return self._maybe_normalize(scores)
 
     def score_decode(self, key, value, layer_idx, *, module=None, hidden_states=None):
         return self._fallback.score_decode(key, value, layer_idx, module=module, hidden_states=hidden_states)
 
 
-def _launch_score(keys: torch.Tensor, values: torch.Tensor, mu: Optional[torch.Tensor],
-                  attn: Optional[torch.Tensor], n_q_heads: int, n_sink: int, eps: float) -> torch.Tensor:
+def _kv_operands(keys: torch.Tensor, values: torch.Tensor):
+    """keys/values as the kernels read them: rows contiguous and 16-byte aligned, equal strides."""
     _lib.require_gpu(keys, "keys")
-    H, T, D = keys.shape
-    if D != _lib.HEAD_DIM:
-        raise ValueError(f"the HIP kernels are written for head_dim {_lib.HEAD_DIM}, got {D}")
+    if keys.shape[-1] != _lib.HEAD_DIM:
+        raise ValueError(f"the HIP kernels are written for head_dim {_lib.HEAD_DIM}, got {keys.shape[-1]}")
     align = 4 if keys.dtype == torch.float32 else 8
     def ok(t):
         return t.stride(-1) == 1 and t.stride(0) % align == 0 and t.stride(1) % align == 0 and t.data_ptr() % 16 == 0
     if not ok(keys) or not ok(values) or keys.stride() != values.stride():
         keys, values = keys.contiguous(), values.contiguous()
+    return keys, values
+
+
+def _launch_score_expected(keys: torch.Tensor, values: torch.Tensor, mu: torch.Tensor,
+                           cov: Optional[torch.Tensor], n_q_heads: int, n_sink: int, eps: float,
+                           use_vnorm: bool) -> torch.Tensor:
+    keys, values = _kv_operands(keys, values)
+    H, T, D = keys.shape
+    dev = keys.device
+    scores = torch.empty(H, T, dtype=torch.float32, device=dev)
+    ws_bytes = lib.odmkv_score_workspace_bytes(H, n_q_heads, T)
+    ws = _lib.workspace(dev, ws_bytes, "score")
+    mu32 = mu.reshape(n_q_heads, D).float().contiguous()
+    cov32 = None if cov is None else cov.reshape(n_q_heads, D, D).float().contiguous()
+    _lib.check(lib.odmkv_score_expected(
+        keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys), H, T, keys.stride(0), keys.stride(1),
+        mu32.data_ptr(), _lib.ptr(cov32), n_q_heads, n_sink, float(eps), int(bool(use_vnorm)),
+        scores.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
+    return scores
+
+
+def _launch_score(keys: torch.Tensor, values: torch.Tensor, mu: Optional[torch.Tensor],
+                  attn: Optional[torch.Tensor], n_q_heads: int, n_sink: int, eps: float) -> torch.Tensor:
+    keys, values = _kv_operands(keys, values)
+    H, T, D = keys.shape
     dev = keys.device
     scores = torch.empty(H, T, dtype=torch.float32, device=dev)
     ws_bytes = lib.odmkv_score_workspace_bytes(H, n_q_heads, T)

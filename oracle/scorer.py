@@ -6,6 +6,7 @@ Follows /root/reference/kvquant/scorer.py
   _pad_sinks_and_normalize                    :321-325  (grain "global" = identity, :118-119)
   RiskScorer.score_prefill                    :385-404
   RiskScorer.score_with_attn                  :406-416
+  ExpectedAttentionScorer.score_prefill       :204-257  (expected_attention_score below)
   _NormFallback.score_prefill                 :145-147 (+ _normalize_scores "layer" :130-134)
 and /root/reference/kvquant/attention_utils.py
   _repeat_kv :19-26, _get_query_states :29-54, _apply_avg_rope :57-115.
@@ -176,3 +177,70 @@ def risk_score_with_attn(keys: torch.Tensor, values: torch.Tensor, attn: torch.T
     kn2 = keys.float().pow(2).sum(dim=-1)
     vn2 = values.float().pow(2).sum(dim=-1)
     return (p + epsilon).pow(2) * (vn2 + (kn2 / float(keys.shape[-1])) * irrep)
+
+
+def avg_rope_matrix(module, like: torch.Tensor, q_len: int, n_future: int) -> Optional[torch.Tensor]:
+    """R_avg [d, d]: element-wise mean over positions [q_len, q_len + n_future) of the RoPE matrices
+    diag(cos_p) + diag(sin_p) P (attention_utils.py:83-105); None where the reference returns its
+    inputs unchanged."""
+    rotary = getattr(module, "rotary_emb", None)
+    if rotary is None or n_future <= 0:
+        return None
+    pos = torch.arange(q_len, q_len + n_future, device=like.device).unsqueeze(0)
+    cos, sin = rotary(like, pos)
+    cos = cos.to(device=like.device, dtype=like.dtype)[0]
+    sin = sin.to(device=like.device, dtype=like.dtype)[0]
+    d = like.shape[-1]
+    half = d // 2
+    eye = torch.eye(d, dtype=like.dtype, device=like.device)
+    perm = torch.zeros(d, d, dtype=like.dtype, device=like.device)
+    perm[half:, :half] = torch.eye(half, dtype=like.dtype, device=like.device)
+    perm[:half, half:] = -torch.eye(half, dtype=like.dtype, device=like.device)
+    return (cos.unsqueeze(-1) * eye + sin.unsqueeze(-1) * perm).mean(dim=0)
+
+
+def query_statistics(module, hidden: torch.Tensor, n_sink: int, n_future: int,
+                     use_covariance: bool):
+    """(mu [1, Hq, d], cov [1, Hq, d, d] or None) after the averaged RoPE: scorer.py:184-202 with
+    attention_utils.py:107-115 (mu' = mu R^T, cov' = R cov R^T)."""
+    if hidden.dim() == 2:
+        hidden = hidden.unsqueeze(0)
+    q_len = hidden.shape[1]
+    if q_len <= n_sink:
+        raise ValueError("not enough tokens to estimate expected attention")
+    q_in = hidden[:, n_sink:]
+    q = query_states(module, q_in)
+    mu = q.mean(dim=2)
+    cov = None
+    if use_covariance:
+        centered = q - mu.unsqueeze(2)
+        cov = torch.einsum("bhsd,bhse->bhde", centered, centered) / q_in.shape[1]
+    r = avg_rope_matrix(module, mu, q_len, n_future)
+    if r is None:
+        return mu, cov
+    mu = torch.matmul(mu, r.T)
+    if cov is not None:
+        cov = torch.matmul(r, torch.matmul(cov, r.T))
+    return mu, cov
+
+
+def expected_attention_score(keys: torch.Tensor, values: torch.Tensor, mu: torch.Tensor,
+                             cov: Optional[torch.Tensor], n_q_heads: int, *, n_sink: int = 4,
+                             epsilon: float = 0.0, use_vnorm: bool = True) -> torch.Tensor:
+    """ExpectedAttentionScorer.score_prefill after the query statistics (scorer.py:227-257),
+    before the final normalisation: keys/values [Hkv, T, d], mu [1, Hq, d], cov [1, Hq, d, d] or
+    None -> [Hkv, T]."""
+    if keys.shape[1] <= n_sink:
+        return torch.ones(keys.shape[:2], dtype=keys.dtype)
+    k_core, v_core = keys[:, n_sink:], values[:, n_sink:]
+    h_kv, t_core, d = k_core.shape
+    groups = n_q_heads // h_kv
+    kt = repeat_kv(k_core.unsqueeze(0), groups).transpose(2, 3)             # [1, Hq, d, Tc]
+    raw = torch.matmul(mu.unsqueeze(2), kt).squeeze(2) / math.sqrt(d)
+    if cov is not None:
+        raw = raw + torch.einsum("bhdt,bhde,bhet->bht", kt, cov, kt) / d / 2
+    raw = torch.softmax(raw, dim=-1)
+    raw = raw.reshape(1, h_kv, groups, t_core).mean(dim=2)
+    if use_vnorm:
+        raw = (raw + epsilon) * v_core.unsqueeze(0).norm(dim=-1)
+    return pad_sinks(raw, n_sink)

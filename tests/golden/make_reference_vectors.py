@@ -160,6 +160,41 @@ def main(ref_root: str) -> None:
     score_case("f16", 2, 4, 48, 16, 24, 21, torch.float16)
     score_case("f32_d128", 2, 8, 160, 128, 64, 24, torch.float32)
 
+    # ExpectedAttentionScorer.score_prefill: covariance on/off, value norm on/off, RoPE, GQA
+    def ea_case(name, hkv, hq, t, d, hidden, seed, *, cov=True, vnorm=True, eps=0.0, rotary=False, n_future=512,
+                grain="global"):
+        gg = torch.Generator().manual_seed(seed)
+        k = torch.randn(hkv, t, d, generator=gg)
+        v = torch.randn(hkv, t, d, generator=gg)
+        h = torch.randn(1, t, hidden, generator=gg)
+        mod = Stub(hidden, hq, d, seed + 1)
+        if rotary:
+            from transformers import LlamaConfig
+            from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+            cfg = LlamaConfig(hidden_size=hq * d, num_attention_heads=hq, num_key_value_heads=hkv,
+                              head_dim=d, rope_theta=10000.0, max_position_embeddings=4096)
+            mod.rotary_emb = LlamaRotaryEmbedding(cfg)
+        sc = ref_scorer.ExpectedAttentionScorer(n_future_positions=n_future, n_sink=4, use_covariance=cov,
+                                                use_vnorm=vnorm, epsilon=eps)
+        sc.normalize_grain = grain
+        with torch.no_grad():
+            res = sc.score_prefill(k, v, 0, module=mod, hidden_states=h)
+            mu, cv = sc._query_statistics(mod, h)
+        out[f"ea_{name}_k"], out[f"ea_{name}_v"], out[f"ea_{name}_h"] = k.numpy(), v.numpy(), h.numpy()
+        out[f"ea_{name}_w"] = mod.q_proj.weight.detach().numpy()
+        out[f"ea_{name}_b"] = mod.q_proj.bias.detach().numpy()
+        out[f"ea_{name}_mu"] = mu.numpy()
+        if cv is not None:
+            out[f"ea_{name}_cov"] = cv.numpy()
+        out[f"ea_{name}_out"] = res.numpy()
+
+    ea_case("cov", 2, 4, 48, 16, 24, 41, eps=1e-2)
+    ea_case("nocov", 2, 4, 48, 16, 24, 42, cov=False)
+    ea_case("novnorm", 3, 3, 40, 16, 24, 43, vnorm=False)
+    ea_case("rope", 2, 8, 64, 32, 40, 44, rotary=True, n_future=64, eps=1e-2)
+    ea_case("d128", 2, 8, 300, 128, 64, 45, eps=1e-2)
+    ea_case("d128_rope_layer", 2, 4, 200, 128, 64, 46, rotary=True, n_future=128, grain="layer")
+
     # score_with_attn and the norm fallback
     gg = torch.Generator().manual_seed(31)
     k = torch.randn(3, 20, 16, generator=gg); v = torch.randn(3, 20, 16, generator=gg)

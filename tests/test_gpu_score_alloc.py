@@ -170,3 +170,64 @@ def test_calibrate_epsilon_matches_oracle():
     assert set(got) == set(want)
     for b in LEVELS:
         assert abs(got[b] - want[b]) <= 1e-6 * max(want[b], 1e-9) + 1e-12
+
+
+# ---- ExpectedAttentionScorer: mean query + query covariance (fp32 matrix cores) -----------------
+@pytest.mark.parametrize("hkv,hq,T,dtype,use_cov,vnorm", [
+    (2, 8, 700, torch.float32, True, True), (8, 32, 2085, torch.float16, True, True),
+    (4, 28, 1500, torch.bfloat16, True, True), (3, 3, 261, torch.float16, True, False),
+    (2, 16, 517, torch.float16, True, True), (2, 4, 300, torch.float32, False, True), (1, 1, 5, torch.float16, True, True)])
+def test_expected_attention_kernel_matches_oracle(hkv, hq, T, dtype, use_cov, vnorm):
+    from kvquant.scorer import _launch_score_expected
+    g = torch.Generator().manual_seed(T + hq)
+    k = torch.randn(hkv, T, 128, generator=g).to(dtype); v = torch.randn(hkv, T, 128, generator=g).to(dtype)
+    mu = torch.randn(1, hq, 128, generator=g)
+    a = torch.randn(1, hq, 128, 24, generator=g) * 0.2        # low rank + diagonal: a covariance
+    cov = a @ a.transpose(-1, -2) + 0.05 * torch.eye(128) if use_cov else None
+    want = osc.expected_attention_score(k.double(), v.double(), mu.double(), None if cov is None else cov.double(),
+                                        hq, n_sink=4, epsilon=1e-2, use_vnorm=vnorm)
+    got = _launch_score_expected(k.to(DEV), v.to(DEV), mu[0].to(DEV), None if cov is None else cov[0].to(DEV),
+                                 hq, 4, 1e-2, vnorm)
+    assert got.shape == (hkv, T) and got.dtype == torch.float32
+    np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=SCORE_RTOL)
+    assert torch.all(got[:, :4] == got[:, 4:].max())
+
+
+def test_expected_attention_strided_cache_rows():
+    """K/V as slices of a wider buffer (head and token strides differ from the dense ones)."""
+    from kvquant.scorer import _launch_score_expected
+    g = torch.Generator().manual_seed(77)
+    big_k = torch.randn(2, 400, 256, generator=g).half().to(DEV); big_v = torch.randn(2, 400, 256, generator=g).half().to(DEV)
+    k, v = big_k[:, 10:350, 128:], big_v[:, 10:350, 128:]
+    mu = torch.randn(1, 4, 128, generator=g)
+    a = torch.randn(1, 4, 128, 128, generator=g) * 0.05
+    cov = a @ a.transpose(-1, -2)
+    want = osc.expected_attention_score(k.cpu().double(), v.cpu().double(), mu.double(), cov.double(), 4,
+                                        n_sink=4, epsilon=0.0, use_vnorm=True)
+    got = _launch_score_expected(k, v, mu[0].to(DEV), cov[0].to(DEV), 4, 4, 0.0, True)
+    np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=SCORE_RTOL)
+
+
+@pytest.mark.parametrize("name", ["d128", "d128_rope_layer"])
+def test_expected_attention_scorer_matches_reference_vectors(golden, name):
+    """The host class end to end (query statistics, averaged RoPE on mean and covariance, kernel,
+    normalisation) against what the reference returned for the same module and tensors."""
+    from kvquant.scorer import ExpectedAttentionScorer
+    from test_oracle_scorer import EA_CASES, _ea_stub
+    hkv, hq, d, use_cov, vnorm, eps, nf, rotary, grain = EA_CASES[name]
+    cfg = dict(hidden_size=hq * d, num_attention_heads=hq, num_key_value_heads=hkv, head_dim=d,
+               rope_theta=10000.0, max_position_embeddings=4096) if rotary else None
+    k, v, h = (torch.from_numpy(golden[f"ea_{name}_{x}"]) for x in "kvh")
+    mod = _ea_stub(golden, name, hq, d, cfg).to(DEV)
+    sc = ExpectedAttentionScorer(n_future_positions=nf, n_sink=4, use_covariance=use_cov, use_vnorm=vnorm, epsilon=eps)
+    sc.normalize_grain = grain
+    with torch.no_grad():
+        mu, cov = sc._query_statistics(mod, h.to(DEV))
+        got = sc.score_prefill(k.to(DEV), v.to(DEV), 0, module=mod, hidden_states=h.to(DEV))
+    np.testing.assert_allclose(mu.cpu().numpy(), golden[f"ea_{name}_mu"], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(cov.cpu().numpy(), golden[f"ea_{name}_cov"], rtol=1e-3, atol=1e-5)
+    np.testing.assert_allclose(got.cpu().numpy(), golden[f"ea_{name}_out"], rtol=SCORE_RTOL, atol=1e-6)
+    # fp16 model and cache: same scores within the 16-bit rounding of the inputs
+    with torch.no_grad():
+        got16 = sc.score_prefill(k.half().to(DEV), v.half().to(DEV), 0, module=mod.half(), hidden_states=h.half().to(DEV))
+    np.testing.assert_allclose(got16.cpu().numpy(), golden[f"ea_{name}_out"], rtol=2e-2, atol=1e-4)

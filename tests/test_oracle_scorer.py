@@ -123,3 +123,83 @@ def test_closed_forms_and_invariants():
     np.testing.assert_allclose(core.numpy(), s1[:, 4:].numpy(), rtol=1e-5)
     # short inputs
     assert torch.all(sc.risk_score_from_mu(k[:, :4], v[:, :4], mu, 4) == 1)
+
+
+# ---- ExpectedAttentionScorer.score_prefill (mean query + query covariance) ---------------------
+def _ea_stub(golden, name, hq, d, rotary_cfg=None):
+    mod = Stub(golden[f"ea_{name}_w"], golden[f"ea_{name}_b"], hq, d)
+    if rotary_cfg is not None:
+        from transformers import LlamaConfig
+        from transformers.models.llama.modeling_llama import LlamaRotaryEmbedding
+        mod.rotary_emb = LlamaRotaryEmbedding(LlamaConfig(**rotary_cfg))
+    return mod
+
+
+EA_CASES = {   # name: (hkv, hq, d, use_covariance, use_vnorm, eps, n_future, rotary, grain)
+    "cov": (2, 4, 16, True, True, 1e-2, 512, False, "global"),
+    "nocov": (2, 4, 16, False, True, 0.0, 512, False, "global"),
+    "novnorm": (3, 3, 16, True, False, 0.0, 512, False, "global"),
+    "rope": (2, 8, 32, True, True, 1e-2, 64, True, "global"),
+    "d128": (2, 8, 128, True, True, 1e-2, 512, False, "global"),
+    "d128_rope_layer": (2, 4, 128, True, True, 0.0, 128, True, "layer"),
+}
+
+
+def ea_oracle(golden, name):
+    """The oracle's expected-attention score of a recorded case -> (scores, mu, cov)."""
+    hkv, hq, d, use_cov, vnorm, eps, nf, rotary, grain = EA_CASES[name]
+    cfg = dict(hidden_size=hq * d, num_attention_heads=hq, num_key_value_heads=hkv, head_dim=d,
+               rope_theta=10000.0, max_position_embeddings=4096) if rotary else None
+    k, v, h = (torch.from_numpy(golden[f"ea_{name}_{x}"]) for x in "kvh")
+    mod = _ea_stub(golden, name, hq, d, cfg)
+    with torch.no_grad():
+        mu, cov = sc.query_statistics(mod, h, 4, nf, use_cov)
+        got = sc.expected_attention_score(k, v, mu, cov, hq, n_sink=4, epsilon=eps, use_vnorm=vnorm)
+    if grain == "layer":
+        got = (got - got.min()) / (got.max() - got.min())
+    return got, mu, cov
+
+
+@pytest.mark.parametrize("name", sorted(EA_CASES))
+def test_expected_attention_matches_reference(golden, name):
+    got, mu, cov = ea_oracle(golden, name)
+    np.testing.assert_allclose(mu.numpy(), golden[f"ea_{name}_mu"], rtol=1e-5, atol=1e-6)
+    if EA_CASES[name][3]:
+        np.testing.assert_allclose(cov.numpy(), golden[f"ea_{name}_cov"], rtol=1e-4, atol=1e-6)
+    else:
+        assert cov is None and f"ea_{name}_cov" not in golden
+    np.testing.assert_allclose(got.numpy(), golden[f"ea_{name}_out"], rtol=5e-5, atol=1e-7)
+
+
+def test_expected_attention_closed_forms():
+    g = torch.Generator().manual_seed(5)
+    hkv, G, T, d = 2, 2, 24, 8
+    k = torch.randn(hkv, T, d, generator=g, dtype=torch.float64)
+    v = torch.randn(hkv, T, d, generator=g, dtype=torch.float64)
+    mu = torch.randn(1, hkv * G, d, generator=g, dtype=torch.float64)
+    a = torch.randn(1, hkv * G, d, d, generator=g, dtype=torch.float64)
+    cov = a @ a.transpose(-1, -2)
+    got = sc.expected_attention_score(k, v, mu, cov, hkv * G, n_sink=4, epsilon=0.5, use_vnorm=True)
+    # brute force, one token at a time
+    want = torch.zeros(hkv, T, dtype=torch.float64)
+    for h in range(hkv):
+        p = torch.zeros(T - 4, dtype=torch.float64)
+        for gq in range(G):
+            q = h * G + gq
+            lg = torch.tensor([float(mu[0, q] @ k[h, t]) / d ** 0.5 + float(k[h, t] @ cov[0, q] @ k[h, t]) / (2 * d)
+                               for t in range(4, T)], dtype=torch.float64)
+            p += torch.exp(lg - lg.max()) / torch.exp(lg - lg.max()).sum() / G
+        want[h, 4:] = (p + 0.5) * torch.tensor([float(v[h, t].norm()) for t in range(4, T)], dtype=torch.float64)
+    want[:, :4] = want[:, 4:].max()
+    np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=1e-12)
+    # a zero covariance is the mean-query score; without the value norm every head's core sums to one
+    zero = sc.expected_attention_score(k, v, mu, torch.zeros_like(cov), hkv * G, n_sink=4, use_vnorm=False)
+    none = sc.expected_attention_score(k, v, mu, None, hkv * G, n_sink=4, use_vnorm=False)
+    np.testing.assert_allclose(zero.numpy(), none.numpy(), rtol=1e-13)
+    np.testing.assert_allclose(none[:, 4:].sum(-1).numpy(), 1.0, rtol=1e-12)
+    # cov = c I adds c |k|^2 / (2d) to every logit of a head: tokens of equal norm keep their ranks
+    kn = k / k.norm(dim=-1, keepdim=True)
+    eye = torch.eye(d, dtype=torch.float64).expand(1, hkv * G, d, d) * 3.0
+    same = sc.expected_attention_score(kn, v, mu, eye, hkv * G, n_sink=4, use_vnorm=False)
+    base = sc.expected_attention_score(kn, v, mu, None, hkv * G, n_sink=4, use_vnorm=False)
+    np.testing.assert_allclose(same.numpy(), base.numpy(), rtol=1e-12)
