@@ -259,6 +259,9 @@ def main() -> int:
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for counter runs under rocprofv3 --pmc: a few eager decode steps and one plain 256 MiB "
                          "device copy (the calibration kernel), nothing else timed")
+    ap.add_argument("--score-expected", action="store_true",
+                    help="time the expected-attention score (mean query + query covariance on the fp32 matrix "
+                         "cores) of one --ctx-token layer, rotating over 8 layers' keys and values, and exit")
     ap.add_argument("--press-e2e", action="store_true",
                     help="instead of the kernel benchmark: a random-init Llama-3-8B-shaped model (--e2e-layers) under the "
                          "press, prefill of --ctx tokens, then greedy decode with the fused kernel and with the dense "
@@ -287,6 +290,39 @@ def main() -> int:
     if args.press_e2e:
         print(json.dumps({"press_e2e": press_e2e(dev, T, args.target, args.e2e_tokens, args.e2e_layers,
                                                    args.e2e_vocab)}))
+        return 0
+
+    if args.score_expected:
+        from kvquant.scorer import _launch_score_expected
+        g = torch.Generator().manual_seed(5)
+        layers = []
+        for _ in range(8):
+            k = torch.randn(n_kv, T, 128, generator=g).half().to(dev)
+            v = torch.randn(n_kv, T, 128, generator=g).half().to(dev)
+            mu = torch.randn(n_q, 128, generator=g).to(dev)
+            a = torch.randn(n_q, 128, 32, generator=g) * 0.2
+            layers.append((k, v, mu, (a @ a.transpose(-1, -2)).to(dev)))
+        out = {}
+        for name, with_cov in (("with_covariance", True), ("mean_query_only", False)):
+            def sweep():
+                for k, v, mu, cov in layers:
+                    _launch_score_expected(k, v, mu, cov if with_cov else None, n_q, 4, 1e-2, True)
+            for _ in range(3):
+                sweep()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(5):
+                sweep()
+            e1.record()
+            torch.cuda.synchronize()
+            out[name + "_ms_per_layer"] = round(e0.elapsed_time(e1) / (5 * len(layers)), 4)
+        flop = 2.0 * n_q * (T - 4) * 128 * 128
+        out["quadratic_form_flop_per_layer"] = flop
+        out["quadratic_form_TFLOPs_lower_bound"] = round(flop / ((out["with_covariance_ms_per_layer"]
+                                                                   - out["mean_query_only_ms_per_layer"]) * 1e-3) / 1e12, 1)
+        out["shape"] = {"Hkv": n_kv, "Hq": n_q, "T": T, "dtype": "fp16"}
+        print(json.dumps({"score_expected": out}))
         return 0
 
     if args.read_ceiling:

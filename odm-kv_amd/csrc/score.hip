@@ -21,6 +21,7 @@ struct ScoreArgs {
     const float* attn;    // [Hkv, T] or null
     const float* cov;     // [Hq, 128, 128] query covariance (expected-attention score only) or null
     int use_vnorm;        // expected-attention score: multiply (p + eps) by |v|
+    int ea_cpw;           // expected-attention score: 256-token chunks a workgroup walks
     float* scores;        // [Hkv, T]
     float* logits;        // [Hq, Tc]
     float* kn2;           // [Hkv, Tc]
@@ -341,53 +342,66 @@ __global__ void score_pad_kernel(ScoreArgs a) {
 //   p[h,t]     = mean over the group of softmax_t(logit[q,:]);   s = (p + eps) * |v|   (or p alone)
 //
 // The quadratic form is a true dense contraction, [T,128] x [128,128] per query head, and runs on
-// the fp32 matrix cores (v_mfma_f32_32x32x2_f32): a wave takes 32 tokens, D = K . Cov/(2d) with the
-// accumulator preset to mu/sqrt(d) in every row, so that logit[t] = sum_c K[t][c] * D[t][c] holds
-// both terms.  Cov/(2d) stays in LDS (64 KB) for the workgroup's life; K is read from HBM by the
+// the fp32 matrix cores (v_mfma_f32_32x32x2_f32): a wave takes 32 tokens, D = Cov/(2d) . K^T with the
+// accumulator preset to mu[c]/sqrt(d), so that logit[t] = sum_c K[t][c] * D[c][t] holds both terms.  Cov/(2d) stays in LDS (64 KB) for the workgroup's life; K is read from HBM by the
 // first head of a group and from the caches by the others.
 // ------------------------------------------------------------------------------------------------
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-#define EA_CHUNKS_PER_WG 2   // 256-token chunks a workgroup walks with one copy of the covariance
+#define EA_MAX_CHUNKS_PER_WG 4   // most 256-token chunks a workgroup walks with one copy of the covariance
 
-// the 32 elements [32*blk, 32*blk+32) of a row, as raw registers; elem() picks one of them
-template <int DT> struct RowBlock;
-template <> struct RowBlock<ODMKV_F32> {
-    float4 r[8];
-    __device__ inline void load(const void* base, size_t off, int blk) {
-        const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + off + blk * 32);
+// the 128 elements of one token's row, as raw registers
+template <int DT> struct RowRegs;
+template <> struct RowRegs<ODMKV_F32> {
+    float4 r[32];
+    __device__ inline void load(const void* base, size_t off) {
+        const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + off);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) r[i] = p[i];
+        for (int i = 0; i < 32; ++i) r[i] = p[i];
     }
-    // element 2*s + half of the block
-    __device__ inline float elem(int s, int half) const {
-        const float4 v = r[s >> 1];
-        const float lo = (s & 1) ? v.z : v.x, hi = (s & 1) ? v.w : v.y;
-        return half ? hi : lo;
+    __device__ inline float at(int e) const {            // e is a compile-time constant where this is used
+        const float4 v = r[e >> 2];
+        return (e & 3) == 0 ? v.x : (e & 3) == 1 ? v.y : (e & 3) == 2 ? v.z : v.w;
+    }
+    // element 2 s + half
+    __device__ inline float pair_elem(int s, int half) const { return half ? at(2 * s + 1) : at(2 * s); }
+    // the four elements e0 + 4 half + 0..3 (e0 a multiple of 8)
+    __device__ inline void quad(int e0, int half, float* x) const {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[j] = half ? at(e0 + 4 + j) : at(e0 + j);
     }
 };
-template <int DT> struct RowBlock {
-    uint4 r[4];
-    __device__ inline void load(const void* base, size_t off, int blk) {
-        const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + off + blk * 32);
+template <int DT> struct RowRegs {
+    uint4 r[16];
+    __device__ inline void load(const void* base, size_t off) {
+        const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + off);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r[i] = p[i];
+        for (int i = 0; i < 16; ++i) r[i] = p[i];
     }
-    __device__ inline float elem(int s, int half) const {
-        const uint4 v = r[s >> 2];
-        const uint32_t w = (s & 3) == 0 ? v.x : (s & 3) == 1 ? v.y : (s & 3) == 2 ? v.z : v.w;
+    __device__ inline uint32_t dword(int i) const {
+        const uint4 v = r[i >> 2];
+        return (i & 3) == 0 ? v.x : (i & 3) == 1 ? v.y : (i & 3) == 2 ? v.z : v.w;
+    }
+    __device__ inline float pair_elem(int s, int half) const {
+        const uint32_t w = dword(s);
         return Elem<DT>::to_f32((uint16_t)(half ? (w >> 16) : (w & 0xffffu)));
     }
+    __device__ inline void quad(int e0, int half, float* x) const {
+        const uint32_t w0 = half ? dword(e0 / 2 + 2) : dword(e0 / 2);
+        const uint32_t w1 = half ? dword(e0 / 2 + 3) : dword(e0 / 2 + 1);
+        x[0] = Elem<DT>::to_f32((uint16_t)(w0 & 0xffffu)); x[1] = Elem<DT>::to_f32((uint16_t)(w0 >> 16));
+        x[2] = Elem<DT>::to_f32((uint16_t)(w1 & 0xffffu)); x[3] = Elem<DT>::to_f32((uint16_t)(w1 >> 16));
+    }
 };
 
-template <int DT>
-__device__ static inline float load_elem(const void* base, size_t off) {
-    if constexpr (DT == ODMKV_F32) return reinterpret_cast<const float*>(base)[off];
-    else return Elem<DT>::to_f32(reinterpret_cast<const uint16_t*>(base)[off]);
-}
-
+// Operand roles: the matrix rows are the covariance's output columns c, the matrix columns the 32
+// tokens (D[c][t] = sum_e Cov[e][c] K[t][e]; the quadratic form only sees the symmetric part of
+// Cov, so Cov[e][c] stands for Cov[c][e]).  A lane then ends with token lane % 32 and the 64
+// columns c = 32 cb + 8 q + 4 (lane / 32) + j: logit[t] = sum_c K[t][c] D[c][t] takes the lane's own
+// row, which it still holds in registers, and one exchange between the two halves of the wave.
 template <int DT>
 __global__ __launch_bounds__(256) void ea_logits_kernel(ScoreArgs a) {
     extern __shared__ __align__(16) float cov_s[];      // [128][128], already divided by 2 d
+    __shared__ __align__(16) float mu_s[HD];            // mu / sqrt(d)
     __shared__ float red_m[4], red_s[4];
     const int hq = blockIdx.y, h = hq / a.G, tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, col = lane & 31, half = lane >> 5;
@@ -400,64 +414,63 @@ __global__ __launch_bounds__(256) void ea_logits_kernel(ScoreArgs a) {
             v.x *= sc; v.y *= sc; v.z *= sc; v.w *= sc;
             dst[e] = v;
         }
+        if (tid < HD) mu_s[tid] = a.mu[(size_t)hq * HD + tid] / 11.313708498984761f;
     }
-    float mu_c[4];
-#pragma unroll
-    for (int cb = 0; cb < 4; ++cb) mu_c[cb] = a.mu[(size_t)hq * HD + cb * 32 + col] / 11.313708498984761f;
+    // sub-tile i of this wave (two per chunk): tokens t0(i) .. t0(i) + 31
+    auto t0_of = [&](int i) { return (blockIdx.x * a.ea_cpw + (i >> 1)) * ROWS_PER_WG + (wave * 2 + (i & 1)) * 32; };
+    auto row_of = [&](int i) {                          // rows past the end repeat the last row and are not stored
+        return (size_t)h * a.sH + (size_t)(a.n_sink + min(t0_of(i) + col, a.Tc - 1)) * a.sT;
+    };
+    RowRegs<DT> cur;
+    cur.load(a.K, row_of(0));
     __syncthreads();
-    for (int cc = 0; cc < EA_CHUNKS_PER_WG; ++cc) {
-        const int chunk = blockIdx.x * EA_CHUNKS_PER_WG + cc;
+    const float* cbase = cov_s + half * HD + col;
+    for (int cc = 0; cc < a.ea_cpw; ++cc) {
+        const int chunk = blockIdx.x * a.ea_cpw + cc;
         if (chunk >= a.nchunks) break;                  // the same for every thread of the workgroup
         float m = -INFINITY, s = 0.0f;
         for (int sub = 0; sub < 2; ++sub) {
-            const int t0 = chunk * ROWS_PER_WG + (wave * 2 + sub) * 32;
-            if (t0 >= a.Tc) break;                      // wave-uniform
-            // operand A: lane = token t0 + col (rows past the end repeat the last row and are not stored)
-            const size_t arow = (size_t)h * a.sH + (size_t)(a.n_sink + min(t0 + col, a.Tc - 1)) * a.sT;
-            f32x16 acc[4];
+            const int it = cc * 2 + sub;
+            const int t0 = t0_of(it);
+            RowRegs<DT> nxt;
+            if constexpr (DT != ODMKV_F32) {            // the next sub-tile's row travels under this one's products
+                if (it < 2 * a.ea_cpw - 1) nxt.load(a.K, row_of(it + 1));
+            }
+            if (t0 < a.Tc) {                            // wave-uniform
+                f32x16 acc[4];
 #pragma unroll
-            for (int cb = 0; cb < 4; ++cb)
+                for (int cb = 0; cb < 4; ++cb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[cb][r] = mu_c[cb];
+                    for (int q = 0; q < 4; ++q) {
+                        const float4 mv = *reinterpret_cast<const float4*>(mu_s + 32 * cb + 8 * q + 4 * half);
+                        acc[cb][4 * q] = mv.x; acc[cb][4 * q + 1] = mv.y; acc[cb][4 * q + 2] = mv.z; acc[cb][4 * q + 3] = mv.w;
+                    }
 #pragma unroll
-            for (int blk = 0; blk < 4; ++blk) {
-                RowBlock<DT> rb;
-                rb.load(a.K, arow, blk);
-#pragma unroll
-                for (int st = 0; st < 16; ++st) {
-                    const float av = rb.elem(st, half);
-                    const float* brow = cov_s + (blk * 32 + 2 * st + half) * HD + col;
+                for (int st = 0; st < 64; ++st) {
+                    const float kv = cur.pair_elem(st, half);
 #pragma unroll
                     for (int cb = 0; cb < 4; ++cb)
-                        acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, brow[cb * 32], acc[cb], 0, 0, 0);
+                        acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(cbase[st * 2 * HD + cb * 32], kv, acc[cb], 0, 0, 0);
+                }
+                float lg = 0.0f;
+#pragma unroll
+                for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float x[4];
+                        cur.quad(32 * cb + 8 * q, half, x);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) lg = __fmaf_rn(x[j], acc[cb][4 * q + j], lg);
+                    }
+                lg += __shfl_xor(lg, 32, WAVE);
+                const int t = t0 + col;
+                if (half == 0 && t < a.Tc) {
+                    a.logits[(size_t)hq * a.Tc + t] = lg;
+                    ms_merge(m, s, lg, 1.0f);
                 }
             }
-            // logit[row] = sum over columns of K[row][c] * D[row][c]; register r of a lane is row
-            // 8 (r / 4) + 4 half + r % 4, column 32 cb + col
-            float part[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = 8 * (r >> 2) + 4 * half + (r & 3);
-                const size_t off = (size_t)h * a.sH + (size_t)(a.n_sink + min(t0 + row, a.Tc - 1)) * a.sT + col;
-                float acc_r = 0.0f;
-#pragma unroll
-                for (int cb = 0; cb < 4; ++cb) acc_r = __fmaf_rn(load_elem<DT>(a.K, off + cb * 32), acc[cb][r], acc_r);
-                part[r] = acc_r;
-            }
-#pragma unroll
-            for (int o = 1; o < 32; o <<= 1)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) part[r] += __shfl_xor(part[r], o, WAVE);
-            // lanes col < 16 of either half own register r = col: 16 + 16 rows per wave
-            float mine = part[0];
-#pragma unroll
-            for (int r = 1; r < 16; ++r) mine = (col & 15) == r ? part[r] : mine;
-            const int rown = col & 15;
-            const int t = t0 + 8 * (rown >> 2) + 4 * half + (rown & 3);
-            if (col < 16 && t < a.Tc) {
-                a.logits[(size_t)hq * a.Tc + t] = mine;
-                ms_merge(m, s, mine, 1.0f);
-            }
+            if constexpr (DT != ODMKV_F32) cur = nxt;
+            else if (it < 2 * a.ea_cpw - 1) cur.load(a.K, row_of(it + 1));
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
@@ -490,24 +503,37 @@ __global__ __launch_bounds__(256) void ea_final_kernel(ScoreArgs a) {
     }
     float best = 0.0f;
     const int t0 = chunk * ROWS_PER_WG;
-    for (int it = 0; it < ROWS_PER_WG / 16; ++it) {
-        const int t = t0 + it * 16 + wave * 4 + rsub;
-        const bool ok = t < a.Tc;
-        float x[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (ok && a.use_vnorm) load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, x);
-        float vn = 0.0f;
+    for (int it0 = 0; it0 < ROWS_PER_WG / 16; it0 += SC_UNROLL_V) {
+        float xs[SC_UNROLL_V][8], lg[SC_UNROLL_V][GMAX];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) vn = __fmaf_rn(x[e], x[e], vn);
-        vn = group16_sum(vn);
-        if (ok && part == 0) {
-            float acc = 0.0f;
+        for (int u = 0; u < SC_UNROLL_V; ++u) {
+            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
 #pragma unroll
-            for (int g = 0; g < GMAX; ++g)
-                if (g < a.G) acc += __expf(a.logits[((size_t)h * a.G + g) * a.Tc + t] - Mg[g]) / Zg[g];
-            const float pt = acc / (float)a.G;
-            const float sc = a.use_vnorm ? (pt + a.eps) * sqrtf(vn) : pt;
-            a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
-            best = fmaxf(best, sc);
+            for (int e = 0; e < 8; ++e) xs[u][e] = 0.0f;
+            if (t < a.Tc) {
+                if (a.use_vnorm) load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, xs[u]);
+#pragma unroll
+                for (int g = 0; g < GMAX; ++g)
+                    if (g < a.G && part == 0) lg[u][g] = a.logits[((size_t)h * a.G + g) * a.Tc + t];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < SC_UNROLL_V; ++u) {
+            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
+            float vn = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) vn = __fmaf_rn(xs[u][e], xs[u][e], vn);
+            vn = group16_sum(vn);
+            if (t < a.Tc && part == 0) {
+                float acc = 0.0f;
+#pragma unroll
+                for (int g = 0; g < GMAX; ++g)
+                    if (g < a.G) acc += __expf(lg[u][g] - Mg[g]) / Zg[g];
+                const float pt = acc / (float)a.G;
+                const float sc = a.use_vnorm ? (pt + a.eps) * sqrtf(vn) : pt;
+                a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
+                best = fmaxf(best, sc);
+            }
         }
     }
     best = wave_max(best);
@@ -586,7 +612,7 @@ extern "C" int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int
     a.K = K; a.V = V; a.sH = stride_h; a.sT = stride_t;
     a.Hkv = Hkv; a.Hq = Hq; a.G = Hq / Hkv; a.Gl = attn ? 0 : Hq / Hkv; a.T = T; a.Tc = T - n_sink; a.n_sink = n_sink;
     a.nchunks = n_chunks(a.Tc); a.eps = eps; a.mu = mu; a.attn = attn; a.scores = scores;
-    a.cov = nullptr; a.use_vnorm = 0;
+    a.cov = nullptr; a.use_vnorm = 0; a.ea_cpw = 1;
     a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
     a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
     a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);
@@ -607,7 +633,16 @@ static int run_expected(ScoreArgs& a, hipStream_t st) {
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds));
             attr_set = true;
         }
-        dim3 g2((a.nchunks + EA_CHUNKS_PER_WG - 1) / EA_CHUNKS_PER_WG, a.Hq);
+        // a workgroup loads its head's covariance (64 KB) once: give it as many chunks as still leaves
+        // two workgroups for every compute unit
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) == hipSuccess) {
+            int v = 0;
+            if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+        }
+        a.ea_cpw = EA_MAX_CHUNKS_PER_WG;
+        while (a.ea_cpw > 1 && (long)((a.nchunks + a.ea_cpw - 1) / a.ea_cpw) * a.Hq < 2L * cus) a.ea_cpw >>= 1;
+        dim3 g2((a.nchunks + a.ea_cpw - 1) / a.ea_cpw, a.Hq);
         hipLaunchKernelGGL((ea_logits_kernel<DT>), g2, block, lds, st, a);
         ODMKV_CHECK_LAUNCH("ea_logits_kernel");
     } else {
@@ -649,7 +684,7 @@ extern "C" int odmkv_score_expected(const void* K, const void* V, int dtype, int
     a.K = K; a.V = V; a.sH = stride_h; a.sT = stride_t;
     a.Hkv = Hkv; a.Hq = Hq; a.G = Hq / Hkv; a.Gl = a.G; a.T = T; a.Tc = T - n_sink; a.n_sink = n_sink;
     a.nchunks = n_chunks(a.Tc); a.eps = eps; a.mu = mu; a.attn = nullptr; a.scores = scores;
-    a.cov = cov; a.use_vnorm = use_vnorm ? 1 : 0;
+    a.cov = cov; a.use_vnorm = use_vnorm ? 1 : 0; a.ea_cpw = 1;
     a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
     a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
     a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);

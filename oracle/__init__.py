@@ -26,7 +26,9 @@ Pin status (what independent evidence fixes each function):
   rotation, 2-entry codebook = sign quantisation), relative MSE against the
   Lloyd-Max distortion table.
 * ``scorer.*``                        pinned: fp64 brute force on tiny inputs,
-  closed forms (uniform attention, G=1), scaling invariants.
+  closed forms (uniform attention, G=1), scaling invariants, and the reference's
+  own outputs in ``tests/golden`` (risk score: 5 cases; expected-attention score
+  with the query covariance: 6 cases incl. RoPE on mean and covariance).
 * ``allocator.optimal_scores_to_bits``  pinned: exhaustive Lagrangian argmin on
   tiny inputs, budget invariants, trivial-case clamps; token choice *inside* a
   group of equal scores at the repair cut-off is implementation-defined in the
