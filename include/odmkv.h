@@ -70,7 +70,8 @@ int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int T,
  *
  * mu: device fp32 [Hq, 128]; cov: device fp32 [Hq, 128, 128] (the RoPE-averaged query covariance),
  * or NULL for the mean-query term alone (use_covariance=False).  The quadratic form runs on the
- * fp32 matrix cores.  K, V, strides, scores and the workspace (odmkv_score_workspace_bytes) are
+ * matrix cores: 16-bit keys with cov split into two fp16 / three bf16 pieces (exact products, fp32
+ * sums), fp32 keys on the fp32 matrix instructions.  K, V, strides, scores and the workspace (odmkv_score_workspace_bytes) are
  * those of odmkv_score.
  */
 int odmkv_score_expected(const void* K, const void* V, int dtype, int Hkv, int T,

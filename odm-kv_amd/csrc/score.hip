@@ -22,6 +22,7 @@ struct ScoreArgs {
     const float* cov;     // [Hq, 128, 128] query covariance (expected-attention score only) or null
     int use_vnorm;        // expected-attention score: multiply (p + eps) by |v|
     int ea_cpw;           // expected-attention score: 256-token chunks a workgroup walks
+    int nstat;            // softmax statistics entries per query head (one per chunk, or one per wave and chunk)
     float* scores;        // [Hkv, T]
     float* logits;        // [Hq, Tc]
     float* kn2;           // [Hkv, Tc]
@@ -173,8 +174,8 @@ __global__ __launch_bounds__(64) void score_stats_kernel(ScoreArgs a) {
     if (hq == 0 && lane == 0) *a.gmax = 0u;
     if (a.Gl == 0) return;                    // attention weights were supplied: nothing to merge
     float m = -INFINITY, s = 0.0f;
-    for (int c = lane; c < a.nchunks; c += WAVE) {
-        const float* st = a.stats + ((size_t)hq * a.nchunks + c) * 2;
+    for (int c = lane; c < a.nstat; c += WAVE) {
+        const float* st = a.stats + ((size_t)hq * a.nstat + c) * 2;
         ms_merge(m, s, st[0], st[1]);
     }
 #pragma unroll
@@ -489,6 +490,158 @@ __global__ __launch_bounds__(256) void ea_logits_kernel(ScoreArgs a) {
     }
 }
 
+// ---- the same contraction for 16-bit keys, on the 16-bit matrix instructions ----------------------
+// K is exact in its own 16-bit type; Cov/(2d) is split into pieces of that type (two fp16 pieces after
+// scaling the head's largest entry to 2^14, or three bf16 pieces), so the products are exact and the
+// sum carries 22-24 bits of every covariance entry relative to the largest: the logits agree with the
+// fp32 kernel to ~1e-6.  v_mfma_f32_32x32x16_{f16,bf16}: operand A = 8 consecutive entries of row c of
+// a piece (one 16-byte LDS read), operand B = 8 consecutive elements of the lane's token row; a wave
+// takes 64 tokens at a time.
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+#define EA_ROW 136           // 16-bit entries per LDS row of a piece: 128 + 8, so that 16-byte reads of
+                             // consecutive rows fall on distinct banks
+
+template <int DT> struct Piece;
+template <> struct Piece<ODMKV_F16> {
+    static constexpr int NP = 2;
+    __device__ static inline f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Piece<ODMKV_BF16> {
+    static constexpr int NP = 3;
+    __device__ static inline f32x16 mfma(uint4 a, uint4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+
+// x -> NP values of the 16-bit type whose sum approximates x (each the rounding of what is left)
+template <int DT>
+__device__ static inline void split_pieces(float x, uint16_t* out) {
+#pragma unroll
+    for (int p = 0; p < Piece<DT>::NP; ++p) {
+        out[p] = Elem<DT>::from_f32(x);
+        x -= Elem<DT>::to_f32(out[p]);
+    }
+}
+
+template <int DT, int NW>
+__global__ __launch_bounds__(NW * 64) void ea_logits16_kernel(ScoreArgs a) {
+    constexpr int NP = Piece<DT>::NP, NT = NW * 64, CPI = NW / 4;      // CPI: 256-token chunks per iteration
+    constexpr int PER = HD * HD / 4 / NT;
+    extern __shared__ __align__(16) uint16_t piece_s[];               // [NP][128][EA_ROW]
+    __shared__ __align__(16) float mu_s[HD];                          // mu / sqrt(d), scaled like the pieces
+    __shared__ float red_a[NW];
+    const int hq = blockIdx.y, h = hq / a.G, tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, col = lane & 31, half = lane >> 5;
+    int kexp = 0;
+    {
+        const float4* src = reinterpret_cast<const float4*>(a.cov + (size_t)hq * HD * HD);
+        float4 v[PER];
+        float amax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            v[i] = src[tid + NT * i];
+            amax = fmaxf(fmaxf(amax, fmaxf(fabsf(v[i].x), fabsf(v[i].y))), fmaxf(fabsf(v[i].z), fabsf(v[i].w)));
+        }
+        amax = wave_max(amax);
+        if (lane == 0) red_a[wave] = amax;
+        __syncthreads();
+        amax = red_a[0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) amax = fmaxf(amax, red_a[w]);
+        if (DT == ODMKV_F16 && amax > 0.0f && amax < INFINITY) {     // fp16 pieces: largest entry of Cov/(2d) -> [2^13, 2^14)
+            int ex;
+            (void)frexpf(amax, &ex);
+            kexp = max(-60, min(60, 14 + 8 - ex));
+        }
+        const float sc = ldexpf(1.0f, kexp - 8);                     // includes the 1 / (2 d)
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e4 = tid + NT * i, row = e4 >> 5, c0 = (e4 & 31) * 4;
+            uint16_t px[NP], py[NP], pz[NP], pw[NP];
+            split_pieces<DT>(v[i].x * sc, px); split_pieces<DT>(v[i].y * sc, py);
+            split_pieces<DT>(v[i].z * sc, pz); split_pieces<DT>(v[i].w * sc, pw);
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+                *reinterpret_cast<uint2*>(piece_s + ((size_t)p * HD + row) * EA_ROW + c0) =
+                    make_uint2((uint32_t)px[p] | ((uint32_t)py[p] << 16), (uint32_t)pz[p] | ((uint32_t)pw[p] << 16));
+        }
+        if (tid < HD) mu_s[tid] = a.mu[(size_t)hq * HD + tid] / 11.313708498984761f * ldexpf(1.0f, kexp);
+    }
+    const float unscale = ldexpf(1.0f, -kexp);
+    __syncthreads();
+    const uint16_t* abase = piece_s + (size_t)col * EA_ROW + 8 * half;
+    for (int itn = 0; itn < a.ea_cpw; ++itn) {
+        const int chunk0 = (blockIdx.x * a.ea_cpw + itn) * CPI;
+        if (chunk0 >= a.nchunks) break;                               // the same for every thread of the workgroup
+        const int t0 = (chunk0 + (wave >> 2)) * ROWS_PER_WG + (wave & 3) * 64;
+        float m = -INFINITY, s = 0.0f;
+        if (t0 < a.Tc) {                                              // wave-uniform
+            // Two blocks of 32 tokens share every A operand: one 16-byte LDS read feeds two matrix
+            // instructions (with one read per instruction the LDS pipe, 128 bytes per clock and compute
+            // unit, is exactly as fast as the matrix pipes and sets the time).  The 32-column blocks of the
+            // covariance go one after the other, so that only two accumulator blocks are live.
+            RowRegs<DT> r0, r1;                                       // rows past the end repeat the last row and are not stored
+            r0.load(a.K, (size_t)h * a.sH + (size_t)(a.n_sink + min(t0 + col, a.Tc - 1)) * a.sT);
+            r1.load(a.K, (size_t)h * a.sH + (size_t)(a.n_sink + min(t0 + 32 + col, a.Tc - 1)) * a.sT);
+            float lg0 = 0.0f, lg1 = 0.0f;
+#pragma unroll
+            for (int cb = 0; cb < 4; ++cb) {
+                f32x16 acc0, acc1;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 mv = *reinterpret_cast<const float4*>(mu_s + 32 * cb + 8 * q + 4 * half);
+                    acc0[4 * q] = mv.x; acc0[4 * q + 1] = mv.y; acc0[4 * q + 2] = mv.z; acc0[4 * q + 3] = mv.w;
+                }
+                acc1 = acc0;
+#pragma unroll
+                for (int st = 0; st < 8; ++st) {
+                    const uint4 b0 = half ? r0.r[2 * st + 1] : r0.r[2 * st];
+                    const uint4 b1 = half ? r1.r[2 * st + 1] : r1.r[2 * st];
+#pragma unroll
+                    for (int p = 0; p < NP; ++p) {
+                        const uint4 av = *reinterpret_cast<const uint4*>(abase + ((size_t)p * HD + 32 * cb) * EA_ROW + 16 * st);
+                        acc0 = Piece<DT>::mfma(av, b0, acc0);
+                        acc1 = Piece<DT>::mfma(av, b1, acc1);
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float x0[4], x1[4];
+                    r0.quad(32 * cb + 8 * q, half, x0);
+                    r1.quad(32 * cb + 8 * q, half, x1);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        lg0 = __fmaf_rn(x0[j], acc0[4 * q + j], lg0);
+                        lg1 = __fmaf_rn(x1[j], acc1[4 * q + j], lg1);
+                    }
+                }
+            }
+            lg0 += __shfl_xor(lg0, 32, WAVE);
+            lg1 += __shfl_xor(lg1, 32, WAVE);
+            const float lg = (half ? lg1 : lg0) * unscale;            // the upper half of the wave stores the second block
+            const int t = t0 + 32 * half + col;
+            if (t < a.Tc) {
+                a.logits[(size_t)hq * a.Tc + t] = lg;
+                ms_merge(m, s, lg, 1.0f);
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float m2 = __shfl_xor(m, o, WAVE), s2 = __shfl_xor(s, o, WAVE);
+            ms_merge(m, s, m2, s2);
+        }
+        // one entry per wave and chunk: the waves of a workgroup never wait for each other in this loop
+        const int chunk = chunk0 + (wave >> 2);
+        if (lane == 0 && chunk < a.nchunks) {
+            float* st = a.stats + ((size_t)hq * a.nstat + chunk * 4 + (wave & 3)) * 2;
+            st[0] = m; st[1] = s;
+        }
+    }
+}
+
 // p from the logits, then (p + eps) * |v| (or p alone), and the running maximum
 template <int DT, int GMAX>
 __global__ __launch_bounds__(256) void ea_final_kernel(ScoreArgs a) {
@@ -553,7 +706,7 @@ static ScoreLayout score_layout(int Hkv, int Hq, int T) {
     L.logits = take((size_t)Hq * Tc * 4);
     L.kn2 = take((size_t)Hkv * Tc * 4);
     L.p = take((size_t)Hkv * Tc * 4);
-    L.stats = take((size_t)Hq * nc * 8);
+    L.stats = take((size_t)Hq * nc * 4 * 8);        // up to one entry per wave and chunk
     L.mz = take((size_t)Hq * 8);
     L.opart = take((size_t)Hkv * nc * HD * 4);
     L.psum = take((size_t)Hkv * nc * 4);
@@ -612,7 +765,7 @@ extern "C" int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int
     a.K = K; a.V = V; a.sH = stride_h; a.sT = stride_t;
     a.Hkv = Hkv; a.Hq = Hq; a.G = Hq / Hkv; a.Gl = attn ? 0 : Hq / Hkv; a.T = T; a.Tc = T - n_sink; a.n_sink = n_sink;
     a.nchunks = n_chunks(a.Tc); a.eps = eps; a.mu = mu; a.attn = attn; a.scores = scores;
-    a.cov = nullptr; a.use_vnorm = 0; a.ea_cpw = 1;
+    a.cov = nullptr; a.use_vnorm = 0; a.ea_cpw = 1; a.nstat = a.nchunks;
     a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
     a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
     a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);
@@ -626,24 +779,36 @@ template <int DT>
 static int run_expected(ScoreArgs& a, hipStream_t st) {
     dim3 grid(a.nchunks, a.Hkv), block(256);
     if (a.cov) {
-        static bool attr_set = false;
-        const int lds = HD * HD * (int)sizeof(float);
-        if (!attr_set) {
-            ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ea_logits_kernel<DT>),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-            attr_set = true;
-        }
-        // a workgroup loads its head's covariance (64 KB) once: give it as many chunks as still leaves
-        // two workgroups for every compute unit
+        // A workgroup prepares its head's covariance (64 KB) once: give it as many chunks as still leaves
+        // `per_cu` workgroups for every compute unit.
         int dev = 0, cus = 256;
         if (hipGetDevice(&dev) == hipSuccess) {
             int v = 0;
             if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
         }
-        a.ea_cpw = EA_MAX_CHUNKS_PER_WG;
-        while (a.ea_cpw > 1 && (long)((a.nchunks + a.ea_cpw - 1) / a.ea_cpw) * a.Hq < 2L * cus) a.ea_cpw >>= 1;
-        dim3 g2((a.nchunks + a.ea_cpw - 1) / a.ea_cpw, a.Hq);
-        hipLaunchKernelGGL((ea_logits_kernel<DT>), g2, block, lds, st, a);
+        auto pick = [&](int cpi, int max_cpw, int per_cu) {
+            int cpw = max_cpw;
+            while (cpw > 1 && (long)((a.nchunks + cpi * cpw - 1) / (cpi * cpw)) * a.Hq < (long)per_cu * cus) cpw >>= 1;
+            a.ea_cpw = cpw;
+            return dim3((a.nchunks + cpi * cpw - 1) / (cpi * cpw), a.Hq);
+        };
+        // the attribute belongs to the function on the current device: set on every call (layers of one
+        // model may live on several devices)
+        if constexpr (DT == ODMKV_F32) {
+            const int lds = HD * HD * (int)sizeof(float);
+            ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ea_logits_kernel<DT>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            const dim3 g2 = pick(1, EA_MAX_CHUNKS_PER_WG, 2);
+            hipLaunchKernelGGL((ea_logits_kernel<DT>), g2, block, lds, st, a);
+        } else {
+            constexpr int NW = DT == ODMKV_F16 ? 4 : 8;        // three bf16 pieces leave room for one workgroup: eight waves
+            const int lds = Piece<DT>::NP * HD * EA_ROW * (int)sizeof(uint16_t);
+            ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&ea_logits16_kernel<DT, NW>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            const dim3 g2 = pick(NW / 4, 8, DT == ODMKV_F16 ? 2 : 1);
+            a.nstat = a.nchunks * 4;
+            hipLaunchKernelGGL((ea_logits16_kernel<DT, NW>), g2, dim3(NW * 64), lds, st, a);
+        }
         ODMKV_CHECK_LAUNCH("ea_logits_kernel");
     } else {
         if (a.G <= 4) hipLaunchKernelGGL((score_logits_kernel<DT, 4>), grid, block, 0, st, a);
@@ -684,7 +849,7 @@ extern "C" int odmkv_score_expected(const void* K, const void* V, int dtype, int
     a.K = K; a.V = V; a.sH = stride_h; a.sT = stride_t;
     a.Hkv = Hkv; a.Hq = Hq; a.G = Hq / Hkv; a.Gl = a.G; a.T = T; a.Tc = T - n_sink; a.n_sink = n_sink;
     a.nchunks = n_chunks(a.Tc); a.eps = eps; a.mu = mu; a.attn = nullptr; a.scores = scores;
-    a.cov = cov; a.use_vnorm = use_vnorm ? 1 : 0; a.ea_cpw = 1;
+    a.cov = cov; a.use_vnorm = use_vnorm ? 1 : 0; a.ea_cpw = 1; a.nstat = a.nchunks;
     a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
     a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
     a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);

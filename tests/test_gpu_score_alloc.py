@@ -231,3 +231,24 @@ def test_expected_attention_scorer_matches_reference_vectors(golden, name):
     with torch.no_grad():
         got16 = sc.score_prefill(k.half().to(DEV), v.half().to(DEV), 0, module=mod.half(), hidden_states=h.half().to(DEV))
     np.testing.assert_allclose(got16.cpu().numpy(), golden[f"ea_{name}_out"], rtol=2e-2, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("cov_scale", [1e-9, 1.0, 3e3])
+def test_expected_attention_covariance_pieces_keep_fp32_accuracy(dtype, cov_scale):
+    """16-bit keys take the 16-bit matrix instructions with the covariance split into fp16 / bf16 pieces
+    (fp16 after scaling the head's largest entry): whatever the covariance's magnitude, the scores must be
+    as close to the fp64 oracle as the fp32 path is, far inside the 1e-3 bar."""
+    from kvquant.scorer import _launch_score_expected
+    g = torch.Generator().manual_seed(91)
+    hkv, hq, T = 2, 8, 900
+    k = (torch.randn(hkv, T, 128, generator=g) * (0.02 if cov_scale > 1 else 1.0)).to(dtype)
+    v = torch.randn(hkv, T, 128, generator=g).to(dtype)
+    mu = torch.randn(1, hq, 128, generator=g)
+    a = torch.randn(1, hq, 128, 24, generator=g) * 0.2
+    cov = (a @ a.transpose(-1, -2) + 0.05 * torch.eye(128)) * cov_scale
+    cov[0, 3] *= 1e-4                                  # heads of very different magnitude
+    want = osc.expected_attention_score(k.double(), v.double(), mu.double(), cov.double(), hq, n_sink=4,
+                                        epsilon=1e-2, use_vnorm=True)
+    got = _launch_score_expected(k.to(DEV), v.to(DEV), mu[0].to(DEV), cov[0].to(DEV), hq, 4, 1e-2, True)
+    np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=2e-5)
