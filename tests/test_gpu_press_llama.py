@@ -32,10 +32,11 @@ def _model(seed=0, layers=2):
     return LlamaForCausalLM(cfg).to(device=DEV, dtype=torch.float16).eval()
 
 
-def _press(target=2.5, buffer_size=128, **kw):
+def _press(target=2.5, buffer_size=128, scorer=None, **kw):
     from kvquant import RiskScorer, TurboQuantPerTokenBackendPress
-    scorer = RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
-    scorer.normalize_grain = "global"
+    if scorer is None:
+        scorer = RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
+        scorer.normalize_grain = "global"
     return TurboQuantPerTokenBackendPress(
         scorer=scorer, bit_levels=LEVELS, target_avg_bits=target, eviction_cost=0.5, seed=42, decode_quant=True,
         sink_tokens=4, layerwise=True, key_quantizer="mse", value_quantizer="mse", buffer_size=buffer_size, **kw)
@@ -308,3 +309,26 @@ def test_bf16_model_fused_matches_dense_path():
     assert states[0]._exact_torch_dtype == torch.bfloat16
     assert (log_f - log_d).abs().max().item() < 0.06
     assert (log_f.argmax(-1) == tok_d).float().mean().item() >= 0.95
+
+
+def test_press_with_expected_attention_scorer():
+    """The press with the reference's other scorer class (mean query + query covariance, the default
+    layer-wise min-max normalisation): the budget holds, sinks and the window stay exact, the fused decode
+    agrees with the dense path, and a 130-step decode crosses a buffer flush."""
+    from kvquant import ExpectedAttentionScorer
+    def scorer():
+        return ExpectedAttentionScorer(n_future_positions=512, n_sink=4, use_covariance=True, use_vnorm=True, epsilon=1e-2)
+    model = _model(5)
+    ids = _ids(600, 21)
+    n_new = 130
+    tok_d, log_d, _, _ = _generate(model, _press(scorer=scorer()), ids, n_new, fused=False)
+    tok_f, log_f, cache, states = _generate(model, _press(scorer=scorer()), ids, n_new, forced=tok_d, fused=True)
+    assert (log_f - log_d).abs().max().item() < LOGIT_ATOL
+    for st in states.values():
+        lm = st._level_map[0, :, :600].float()
+        assert torch.all(lm[:, :4] == 16) and torch.all(lm[:, 600 - 128:] == 16)
+        core = lm[:, 4:600 - 128]
+        assert set(core.unique().tolist()) <= set(float(b) for b in LEVELS)
+        # the budget is met over all non-sink tokens before the window is forced to 16 bits, so the mean over
+        # the tokens in front of the window sits near the target, not exactly under it
+        assert abs(core.mean().item() - 2.5) < 0.1
