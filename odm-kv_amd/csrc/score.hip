@@ -52,6 +52,33 @@ __device__ static inline void load8(const void* base, size_t elem_off, float* x)
     }
 }
 
+// the same 8 elements as raw registers (so that a later trip's rows can be requested before the current
+// trip's are converted and used), and their conversion
+template <int DT> struct Raw8 { uint4 a; };
+template <> struct Raw8<ODMKV_F32> { float4 a, b; };
+template <int DT>
+__device__ static inline void load8_raw(const void* base, size_t elem_off, Raw8<DT>& r) {
+    if constexpr (DT == ODMKV_F32) {
+        const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(base) + elem_off);
+        r.a = p[0]; r.b = p[1];
+    } else {
+        r.a = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + elem_off);
+    }
+}
+template <int DT>
+__device__ static inline void cvt8(const Raw8<DT>& r, float* x) {
+    if constexpr (DT == ODMKV_F32) {
+        x[0] = r.a.x; x[1] = r.a.y; x[2] = r.a.z; x[3] = r.a.w; x[4] = r.b.x; x[5] = r.b.y; x[6] = r.b.z; x[7] = r.b.w;
+    } else {
+        const uint32_t w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            x[2 * e] = Elem<DT>::to_f32((uint16_t)(w[e] & 0xffffu));
+            x[2 * e + 1] = Elem<DT>::to_f32((uint16_t)(w[e] >> 16));
+        }
+    }
+}
+
 // sum over the 16 lanes that share a row, by data-parallel-primitive moves (no LDS traffic): inside the
 // quad, then the neighbouring quad, then the other half of the 16-lane row.  Every lane ends with the
 // total; the order of the additions is fixed per lane (only lane 0 of the row is used).
@@ -94,7 +121,7 @@ __global__ __launch_bounds__(256) void score_logits_kernel(ScoreArgs a) {
     float m[GMAX], s[GMAX];
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) { m[g] = -INFINITY; s[g] = 0.0f; }
-    const float inv_div = 11.313708498984761f;        // sqrt(128)
+    const float inv_sqrt_d = 0.08838834764831845f;    // 1 / sqrt(128): a multiplication, one rounding like the division
     const int t0 = chunk * ROWS_PER_WG;
     // A group of 16 lanes takes four consecutive rows per trip (all four requested before any is
     // used).  The row sums leave the reduction in every lane of the group, so lane u < 4 of the group
@@ -102,17 +129,23 @@ __global__ __launch_bounds__(256) void score_logits_kernel(ScoreArgs a) {
     // and keeps the running softmax statistics of its rows.
     static_assert(SC_UNROLL == 4, "four rows per lane group and trip");
     const bool owner = part < SC_UNROLL;
+    // rows of the next trip are requested before the current trip's are used; rows past the end repeat the
+    // last row (never stored)
+    auto request = [&](int it0, Raw8<DT>* raw) {
+        const int tb = t0 + it0 * 16 + (wave * 4 + rsub) * SC_UNROLL;
+#pragma unroll
+        for (int u = 0; u < SC_UNROLL; ++u)
+            load8_raw<DT>(a.K, (size_t)h * a.sH + (size_t)(a.n_sink + min(tb + u, a.Tc - 1)) * a.sT + part * 8, raw[u]);
+    };
+    Raw8<DT> raw[SC_UNROLL], nraw[SC_UNROLL];
+    request(0, raw);
+#pragma unroll                 // straight-line code: the wait before a trip's first use counts only that trip's loads
     for (int it0 = 0; it0 < ROWS_PER_WG / 16; it0 += SC_UNROLL) {
         const int tb = t0 + it0 * 16 + (wave * 4 + rsub) * SC_UNROLL;
+        if (it0 + SC_UNROLL < ROWS_PER_WG / 16) request(it0 + SC_UNROLL, nraw);
         float xs[SC_UNROLL][8];
 #pragma unroll
-        for (int u = 0; u < SC_UNROLL; ++u) {
-            if (tb + u < a.Tc) load8<DT>(a.K, (size_t)h * a.sH + (size_t)(a.n_sink + tb + u) * a.sT + part * 8, xs[u]);
-            else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) xs[u][e] = 0.0f;
-            }
-        }
+        for (int u = 0; u < SC_UNROLL; ++u) cvt8<DT>(raw[u], xs[u]);
         float kn_own = 0.0f, d_own[GMAX];
 #pragma unroll
         for (int g = 0; g < GMAX; ++g) d_own[g] = 0.0f;
@@ -130,7 +163,7 @@ __global__ __launch_bounds__(256) void score_logits_kernel(ScoreArgs a) {
                     float d = 0.0f;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) d = __fmaf_rn(x[e], mu_r[g][e], d);
-                    d = group16_sum(d) / inv_div;
+                    d = group16_sum(d) * inv_sqrt_d;
                     d_own[g] = part == u ? d : d_own[g];
                 }
             }
@@ -146,6 +179,8 @@ __global__ __launch_bounds__(256) void score_logits_kernel(ScoreArgs a) {
                 }
             }
         }
+#pragma unroll
+        for (int u = 0; u < SC_UNROLL; ++u) raw[u] = nraw[u];
     }
     // only the owner lanes hold statistics; butterfly over the wave, then over the 4 waves
 #pragma unroll
@@ -197,8 +232,9 @@ __global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) {
         Mg[g] = (a.attn == nullptr && g < a.G) ? a.mz[2 * (h * a.G + g)] : 0.0f;
-        Zg[g] = (a.attn == nullptr && g < a.G) ? a.mz[2 * (h * a.G + g) + 1] : 1.0f;
+        Zg[g] = (a.attn == nullptr && g < a.G) ? 1.0f / a.mz[2 * (h * a.G + g) + 1] : 1.0f;   // reciprocal of the sum
     }
+    const float inv_g = 1.0f / (float)a.G;
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     float ps = 0.0f;
     const int t0 = chunk * ROWS_PER_WG;
@@ -228,8 +264,8 @@ __global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
                     float acc = 0.0f;
 #pragma unroll
                     for (int g = 0; g < GMAX; ++g)
-                        if (g < a.G) acc += __expf(lg[u][g] - Mg[g]) / Zg[g];
-                    pt = acc / (float)a.G;
+                        if (g < a.G) acc = __fmaf_rn(__expf(lg[u][g] - Mg[g]), Zg[g], acc);
+                    pt = acc * inv_g;
                 }
                 if (part == 0) { a.p[(size_t)h * a.Tc + t] = pt; ps += pt; }
 #pragma unroll
@@ -315,7 +351,7 @@ __global__ __launch_bounds__(256) void score_final_kernel(ScoreArgs a) {
             ir = group16_sum(ir);
             if (ok && part == 0) {
                 const float pe = pin[u] + a.eps;
-                const float kterm = (knin[u] / (float)HD) * ir;
+                const float kterm = (knin[u] * (1.0f / (float)HD)) * ir;      // 1/128: exact
                 const float sc = (pe * pe) * (vn + kterm);
                 a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
                 best = fmaxf(best, sc);
@@ -652,8 +688,9 @@ __global__ __launch_bounds__(256) void ea_final_kernel(ScoreArgs a) {
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) {
         Mg[g] = g < a.G ? a.mz[2 * (h * a.G + g)] : 0.0f;
-        Zg[g] = g < a.G ? a.mz[2 * (h * a.G + g) + 1] : 1.0f;
+        Zg[g] = g < a.G ? 1.0f / a.mz[2 * (h * a.G + g) + 1] : 1.0f;   // reciprocal of the sum
     }
+    const float inv_g = 1.0f / (float)a.G;
     float best = 0.0f;
     const int t0 = chunk * ROWS_PER_WG;
     for (int it0 = 0; it0 < ROWS_PER_WG / 16; it0 += SC_UNROLL_V) {
@@ -681,8 +718,8 @@ __global__ __launch_bounds__(256) void ea_final_kernel(ScoreArgs a) {
                 float acc = 0.0f;
 #pragma unroll
                 for (int g = 0; g < GMAX; ++g)
-                    if (g < a.G) acc += __expf(lg[u][g] - Mg[g]) / Zg[g];
-                const float pt = acc / (float)a.G;
+                    if (g < a.G) acc = __fmaf_rn(__expf(lg[u][g] - Mg[g]), Zg[g], acc);
+                const float pt = acc * inv_g;
                 const float sc = a.use_vnorm ? (pt + a.eps) * sqrtf(vn) : pt;
                 a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
                 best = fmaxf(best, sc);
