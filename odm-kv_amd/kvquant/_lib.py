@@ -108,7 +108,19 @@ def require_gpu(t: torch.Tensor, what: str) -> None:
         raise RuntimeError(f"{what} must live on the GPU: the ODM-KV kernels have no CPU path")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device) -> int:
+    """The current stream of `device` as a raw handle (called twice per layer and decode step: the raw
+    query is several times cheaper than building a torch.cuda.Stream object)."""
+    if _raw_stream is not None:
+        idx = getattr(device, "index", None)
+        if idx is None:
+            idx = torch.device(device).index
+        if idx is None:
+            idx = torch.cuda.current_device()
+        return _raw_stream(idx)
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -121,7 +133,7 @@ _ws_cache: dict[tuple, torch.Tensor] = {}
 
 def workspace(device, nbytes: int, tag: str = "") -> torch.Tensor:
     """A reusable scratch buffer per (device, stream, tag); grown, never shrunk."""
-    key = (str(device), torch.cuda.current_stream(device).cuda_stream, tag)
+    key = (str(device), stream_ptr(device), tag)
     buf = _ws_cache.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)

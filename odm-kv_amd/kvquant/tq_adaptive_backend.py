@@ -113,6 +113,7 @@ class TurboQuantAdaptiveKVCacheState:
         self.seq_len = 0
         self._nseg = 0
         self._counts = None           # np.int64 [5, nseg]   tokens stored per level and segment
+        self._exact_room = None       # tokens every exact segment can still take (None: not known)
         self._seg_tile = None         # np.int64 [5, nseg+1] first tile of each segment
         self._bufs = None
         self._level_store = None      # uint8 [B, H, capacity]: bit level of every position (grown by doubling)
@@ -255,6 +256,7 @@ class TurboQuantAdaptiveKVCacheState:
                 new["seg_count"][li].copy_(old["seg_count"][li])
         self._bufs = new
         self._seg_tile = seg_tile
+        self._exact_room = None
         self._make_struct()
 
     # ------------------------------------------------------------------ validation
@@ -323,6 +325,7 @@ class TurboQuantAdaptiveKVCacheState:
             self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
             C.byref(self._packed), ws.data_ptr(), ws_bytes, st))
         self._counts = new_counts
+        self._exact_room = None
         lm = bits.to(torch.uint8)
         if _pos_offset is None:
             self._extend_levels(lm)
@@ -342,17 +345,27 @@ class TurboQuantAdaptiveKVCacheState:
             bits = torch.full((B, H, T), 16, dtype=torch.int32, device=self.device)
             self.append(keys, values, bits)
             return
-        new_counts = self._counts.copy()
-        new_counts[4] += 1
         had = self._seg_tile
-        self._ensure_capacity(new_counts)
+        room = self._exact_room
+        new_counts = None
+        if room is None or room <= 0:
+            new_counts = self._counts.copy()
+            new_counts[4] += 1
+            self._ensure_capacity(new_counts)
+            # tokens every exact segment can still take before a tile has to be added (the usual decode step
+            # then skips the capacity arithmetic)
+            room = int((np.diff(self._seg_tile[4]) * TILE - new_counts[4]).min()) + 1
         # the token is read where it lies (the newest row of the model's cache): no staging copies
         k, v = keys[:, :, 0, :], values[:, :, 0, :]
         if k.stride(2) != 1 or v.stride() != k.stride():
             k, v = k.contiguous(), v.contiguous()
         _lib.check(lib.odmkv_append_exact(C.byref(self._packed), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1),
                                           self.seq_len, _lib.stream_ptr(self.device)))
-        self._counts = new_counts
+        if new_counts is None:
+            self._counts[4] += 1
+        else:
+            self._counts = new_counts
+        self._exact_room = room - 1
         if self._level_store.shape[2] < self.seq_len + 1:
             self._extend_levels(torch.full((B, H, 1), 16, dtype=torch.uint8, device=self.device))
         # otherwise nothing to write: the level store reads 16 behind seq_len (an exact token leaves
@@ -378,6 +391,7 @@ class TurboQuantAdaptiveKVCacheState:
                 if c:
                     first = int(self._seg_tile[li, s]) * TILE
                     self._counts[li, s] = int(np.searchsorted(pos[first:first + c], seq_len, side="left"))
+                    self._exact_room = None
             self._bufs["seg_count"][li].copy_(torch.from_numpy(self._counts[li].astype(np.int32)))
         self._items = None
 
@@ -481,6 +495,7 @@ class TurboQuantAdaptiveKVCacheState:
         bits = new_bits.to(device=self.device, dtype=torch.int32).reshape(B, H, n_buf)
         # drop the buffered tokens from the exact segments, then append them at their new levels
         self._counts[4] -= n_buf
+        self._exact_room = None
         self._bufs["seg_count"][4].copy_(torch.from_numpy(self._counts[4].astype(np.int32)))
         self.append(k, v, bits, _pos_offset=start)
 
