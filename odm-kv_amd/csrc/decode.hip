@@ -393,6 +393,9 @@ __device__ static inline void compute_tile(const TileData<W>& t, int nvalid, int
     PV_STEP(8) PV_STEP(9) PV_STEP(10) PV_STEP(11) PV_STEP(12) PV_STEP(13) PV_STEP(14) PV_STEP(15)
 }
 
+// LDS row of one head's query halves: 32 steps of 16 bytes plus one of padding, so that the four heads a
+// wavefront reads in one instruction (lane % 4) sit on different banks
+#define QS 33
 // stage the group's queries (fp16 high/low halves per 4-dim step) in LDS; heads beyond the group are 0
 template <int NP>
 __device__ static inline uint4 load_query_slice(const DecodeArgs& a, const uint4* src, int tid, int nheads) {
@@ -400,7 +403,7 @@ __device__ static inline uint4 load_query_slice(const DecodeArgs& a, const uint4
 }
 template <int NP>
 __device__ static inline void stage_queries(uint4 v, uint4* qsh, int tid) {
-    if (tid < 4 * NP * 32) qsh[tid] = v;
+    if (tid < 4 * NP * 32) qsh[(tid >> 5) * QS + (tid & 31)] = v;
 }
 template <int NP>
 __device__ static inline void fetch_queries(const uint4* qsh, int lane, h4* qr, h4* ql) {
@@ -408,7 +411,7 @@ __device__ static inline void fetch_queries(const uint4* qsh, int lane, h4* qr, 
     for (int p = 0; p < NP; ++p)
 #pragma unroll
         for (int s = 0; s < 32; ++s) {
-            const uint4 v = qsh[(4 * p + (lane & 3)) * 32 + s];
+            const uint4 v = qsh[(4 * p + (lane & 3)) * QS + s];
             qr[p * 32 + s] = as_h4(v.x, v.y);
             ql[p * 32 + s] = as_h4(v.z, v.w);
         }
@@ -562,7 +565,7 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
     for (int p = 0; p < NP; ++p)
 #pragma unroll
         for (int s = 0; s < 32; ++s) {
-            const uint2 v = *reinterpret_cast<const uint2*>(&qsh[(4 * p + (lane & 3)) * 32 + s]);
+            const uint2 v = *reinterpret_cast<const uint2*>(&qsh[(4 * p + (lane & 3)) * QS + s]);
             qr[p * 32 + s] = as_h4(v.x, v.y);
         }
     while (nvalid > 0) {
@@ -580,7 +583,7 @@ template <int NP, bool MULTI, bool ORDERED>
 __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs a) {
     __shared__ __align__(16) uint8_t lut[LUT_BYTES];     // centroid table; reused to combine the wavefronts
     __shared__ float wm[NWAVES][4 * NP], wl[NWAVES][4 * NP];
-    __shared__ uint4 qsh[4 * NP * 32];
+    __shared__ uint4 qsh[4 * NP * QS];
 
     // A GQA group of more than four query heads is served four heads at a time by separate workgroups
     // of the same item (the item's codes are read once per pass; the second read mostly hits the caches).
