@@ -80,6 +80,24 @@ int odmkv_score_expected(const void* K, const void* V, int dtype, int Hkv, int T
                          int use_vnorm, float* scores, void* workspace, size_t workspace_bytes,
                          void* stream);
 
+/* Observation-window attention mass (the per-query form of the scorer's attention estimate; the
+ * reference scores with one query per head, the mean query: kvquant/scorer.py:285-318, and has no
+ * counterpart of this entry point):
+ *
+ *   p[h,t] = mean over the W window queries and the G heads of kv-head h of
+ *            softmax_t( Q[q,w] . K[h,t] * scaling ),  t >= n_sink,
+ *   causal inside the window: query w stands at position q_pos0 + w and sees keys at positions <= its own.
+ *
+ * K: [Hkv, T, 128] float16 or bfloat16 (strides as for odmkv_score); Q: [Hq, W, 128] of the same type,
+ * contiguous, already rotated to their positions (post-RoPE); q_pos0 >= n_sink.  p: device fp32
+ * [Hkv, T - n_sink] out; it can be handed to odmkv_score as `attn` over the core tokens.  Runs on the
+ * 16-bit matrix cores, two passes over K, logits are not stored.
+ */
+size_t odmkv_window_attention_workspace_bytes(int Hkv, int Hq, int W, int T);
+int odmkv_window_attention(const void* K, int dtype, int Hkv, int T, int64_t stride_h, int64_t stride_t,
+                           const void* Q, int Hq, int W, int q_pos0, int n_sink, float scaling,
+                           float* p, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Allocator.  Replaces optimal_scores_to_bits (kvquant/allocator.py:459-663) for a batch of
  * independent rows (one row = one (layer, sequence): the flattened [Hkv, T] scores).

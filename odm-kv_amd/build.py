@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libodmkv.so")
-SOURCES = ["error.hip", "score.hip", "allocate.hip", "pack.hip", "rows.hip", "decode.hip"]
+SOURCES = ["error.hip", "score.hip", "window.hip", "allocate.hip", "pack.hip", "rows.hip", "decode.hip"]
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

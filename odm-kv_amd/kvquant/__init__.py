@@ -9,6 +9,7 @@ from kvquant.allocator import (
     calibrate_epsilon, effective_bits, DEFAULT_BIT_LEVELS,
 )
 from kvquant.scorer import BaseScorer, ExpectedAttentionScorer, RiskScorer
+from kvquant.scorer import WindowRiskScorer          # not in the reference: per-query observation-window variant (opt-in)
 
 _LAZY = {
     "TurboQuantPerTokenBackendPress": "kvquant.adaptive_backend_press",

@@ -212,3 +212,70 @@ class RiskScorer(ExpectedAttentionScorer):
     def score_with_attn(self, keys, values, attn_weights, *, module=None):
         H = keys.shape[0]
         return _launch_score(keys, values, None, attn_weights, H, 0, self.epsilon)
+
+
+def _launch_window_attention(keys: torch.Tensor, queries: torch.Tensor, n_sink: int, q_pos0: int,
+                             scaling: float) -> torch.Tensor:
+    """p fp32 [Hkv, T - n_sink]: attention mass of the window queries [Hq, W, d] (rotated to positions
+    q_pos0 .. q_pos0 + W - 1) over the core keys, per-query causal softmax, mean over queries and group."""
+    _lib.require_gpu(keys, "keys")
+    if keys.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError(f"window attention runs on the 16-bit matrix cores: keys must be float16 or bfloat16, got {keys.dtype}")
+    if keys.shape[-1] != _lib.HEAD_DIM:
+        raise ValueError(f"the HIP kernels are written for head_dim {_lib.HEAD_DIM}, got {keys.shape[-1]}")
+    if keys.stride(-1) != 1 or keys.stride(0) % 8 or keys.stride(1) % 8 or keys.data_ptr() % 16:
+        keys = keys.contiguous()
+    H, T, D = keys.shape
+    Hq, W, _ = queries.shape
+    q = queries.to(keys.dtype).contiguous()
+    dev = keys.device
+    p = torch.empty(H, T - n_sink, dtype=torch.float32, device=dev)
+    ws_bytes = lib.odmkv_window_attention_workspace_bytes(H, Hq, W, T)
+    ws = _lib.workspace(dev, ws_bytes, "window")
+    _lib.check(lib.odmkv_window_attention(
+        keys.data_ptr(), _lib.dtype_code(keys), H, T, keys.stride(0), keys.stride(1), q.data_ptr(), Hq, W,
+        int(q_pos0), int(n_sink), float(scaling), p.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
+    return p
+
+
+class WindowRiskScorer(RiskScorer):
+    """The risk score with the attention estimate taken from the prompt's last `window` queries, each
+    with its own causal softmax, instead of from the one mean query (not in the reference; opt-in).
+
+        p_j = mean over window queries and GQA group of softmax_j(q . k_j / sqrt(d)),   s_j as in RiskScorer
+
+    The queries are the module's own (q_proj / q_norm, RoPE at their positions); keys must be 16-bit."""
+
+    def __init__(self, *, window: int = 64, **kw):
+        super().__init__(**kw)
+        if window < 1:
+            raise ValueError("window must be at least 1")
+        self.window = int(window)
+
+    def _window_queries(self, module: nn.Module, hidden_states: torch.Tensor, w: int) -> torch.Tensor:
+        q_len = hidden_states.shape[1]
+        q = _get_query_states(module, hidden_states[:, q_len - w:])              # [1, Hq, w, d], pre-RoPE
+        rotary_emb = getattr(module, "rotary_emb", None)
+        if rotary_emb is not None:
+            pos = torch.arange(q_len - w, q_len, device=q.device).unsqueeze(0)
+            cos, sin = _aligned_rotary_outputs(rotary_emb, q, pos)
+            q = _apply_rotary_pos_emb_q(q, cos, sin)
+        return q[0]
+
+    def score_prefill(self, keys, values, layer_idx, *, module=None, hidden_states=None):
+        if module is None or hidden_states is None:
+            return self._fallback.score_prefill(keys, values, layer_idx)
+        if keys.shape[1] <= self.n_sink:
+            return torch.ones(keys.shape[:2], device=keys.device, dtype=keys.dtype)
+        if hidden_states.dim() == 2:
+            hidden_states = hidden_states.unsqueeze(0)
+        H, T, D = keys.shape
+        w = min(self.window, T - self.n_sink, hidden_states.shape[1])
+        try:
+            queries = self._window_queries(module, hidden_states, w)
+        except (AttributeError, NotImplementedError):
+            return self._fallback.score_prefill(keys, values, layer_idx)
+        p = _launch_window_attention(keys, queries, self.n_sink, T - w, D ** -0.5)
+        core = _launch_score(keys[:, self.n_sink:], values[:, self.n_sink:], None, p, H, 0, self.epsilon)
+        top = core.max().reshape(1, 1).expand(H, self.n_sink)
+        return self._maybe_normalize(torch.cat([top, core], dim=1))

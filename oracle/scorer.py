@@ -7,6 +7,9 @@ Follows /root/reference/kvquant/scorer.py
   RiskScorer.score_prefill                    :385-404
   RiskScorer.score_with_attn                  :406-416
   ExpectedAttentionScorer.score_prefill       :204-257  (expected_attention_score below)
+window_attention / window_risk_score have no counterpart in the reference (it scores with the mean
+query only): they restate the textbook definition, causal softmax attention of each of the last W
+queries averaged over queries and GQA group, and are pinned by brute force and special cases only.
   _NormFallback.score_prefill                 :145-147 (+ _normalize_scores "layer" :130-134)
 and /root/reference/kvquant/attention_utils.py
   _repeat_kv :19-26, _get_query_states :29-54, _apply_avg_rope :57-115.
@@ -244,3 +247,29 @@ def expected_attention_score(keys: torch.Tensor, values: torch.Tensor, mu: torch
     if use_vnorm:
         raw = (raw + epsilon) * v_core.unsqueeze(0).norm(dim=-1)
     return pad_sinks(raw, n_sink)
+
+
+def window_attention(keys: torch.Tensor, queries: torch.Tensor, n_sink: int, q_pos0: int,
+                     scaling: Optional[float] = None) -> torch.Tensor:
+    """p [1, Hkv, T - n_sink]: mean over the W window queries and the GQA group of
+    softmax_t(q . k_t * scaling) over core tokens, query w (at position q_pos0 + w) seeing keys at
+    positions <= its own.  keys [Hkv, T, d], queries [Hq, W, d] (already rotated to their positions)."""
+    core = keys[:, n_sink:]
+    h_kv, t_core, d = core.shape
+    h_q, w, _ = queries.shape
+    groups = h_q // h_kv
+    scale = d ** -0.5 if scaling is None else scaling
+    kx = repeat_kv(core.unsqueeze(0), groups)[0]                                  # [Hq, Tc, d]
+    logits = torch.einsum("qwd,qtd->qwt", queries, kx) * scale
+    key_pos = n_sink + torch.arange(t_core)
+    q_pos = q_pos0 + torch.arange(w)
+    logits = logits.masked_fill(key_pos[None, None, :] > q_pos[None, :, None], float("-inf"))
+    a = torch.softmax(logits, dim=-1)
+    return a.reshape(h_kv, groups * w, t_core).mean(dim=1).unsqueeze(0)
+
+
+def window_risk_score(keys: torch.Tensor, values: torch.Tensor, queries: torch.Tensor, q_pos0: int, *,
+                      n_sink: int = 4, epsilon: float = 1e-2, scaling: Optional[float] = None) -> torch.Tensor:
+    """The risk score with the window attention mass in place of the mean query's: [Hkv, T]."""
+    p = window_attention(keys, queries, n_sink, q_pos0, scaling)
+    return pad_sinks(risk_from_attention(p, keys[:, n_sink:], values[:, n_sink:], epsilon), n_sink)

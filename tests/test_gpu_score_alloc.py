@@ -252,3 +252,55 @@ def test_expected_attention_covariance_pieces_keep_fp32_accuracy(dtype, cov_scal
                                         epsilon=1e-2, use_vnorm=True)
     got = _launch_score_expected(k.to(DEV), v.to(DEV), mu[0].to(DEV), cov[0].to(DEV), hq, 4, 1e-2, True)
     np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=2e-5)
+
+
+# ---- observation-window attention on the 16-bit matrix cores --------------------------------------
+@pytest.mark.parametrize("hkv,hq,T,W,dtype", [
+    (2, 8, 700, 64, torch.float16), (8, 32, 2085, 64, torch.float16), (4, 28, 1500, 32, torch.bfloat16),
+    (2, 16, 517, 64, torch.float16), (3, 3, 261, 13, torch.bfloat16), (1, 4, 300, 1, torch.float16),
+    (2, 4, 40, 30, torch.float16), (1, 8, 1000, 128, torch.bfloat16)])
+def test_window_attention_kernel_matches_oracle(hkv, hq, T, W, dtype):
+    from kvquant.scorer import _launch_window_attention
+    g = torch.Generator().manual_seed(T + W)
+    k = torch.randn(hkv, T, 128, generator=g).to(dtype)
+    q = (torch.randn(hq, W, 128, generator=g) * 1.5).to(dtype)
+    want = osc.window_attention(k.double(), q.double(), 4, T - W)[0]
+    got = _launch_window_attention(k.to(DEV), q.to(DEV), 4, T - W, 128 ** -0.5)
+    assert got.shape == (hkv, T - 4) and got.dtype == torch.float32
+    np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=SCORE_RTOL, atol=1e-12)
+    np.testing.assert_allclose(got.sum(-1).cpu().numpy(), 1.0, rtol=1e-4)
+
+
+def test_window_attention_rejects_fp32_keys():
+    from kvquant.scorer import _launch_window_attention
+    k = torch.randn(1, 64, 128, device=DEV)
+    with pytest.raises(ValueError):
+        _launch_window_attention(k, torch.randn(2, 8, 128, device=DEV), 4, 56, 128 ** -0.5)
+
+
+@pytest.mark.parametrize("dtype,rotary", [(torch.float16, True), (torch.bfloat16, False)])
+def test_window_risk_scorer_matches_oracle(dtype, rotary):
+    """The host class end to end: the module's own queries of the last `window` positions (RoPE at their
+    positions), window attention, risk score, sink padding."""
+    from kvquant.scorer import WindowRiskScorer
+    from kvquant.attention_utils import _apply_rotary_pos_emb_q
+    hkv, hq, T, W = 2, 8, 900, 48
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn(hkv, T, 128, generator=g).to(dtype); v = torch.randn(hkv, T, 128, generator=g).to(dtype)
+    h = torch.randn(1, T, 96, generator=g).to(dtype)
+    mod = Stub(96, hq, 128, 17, rotary=rotary, n_kv=hkv).to(dtype)
+    sc = WindowRiskScorer(window=W, n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
+    sc.normalize_grain = "global"
+    with torch.no_grad():
+        got = sc.score_prefill(k.to(DEV), v.to(DEV), 0, module=mod.to(DEV), hidden_states=h.to(DEV))
+        # the oracle takes the same 16-bit queries the kernel was given
+        mod = mod.cpu()
+        q = osc.query_states(mod, h[:, T - W:])
+        if rotary:
+            cos, sin = mod.rotary_emb(q, torch.arange(T - W, T).unsqueeze(0))
+            q = _apply_rotary_pos_emb_q(q, cos.to(q.dtype), sin.to(q.dtype))
+        want = osc.window_risk_score(k.double(), v.double(), q[0].to(dtype).double(), T - W, n_sink=4, epsilon=1e-2)
+    assert got.shape == (hkv, T) and got.dtype == torch.float32
+    # the queries come out of a 16-bit GEMM on either side (CPU and GPU round differently): 16-bit tolerance
+    np.testing.assert_allclose(got.cpu().numpy(), want.numpy(), rtol=3e-2)
+    assert torch.all(got[:, :4] == got[:, 4:].max())

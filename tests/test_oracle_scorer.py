@@ -203,3 +203,45 @@ def test_expected_attention_closed_forms():
     same = sc.expected_attention_score(kn, v, mu, eye, hkv * G, n_sink=4, use_vnorm=False)
     base = sc.expected_attention_score(kn, v, mu, None, hkv * G, n_sink=4, use_vnorm=False)
     np.testing.assert_allclose(same.numpy(), base.numpy(), rtol=1e-12)
+
+
+# ---- observation-window attention (no counterpart in the reference: pinned by definition and special cases) ----
+def test_window_attention_brute_force_and_special_cases():
+    g = torch.Generator().manual_seed(8)
+    hkv, G, T, d, W, n_sink = 2, 2, 20, 8, 5, 3
+    k = torch.randn(hkv, T, d, generator=g, dtype=torch.float64)
+    v = torch.randn(hkv, T, d, generator=g, dtype=torch.float64)
+    q = torch.randn(hkv * G, W, d, generator=g, dtype=torch.float64)
+    q_pos0 = T - W
+    got = sc.window_attention(k, q, n_sink, q_pos0)[0]
+    want = torch.zeros(hkv, T - n_sink, dtype=torch.float64)
+    for h in range(hkv):
+        for gq in range(G):
+            for w in range(W):
+                last = q_pos0 + w                                     # the query sees keys at positions n_sink .. last
+                lg = torch.tensor([float(q[h * G + gq, w] @ k[h, t]) / d ** 0.5 for t in range(n_sink, last + 1)],
+                                  dtype=torch.float64)
+                pr = torch.exp(lg - lg.max()); pr = pr / pr.sum()
+                want[h, : last + 1 - n_sink] += pr / (G * W)
+    np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=1e-12, atol=1e-15)
+    np.testing.assert_allclose(got.sum(-1).numpy(), 1.0, rtol=1e-12)                 # a mean of distributions
+    assert got[:, -1].max() < 1.0 / W                                                # the last key is seen by one query in W
+    # one query at the last position, no key after it: the mean-query attention with that query as the mean
+    one = sc.window_attention(k, q[:, -1:], n_sink, T - 1)
+    ref = sc.expected_attention(k, q[:, -1].unsqueeze(0), n_sink, hkv * G)
+    np.testing.assert_allclose(one.numpy(), ref.numpy(), rtol=1e-12)
+    # a window far behind the keys (no causal cut) with identical queries equals that one query's softmax
+    same = sc.window_attention(k, q[:, :1].expand(-1, 4, -1), n_sink, T + 10)
+    ref = sc.expected_attention(k, q[:, 0].unsqueeze(0), n_sink, hkv * G)
+    np.testing.assert_allclose(same.numpy(), ref.numpy(), rtol=1e-12)
+    # zero queries: uniform over the keys each query sees
+    uni = sc.window_attention(k, torch.zeros_like(q), n_sink, q_pos0)[0]
+    cnt = torch.tensor([sum(1.0 / (q_pos0 + w + 1 - n_sink) for w in range(W) if n_sink + t <= q_pos0 + w) / W
+                        for t in range(T - n_sink)], dtype=torch.float64)
+    np.testing.assert_allclose(uni[0].numpy(), cnt.numpy(), rtol=1e-12)
+    # and the score built on it follows the risk formula with that p
+    s = sc.window_risk_score(k, v, q, q_pos0, n_sink=n_sink, epsilon=1e-2)
+    p = sc.window_attention(k, q, n_sink, q_pos0)
+    np.testing.assert_allclose(s[:, n_sink:].numpy(),
+                               sc.risk_from_attention(p, k[:, n_sink:], v[:, n_sink:], 1e-2)[0].numpy(), rtol=1e-12)
+    assert torch.all(s[:, :n_sink] == s[:, n_sink:].max())
