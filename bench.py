@@ -262,6 +262,9 @@ def main() -> int:
     ap.add_argument("--score-expected", action="store_true",
                     help="time the expected-attention score (mean query + query covariance on the fp32 matrix "
                          "cores) of one --ctx-token layer, rotating over 8 layers' keys and values, and exit")
+    ap.add_argument("--score-window", action="store_true",
+                    help="time the observation-window attention mass (last 64 queries of every head, per-query causal "
+                         "softmax, 16-bit matrix cores) and the risk score built on it for one --ctx-token layer, and exit")
     ap.add_argument("--press-e2e", action="store_true",
                     help="instead of the kernel benchmark: a random-init Llama-3-8B-shaped model (--e2e-layers) under the "
                          "press, prefill of --ctx tokens, then greedy decode with the fused kernel and with the dense "
@@ -323,6 +326,38 @@ def main() -> int:
                                                                    - out["mean_query_only_ms_per_layer"]) * 1e-3) / 1e12, 1)
         out["shape"] = {"Hkv": n_kv, "Hq": n_q, "T": T, "dtype": "fp16"}
         print(json.dumps({"score_expected": out}))
+        return 0
+
+    if args.score_window:
+        from kvquant.scorer import _launch_window_attention
+        g = torch.Generator().manual_seed(6)
+        W = 64
+        layers = []
+        for _ in range(8):
+            k = torch.randn(n_kv, T, 128, generator=g).half().to(dev)
+            v = torch.randn(n_kv, T, 128, generator=g).half().to(dev)
+            q = torch.randn(n_q, W, 128, generator=g).half().to(dev)
+            layers.append((k, v, q))
+        out = {}
+        for name in ("window_attention", "window_risk_score"):
+            def sweep():
+                for k, v, q in layers:
+                    p = _launch_window_attention(k, q, 4, T - W, 128 ** -0.5)
+                    if name == "window_risk_score":
+                        _launch_score(k[:, 4:], v[:, 4:], None, p, n_kv, 0, 1e-2)
+            for _ in range(3):
+                sweep()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(5):
+                sweep()
+            e1.record()
+            torch.cuda.synchronize()
+            out[name + "_ms_per_layer"] = round(e0.elapsed_time(e1) / (5 * len(layers)), 4)
+        out["flop_per_pass"] = 2.0 * n_q * W * (T - 4) * 128
+        out["shape"] = {"Hkv": n_kv, "Hq": n_q, "T": T, "window": W, "dtype": "fp16"}
+        print(json.dumps({"score_window": out}))
         return 0
 
     if args.read_ceiling:

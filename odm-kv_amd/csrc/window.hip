@@ -9,8 +9,8 @@
 // Two passes over K, the logits are never stored:
 //   pass 1  rows of the matrix product = tokens, columns = queries: a lane owns a query and keeps that
 //           query's running (max, sum) over the tokens it sees; per-wave results go to `stats`
-//   stats   merge per query -> (M, 1/Z)
-//   pass 2  rows = queries, columns = tokens: a lane owns a token and sums exp2(s - M) / Z over the queries
+//   stats   merge per query -> M + log2 Z
+//   pass 2  rows = queries, columns = tokens: a lane owns a token and sums exp2(s - M - log2 Z) over the queries
 // The same two operand fragments serve both passes; only their roles (A or B) swap.  The queries of a
 // kv-head (up to 256 at a time) sit in LDS, a wave holds the rows of its 64 tokens in registers and every
 // 16-byte LDS read of a query fragment feeds two matrix instructions.
@@ -31,7 +31,7 @@ struct WinArgs {
     int Hkv, G, W, R, T, Tc, n_sink, nchunks, nstat, qpos0;
     float c;              // scaling * log2(e): logits in base-2 units
     float* stats;         // [Hkv R][nstat][2]
-    float* mz;            // [Hkv R][2]: maximum and reciprocal sum
+    float* mz;            // [Hkv R]: maximum + log2(sum), both in base-2 units
     float* p;             // [Hkv][Tc]
 };
 
@@ -63,13 +63,14 @@ __device__ static inline uint4 pick_half(int half, const uint4& lo, const uint4&
 template <int DT, int PASS>
 __global__ __launch_bounds__(256) void window_kernel(WinArgs a) {
     extern __shared__ __align__(16) uint16_t q_s[];                 // [WIN_ROWS][WIN_QROW]
-    __shared__ float2 mz_s[WIN_ROWS];
+    __shared__ float ml_s[WIN_ROWS];
     const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, col = lane & 31, half = lane >> 5;
     const int t0 = chunk * WIN_CHUNK + wave * 64;                    // first of this wave's 64 core tokens
     const bool active = t0 < a.Tc;                                  // wave-uniform
     // keys at or before every window query need no causal test: only the last tokens do
     const bool need_mask = a.n_sink + t0 + 63 > a.qpos0;
+    const bool tail = t0 + 64 > a.Tc;                               // some of the wave's tokens lie past the end
     uint4 k0[16], k1[16];                                           // the rows of tokens t0 + col and t0 + 32 + col
     if (active) {                                                   // rows past the end repeat the last row and are masked
         const uint4* p0 = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.K) + (size_t)h * a.sH +
@@ -84,17 +85,24 @@ __global__ __launch_bounds__(256) void window_kernel(WinArgs a) {
     for (int rg = 0; rg < a.R; rg += WIN_ROWS) {
         const int nr = min(WIN_ROWS, a.R - rg), nrb = (nr + 31) >> 5;
         __syncthreads();                                            // the previous group's reads are done
-        for (int e = tid; e < nrb * 32 * 16; e += 256) {
-            const int row = e >> 4, pc = e & 15;
-            const uint4 v = row < nr ? qsrc[(size_t)(rg + row) * 16 + pc] : make_uint4(0u, 0u, 0u, 0u);
-            *reinterpret_cast<uint4*>(q_s + (size_t)row * WIN_QROW + pc * 8) = v;
+        {
+            // all of a thread's 16-byte pieces are requested before the first is stored (one round trip to
+            // the caches instead of sixteen)
+            uint4 stage[WIN_ROWS * 16 / 256];
+#pragma unroll
+            for (int i = 0; i < WIN_ROWS * 16 / 256; ++i) {
+                const int e = tid + 256 * i, row = e >> 4, pc = e & 15;
+                stage[i] = row < nr ? qsrc[(size_t)(rg + row) * 16 + pc] : make_uint4(0u, 0u, 0u, 0u);
+            }
+#pragma unroll
+            for (int i = 0; i < WIN_ROWS * 16 / 256; ++i) {
+                const int e = tid + 256 * i, row = e >> 4, pc = e & 15;
+                if (row < nrb * 32) *reinterpret_cast<uint4*>(q_s + (size_t)row * WIN_QROW + pc * 8) = stage[i];
+            }
         }
         if (PASS == 2) {
-            for (int e = tid; e < nrb * 32; e += 256) {
-                // queries beyond the last take weight 0
-                mz_s[e] = e < nr ? make_float2(a.mz[2 * ((size_t)h * a.R + rg + e)], a.mz[2 * ((size_t)h * a.R + rg + e) + 1])
-                                 : make_float2(0.0f, 0.0f);
-            }
+            // queries beyond the last take weight 0: exp2(0 - inf)
+            for (int e = tid; e < nrb * 32; e += 256) ml_s[e] = e < nr ? a.mz[(size_t)h * a.R + rg + e] : INFINITY;
         }
         __syncthreads();
         if (!active) {
@@ -124,20 +132,32 @@ __global__ __launch_bounds__(256) void window_kernel(WinArgs a) {
                 // this lane's query: row rho of the kv-head; its position decides which of the last keys it sees
                 const int rho = rg + rb * 32 + col;
                 const int qpos = a.qpos0 + rho % a.W;
-                float s0[16], s1[16], mx = -INFINITY;
+                float mx = -INFINITY, z = 0.0f;
+                if (!need_mask && !tail) {
+                    // every token of the wave is a key every query sees: the maximum is taken on the raw
+                    // products (the scale is positive) and the scale folds into the exponent
+                    float mr = acc0[0];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int ta = t0 + acc_row(r, half), tb = ta + 32;
-                    const bool va = ta < a.Tc && (!need_mask || a.n_sink + ta <= qpos);
-                    const bool vb = tb < a.Tc && (!need_mask || a.n_sink + tb <= qpos);
-                    s0[r] = va ? acc0[r] * a.c : -INFINITY;
-                    s1[r] = vb ? acc1[r] * a.c : -INFINITY;
-                    mx = fmaxf(mx, fmaxf(s0[r], s1[r]));
-                }
-                float z = 0.0f;
-                if (mx > -INFINITY) {
+                    for (int r = 0; r < 16; ++r) mr = fmaxf(mr, fmaxf(acc0[r], acc1[r]));
+                    mx = mr * a.c;
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) z += __builtin_amdgcn_exp2f(s0[r] - mx) + __builtin_amdgcn_exp2f(s1[r] - mx);
+                    for (int r = 0; r < 16; ++r)
+                        z += __builtin_amdgcn_exp2f(__fmaf_rn(acc0[r], a.c, -mx)) + __builtin_amdgcn_exp2f(__fmaf_rn(acc1[r], a.c, -mx));
+                } else {
+                    float s0[16], s1[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int ta = t0 + acc_row(r, half), tb = ta + 32;
+                        const bool va = ta < a.Tc && a.n_sink + ta <= qpos;
+                        const bool vb = tb < a.Tc && a.n_sink + tb <= qpos;
+                        s0[r] = va ? acc0[r] * a.c : -INFINITY;
+                        s1[r] = vb ? acc1[r] * a.c : -INFINITY;
+                        mx = fmaxf(mx, fmaxf(s0[r], s1[r]));
+                    }
+                    if (mx > -INFINITY) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) z += __builtin_amdgcn_exp2f(s0[r] - mx) + __builtin_amdgcn_exp2f(s1[r] - mx);
+                    }
                 }
                 // the other half of the wave holds the same query's other tokens
                 const float m2 = __shfl_xor(mx, 32, WAVE), z2 = __shfl_xor(z, 32, WAVE);
@@ -151,9 +171,9 @@ __global__ __launch_bounds__(256) void window_kernel(WinArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int row = rb * 32 + acc_row(r, half);
-                    const float2 mz = mz_s[row];
-                    float ea = __builtin_amdgcn_exp2f(__fmaf_rn(acc0[r], a.c, -mz.x)) * mz.y;
-                    float eb = __builtin_amdgcn_exp2f(__fmaf_rn(acc1[r], a.c, -mz.x)) * mz.y;
+                    const float ml = ml_s[row];                     // M + log2 Z: exp2(s - ml) = exp2(s - M) / Z
+                    float ea = __builtin_amdgcn_exp2f(__fmaf_rn(acc0[r], a.c, -ml));
+                    float eb = __builtin_amdgcn_exp2f(__fmaf_rn(acc1[r], a.c, -ml));
                     if (need_mask) {
                         const int qpos = a.qpos0 + (rg + row) % a.W;
                         if (a.n_sink + ta > qpos) ea = 0.0f;
@@ -186,11 +206,8 @@ __global__ __launch_bounds__(64) void window_stats_kernel(WinArgs a) {
         const float m2 = __shfl_xor(m, o, WAVE), s2 = __shfl_xor(s, o, WAVE);
         ms2_merge(m, s, m2, s2);
     }
-    if (lane == 0) {
-        // a query that sees no key at all (cannot happen when the window lies behind the sinks) votes for nothing
-        a.mz[2 * row] = m > -INFINITY ? m : 0.0f;
-        a.mz[2 * row + 1] = s > 0.0f ? 1.0f / s : 0.0f;
-    }
+    // M + log2 Z; a query that sees no key at all (cannot happen when the window lies behind the sinks) votes for nothing
+    if (lane == 0) a.mz[row] = (m > -INFINITY && s > 0.0f) ? m + __builtin_amdgcn_logf(s) : INFINITY;
 }
 
 static inline int win_chunks(int Tc) { return (Tc + WIN_CHUNK - 1) / WIN_CHUNK; }

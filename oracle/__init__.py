@@ -29,6 +29,8 @@ Pin status (what independent evidence fixes each function):
   closed forms (uniform attention, G=1), scaling invariants, and the reference's
   own outputs in ``tests/golden`` (risk score: 5 cases; expected-attention score
   with the query covariance: 6 cases incl. RoPE on mean and covariance).
+  ``scorer.window_attention`` has no counterpart in the reference: **parity
+  unpinned** there, pinned by brute force and special cases only.
 * ``allocator.optimal_scores_to_bits``  pinned: exhaustive Lagrangian argmin on
   tiny inputs, budget invariants, trivial-case clamps; token choice *inside* a
   group of equal scores at the repair cut-off is implementation-defined in the
