@@ -311,12 +311,18 @@ def test_bf16_model_fused_matches_dense_path():
     assert (log_f.argmax(-1) == tok_d).float().mean().item() >= 0.95
 
 
-def test_press_with_expected_attention_scorer():
+@pytest.mark.parametrize("kind", ["expected_attention", "window_risk"])
+def test_press_with_other_scorers(kind):
     """The press with the reference's other scorer class (mean query + query covariance, the default
-    layer-wise min-max normalisation): the budget holds, sinks and the window stay exact, the fused decode
-    agrees with the dense path, and a 130-step decode crosses a buffer flush."""
-    from kvquant import ExpectedAttentionScorer
+    layer-wise min-max normalisation) and with the observation-window risk scorer: the budget holds, sinks
+    and the window stay exact, the fused decode agrees with the dense path, and a 130-step decode crosses
+    a buffer flush."""
+    from kvquant import ExpectedAttentionScorer, WindowRiskScorer
     def scorer():
+        if kind == "window_risk":
+            sc = WindowRiskScorer(window=64, n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)
+            sc.normalize_grain = "global"
+            return sc
         return ExpectedAttentionScorer(n_future_positions=512, n_sink=4, use_covariance=True, use_vnorm=True, epsilon=1e-2)
     model = _model(5)
     ids = _ids(600, 21)
