@@ -12,8 +12,8 @@
 //   stats   merge per query -> M + log2 Z
 //   pass 2  rows = queries, columns = tokens: a lane owns a token and sums exp2(s - M - log2 Z) over the queries
 // The same two operand fragments serve both passes; only their roles (A or B) swap.  The queries of a
-// kv-head (up to 256 at a time) sit in LDS, a wave holds the rows of its 64 tokens in registers and every
-// 16-byte LDS read of a query fragment feeds two matrix instructions.
+// kv-head (up to 256 at a time) sit in LDS, a wave holds its 64 tokens in registers (each lane the half row it
+// contracts) and every 16-byte LDS read of a query fragment feeds two matrix instructions.
 #include "common.h"
 
 #define WIN_CHUNK 256        // tokens per workgroup (4 waves x 64)
@@ -54,12 +54,6 @@ __device__ static inline void ms2_merge(float& m, float& s, float m2, float s2) 
 // index (0..31) inside a 32-row block of accumulator register r of a lane in wave half `half`
 __device__ static inline int acc_row(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }
 
-// lo for the lower half of the wave, hi for the upper one: selected register by register (an index into the
-// row array that depends on the lane would move the array to scratch memory)
-__device__ static inline uint4 pick_half(int half, const uint4& lo, const uint4& hi) {
-    return make_uint4(half ? hi.x : lo.x, half ? hi.y : lo.y, half ? hi.z : lo.z, half ? hi.w : lo.w);
-}
-
 template <int DT, int PASS>
 __global__ __launch_bounds__(256) void window_kernel(WinArgs a) {
     extern __shared__ __align__(16) uint16_t q_s[];                 // [WIN_ROWS][WIN_QROW]
@@ -71,14 +65,18 @@ __global__ __launch_bounds__(256) void window_kernel(WinArgs a) {
     // keys at or before every window query need no causal test: only the last tokens do
     const bool need_mask = a.n_sink + t0 + 63 > a.qpos0;
     const bool tail = t0 + 64 > a.Tc;                               // some of the wave's tokens lie past the end
-    uint4 k0[16], k1[16];                                           // the rows of tokens t0 + col and t0 + 32 + col
+    // Operand fragments: the matrix instruction contracts over 16 elements per step, 8 from either half of
+    // the wave; which 8 is free as long as both operands agree.  Here half h of the wave takes elements
+    // 64 h + 8 st .. + 7 in step st, so a lane reads one contiguous 128-byte half row of its token (a whole
+    // cache line, used by that lane alone) and nothing it does not use.
+    uint4 k0[8], k1[8];                                             // half rows of tokens t0 + col and t0 + 32 + col
     if (active) {                                                   // rows past the end repeat the last row and are masked
         const uint4* p0 = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.K) + (size_t)h * a.sH +
-                                                          (size_t)(a.n_sink + min(t0 + col, a.Tc - 1)) * a.sT);
+                                                          (size_t)(a.n_sink + min(t0 + col, a.Tc - 1)) * a.sT + 64 * half);
         const uint4* p1 = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.K) + (size_t)h * a.sH +
-                                                          (size_t)(a.n_sink + min(t0 + 32 + col, a.Tc - 1)) * a.sT);
+                                                          (size_t)(a.n_sink + min(t0 + 32 + col, a.Tc - 1)) * a.sT + 64 * half);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { k0[i] = p0[i]; k1[i] = p1[i]; }
+        for (int i = 0; i < 8; ++i) { k0[i] = p0[i]; k1[i] = p1[i]; }
     }
     float pacc0 = 0.0f, pacc1 = 0.0f;
     const uint4* qsrc = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.Q) + (size_t)h * a.R * HD);
@@ -119,12 +117,11 @@ __global__ __launch_bounds__(256) void window_kernel(WinArgs a) {
             f32x16 acc0, acc1;
 #pragma unroll
             for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
-            const uint16_t* qrow = q_s + (size_t)(rb * 32 + col) * WIN_QROW + 8 * half;
+            const uint16_t* qrow = q_s + (size_t)(rb * 32 + col) * WIN_QROW + 64 * half;
 #pragma unroll
             for (int st = 0; st < 8; ++st) {
-                const uint4 qv = *reinterpret_cast<const uint4*>(qrow + 16 * st);
-                const uint4 ka = pick_half(half, k0[2 * st], k0[2 * st + 1]);
-                const uint4 kb = pick_half(half, k1[2 * st], k1[2 * st + 1]);
+                const uint4 qv = *reinterpret_cast<const uint4*>(qrow + 8 * st);
+                const uint4 ka = k0[st], kb = k1[st];
                 if (PASS == 1) { acc0 = win_mfma<DT>(ka, qv, acc0); acc1 = win_mfma<DT>(kb, qv, acc1); }
                 else { acc0 = win_mfma<DT>(qv, ka, acc0); acc1 = win_mfma<DT>(qv, kb, acc1); }
             }
