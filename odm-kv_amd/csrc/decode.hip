@@ -397,44 +397,43 @@ __device__ static inline void compute_tile(const TileData<W>& t, int nvalid, int
 // wavefront reads in one instruction (lane % 4) sit on different banks
 #define QS 33
 // stage the group's queries (fp16 high/low halves per 4-dim step) in LDS; heads beyond the group are 0
-template <int NP>
-__device__ static inline uint4 load_query_slice(const DecodeArgs& a, const uint4* src, int tid, int nheads) {
-    return (tid < 4 * NP * 32 && (tid >> 5) < nheads) ? src[tid] : make_uint4(0u, 0u, 0u, 0u);
+// nq: query heads staged by the workgroup (4, or 8 when its two wave groups serve four heads each)
+__device__ static inline uint4 load_query_slice(const uint4* src, int tid, int nq, int nheads) {
+    return (tid < nq * 32 && (tid >> 5) < nheads) ? src[tid] : make_uint4(0u, 0u, 0u, 0u);
 }
-template <int NP>
-__device__ static inline void stage_queries(uint4 v, uint4* qsh, int tid) {
-    if (tid < 4 * NP * 32) qsh[(tid >> 5) * QS + (tid & 31)] = v;
+__device__ static inline void stage_queries(uint4 v, uint4* qsh, int tid, int nq) {
+    if (tid < nq * 32) qsh[(tid >> 5) * QS + (tid & 31)] = v;
 }
-template <int NP>
-__device__ static inline void fetch_queries(const uint4* qsh, int lane, h4* qr, h4* ql) {
+// hbase: first of the four heads this wavefront serves
+__device__ static inline void fetch_queries(const uint4* qsh, int lane, int hbase, h4* qr, h4* ql) {
 #pragma unroll
-    for (int p = 0; p < NP; ++p)
-#pragma unroll
-        for (int s = 0; s < 32; ++s) {
-            const uint4 v = qsh[(4 * p + (lane & 3)) * QS + s];
-            qr[p * 32 + s] = as_h4(v.x, v.y);
-            ql[p * 32 + s] = as_h4(v.z, v.w);
-        }
+    for (int s = 0; s < 32; ++s) {
+        const uint4 v = qsh[(hbase + (lane & 3)) * QS + s];
+        qr[s] = as_h4(v.x, v.y);
+        ql[s] = as_h4(v.z, v.w);
+    }
 }
 
-// One work item of a quantised level.
-template <int W, int NP>
-__device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq0, int nheads, int tile0, int ntiles, int ntok,
+// One work item of a quantised level.  TW wavefronts walk the item's tiles for the same four heads (all
+// eight, or four per head group when the workgroup serves eight heads); wq is this wavefront's place among them.
+template <int W, int NP, int TW>
+__device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq_first, int nq, int nheads_all, int hbase,
+                                              int tile0, int ntiles, int ntok,
                                               int tid, uint8_t* lut, uint4* qsh, WaveState<NP>& st) {
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = tid >> 6, lane = tid & 63, wq = wave % TW;
     const uint32_t slot4 = (lane & 31) * 4;
     const float vsc = a.inv_s[li], ksc = a.inv_s[li] * a.scaling * LOG2E;
     // The table needs nothing from memory and is built before the tiles are requested: behind a
     // wavefront's tile requests its LDS traffic would wait for the memory pipeline to accept them
     // (every wavefront of the chip asks for its tiles at the same moment).  Loads return in issue
     // order: the (small) query slice goes first so that staging it does not have to wait for the tile.
-    const uint4 qslice = load_query_slice<NP>(a, a.qrot + (size_t)bq0 * 32, tid, nheads);   // one request: lands while the table is built
+    const uint4 qslice = load_query_slice(a.qrot + (size_t)bq_first * 32, tid, nq, nheads_all);   // one request: lands while the table is built
     build_lut<W>(lut, a, tid);
     TileData<W> cur;
-    int tt = wave;
+    int tt = wq;
     int nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
     if (nvalid > 0) load_tile<W>(cur, a, li, tile0 + tt, lane);
-    stage_queries<NP>(qslice, qsh, tid);
+    stage_queries(qslice, qsh, tid, nq);
     lds_barrier();
     TRACE(1)
     // second buffer (not for the widest rows: the registers go to the query there), requested before
@@ -442,17 +441,17 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     TileData<W> nxt;
     int nv1 = 0;
     if constexpr (W != 8) {
-        nv1 = tt + NWAVES < ntiles ? min(ntok - (tt + NWAVES) * TILE, TILE) : 0;
-        if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + NWAVES, lane);
+        nv1 = tt + TW < ntiles ? min(ntok - (tt + TW) * TILE, TILE) : 0;
+        if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + TW, lane);
     }
     h4 qr[NP * 32], ql[NP * 32];
-    fetch_queries<NP>(qsh, lane, qr, ql);
+    fetch_queries(qsh, lane, hbase, qr, ql);
     if (nvalid <= 0) return;
     TRACE(2)
     if constexpr (W == 8) {
         while (true) {
             compute_tile<W, NP>(cur, nvalid, lane, lut, slot4, qr, ql, ksc, vsc, st);
-            tt += NWAVES;
+            tt += TW;
             nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
             if (nvalid <= 0) break;
             load_tile<W>(cur, a, li, tile0 + tt, lane);
@@ -461,13 +460,13 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
         while (true) {
             compute_tile<W, NP>(cur, nvalid, lane, lut, slot4, qr, ql, ksc, vsc, st);
             if (nv1 <= 0) break;
-            tt += 2 * NWAVES;
+            tt += 2 * TW;
             nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
             if (nvalid > 0) load_tile<W>(cur, a, li, tile0 + tt, lane);
             compute_tile<W, NP>(nxt, nv1, lane, lut, slot4, qr, ql, ksc, vsc, st);
             if (nvalid <= 0) break;
-            nv1 = tt + NWAVES < ntiles ? min(ntok - (tt + NWAVES) * TILE, TILE) : 0;
-            if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + NWAVES, lane);
+            nv1 = tt + TW < ntiles ? min(ntok - (tt + TW) * TILE, TILE) : 0;
+            if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + TW, lane);
         }
     }
 }
@@ -546,55 +545,58 @@ __device__ static inline void compute_exact_tile(const ExactTile& t, bool bf, in
 
 // Exact (16-bit) tokens: the query is the fp16-rounded one itself (its low halves are zero), so only
 // the high halves are fetched.  The first tile's loads are issued before anything is waited for.
-template <int NP>
-__device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int bq0, int nheads, int tile0, int ntiles, int seg_first,
+template <int NP, int TW>
+__device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int bq_first, int nq, int nheads_all, int hbase,
+                                              int tile0, int ntiles, int seg_first,
                                               int tid, uint4* qsh, WaveState<NP>& st) {
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = tid >> 6, lane = tid & 63, wq = wave % TW;
     const bool bf = a.s.exact_dtype == ODMKV_BF16;
     const float esc = a.scaling * LOG2E;
-    const uint4 qslice = load_query_slice<NP>(a, a.qs + (size_t)bq0 * 32, tid, nheads);
+    const uint4 qslice = load_query_slice(a.qs + (size_t)bq_first * 32, tid, nq, nheads_all);
     const int count = a.s.seg_count[4][bh];          // exact segments grow between work-list rebuilds
     ExactTile cur;
-    int tt = wave;
+    int tt = wq;
     int nvalid = tt < ntiles ? min(count - (tile0 + tt - seg_first) * TILE, TILE) : 0;
     if (nvalid > 0) load_exact_tile(cur, a, tile0 + tt, lane);
-    stage_queries<NP>(qslice, qsh, tid);
+    stage_queries(qslice, qsh, tid, nq);
     lds_barrier();
     h4 qr[NP * 32];
 #pragma unroll
     for (int p = 0; p < NP; ++p)
 #pragma unroll
         for (int s = 0; s < 32; ++s) {
-            const uint2 v = *reinterpret_cast<const uint2*>(&qsh[(4 * p + (lane & 3)) * QS + s]);
+            const uint2 v = *reinterpret_cast<const uint2*>(&qsh[(hbase + 4 * p + (lane & 3)) * QS + s]);
             qr[p * 32 + s] = as_h4(v.x, v.y);
         }
     while (nvalid > 0) {
         compute_exact_tile<NP>(cur, bf, nvalid, lane, esc, qr, st);
-        tt += NWAVES;
+        tt += TW;
         nvalid = tt < ntiles ? min(count - (tile0 + tt - seg_first) * TILE, TILE) : 0;
         if (nvalid > 0) load_exact_tile(cur, a, tile0 + tt, lane);
     }
 }
 
 // ------------------------------------------------------------------------------------------------
-// main kernel: four query heads per workgroup (NP = 1); larger GQA groups take one workgroup pass per four heads
+// main kernel: four query heads per workgroup; a larger GQA group (SPLIT) is served by the two halves of
+// the workgroup, wavefronts 0-3 the first four heads and wavefronts 4-7 the rest, over the same tiles
+// (the second read of a tile hits the compute unit's own cache): one set-up and one launch wave per item
 // ------------------------------------------------------------------------------------------------
-template <int NP, bool MULTI, bool ORDERED>
+template <int NP, bool SPLIT, bool ORDERED>
 __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs a) {
+    constexpr int NQ = SPLIT ? 8 : 4;                     // query heads of the workgroup
+    constexpr int TW = SPLIT ? NWAVES / 2 : NWAVES;       // wavefronts that share the item's tiles for the same heads
     __shared__ __align__(16) uint8_t lut[LUT_BYTES];     // centroid table; reused to combine the wavefronts
-    __shared__ float wm[NWAVES][4 * NP], wl[NWAVES][4 * NP];
-    __shared__ uint4 qsh[4 * NP * QS];
+    __shared__ float wm[NWAVES][4], wl[NWAVES][4];
+    __shared__ uint4 qsh[NQ * QS];
 
-    // A GQA group of more than four query heads is served four heads at a time by separate workgroups
-    // of the same item (the item's codes are read once per pass; the second read mostly hits the caches).
-    const int item = ORDERED ? a.order[blockIdx.x] : (int)blockIdx.x, pass = MULTI ? (int)blockIdx.y : 0;
+    const int item = ORDERED ? a.order[blockIdx.x] : (int)blockIdx.x;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int hbase = SPLIT ? 4 * (wave / TW) : 0;       // first head (within the group) this wavefront serves
     TRACE(0)
     const int4 d0 = reinterpret_cast<const int4*>(a.items)[2 * item];       // bh, level, first tile, tiles
     const int4 d1 = reinterpret_cast<const int4*>(a.items)[2 * item + 1];   // tokens, first tile of the segment
     const int bh = d0.x, li = d0.y, tile0 = d0.z, ntiles = d0.w;
-    const int bq0 = (bh / a.s.Hkv) * a.Hq + (bh % a.s.Hkv) * a.G + 4 * NP * pass;   // first query head of this pass
-    const int nheads = MULTI ? min(a.G - 4 * NP * pass, 4 * NP) : a.G;
+    const int bq_first = (bh / a.s.Hkv) * a.Hq + (bh % a.s.Hkv) * a.G;      // first query head of the group
 
     WaveState<NP> st;
 #pragma unroll
@@ -603,43 +605,41 @@ __global__ __launch_bounds__(NWAVES * 64, 2) void decode_main_kernel(DecodeArgs 
         st.acc[p][0] = (f4){0.f, 0.f, 0.f, 0.f}; st.acc[p][1] = (f4){0.f, 0.f, 0.f, 0.f};
     }
     switch (li) {
-        case 0: run_quant_level<2, NP>(a, 0, bq0, nheads, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
-        case 1: run_quant_level<3, NP>(a, 1, bq0, nheads, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
-        case 2: run_quant_level<4, NP>(a, 2, bq0, nheads, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
-        case 3: run_quant_level<8, NP>(a, 3, bq0, nheads, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
-        default: run_exact_level<NP>(a, bh, bq0, nheads, tile0, ntiles, d1.y, tid, qsh, st); break;
+        case 0: run_quant_level<2, NP, TW>(a, 0, bq_first, NQ, a.G, hbase, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        case 1: run_quant_level<3, NP, TW>(a, 1, bq_first, NQ, a.G, hbase, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        case 2: run_quant_level<4, NP, TW>(a, 2, bq_first, NQ, a.G, hbase, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        case 3: run_quant_level<8, NP, TW>(a, 3, bq_first, NQ, a.G, hbase, tile0, ntiles, d1.x, tid, lut, qsh, st); break;
+        default: run_exact_level<NP, TW>(a, bh, bq_first, NQ, a.G, hbase, tile0, ntiles, d1.y, tid, qsh, st); break;
     }
 
-    // ---- combine the four wavefronts (the table is no longer needed) ----
+    // ---- combine the wavefronts that served the same heads (the table is no longer needed) ----
     TRACE(3)
     __syncthreads();
     TRACE(4)
-    float* wacc = reinterpret_cast<float*>(lut);          // [NWAVES][4*NP][128]
-    constexpr int GP = 4 * NP;
-#pragma unroll
-    for (int p = 0; p < NP; ++p) {
-        const float ls = head_sum(st.l[p]);
-        if (lane < 4) { wm[wave][4 * p + lane] = st.m[p]; wl[wave][4 * p + lane] = ls; }
+    float* wacc = reinterpret_cast<float*>(lut);          // [NWAVES][4][128]
+    {
+        const float ls = head_sum(st.l[0]);
+        if (lane < 4) { wm[wave][lane] = st.m[0]; wl[wave][lane] = ls; }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            wacc[((wave * GP) + 4 * p + i) * HD + lane] = st.acc[p][0][i];
-            wacc[((wave * GP) + 4 * p + i) * HD + lane + 64] = st.acc[p][1][i];
+            wacc[(wave * 4 + i) * HD + lane] = st.acc[0][0][i];
+            wacc[(wave * 4 + i) * HD + lane + 64] = st.acc[0][1][i];
         }
     }
     __syncthreads();
-    float* dst = a.partial + (MULTI ? ((size_t)item * a.gp + GP * pass) : (size_t)item * GP) * PSTRIDE;
-    for (int e = tid; e < GP * HD; e += NWAVES * 64) {
-        const int g = e / HD, j = e % HD;
-        float M = wm[0][g];
+    float* dst = a.partial + (size_t)item * NQ * PSTRIDE;
+    for (int e = tid; e < NQ * HD; e += NWAVES * 64) {
+        const int g = e / HD, j = e % HD, gl = g & 3, w0 = SPLIT ? (g >> 2) * TW : 0;
+        float M = wm[w0][gl];
 #pragma unroll
-        for (int w = 1; w < NWAVES; ++w) M = fmaxf(M, wm[w][g]);
+        for (int w = 1; w < TW; ++w) M = fmaxf(M, wm[w0 + w][gl]);
         float s = 0.0f, L = 0.0f;
         if (M > -INFINITY) {
 #pragma unroll
-            for (int w = 0; w < NWAVES; ++w) {
-                const float f = __builtin_amdgcn_exp2f(wm[w][g] - M);
-                s = __fmaf_rn(wacc[((w * GP) + g) * HD + j], f, s);
-                L = __fmaf_rn(wl[w][g], f, L);
+            for (int w = 0; w < TW; ++w) {
+                const float f = __builtin_amdgcn_exp2f(wm[w0 + w][gl] - M);
+                s = __fmaf_rn(wacc[((w0 + w) * 4 + gl) * HD + j], f, s);
+                L = __fmaf_rn(wl[w0 + w][gl], f, L);
             }
         }
         dst[g * PSTRIDE + j] = s;
@@ -899,8 +899,8 @@ extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, floa
         // (the plain case keeps its own instantiation: a branch on either option at the kernel's start costs it 0.25 us)
         if (GP == 4 && !a.order) hipExtLaunchKernelGGL((decode_main_kernel<1, false, false>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
         else if (GP == 4) hipExtLaunchKernelGGL((decode_main_kernel<1, false, true>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
-        else if (!a.order) hipExtLaunchKernelGGL((decode_main_kernel<1, true, false>), dim3(n_items, GP / 4), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
-        else hipExtLaunchKernelGGL((decode_main_kernel<1, true, true>), dim3(n_items, GP / 4), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
+        else if (!a.order) hipExtLaunchKernelGGL((decode_main_kernel<1, true, false>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
+        else hipExtLaunchKernelGGL((decode_main_kernel<1, true, true>), dim3(n_items), dim3(NWAVES * 64), 0, st, e0, e1, 0, a);
         ODMKV_CHECK_LAUNCH("decode_main_kernel");
         if (rec) ++g_prof_used;
     }
