@@ -252,6 +252,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--ctx", type=int, default=32768)
     ap.add_argument("--target", type=float, default=2.0)
+    ap.add_argument("--kv-heads", type=int, default=8, help="KV heads (default 8: Llama-3-8B; --kv-heads 4 --q-heads 28 --layers 28 "
+                                                            "--target 3.0 is configuration c5, Qwen2.5-7B)")
+    ap.add_argument("--q-heads", type=int, default=32)
     ap.add_argument("--cpu-sample-ctx", type=int, default=8192)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--read-ceiling", action="store_true",
@@ -288,7 +291,7 @@ def main() -> int:
         return 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    n_kv, n_q, T, NL = 8, 32, args.ctx, args.layers
+    n_kv, n_q, T, NL = args.kv_heads, args.q_heads, args.ctx, args.layers
 
     if args.press_e2e:
         print(json.dumps({"press_e2e": press_e2e(dev, T, args.target, args.e2e_tokens, args.e2e_layers,
@@ -564,7 +567,7 @@ def main() -> int:
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 products, f32 accumulate (2/3/4/8-bit codes)", "data": "synthetic",
-        "config": {"workload": f"c2 kernel-only: {NL} layers x [Hkv 8, T {T}, d 128] fp16, Hq 32, {args.target} avg bits, "
+        "config": {"workload": f"{'c2' if (n_kv, n_q, NL) == (8, 32, 32) else 'custom'} kernel-only: {NL} layers x [Hkv {n_kv}, T {T}, d 128] fp16, Hq {n_q}, {args.target} avg bits, "
                                "1 decode token per step over all layers' packed caches",
                    "levels": list(LEVELS), "n_sink": 4, "window": 128, "launch": launch_mode},
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
