@@ -237,3 +237,23 @@ def test_decode_error_is_mostly_the_dense_cache_rounding():
     e16, e32, oracle_gap = rel_err(got, want16), rel_err(got, want32), rel_err(want16, want32)
     assert e16 < ATTN_RTOL
     assert e32 < 5e-4 and e32 < e16 and e32 < oracle_gap, (e16, e32, oracle_gap)
+
+
+@pytest.mark.parametrize("G", [5, 8])
+def test_large_group_with_more_items_than_compute_units(G):
+    """A GQA group of more than four heads is served by the two halves of each workgroup; with more work items
+    than compute units the kernel also follows the host's dispatch order.  Both cuts must give the oracle's result."""
+    g = torch.Generator().manual_seed(40 + G)
+    B, Hkv, T = 2, 2, 6000
+    k = torch.randn(B, Hkv, T, 128, generator=g).half(); v = torch.randn(B, Hkv, T, 128, generator=g).half()
+    bits = _rand_bits(g, (B, Hkv, T), (0.1, 0.5, 0.2, 0.1, 0.05, 0.05))
+    bits[..., :4] = 16; bits[..., -32:] = 16
+    st, ref = _pair(k, v, bits)
+    q = torch.randn(B, Hkv * G, 128, generator=g).half().float()
+    want = decode_attention_state(q, ref)
+    st._build_items(1 << 20, 1)                       # one- and two-tile items: several per compute unit
+    assert st._items[2] > torch.cuda.get_device_properties(0).multi_processor_count and st._item_order is not None
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
+    st._build_items(16, 1 << 30)                      # a few long items: every wave walks several tiles
+    assert st._item_order is None
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
