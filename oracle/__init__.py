@@ -35,7 +35,17 @@ Pin status (what independent evidence fixes each function):
   tiny inputs, budget invariants, trivial-case clamps; token choice *inside* a
   group of equal scores at the repair cut-off is implementation-defined in the
   reference (unstable argsort) and therefore **parity unpinned** there.
-* ``kvstate.*``                       pinned: partition/round-trip invariants.
-* ``attention.decode_attention``      pinned: equals torch SDPA on an all-exact
-  cache, single-token and permutation special cases.
+* ``kvstate.*``                       pinned by tests/test_oracle_kvstate_attention.py:
+  every position lands in exactly one level, ``materialize`` equals the
+  golden-pinned ``quantizer.dequantize`` at quantised positions, the input at
+  16-bit ones and zero at evicted ones, ``materialize_quantized_into`` leaves the
+  other two alone, ``truncate`` drops exactly the positions behind the cut,
+  ``append_all_exact`` + ``flush_buffer`` re-route exactly the buffered tokens.
+* ``attention.decode_attention``      pinned by the same file: equals torch's
+  ``scaled_dot_product_attention`` in fp64 (G = 1, 4, 7, with mask and scale),
+  returns the value of a single visible token, is invariant under a permutation
+  of the tokens, under dropping the evicted ones and under a split of the token
+  axis merged by log-sum-exp.
+* ``flush.*``                         the decode-time flush scoring; see that
+  module's header for its pins.
 """

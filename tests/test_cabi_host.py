@@ -95,3 +95,15 @@ def test_host_ratio_and_container_match_reference(golden):
     for b in (1, 2, 3, 4, 8):
         codes = torch.from_numpy(golden[f"pack_b{b}_codes"])
         assert (_pack_indices(codes, b).numpy() == golden[f"pack_b{b}_bytes"]).all()
+
+
+def test_product_rotation_is_the_reference_matrix(golden):
+    """The product's own random_rotation (not the oracle's copy) against the matrix the reference
+    drew for seed 42 on the CPU generator (kvquant/tq_backend.py:25-36)."""
+    import torch
+    from kvquant.tq_backend import cached_rotation, random_rotation
+    pi = random_rotation(128, "cpu", torch.float32, seed=42)
+    assert pi.dtype == torch.float32 and (pi.numpy() == golden["pi_seed42"]).all()
+    assert (cached_rotation(128, "cpu", 42).numpy() == golden["pi_seed42"]).all()
+    # another seed is another matrix; the value rotation of a state is seed + 2000
+    assert not (random_rotation(128, "cpu", torch.float32, seed=2042).numpy() == golden["pi_seed42"]).all()

@@ -338,3 +338,73 @@ def test_press_with_other_scorers(kind):
         # the budget is met over all non-sink tokens before the window is forced to 16 bits, so the mean over
         # the tokens in front of the window sits near the target, not exactly under it
         assert abs(core.mean().item() - 2.5) < 0.1
+
+
+@torch.inference_mode()
+def test_flush_levels_match_the_oracle():
+    """Decode-time flush (reference: kvquant/adaptive_backend_press.py:464-665, 198-241) against
+    oracle.flush on the same buffered tokens: attention weights of the current query, normalised risk
+    scores, and the levels from the level shares recorded at prefill."""
+    from transformers import DynamicCache
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+    from oracle import flush as ofl
+    model = _model(9)
+    T, n_buf = 500, 128
+    ids = _ids(T, 61)
+    forced = torch.randint(0, 1000, (n_buf + 3,), generator=torch.Generator().manual_seed(62)).to(DEV)
+    press = _press(target=2.5)
+    rec = {}
+    orig_flush, orig_attn, orig_alloc = press._flush_decode_buffer, press._flush_attention, press._allocate_bits_via_cached_ratios
+
+    def spy_flush(state, layer_idx, cache, module, hidden_states=None):
+        r = rec.setdefault(layer_idx, {})
+        pos, k, v = state.get_buffer_tokens(press._buffer_start_seqs[layer_idx])
+        r.update(pos=pos.cpu().numpy(), k=k.float().cpu(), v=v.float().cpu(), hidden=hidden_states.clone(),
+                 seq_len=state.seq_len, module=module, observed={h: press._observed_ratios[(layer_idx, h)] for h in range(state.num_heads)})
+        press._cur = r
+        orig_flush(state, layer_idx, cache, module, hidden_states)
+        r["levels"] = state._level_map[0].cpu().numpy().copy()
+
+    def spy_attn(*a, **kw):
+        out = orig_attn(*a, **kw)
+        press._cur["attn"] = out.float().cpu()
+        return out
+
+    def spy_alloc(scores, positions, *a, **kw):
+        out = orig_alloc(scores, positions, *a, **kw)
+        press._cur["scores"] = scores.float().cpu()
+        press._cur["bits"] = out.cpu()
+        return out
+
+    press._flush_decode_buffer, press._flush_attention, press._allocate_bits_via_cached_ratios = spy_flush, spy_attn, spy_alloc
+    cache = DynamicCache()
+    with press(model):
+        model.model(input_ids=ids, past_key_values=cache)
+        for step in range(forced.shape[0]):
+            model(input_ids=forced[step].view(1, 1), past_key_values=cache, position_ids=torch.tensor([[T + step]], device=DEV))
+    assert sorted(rec) == [0, 1]
+    for layer_idx, r in rec.items():
+        assert r["pos"].shape[0] == 2 * n_buf and r["seq_len"] == T + n_buf
+        # the query of the newest position through the model's own projection and rotary code
+        m = r["module"]
+        q = m.q_proj(r["hidden"]).view(1, 1, 4, 128).transpose(1, 2)
+        cos, sin = model.model.rotary_emb(q, torch.tensor([[r["seq_len"] - 1]], device=DEV))
+        q, _ = apply_rotary_pos_emb(q, q, cos, sin)
+        q_last = q[:, :, -1, :].float().cpu()
+        attn, scores, bits = ofl.flush_levels(q_last, r["k"], r["v"], r["pos"], 2, r["observed"], (2, 3, 4, 8, 16))
+        # (1) attention weights: the press works in the model's fp16
+        np.testing.assert_allclose(r["attn"].numpy(), attn.numpy(), rtol=2e-2, atol=1e-6)
+        # (2) scores on the press's own weights: kernel against the oracle's formula
+        want_scores = ofl.flush_scores(r["k"], r["v"], r["attn"], r["pos"], 2)
+        np.testing.assert_allclose(r["scores"].numpy(), want_scores.numpy(), rtol=1e-3, atol=1e-6)
+        # (3) levels on the press's own scores: bit for bit
+        want_bits = ofl.cached_ratio_bits(r["scores"], r["pos"], 2, r["observed"], (2, 3, 4, 8, 16))
+        assert torch.equal(r["bits"], want_bits)
+        # (4) the whole chain from the oracle's own weights: the same tier sizes, and a different level only
+        # for tokens whose score sits at a tier boundary (fp16 rounding of the weights moves the ranks there)
+        assert sorted(bits.tolist()) == sorted(r["bits"].tolist())
+        assert (bits != r["bits"]).float().mean().item() < 0.05
+        # (5) the store took them: buffered positions now hold those levels, later tokens stay exact
+        lm = r["levels"]
+        assert (lm[r["pos"][:, 1], r["pos"][:, 2]] == r["bits"].numpy()).all()
+        assert not (r["bits"] == 0).any()                 # no decode-time eviction
