@@ -249,6 +249,25 @@ int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
                       void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                       void* stream);
 
+/* The same call without a workspace, for callers that cannot allocate device memory and have none
+ * to hand over (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.  The prepared queries and the per-item partial results live in
+ * a fixed array of ODMKV_STATIC_SCRATCH_BYTES inside the library's device image (held by every GPU
+ * the library runs on until the process ends); a call whose odmkv_decode_workspace_bytes(B, Hq,
+ * n_items) exceeds it fails with ODMKV_ENOSPACE and launches nothing.  The call allocates and
+ * frees nothing.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream do not.  The first call on a device looks the
+ * array's address up (no stream work); make it outside graph capture.  Everything else is
+ * odmkv_decode_attn. */
+#define ODMKV_STATIC_SCRATCH_BYTES (8u << 20)
+int odmkv_decode_attn_static(const void* q, int q_dtype, int B, int Hq, float scaling,
+                             const odmkv_packed_t* store,
+                             const int32_t* items, int n_items, const int32_t* item_range,
+                             const int32_t* dispatch_order,
+                             const float* pi_k_t, const float* pi_v, const float* codebooks,
+                             const float* codebooks_host, const float* inv_scales,
+                             void* out, int out_dtype, float* lse, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Measurement hooks (no counterpart in the reference).  While enabled, every odmkv_decode_attn
  * call records a pair of HIP events around its main (streaming) kernel on the caller's stream;

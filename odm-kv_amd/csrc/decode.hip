@@ -850,14 +850,14 @@ extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     return 2 * q + align_up((size_t)n_items * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
 }
 
-extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
-                                 const odmkv_packed_t* store,
-                                 const int32_t* items, int n_items, const int32_t* item_range,
-                                 const int32_t* dispatch_order,
-                                 const float* pi_k_t, const float* pi_v, const float* codebooks,
-                                 const float* codebooks_host, const float* inv_scales,
-                                 void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
-                                 void* stream) {
+static int decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling,
+                         const odmkv_packed_t* store,
+                         const int32_t* items, int n_items, const int32_t* item_range,
+                         const int32_t* dispatch_order,
+                         const float* pi_k_t, const float* pi_v, const float* codebooks,
+                         const float* codebooks_host, const float* inv_scales,
+                         void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
+                         void* stream) {
     ODMKV_CHECK_ARG(q_dtype == ODMKV_F16 || q_dtype == ODMKV_BF16 || q_dtype == ODMKV_F32, "decode_attn: bad query dtype %d", q_dtype);
     ODMKV_CHECK_ARG(out_dtype == ODMKV_F16 || out_dtype == ODMKV_BF16 || out_dtype == ODMKV_F32, "decode_attn: bad output dtype %d", out_dtype);
     ODMKV_CHECK_ARG(codebooks_host != nullptr, "decode_attn: null host copy of the centroid tables");
@@ -910,4 +910,62 @@ extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, floa
         ODMKV_CHECK_LAUNCH("decode_merge_kernel");
     }
     return 0;
+}
+
+extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
+                                 const odmkv_packed_t* store,
+                                 const int32_t* items, int n_items, const int32_t* item_range,
+                                 const int32_t* dispatch_order,
+                                 const float* pi_k_t, const float* pi_v, const float* codebooks,
+                                 const float* codebooks_host, const float* inv_scales,
+                                 void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
+                                 void* stream) {
+    return decode_launch(q, q_dtype, B, Hq, scaling, store, items, n_items, item_range, dispatch_order, pi_k_t, pi_v,
+                         codebooks, codebooks_host, inv_scales, out, out_dtype, lse, workspace, workspace_bytes, stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same call for callers that cannot allocate and have no workspace to hand over: the partial
+// results and the prepared queries live in a fixed array of the library's own device image.
+// ------------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[ODMKV_STATIC_SCRATCH_BYTES];
+
+#include <mutex>
+#define ODMKV_MAX_DEVICES 64
+static void* g_scratch_ptr[ODMKV_MAX_DEVICES];      // device address of `scratch` per device, looked up once
+static std::mutex g_scratch_mutex;
+
+// the address of this device's copy of `scratch` (every device that loads the library holds its own)
+static int static_scratch(void** ptr) {
+    int dev = -1;
+    ODMKV_CHECK_HIP(hipGetDevice(&dev));
+    ODMKV_CHECK_ARG(dev >= 0 && dev < ODMKV_MAX_DEVICES, "decode_attn_static: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        ODMKV_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" int odmkv_decode_attn_static(const void* q, int q_dtype, int B, int Hq, float scaling,
+                                        const odmkv_packed_t* store,
+                                        const int32_t* items, int n_items, const int32_t* item_range,
+                                        const int32_t* dispatch_order,
+                                        const float* pi_k_t, const float* pi_v, const float* codebooks,
+                                        const float* codebooks_host, const float* inv_scales,
+                                        void* out, int out_dtype, float* lse, void* stream) {
+    ODMKV_CHECK_ARG(B > 0 && Hq > 0 && n_items >= 0, "decode_attn_static: bad shape B=%d Hq=%d items=%d", B, Hq, n_items);
+    const size_t need = odmkv_decode_workspace_bytes(B, Hq, n_items);
+    if (need > (size_t)ODMKV_STATIC_SCRATCH_BYTES) {
+        odmkv_set_error("decode_attn_static: B=%d Hq=%d items=%d need %zu bytes of scratch, the fixed array holds %zu; "
+                        "use odmkv_decode_attn with a workspace", B, Hq, n_items, need, (size_t)ODMKV_STATIC_SCRATCH_BYTES);
+        return ODMKV_ENOSPACE;
+    }
+    void* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    return decode_launch(q, q_dtype, B, Hq, scaling, store, items, n_items, item_range, dispatch_order, pi_k_t, pi_v,
+                         codebooks, codebooks_host, inv_scales, out, out_dtype, lse, ws, (size_t)ODMKV_STATIC_SCRATCH_BYTES, stream);
 }
