@@ -10,11 +10,11 @@ over all layers' packed caches, launched layer after layer on one stream.  The p
 32 layers (~0.6 GB) do not fit the 256 MB last-level cache, so every step streams them from HBM.
 
 Prints ONE JSON line:
-  value          whole-job GB/s = packed bytes of all layers / mean step time (prep + main + merge
+  value          whole-job GB/s = packed bytes of all layers / mean step time (query preparation + main
                  kernels and launch gaps included; inputs resident in HBM; the step is replayed as
                  one HIP graph unless --no-graph)
-  roofline       the main streaming kernel alone: packed bytes per launch / its mean duration from
-                 HIP events recorded around it on its own stream, against 8 TB/s
+  roofline       the main kernel alone (streaming + the merge at its end): packed bytes per launch / its
+                 mean duration from HIP events on its own stream, against 8 TB/s
   cpu_baseline   the oracle's restatement of the reference's CPU decode step (SDPA over the
                  re-materialised cache) on this box's host cores, in the same unit
 and, as extra fields, the per-layer score+allocate+pack time (the second half of the metric).
@@ -35,25 +35,60 @@ for p in (ROOT, os.path.join(ROOT, "odm-kv_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the main decode kernel on the default workload, from the L2 counters
-# (FETCH_SIZE and WRITE_SIZE, one rocprofv3 --pmc run each, scaled by a 256 MiB copy of known size):
-# 20.16 MB fetched + 0.54 MB written.  Applies to --layers 32 --ctx 32768 --target 2.0 only.
-MEASURED_TRAFFIC_BYTES = 20.70e6
+# HBM bytes per launch of the main decode kernel on the default workload, NOT measured by this run: from
+# the L2 counters of two rocprofv3 --pmc runs of `python bench.py --traffic-probe` (FETCH_SIZE, WRITE_SIZE),
+# each scaled by what the same counter reads for a 256 MiB device copy; the figures and the commands are in
+# profiles/decode_main_c2_32k_hbm_traffic.txt.  Applies to --layers 32 --ctx 32768 --target 2.0 only.
+TRAFFIC_FROM_PROFILE_BYTES = None
 LEVELS = (0, 2, 3, 4, 8, 16)
 
 
-def make_layer(seed, n_kv, n_q, T, dev):
-    """K, V ~ N(0,1) fp16 with 8x sinks, expected query mu, decode query q: drawn on the GPU."""
-    import torch
-    g = torch.Generator(device=dev)
-    g.manual_seed(seed)
-    k = torch.randn(n_kv, T, 128, generator=g, device=dev)
-    v = torch.randn(n_kv, T, 128, generator=g, device=dev)
-    k[:, :4] *= 8
-    v[:, :4] *= 8
-    mu = torch.randn(n_q, 64, 128, generator=g, device=dev).mean(dim=1)
-    q = torch.randn(1, n_q, 128, generator=g, device=dev).half().float()
-    return k.half(), v.half(), mu, q
+def make_layer(li, n_kv, n_q, T, dev):
+    """One layer of the workload, drawn from the CPU generator (the same numbers on every machine):
+    K, V ~ N(0,1) fp16 with 8x sinks, expected query mu, decode query q."""
+    import synthetic
+    if (n_kv, n_q) == (8, 32):
+        L = synthetic.config("c2", layer=li, T=T)
+    elif (n_kv, n_q) == (4, 28):
+        L = synthetic.config("c5", layer=li, T=T)
+    else:
+        L = synthetic.gaussian_layer(2002 + li, n_kv, n_q, T)
+    return L.keys.to(dev), L.values.to(dev), L.mu.to(dev), L.query[None].to(dev)
+
+
+def load_bench_lib():
+    """libodmkv_bench.so: the product library's object files plus the measurement entry points of
+    include/odmkv_bench.h (stage selection per call, kernel timing, a plain read)."""
+    from kvquant import _lib
+    path = os.path.join(ROOT, "odm-kv_amd", "lib", "libodmkv_bench.so")
+    lib = C.CDLL(path)
+    i32, vp, f32, sz = C.c_int, C.c_void_p, C.c_float, C.c_size_t
+    lib.odmkv_last_error.restype = C.c_char_p
+    lib.odmkv_bench_timer_create.argtypes = [i32, C.POINTER(vp)]
+    lib.odmkv_bench_timer_collect.argtypes = [vp, C.POINTER(C.c_float), i32, C.POINTER(C.c_int)]
+    lib.odmkv_bench_timer_destroy.argtypes = [vp]
+    lib.odmkv_bench_decode_attn.argtypes = [vp, i32, i32, i32, f32, C.POINTER(_lib.Packed), vp, i32, vp, vp, vp, vp, vp,
+                                            C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp, sz, vp, i32, vp]
+    lib.odmkv_bench_probe_read.argtypes = [vp, sz, i32, vp, vp]
+    lib.odmkv_decode_workspace_bytes.restype = sz
+    lib.odmkv_decode_workspace_bytes.argtypes = [i32, i32, i32]
+    return lib
+
+
+def bench_decode(blib, st, q, out, ws, stage_mask=7, timer=None):
+    """The call of TurboQuantAdaptiveKVCacheState.decode_attention through the measurement library."""
+    from kvquant import _lib
+    if st._items is None:
+        st._build_items()
+    items, ranges, n_items = st._items
+    B, Hq, _ = q.shape
+    rc = blib.odmkv_bench_decode_attn(
+        q.data_ptr(), _lib.dtype_code(q), B, Hq, 128 ** -0.5, C.byref(st._packed), items.data_ptr(), n_items,
+        ranges.data_ptr(), _lib.ptr(st._item_order), st._pi_k_t.data_ptr(), st.pi_v.data_ptr(), st._decode_cb.data_ptr(),
+        st._decode_cb_host, st._decode_inv, out.data_ptr(), _lib.dtype_code(out), None, ws.data_ptr(), ws.numel(),
+        _lib.stream_ptr(q.device), stage_mask, timer)
+    if rc != 0:
+        raise RuntimeError(blib.odmkv_last_error().decode())
 
 
 def parity_gate(dev):
@@ -363,6 +398,7 @@ def main() -> int:
         print(json.dumps({"score_window": out}))
         return 0
 
+    blib = load_bench_lib()
     if args.read_ceiling:
         # what can ONE launch of a given size reach?  buffers rotate through 2 GiB so every launch reads HBM
         pool = torch.ones(2 << 30, dtype=torch.uint8, device=dev)
@@ -374,8 +410,9 @@ def main() -> int:
             for grid in (1024, 2048, 4096):
                 def sweep():
                     for it in range(nbuf):
-                        _lib.check(_lib.lib.odmkv_probe_read(pool.data_ptr() + it * stride, nbytes, grid, sink.data_ptr(),
-                                                             _lib.stream_ptr(dev)))
+                        rc = blib.odmkv_bench_probe_read(pool.data_ptr() + it * stride, nbytes, grid, sink.data_ptr(),
+                                                         _lib.stream_ptr(dev))
+                        assert rc == 0, blib.odmkv_last_error()
                 # the launches of one sweep over the buffers go back to back (one graph), timed between two
                 # events: event pairs around single launches would add about 2 us to each
                 side = torch.cuda.Stream()
@@ -408,7 +445,7 @@ def main() -> int:
     states, qs, t_stage = [], [], {"score": [], "alloc": [], "pack": [], "total": []}
     dense0 = None
     for li in range(NL):
-        k, v, mu, q = make_layer(2002 + li, n_kv, n_q, T, dev)
+        k, v, mu, q = make_layer(li, n_kv, n_q, T, dev)
         for rep in range(2 if li == 0 else 1):               # the first pass also warms allocators
             st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=dev, dtype=torch.float16, key_quantizer="mse",
                                                 value_quantizer="mse", seed=42 + 7 * li)
@@ -454,15 +491,29 @@ def main() -> int:
         for st, q in zip(states, qs):
             st.decode_attention(q)
 
+    # the measurement calls go through libodmkv_bench.so with the stores' own buffers; outputs and workspaces
+    # are allocated once, outside every timed region
+    for st in states:
+        if st._items is None:
+            st._build_items()
+    ws_bytes = max(blib.odmkv_decode_workspace_bytes(1, n_q, st._items[2]) for st in states)
+    b_ws = [torch.empty(ws_bytes, dtype=torch.uint8, device=dev) for _ in states]
+    b_out = [torch.empty(1, n_q, 128, dtype=torch.float32, device=dev) for _ in states]
+
+    def bench_step(stage_mask=7, timer=None):
+        for st, q, o, w in zip(states, qs, b_out, b_ws):
+            bench_decode(blib, st, q, o, w, stage_mask, timer)
+
     def collect_kernel_ms(n_launches, fn):
-        """Durations of the main streaming kernel from the library's HIP events (launch stream)."""
-        _lib.check(_lib.lib.odmkv_profile_enable(n_launches + 8))
-        fn()
+        """Durations of the main kernel from HIP events attached to its dispatches (launch stream)."""
+        timer = C.c_void_p()
+        assert blib.odmkv_bench_timer_create(n_launches + 8, C.byref(timer)) == 0, blib.odmkv_last_error()
+        fn(timer)
         torch.cuda.synchronize()
         buf = (C.c_float * (n_launches + 8))()
         n = C.c_int(0)
-        _lib.check(_lib.lib.odmkv_profile_collect(buf, len(buf), C.byref(n)))
-        _lib.check(_lib.lib.odmkv_profile_disable())
+        assert blib.odmkv_bench_timer_collect(timer, buf, len(buf), C.byref(n)) == 0, blib.odmkv_last_error()
+        blib.odmkv_bench_timer_destroy(timer)
         return sorted(buf[i] for i in range(n.value))
 
     if args.traffic_probe:
@@ -480,7 +531,7 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
 
-    # the timed region replays one captured step (96 kernels) so that the host's per-call work does
+    # the timed region replays one captured step (64 kernels) so that the host's per-call work does
     # not sit between the kernels; falls back to launching from Python if capture is not possible
     graph, launch_mode = None, "python"
     if not args.no_graph:
@@ -512,42 +563,39 @@ def main() -> int:
 
     # kernel durations: an eager pass over the same rotating 32 buffers, then one buffer alone (cache-resident)
     prof_steps = min(args.steps, 20)
-    kernel_ms = collect_kernel_ms(prof_steps * NL, lambda: [step() for _ in range(prof_steps)])
-    hot_ms = collect_kernel_ms(200, lambda: [states[0].decode_attention(qs[0]) for _ in range(200)])
+    kernel_ms = collect_kernel_ms(prof_steps * NL, lambda t: [bench_step(7, t) for _ in range(prof_steps)])
+    hot_ms = collect_kernel_ms(200, lambda t: [bench_decode(blib, states[0], qs[0], b_out[0], b_ws[0], 7, t) for _ in range(200)])
 
-    def main_kernel_alone_ms(reps):
-        """Average duration of the main kernel over the rotating buffers: the step's 32 main-kernel
-        launches alone (no preparation, no merge: they reuse what the last full step left in the
-        workspaces), captured as one graph and replayed between two HIP events on the launch stream.
-        Per-launch event pairs (above) add about 2 us to every launch; this does not."""
-        old = _lib.lib.odmkv_decode_stage_mask(2)
-        try:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                step()
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            gk = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gk):
-                step()
-            for _ in range(3):
-                gk.replay()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            e0.record()
-            for _ in range(reps):
-                gk.replay()
-            e1.record()
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) / (reps * NL)
-        finally:
-            _lib.lib.odmkv_decode_stage_mask(old)
+    def graph_ms_per_launch(stage_mask, reps):
+        """The step's 32 decode calls with the given stages, captured as one graph and replayed between two
+        HIP events on the launch stream; elapsed / launches.  Per-launch event pairs (above) add about 2 us
+        to every launch; this does not."""
+        bench_step(7)                                    # a full call fills the workspaces the partial stages reuse
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            bench_step(stage_mask)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        gk = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gk):
+            bench_step(stage_mask)
+        for _ in range(3):
+            gk.replay()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            gk.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (reps * NL)
 
-    kern_alone_ms = None
+    kern_alone_ms = stream_only_ms = None
     if graph is not None:
         try:
-            kern_alone_ms = main_kernel_alone_ms(min(args.steps, 50))
+            kern_alone_ms = graph_ms_per_launch(6, min(args.steps, 50))      # main kernel with its merge, no preparation
+            stream_only_ms = graph_ms_per_launch(2, min(args.steps, 50))     # its streaming part alone
         except Exception as exc:                                   # noqa: BLE001
             print(f"main-kernel-only graph not available ({exc}); using per-launch events", file=sys.stderr)
             torch.cuda.synchronize()
@@ -578,10 +626,13 @@ def main() -> int:
         "parity": {"gate_attn_rel_err": gate_err, "full_size_fused_vs_dense_rel_err": full_err},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES if (NL, T, args.target) == (32, 32768, 2.0) else None,
+                     "traffic": TRAFFIC_FROM_PROFILE_BYTES if (NL, T, args.target) == (32, 32768, 2.0) else None,
+                     "traffic_source": "profiles/decode_main_c2_32k_hbm_traffic.txt (rocprofv3 --pmc runs, not this run)",
                      "kernel": "decode_main_kernel", "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
-                     "kernel_avg_method": ("32 main-kernel launches alone as one graph, replayed between two HIP events"
+                     "kernel_avg_method": ("the step's main-kernel launches (streaming + merge, no query preparation) alone "
+                                           "as one graph, replayed between two HIP events"
                                            if kern_alone_ms is not None else "per-launch HIP event pairs"),
+                     "streaming_part_only_us": None if stream_only_ms is None else round(stream_only_ms * 1e3, 2),
                      "per_launch_events_avg_us": round(events_avg_ms * 1e3, 2),
                      "per_launch_events_median_us": round(pct(kernel_ms, 50) * 1e3, 2),
                      "per_launch_events_p10_us": round(pct(kernel_ms, 10) * 1e3, 2),
@@ -589,11 +640,12 @@ def main() -> int:
                      "single_buffer_cache_resident_median_us": round(pct(hot_ms, 50) * 1e3, 2)},
     }
     if not args.no_cpu:
-        threads = os.cpu_count() or 1
-        threads = min(threads, 16)
+        # the GPU box hands one job a 16-thread share of its host, whatever os.cpu_count() shows
+        threads = min(os.cpu_count() or 1, 16)
         cb = cpu_baseline(args.cpu_sample_ctx, n_kv, n_q, eps, threads)
         out["cpu_baseline"] = {
-            "value": round(cb["packed_bytes"] / cb["t_sdpa"] / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "value": round(cb["packed_bytes"] / cb["t_sdpa"] / 1e9, 3), "unit": "GB/s", "cores": threads,
+            "host_cpu_count": os.cpu_count(), "kind": "port",
             "sample": f"one layer, T={args.cpu_sample_ctx}: oracle compress, then median of 5 torch-CPU fp32 SDPA calls over "
                       "the re-materialised dense cache (what a reference decode step costs), packed bytes / time",
             "sdpa_ms": round(cb["t_sdpa"] * 1e3, 2), "materialize_ms": round(cb["t_materialize"] * 1e3, 1),

@@ -268,28 +268,6 @@ int odmkv_decode_attn_static(const void* q, int q_dtype, int B, int Hq, float sc
                              const float* codebooks_host, const float* inv_scales,
                              void* out, int out_dtype, float* lse, void* stream);
 
-/* ---------------------------------------------------------------------------------------------
- * Measurement hooks (no counterpart in the reference).  While enabled, every odmkv_decode_attn
- * call records a pair of HIP events around its main (streaming) kernel on the caller's stream;
- * odmkv_profile_collect waits for them and returns the kernel durations in milliseconds.
- * The event pool is created by odmkv_profile_enable and destroyed by odmkv_profile_disable.
- */
-int odmkv_profile_enable(int max_records);
-int odmkv_profile_collect(float* ms, int capacity, int* n_out);
-int odmkv_profile_disable(void);
-
-/* Which of the three kernels of odmkv_decode_attn later calls launch: bit 0 the query preparation,
- * bit 1 the main (streaming) kernel, bit 2 the merge.  7 (the default) is the product behaviour; any
- * other value is for timing one kernel in isolation over buffers that a full call has filled
- * (e.g. 2: the main kernel alone, back to back, between two events).  Returns the previous mask. */
-int odmkv_decode_stage_mask(int mask);
-
-/* Yardstick for the roofline (no counterpart in the reference): a plain streaming read of `bytes`
- * bytes at `buf` (device, 16-byte aligned) by `grid` workgroups of 256 threads; `sink` is a device
- * word that is practically never written.  Timing it over buffers that rotate through more than
- * the last-level cache shows what one launch of that size can reach on the machine. */
-int odmkv_probe_read(const void* buf, size_t bytes, int grid, void* sink, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

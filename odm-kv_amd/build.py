@@ -1,4 +1,6 @@
-"""Builds libodmkv.so (the HIP kernels and their C ABI) for gfx950 with hipcc.
+"""Builds libodmkv.so (the HIP kernels and their C ABI) for gfx950 with hipcc, and
+libodmkv_bench.so: the same object files plus the measurement entry points of csrc/bench_hooks.hip
+(include/odmkv_bench.h), which the product library does not export.
 
     python odm-kv_amd/build.py [--force]
 
@@ -18,7 +20,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libodmkv.so")
+BENCH_LIB = os.path.join(LIBDIR, "libodmkv_bench.so")
 SOURCES = ["error.hip", "score.hip", "window.hip", "allocate.hip", "pack.hip", "rows.hip", "decode.hip"]
+BENCH_SOURCES = ["bench_hooks.hip"]
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -31,9 +35,11 @@ def _newest(paths):
 
 
 def build(force: bool = False, verbose: bool = True) -> str:
-    srcs = [os.path.join(CSRC, s) for s in SOURCES]
-    deps = srcs + [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "quant.h"), os.path.join(HERE, "..", "include", "odmkv.h"), __file__]
-    if not force and os.path.exists(LIB) and os.path.getmtime(LIB) >= _newest(deps):
+    srcs = [os.path.join(CSRC, s) for s in SOURCES + BENCH_SOURCES]
+    deps = srcs + [os.path.join(CSRC, h) for h in ("common.h", "quant.h", "decode.h")] + [
+        os.path.join(HERE, "..", "include", "odmkv.h"), os.path.join(HERE, "..", "include", "odmkv_bench.h"), __file__]
+    if (not force and os.path.exists(LIB) and os.path.exists(BENCH_LIB)
+            and min(os.path.getmtime(LIB), os.path.getmtime(BENCH_LIB)) >= _newest(deps)):
         return LIB
     os.makedirs(LIBDIR, exist_ok=True)
     objdir = os.path.join(HERE, "build")
@@ -54,10 +60,12 @@ def build(force: bool = False, verbose: bool = True) -> str:
 
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         objs = list(ex.map(compile_one, srcs))
-    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+    product = objs[:len(SOURCES)]
+    for lib, parts in ((LIB, product), (BENCH_LIB, objs)):
+        cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *parts]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
     return LIB
 
 

@@ -1,0 +1,44 @@
+// Internal interface of the fused decode attention: shared by the product entry points (decode.hip)
+// and the measurement entry points (bench_hooks.hip, a library of its own).  Not part of the C ABI.
+#pragma once
+#include "quant.h"
+#include <hip/hip_ext.h>
+
+#define PSTRIDE 132          // floats per (item, head) partial result: 128 acc + m + l + 2 pad
+#ifndef DECODE_NWAVES
+#define DECODE_NWAVES 8      // wavefronts of a workgroup of the main kernel
+#endif
+
+struct DecodeArgs {
+    odmkv_packed_t s;
+    const void* q;
+    int q_dt, out_dt;   // element types of q and out (ODMKV_F16 / BF16 / F32)
+    int Hq, G, B;
+    float scaling;
+    const int32_t* items;
+    const int32_t* item_range;
+    const int32_t* order;      // order[k] = item that workgroup k takes (long items first), or null: item k
+    const float* pi_k_t;   // Pi_k transposed
+    const float* pi_v;
+    const float* cb;
+    uint4* qrot;      // [B*Hq][2][128] fp16: high and low halves of Pi_k q16
+    uint4* qs;        // [B*Hq][2][128] q16 itself for the exact tokens (fp16 + zeros, or bf16 high + low pieces)
+    unsigned int* tickets;   // [B*Hkv] items of the (sequence, kv-head) that have finished
+    float inv_s[4];   // 1 / table scale per width
+    float cbs[28];    // scaled centroids of widths 2, 3, 4 (kept in scalar registers; 8-bit ones stay in memory)
+    int gp;           // head slots per item in `partial`: 4 or 8
+    float* partial;   // [n_items, gp, PSTRIDE]
+    void* out;
+    float* lse;
+};
+
+// stage_mask: bit 0 the query preparation, bit 1 the main kernel, bit 2 the merge at its end (7 = the
+// product call).  ev_start / ev_stop: hipEvent_t attached to the main kernel's dispatch, or null.
+int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling,
+                        const odmkv_packed_t* store,
+                        const int32_t* items, int n_items, const int32_t* item_range,
+                        const int32_t* dispatch_order,
+                        const float* pi_k_t, const float* pi_v, const float* codebooks,
+                        const float* codebooks_host, const float* inv_scales,
+                        void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
+                        void* stream, int stage_mask, void* ev_start, void* ev_stop);

@@ -1,9 +1,10 @@
 // Packed mixed-width KV store: level counts, position compaction, TurboQuant-MSE quantise + pack,
 // exact-row gather, decode-time append, and dequantise-to-dense.
 //
-// One wavefront owns one 64-token tile.  The quantiser runs the rotation on the fp32 matrix cores
-// one k at a time; the dequantiser keeps a token per lane and walks the rotation matrix through
-// scalar (wave-uniform) loads.  Both keep the sequential fp32 summation order of the definition.
+// One wavefront owns one 64-token tile.  The quantiser and the dequantiser run the rotation on the
+// fp32 matrix cores one k at a time, a token per lane, and keep the sequential fp32 summation order of
+// the definition; the tile's own layout (what the decode kernel's matrix operands want, quant.h) is
+// produced and consumed by a re-layout through LDS.
 #include <algorithm>
 #include "quant.h"
 
@@ -337,13 +338,21 @@ __device__ static __forceinline__ void stage_direct_k(const f32x32& a0, const f3
     }
 }
 
+// lane (n, j) gathers dims 32j..32j+31 of slots 4n..4n+3 from the staged token streams
 template <int W>
 __device__ static __forceinline__ void store_direct_k(const uint8_t* stage, uint8_t* kcodes, int tile, int lane) {
+    const int n = lane & 15, j = lane >> 4;
+    uint32_t words[4 * W];
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int i = 0; i < W; ++i)
+            words[b * W + i] = *reinterpret_cast<const uint32_t*>(stage + (4 * n + b) * Direct<W>::ROW_K + 4 * W * j + 4 * i);
     uint8_t* dst = kcodes + (size_t)tile * (TILE * 16 * W);
 #pragma unroll
     for (int ch = 0; ch < W; ++ch)
         *reinterpret_cast<uint4*>(dst + ((size_t)ch * TILE + lane) * 16) =
-            *reinterpret_cast<const uint4*>(stage + lane * Direct<W>::ROW_K + 16 * ch);
+            make_uint4(words[4 * ch], words[4 * ch + 1], words[4 * ch + 2], words[4 * ch + 3]);
 }
 
 template <int W>
@@ -357,77 +366,99 @@ __device__ static __forceinline__ void stage_direct_v(const f32x32& acc, int g, 
     }
 }
 
+// lane (n, j) gathers slots 32k+8j..+7 (k = 0, 1) of dims 16m+n (m = 0..7) from the staged dim streams:
+// W bytes per (k, m)
 template <int W>
 __device__ static __forceinline__ void store_direct_v(const uint8_t* stage, uint8_t* vcodes, int tile, int lane) {
-    uint8_t* dst = vcodes + (size_t)tile * (HD * 8 * W);
+    const int n = lane & 15, j = lane >> 4;
+    uint32_t words[4 * W];
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-        const int j = lane + 64 * half;
+    for (int i = 0; i < 4 * W; ++i) words[i] = 0u;
 #pragma unroll
-        for (int u = 0; u < W / 2; ++u) {                                  // 16-byte units of the dim's stream
-            const uint2 x = *reinterpret_cast<const uint2*>(stage + j * Direct<W>::ROW_V + 16 * u);
-            const uint2 y = *reinterpret_cast<const uint2*>(stage + j * Direct<W>::ROW_V + 16 * u + 8);
-            *reinterpret_cast<uint4*>(dst + ((size_t)u * HD + j) * 16) = make_uint4(x.x, x.y, y.x, y.y);
+    for (int k = 0; k < 2; ++k)
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const uint8_t* src = stage + (16 * m + n) * Direct<W>::ROW_V + (4 * k + j) * W;
+            const int g = 8 * k + m;                                       // group of 8 codes = W bytes of the lane's stream
+            if constexpr (W == 2) words[g >> 1] |= (uint32_t)(*reinterpret_cast<const uint16_t*>(src)) << (16 * (g & 1));
+            else if constexpr (W == 4) words[g] = *reinterpret_cast<const uint32_t*>(src);
+            else { const uint2 v = *reinterpret_cast<const uint2*>(src); words[2 * g] = v.x; words[2 * g + 1] = v.y; }
         }
-    }
+    uint8_t* dst = vcodes + (size_t)tile * (TILE * 16 * W);
+#pragma unroll
+    for (int ch = 0; ch < W; ++ch)
+        *reinterpret_cast<uint4*>(dst + ((size_t)ch * TILE + lane) * 16) =
+            make_uint4(words[4 * ch], words[4 * ch + 1], words[4 * ch + 2], words[4 * ch + 3]);
 }
 
-template <int W>
-__device__ static __forceinline__ void pack_store_k(const uint8_t* stage, uint8_t* kcodes, int tile, int lane) {
+// Generic stores (any width; tiles that already hold `lo` tokens keep them: KEEP).  Slots at and behind
+// `hi` receive the codes of zero rows; they are not counted by anybody until a later call fills them.
+template <int W, bool KEEP>
+__device__ static __forceinline__ void pack_store_k(const uint8_t* stage, uint8_t* kcodes, int tile, int lane, int lo) {
+    const int n = lane & 15, j = lane >> 4;
+    uint8_t* dst = kcodes + (size_t)tile * (TILE * 16 * W);
     uint32_t words[4 * W];
 #pragma unroll
     for (int k = 0; k < 4 * W; ++k) words[k] = 0;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        const uint4 v = *reinterpret_cast<const uint4*>(stage + lane * CODE_ROW + 16 * c);
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    for (int b = 0; b < 4; ++b) {
+        const uint4 v0 = *reinterpret_cast<const uint4*>(stage + (4 * n + b) * CODE_ROW + 32 * j);
+        const uint4 v1 = *reinterpret_cast<const uint4*>(stage + (4 * n + b) * CODE_ROW + 32 * j + 16);
+        const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
-        for (int e = 0; e < 16; ++e) put_code<W>(words, 16 * c + e, (w[e >> 2] >> (8 * (e & 3))) & 0xffu);
+        for (int e = 0; e < 32; ++e) put_code<W>(words, 32 * b + e, (w[e >> 2] >> (8 * (e & 3))) & 0xffu);
     }
-    uint8_t* dst = kcodes + (size_t)tile * (TILE * 16 * W);
+    if constexpr (KEEP) {
+        // a slot's codes are W whole words of the lane's stream
+#pragma unroll
+        for (int c = 0; c < W; ++c) {
+            const uint4 old = *reinterpret_cast<const uint4*>(dst + ((size_t)c * TILE + lane) * 16);
+            const uint32_t o[4] = {old.x, old.y, old.z, old.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int b = (4 * c + i) / W;
+                if (4 * n + b < lo) words[4 * c + i] = o[i];
+            }
+        }
+    }
 #pragma unroll
     for (int c = 0; c < W; ++c)
         *reinterpret_cast<uint4*>(dst + ((size_t)c * TILE + lane) * 16) =
             make_uint4(words[4 * c], words[4 * c + 1], words[4 * c + 2], words[4 * c + 3]);
 }
 
-template <int W>
-__device__ static __forceinline__ void pack_store_v(const uint8_t* stage, uint8_t* vcodes, int tile, int lane, int lo, int hi) {
-    uint8_t* dst = vcodes + (size_t)tile * (HD * 8 * W);
+template <int W, bool KEEP>
+__device__ static __forceinline__ void pack_store_v(const uint8_t* stage, uint8_t* vcodes, int tile, int lane, int lo) {
+    const int n = lane & 15, j = lane >> 4;
+    uint8_t* dst = vcodes + (size_t)tile * (TILE * 16 * W);
+    uint32_t old[4 * W];
+    if constexpr (KEEP) {
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-        const int j = lane + 64 * half;
-        uint32_t words[2 * W];
+        for (int c = 0; c < W; ++c) {
+            const uint4 o = *reinterpret_cast<const uint4*>(dst + ((size_t)c * TILE + lane) * 16);
+            old[4 * c] = o.x; old[4 * c + 1] = o.y; old[4 * c + 2] = o.z; old[4 * c + 3] = o.w;
+        }
+    }
+    uint32_t words[4 * W];
 #pragma unroll
-        for (int k = 0; k < 2 * W; ++k) words[k] = 0;
+    for (int k = 0; k < 4 * W; ++k) words[k] = 0;
 #pragma unroll
-        for (int t8 = 0; t8 < 8; ++t8) {
-            const uint2 v = *reinterpret_cast<const uint2*>(stage + j * CODE_ROW_T + 8 * t8);
+    for (int k = 0; k < 2; ++k)
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const uint2 v = *reinterpret_cast<const uint2*>(stage + (16 * m + n) * CODE_ROW_T + 32 * k + 8 * j);
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const int t = 8 * t8 + e;
+                const int ci = 64 * k + 8 * m + e;
                 uint32_t c = ((e < 4 ? v.x : v.y) >> (8 * (e & 3))) & 0xffu;
-                c = (t >= lo && t < hi) ? c : 0u;
-                put_code<W>(words, t, c);
-            }
-        }
-        if (lo > 0) {
-            // tokens below `lo` were packed earlier: keep their bits
-            const int keep_bits = lo * W;
-#pragma unroll
-            for (int k = 0; k < 2 * W; ++k) {
-                const int nb = keep_bits - 32 * k;
-                if (nb > 0) {
-                    const uint32_t old = *reinterpret_cast<const uint32_t*>(dst + v_word_offset<W>(k, j));
-                    const uint32_t mask = nb >= 32 ? 0xffffffffu : ((1u << nb) - 1u);
-                    words[k] = (old & mask) | (words[k] & ~mask);
-                }
+                if constexpr (KEEP) c = (32 * k + 8 * j + e < lo) ? get_code<W>(old, ci) : c;     // stored earlier: keep
+                put_code<W>(words, ci, c);
             }
         }
 #pragma unroll
-        for (int k = 0; k < 2 * W; ++k)
-            *reinterpret_cast<uint32_t*>(dst + v_word_offset<W>(k, j)) = words[k];
-    }
+    for (int c = 0; c < W; ++c)
+        *reinterpret_cast<uint4*>(dst + ((size_t)c * TILE + lane) * 16) =
+            make_uint4(words[4 * c], words[4 * c + 1], words[4 * c + 2], words[4 * c + 3]);
 }
 
 // LDS writes of this wave visible to its own later reads (no other wave touches its staging area)
@@ -616,23 +647,28 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
                 }
             }
             wave_lds_fence();
-            if (valid) {
-                if (direct) {
-                    switch (li) {
-                        case 0: store_direct_k<2>(stage, a.s.kcodes[0], tile, ln); break;
-                        case 2: store_direct_k<4>(stage, a.s.kcodes[2], tile, ln); break;
-                        default: store_direct_k<8>(stage, a.s.kcodes[3], tile, ln); break;
-                    }
-                } else {
-                    switch (li) {
-                        case 0: pack_store_k<2>(stage, a.s.kcodes[0], tile, ln); break;
-                        case 1: pack_store_k<3>(stage, a.s.kcodes[1], tile, ln); break;
-                        case 2: pack_store_k<4>(stage, a.s.kcodes[2], tile, ln); break;
-                        default: pack_store_k<8>(stage, a.s.kcodes[3], tile, ln); break;
-                    }
+            if (direct) {
+                switch (li) {
+                    case 0: store_direct_k<2>(stage, a.s.kcodes[0], tile, ln); break;
+                    case 2: store_direct_k<4>(stage, a.s.kcodes[2], tile, ln); break;
+                    default: store_direct_k<8>(stage, a.s.kcodes[3], tile, ln); break;
                 }
-                a.s.knorm[li][slot] = norm;
+            } else if (lo > 0) {
+                switch (li) {
+                    case 0: pack_store_k<2, true>(stage, a.s.kcodes[0], tile, ln, lo); break;
+                    case 1: pack_store_k<3, true>(stage, a.s.kcodes[1], tile, ln, lo); break;
+                    case 2: pack_store_k<4, true>(stage, a.s.kcodes[2], tile, ln, lo); break;
+                    default: pack_store_k<8, true>(stage, a.s.kcodes[3], tile, ln, lo); break;
+                }
+            } else {
+                switch (li) {
+                    case 0: pack_store_k<2, false>(stage, a.s.kcodes[0], tile, ln, 0); break;
+                    case 1: pack_store_k<3, false>(stage, a.s.kcodes[1], tile, ln, 0); break;
+                    case 2: pack_store_k<4, false>(stage, a.s.kcodes[2], tile, ln, 0); break;
+                    default: pack_store_k<8, false>(stage, a.s.kcodes[3], tile, ln, 0); break;
+                }
             }
+            if (valid) a.s.knorm[li][slot] = norm;
         } else {
             if (direct) {
                 switch (li) {
@@ -661,11 +697,20 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
                              stage_codes_v<8>(acc2, 2, cb, stage, ln); stage_codes_v<8>(acc3, 3, cb, stage, ln); break;
                 }
                 wave_lds_fence();
-                switch (li) {
-                    case 0: pack_store_v<2>(stage, a.s.vcodes[0], tile, ln, lo, hi); break;
-                    case 1: pack_store_v<3>(stage, a.s.vcodes[1], tile, ln, lo, hi); break;
-                    case 2: pack_store_v<4>(stage, a.s.vcodes[2], tile, ln, lo, hi); break;
-                    default: pack_store_v<8>(stage, a.s.vcodes[3], tile, ln, lo, hi); break;
+                if (lo > 0) {
+                    switch (li) {
+                        case 0: pack_store_v<2, true>(stage, a.s.vcodes[0], tile, ln, lo); break;
+                        case 1: pack_store_v<3, true>(stage, a.s.vcodes[1], tile, ln, lo); break;
+                        case 2: pack_store_v<4, true>(stage, a.s.vcodes[2], tile, ln, lo); break;
+                        default: pack_store_v<8, true>(stage, a.s.vcodes[3], tile, ln, lo); break;
+                    }
+                } else {
+                    switch (li) {
+                        case 0: pack_store_v<2, false>(stage, a.s.vcodes[0], tile, ln, 0); break;
+                        case 1: pack_store_v<3, false>(stage, a.s.vcodes[1], tile, ln, 0); break;
+                        case 2: pack_store_v<4, false>(stage, a.s.vcodes[2], tile, ln, 0); break;
+                        default: pack_store_v<8, false>(stage, a.s.vcodes[3], tile, ln, 0); break;
+                    }
                 }
             }
             if (valid) a.s.vnorm[li][slot] = norm;
@@ -718,12 +763,11 @@ __global__ __launch_bounds__(64) void exact_gather_kernel(ExactArgs a) {
         pk.y = Elem<ODT>::from_f32(x[8 * c + 2]) | ((uint32_t)Elem<ODT>::from_f32(x[8 * c + 3]) << 16);
         pk.z = Elem<ODT>::from_f32(x[8 * c + 4]) | ((uint32_t)Elem<ODT>::from_f32(x[8 * c + 5]) << 16);
         pk.w = Elem<ODT>::from_f32(x[8 * c + 6]) | ((uint32_t)Elem<ODT>::from_f32(x[8 * c + 7]) << 16);
-        *reinterpret_cast<uint4*>(kd + ((size_t)c * TILE + lane) * 8) = pk;
+        *reinterpret_cast<uint4*>(kd + exact_k_index(lane, 8 * c)) = pk;
     }
     load_row<DT>(a.V, off, x);
 #pragma unroll
-    for (int j = 0; j < HD; ++j)
-        vd[((size_t)(lane >> 2) * HD + j) * 4 + (lane & 3)] = Elem<ODT>::from_f32(x[j]);
+    for (int j = 0; j < HD; ++j) vd[exact_v_index(lane, j)] = Elem<ODT>::from_f32(x[j]);
 }
 
 // one new token per (b, h) behind the stored exact tokens
@@ -739,8 +783,8 @@ __global__ __launch_bounds__(128) void append_exact_kernel(odmkv_packed_t s, con
     const int l = cnt % TILE;
     uint16_t* kd = s.kexact + (size_t)tile * TILE * HD;
     uint16_t* vd = s.vexact + (size_t)tile * TILE * HD;
-    kd[((size_t)(j >> 3) * TILE + l) * 8 + (j & 7)] = k[src];
-    vd[((size_t)(l >> 2) * HD + j) * 4 + (l & 3)] = v[src];
+    kd[exact_k_index(l, j)] = k[src];
+    vd[exact_v_index(l, j)] = v[src];
     __syncthreads();
     if (j == 0) {
         s.pos[4][(size_t)tile * TILE + l] = pos;
@@ -946,24 +990,34 @@ __global__ __launch_bounds__(DQ_NW * 64) void dequant_kernel(DequantArgs a, int 
             offs[lane] = write ? (long long)((size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH + (size_t)t * a.sT) : -1ll;
             norms[lane] = valid ? (is_v ? a.vnorm[slot] : a.knorm[slot]) : 0.0f;
         }
-        uint32_t words[4 * W];                                       // keys: the token's code words
-        if (!is_v) {
-            const uint8_t* src = a.kcodes + (size_t)tile * (TILE * 16 * W);
+        // the lane's 128 codes -> one byte each in LDS, [token][dim]: the matrix instructions below want a
+        // token per lane, the tile keeps (4 tokens x 32 dims) of keys or (16 tokens x 8 dims) of values per lane
+        {
+            const int n = lane & 15, j = lane >> 4;
+            const uint8_t* src = (is_v ? a.vcodes : a.kcodes) + (size_t)tile * (TILE * 16 * W);
+            uint32_t words[4 * W];
 #pragma unroll
             for (int c = 0; c < W; ++c) {
                 const uint4 v = *reinterpret_cast<const uint4*>(src + ((size_t)c * TILE + lane) * 16);
                 words[4 * c] = v.x; words[4 * c + 1] = v.y; words[4 * c + 2] = v.z; words[4 * c + 3] = v.w;
             }
-        } else {                                                     // values are stored dim-major: transpose through LDS
-            const uint8_t* src = a.vcodes + (size_t)tile * (HD * 8 * W);
+            if (!is_v) {
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int j = lane + 64 * half;
-                uint32_t vw[2 * W];
+                for (int b = 0; b < 4; ++b)
 #pragma unroll
-                for (int k = 0; k < 2 * W; ++k) vw[k] = *reinterpret_cast<const uint32_t*>(src + v_word_offset<W>(k, j));
+                    for (int i = 0; i < 32; i += 4) {
+                        const uint32_t w4 = get_code<W>(words, 32 * b + i) | (get_code<W>(words, 32 * b + i + 1) << 8) |
+                                            (get_code<W>(words, 32 * b + i + 2) << 16) | (get_code<W>(words, 32 * b + i + 3) << 24);
+                        *reinterpret_cast<uint32_t*>(&codes[(4 * n + b) * CODE_ROW + 32 * j + i]) = w4;
+                    }
+            } else {
 #pragma unroll
-                for (int t = 0; t < TILE; ++t) codes[t * CODE_ROW + j] = (uint8_t)get_code<W>(vw, t);
+                for (int k = 0; k < 2; ++k)
+#pragma unroll
+                    for (int m = 0; m < 8; ++m)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            codes[(32 * k + 8 * j + e) * CODE_ROW + 16 * m + n] = (uint8_t)get_code<W>(words, 64 * k + 8 * m + e);
             }
         }
         wave_lds_fence();
@@ -974,10 +1028,7 @@ __global__ __launch_bounds__(DQ_NW * 64) void dequant_kernel(DequantArgs a, int 
 #pragma unroll
         for (int i0 = 0; i0 < HD; i0 += DQ_GROUP) {
             float y[DQ_GROUP];
-            if (!is_v) {
-#pragma unroll
-                for (int g = 0; g < DQ_GROUP; ++g) y[g] = cb[get_code<W>(words, i0 + g)];
-            } else {
+            {
                 const uint4 v = *reinterpret_cast<const uint4*>(&codes[lane * CODE_ROW + i0]);
                 const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -1034,8 +1085,8 @@ __global__ __launch_bounds__(64) void exact_scatter_kernel(odmkv_packed_t s, voi
     typename Elem<DT>::raw* kd = reinterpret_cast<typename Elem<DT>::raw*>(K) + off;
     typename Elem<DT>::raw* vd = reinterpret_cast<typename Elem<DT>::raw*>(V) + off;
     for (int j = 0; j < HD; ++j) {
-        const uint16_t kr = ks[((size_t)(j >> 3) * TILE + lane) * 8 + (j & 7)];
-        const uint16_t vr = vs[((size_t)(lane >> 2) * HD + j) * 4 + (lane & 3)];
+        const uint16_t kr = ks[exact_k_index(lane, j)];
+        const uint16_t vr = vs[exact_v_index(lane, j)];
         const float kf = src_bf16 ? Elem<ODMKV_BF16>::to_f32(kr) : Elem<ODMKV_F16>::to_f32(kr);
         const float vf = src_bf16 ? Elem<ODMKV_BF16>::to_f32(vr) : Elem<ODMKV_F16>::to_f32(vr);
         kd[j] = Elem<DT>::from_f32(kf);

@@ -17,12 +17,21 @@ __device__ static inline void put_code(uint32_t* w, int i, uint32_t c) {
     if (sh + W > 32) w[k + 1] |= c >> (32 - sh);
 }
 
-// V layout: word k (of 2W) of dim j lives in a unit of U bytes
-template <int W>
-__device__ static inline size_t v_word_offset(int k, int j) {
-    constexpr int U = (W == 3) ? 8 : 16;
-    constexpr int WPU = U / 4;
-    return ((size_t)(k / WPU) * HD + j) * U + (size_t)(k % WPU) * 4;
+// ---- tile layouts (see include/odmkv.h) ----------------------------------------------------------
+// Every tile buffer is W (codes) or 16 (exact rows) chunks of 16 bytes per lane; chunk c of lane l sits
+// at byte (c*64 + l)*16 of the tile.  Lane l = 16j + n.
+//   key codes:    the lane's 128 codes are  code 32b + i   = dim 32j + i   of slot 4n + b
+//   value codes:  the lane's 128 codes are  code 64k + 8m + e = slot 32k + 8j + e  of dim 16m + n
+//   exact keys:   chunk 4b + k of the lane  = dims 32j + 8k .. + 7 of slot 4n + b
+//   exact values: chunk 8k + m of the lane  = slots 32k + 8j .. + 7 of dim 16m + n
+// index (in 16-bit elements) of element (slot, dim) inside an exact tile
+__host__ __device__ static inline int exact_k_index(int slot, int dim) {
+    const int n = slot >> 2, b = slot & 3, j = dim >> 5, k = (dim >> 3) & 3, e = dim & 7;
+    return (((4 * b + k) * TILE) + 16 * j + n) * 8 + e;
+}
+__host__ __device__ static inline int exact_v_index(int slot, int dim) {
+    const int k = slot >> 5, j = (slot >> 3) & 3, e = slot & 7, m = dim >> 4, n = dim & 15;
+    return (((8 * k + m) * TILE) + 16 * j + n) * 8 + e;
 }
 
 template <int DT>

@@ -67,11 +67,6 @@ def _load() -> C.CDLL:
                                         C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp, sz, vp]),
         "odmkv_decode_attn_static": (C.c_int, [vp, i32, i32, i32, f32, C.POINTER(Packed), vp, i32, vp, vp, vp, vp, vp,
                                                C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp]),
-        "odmkv_profile_enable": (C.c_int, [i32]),
-        "odmkv_profile_collect": (C.c_int, [C.POINTER(C.c_float), i32, C.POINTER(C.c_int)]),
-        "odmkv_profile_disable": (C.c_int, []),
-        "odmkv_decode_stage_mask": (C.c_int, [i32]),
-        "odmkv_probe_read": (C.c_int, [vp, sz, i32, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -86,8 +81,7 @@ EXPORTS = ("odmkv_version", "odmkv_last_error", "odmkv_score_workspace_bytes", "
            "odmkv_allocate_workspace_bytes", "odmkv_allocate", "odmkv_level_counts",
            "odmkv_pack_workspace_bytes", "odmkv_quant_pack", "odmkv_quantize_rows",
            "odmkv_dequantize_rows", "odmkv_dequant", "odmkv_append_exact",
-           "odmkv_decode_workspace_bytes", "odmkv_decode_attn", "odmkv_decode_attn_static",
-           "odmkv_profile_enable", "odmkv_profile_collect", "odmkv_profile_disable", "odmkv_decode_stage_mask", "odmkv_probe_read")
+           "odmkv_decode_workspace_bytes", "odmkv_decode_attn", "odmkv_decode_attn_static")
 
 
 def check(rc: int) -> None:

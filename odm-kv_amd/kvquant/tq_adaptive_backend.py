@@ -8,7 +8,8 @@ makes possible: ``decode_attention`` (fused LUT attention straight from the pack
 ``packed_bytes``.
 
 Layout (see include/odmkv.h): per bit level, tokens of one (sequence, kv-head) form a segment of
-64-token tiles in ascending position; keys are stored token-major, values dim-major, norms fp32.
+64-token tiles in ascending position; codes lie in the order the decode kernel's matrix operands take
+them (keys: 4 tokens x 32 dims per 16*w bytes, values: 16 tokens x 8 dims), norms fp32.
 Evicted (0-bit) tokens are not stored at all.  The host keeps a mirror of every segment's length,
 so that after the one synchronisation an ``append`` needs (to size the buffers from the level
 counts) no later call has to read anything back.
@@ -28,7 +29,19 @@ from .tq_backend import (cached_rotation, codebook_table, decode_tables, normali
                          normalize_value_quantizer)
 
 _LEVEL_INDEX = {2: 0, 3: 1, 4: 2, 8: 3, 16: 4}
-_MAX_ITEMS_PER_SEGMENT = 1024        # ODMKV_MAX_ITEMS_PER_SEGMENT of include/odmkv.h
+
+
+def _exact_index_tables():
+    """[64, 128] element index of (slot, dim) inside an exact tile, for keys and for values
+    (the layouts of include/odmkv.h)."""
+    slot = np.arange(TILE)[:, None]
+    dim = np.arange(HEAD_DIM)[None, :]
+    k_idx = (((4 * (slot & 3) + ((dim >> 3) & 3)) * TILE) + 16 * (dim >> 5) + (slot >> 2)) * 8 + (dim & 7)
+    v_idx = (((8 * (slot >> 5) + (dim >> 4)) * TILE) + 16 * ((slot >> 3) & 3) + (dim & 15)) * 8 + (slot & 7)
+    return k_idx.astype(np.int64), v_idx.astype(np.int64)
+
+
+_EXACT_K_IDX, _EXACT_V_IDX = _exact_index_tables()
 _TILE_BYTES = [TILE * 16 * w + 2 * TILE * 4 for w in WIDTHS] + [2 * TILE * HEAD_DIM * 2]
 
 
@@ -464,10 +477,12 @@ class TurboQuantAdaptiveKVCacheState:
         if slots.size == 0:
             return None
         bh = np.concatenate(bh)
-        st = torch.from_numpy(slots).to(self.device)
-        nt = self._bufs["kexact"].numel() // (TILE * HEAD_DIM)
-        krows = self._bufs["kexact"].view(nt, 16, TILE, 8).permute(0, 2, 1, 3).reshape(nt * TILE, HEAD_DIM)[st]
-        vrows = self._bufs["vexact"].view(nt, 16, HEAD_DIM, 4).permute(0, 1, 3, 2).reshape(nt * TILE, HEAD_DIM)[st]
+        # element (slot, dim) of tile t sits at t * 8192 + index table[slot % 64, dim]
+        base = torch.from_numpy((slots // TILE) * (TILE * HEAD_DIM)).to(self.device)[:, None]
+        kidx = base + torch.from_numpy(_EXACT_K_IDX[slots % TILE]).to(self.device)
+        vidx = base + torch.from_numpy(_EXACT_V_IDX[slots % TILE]).to(self.device)
+        krows = self._bufs["kexact"].view(-1)[kidx]
+        vrows = self._bufs["vexact"].view(-1)[vidx]
         p3 = np.stack([bh // self.num_heads, bh % self.num_heads, pos_host[slots]], axis=-1).astype(np.int64)
         return torch.from_numpy(p3).to(self.device), krows, vrows
 
@@ -524,17 +539,10 @@ class TurboQuantAdaptiveKVCacheState:
         def n_pieces(per_item: int) -> int:
             return sum(-(-nt // step_of(per_item, li)) for _, li, nt in runs)
 
-        def most_per_segment(per_item: int) -> int:
-            per = np.zeros(self._nseg, np.int64)
-            for s, li, nt in runs:
-                per[s] += -(-nt // step_of(per_item, li))
-            return int(per.max()) if len(runs) else 0
-
         def fit(target: int) -> int:
-            # the coarsest cut with at most `target` items (a run's last piece may be short) and no
-            # segment above the merge kernel's limit
+            # the coarsest cut with at most `target` items (a run's last piece may be short)
             per_item = max(total // max(target, 1), min_item_bytes)
-            while (n_pieces(per_item) > target or most_per_segment(per_item) > _MAX_ITEMS_PER_SEGMENT) and per_item < total:
+            while n_pieces(per_item) > target and per_item < total:
                 per_item += max(per_item // 64, 1)
             return per_item
 

@@ -13,19 +13,23 @@ def _bits_to_codes(byte_rows: np.ndarray, w: int) -> np.ndarray:
     return (bits << np.arange(w, dtype=np.uint16)).sum(axis=-1).astype(np.uint8)
 
 
+def _lane_streams(buf: np.ndarray, nt: int, w: int) -> np.ndarray:
+    """Tile buffer -> [nt, 64 lanes, 128 codes]: chunk c of lane l sits at byte (c*64 + l)*16 of its tile."""
+    chunks = buf[: nt * TILE * 16 * w].reshape(nt, w, TILE, 16)
+    return _bits_to_codes(chunks.transpose(0, 2, 1, 3).reshape(nt, TILE, 16 * w), w)
+
+
 def decode_level(state, li: int):
     """-> dict(bh, pos, kcodes [N,128], vcodes [N,128], knorm, vnorm) over the stored tokens."""
     w = WIDTHS[li]
     b = state._bufs
     nt = int(state._seg_tile[li, -1])
-    kc = b["kcodes"][li].cpu().numpy()[: nt * TILE * 16 * w].reshape(nt, w, TILE, 16)
-    k_rows = kc.transpose(0, 2, 1, 3).reshape(nt, TILE, 16 * w)               # token-major streams
-    kcodes = _bits_to_codes(k_rows, w)                                        # [nt, 64, 128]
-    U = 8 if w == 3 else 16
-    nu = 8 * w // U
-    vc = b["vcodes"][li].cpu().numpy()[: nt * HD * 8 * w].reshape(nt, nu, HD, U)
-    v_rows = vc.transpose(0, 2, 1, 3).reshape(nt, HD, 8 * w)                  # dim-major streams
-    vcodes = _bits_to_codes(v_rows, w).transpose(0, 2, 1)                     # [nt, 64 tokens, 128 dims]
+    # keys: lane 16j+n, code 32b+i = dim 32j+i of slot 4n+b
+    ks = _lane_streams(b["kcodes"][li].cpu().numpy(), nt, w).reshape(nt, 4, 16, 4, 32)        # [t, j, n, b, i]
+    kcodes = ks.transpose(0, 2, 3, 1, 4).reshape(nt, TILE, HD)                                # [t, slot=4n+b, dim=32j+i]
+    # values: lane 16j+n, code 64k+8m+e = slot 32k+8j+e of dim 16m+n
+    vs = _lane_streams(b["vcodes"][li].cpu().numpy(), nt, w).reshape(nt, 4, 16, 2, 8, 8)      # [t, j, n, k, m, e]
+    vcodes = vs.transpose(0, 3, 1, 5, 4, 2).reshape(nt, TILE, HD)                             # [t, slot=32k+8j+e, dim=16m+n]
     kn = b["knorm"][li].cpu().numpy()[: nt * TILE].reshape(nt, TILE)
     vn = b["vnorm"][li].cpu().numpy()[: nt * TILE].reshape(nt, TILE)
     pos = b["pos"][li].cpu().numpy()[: nt * TILE].reshape(nt, TILE)
@@ -46,8 +50,10 @@ def decode_exact(state):
     nt = int(state._seg_tile[4, -1])
     ke = b["kexact"].view(-1).cpu().view(dtype=__import__("torch").int16).numpy()[: nt * TILE * HD]
     ve = b["vexact"].view(-1).cpu().view(dtype=__import__("torch").int16).numpy()[: nt * TILE * HD]
-    krows = ke.reshape(nt, 16, TILE, 8).transpose(0, 2, 1, 3).reshape(nt, TILE, HD)
-    vrows = ve.reshape(nt, 16, HD, 4).transpose(0, 1, 3, 2).reshape(nt, TILE, HD)
+    # keys: chunk 4b+k of lane 16j+n = dims 32j+8k..+7 of slot 4n+b
+    krows = ke.reshape(nt, 4, 4, 4, 16, 8).transpose(0, 4, 1, 3, 2, 5).reshape(nt, TILE, HD)  # [t,b,k,j,n,e] -> [t, n, b, j, k, e]
+    # values: chunk 8k+m of lane 16j+n = slots 32k+8j..+7 of dim 16m+n
+    vrows = ve.reshape(nt, 2, 8, 4, 16, 8).transpose(0, 1, 3, 5, 2, 4).reshape(nt, TILE, HD)  # [t,k,m,j,n,e] -> [t, k, j, e, m, n]
     pos = b["pos"][4].cpu().numpy()[: nt * TILE].reshape(nt, TILE)
     out = {k: [] for k in ("bh", "pos", "k", "v")}
     for s in range(state._nseg):

@@ -99,9 +99,9 @@ def test_decode_special_cases():
     assert rel_err(st.decode_attention(q.to(DEV)).cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
 
 
-def test_work_list_respects_the_per_segment_item_limit():
-    """One long (sequence, kv-head) cut into one-tile items would exceed the number of items the merge
-    kernel takes per segment; the work-list builder must cut coarser, and the result must not change."""
+def test_one_segment_cut_into_more_than_a_thousand_items():
+    """One long (sequence, kv-head) cut into one-tile items: the merge at the end of the main kernel walks
+    the items of a segment in chunks, so their number has no limit; the result must not change."""
     g = torch.Generator().manual_seed(5)
     T = 70000
     k = torch.randn(1, 1, T, 128, generator=g).half(); v = torch.randn(1, 1, T, 128, generator=g).half()
@@ -111,8 +111,7 @@ def test_work_list_respects_the_per_segment_item_limit():
     want = decode_attention_state(q, ref)
     st._build_items(1 << 20, 1)                       # as many, as small items as the builder will give
     items, ranges, n_items = st._items
-    per_segment = np.diff(ranges.cpu().numpy())
-    assert per_segment.max() <= 1024 and n_items >= 512
+    assert n_items > 1024
     assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
     st._build_items(8, 1 << 30)                       # and a handful of huge ones
     assert st._items[2] <= 8
