@@ -67,7 +67,7 @@ def load_bench_lib():
     lib.odmkv_bench_timer_create.argtypes = [i32, C.POINTER(vp)]
     lib.odmkv_bench_timer_collect.argtypes = [vp, C.POINTER(C.c_float), i32, C.POINTER(C.c_int)]
     lib.odmkv_bench_timer_destroy.argtypes = [vp]
-    lib.odmkv_bench_decode_attn.argtypes = [vp, i32, i32, i32, f32, C.POINTER(_lib.Packed), vp, i32, vp, vp, vp, vp, vp,
+    lib.odmkv_bench_decode_attn.argtypes = [vp, i32, i32, i32, f32, C.POINTER(_lib.Packed), C.POINTER(_lib.Worklist), vp, vp, vp,
                                             C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp, sz, vp, i32, vp]
     lib.odmkv_bench_probe_read.argtypes = [vp, sz, i32, vp, vp]
     lib.odmkv_decode_workspace_bytes.restype = sz
@@ -80,11 +80,10 @@ def bench_decode(blib, st, q, out, ws, stage_mask=7, timer=None):
     from kvquant import _lib
     if st._items is None:
         st._build_items()
-    items, ranges, n_items = st._items
     B, Hq, _ = q.shape
     rc = blib.odmkv_bench_decode_attn(
-        q.data_ptr(), _lib.dtype_code(q), B, Hq, 128 ** -0.5, C.byref(st._packed), items.data_ptr(), n_items,
-        ranges.data_ptr(), _lib.ptr(st._item_order), st._pi_k_t.data_ptr(), st.pi_v.data_ptr(), st._decode_cb.data_ptr(),
+        q.data_ptr(), _lib.dtype_code(q), B, Hq, 128 ** -0.5, C.byref(st._packed), C.byref(st._worklist),
+        st._pi_k_t.data_ptr(), st.pi_v.data_ptr(), st._decode_cb.data_ptr(),
         st._decode_cb_host, st._decode_inv, out.data_ptr(), _lib.dtype_code(out), None, ws.data_ptr(), ws.numel(),
         _lib.stream_ptr(q.device), stage_mask, timer)
     if rc != 0:

@@ -126,19 +126,19 @@ int odmkv_allocate(const float* scores, int rows, int n,
  * (kvquant/tq_backend.py:185-197, 103-125) as the quantiser.
  *
  * Tokens of one (sequence b, kv-head h) stored at one bit level form a segment; a segment is a
- * whole number of 64-token tiles, tokens in ascending position, the tail of the last tile
- * padded (pos = -1, norm = 0).  Level index li = 0..3 means 2, 3, 4, 8 bits; "exact" tokens
- * (16 bits) are fp16/bf16 rows.  Within a tile of width w:
- *   K codes, token-major:  the 16*w bytes of token l are w chunks of 16 bytes; chunk c of token
- *            l sits at byte (c*64 + l)*16 of the tile.  The token's code stream is little
- *            endian: code i occupies bits [i*w, i*w + w).
- *   V codes, dim-major:    the 8*w bytes of dim j hold the codes of the 64 tokens, token t at
- *            bits [t*w, t*w + w); they are split into units of U bytes (U = 16 for w = 2, 4, 8
- *            and U = 8 for w = 3), unit u of dim j at byte (u*128 + j)*U of the tile.
- *   norms fp32 [64], pos int32 [64] per tile.
- *   exact K, token-major:  chunk c (16 bytes = 8 elements) of token l at byte (c*64 + l)*16.
- *   exact V, dim-major in groups of 4 tokens: element (t, j) at 2-byte index
- *            ((t/4)*128 + j)*4 + t%4 of the tile.
+ * whole number of 64-token tiles, tokens in ascending position ("slot" s = 0..63 of a tile), the tail
+ * of the last tile padded (pos = -1, norm = 0).  Level index li = 0..3 means 2, 3, 4, 8 bits; "exact"
+ * tokens (16 bits) are fp16/bf16 rows.  The code and row buffers of a tile are laid out for the
+ * 16x16x32 matrix instructions of the decode kernel: every buffer is C chunks of 16 bytes per lane
+ * l = 0..63 (C = w for codes of width w, C = 16 for exact rows), chunk c of lane l at byte
+ * (c*64 + l)*16 of the tile, and with l = 16*j + n the lane's 16*C bytes hold
+ *   K codes:  128 codes as one little-endian bit stream (code i at bits [i*w, i*w + w));
+ *             code 32*b + i  is dim 32*j + i  of slot 4*n + b          (b = 0..3, i = 0..31)
+ *   V codes:  128 codes likewise; code 64*k + 8*m + e  is slot 32*k + 8*j + e  of dim 16*m + n
+ *                                                                        (k = 0..1, m = 0..7, e = 0..7)
+ *   exact K:  chunk 4*b + k  = the 8 elements  dims 32*j + 8*k .. + 7  of slot 4*n + b
+ *   exact V:  chunk 8*k + m  = the 8 elements  slots 32*k + 8*j .. + 7 of dim 16*m + n
+ *   norms fp32 [64], pos int32 [64] per tile, in slot order.
  */
 typedef struct odmkv_packed {
     int32_t B, Hkv;                      /* segments are indexed bh = b*Hkv + h */
@@ -219,15 +219,8 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  * over the stored (non-evicted) tokens.  Evicted tokens are simply absent.
  *
  * q: device [B, Hq, 128] of q_dtype (ODMKV_F16 / ODMKV_BF16 / ODMKV_F32), contiguous: the model's
- * query states are passed as they are.  items: device int32 [n_items, 8] work list, sorted by bh:
- * (bh, level index 0..4, first tile, tile count, tokens held by those tiles, first tile of the
- * segment, 0, 0); for the exact level (index 4) the token count is read from seg_count instead,
- * so that tokens appended since the list was built are seen.  item_range: device int32
- * [B*Hkv + 1] first item of each bh; a bh may have at most ODMKV_MAX_ITEMS_PER_SEGMENT items (the
- * caller builds the list and keeps to it; one item per compute unit is what performs best).
- * dispatch_order: device int32 [n_items], a permutation of the items in the order the workgroups
- * should take them (longest first, when there are more items than compute units), or NULL for the
- * list's own order.
+ * query states are passed as they are.  work: the work list (below), built by the caller once per
+ * change of the store.
  * out: device [B, Hq, 128] of out_dtype (accumulated in fp32, rounded once on the store);
  * lse: device fp32 [B, Hq] or NULL (log-sum-exp of the scaled logits).
  * pi_k_t is the key rotation TRANSPOSED (row-major [128,128] of Pi_k^T), pi_v the value rotation as is.
@@ -236,14 +229,29 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  * `codebooks` here holds the centroids of each width times a per-width scale chosen on the host
  * so that the scaled values are (nearly) exact in fp16, codebooks_host a host copy of the same 284
  * floats (the small tables travel as kernel arguments), and inv_scales (host, 4 floats) the
- * reciprocals of those scales.
+ * reciprocals of those scales.  Exact rows are multiplied in their own type (fp16, or bf16 with the
+ * query and the softmax weights split into two bf16 pieces each): nothing is narrowed.
+ *
+ * Work list.  items: device int32 [n_items, 8], sorted by bh: (bh, level index 0..4, first tile,
+ * tile count, tokens held by those tiles, first tile of the segment, 0, 0); for the exact level
+ * (index 4) the token count is read from seg_count instead, so that tokens appended since the list
+ * was built are seen.  item_range: device int32 [B*Hkv + 1] first item of each bh (any number of
+ * items per bh; one item per compute unit is what performs best; a bh without items gets zeros and
+ * lse = -inf).  One workgroup of the main kernel runs one item.
+ * dispatch_order: NULL (workgroup k takes item k), or device int32 [n_items], a permutation of the
+ * items in the order the workgroups should take them (longest first, when there are more items than
+ * compute units).
  */
-#define ODMKV_MAX_ITEMS_PER_SEGMENT 1024
+typedef struct odmkv_worklist {
+    const int32_t* items;            /* device [n_items, 8] */
+    const int32_t* item_range;       /* device [B*Hkv + 1] */
+    const int32_t* dispatch_order;   /* device [n_items] or NULL */
+    int32_t n_items;
+} odmkv_worklist_t;
+
 size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);
 int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
-                      const odmkv_packed_t* store,
-                      const int32_t* items, int n_items, const int32_t* item_range,
-                      const int32_t* dispatch_order,
+                      const odmkv_packed_t* store, const odmkv_worklist_t* work,
                       const float* pi_k_t, const float* pi_v, const float* codebooks,
                       const float* codebooks_host, const float* inv_scales,
                       void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
@@ -261,9 +269,7 @@ int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
  * odmkv_decode_attn. */
 #define ODMKV_STATIC_SCRATCH_BYTES (8u << 20)
 int odmkv_decode_attn_static(const void* q, int q_dtype, int B, int Hq, float scaling,
-                             const odmkv_packed_t* store,
-                             const int32_t* items, int n_items, const int32_t* item_range,
-                             const int32_t* dispatch_order,
+                             const odmkv_packed_t* store, const odmkv_worklist_t* work,
                              const float* pi_k_t, const float* pi_v, const float* codebooks,
                              const float* codebooks_host, const float* inv_scales,
                              void* out, int out_dtype, float* lse, void* stream);

@@ -26,9 +26,7 @@ int odmkv_bench_timer_destroy(void* timer);
  * alone over buffers a full call has filled (its output is then not written).  timer: NULL, or a
  * timer whose next event pair is attached to the main kernel. */
 int odmkv_bench_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
-                            const odmkv_packed_t* store,
-                            const int32_t* items, int n_items, const int32_t* item_range,
-                            const int32_t* dispatch_order,
+                            const odmkv_packed_t* store, const odmkv_worklist_t* work,
                             const float* pi_k_t, const float* pi_v, const float* codebooks,
                             const float* codebooks_host, const float* inv_scales,
                             void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,

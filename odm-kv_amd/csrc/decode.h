@@ -23,7 +23,6 @@ struct DecodeArgs {
     const float* cb;
     uint4* qrot;      // [B*Hq][2][128] fp16: high and low halves of Pi_k q16
     uint4* qs;        // [B*Hq][2][128] q16 itself for the exact tokens (fp16 + zeros, or bf16 high + low pieces)
-    unsigned int* tickets;   // [B*Hkv] items of the (sequence, kv-head) that have finished
     float inv_s[4];   // 1 / table scale per width
     float cbs[28];    // scaled centroids of widths 2, 3, 4 (kept in scalar registers; 8-bit ones stay in memory)
     int gp;           // head slots per item in `partial`: 4 or 8
@@ -32,12 +31,10 @@ struct DecodeArgs {
     float* lse;
 };
 
-// stage_mask: bit 0 the query preparation, bit 1 the main kernel, bit 2 the merge at its end (7 = the
+// stage_mask: bit 0 the query preparation, bit 1 the main kernel, bit 2 the merge (7 = the
 // product call).  ev_start / ev_stop: hipEvent_t attached to the main kernel's dispatch, or null.
 int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling,
-                        const odmkv_packed_t* store,
-                        const int32_t* items, int n_items, const int32_t* item_range,
-                        const int32_t* dispatch_order,
+                        const odmkv_packed_t* store, const odmkv_worklist_t* work,
                         const float* pi_k_t, const float* pi_v, const float* codebooks,
                         const float* codebooks_host, const float* inv_scales,
                         void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,

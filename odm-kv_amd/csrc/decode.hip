@@ -1,14 +1,16 @@
 // Fused LUT decode attention over the packed mixed-width KV store (one query token per sequence).
 //
-// Two launches per call:
+// Three launches per call:
 //   1. prep:  q16 = the query rounded to fp16 (what a model in fp16/bf16 hands over anyway);
 //             q' = Pi_k q16 in fp32, stored as fp16 high + low halves (queries in the rotated basis of
-//             the quantised keys); q16 itself for the exact tokens; the merge tickets are cleared.
+//             the quantised keys); q16 itself for the exact tokens.
 //   2. main:  one workgroup per work item = a run of 64-token tiles of one (sequence, kv-head,
-//             level).  The packed bytes are read once from HBM; nothing else is.  The workgroup that
-//             finishes last among the items of a (sequence, kv-head) merges their partial results by
-//             log-sum-exp, rotates the quantised part back to the model basis (acc . Pi_v), adds the
-//             exact part, normalises and writes the output.
+//             level).  The packed bytes are read once from HBM; nothing else is.
+//   3. merge: log-sum-exp merge of a kv-head's items per query head, rotation of the quantised
+//             part back to the model basis (acc . Pi_v), addition of the exact part, normalise.
+// (Merging inside the main kernel, by the workgroup that finishes last among a kv-head's items, was built
+// and measured: the count and the other workgroups' results have to cross the device at agent scope, two
+// to three dependent trips to memory of 2-3 us each under the streaming load, against one launch of 4 us.)
 //
 // Main kernel, per wavefront and tile, on v_mfma_f32_16x16x32_f16 (D[16x16] += A[16x32] B[32x16];
 // lane l supplies A[l%16][8(l/16)+e] and B[8(l/16)+e][l%16], e = 0..7, and holds D[4(l/16)+r][l%16]):
@@ -39,19 +41,16 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 #define PROW 144            // bytes per head row of a wave's p buffer: 64 x 16 bit + 16 of padding (bank spread)
 #define PBUF (16 * PROW)    // one p buffer (8 head rows used)
 #define QROW 256            // bytes of one query row (128 x 16 bit)
-#define MERGE_CHUNK 256     // items whose weights are held in LDS at a time by the merge
 
-// dynamic LDS of the main kernel: [table | combine area | Pi_v of the merge] [p buffers | merge scratch] [per-wave scalars]
+// LDS of the main kernel: [table | combine area | Pi_v of the merge] [p buffers | merge scratch] [per-wave scalars]
 #define LDS_PBUFS LUT_BYTES
 #define LDS_SCALARS (LDS_PBUFS + DECODE_NWAVES * 2 * PBUF)
 #define LDS_TOTAL (LDS_SCALARS + DECODE_NWAVES * 3 * 8 * 4)
 static_assert(DECODE_NWAVES * ODMKV_MAX_GROUP * HD * 4 <= LUT_BYTES, "combine area must fit the table's space");
-static_assert((MERGE_CHUNK * ODMKV_MAX_GROUP + 3 * ODMKV_MAX_GROUP + ODMKV_MAX_GROUP * HD) * 4 <= DECODE_NWAVES * 2 * PBUF,
-              "merge scratch must fit the p buffers' space");
-static_assert(DECODE_NWAVES >= ODMKV_MAX_GROUP && (256 / DECODE_NWAVES) % 4 == 0, "wave count");
+static_assert((256 / DECODE_NWAVES) % 4 == 0, "wave count");
 
 // ------------------------------------------------------------------------------------------------
-// prep: rotate the queries, clear the tickets
+// prep: rotate the queries
 // ------------------------------------------------------------------------------------------------
 __device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
 
@@ -72,17 +71,6 @@ __global__ __launch_bounds__(PREP_THREADS) void decode_prep_kernel(DecodeArgs a)
     float pk[JN];
 #pragma unroll
     for (int jj = 0; jj < JN; ++jj) pk[jj] = a.pi_k_t[(size_t)(js * JN + jj) * HD + i];
-    if (blockIdx.x == 0)                     // every (sequence, kv-head) starts the call with no finished item
-        for (int t = tid; t < a.B * a.s.Hkv; t += PREP_THREADS) a.tickets[t] = 0u;
-    if (quarter == 0 && tid < HD) {          // a (sequence, kv-head) that stores nothing has no workgroup to write its rows
-        const int bh = (bq / a.Hq) * a.s.Hkv + (bq % a.Hq) / a.G;
-        if (a.item_range[bh + 1] == a.item_range[bh]) {
-            const size_t oi = (size_t)bq * HD + tid;
-            if (a.out_dt == ODMKV_F32) reinterpret_cast<float*>(a.out)[oi] = 0.0f;
-            else reinterpret_cast<uint16_t*>(a.out)[oi] = 0;
-            if (a.lse && tid == 0) a.lse[bq] = -INFINITY;
-        }
-    }
     if (tid < HD) {
         // the query is consumed at fp16 precision, like the attention it replaces (model dtype)
         const size_t qi = (size_t)bq * HD + tid;
@@ -157,6 +145,24 @@ __device__ static inline float row_max(float v) {
     v = fmaxf(v, dpp<DPP_ROR(2)>(v));
     v = fmaxf(v, dpp<DPP_ROR(1)>(v));
     return v;
+}
+// the same for two values at once, as fused DPP instructions (the two chains fill each other's wait states)
+__device__ static inline void row_max2(float& a, float& b) {
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_max_f32_dpp %1, %1, %1 row_ror:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(a), "+v"(b));
 }
 __device__ static inline float row_sum(float v) {
     v += dpp<DPP_ROR(8)>(v);
@@ -301,10 +307,13 @@ __device__ static inline uint32_t pack_h2(float a, float b) {
 __device__ static inline void softmax_tile(WaveState& st, const float* tA, const float* tB, int lane,
                                            float* alpha_sh, float* pA, float* pB) {
     const int n = lane & 15, j = lane >> 4;
-    const float mxA = row_max(fmaxf(fmaxf(tA[0], tA[1]), fmaxf(tA[2], tA[3])));
-    const float mxB = row_max(fmaxf(fmaxf(tB[0], tB[1]), fmaxf(tB[2], tB[3])));
-    const float mnA = fmaxf(st.mA, mxA), mnB = fmaxf(st.mB, mxB);
-    if (__builtin_amdgcn_ballot_w64(mnA != st.mA || mnB != st.mB) != 0) {       // wave-uniform: some maximum moved
+    float mxA = fmaxf(fmaxf(tA[0], tA[1]), fmaxf(tA[2], tA[3]));
+    float mxB = fmaxf(fmaxf(tB[0], tB[1]), fmaxf(tB[2], tB[3]));
+    // the running maxima move only when some lane sees a larger logit (wave-uniform test): no cross-lane
+    // reduction otherwise
+    if (__builtin_amdgcn_ballot_w64(mxA > st.mA || mxB > st.mB) != 0) {
+        row_max2(mxA, mxB);
+        const float mnA = fmaxf(st.mA, mxA), mnB = fmaxf(st.mB, mxB);
         const float aA = __builtin_amdgcn_exp2f(st.mA - mnA), aB = __builtin_amdgcn_exp2f(st.mB - mnB);   // first tile: exp2(-inf) = 0
         st.lA *= aA; st.lB *= aB;
         st.mA = mnA; st.mB = mnB;
@@ -314,6 +323,7 @@ __device__ static inline void softmax_tile(WaveState& st, const float* tA, const
 #pragma unroll
         for (int nb = 0; nb < 8; ++nb) st.acc[nb] *= al;
     }
+    const float mnA = st.mA, mnB = st.mB;
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
         pA[b] = __builtin_amdgcn_exp2f(tA[b] - mnA);      // padded slots: -inf -> 0
@@ -549,148 +559,17 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
 }
 
 // ------------------------------------------------------------------------------------------------
-// merge of a (sequence, kv-head): log-sum-exp over its items' partial results, quantised part rotated
-// back, exact part added.  Run by the workgroup that finished last; the partial results were written
-// through to memory (agent-scope stores) and are read past the caches (agent-scope loads).
-// ------------------------------------------------------------------------------------------------
-__device__ static inline float ld_agent(const float* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ static inline void st_agent(float* p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-template <int GP>
-__device__ static inline void merge_segment(const DecodeArgs& a, int bh, int tid, uint8_t* smem) {
-    constexpr int NT = DECODE_NWAVES * 64;
-    constexpr int HP = NT / HD;                    // heads handled per pass
-    constexpr int NP = (GP + HP - 1) / HP;         // passes
-    constexpr int PER_LANE = MERGE_CHUNK / 64;
-    float* pis = reinterpret_cast<float*>(smem);                       // Pi_v [HD][HD] (64 KB, the table's space)
-    float* wts = reinterpret_cast<float*>(smem + LDS_PBUFS);           // [MERGE_CHUNK][GP] weight; the sign bit marks exact items
-    float* red = wts + MERGE_CHUNK * GP;                               // [GP][3]: running maximum, running sum, rescale of this chunk
-    float* rot = red + 3 * GP;                                         // [GP][HD] merged quantised part
-    const int wave = tid >> 6, lane = tid & 63;
-    const int i0 = a.item_range[bh], n = a.item_range[bh + 1] - i0;
-    const int b = bh / a.s.Hkv, hkv = bh % a.s.Hkv;
-    // Pi_v -> LDS, requested first: it depends on nothing
-    {
-        constexpr int NV = HD * HD / 4 / NT;
-        const float4* __restrict__ src = reinterpret_cast<const float4*>(a.pi_v);
-        float4 tmp[NV];
-#pragma unroll
-        for (int k = 0; k < NV; ++k) tmp[k] = src[k * NT + tid];
-#pragma unroll
-        for (int k = 0; k < NV; ++k) reinterpret_cast<float4*>(pis)[k * NT + tid] = tmp[k];
-    }
-    if (tid < GP) { red[3 * tid] = -INFINITY; red[3 * tid + 1] = 0.0f; red[3 * tid + 2] = 0.0f; }
-    float arot[NP], aex[NP];
-#pragma unroll
-    for (int p = 0; p < NP; ++p) { arot[p] = 0.0f; aex[p] = 0.0f; }
-    __syncthreads();
-    for (int c0 = 0; c0 < n; c0 += MERGE_CHUNK) {
-        const int nc = min(n - c0, MERGE_CHUNK);
-        // wavefront g weighs head g: new running maximum, weights of the chunk's items against it, running sum
-        if (wave < GP) {
-            const int g = wave;
-            const float Mold = red[3 * g], Lold = red[3 * g + 1];
-            float m[PER_LANE], l[PER_LANE];
-            float mx = -INFINITY;
-#pragma unroll
-            for (int k = 0; k < PER_LANE; ++k) {
-                const int it = lane + 64 * k;
-                m[k] = -INFINITY; l[k] = 0.0f;
-                if (it < nc) {
-                    const float* p = a.partial + ((size_t)(i0 + c0 + it) * GP + g) * PSTRIDE + HD;
-                    m[k] = ld_agent(p); l[k] = ld_agent(p + 1);
-                }
-                mx = fmaxf(mx, m[k]);
-            }
-            const float M = fmaxf(Mold, wave_max(mx));
-            float sum = 0.0f;
-#pragma unroll
-            for (int k = 0; k < PER_LANE; ++k) {
-                const int it = lane + 64 * k;
-                if (it < nc) {
-                    const float f = M > -INFINITY ? __builtin_amdgcn_exp2f(m[k] - M) : 0.0f;
-                    wts[it * GP + g] = a.items[8 * (i0 + c0 + it) + 1] == 4 ? -f : f;
-                    sum = __fmaf_rn(l[k], f, sum);
-                }
-            }
-            sum = wave_sum(sum);
-            if (lane == 0) {
-                const float sc = Mold > -INFINITY ? __builtin_amdgcn_exp2f(Mold - M) : 0.0f;
-                red[3 * g] = M; red[3 * g + 1] = __fmaf_rn(Lold, sc, sum); red[3 * g + 2] = sc;
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            const int g = p * HP + tid / HD, dim = tid % HD;
-            if (g < GP) {
-                const float sc = red[3 * g + 2];
-                float r = arot[p] * sc, x = aex[p] * sc;
-                const float* src = a.partial + ((size_t)(i0 + c0) * GP + g) * PSTRIDE + dim;
-                int it = 0;
-                for (; it + 8 <= nc; it += 8) {
-                    float v[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) v[u] = ld_agent(src + (size_t)(it + u) * GP * PSTRIDE);
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) {
-                        const float w = wts[(it + u) * GP + g];
-                        if (__float_as_uint(w) >> 31) x = __fmaf_rn(v[u], -w, x);
-                        else r = __fmaf_rn(v[u], w, r);
-                    }
-                }
-                for (; it < nc; ++it) {
-                    const float v = ld_agent(src + (size_t)it * GP * PSTRIDE);
-                    const float w = wts[it * GP + g];
-                    if (__float_as_uint(w) >> 31) x = __fmaf_rn(v, -w, x);
-                    else r = __fmaf_rn(v, w, r);
-                }
-                arot[p] = r; aex[p] = x;
-            }
-        }
-        __syncthreads();                               // the weights are overwritten by the next chunk
-    }
-    // rotate back and write
-#pragma unroll
-    for (int p = 0; p < NP; ++p) {
-        const int g = p * HP + tid / HD;
-        if (g < GP) rot[g * HD + tid % HD] = arot[p];
-    }
-    __syncthreads();
-#pragma unroll
-    for (int p = 0; p < NP; ++p) {
-        const int g = p * HP + tid / HD, dim = tid % HD;
-        if (g < a.G) {
-            float o = 0.0f;
-#pragma unroll 16
-            for (int i = 0; i < HD; ++i) o = __fmaf_rn(rot[g * HD + i], pis[i * HD + dim], o);
-            const float M = red[3 * g], L = red[3 * g + 1];
-            const float o32 = L > 0.0f ? (o + aex[p]) / L : 0.0f;
-            const int bq = b * a.Hq + hkv * a.G + g;
-            const size_t oi = (size_t)bq * HD + dim;
-            if (a.out_dt == ODMKV_F32) reinterpret_cast<float*>(a.out)[oi] = o32;
-            else if (a.out_dt == ODMKV_F16) reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_F16>::from_f32(o32);
-            else reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_BF16>::from_f32(o32);
-            if (a.lse && dim == 0) a.lse[bq] = L > 0.0f ? (M + __log2f(L)) * LN2 : -INFINITY;
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
 // main kernel
 // ------------------------------------------------------------------------------------------------
 template <int GP, bool ORDERED>
-__global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeArgs a, int stage_mask) {
-    extern __shared__ __align__(16) uint8_t smem[];
-    uint8_t* lut = smem;                                               // centroid table; reused to combine the wavefronts and to merge
+__global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeArgs a) {
+    // one static LDS block: the table sits at LDS address 0 and that is known when the kernel is compiled, so a
+    // lookup address needs no base added
+    __shared__ __align__(16) uint8_t smem[LDS_TOTAL];
+    uint8_t* lut = smem;                                               // centroid table; reused to combine the wavefronts
     float* alphas = reinterpret_cast<float*>(smem + LDS_SCALARS);      // [NWAVES][8]
     float* wm = alphas + DECODE_NWAVES * 8;                            // [NWAVES][8]
     float* wl = wm + DECODE_NWAVES * 8;                                // [NWAVES][8]
-    __shared__ int last_flag;
 
     const int item = ORDERED ? a.order[blockIdx.x] : (int)blockIdx.x;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -718,7 +597,7 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
 
     // ---- combine the wavefronts (the table is no longer needed) ----
     __syncthreads();
-    float* wacc = reinterpret_cast<float*>(lut);          // [NWAVES][GP][128]
+    float* wacc = reinterpret_cast<float*>(lut);          // [NWAVES][128 dims][GP heads]
     {
         const int n = lane & 15, j = lane >> 4;
         const float lsA = row_sum(st.lA), lsB = row_sum(st.lB);
@@ -728,9 +607,7 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
         }
         if (4 * j < GP) {
 #pragma unroll
-            for (int nb = 0; nb < 8; ++nb)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) wacc[(wave * GP + 4 * j + r) * HD + 16 * nb + n] = st.acc[nb][r];
+            for (int nb = 0; nb < 8; ++nb) *reinterpret_cast<f4*>(&wacc[((wave * HD) + 16 * nb + n) * GP + 4 * j]) = st.acc[nb];
         }
     }
     __syncthreads();
@@ -745,26 +622,152 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
 #pragma unroll
             for (int w = 0; w < DECODE_NWAVES; ++w) {
                 const float f = __builtin_amdgcn_exp2f(wm[w * 8 + g] - M);
-                s = __fmaf_rn(wacc[(w * GP + g) * HD + dim], f, s);
+                s = __fmaf_rn(wacc[(w * HD + dim) * GP + g], f, s);
                 L = __fmaf_rn(wl[w * 8 + g], f, L);
             }
         }
-        st_agent(dst + g * PSTRIDE + dim, s);
-        if (dim == 0) { st_agent(dst + g * PSTRIDE + HD, M); st_agent(dst + g * PSTRIDE + HD + 1, L); }
+        dst[g * PSTRIDE + dim] = s;
+        if (dim == 0) { dst[g * PSTRIDE + HD] = M; dst[g * PSTRIDE + HD + 1] = L; }
     }
-    if (!(stage_mask & 4)) return;                         // measurement: the streaming part alone
-    // ---- the last workgroup of this (sequence, kv-head) merges ----
-    __builtin_amdgcn_s_waitcnt(0);                         // the stores have reached the memory side
+}
+
+// ------------------------------------------------------------------------------------------------
+// merge: MERGE_SPLIT workgroups per query head
+// ------------------------------------------------------------------------------------------------
+#define MERGE_THREADS 512
+#define MERGE_SLICES (MERGE_THREADS / HD)
+#ifndef MERGE_SPLIT
+#define MERGE_SPLIT 4
+#endif
+#define MERGE_CHUNK 1024          // items whose weights are held in LDS at a time
+
+template <int GP>
+__global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs a) {
+    __shared__ float wts[MERGE_CHUNK];               // exp2(m_item - M); the sign bit marks exact items
+    __shared__ float red[MERGE_THREADS / 64];
+    __shared__ float part[2][MERGE_SLICES][HD];      // [rotated | exact][slice][dim]
+    __shared__ float rot[HD];
+    __shared__ float Lsh;
+    // MERGE_SPLIT workgroups per query head: each merges the head's partial results in full (they are small and
+    // shared through the caches) and rotates back a quarter of the output dims, so that no workgroup has to pull
+    // the whole 64 KB rotation through one compute unit
+    const int bq = blockIdx.x / MERGE_SPLIT, quarter = blockIdx.x % MERGE_SPLIT;
+    const int tid = threadIdx.x, j = tid & (HD - 1), slice = tid >> 7;
+    const int b = bq / a.Hq, hq = bq % a.Hq;
+    const int bh = b * a.s.Hkv + hq / a.G, g = hq % a.G;
+    const int i0 = a.item_range[bh], n = a.item_range[bh + 1] - i0;
+    // Everything that does not depend on the weights is requested now, in one round trip: this thread's
+    // share of the value rotation, the first MERGE_PRE accumulator values of its slice, its item's (m, l, level)
+    constexpr int QD = HD / MERGE_SPLIT;                 // output dims of this workgroup
+    constexpr int RS = MERGE_THREADS / QD;                // row slices of the rotation
+    constexpr int IN = HD / RS;                           // rows per slice
+    const int jj = tid % QD, rs = tid / QD;
+    float pv[IN];
+#pragma unroll
+    for (int ii = 0; ii < IN; ++ii) pv[ii] = a.pi_v[(size_t)(rs * IN + ii) * HD + quarter * QD + jj];
+    constexpr int MERGE_PRE = 16;
+    float pre[MERGE_PRE];
+#pragma unroll
+    for (int k = 0; k < MERGE_PRE; ++k) {
+        const int it = slice + k * MERGE_SLICES;
+        pre[k] = it < n ? a.partial[((size_t)(i0 + it) * GP + g) * PSTRIDE + j] : 0.0f;
+    }
+    float my_m = -INFINITY, my_l = 0.0f;
+    int my_level = 0;
+    if (tid < n) {
+        const float* p = a.partial + ((size_t)(i0 + tid) * GP + g) * PSTRIDE;
+        my_m = p[HD]; my_l = p[HD + 1];
+        my_level = a.items[8 * (i0 + tid) + 1];
+    }
+    // maximum over all the items
+    float mx = my_m;
+    for (int it = tid + MERGE_THREADS; it < n; it += MERGE_THREADS)
+        mx = fmaxf(mx, a.partial[((size_t)(i0 + it) * GP + g) * PSTRIDE + HD]);
+    mx = wave_max(mx);
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    float M = red[0];
+#pragma unroll
+    for (int w = 1; w < MERGE_THREADS / 64; ++w) M = fmaxf(M, red[w]);
+    __syncthreads();
+    // weights, the normaliser and the weighted sums, MERGE_CHUNK items at a time (one round for the usual work list)
+    float lpart = 0.0f, arot = 0.0f, aex = 0.0f;
+    for (int c0 = 0; c0 < n; c0 += MERGE_CHUNK) {
+        const int nc = min(n - c0, MERGE_CHUNK);
+        if (c0 == 0 && tid < nc) {
+            const float f = M > -INFINITY ? __builtin_amdgcn_exp2f(my_m - M) : 0.0f;
+            lpart = my_l * f;
+            wts[tid] = my_level == 4 ? -f : f;
+        }
+        for (int it = tid + (c0 == 0 ? MERGE_THREADS : 0); it < nc; it += MERGE_THREADS) {
+            const float* p = a.partial + ((size_t)(i0 + c0 + it) * GP + g) * PSTRIDE;
+            const float f = M > -INFINITY ? __builtin_amdgcn_exp2f(p[HD] - M) : 0.0f;
+            lpart = __fmaf_rn(p[HD + 1], f, lpart);
+            wts[it] = a.items[8 * (i0 + c0 + it) + 1] == 4 ? -f : f;
+        }
+        __syncthreads();                                   // weights written
+        int first = slice;
+        if (c0 == 0) {
+#pragma unroll
+            for (int k = 0; k < MERGE_PRE; ++k) {
+                const int it = slice + k * MERGE_SLICES;
+                if (it < nc) {
+                    const float w = wts[it];
+                    if (__float_as_uint(w) >> 31) aex = __fmaf_rn(pre[k], -w, aex);
+                    else arot = __fmaf_rn(pre[k], w, arot);
+                }
+            }
+            first = slice + MERGE_PRE * MERGE_SLICES;
+        }
+#pragma unroll 4
+        for (int it = first; it < nc; it += MERGE_SLICES) {
+            const float w = wts[it];
+            const float v = a.partial[((size_t)(i0 + c0 + it) * GP + g) * PSTRIDE + j];
+            if (__float_as_uint(w) >> 31) aex = __fmaf_rn(v, -w, aex);
+            else arot = __fmaf_rn(v, w, arot);
+        }
+        __syncthreads();                                   // the weights are overwritten by the next round
+    }
+    lpart = wave_sum(lpart);
+    if ((tid & 63) == 0) red[tid >> 6] = lpart;
+    part[0][slice][j] = arot;
+    part[1][slice][j] = aex;
     __syncthreads();
     if (tid == 0) {
-        const unsigned int need = (unsigned int)(a.item_range[bh + 1] - a.item_range[bh]);
-        const unsigned int t = __hip_atomic_fetch_add(&a.tickets[bh], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        last_flag = (t == need - 1u);
-        if (last_flag) __hip_atomic_store(&a.tickets[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        float L = 0.0f;
+        for (int w = 0; w < MERGE_THREADS / 64; ++w) L += red[w];
+        Lsh = L;
+    }
+    if (tid < HD) {
+        float r = 0.0f;
+#pragma unroll
+        for (int s = 0; s < MERGE_SLICES; ++s) r += part[0][s][tid];
+        rot[tid] = r;
     }
     __syncthreads();
-    if (!last_flag) return;
-    merge_segment<GP>(a, bh, tid, smem);
+    // rotate the quantised part back: out_j = sum_i rot_i Pi_v[i][j] for this workgroup's dims; the slices split the i range
+    float o = 0.0f;
+#pragma unroll
+    for (int ii = 0; ii < IN; ++ii) o = __fmaf_rn(rot[rs * IN + ii], pv[ii], o);
+    __syncthreads();
+    float* part2 = &part[0][0][0];                        // [RS][QD], the first half of `part` is free again
+    part2[rs * QD + jj] = o;
+    __syncthreads();
+    if (tid < QD) {
+        const int dim = quarter * QD + tid;
+        float tot = 0.0f;
+#pragma unroll
+        for (int r = 0; r < RS; ++r) tot += part2[r * QD + tid];
+#pragma unroll
+        for (int s = 0; s < MERGE_SLICES; ++s) tot += part[1][s][dim];
+        const float L = Lsh;
+        const float o32 = L > 0.0f ? tot / L : 0.0f;
+        const size_t oi = (size_t)bq * HD + dim;
+        if (a.out_dt == ODMKV_F32) reinterpret_cast<float*>(a.out)[oi] = o32;
+        else if (a.out_dt == ODMKV_F16) reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_F16>::from_f32(o32);
+        else reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_BF16>::from_f32(o32);
+        if (a.lse && tid == 0 && quarter == 0) a.lse[bq] = L > 0.0f ? (M + __log2f(L)) * LN2 : -INFINITY;
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -775,28 +778,18 @@ static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
 extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     if (B <= 0 || Hq <= 0 || n_items < 0) return 0;
     const size_t q = align_up((size_t)B * Hq * 2 * QROW, 256);
-    return 2 * q + align_up((size_t)B * Hq * sizeof(unsigned int), 256) +
-           align_up((size_t)n_items * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
+    return 2 * q + align_up((size_t)n_items * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
 }
 
 template <int GP, bool ORDERED>
-static int launch_main(const DecodeArgs& a, int n_items, int stage_mask, hipEvent_t e0, hipEvent_t e1, hipStream_t st) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&decode_main_kernel<GP, ORDERED>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL));
-        attr_set = true;
-    }
-    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED>), dim3(n_items), dim3(DECODE_NWAVES * 64), LDS_TOTAL, st, e0, e1, 0,
-                          a, stage_mask);
+static int launch_main(const DecodeArgs& a, int grid, hipEvent_t e0, hipEvent_t e1, hipStream_t st) {
+    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED>), dim3(grid), dim3(DECODE_NWAVES * 64), 0, st, e0, e1, 0, a);
     ODMKV_CHECK_LAUNCH("decode_main_kernel");
     return 0;
 }
 
 int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling,
-                        const odmkv_packed_t* store,
-                        const int32_t* items, int n_items, const int32_t* item_range,
-                        const int32_t* dispatch_order,
+                        const odmkv_packed_t* store, const odmkv_worklist_t* work,
                         const float* pi_k_t, const float* pi_v, const float* codebooks,
                         const float* codebooks_host, const float* inv_scales,
                         void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
@@ -805,14 +798,16 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     ODMKV_CHECK_ARG(out_dtype == ODMKV_F16 || out_dtype == ODMKV_BF16 || out_dtype == ODMKV_F32, "decode_attn: bad output dtype %d", out_dtype);
     ODMKV_CHECK_ARG(codebooks_host != nullptr, "decode_attn: null host copy of the centroid tables");
     ODMKV_CHECK_ARG(inv_scales != nullptr, "decode_attn: null table scales");
-    ODMKV_CHECK_ARG(q && store && item_range && pi_k_t && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
-    ODMKV_CHECK_ARG(n_items == 0 || items, "decode_attn: null work list");
+    ODMKV_CHECK_ARG(q && store && work && pi_k_t && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
+    const int n_items = work->n_items;
+    ODMKV_CHECK_ARG(n_items >= 0, "decode_attn: negative item count");
+    ODMKV_CHECK_ARG(work->item_range, "decode_attn: null item ranges");
+    ODMKV_CHECK_ARG(n_items == 0 || work->items, "decode_attn: null work list");
     ODMKV_CHECK_ARG(B > 0 && Hq > 0 && store->B == B && store->Hkv > 0 && Hq % store->Hkv == 0,
                     "decode_attn: bad head counts B=%d Hq=%d store(B=%d,Hkv=%d)", B, Hq, store->B, store->Hkv);
     ODMKV_CHECK_ARG(store->exact_dtype == ODMKV_F16 || store->exact_dtype == ODMKV_BF16, "decode_attn: exact dtype must be fp16 or bf16");
     const int G = Hq / store->Hkv;
     ODMKV_CHECK_ARG(G <= ODMKV_MAX_GROUP, "decode_attn: GQA group %d exceeds %d", G, ODMKV_MAX_GROUP);
-    ODMKV_CHECK_ARG(n_items >= 0, "decode_attn: negative item count");
     if (workspace_bytes < odmkv_decode_workspace_bytes(B, Hq, n_items)) {
         odmkv_set_error("decode_attn: workspace of %zu bytes, %zu needed", workspace_bytes, odmkv_decode_workspace_bytes(B, Hq, n_items));
         return ODMKV_ENOSPACE;
@@ -820,15 +815,14 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     hipStream_t st = (hipStream_t)stream;
     DecodeArgs a;
     a.s = *store; a.q = q; a.q_dt = q_dtype; a.out_dt = out_dtype; a.Hq = Hq; a.G = G; a.B = B; a.scaling = scaling;
-    a.items = items; a.item_range = item_range; a.order = dispatch_order;
+    a.items = work->items; a.item_range = work->item_range; a.order = work->dispatch_order;
     a.pi_k_t = pi_k_t; a.pi_v = pi_v; a.cb = codebooks;
     for (int w = 0; w < 4; ++w) a.inv_s[w] = inv_scales[w];
     for (int k = 0; k < 28; ++k) a.cbs[k] = codebooks_host[k];
     const size_t qbytes = align_up((size_t)B * Hq * 2 * QROW, 256);
     a.qrot = (uint4*)workspace;
     a.qs = (uint4*)((char*)workspace + qbytes);
-    a.tickets = (unsigned int*)((char*)workspace + 2 * qbytes);
-    a.partial = (float*)((char*)workspace + 2 * qbytes + align_up((size_t)B * Hq * sizeof(unsigned int), 256));
+    a.partial = (float*)((char*)workspace + 2 * qbytes);
     a.out = out; a.lse = lse;
     if (stage_mask & 1) {
         hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq * PREP_SPLIT), dim3(PREP_THREADS), 0, st, a);
@@ -841,31 +835,33 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
         // start and end timestamps, not those of separate marker packets
         hipEvent_t e0 = (hipEvent_t)ev_start, e1 = (hipEvent_t)ev_stop;
         int rc;
-        if (GP == 4 && !a.order) rc = launch_main<4, false>(a, n_items, stage_mask, e0, e1, st);
-        else if (GP == 4) rc = launch_main<4, true>(a, n_items, stage_mask, e0, e1, st);
-        else if (!a.order) rc = launch_main<8, false>(a, n_items, stage_mask, e0, e1, st);
-        else rc = launch_main<8, true>(a, n_items, stage_mask, e0, e1, st);
+        if (GP == 4 && !a.order) rc = launch_main<4, false>(a, n_items, e0, e1, st);
+        else if (GP == 4) rc = launch_main<4, true>(a, n_items, e0, e1, st);
+        else if (!a.order) rc = launch_main<8, false>(a, n_items, e0, e1, st);
+        else rc = launch_main<8, true>(a, n_items, e0, e1, st);
         if (rc) return rc;
+    }
+    if (stage_mask & 4) {
+        if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq * MERGE_SPLIT), dim3(MERGE_THREADS), 0, st, a);
+        else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq * MERGE_SPLIT), dim3(MERGE_THREADS), 0, st, a);
+        ODMKV_CHECK_LAUNCH("decode_merge_kernel");
     }
     return 0;
 }
 
 extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
-                                 const odmkv_packed_t* store,
-                                 const int32_t* items, int n_items, const int32_t* item_range,
-                                 const int32_t* dispatch_order,
+                                 const odmkv_packed_t* store, const odmkv_worklist_t* work,
                                  const float* pi_k_t, const float* pi_v, const float* codebooks,
                                  const float* codebooks_host, const float* inv_scales,
                                  void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                                  void* stream) {
-    return odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, items, n_items, item_range, dispatch_order, pi_k_t, pi_v,
-                               codebooks, codebooks_host, inv_scales, out, out_dtype, lse, workspace, workspace_bytes, stream,
-                               7, nullptr, nullptr);
+    return odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, work, pi_k_t, pi_v, codebooks, codebooks_host, inv_scales,
+                               out, out_dtype, lse, workspace, workspace_bytes, stream, 7, nullptr, nullptr);
 }
 
 // ------------------------------------------------------------------------------------------------
 // The same call for callers that cannot allocate and have no workspace to hand over: the prepared
-// queries, the tickets and the partial results live in a fixed array of the library's own device image.
+// queries and the partial results live in a fixed array of the library's own device image.
 // ------------------------------------------------------------------------------------------------
 static __device__ __align__(256) unsigned char scratch[ODMKV_STATIC_SCRATCH_BYTES];
 
@@ -890,22 +886,20 @@ static int static_scratch(void** ptr) {
 }
 
 extern "C" int odmkv_decode_attn_static(const void* q, int q_dtype, int B, int Hq, float scaling,
-                                        const odmkv_packed_t* store,
-                                        const int32_t* items, int n_items, const int32_t* item_range,
-                                        const int32_t* dispatch_order,
+                                        const odmkv_packed_t* store, const odmkv_worklist_t* work,
                                         const float* pi_k_t, const float* pi_v, const float* codebooks,
                                         const float* codebooks_host, const float* inv_scales,
                                         void* out, int out_dtype, float* lse, void* stream) {
-    ODMKV_CHECK_ARG(B > 0 && Hq > 0 && n_items >= 0, "decode_attn_static: bad shape B=%d Hq=%d items=%d", B, Hq, n_items);
-    const size_t need = odmkv_decode_workspace_bytes(B, Hq, n_items);
+    ODMKV_CHECK_ARG(work != nullptr, "decode_attn_static: null work list");
+    ODMKV_CHECK_ARG(B > 0 && Hq > 0 && work->n_items >= 0, "decode_attn_static: bad shape B=%d Hq=%d items=%d", B, Hq, work->n_items);
+    const size_t need = odmkv_decode_workspace_bytes(B, Hq, work->n_items);
     if (need > (size_t)ODMKV_STATIC_SCRATCH_BYTES) {
         odmkv_set_error("decode_attn_static: B=%d Hq=%d items=%d need %zu bytes of scratch, the fixed array holds %zu; "
-                        "use odmkv_decode_attn with a workspace", B, Hq, n_items, need, (size_t)ODMKV_STATIC_SCRATCH_BYTES);
+                        "use odmkv_decode_attn with a workspace", B, Hq, work->n_items, need, (size_t)ODMKV_STATIC_SCRATCH_BYTES);
         return ODMKV_ENOSPACE;
     }
     void* ws = nullptr;
     if (int rc = static_scratch(&ws)) return rc;
-    return odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, items, n_items, item_range, dispatch_order, pi_k_t, pi_v,
-                               codebooks, codebooks_host, inv_scales, out, out_dtype, lse, ws, (size_t)ODMKV_STATIC_SCRATCH_BYTES,
-                               stream, 7, nullptr, nullptr);
+    return odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, work, pi_k_t, pi_v, codebooks, codebooks_host, inv_scales,
+                               out, out_dtype, lse, ws, (size_t)ODMKV_STATIC_SCRATCH_BYTES, stream, 7, nullptr, nullptr);
 }

@@ -36,6 +36,14 @@ class Packed(C.Structure):
     ]
 
 
+class Worklist(C.Structure):
+    """struct odmkv_worklist of include/odmkv.h."""
+    _fields_ = [
+        ("items", C.c_void_p), ("item_range", C.c_void_p), ("dispatch_order", C.c_void_p),
+        ("n_items", C.c_int32),
+    ]
+
+
 def _load() -> C.CDLL:
     if not os.path.exists(LIB_PATH):
         raise ImportError(
@@ -63,9 +71,9 @@ def _load() -> C.CDLL:
         "odmkv_dequant": (C.c_int, [C.POINTER(Packed), vp, vp, i32, i32, i64, i64, i64, vp, vp, vp, i32, vp]),
         "odmkv_append_exact": (C.c_int, [C.POINTER(Packed), vp, vp, i64, i64, i32, vp]),
         "odmkv_decode_workspace_bytes": (sz, [i32, i32, i32]),
-        "odmkv_decode_attn": (C.c_int, [vp, i32, i32, i32, f32, C.POINTER(Packed), vp, i32, vp, vp, vp, vp, vp,
+        "odmkv_decode_attn": (C.c_int, [vp, i32, i32, i32, f32, C.POINTER(Packed), C.POINTER(Worklist), vp, vp, vp,
                                         C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp, sz, vp]),
-        "odmkv_decode_attn_static": (C.c_int, [vp, i32, i32, i32, f32, C.POINTER(Packed), vp, i32, vp, vp, vp, vp, vp,
+        "odmkv_decode_attn_static": (C.c_int, [vp, i32, i32, i32, f32, C.POINTER(Packed), C.POINTER(Worklist), vp, vp, vp,
                                                C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp]),
     }
     for name, (res, args) in sig.items():

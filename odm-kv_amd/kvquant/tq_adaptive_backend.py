@@ -133,6 +133,7 @@ class TurboQuantAdaptiveKVCacheState:
         self._masked = None           # cached (indices of evicted positions,) or None when stale
         self._items = None
         self._item_order = None
+        self._worklist = None         # ctypes twin of odmkv_worklist_t over the tensors above
         self._items_choice = None     # (winning items-per-compute-unit multiple, packed bytes it was chosen at)
         self._packed = None
 
@@ -559,7 +560,7 @@ class TurboQuantAdaptiveKVCacheState:
 
         def cost(item) -> float:                     # microseconds of one workgroup, roughly
             rounds = -(-item[3] // 8)
-            return (3.0 + 1.0 * rounds) if item[1] == 4 else (3.5 + 1.5 * rounds)
+            return (3.0 + 1.0 * rounds) if item[1] == 4 else (3.0 + 1.0 * rounds)
 
         def makespan(items) -> float:
             import heapq
@@ -592,10 +593,14 @@ class TurboQuantAdaptiveKVCacheState:
         order = None
         if len(items) > n_cu:
             order = np.argsort(-np.asarray([cost(it) for it in items]), kind="stable").astype(np.int32)
-            order = torch.from_numpy(order).to(self.device)
+        self._item_order = None if order is None else torch.from_numpy(order).to(self.device)
         self._items = (torch.from_numpy(arr).to(self.device),
                        torch.from_numpy(ranges.astype(np.int32)).to(self.device), len(items))
-        self._item_order = order
+        w = _lib.Worklist()
+        w.items, w.item_range = self._items[0].data_ptr(), self._items[1].data_ptr()
+        w.dispatch_order = _lib.ptr(self._item_order)
+        w.n_items = len(items)
+        self._worklist = w
 
     def decode_attention(self, query: torch.Tensor, scaling: Optional[float] = None,
                          return_lse: bool = False, out_dtype: torch.dtype = torch.float32):
@@ -622,8 +627,8 @@ class TurboQuantAdaptiveKVCacheState:
         ws_bytes = lib.odmkv_decode_workspace_bytes(B, Hq, n_items)
         ws = _lib.workspace(self.device, ws_bytes, "decode")
         _lib.check(lib.odmkv_decode_attn(
-            q.data_ptr(), _lib.dtype_code(q), B, Hq, scale, C.byref(self._packed), items.data_ptr(), n_items,
-            ranges.data_ptr(), _lib.ptr(self._item_order), self._pi_k_t.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
+            q.data_ptr(), _lib.dtype_code(q), B, Hq, scale, C.byref(self._packed), C.byref(self._worklist),
+            self._pi_k_t.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
             self._decode_cb_host, self._decode_inv, out.data_ptr(), _lib.dtype_code(out), _lib.ptr(lse), ws.data_ptr(), ws_bytes,
             _lib.stream_ptr(self.device)))
         return (out, lse) if return_lse else out

@@ -25,6 +25,15 @@ def test_exports_every_declared_symbol(lib):
         assert hasattr(lib, name), f"{name} is declared in odmkv.h but not exported"
     from kvquant import _lib
     assert set(_lib.EXPORTS) == declared
+    # the measurement entry points live in a library of their own and are not part of the product ABI
+    bench_header = open(os.path.join(ROOT, "include", "odmkv_bench.h")).read()
+    bench_declared = set(re.findall(r"\b(odmkv_bench_[a-z_]+)\s*\(", bench_header))
+    assert len(bench_declared) >= 5
+    blib = C.CDLL(os.path.join(ROOT, "odm-kv_amd", "lib", "libodmkv_bench.so"))
+    for name in bench_declared:
+        assert hasattr(blib, name) and not hasattr(lib, name)
+    for name in declared:
+        assert hasattr(blib, name)
 
 
 def test_version_and_error_slot(lib):
@@ -59,12 +68,14 @@ def test_argument_checks_without_a_gpu(lib):
     # unsupported width
     rc = lib.odmkv_quantize_rows(p, 0, C.c_int64(4), C.c_int64(128), 5, p, p, p, p, None)
     assert rc == -1 and b"width" in lib.odmkv_last_error()
-    rc = lib.odmkv_decode_attn(None, 2, 1, 8, C.c_float(1.0), None, None, 0, None, None, None, None, None, None, None,
+    rc = lib.odmkv_decode_attn(None, 2, 1, 8, C.c_float(1.0), None, None, None, None, None, None, None,
                                None, 2, None, None, C.c_size_t(0), None)
     assert rc == -1
-    rc = lib.odmkv_decode_attn(p, 7, 1, 8, C.c_float(1.0), None, None, 0, None, None, None, None, None, None, None,
+    rc = lib.odmkv_decode_attn(p, 7, 1, 8, C.c_float(1.0), None, None, None, None, None, None, None,
                                p, 2, None, None, C.c_size_t(0), None)
     assert rc == -1 and b"query dtype" in lib.odmkv_last_error()
+    rc = lib.odmkv_decode_attn_static(p, 0, 1, 8, C.c_float(1.0), None, None, None, None, None, None, None, p, 2, None, None)
+    assert rc == -1 and b"work list" in lib.odmkv_last_error()
 
 
 def test_host_modules_import_and_validate():
