@@ -21,8 +21,6 @@ struct DecodeArgs {
     const float* pi_k_t;   // Pi_k transposed
     const float* pi_v;
     const float* cb;
-    uint4* qrot;      // [B*Hq][2][128] fp16: high and low halves of Pi_k q16
-    uint4* qs;        // [B*Hq][2][128] q16 itself for the exact tokens (fp16 + zeros, or bf16 high + low pieces)
     float inv_s[4];   // 1 / table scale per width
     float cbs[28];    // scaled centroids of widths 2, 3, 4 (kept in scalar registers; 8-bit ones stay in memory)
     int gp;           // head slots per item in `partial`: 4 or 8
@@ -31,8 +29,8 @@ struct DecodeArgs {
     float* lse;
 };
 
-// stage_mask: bit 0 the query preparation, bit 1 the main kernel, bit 2 the merge (7 = the
-// product call).  ev_start / ev_stop: hipEvent_t attached to the main kernel's dispatch, or null.
+// stage_mask: bit 1 the main kernel (query rotation included), bit 2 the merge (6 or 7 = the product
+// call; bit 0 is unused).  ev_start / ev_stop: hipEvent_t attached to the main kernel's dispatch, or null.
 int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling,
                         const odmkv_packed_t* store, const odmkv_worklist_t* work,
                         const float* pi_k_t, const float* pi_v, const float* codebooks,

@@ -34,83 +34,29 @@ typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f2 __attribute__((ext_vector_type(2)));
 
 #define LUT_BYTES 65536
 #define LOG2E 1.4426950408889634f
 #define LN2 0.6931471805599453f
-#define PROW 144            // bytes per head row of a wave's p buffer: 64 x 16 bit + 16 of padding (bank spread)
-#define PBUF (16 * PROW)    // one p buffer (8 head rows used)
-#define QROW 256            // bytes of one query row (128 x 16 bit)
+#define UNIT 32             // tokens of a unit of work: half a tile
+#define PROW 96             // bytes per head row of a wave's p buffer: 32 x 16 bit + padding (bank spread)
+#define PBUF (8 * PROW)     // one p buffer: 8 head rows
 
-// LDS of the main kernel: [table | combine area | Pi_v of the merge] [p buffers | merge scratch] [per-wave scalars]
-#define LDS_PBUFS LUT_BYTES
+// LDS of the main kernel: [table, later the combine area] [partial sums of the query rotation] [rotated query rows]
+// [p buffers] [per-wave scalars]
+#define ROT_SLICES (DECODE_NWAVES * 64 / 32)     // slices of the rotation's sum: a thread covers 4 dims x HD / ROT_SLICES terms
+#define ROT_TERMS (HD / ROT_SLICES)
+#define QROW_LDS 272                             // bytes of a query row in LDS: 128 x 16 bit + 16 (bank spread)
+#define LDS_ROT LUT_BYTES
+#define LDS_QROWS (LDS_ROT + ROT_SLICES * ODMKV_MAX_GROUP * HD * 4)
+#define LDS_PBUFS (LDS_QROWS + 16 * QROW_LDS)
 #define LDS_SCALARS (LDS_PBUFS + DECODE_NWAVES * 2 * PBUF)
-#define LDS_TOTAL (LDS_SCALARS + DECODE_NWAVES * 3 * 8 * 4)
+#define LDS_TOTAL (LDS_SCALARS + DECODE_NWAVES * 4 * 8 * 4 + 8 * 4)
 static_assert(DECODE_NWAVES * ODMKV_MAX_GROUP * HD * 4 <= LUT_BYTES, "combine area must fit the table's space");
-static_assert((256 / DECODE_NWAVES) % 4 == 0, "wave count");
+static_assert((256 / DECODE_NWAVES) % 4 == 0 && DECODE_NWAVES <= 16 && ROT_TERMS == 8, "wave count");
 
-// ------------------------------------------------------------------------------------------------
-// prep: rotate the queries
-// ------------------------------------------------------------------------------------------------
 __device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
-
-#ifndef PREP_SPLIT
-#define PREP_SPLIT 4                       // workgroups per query head, each producing HD / PREP_SPLIT rotated dims
-#endif
-#define PREP_THREADS 512
-__global__ __launch_bounds__(PREP_THREADS) void decode_prep_kernel(DecodeArgs a) {
-    constexpr int QD = HD / PREP_SPLIT;     // rotated dims of this workgroup
-    constexpr int JS = PREP_THREADS / QD;   // slices of the sum over j
-    constexpr int JN = HD / JS;             // terms per slice
-    __shared__ float qsh[HD];
-    __shared__ float part[JS][QD];
-    const int bq = blockIdx.x / PREP_SPLIT, quarter = blockIdx.x % PREP_SPLIT, tid = threadIdx.x;
-    const int ii = tid % QD, js = tid / QD, i = quarter * QD + ii;
-    // this thread's JN elements of column i of Pi_k (rows of the transposed matrix): all requested at once.
-    // No workgroup pulls the whole 64 KB matrix through one compute unit.
-    float pk[JN];
-#pragma unroll
-    for (int jj = 0; jj < JN; ++jj) pk[jj] = a.pi_k_t[(size_t)(js * JN + jj) * HD + i];
-    if (tid < HD) {
-        // the query is consumed at fp16 precision, like the attention it replaces (model dtype)
-        const size_t qi = (size_t)bq * HD + tid;
-        const float qf = a.q_dt == ODMKV_F32 ? reinterpret_cast<const float*>(a.q)[qi]
-                       : a.q_dt == ODMKV_F16 ? Elem<ODMKV_F16>::to_f32(reinterpret_cast<const uint16_t*>(a.q)[qi])
-                                             : Elem<ODMKV_BF16>::to_f32(reinterpret_cast<const uint16_t*>(a.q)[qi]);
-        const __half q16 = __float2half_rn(qf);
-        const float q32 = __half2float(q16);
-        qsh[tid] = q32;
-        if (tid / QD == quarter) {           // the un-rotated copy (for exact tiles): every workgroup writes its own dims
-            uint16_t* qs16 = reinterpret_cast<uint16_t*>(a.qs) + (size_t)bq * 2 * HD;
-            if (a.s.exact_dtype == ODMKV_BF16) {
-                // exact bf16 rows meet the query on the bf16 matrix instructions: q16 = hi + lo exactly
-                // (11 significant bits in two pieces of 8)
-                const uint16_t hi = Elem<ODMKV_BF16>::from_f32(q32);
-                qs16[tid] = hi;
-                qs16[HD + tid] = Elem<ODMKV_BF16>::from_f32(q32 - Elem<ODMKV_BF16>::to_f32(hi));
-            } else {
-                qs16[tid] = __half_as_ushort(q16);
-                qs16[HD + tid] = 0;
-            }
-        }
-    }
-    __syncthreads();
-    // q'_i = sum_j Pi_k[i][j] q_j: every slice sums its share of j in order, the slices are added in order
-    float acc = 0.0f;
-#pragma unroll
-    for (int jj = 0; jj < JN; ++jj) acc = __fmaf_rn(pk[jj], qsh[js * JN + jj], acc);
-    part[js][ii] = acc;
-    __syncthreads();
-    if (tid < QD) {
-        float tot = part[0][tid];
-#pragma unroll
-        for (int sl = 1; sl < JS; ++sl) tot += part[sl][tid];
-        uint16_t* qr16 = reinterpret_cast<uint16_t*>(a.qrot) + (size_t)bq * 2 * HD;
-        const __half hi = __float2half_rn(tot);
-        qr16[i] = __half_as_ushort(hi);
-        qr16[HD + i] = (uint16_t)half_bits(tot - __half2float(hi));
-    }
-}
 
 // ------------------------------------------------------------------------------------------------
 // small helpers
@@ -294,6 +240,41 @@ __device__ static inline uint4 stream_load(const uint4* p) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// eight consecutive elements of the query: the request (one or two 16-byte loads) and, apart from it, the
+// conversion to floats rounded to fp16 (the precision at which the attention this call replaces consumes its
+// query).  Keeping them apart lets other requests be issued before the first value is needed.
+struct RawQ8 { uint4 x, y; };
+__device__ static inline RawQ8 request_q8(const void* q, int dt, size_t elem) {
+    RawQ8 r;
+    if (dt == ODMKV_F32) {
+        r.x = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(q) + elem);
+        r.y = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(q) + elem + 4);
+    } else {
+        r.x = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(q) + elem);
+        r.y = make_uint4(0u, 0u, 0u, 0u);
+    }
+    return r;
+}
+__device__ static inline void convert_q8(const RawQ8& r, int dt, float* out) {
+    const uint32_t w[8] = {r.x.x, r.x.y, r.x.z, r.x.w, r.y.x, r.y.y, r.y.z, r.y.w};
+    if (dt == ODMKV_F32) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = __half2float(__float2half_rn(__uint_as_float(w[e])));
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint16_t bits = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+            out[e] = dt == ODMKV_F16 ? Elem<ODMKV_F16>::to_f32(bits) : __half2float(__float2half_rn(Elem<ODMKV_BF16>::to_f32(bits)));
+        }
+    }
+}
+__device__ static inline void load_q8(const void* q, int dt, size_t elem, float* out) { convert_q8(request_q8(q, dt, elem), dt, out); }
+
+__device__ static inline uint32_t bf16_pair(float a, float b) {
+    return (uint32_t)Elem<ODMKV_BF16>::from_f32(a) | ((uint32_t)Elem<ODMKV_BF16>::from_f32(b) << 16);
+}
+__device__ static inline float bf16_rest(float a) { return a - Elem<ODMKV_BF16>::to_f32(Elem<ODMKV_BF16>::from_f32(a)); }
+
 __device__ static inline uint32_t pack_h2(float a, float b) {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
     union { h2 h; uint32_t u; } x;
@@ -301,194 +282,262 @@ __device__ static inline uint32_t pack_h2(float a, float b) {
     return x.u;
 }
 
-// Softmax step of one tile for this lane's two heads.  tA/tB: base-2 logits of slots 4n..4n+3 (padding:
-// -inf).  Returns the weights p (relative to the new running maxima), updates (m, l), and rescales the
-// accumulators when a maximum moved.
-__device__ static inline void softmax_tile(WaveState& st, const float* tA, const float* tB, int lane,
+// Softmax step of one unit (32 tokens) for this lane's two heads.  tA/tB: base-2 logits of the lane's two
+// slots (padding: -inf).  Returns the weights p = exp2(t - m) and updates (m, l).  m is a reference point, not
+// the exact running maximum: it moves (and the accumulators are rescaled) only when a logit exceeds it by more
+// than SOFTMAX_SLACK, so p stays below 2^SOFTMAX_SLACK and most units need neither a cross-lane reduction nor a
+// pass over the accumulators.  Any reference point gives the same quotient sum(p v) / sum(p).
+// The weights are kept 2^P_SHIFT times larger than that: they reach the matrix instructions as fp16, whose normal
+// range ends at 6e-5, and in a long context next to a dominant token most weights lie far below (rounded to a few bits,
+// or to zero, as they would otherwise be).  The normaliser carries the same factor, so the quotient does not; the
+// merge takes it out of the log-sum-exp.
+#define SOFTMAX_SLACK 3.0f
+#define P_SHIFT 8.0f
+#define FP16_MAX 65504.0f
+__device__ static inline void softmax_unit(WaveState& st, const float* tA, const float* tB, int lane,
                                            float* alpha_sh, float* pA, float* pB) {
     const int n = lane & 15, j = lane >> 4;
-    float mxA = fmaxf(fmaxf(tA[0], tA[1]), fmaxf(tA[2], tA[3]));
-    float mxB = fmaxf(fmaxf(tB[0], tB[1]), fmaxf(tB[2], tB[3]));
-    // the running maxima move only when some lane sees a larger logit (wave-uniform test): no cross-lane
-    // reduction otherwise
-    if (__builtin_amdgcn_ballot_w64(mxA > st.mA || mxB > st.mB) != 0) {
+    float mxA = fmaxf(tA[0], tA[1]);
+    float mxB = fmaxf(tB[0], tB[1]);
+    if (__builtin_amdgcn_ballot_w64(mxA > st.mA + SOFTMAX_SLACK || mxB > st.mB + SOFTMAX_SLACK) != 0) {      // wave-uniform
         row_max2(mxA, mxB);
         const float mnA = fmaxf(st.mA, mxA), mnB = fmaxf(st.mB, mxB);
-        const float aA = __builtin_amdgcn_exp2f(st.mA - mnA), aB = __builtin_amdgcn_exp2f(st.mB - mnB);   // first tile: exp2(-inf) = 0
-        st.lA *= aA; st.lB *= aB;
+        if (__builtin_amdgcn_ballot_w64(st.mA > -INFINITY || st.mB > -INFINITY) != 0) {     // not the wave's first unit
+            const float aA = __builtin_amdgcn_exp2f(st.mA - mnA), aB = __builtin_amdgcn_exp2f(st.mB - mnB);
+            st.lA *= aA; st.lB *= aB;
+            if (n == 0) { alpha_sh[2 * j] = aA; alpha_sh[2 * j + 1] = aB; }
+            wave_lds_fence();
+            const f4 al = *reinterpret_cast<const f4*>(alpha_sh + 4 * (j & 1));      // heads 4j..4j+3 of the output rows
+#pragma unroll
+            for (int nb = 0; nb < 8; ++nb) st.acc[nb] *= al;
+        }
         st.mA = mnA; st.mB = mnB;
-        if (n == 0) { alpha_sh[2 * j] = aA; alpha_sh[2 * j + 1] = aB; }
-        wave_lds_fence();
-        const f4 al = *reinterpret_cast<const f4*>(alpha_sh + 4 * (j & 1));      // heads 4j..4j+3 of the output rows
-#pragma unroll
-        for (int nb = 0; nb < 8; ++nb) st.acc[nb] *= al;
     }
-    const float mnA = st.mA, mnB = st.mB;
+    const float mnA = st.mA - P_SHIFT, mnB = st.mB - P_SHIFT;
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
+    for (int b = 0; b < 2; ++b) {
         pA[b] = __builtin_amdgcn_exp2f(tA[b] - mnA);      // padded slots: -inf -> 0
         pB[b] = __builtin_amdgcn_exp2f(tB[b] - mnB);
     }
-    st.lA += (pA[0] + pA[1]) + (pA[2] + pA[3]);
-    st.lB += (pB[0] + pB[1]) + (pB[2] + pB[3]);
+    st.lA += pA[0] + pA[1];
+    st.lB += pB[0] + pB[1];
 }
 
-// ---- quantised tiles -----------------------------------------------------------------------------
-// A lane's 16*W bytes of key codes: 128 codes, code 32b+i = dim 32j+i of slot 4n+b.
-// A lane's 16*W bytes of value codes: 128 codes, code 64kb+8nb+e = slot 32kb+8j+e of dim 16nb+n.
+// this lane's two slots inside a unit are 2 * pair_slot(n) and the next one (see key_slot)
+__device__ static inline int pair_slot(int n) { return 8 * (n >> 2) + 2 * (n & 3); }
+
+// ---- quantised units -----------------------------------------------------------------------------
+// Unit h of a tile = slots 32h .. 32h+31 = the h-th half of every lane's code bytes:
+//   keys:   the lane's 64 codes of the unit are  code 32b + i = dim 32j + i of slot 32h + pair_slot(n) + b
+//   values: the lane's 64 codes of the unit are  code 8m + e  = slot 32h + 8j + e of dim 16m + n
 template <int W>
-struct TileData {
-    uint32_t kw[4 * W];
-    uint32_t vw[4 * W];
-    f4 kn, vn;
+struct Unit {
+    uint32_t kw[2 * W];
+    uint32_t vw[2 * W];
+    f2 kn, vn;
 };
 
+// the h-th half (8 * W bytes) of a lane's 16 * W bytes of a tile buffer
 template <int W>
-__device__ static inline void load_tile(TileData<W>& t, const DecodeArgs& a, int li, int tile, int lane) {
-    const uint8_t* ksrc = a.s.kcodes[li] + (size_t)tile * (TILE * 16 * W);
-    const uint8_t* vsrc = a.s.vcodes[li] + (size_t)tile * (TILE * 16 * W);
+__device__ static inline void load_half_stream(uint32_t* w, const uint8_t* tile_base, int h, int lane) {
+    if constexpr (W == 3) {
+        // 24 bytes: chunk 0 and half of chunk 1, or the other half of chunk 1 and chunk 2
+        const uint8_t* mid = tile_base + ((size_t)TILE + lane) * 16;
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        if (h == 0) {
+            const uint4 x = stream_load(reinterpret_cast<const uint4*>(tile_base + (size_t)lane * 16));
+            const u32x2 y = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(mid));
+            w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w; w[4] = y.x; w[5] = y.y;
+        } else {
+            const u32x2 y = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(mid + 8));
+            const uint4 x = stream_load(reinterpret_cast<const uint4*>(tile_base + ((size_t)2 * TILE + lane) * 16));
+            w[0] = y.x; w[1] = y.y; w[2] = x.x; w[3] = x.y; w[4] = x.z; w[5] = x.w;
+        }
+    } else {
+        constexpr int C = W / 2;                            // whole 16-byte chunks per half
 #pragma unroll
-    for (int c = 0; c < W; ++c) {
-        const uint4 v = stream_load(reinterpret_cast<const uint4*>(ksrc + ((size_t)c * TILE + lane) * 16));
-        t.kw[4 * c] = v.x; t.kw[4 * c + 1] = v.y; t.kw[4 * c + 2] = v.z; t.kw[4 * c + 3] = v.w;
+        for (int c = 0; c < C; ++c) {
+            const uint4 v = stream_load(reinterpret_cast<const uint4*>(tile_base + ((size_t)(C * h + c) * TILE + lane) * 16));
+            w[4 * c] = v.x; w[4 * c + 1] = v.y; w[4 * c + 2] = v.z; w[4 * c + 3] = v.w;
+        }
     }
-#pragma unroll
-    for (int c = 0; c < W; ++c) {
-        const uint4 v = stream_load(reinterpret_cast<const uint4*>(vsrc + ((size_t)c * TILE + lane) * 16));
-        t.vw[4 * c] = v.x; t.vw[4 * c + 1] = v.y; t.vw[4 * c + 2] = v.z; t.vw[4 * c + 3] = v.w;
-    }
-    const size_t quad = (size_t)tile * TILE + 4 * (lane & 15);
-    t.kn = __builtin_nontemporal_load(reinterpret_cast<const f4*>(a.s.knorm[li] + quad));
-    t.vn = __builtin_nontemporal_load(reinterpret_cast<const f4*>(a.s.vnorm[li] + quad));
 }
 
 template <int W>
-__device__ static inline void compute_tile(const TileData<W>& t, int nvalid, int lane, const uint8_t* lut,
+__device__ static inline void load_unit(Unit<W>& t, const DecodeArgs& a, int li, int unit, int lane) {
+    const int tile = unit >> 1, h = unit & 1;               // wave-uniform
+    load_half_stream<W>(t.kw, a.s.kcodes[li] + (size_t)tile * (TILE * 16 * W), h, lane);
+    load_half_stream<W>(t.vw, a.s.vcodes[li] + (size_t)tile * (TILE * 16 * W), h, lane);
+    const size_t pair = (size_t)unit * UNIT + pair_slot(lane & 15);
+    t.kn = __builtin_nontemporal_load(reinterpret_cast<const f2*>(a.s.knorm[li] + pair));
+    t.vn = __builtin_nontemporal_load(reinterpret_cast<const f2*>(a.s.vnorm[li] + pair));
+}
+
+template <int W>
+__device__ static inline void compute_unit(const Unit<W>& t, int nvalid, int lane, const uint8_t* lut,
                                            uint32_t slot4, const h8* qa, float ksc, float vsc,
                                            uint8_t* pbuf, float* alpha_sh, WaveState& st) {
     const int n = lane & 15, j = lane >> 4;
-    // ---- keys: D[q row][token] ----
-    f4 dk[4];
-#pragma unroll
-    for (int b = 0; b < 4; ++b) dk[b] = (f4){0.f, 0.f, 0.f, 0.f};
+    // ---- keys: D[q row][token], two token blocks x four dim blocks ----
+    f4 dk[2];
+    dk[0] = (f4){0.f, 0.f, 0.f, 0.f};
+    dk[1] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) dk[b] = MFMA_F16(qa[kb], lut8<W>(t.kw, 4 * b + kb, lut, slot4), dk[b]);
-    float tA[4], tB[4];
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const float kn = t.kn[b] * ksc;
-        tA[b] = (dk[b][0] + dk[b][1]) * kn;
-        tB[b] = (dk[b][2] + dk[b][3]) * kn;
+        for (int b = 0; b < 2; ++b) dk[b] = MFMA_F16(qa[kb], lut8<W>(t.kw, 4 * b + kb, lut, slot4), dk[b]);
+    float tA[2], tB[2];
+    {
+        const float kn0 = t.kn.x * ksc, kn1 = t.kn.y * ksc;
+        tA[0] = (dk[0][0] + dk[0][1]) * kn0; tB[0] = (dk[0][2] + dk[0][3]) * kn0;
+        tA[1] = (dk[1][0] + dk[1][1]) * kn1; tB[1] = (dk[1][2] + dk[1][3]) * kn1;
     }
-    if (nvalid < TILE) {                                   // the last tile of a run (wave-uniform)
+    if (nvalid < UNIT) {                                   // the last unit of a run (wave-uniform)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const bool ok = 4 * n + b < nvalid;
+        for (int b = 0; b < 2; ++b) {
+            const bool ok = pair_slot(n) + b < nvalid;
             tA[b] = ok ? tA[b] : -INFINITY;
             tB[b] = ok ? tB[b] : -INFINITY;
         }
     }
-    float pA[4], pB[4];
-    softmax_tile(st, tA, tB, lane, alpha_sh, pA, pB);
+    float pA[2], pB[2];
+    softmax_unit(st, tA, tB, lane, alpha_sh, pA, pB);
     {
-        float vn[4];
-#pragma unroll
-        for (int b = 0; b < 4; ++b) vn[b] = t.vn[b] * vsc;
-        *reinterpret_cast<uint2*>(pbuf + (2 * j) * PROW + 8 * n) =
-            make_uint2(pack_h2(pA[0] * vn[0], pA[1] * vn[1]), pack_h2(pA[2] * vn[2], pA[3] * vn[3]));
-        *reinterpret_cast<uint2*>(pbuf + (2 * j + 1) * PROW + 8 * n) =
-            make_uint2(pack_h2(pB[0] * vn[0], pB[1] * vn[1]), pack_h2(pB[2] * vn[2], pB[3] * vn[3]));
+        // p |v| as fp16 into the lane's two slots (bytes 2 * pair_slot(n) = 4n .. 4n+3) of rows 2j and 2j+1
+        const float vn0 = t.vn.x * vsc, vn1 = t.vn.y * vsc;
+        // (the clamp only matters for value norms thousands of times the table's scale: no infinities)
+        *reinterpret_cast<uint32_t*>(pbuf + (2 * j) * PROW + 4 * n) = pack_h2(fminf(pA[0] * vn0, FP16_MAX), fminf(pA[1] * vn1, FP16_MAX));
+        *reinterpret_cast<uint32_t*>(pbuf + (2 * j + 1) * PROW + 4 * n) = pack_h2(fminf(pB[0] * vn0, FP16_MAX), fminf(pB[1] * vn1, FP16_MAX));
     }
     wave_lds_fence();
-    // ---- values: D[head][dim] ----
+    // ---- values: D[head][dim], eight dim blocks ----
+    const h8 pa = as_h8(*reinterpret_cast<const uint4*>(pbuf + (n & 7) * PROW + 16 * j));
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-        const h8 pa = as_h8(*reinterpret_cast<const uint4*>(pbuf + (n & 7) * PROW + (32 * kb + 8 * j) * 2));
-#pragma unroll
-        for (int nb = 0; nb < 8; ++nb) st.acc[nb] = MFMA_F16(pa, lut8<W>(t.vw, 8 * kb + nb, lut, slot4), st.acc[nb]);
-    }
-    wave_lds_fence();                                      // the p buffer is free for the next tile
+    for (int m = 0; m < 8; ++m) st.acc[m] = MFMA_F16(pa, lut8<W>(t.vw, m, lut, slot4), st.acc[m]);
+    wave_lds_fence();                                      // the p buffer is free for the next unit
 }
 
 // the A operand of the key products: rows 2h, 2h+1 = high, low half of head h; row `n` of this lane,
-// dims 32j + 8kb .. + 7 for step kb.  Rows behind the group's heads are zero.
-__device__ static inline void load_queries(const uint8_t* rows, int lane, int nheads, uint4* q) {
+// dims 32j + 8kb .. + 7 for step kb, from the query rows in LDS.  Rows behind the group's slots are zero.
+__device__ static inline void load_queries(const uint8_t* qrows, int lane, int nrows, h8* qa) {
     const int n = lane & 15, j = lane >> 4;
-    const bool on = n < 2 * nheads;
+    const bool on = n < nrows;
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb)
-        q[kb] = on ? *reinterpret_cast<const uint4*>(rows + n * QROW + (32 * j + 8 * kb) * 2) : make_uint4(0u, 0u, 0u, 0u);
+        qa[kb] = as_h8(on ? *reinterpret_cast<const uint4*>(qrows + n * QROW_LDS + (32 * j + 8 * kb) * 2) : make_uint4(0u, 0u, 0u, 0u));
 }
 
-// One work item of a quantised level: the workgroup's wavefronts walk the item's tiles.
-template <int W>
+// The queries in the rotated basis of the quantised keys, q' = Pi_k q16, as fp16 high + low halves.  Thread
+// (i4 = tid % 32, slice = tid / 32) holds Pi_k^T[8 slice .. + 7][4 i4 .. + 3] (requested when the kernel starts, before
+// the work item is known) and sums its eight terms for every head of the group, in order; the slices are added in
+// order by the thread that owns (head, dim).  Every workgroup of a KV head repeats this: the matrix comes out of the
+// L2 cache, and the work hides behind the first unit's way from memory.
+template <int GP>
+__device__ static inline void rotate_request(const DecodeArgs& a, int bq_first, RawQ8* raw, int tid) {
+    const int slice = tid >> 5;
+#pragma unroll
+    for (int g = 0; g < GP; ++g)
+        if (g < a.G) raw[g] = request_q8(a.q, a.q_dt, (size_t)(bq_first + g) * HD + slice * ROT_TERMS);
+}
+template <int GP>
+__device__ static inline void rotate_partial(const DecodeArgs& a, const RawQ8* raw, const f4* pk, float* rot, int tid) {
+    const int i4 = tid & 31, slice = tid >> 5;
+#pragma unroll
+    for (int g = 0; g < GP; ++g) {
+        f4 acc = (f4){0.f, 0.f, 0.f, 0.f};
+        if (g < a.G) {                                     // wave-uniform
+            float qv[8];
+            convert_q8(raw[g], a.q_dt, qv);
+#pragma unroll
+            for (int t = 0; t < ROT_TERMS; ++t)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] = __fmaf_rn(pk[t][e], qv[t], acc[e]);
+        }
+        *reinterpret_cast<f4*>(rot + ((size_t)(slice * GP + g) * HD) + 4 * i4) = acc;
+    }
+}
+template <int GP>
+__device__ static inline void rotate_finish(const float* rot, uint8_t* qrows, int tid) {
+    for (int o = tid; o < GP * HD; o += DECODE_NWAVES * 64) {
+        const int g = o / HD, dim = o % HD;
+        float tot = rot[(size_t)g * HD + dim];
+#pragma unroll
+        for (int sl = 1; sl < ROT_SLICES; ++sl) tot += rot[((size_t)sl * GP + g) * HD + dim];
+        const __half hi = __float2half_rn(tot);
+        *reinterpret_cast<uint16_t*>(qrows + (2 * g) * QROW_LDS + dim * 2) = __half_as_ushort(hi);
+        *reinterpret_cast<uint16_t*>(qrows + (2 * g + 1) * QROW_LDS + dim * 2) = (uint16_t)half_bits(tot - __half2float(hi));
+    }
+}
+
+// One work item of a quantised level: the workgroup's wavefronts walk the item's units.
+template <int W, int GP>
 __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq_first, int tile0, int ntiles, int ntok,
-                                              int tid, uint8_t* lut, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
+                                              int tid, const f4* pk, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
+    uint8_t* lut = smem;
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
     const float vsc = a.inv_s[li], ksc = a.inv_s[li] * a.scaling * LOG2E;
-    // The table needs nothing from memory and is built before the tiles are requested: behind a
-    // wavefront's tile requests its LDS traffic would wait for the memory pipeline to accept them.
-    // Loads return in issue order: the (small) query rows go first.
-    uint4 qraw[4];
-    load_queries(reinterpret_cast<const uint8_t*>(a.qrot) + (size_t)bq_first * 2 * QROW, lane, a.G, qraw);
+    const int unit0 = 2 * tile0;
+    const auto tokens_of = [&](int u) { return min(ntok - u * UNIT, UNIT); };    // <= 0 behind the item's last token
+    // Each wavefront requests its first unit, then rotates the queries and builds its share of the table while memory
+    // answers; the second unit is requested after that (LDS stores behind a long queue of requests wait until the
+    // memory pipeline has accepted them: with both units requested first the table was ready a microsecond later).
+    // Loads return in issue order: the (small) query goes first.
+    RawQ8 qraw[GP];
+    rotate_request<GP>(a, bq_first, qraw, tid);
+    Unit<W> cur;
+    int u = wave;
+    int nvalid = tokens_of(u);
+    if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
     build_lut<W>(lut, a, tid);
-    TileData<W> cur;
-    int tt = wave;
-    int nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
-    if (nvalid > 0) load_tile<W>(cur, a, li, tile0 + tt, lane);
+    rotate_partial<GP>(a, qraw, pk, reinterpret_cast<float*>(smem + LDS_ROT), tid);
     lds_barrier();
-    // second buffer (not for the widest rows), requested before the first tile is used
-    TileData<W> nxt;
+    rotate_finish<GP>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
+    lds_barrier();
+    // second buffer (not for the widest rows), requested before the first unit is used
+    Unit<W> nxt;
     int nv1 = 0;
     if constexpr (W != 8) {
-        nv1 = tt + DECODE_NWAVES < ntiles ? min(ntok - (tt + DECODE_NWAVES) * TILE, TILE) : 0;
-        if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + DECODE_NWAVES, lane);
+        nv1 = tokens_of(u + DECODE_NWAVES);
+        if (nv1 > 0) load_unit<W>(nxt, a, li, unit0 + u + DECODE_NWAVES, lane);
     }
     if (nvalid <= 0) return;
     h8 qa[4];
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb) qa[kb] = as_h8(qraw[kb]);
+    load_queries(smem + LDS_QROWS, lane, 2 * GP, qa);
     if constexpr (W == 8) {
         while (true) {
-            compute_tile<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
-            tt += DECODE_NWAVES;
-            nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
+            compute_unit<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
+            u += DECODE_NWAVES;
+            nvalid = tokens_of(u);
             if (nvalid <= 0) break;
-            load_tile<W>(cur, a, li, tile0 + tt, lane);
+            load_unit<W>(cur, a, li, unit0 + u, lane);
         }
     } else {
         while (true) {
-            compute_tile<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
+            compute_unit<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
             if (nv1 <= 0) break;
-            tt += 2 * DECODE_NWAVES;
-            nvalid = tt < ntiles ? min(ntok - tt * TILE, TILE) : 0;
-            if (nvalid > 0) load_tile<W>(cur, a, li, tile0 + tt, lane);
-            compute_tile<W>(nxt, nv1, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
+            u += 2 * DECODE_NWAVES;
+            nvalid = tokens_of(u);
+            if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
+            compute_unit<W>(nxt, nv1, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
             if (nvalid <= 0) break;
-            nv1 = tt + DECODE_NWAVES < ntiles ? min(ntok - (tt + DECODE_NWAVES) * TILE, TILE) : 0;
-            if (nv1 > 0) load_tile<W>(nxt, a, li, tile0 + tt + DECODE_NWAVES, lane);
+            nv1 = tokens_of(u + DECODE_NWAVES);
+            if (nv1 > 0) load_unit<W>(nxt, a, li, unit0 + u + DECODE_NWAVES, lane);
         }
     }
 }
 
-// ---- exact (fp16 / bf16) tiles ---------------------------------------------------------------------
-// Keys of a tile: chunk 4b+kb of lane (n, j) = dims 32j+8kb..+7 of slot 4n+b.  Values: chunk 8kb+nb of
-// lane (n, j) = slots 32kb+8j..+7 of dim 16nb+n.  Chunk c of lane l sits at byte (c*64 + l)*16 of the tile.
-struct ExactHalf { uint4 c[16]; };
+// ---- exact (fp16 / bf16) units ---------------------------------------------------------------------
+// Unit h of a tile is chunks 8h .. 8h+7 of every lane.  Keys: chunk 8h + 4b + kb of lane (n, j) = dims
+// 32j+8kb..+7 of slot 32h + pair_slot(n) + b.  Values: chunk 8h + m = slots 32h+8j..+7 of dim 16m+n.
+// Chunk c of lane l sits at byte (c*64 + l)*16 of the tile.
+struct ExactUnit { uint4 c[8]; };
 
-__device__ static inline void load_exact_half(ExactHalf& t, const uint16_t* base, int tile, int lane) {
-    const uint8_t* src = reinterpret_cast<const uint8_t*>(base) + (size_t)tile * (TILE * HD * 2);
+__device__ static inline void load_exact_unit(ExactUnit& t, const uint16_t* base, int unit, int lane) {
+    const uint8_t* src = reinterpret_cast<const uint8_t*>(base) + (size_t)(unit >> 1) * (TILE * HD * 2) + (size_t)(unit & 1) * (8 * TILE * 16);
 #pragma unroll
-    for (int c = 0; c < 16; ++c) t.c[c] = stream_load(reinterpret_cast<const uint4*>(src + ((size_t)c * TILE + lane) * 16));
+    for (int c = 0; c < 8; ++c) t.c[c] = stream_load(reinterpret_cast<const uint4*>(src + ((size_t)c * TILE + lane) * 16));
 }
-
-__device__ static inline uint32_t bf16_pair(float a, float b) {
-    return (uint32_t)Elem<ODMKV_BF16>::from_f32(a) | ((uint32_t)Elem<ODMKV_BF16>::from_f32(b) << 16);
-}
-__device__ static inline float bf16_rest(float a) { return a - Elem<ODMKV_BF16>::to_f32(Elem<ODMKV_BF16>::from_f32(a)); }
 
 // BF: the store keeps bf16 rows; they meet the query (bf16 high + low piece of q16, exact) and the
 // softmax weights (bf16 high + low piece) on the bf16 matrix instructions, products exact, sums fp32.
@@ -497,62 +546,75 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
                                               int tid, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
     const int wave = tid >> 6, lane = tid & 63, n = lane & 15, j = lane >> 4;
     const float esc = a.scaling * LOG2E;
+    // the query itself (no rotation): row 2h = q16 of head h, row 2h+1 = zero for fp16 rows; for bf16 rows the two
+    // bf16 pieces of q16 (11 significant bits in two pieces of 8: exact)
     uint4 qraw[4];
-    load_queries(reinterpret_cast<const uint8_t*>(a.qs) + (size_t)bq_first * 2 * QROW, lane, a.G, qraw);
-    const int count = a.s.seg_count[4][bh];          // exact segments grow between work-list rebuilds
-    for (int tt = wave; tt < ntiles; tt += DECODE_NWAVES) {
-        const int nvalid = min(count - (tile0 + tt - seg_first) * TILE, TILE);
-        if (nvalid <= 0) break;
-        ExactHalf k;
-        load_exact_half(k, a.s.kexact, tile0 + tt, lane);
-        f4 dk[4];
+    {
+        const int h = n >> 1, lo = n & 1;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) dk[b] = (f4){0.f, 0.f, 0.f, 0.f};
+        for (int kb = 0; kb < 4; ++kb) {
+            uint32_t w[4] = {0u, 0u, 0u, 0u};
+            if (h < a.G && (BF || !lo)) {
+                float qv[8];
+                load_q8(a.q, a.q_dt, (size_t)(bq_first + h) * HD + 32 * j + 8 * kb, qv);
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    if constexpr (BF) w[e >> 1] = lo ? bf16_pair(bf16_rest(qv[e]), bf16_rest(qv[e + 1])) : bf16_pair(qv[e], qv[e + 1]);
+                    else w[e >> 1] = pack_h2(qv[e], qv[e + 1]);
+                }
+            }
+            qraw[kb] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+    const int count = a.s.seg_count[4][bh] - (tile0 - seg_first) * TILE;     // exact segments grow between work-list rebuilds
+    for (int u = wave; u < 2 * ntiles; u += DECODE_NWAVES) {
+        const int nvalid = min(count - u * UNIT, UNIT);
+        if (nvalid <= 0) break;
+        ExactUnit k;
+        load_exact_unit(k, a.s.kexact, 2 * tile0 + u, lane);
+        f4 dk[2];
+        dk[0] = (f4){0.f, 0.f, 0.f, 0.f};
+        dk[1] = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
+            for (int b = 0; b < 2; ++b) {
                 if constexpr (BF) dk[b] = MFMA_BF16(as_bf8(qraw[kb]), as_bf8(k.c[4 * b + kb]), dk[b]);
                 else dk[b] = MFMA_F16(as_h8(qraw[kb]), as_h8(k.c[4 * b + kb]), dk[b]);
             }
-        ExactHalf v;
-        load_exact_half(v, a.s.vexact, tile0 + tt, lane);
-        float tA[4], tB[4];
+        ExactUnit v;
+        load_exact_unit(v, a.s.vexact, 2 * tile0 + u, lane);
+        float tA[2], tB[2];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const bool ok = 4 * n + b < nvalid;
+        for (int b = 0; b < 2; ++b) {
+            const bool ok = pair_slot(n) + b < nvalid;
             tA[b] = ok ? (dk[b][0] + dk[b][1]) * esc : -INFINITY;
             tB[b] = ok ? (dk[b][2] + dk[b][3]) * esc : -INFINITY;
         }
-        float pA[4], pB[4];
-        softmax_tile(st, tA, tB, lane, alpha_sh, pA, pB);
+        float pA[2], pB[2];
+        softmax_unit(st, tA, tB, lane, alpha_sh, pA, pB);
         if constexpr (BF) {
             // p = hi + lo in bf16: two p buffers, two products
-            *reinterpret_cast<uint2*>(pbuf + (2 * j) * PROW + 8 * n) = make_uint2(bf16_pair(pA[0], pA[1]), bf16_pair(pA[2], pA[3]));
-            *reinterpret_cast<uint2*>(pbuf + (2 * j + 1) * PROW + 8 * n) = make_uint2(bf16_pair(pB[0], pB[1]), bf16_pair(pB[2], pB[3]));
-            *reinterpret_cast<uint2*>(pbuf + PBUF + (2 * j) * PROW + 8 * n) =
-                make_uint2(bf16_pair(bf16_rest(pA[0]), bf16_rest(pA[1])), bf16_pair(bf16_rest(pA[2]), bf16_rest(pA[3])));
-            *reinterpret_cast<uint2*>(pbuf + PBUF + (2 * j + 1) * PROW + 8 * n) =
-                make_uint2(bf16_pair(bf16_rest(pB[0]), bf16_rest(pB[1])), bf16_pair(bf16_rest(pB[2]), bf16_rest(pB[3])));
+            *reinterpret_cast<uint32_t*>(pbuf + (2 * j) * PROW + 4 * n) = bf16_pair(pA[0], pA[1]);
+            *reinterpret_cast<uint32_t*>(pbuf + (2 * j + 1) * PROW + 4 * n) = bf16_pair(pB[0], pB[1]);
+            *reinterpret_cast<uint32_t*>(pbuf + PBUF + (2 * j) * PROW + 4 * n) = bf16_pair(bf16_rest(pA[0]), bf16_rest(pA[1]));
+            *reinterpret_cast<uint32_t*>(pbuf + PBUF + (2 * j + 1) * PROW + 4 * n) = bf16_pair(bf16_rest(pB[0]), bf16_rest(pB[1]));
         } else {
-            *reinterpret_cast<uint2*>(pbuf + (2 * j) * PROW + 8 * n) = make_uint2(pack_h2(pA[0], pA[1]), pack_h2(pA[2], pA[3]));
-            *reinterpret_cast<uint2*>(pbuf + (2 * j + 1) * PROW + 8 * n) = make_uint2(pack_h2(pB[0], pB[1]), pack_h2(pB[2], pB[3]));
+            *reinterpret_cast<uint32_t*>(pbuf + (2 * j) * PROW + 4 * n) = pack_h2(pA[0], pA[1]);
+            *reinterpret_cast<uint32_t*>(pbuf + (2 * j + 1) * PROW + 4 * n) = pack_h2(pB[0], pB[1]);
         }
         wave_lds_fence();
+        const uint4 phi = *reinterpret_cast<const uint4*>(pbuf + (n & 7) * PROW + 16 * j);
+        if constexpr (BF) {
+            const uint4 plo = *reinterpret_cast<const uint4*>(pbuf + PBUF + (n & 7) * PROW + 16 * j);
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            const uint4 phi = *reinterpret_cast<const uint4*>(pbuf + (n & 7) * PROW + (32 * kb + 8 * j) * 2);
-            if constexpr (BF) {
-                const uint4 plo = *reinterpret_cast<const uint4*>(pbuf + PBUF + (n & 7) * PROW + (32 * kb + 8 * j) * 2);
-#pragma unroll
-                for (int nb = 0; nb < 8; ++nb) {
-                    st.acc[nb] = MFMA_BF16(as_bf8(phi), as_bf8(v.c[8 * kb + nb]), st.acc[nb]);
-                    st.acc[nb] = MFMA_BF16(as_bf8(plo), as_bf8(v.c[8 * kb + nb]), st.acc[nb]);
-                }
-            } else {
-#pragma unroll
-                for (int nb = 0; nb < 8; ++nb) st.acc[nb] = MFMA_F16(as_h8(phi), as_h8(v.c[8 * kb + nb]), st.acc[nb]);
+            for (int m = 0; m < 8; ++m) {
+                st.acc[m] = MFMA_BF16(as_bf8(phi), as_bf8(v.c[m]), st.acc[m]);
+                st.acc[m] = MFMA_BF16(as_bf8(plo), as_bf8(v.c[m]), st.acc[m]);
             }
+        } else {
+#pragma unroll
+            for (int m = 0; m < 8; ++m) st.acc[m] = MFMA_F16(as_h8(phi), as_h8(v.c[m]), st.acc[m]);
         }
         wave_lds_fence();
     }
@@ -570,13 +632,24 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
     float* alphas = reinterpret_cast<float*>(smem + LDS_SCALARS);      // [NWAVES][8]
     float* wm = alphas + DECODE_NWAVES * 8;                            // [NWAVES][8]
     float* wl = wm + DECODE_NWAVES * 8;                                // [NWAVES][8]
+    float* wf = wl + DECODE_NWAVES * 8;                                // [NWAVES][8]
+    float* wM = wf + DECODE_NWAVES * 8;                                // [8]
 
-    const int item = ORDERED ? a.order[blockIdx.x] : (int)blockIdx.x;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    // this thread's share of Pi_k^T for the query rotation: the same for every item, requested first
+    f4 pk[ROT_TERMS];
+#pragma unroll
+    for (int t = 0; t < ROT_TERMS; ++t)
+        pk[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
+    const int item = ORDERED ? a.order[blockIdx.x] : (int)blockIdx.x;
     const int4 d0 = reinterpret_cast<const int4*>(a.items)[2 * item];       // bh, level, first tile, tiles
     const int4 d1 = reinterpret_cast<const int4*>(a.items)[2 * item + 1];   // tokens, first tile of the segment
     const int bh = d0.x, li = d0.y, tile0 = d0.z, ntiles = d0.w;
     const int bq_first = (bh / a.s.Hkv) * a.Hq + (bh % a.s.Hkv) * a.G;      // first query head of the group
+
+    // where this item's result goes: fetched now, not when the workgroup is about to finish
+    float* dst = a.partial + (size_t)item * GP * PSTRIDE;
+    asm volatile("" : "+s"(dst));
 
     WaveState st;
     st.mA = -INFINITY; st.mB = -INFINITY; st.lA = 0.0f; st.lB = 0.0f;
@@ -585,10 +658,10 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
     uint8_t* pbuf = smem + LDS_PBUFS + wave * 2 * PBUF;
     float* alpha_sh = alphas + wave * 8;
     switch (li) {
-        case 0: run_quant_level<2>(a, 0, bq_first, tile0, ntiles, d1.x, tid, lut, pbuf, alpha_sh, st); break;
-        case 1: run_quant_level<3>(a, 1, bq_first, tile0, ntiles, d1.x, tid, lut, pbuf, alpha_sh, st); break;
-        case 2: run_quant_level<4>(a, 2, bq_first, tile0, ntiles, d1.x, tid, lut, pbuf, alpha_sh, st); break;
-        case 3: run_quant_level<8>(a, 3, bq_first, tile0, ntiles, d1.x, tid, lut, pbuf, alpha_sh, st); break;
+        case 0: run_quant_level<2, GP>(a, 0, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
+        case 1: run_quant_level<3, GP>(a, 1, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
+        case 2: run_quant_level<4, GP>(a, 2, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
+        case 3: run_quant_level<8, GP>(a, 3, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
         default:
             if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
             else run_exact_level<false>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
@@ -596,14 +669,24 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
     }
 
     // ---- combine the wavefronts (the table is no longer needed) ----
+    // Every wavefront publishes its maxima; after the barrier it takes the maximum over all wavefronts (lane n of a
+    // row reads wavefront n's value), derives its own factor exp2(m - M) and publishes the factor, its scaled share of
+    // the normaliser and its accumulators as they are.  After a second barrier one thread per (head, dim) forms the
+    // weighted sum over the wavefronts.
+    const int n = lane & 15, j = lane >> 4;
+    const float lsA = row_sum(st.lA), lsB = row_sum(st.lB);
+    if (n == 0) { wm[wave * 8 + 2 * j] = st.mA; wm[wave * 8 + 2 * j + 1] = st.mB; }
     __syncthreads();
     float* wacc = reinterpret_cast<float*>(lut);          // [NWAVES][128 dims][GP heads]
     {
-        const int n = lane & 15, j = lane >> 4;
-        const float lsA = row_sum(st.lA), lsB = row_sum(st.lB);
+        float MA = n < DECODE_NWAVES ? wm[n * 8 + 2 * j] : -INFINITY, MB = n < DECODE_NWAVES ? wm[n * 8 + 2 * j + 1] : -INFINITY;
+        row_max2(MA, MB);
+        const float fA = st.mA > -INFINITY ? __builtin_amdgcn_exp2f(st.mA - MA) : 0.0f;
+        const float fB = st.mB > -INFINITY ? __builtin_amdgcn_exp2f(st.mB - MB) : 0.0f;
         if (n == 0 && 2 * j < GP) {
-            wm[wave * 8 + 2 * j] = st.mA; wm[wave * 8 + 2 * j + 1] = st.mB;
-            wl[wave * 8 + 2 * j] = lsA; wl[wave * 8 + 2 * j + 1] = lsB;
+            wf[wave * 8 + 2 * j] = fA; wf[wave * 8 + 2 * j + 1] = fB;
+            wl[wave * 8 + 2 * j] = lsA * fA; wl[wave * 8 + 2 * j + 1] = lsB * fB;
+            if (wave == 0) { wM[2 * j] = MA; wM[2 * j + 1] = MB; }
         }
         if (4 * j < GP) {
 #pragma unroll
@@ -611,23 +694,20 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
         }
     }
     __syncthreads();
-    float* dst = a.partial + (size_t)item * GP * PSTRIDE;
     for (int e = tid; e < GP * HD; e += DECODE_NWAVES * 64) {
-        const int g = e / HD, dim = e % HD;
-        float M = wm[g];
+        const int g = e % GP, dim = e / GP;               // consecutive threads walk consecutive LDS words
+        float s = 0.0f;
 #pragma unroll
-        for (int w = 1; w < DECODE_NWAVES; ++w) M = fmaxf(M, wm[w * 8 + g]);
-        float s = 0.0f, L = 0.0f;
-        if (M > -INFINITY) {
-#pragma unroll
-            for (int w = 0; w < DECODE_NWAVES; ++w) {
-                const float f = __builtin_amdgcn_exp2f(wm[w * 8 + g] - M);
-                s = __fmaf_rn(wacc[(w * HD + dim) * GP + g], f, s);
-                L = __fmaf_rn(wl[w * 8 + g], f, L);
-            }
-        }
+        for (int w = 0; w < DECODE_NWAVES; ++w) s = __fmaf_rn(wacc[w * HD * GP + e], wf[w * 8 + g], s);
         dst[g * PSTRIDE + dim] = s;
-        if (dim == 0) { dst[g * PSTRIDE + HD] = M; dst[g * PSTRIDE + HD + 1] = L; }
+    }
+    if (tid >= DECODE_NWAVES * 64 - GP) {                 // the last wavefront has the least to do above
+        const int g = tid - (DECODE_NWAVES * 64 - GP);
+        float L = 0.0f;
+#pragma unroll
+        for (int w = 0; w < DECODE_NWAVES; ++w) L += wl[w * 8 + g];
+        dst[g * PSTRIDE + HD] = wM[g];
+        dst[g * PSTRIDE + HD + 1] = L;
     }
 }
 
@@ -766,7 +846,7 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
         if (a.out_dt == ODMKV_F32) reinterpret_cast<float*>(a.out)[oi] = o32;
         else if (a.out_dt == ODMKV_F16) reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_F16>::from_f32(o32);
         else reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_BF16>::from_f32(o32);
-        if (a.lse && tid == 0 && quarter == 0) a.lse[bq] = L > 0.0f ? (M + __log2f(L)) * LN2 : -INFINITY;
+        if (a.lse && tid == 0 && quarter == 0) a.lse[bq] = L > 0.0f ? (M + __log2f(L) - P_SHIFT) * LN2 : -INFINITY;
     }
 }
 
@@ -777,8 +857,7 @@ static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
 
 extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     if (B <= 0 || Hq <= 0 || n_items < 0) return 0;
-    const size_t q = align_up((size_t)B * Hq * 2 * QROW, 256);
-    return 2 * q + align_up((size_t)n_items * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
+    return align_up((size_t)(n_items > 0 ? n_items : 1) * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
 }
 
 template <int GP, bool ORDERED>
@@ -799,6 +878,7 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     ODMKV_CHECK_ARG(codebooks_host != nullptr, "decode_attn: null host copy of the centroid tables");
     ODMKV_CHECK_ARG(inv_scales != nullptr, "decode_attn: null table scales");
     ODMKV_CHECK_ARG(q && store && work && pi_k_t && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
+    ODMKV_CHECK_ARG(((uintptr_t)q & 15) == 0, "decode_attn: the query must be 16-byte aligned");
     const int n_items = work->n_items;
     ODMKV_CHECK_ARG(n_items >= 0, "decode_attn: negative item count");
     ODMKV_CHECK_ARG(work->item_range, "decode_attn: null item ranges");
@@ -819,15 +899,8 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     a.pi_k_t = pi_k_t; a.pi_v = pi_v; a.cb = codebooks;
     for (int w = 0; w < 4; ++w) a.inv_s[w] = inv_scales[w];
     for (int k = 0; k < 28; ++k) a.cbs[k] = codebooks_host[k];
-    const size_t qbytes = align_up((size_t)B * Hq * 2 * QROW, 256);
-    a.qrot = (uint4*)workspace;
-    a.qs = (uint4*)((char*)workspace + qbytes);
-    a.partial = (float*)((char*)workspace + 2 * qbytes);
+    a.partial = (float*)workspace;
     a.out = out; a.lse = lse;
-    if (stage_mask & 1) {
-        hipLaunchKernelGGL(decode_prep_kernel, dim3(B * Hq * PREP_SPLIT), dim3(PREP_THREADS), 0, st, a);
-        ODMKV_CHECK_LAUNCH("decode_prep_kernel");
-    }
     const int GP = group_pad(G);
     a.gp = GP;
     if (n_items > 0 && (stage_mask & 2)) {

@@ -338,7 +338,7 @@ __device__ static __forceinline__ void stage_direct_k(const f32x32& a0, const f3
     }
 }
 
-// lane (n, j) gathers dims 32j..32j+31 of slots 4n..4n+3 from the staged token streams
+// lane (n, j) gathers dims 32j..32j+31 of its four slots key_slot(n, 0..3) from the staged token streams
 template <int W>
 __device__ static __forceinline__ void store_direct_k(const uint8_t* stage, uint8_t* kcodes, int tile, int lane) {
     const int n = lane & 15, j = lane >> 4;
@@ -347,7 +347,7 @@ __device__ static __forceinline__ void store_direct_k(const uint8_t* stage, uint
     for (int b = 0; b < 4; ++b)
 #pragma unroll
         for (int i = 0; i < W; ++i)
-            words[b * W + i] = *reinterpret_cast<const uint32_t*>(stage + (4 * n + b) * Direct<W>::ROW_K + 4 * W * j + 4 * i);
+            words[b * W + i] = *reinterpret_cast<const uint32_t*>(stage + key_slot(n, b) * Direct<W>::ROW_K + 4 * W * j + 4 * i);
     uint8_t* dst = kcodes + (size_t)tile * (TILE * 16 * W);
 #pragma unroll
     for (int ch = 0; ch < W; ++ch)
@@ -402,8 +402,8 @@ __device__ static __forceinline__ void pack_store_k(const uint8_t* stage, uint8_
     for (int k = 0; k < 4 * W; ++k) words[k] = 0;
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-        const uint4 v0 = *reinterpret_cast<const uint4*>(stage + (4 * n + b) * CODE_ROW + 32 * j);
-        const uint4 v1 = *reinterpret_cast<const uint4*>(stage + (4 * n + b) * CODE_ROW + 32 * j + 16);
+        const uint4 v0 = *reinterpret_cast<const uint4*>(stage + key_slot(n, b) * CODE_ROW + 32 * j);
+        const uint4 v1 = *reinterpret_cast<const uint4*>(stage + key_slot(n, b) * CODE_ROW + 32 * j + 16);
         const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
         for (int e = 0; e < 32; ++e) put_code<W>(words, 32 * b + e, (w[e >> 2] >> (8 * (e & 3))) & 0xffu);
@@ -417,7 +417,7 @@ __device__ static __forceinline__ void pack_store_k(const uint8_t* stage, uint8_
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int b = (4 * c + i) / W;
-                if (4 * n + b < lo) words[4 * c + i] = o[i];
+                if (key_slot(n, b) < lo) words[4 * c + i] = o[i];
             }
         }
     }
@@ -1008,7 +1008,7 @@ __global__ __launch_bounds__(DQ_NW * 64) void dequant_kernel(DequantArgs a, int 
                     for (int i = 0; i < 32; i += 4) {
                         const uint32_t w4 = get_code<W>(words, 32 * b + i) | (get_code<W>(words, 32 * b + i + 1) << 8) |
                                             (get_code<W>(words, 32 * b + i + 2) << 16) | (get_code<W>(words, 32 * b + i + 3) << 24);
-                        *reinterpret_cast<uint32_t*>(&codes[(4 * n + b) * CODE_ROW + 32 * j + i]) = w4;
+                        *reinterpret_cast<uint32_t*>(&codes[key_slot(n, b) * CODE_ROW + 32 * j + i]) = w4;
                     }
             } else {
 #pragma unroll

@@ -20,13 +20,19 @@ __device__ static inline void put_code(uint32_t* w, int i, uint32_t c) {
 // ---- tile layouts (see include/odmkv.h) ----------------------------------------------------------
 // Every tile buffer is W (codes) or 16 (exact rows) chunks of 16 bytes per lane; chunk c of lane l sits
 // at byte (c*64 + l)*16 of the tile.  Lane l = 16j + n.
-//   key codes:    the lane's 128 codes are  code 32b + i   = dim 32j + i   of slot 4n + b
+//   key codes:    the lane's 128 codes are  code 32b + i   = dim 32j + i   of slot key_slot(n, b)
 //   value codes:  the lane's 128 codes are  code 64k + 8m + e = slot 32k + 8j + e  of dim 16m + n
-//   exact keys:   chunk 4b + k of the lane  = dims 32j + 8k .. + 7 of slot 4n + b
+//   exact keys:   chunk 4b + k of the lane  = dims 32j + 8k .. + 7 of slot key_slot(n, b)
 //   exact values: chunk 8k + m of the lane  = slots 32k + 8j .. + 7 of dim 16m + n
+// Both halves of a lane's code bytes (and chunks 0-7 / 8-15 of its exact rows) belong to the same 32 slots,
+// 32h .. 32h + 31: half a tile is a unit of work of its own.
+// slot of key block b (0..3), column n (0..15): the two blocks of a half interleave, so that a lane's two
+// softmax weights of a half sit next to each other in slot order
+__host__ __device__ static inline int key_slot(int n, int b) { return 32 * (b >> 1) + 8 * (n >> 2) + 2 * (n & 3) + (b & 1); }
 // index (in 16-bit elements) of element (slot, dim) inside an exact tile
 __host__ __device__ static inline int exact_k_index(int slot, int dim) {
-    const int n = slot >> 2, b = slot & 3, j = dim >> 5, k = (dim >> 3) & 3, e = dim & 7;
+    const int b = 2 * (slot >> 5) + (slot & 1), n = 4 * ((slot >> 3) & 3) + ((slot >> 1) & 3);
+    const int j = dim >> 5, k = (dim >> 3) & 3, e = dim & 7;
     return (((4 * b + k) * TILE) + 16 * j + n) * 8 + e;
 }
 __host__ __device__ static inline int exact_v_index(int slot, int dim) {

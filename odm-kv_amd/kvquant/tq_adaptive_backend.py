@@ -36,7 +36,8 @@ def _exact_index_tables():
     (the layouts of include/odmkv.h)."""
     slot = np.arange(TILE)[:, None]
     dim = np.arange(HEAD_DIM)[None, :]
-    k_idx = (((4 * (slot & 3) + ((dim >> 3) & 3)) * TILE) + 16 * (dim >> 5) + (slot >> 2)) * 8 + (dim & 7)
+    kb, kn = 2 * (slot >> 5) + (slot & 1), 4 * ((slot >> 3) & 3) + ((slot >> 1) & 3)      # key block and column of the slot
+    k_idx = (((4 * kb + ((dim >> 3) & 3)) * TILE) + 16 * (dim >> 5) + kn) * 8 + (dim & 7)
     v_idx = (((8 * (slot >> 5) + (dim >> 4)) * TILE) + 16 * ((slot >> 3) & 3) + (dim & 15)) * 8 + (slot & 7)
     return k_idx.astype(np.int64), v_idx.astype(np.int64)
 
@@ -421,9 +422,11 @@ class TurboQuantAdaptiveKVCacheState:
             self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
             1 if include_exact else 0, _lib.stream_ptr(self.device)))
 
-    def materialize(self) -> tuple[torch.Tensor, torch.Tensor]:
+    def materialize(self, dtype: torch.dtype | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+        """Dense (keys, values) of the whole store in the state's dtype, as the reference returns them; `dtype`
+        (an addition) asks for another one: float32 keeps the dequantised values unrounded."""
         keys = torch.zeros(self.batch_size, self.num_heads, self.seq_len, self.head_dim,
-                           device=self.device, dtype=self.dtype)
+                           device=self.device, dtype=self.dtype if dtype is None else dtype)
         values = torch.zeros_like(keys)
         self._dequant_into(keys, values, True)
         return keys, values

@@ -4,6 +4,8 @@ import numpy as np
 
 TILE, HD = 64, 128
 WIDTHS = (2, 3, 4, 8)
+# slot of key block b (0..3), column n (0..15) of a tile: [n, b]
+KEY_SLOT = np.array([[32 * (b >> 1) + 8 * (n >> 2) + 2 * (n & 3) + (b & 1) for b in range(4)] for n in range(16)])
 
 
 def _bits_to_codes(byte_rows: np.ndarray, w: int) -> np.ndarray:
@@ -24,9 +26,10 @@ def decode_level(state, li: int):
     w = WIDTHS[li]
     b = state._bufs
     nt = int(state._seg_tile[li, -1])
-    # keys: lane 16j+n, code 32b+i = dim 32j+i of slot 4n+b
+    # keys: lane 16j+n, code 32b+i = dim 32j+i of slot key_slot(n, b)
     ks = _lane_streams(b["kcodes"][li].cpu().numpy(), nt, w).reshape(nt, 4, 16, 4, 32)        # [t, j, n, b, i]
-    kcodes = ks.transpose(0, 2, 3, 1, 4).reshape(nt, TILE, HD)                                # [t, slot=4n+b, dim=32j+i]
+    kcodes = np.empty((nt, TILE, HD), np.uint8)
+    kcodes[:, KEY_SLOT.reshape(-1)] = ks.transpose(0, 2, 3, 1, 4).reshape(nt, TILE, HD)       # rows (n, b) -> their slots
     # values: lane 16j+n, code 64k+8m+e = slot 32k+8j+e of dim 16m+n
     vs = _lane_streams(b["vcodes"][li].cpu().numpy(), nt, w).reshape(nt, 4, 16, 2, 8, 8)      # [t, j, n, k, m, e]
     vcodes = vs.transpose(0, 3, 1, 5, 4, 2).reshape(nt, TILE, HD)                             # [t, slot=32k+8j+e, dim=16m+n]
@@ -50,8 +53,9 @@ def decode_exact(state):
     nt = int(state._seg_tile[4, -1])
     ke = b["kexact"].view(-1).cpu().view(dtype=__import__("torch").int16).numpy()[: nt * TILE * HD]
     ve = b["vexact"].view(-1).cpu().view(dtype=__import__("torch").int16).numpy()[: nt * TILE * HD]
-    # keys: chunk 4b+k of lane 16j+n = dims 32j+8k..+7 of slot 4n+b
-    krows = ke.reshape(nt, 4, 4, 4, 16, 8).transpose(0, 4, 1, 3, 2, 5).reshape(nt, TILE, HD)  # [t,b,k,j,n,e] -> [t, n, b, j, k, e]
+    # keys: chunk 4b+k of lane 16j+n = dims 32j+8k..+7 of slot key_slot(n, b)
+    krows = np.empty((nt, TILE, HD), ke.dtype)
+    krows[:, KEY_SLOT.reshape(-1)] = ke.reshape(nt, 4, 4, 4, 16, 8).transpose(0, 4, 1, 3, 2, 5).reshape(nt, TILE, HD)  # [t,b,k,j,n,e] -> [t, (n, b), (j, k, e)]
     # values: chunk 8k+m of lane 16j+n = slots 32k+8j..+7 of dim 16m+n
     vrows = ve.reshape(nt, 2, 8, 4, 16, 8).transpose(0, 1, 3, 5, 2, 4).reshape(nt, TILE, HD)  # [t,k,m,j,n,e] -> [t, k, j, e, m, n]
     pos = b["pos"][4].cpu().numpy()[: nt * TILE].reshape(nt, TILE)
