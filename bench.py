@@ -443,23 +443,37 @@ def main() -> int:
     # ---- compress every layer: score -> allocate -> window -> pack (timed per layer) ----
     states, qs, t_stage = [], [], {"score": [], "alloc": [], "pack": [], "total": []}
     dense0 = None
-    for li in range(NL):
-        k, v, mu, q = make_layer(li, n_kv, n_q, T, dev)
-        for rep in range(2 if li == 0 else 1):               # the first pass also warms allocators
-            st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=dev, dtype=torch.float16, key_quantizer="mse",
-                                                value_quantizer="mse", seed=42 + 7 * li)
-            ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
-            torch.cuda.synchronize()
+
+    def compress(k, v, mu, seed, ev=None):
+        st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=dev, dtype=torch.float16, key_quantizer="mse",
+                                            value_quantizer="mse", seed=seed)
+        if ev:
             ev[0].record()
-            s = _launch_score(k, v, mu, None, n_q, 4, 1e-2)
+        s = _launch_score(k, v, mu, None, n_q, 4, 1e-2)
+        if ev:
             ev[1].record()
-            bits = optimal_scores_to_bits_batched(s.reshape(1, -1), LEVELS, [args.target], eps, n_sink=4, period=T,
-                                                  eviction_cost=0.5).reshape(n_kv, T)
-            bits[:, -128:] = 16
+        bits = optimal_scores_to_bits_batched(s.reshape(1, -1), LEVELS, [args.target], eps, n_sink=4, period=T,
+                                              eviction_cost=0.5).reshape(n_kv, T)
+        bits[:, -128:] = 16
+        if ev:
             ev[2].record()
-            st.prefill(k[None], v[None], bits[None])
+        st.prefill(k[None], v[None], bits[None])
+        if ev:
             ev[3].record()
-            torch.cuda.synchronize()
+        return st, bits
+
+    warm = None
+    for li in range(NL):
+        k, v, mu, q = make_layer(li, n_kv, n_q, T, dev)        # about a second of CPU work: the GPU idles meanwhile
+        # an untimed pass over OTHER data first (the previous layer's; for the first layer its own, which also warms
+        # the allocators): the device is busy and at its clocks again when the timed pass starts, and the timed
+        # pass still reads keys and values that no kernel has touched
+        compress(*(warm if warm is not None else (k, v, mu)), seed=41)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        torch.cuda.synchronize()
+        st, bits = compress(k, v, mu, 42 + 7 * li, ev)
+        torch.cuda.synchronize()
+        warm = (k, v, mu)
         # device events on the launch stream, no host synchronisation between the stages (the pack
         # stage's own read-back of the level counts is inside its interval)
         t_stage["score"].append(ev[0].elapsed_time(ev[1]) * 1e-3)

@@ -132,7 +132,7 @@ __device__ static inline void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt
 //   W = 2: index = byte (4 codes) -> 4 halfs (8 bytes),  row = 256 bytes
 //   W = 3: index = 6 bits (2 codes) -> 2 halfs (4 bytes), row = 128 bytes
 //   W = 4: index = byte (2 codes) -> 2 halfs,             row = 128 bytes
-//   W = 8: index = byte (1 code)  -> the half in both halves of a dword, row = 128 bytes
+//   W = 8: index = byte (1 code)  -> the centroid's fp16 high half (low word) and low half (high word), row = 128 bytes
 // ------------------------------------------------------------------------------------------------
 // pick table[idx] from a table that lives in scalar registers (no memory access: every workgroup
 // of a launch would otherwise hammer the same cache line)
@@ -172,7 +172,13 @@ __device__ static inline void build_lut(uint8_t* lut, const DecodeArgs& a, int t
         uint32_t v;
         if constexpr (W == 3) { v = half_bits(pick<8>(a.cbs + 4, tid & 7)) | (half_bits(pick<8>(a.cbs + 4, (tid >> 3) & 7)) << 16); }
         else if constexpr (W == 4) { v = half_bits(pick<16>(a.cbs + 12, tid & 15)) | (half_bits(pick<16>(a.cbs + 12, (tid >> 4) & 15)) << 16); }
-        else { v = half_bits(a.cb[codebook_offset(3) + (tid & 255)]) * 0x10001u; }
+        else {
+            // the 256-entry table does not round well to fp16 as a whole (no common scale suits 128 magnitudes): an
+            // entry keeps the centroid's high half and, in its upper 16 bits, the low half
+            const float c = a.cb[codebook_offset(3) + (tid & 255)];
+            const __half hi = __float2half_rn(c);
+            v = (uint32_t)__half_as_ushort(hi) | (half_bits(c - __half2float(hi)) << 16);
+        }
         const bool on = wave < 4 && (W != 3 || wave == 0);  // 256 entries (64 for the 3-bit table): four wavefronts' worth
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -205,7 +211,7 @@ __device__ static inline h4 lut4(const uint32_t* w, int s, const uint8_t* lut, u
         const uint32_t t1 = *reinterpret_cast<const uint32_t*>(lut + (((x >> 8) & 0xffu) << 7) + slot4);
         const uint32_t t2 = *reinterpret_cast<const uint32_t*>(lut + (((x >> 16) & 0xffu) << 7) + slot4);
         const uint32_t t3 = *reinterpret_cast<const uint32_t*>(lut + ((x >> 24) << 7) + slot4);
-        return as_h4((t0 & 0xffffu) | (t1 & 0xffff0000u), (t2 & 0xffffu) | (t3 & 0xffff0000u));
+        return as_h4(__builtin_amdgcn_perm(t1, t0, 0x05040100u), __builtin_amdgcn_perm(t3, t2, 0x05040100u));     // the high halves
     } else {
         const int bit = 12 * s, k = bit >> 5, sh = bit & 31;
         uint32_t x = w[k] >> sh;
@@ -214,6 +220,23 @@ __device__ static inline h4 lut4(const uint32_t* w, int s, const uint8_t* lut, u
         const uint32_t hi = *reinterpret_cast<const uint32_t*>(lut + (((x >> 6) & 63u) << 7) + slot4);
         return as_h4(lo, hi);
     }
+}
+// 8-bit codes 8g..8g+7: the high halves and the low halves of the centroids, two matrix operands
+__device__ static inline void lut8_split(const uint32_t* w, int g, const uint8_t* lut, uint32_t slot4, h8& hi, h8& lo) {
+    uint32_t t[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t x = w[2 * g + (e >> 2)] >> (8 * (e & 3));
+        t[e] = *reinterpret_cast<const uint32_t*>(lut + ((x & 0xffu) << 7) + slot4);
+    }
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        h[e] = __builtin_amdgcn_perm(t[2 * e + 1], t[2 * e], 0x05040100u);       // low words of the two entries
+        l[e] = __builtin_amdgcn_perm(t[2 * e + 1], t[2 * e], 0x07060302u);       // high words
+    }
+    hi = join(as_h4(h[0], h[1]), as_h4(h[2], h[3]));
+    lo = join(as_h4(l[0], l[1]), as_h4(l[2], l[3]));
 }
 // centroids of codes 8g..8g+7 of the stream: one matrix operand
 template <int W>
@@ -385,7 +408,16 @@ __device__ static inline void compute_unit(const Unit<W>& t, int nvalid, int lan
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int b = 0; b < 2; ++b) dk[b] = MFMA_F16(qa[kb], lut8<W>(t.kw, 4 * b + kb, lut, slot4), dk[b]);
+        for (int b = 0; b < 2; ++b) {
+            if constexpr (W == 8) {
+                h8 chi, clo;
+                lut8_split(t.kw, 4 * b + kb, lut, slot4, chi, clo);
+                dk[b] = MFMA_F16(qa[kb], chi, dk[b]);
+                dk[b] = MFMA_F16(qa[kb], clo, dk[b]);
+            } else {
+                dk[b] = MFMA_F16(qa[kb], lut8<W>(t.kw, 4 * b + kb, lut, slot4), dk[b]);
+            }
+        }
     float tA[2], tB[2];
     {
         const float kn0 = t.kn.x * ksc, kn1 = t.kn.y * ksc;
@@ -413,7 +445,16 @@ __device__ static inline void compute_unit(const Unit<W>& t, int nvalid, int lan
     // ---- values: D[head][dim], eight dim blocks ----
     const h8 pa = as_h8(*reinterpret_cast<const uint4*>(pbuf + (n & 7) * PROW + 16 * j));
 #pragma unroll
-    for (int m = 0; m < 8; ++m) st.acc[m] = MFMA_F16(pa, lut8<W>(t.vw, m, lut, slot4), st.acc[m]);
+    for (int m = 0; m < 8; ++m) {
+        if constexpr (W == 8) {
+            h8 chi, clo;
+            lut8_split(t.vw, m, lut, slot4, chi, clo);
+            st.acc[m] = MFMA_F16(pa, chi, st.acc[m]);
+            st.acc[m] = MFMA_F16(pa, clo, st.acc[m]);
+        } else {
+            st.acc[m] = MFMA_F16(pa, lut8<W>(t.vw, m, lut, slot4), st.acc[m]);
+        }
+    }
     wave_lds_fence();                                      // the p buffer is free for the next unit
 }
 

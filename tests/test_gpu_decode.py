@@ -238,6 +238,31 @@ def test_decode_error_is_mostly_the_dense_cache_rounding():
     assert e32 < 5e-4 and e32 < e16 and e32 < oracle_gap, (e16, e32, oracle_gap)
 
 
+@pytest.mark.parametrize("mix", ["all-8-bit", "half-8-bit"])
+def test_eight_bit_tokens_keep_the_margin(mix):
+    """The 256-entry table cannot be scaled so that all its entries round well to fp16 (up to 3.4e-4 relative per
+    entry): the kernel keeps each entry as an fp16 high + low pair.  Against the oracle that materialises in fp32
+    the worst head of stores that are all or half 8-bit stays within 5e-4, half the stated tolerance, like the
+    other widths (what remains is the fp16 rounding of the softmax weights)."""
+    worst = 0.0
+    for seed in range(4):
+        g = torch.Generator().manual_seed(900 + seed)
+        B, H, G, T = 1, 4, 4, 2048
+        k = torch.randn(B, H, T, 128, generator=g).half()
+        v = torch.randn(B, H, T, 128, generator=g).half()
+        bits = torch.full((B, H, T), 8, dtype=torch.int32)
+        if mix == "half-8-bit":
+            bits[torch.rand(B, H, T, generator=g) < 0.5] = 2
+        st, ref16 = _pair(k, v, bits)
+        ref32 = KVState(128, (0, 2, 3, 4, 8, 16), dtype=torch.float32, seed=42, order="canonical")
+        ref32.prefill(k.float(), v.float(), bits)
+        q = torch.randn(B, H * G, 128, generator=g).half()
+        got = st.decode_attention(q.to(DEV)).cpu()
+        assert rel_err(got, decode_attention_state(q.float(), ref16)) < ATTN_RTOL
+        worst = max(worst, rel_err(got, decode_attention_state(q.float(), ref32)))
+    assert worst < 5e-4, worst
+
+
 @pytest.mark.parametrize("G", [5, 8])
 def test_large_group_with_more_items_than_compute_units(G):
     """A GQA group of more than four heads is served by the two halves of each workgroup; with more work items
