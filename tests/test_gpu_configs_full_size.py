@@ -110,10 +110,14 @@ def test_c4_long_context_heavy_eviction():
     _check_attention(st, [L], 4)
     # 128 decode steps keep new tokens exact and visible
     g = torch.Generator().manual_seed(9)
-    for step in range(3):
-        kn = torch.randn(1, 8, 1, 128, generator=g).half().to(DEV)
-        st.append_all_exact(kn, torch.randn(1, 8, 1, 128, generator=g).half().to(DEV))
-    assert st.seq_len == 131072 + 3
+    new_k = torch.randn(128, 1, 8, 1, 128, generator=g).half().to(DEV)
+    new_v = torch.randn(128, 1, 8, 1, 128, generator=g).half().to(DEV)
+    for step in range(128):
+        st.append_all_exact(new_k[step], new_v[step])
+        if step in (0, 63):                              # attention stays right while the exact segment grows
+            _check_attention(st, [L], 4)
+    assert st.seq_len == 131072 + 128
+    assert (st._level_map[0, :, 131072:] == 16).all()
     _check_attention(st, [L], 4)
 
 
@@ -130,6 +134,20 @@ def test_c5_group_of_seven_heavy_tailed_values():
     assert len(used) >= 4, used                          # a 3-bit budget on heavy tails spreads over the levels
     _check_levels(st, stored)
     _check_attention(st, [L], 7)
+
+
+def test_c2_one_layer_pack_and_decode_at_full_size():
+    L = synthetic.config("c2", layer=5)
+    st, bits, stored, scores = _compress([L], [2.0])
+    n_active = 8 * (32768 - 4)
+    assert abs(bits[0, :, 4:].sum().item() - 2.0 * n_active) <= 8
+    assert (bits[0, :, :4] == 16).all()
+    sink = torch.zeros(8, 32768, dtype=torch.bool)
+    sink[:, :4] = True
+    want = oal.optimal_scores_to_bits(scores[0].cpu(), LEVELS, 2.0, EPS, sink, eviction_cost=0.5)
+    assert torch.equal(bits[0].cpu(), want)
+    _check_levels(st, stored)
+    _check_attention(st, [L], 4)
 
 
 def test_c2_one_layer_score_matches_oracle_at_full_size():
