@@ -293,6 +293,10 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--read-ceiling", action="store_true",
                     help="time a plain streaming read kernel at the decode kernel's launch sizes (cold buffers) and exit")
+    ap.add_argument("--decode-shape", choices=["c3", "c4"],
+                    help="time the fused decode call on six stores of configuration c3's (16 sequences x 8192 tokens, "
+                         "cycling budgets) or c4's (131072 tokens, heavy eviction) shape, compressed by the real pipeline, "
+                         "rotating over the stores so that every call reads HBM; prints main-kernel and whole-call times and exits")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for counter runs under rocprofv3 --pmc: a few eager decode steps and one plain 256 MiB "
                          "device copy (the calibration kernel), nothing else timed")
@@ -439,6 +443,72 @@ def main() -> int:
         return 0
 
     eps, gate_err = parity_gate(dev)
+
+    if args.decode_shape:
+        import synthetic
+        name, n_stores = args.decode_shape, 6
+        sts, sqs = [], []
+        for li in range(n_stores):
+            if name == "c3":
+                Ls = [synthetic.gaussian_layer(3003 + 100 * li + s, 8, 32, 8192) for s in range(16)]
+                targets = [synthetic.C3_TARGETS[s % 3] for s in range(16)]
+            else:
+                Ls = [synthetic.lognormal_norm_layer(4004 + li, 8, 32, 131072)]
+                targets = [2.0]
+            Bs, Ts = len(Ls), Ls[0].keys.shape[1]
+            k = torch.stack([L.keys for L in Ls]).to(dev)
+            v = torch.stack([L.values for L in Ls]).to(dev)
+            sc = torch.stack([_launch_score(k[b], v[b], Ls[b].mu.to(dev), None, 32, 4, 1e-2) for b in range(Bs)])
+            bits = optimal_scores_to_bits_batched(sc.reshape(Bs, -1), LEVELS, targets, eps, n_sink=4, period=Ts,
+                                                  eviction_cost=0.5).reshape(Bs, 8, Ts)
+            bits[..., -128:] = 16
+            st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=dev, dtype=torch.float16, key_quantizer="mse",
+                                                value_quantizer="mse", seed=42 + li)
+            st.prefill(k, v, bits)
+            st._build_items()
+            sts.append(st)
+            sqs.append(torch.stack([L.query for L in Ls]).to(dev))
+            del k, v, sc, bits
+        Bs = sqs[0].shape[0]
+        ws_bytes = max(blib.odmkv_decode_workspace_bytes(Bs, 32, st._items[2]) for st in sts)
+        wss = [torch.empty(ws_bytes, dtype=torch.uint8, device=dev) for _ in sts]
+        outs = [torch.empty(Bs, 32, 128, dtype=torch.float32, device=dev) for _ in sts]
+
+        def sweep(mask):
+            for st, q, o, w in zip(sts, sqs, outs, wss):
+                bench_decode(blib, st, q, o, w, mask)
+
+        def graph_us(mask, reps=20):
+            sweep(7)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                sweep(mask)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            gk = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gk):
+                sweep(mask)
+            for _ in range(3):
+                gk.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(reps):
+                gk.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / (reps * n_stores) * 1e3
+
+        pb = sum(st.packed_bytes() for st in sts) / n_stores
+        main_us, call_us = graph_us(2), graph_us(6)
+        print(json.dumps({"decode_shape": name, "stores": n_stores, "sequences": Bs, "tokens": int(sts[0].seq_len),
+                          "packed_bytes_per_store": int(pb), "work_items": int(sts[0]._items[2]),
+                          "level_counts": {str(b): int(sum(st.level_counts()[b] for st in sts) / n_stores) for b in LEVELS},
+                          "main_kernel_us": round(main_us, 2), "main_kernel_GBps": round(pb / main_us / 1e3, 1),
+                          "main_kernel_frac_of_8TBps": round(pb / main_us / 1e3 / 8000.0, 4),
+                          "whole_call_us": round(call_us, 2), "whole_call_GBps": round(pb / call_us / 1e3, 1)}))
+        return 0
 
     # ---- compress every layer: score -> allocate -> window -> pack (timed per layer) ----
     states, qs, t_stage = [], [], {"score": [], "alloc": [], "pack": [], "total": []}
@@ -611,11 +681,11 @@ def main() -> int:
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / (reps * NL)
 
-    kern_alone_ms = stream_only_ms = None
+    kern_alone_ms = with_merge_ms = None
     if graph is not None:
         try:
-            kern_alone_ms = graph_ms_per_launch(6, min(args.steps, 50))      # main kernel with its merge, no preparation
-            stream_only_ms = graph_ms_per_launch(2, min(args.steps, 50))     # its streaming part alone
+            kern_alone_ms = graph_ms_per_launch(2, min(args.steps, 50))      # the main kernel alone, back to back
+            with_merge_ms = graph_ms_per_launch(6, min(args.steps, 50))      # with its merge: the whole call
         except Exception as exc:                                   # noqa: BLE001
             print(f"main-kernel-only graph not available ({exc}); using per-launch events", file=sys.stderr)
             torch.cuda.synchronize()
@@ -649,10 +719,10 @@ def main() -> int:
                      "traffic": TRAFFIC_FROM_PROFILE_BYTES if (NL, T, args.target) == (32, 32768, 2.0) else None,
                      "traffic_source": "profiles/decode_main_c2_32k_hbm_traffic.txt (rocprofv3 --pmc runs, not this run)",
                      "kernel": "decode_main_kernel", "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
-                     "kernel_avg_method": ("the step's main-kernel launches (streaming + merge, no query preparation) alone "
-                                           "as one graph, replayed between two HIP events"
+                     "kernel_avg_method": ("the step's main-kernel launches alone (no merge) as one graph, replayed between two "
+                                           "HIP events on the launch stream: elapsed / launches, launch gaps included"
                                            if kern_alone_ms is not None else "per-launch HIP event pairs"),
-                     "streaming_part_only_us": None if stream_only_ms is None else round(stream_only_ms * 1e3, 2),
+                     "with_merge_kernel_us": None if with_merge_ms is None else round(with_merge_ms * 1e3, 2),
                      "per_launch_events_avg_us": round(events_avg_ms * 1e3, 2),
                      "per_launch_events_median_us": round(pct(kernel_ms, 50) * 1e3, 2),
                      "per_launch_events_p10_us": round(pct(kernel_ms, 10) * 1e3, 2),

@@ -5,9 +5,6 @@
 #include <hip/hip_ext.h>
 
 #define PSTRIDE 132          // floats per (item, head) partial result: 128 acc + m + l + 2 pad
-#ifndef DECODE_NWAVES
-#define DECODE_NWAVES 8      // wavefronts of a workgroup of the main kernel
-#endif
 
 struct DecodeArgs {
     odmkv_packed_t s;

@@ -44,17 +44,25 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 #define PBUF (8 * PROW)     // one p buffer: 8 head rows
 
 // LDS of the main kernel: [table, later the combine area] [partial sums of the query rotation] [rotated query rows]
-// [p buffers] [per-wave scalars]
-#define ROT_SLICES (DECODE_NWAVES * 64 / 32)     // slices of the rotation's sum: a thread covers 4 dims x HD / ROT_SLICES terms
+// [p buffers] [per-wave scalars].  NW = wavefronts of the workgroup: 8 (short items: less set-up and a lighter combine)
+// or 16 (long items: four wavefronts per SIMD keep its issue slots full).
+#define ROT_THREADS 512                          // threads that rotate the queries (the first 512 of the workgroup)
+#define ROT_SLICES (ROT_THREADS / 32)            // slices of the rotation's sum: a thread covers 4 dims x HD / ROT_SLICES terms
 #define ROT_TERMS (HD / ROT_SLICES)
 #define QROW_LDS 272                             // bytes of a query row in LDS: 128 x 16 bit + 16 (bank spread)
 #define LDS_ROT LUT_BYTES
 #define LDS_QROWS (LDS_ROT + ROT_SLICES * ODMKV_MAX_GROUP * HD * 4)
 #define LDS_PBUFS (LDS_QROWS + 16 * QROW_LDS)
-#define LDS_SCALARS (LDS_PBUFS + DECODE_NWAVES * 2 * PBUF)
-#define LDS_TOTAL (LDS_SCALARS + DECODE_NWAVES * 4 * 8 * 4 + 8 * 4)
-static_assert(DECODE_NWAVES * ODMKV_MAX_GROUP * HD * 4 <= LUT_BYTES, "combine area must fit the table's space");
-static_assert((256 / DECODE_NWAVES) % 4 == 0 && DECODE_NWAVES <= 16 && ROT_TERMS == 8, "wave count");
+static_assert(ODMKV_MAX_GROUP * HD * 4 <= 16 * QROW_LDS, "the staged query shares the rotated rows' space");
+template <int NW>
+struct Lds {
+    static constexpr int SCALARS = LDS_PBUFS + NW * 2 * PBUF;
+    static constexpr int TOTAL = SCALARS + NW * 4 * 8 * 4 + 8 * 4;
+    static_assert(NW * ODMKV_MAX_GROUP * HD * 4 <= LUT_BYTES, "combine area must fit the table's space");
+    static_assert((256 / NW) % 4 == 0 && NW <= 16 && NW * 64 >= ROT_THREADS, "wave count");
+    static_assert(TOTAL <= 160 * 1024, "LDS of one workgroup");
+};
+static_assert(ROT_TERMS == 8, "rotation slices");
 
 __device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
 
@@ -149,7 +157,7 @@ __device__ static inline float pick(const float* t, uint32_t idx) {
 // apart), so the wavefront writes row after row instead: the lanes of one store instruction cover
 // consecutive 16-byte pieces of four (eight) rows, and fetch the row's entry from its owner by a
 // cross-lane read.
-template <int W>
+template <int W, int NW>
 __device__ static inline void build_lut(uint8_t* lut, const DecodeArgs& a, int tid) {
     const int lane = tid & 63, wave = tid >> 6;
     if constexpr (W == 2) {
@@ -161,7 +169,7 @@ __device__ static inline void build_lut(uint8_t* lut, const DecodeArgs& a, int t
         for (int k = 0; k < 4; ++k) h[k] = half_bits(a.cbs[k]);
         const auto sel = [&](int k) { return k == 0 ? h[0] : k == 1 ? h[1] : k == 2 ? h[2] : h[3]; };
         const uint32_t own = sel(lane >> 4);
-        constexpr int ROWS = 256 / DECODE_NWAVES;             // rows of this wavefront
+        constexpr int ROWS = 256 / NW;             // rows of this wavefront
 #pragma unroll
         for (int i = 0; i < ROWS / 4; ++i) {
             const int base = wave * ROWS + i * 4;            // wave-uniform; the row is base + (lane >> 4)
@@ -473,33 +481,29 @@ __device__ static inline void load_queries(const uint8_t* qrows, int lane, int n
 // the work item is known) and sums its eight terms for every head of the group, in order; the slices are added in
 // order by the thread that owns (head, dim).  Every workgroup of a KV head repeats this: the matrix comes out of the
 // L2 cache, and the work hides behind the first unit's way from memory.
+// The query of the group's heads goes through LDS: thread t < 16 G requests eight elements (request_q8), and
+// stages them as floats once they are there; after a barrier every rotating thread reads the eight terms of its slice.
 template <int GP>
-__device__ static inline void rotate_request(const DecodeArgs& a, int bq_first, RawQ8* raw, int tid) {
-    const int slice = tid >> 5;
-#pragma unroll
-    for (int g = 0; g < GP; ++g)
-        if (g < a.G) raw[g] = request_q8(a.q, a.q_dt, (size_t)(bq_first + g) * HD + slice * ROT_TERMS);
-}
-template <int GP>
-__device__ static inline void rotate_partial(const DecodeArgs& a, const RawQ8* raw, const f4* pk, float* rot, int tid) {
+__device__ static inline void rotate_partial(const DecodeArgs& a, const float* qsh, const f4* pk, float* rot, int tid) {
     const int i4 = tid & 31, slice = tid >> 5;
+    if (tid >= ROT_THREADS) return;
 #pragma unroll
     for (int g = 0; g < GP; ++g) {
         f4 acc = (f4){0.f, 0.f, 0.f, 0.f};
         if (g < a.G) {                                     // wave-uniform
-            float qv[8];
-            convert_q8(raw[g], a.q_dt, qv);
+            const f4 q0 = *reinterpret_cast<const f4*>(qsh + g * HD + slice * ROT_TERMS);
+            const f4 q1 = *reinterpret_cast<const f4*>(qsh + g * HD + slice * ROT_TERMS + 4);
 #pragma unroll
             for (int t = 0; t < ROT_TERMS; ++t)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[e] = __fmaf_rn(pk[t][e], qv[t], acc[e]);
+                for (int e = 0; e < 4; ++e) acc[e] = __fmaf_rn(pk[t][e], t < 4 ? q0[t] : q1[t - 4], acc[e]);
         }
         *reinterpret_cast<f4*>(rot + ((size_t)(slice * GP + g) * HD) + 4 * i4) = acc;
     }
 }
-template <int GP>
+template <int GP, int NW>
 __device__ static inline void rotate_finish(const float* rot, uint8_t* qrows, int tid) {
-    for (int o = tid; o < GP * HD; o += DECODE_NWAVES * 64) {
+    for (int o = tid; o < GP * HD; o += NW * 64) {
         const int g = o / HD, dim = o % HD;
         float tot = rot[(size_t)g * HD + dim];
 #pragma unroll
@@ -511,7 +515,7 @@ __device__ static inline void rotate_finish(const float* rot, uint8_t* qrows, in
 }
 
 // One work item of a quantised level: the workgroup's wavefronts walk the item's units.
-template <int W, int GP>
+template <int W, int GP, int NW>
 __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq_first, int tile0, int ntiles, int ntok,
                                               int tid, const f4* pk, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
     uint8_t* lut = smem;
@@ -524,23 +528,38 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     // answers; the second unit is requested after that (LDS stores behind a long queue of requests wait until the
     // memory pipeline has accepted them: with both units requested first the table was ready a microsecond later).
     // Loads return in issue order: the (small) query goes first.
-    RawQ8 qraw[GP];
-    rotate_request<GP>(a, bq_first, qraw, tid);
+    RawQ8 qraw;
+    const bool stages_q = tid < 16 * a.G;
+    if (stages_q) qraw = request_q8(a.q, a.q_dt, (size_t)bq_first * HD + 8 * tid);
     Unit<W> cur;
     int u = wave;
     int nvalid = tokens_of(u);
     if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
-    build_lut<W>(lut, a, tid);
-    rotate_partial<GP>(a, qraw, pk, reinterpret_cast<float*>(smem + LDS_ROT), tid);
+    f4 pk_late[ROT_TERMS];
+    if constexpr (NW != 8) {
+#pragma unroll
+        for (int t = 0; t < ROT_TERMS; ++t)
+            if (tid < ROT_THREADS) pk_late[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
+    }
+    build_lut<W, NW>(lut, a, tid);
+    float* qsh = reinterpret_cast<float*>(smem + LDS_QROWS);       // [G][128] floats; the rotated rows take this place later
+    if (stages_q) {
+        float qv[8];
+        convert_q8(qraw, a.q_dt, qv);
+        *reinterpret_cast<f4*>(qsh + 8 * tid) = (f4){qv[0], qv[1], qv[2], qv[3]};
+        *reinterpret_cast<f4*>(qsh + 8 * tid + 4) = (f4){qv[4], qv[5], qv[6], qv[7]};
+    }
     lds_barrier();
-    rotate_finish<GP>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
+    rotate_partial<GP>(a, qsh, NW == 8 ? pk : pk_late, reinterpret_cast<float*>(smem + LDS_ROT), tid);
+    lds_barrier();
+    rotate_finish<GP, NW>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
     lds_barrier();
     // second buffer (not for the widest rows), requested before the first unit is used
     Unit<W> nxt;
     int nv1 = 0;
     if constexpr (W != 8) {
-        nv1 = tokens_of(u + DECODE_NWAVES);
-        if (nv1 > 0) load_unit<W>(nxt, a, li, unit0 + u + DECODE_NWAVES, lane);
+        nv1 = tokens_of(u + NW);
+        if (nv1 > 0) load_unit<W>(nxt, a, li, unit0 + u + NW, lane);
     }
     if (nvalid <= 0) return;
     h8 qa[4];
@@ -548,7 +567,7 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     if constexpr (W == 8) {
         while (true) {
             compute_unit<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
-            u += DECODE_NWAVES;
+            u += NW;
             nvalid = tokens_of(u);
             if (nvalid <= 0) break;
             load_unit<W>(cur, a, li, unit0 + u, lane);
@@ -557,13 +576,13 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
         while (true) {
             compute_unit<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
             if (nv1 <= 0) break;
-            u += 2 * DECODE_NWAVES;
+            u += 2 * NW;
             nvalid = tokens_of(u);
             if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
             compute_unit<W>(nxt, nv1, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
             if (nvalid <= 0) break;
-            nv1 = tokens_of(u + DECODE_NWAVES);
-            if (nv1 > 0) load_unit<W>(nxt, a, li, unit0 + u + DECODE_NWAVES, lane);
+            nv1 = tokens_of(u + NW);
+            if (nv1 > 0) load_unit<W>(nxt, a, li, unit0 + u + NW, lane);
         }
     }
 }
@@ -582,7 +601,7 @@ __device__ static inline void load_exact_unit(ExactUnit& t, const uint16_t* base
 
 // BF: the store keeps bf16 rows; they meet the query (bf16 high + low piece of q16, exact) and the
 // softmax weights (bf16 high + low piece) on the bf16 matrix instructions, products exact, sums fp32.
-template <bool BF>
+template <bool BF, int NW>
 __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int bq_first, int tile0, int ntiles, int seg_first,
                                               int tid, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
     const int wave = tid >> 6, lane = tid & 63, n = lane & 15, j = lane >> 4;
@@ -608,7 +627,7 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
         }
     }
     const int count = a.s.seg_count[4][bh] - (tile0 - seg_first) * TILE;     // exact segments grow between work-list rebuilds
-    for (int u = wave; u < 2 * ntiles; u += DECODE_NWAVES) {
+    for (int u = wave; u < 2 * ntiles; u += NW) {
         const int nvalid = min(count - u * UNIT, UNIT);
         if (nvalid <= 0) break;
         ExactUnit k;
@@ -664,24 +683,25 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
 // ------------------------------------------------------------------------------------------------
 // main kernel
 // ------------------------------------------------------------------------------------------------
-template <int GP, bool ORDERED>
-__global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeArgs a) {
+template <int GP, bool ORDERED, int NW>
+__global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
     // one static LDS block: the table sits at LDS address 0 and that is known when the kernel is compiled, so a
     // lookup address needs no base added
-    __shared__ __align__(16) uint8_t smem[LDS_TOTAL];
+    __shared__ __align__(16) uint8_t smem[Lds<NW>::TOTAL];
     uint8_t* lut = smem;                                               // centroid table; reused to combine the wavefronts
-    float* alphas = reinterpret_cast<float*>(smem + LDS_SCALARS);      // [NWAVES][8]
-    float* wm = alphas + DECODE_NWAVES * 8;                            // [NWAVES][8]
-    float* wl = wm + DECODE_NWAVES * 8;                                // [NWAVES][8]
-    float* wf = wl + DECODE_NWAVES * 8;                                // [NWAVES][8]
-    float* wM = wf + DECODE_NWAVES * 8;                                // [8]
+    float* alphas = reinterpret_cast<float*>(smem + Lds<NW>::SCALARS);      // [NWAVES][8]
+    float* wm = alphas + NW * 8;                            // [NWAVES][8]
+    float* wl = wm + NW * 8;                                // [NWAVES][8]
+    float* wf = wl + NW * 8;                                // [NWAVES][8]
+    float* wM = wf + NW * 8;                                // [8]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     // this thread's share of Pi_k^T for the query rotation: the same for every item, requested first
+    // (eight wavefronts only: sixteen have half the registers, and their long items do not feel the wait)
     f4 pk[ROT_TERMS];
 #pragma unroll
     for (int t = 0; t < ROT_TERMS; ++t)
-        pk[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
+        if (NW == 8 && tid < ROT_THREADS) pk[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
     const int item = ORDERED ? a.order[blockIdx.x] : (int)blockIdx.x;
     const int4 d0 = reinterpret_cast<const int4*>(a.items)[2 * item];       // bh, level, first tile, tiles
     const int4 d1 = reinterpret_cast<const int4*>(a.items)[2 * item + 1];   // tokens, first tile of the segment
@@ -699,13 +719,13 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
     uint8_t* pbuf = smem + LDS_PBUFS + wave * 2 * PBUF;
     float* alpha_sh = alphas + wave * 8;
     switch (li) {
-        case 0: run_quant_level<2, GP>(a, 0, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
-        case 1: run_quant_level<3, GP>(a, 1, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
-        case 2: run_quant_level<4, GP>(a, 2, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
-        case 3: run_quant_level<8, GP>(a, 3, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
+        case 0: run_quant_level<2, GP, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
+        case 1: run_quant_level<3, GP, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
+        case 2: run_quant_level<4, GP, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
+        case 3: run_quant_level<8, GP, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
         default:
-            if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
-            else run_exact_level<false>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
+            if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
+            else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
             break;
     }
 
@@ -720,7 +740,7 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
     __syncthreads();
     float* wacc = reinterpret_cast<float*>(lut);          // [NWAVES][128 dims][GP heads]
     {
-        float MA = n < DECODE_NWAVES ? wm[n * 8 + 2 * j] : -INFINITY, MB = n < DECODE_NWAVES ? wm[n * 8 + 2 * j + 1] : -INFINITY;
+        float MA = n < NW ? wm[n * 8 + 2 * j] : -INFINITY, MB = n < NW ? wm[n * 8 + 2 * j + 1] : -INFINITY;
         row_max2(MA, MB);
         const float fA = st.mA > -INFINITY ? __builtin_amdgcn_exp2f(st.mA - MA) : 0.0f;
         const float fB = st.mB > -INFINITY ? __builtin_amdgcn_exp2f(st.mB - MB) : 0.0f;
@@ -735,18 +755,18 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
         }
     }
     __syncthreads();
-    for (int e = tid; e < GP * HD; e += DECODE_NWAVES * 64) {
+    for (int e = tid; e < GP * HD; e += NW * 64) {
         const int g = e % GP, dim = e / GP;               // consecutive threads walk consecutive LDS words
         float s = 0.0f;
 #pragma unroll
-        for (int w = 0; w < DECODE_NWAVES; ++w) s = __fmaf_rn(wacc[w * HD * GP + e], wf[w * 8 + g], s);
+        for (int w = 0; w < NW; ++w) s = __fmaf_rn(wacc[w * HD * GP + e], wf[w * 8 + g], s);
         dst[g * PSTRIDE + dim] = s;
     }
-    if (tid >= DECODE_NWAVES * 64 - GP) {                 // the last wavefront has the least to do above
-        const int g = tid - (DECODE_NWAVES * 64 - GP);
+    if (tid >= NW * 64 - GP) {                 // the last wavefront has the least to do above
+        const int g = tid - (NW * 64 - GP);
         float L = 0.0f;
 #pragma unroll
-        for (int w = 0; w < DECODE_NWAVES; ++w) L += wl[w * 8 + g];
+        for (int w = 0; w < NW; ++w) L += wl[w * 8 + g];
         dst[g * PSTRIDE + HD] = wM[g];
         dst[g * PSTRIDE + HD + 1] = L;
     }
@@ -757,12 +777,11 @@ __global__ __launch_bounds__(DECODE_NWAVES * 64) void decode_main_kernel(DecodeA
 // ------------------------------------------------------------------------------------------------
 #define MERGE_THREADS 512
 #define MERGE_SLICES (MERGE_THREADS / HD)
-#ifndef MERGE_SPLIT
-#define MERGE_SPLIT 4
-#endif
 #define MERGE_CHUNK 1024          // items whose weights are held in LDS at a time
 
-template <int GP>
+// MERGE_SPLIT: workgroups per query head (4 when there are few heads, so that the launch still covers the device;
+// 1 for large batches, where every further workgroup only repeats the reading)
+template <int GP, int MERGE_SPLIT>
 __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs a) {
     __shared__ float wts[MERGE_CHUNK];               // exp2(m_item - M); the sign bit marks exact items
     __shared__ float red[MERGE_THREADS / 64];
@@ -901,9 +920,9 @@ extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     return align_up((size_t)(n_items > 0 ? n_items : 1) * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
 }
 
-template <int GP, bool ORDERED>
+template <int GP, bool ORDERED, int NW>
 static int launch_main(const DecodeArgs& a, int grid, hipEvent_t e0, hipEvent_t e1, hipStream_t st) {
-    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED>), dim3(grid), dim3(DECODE_NWAVES * 64), 0, st, e0, e1, 0, a);
+    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED, NW>), dim3(grid), dim3(NW * 64), 0, st, e0, e1, 0, a);
     ODMKV_CHECK_LAUNCH("decode_main_kernel");
     return 0;
 }
@@ -922,6 +941,8 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     ODMKV_CHECK_ARG(((uintptr_t)q & 15) == 0, "decode_attn: the query must be 16-byte aligned");
     const int n_items = work->n_items;
     ODMKV_CHECK_ARG(n_items >= 0, "decode_attn: negative item count");
+    ODMKV_CHECK_ARG(work->wavefronts == 0 || work->wavefronts == 8 || work->wavefronts == 16,
+                    "decode_attn: %d wavefronts per work item (0, 8 or 16)", work->wavefronts);
     ODMKV_CHECK_ARG(work->item_range, "decode_attn: null item ranges");
     ODMKV_CHECK_ARG(n_items == 0 || work->items, "decode_attn: null work list");
     ODMKV_CHECK_ARG(B > 0 && Hq > 0 && store->B == B && store->Hkv > 0 && Hq % store->Hkv == 0,
@@ -948,16 +969,26 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
         // when measuring, the events are attached to the dispatch itself: they carry the kernel's own
         // start and end timestamps, not those of separate marker packets
         hipEvent_t e0 = (hipEvent_t)ev_start, e1 = (hipEvent_t)ev_stop;
+        const bool wide = work->wavefronts == 16;
         int rc;
-        if (GP == 4 && !a.order) rc = launch_main<4, false>(a, n_items, e0, e1, st);
-        else if (GP == 4) rc = launch_main<4, true>(a, n_items, e0, e1, st);
-        else if (!a.order) rc = launch_main<8, false>(a, n_items, e0, e1, st);
-        else rc = launch_main<8, true>(a, n_items, e0, e1, st);
+        if (GP == 4 && !a.order) rc = wide ? launch_main<4, false, 16>(a, n_items, e0, e1, st) : launch_main<4, false, 8>(a, n_items, e0, e1, st);
+        else if (GP == 4) rc = wide ? launch_main<4, true, 16>(a, n_items, e0, e1, st) : launch_main<4, true, 8>(a, n_items, e0, e1, st);
+        else if (!a.order) rc = wide ? launch_main<8, false, 16>(a, n_items, e0, e1, st) : launch_main<8, false, 8>(a, n_items, e0, e1, st);
+        else rc = wide ? launch_main<8, true, 16>(a, n_items, e0, e1, st) : launch_main<8, true, 8>(a, n_items, e0, e1, st);
         if (rc) return rc;
     }
     if (stage_mask & 4) {
-        if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4>), dim3(B * Hq * MERGE_SPLIT), dim3(MERGE_THREADS), 0, st, a);
-        else hipLaunchKernelGGL((decode_merge_kernel<8>), dim3(B * Hq * MERGE_SPLIT), dim3(MERGE_THREADS), 0, st, a);
+        const int heads = B * Hq;
+        if (heads >= 256) {
+            if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4, 1>), dim3(heads), dim3(MERGE_THREADS), 0, st, a);
+            else hipLaunchKernelGGL((decode_merge_kernel<8, 1>), dim3(heads), dim3(MERGE_THREADS), 0, st, a);
+        } else if (heads >= 128) {
+            if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4, 2>), dim3(heads * 2), dim3(MERGE_THREADS), 0, st, a);
+            else hipLaunchKernelGGL((decode_merge_kernel<8, 2>), dim3(heads * 2), dim3(MERGE_THREADS), 0, st, a);
+        } else {
+            if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4, 4>), dim3(heads * 4), dim3(MERGE_THREADS), 0, st, a);
+            else hipLaunchKernelGGL((decode_merge_kernel<8, 4>), dim3(heads * 4), dim3(MERGE_THREADS), 0, st, a);
+        }
         ODMKV_CHECK_LAUNCH("decode_merge_kernel");
     }
     return 0;

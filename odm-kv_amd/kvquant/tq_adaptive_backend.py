@@ -44,6 +44,10 @@ def _exact_index_tables():
 
 _EXACT_K_IDX, _EXACT_V_IDX = _exact_index_tables()
 _TILE_BYTES = [TILE * 16 * w + 2 * TILE * 4 for w in WIDTHS] + [2 * TILE * HEAD_DIM * 2]
+# what one compute unit was measured to need per 64-token tile of each level (nanoseconds; 2, 3, 4, 8 bits, exact rows)
+# and per work item (microseconds: start, table, query rotation, combining the wavefronts)
+_TILE_COST = [300, 420, 450, 890, 1310]
+_ITEM_FIXED_US = 4.0
 
 
 class _Buffers:
@@ -521,24 +525,28 @@ class TurboQuantAdaptiveKVCacheState:
     # ------------------------------------------------------------------ fused attention
     def _build_items(self, target_items: Optional[int] = None, min_item_bytes: Optional[int] = None) -> None:
         """The decode work list: every (segment, level) run of tiles cut into items of about equal
-        bytes, one workgroup (one compute unit, eight wavefronts) per item.
+        cost, one workgroup (one compute unit) per item.
 
+        The cost of a tile is what the kernel was measured to need for it per level (the 2-bit loop is
+        bound by instruction issue, the wider ones and the exact rows by memory), plus a fixed part per item.
         With a target the cut is the coarsest one that does not exceed it.  Without one, a few cuts
         are compared by the time a longest-first assignment of their items to the compute units
-        would take (a small cost model of the kernel: fixed set-up plus a round of eight tiles at a
-        time), and the best is kept; when it has more items than compute units, the order in which
-        the workgroups take the items (longest first) is handed to the kernel as well."""
+        would take, and the best is kept; when it has more items than compute units, the order in which
+        the workgroups take the items (longest first) is handed to the kernel as well.  Items of sixteen
+        tiles and more on average are run by sixteen wavefronts, shorter ones by eight."""
         import os
         n_cu = torch.cuda.get_device_properties(self.device).multi_processor_count
         env_target = int(os.environ.get("ODMKV_DECODE_ITEMS", 0))
         min_item_bytes = int(os.environ.get("ODMKV_DECODE_MIN_ITEM_BYTES", 16384)) if min_item_bytes is None else min_item_bytes
         used = (self._counts + TILE - 1) // TILE
         used[4] = np.diff(self._seg_tile[4])              # exact segments grow between rebuilds
-        total = sum(int(used[li].sum()) * _TILE_BYTES[li] for li in range(5))
+        total_bytes = sum(int(used[li].sum()) * _TILE_BYTES[li] for li in range(5))
+        total = sum(int(used[li].sum()) * _TILE_COST[li] for li in range(5))      # cost units: nanoseconds of one compute unit
+        min_item_bytes = min_item_bytes * _TILE_COST[0] // _TILE_BYTES[0]          # the same floor, as a cost
         runs = [(s, li, int(used[li, s])) for s in range(self._nseg) for li in range(5) if used[li, s] > 0]
 
         def step_of(per_item: int, li: int) -> int:
-            return max(1, int(round(per_item / _TILE_BYTES[li])))
+            return max(1, int(round(per_item / _TILE_COST[li])))
 
         def n_pieces(per_item: int) -> int:
             return sum(-(-nt // step_of(per_item, li)) for _, li, nt in runs)
@@ -562,8 +570,7 @@ class TurboQuantAdaptiveKVCacheState:
             return items
 
         def cost(item) -> float:                     # microseconds of one workgroup, roughly
-            rounds = -(-item[3] // 8)
-            return (3.0 + 1.0 * rounds) if item[1] == 4 else (3.0 + 1.0 * rounds)
+            return _ITEM_FIXED_US + item[3] * _TILE_COST[item[1]] * 1e-3
 
         def makespan(items) -> float:
             import heapq
@@ -579,7 +586,7 @@ class TurboQuantAdaptiveKVCacheState:
             # the comparison is repeated only when the store has grown by more than 5 % since the
             # last one (a decode-time flush adds a fraction of a percent): until then its winner is re-cut
             chosen = self._items_choice
-            if chosen is not None and abs(total - chosen[1]) <= 0.05 * chosen[1]:
+            if chosen is not None and abs(total_bytes - chosen[1]) <= 0.05 * chosen[1]:
                 items = cut(fit(int(n_cu * chosen[0])))
             else:
                 best = None
@@ -589,7 +596,7 @@ class TurboQuantAdaptiveKVCacheState:
                     if best is None or t < best[0] - 1e-9:
                         best = (t, cand, mult)
                 items = best[1]
-                self._items_choice = (best[2], total)
+                self._items_choice = (best[2], total_bytes)
         arr = np.asarray(items, np.int32).reshape(-1, 8)
         per_seg = np.bincount(arr[:, 0], minlength=self._nseg) if len(items) else np.zeros(self._nseg, np.int64)
         ranges = np.concatenate([[0], np.cumsum(per_seg)])          # items are generated in segment order
@@ -603,6 +610,8 @@ class TurboQuantAdaptiveKVCacheState:
         w.items, w.item_range = self._items[0].data_ptr(), self._items[1].data_ptr()
         w.dispatch_order = _lib.ptr(self._item_order)
         w.n_items = len(items)
+        quant = arr[arr[:, 1] < 4, 3] if len(items) else arr[:0, 3]
+        w.wavefronts = int(os.environ.get("ODMKV_DECODE_WAVES", 0)) or (16 if quant.size and quant.mean() >= 16 else 8)
         self._worklist = w
 
     def decode_attention(self, query: torch.Tensor, scaling: Optional[float] = None,

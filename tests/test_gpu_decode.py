@@ -238,6 +238,23 @@ def test_decode_error_is_mostly_the_dense_cache_rounding():
     assert e32 < 5e-4 and e32 < e16 and e32 < oracle_gap, (e16, e32, oracle_gap)
 
 
+@pytest.mark.parametrize("B", [4, 8])
+def test_many_query_heads_take_fewer_merge_workgroups_per_head(B):
+    """The merge runs four workgroups per query head for a handful of heads, two from 128 heads on and one from
+    256 on (B x 32 heads here): the result is the oracle's whichever way the head's dims are split."""
+    g = torch.Generator().manual_seed(60 + B)
+    H, G, T = 8, 4, 200
+    k = torch.randn(B, H, T, 128, generator=g).half()
+    v = torch.randn(B, H, T, 128, generator=g).half()
+    bits = _rand_bits(g, (B, H, T), (0.15, 0.4, 0.2, 0.1, 0.05, 0.1))
+    bits[..., :4] = 16
+    st, ref = _pair(k, v, bits)
+    q = torch.randn(B, H * G, 128, generator=g).half()
+    got, lse = st.decode_attention(q.to(DEV), return_lse=True)
+    assert rel_err(got.cpu(), decode_attention_state(q.float(), ref)) < ATTN_RTOL
+    assert torch.isfinite(lse).all()
+
+
 @pytest.mark.parametrize("mix", ["all-8-bit", "half-8-bit"])
 def test_eight_bit_tokens_keep_the_margin(mix):
     """The 256-entry table cannot be scaled so that all its entries round well to fp16 (up to 3.4e-4 relative per
