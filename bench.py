@@ -39,7 +39,7 @@ HBM_PEAK_GBS = 8000.0
 # the L2 counters of two rocprofv3 --pmc runs of `python bench.py --traffic-probe` (FETCH_SIZE, WRITE_SIZE),
 # each scaled by what the same counter reads for a 256 MiB device copy; the figures and the commands are in
 # profiles/decode_main_c2_32k_hbm_traffic.txt.  Applies to --layers 32 --ctx 32768 --target 2.0 only.
-TRAFFIC_FROM_PROFILE_BYTES = None
+TRAFFIC_FROM_PROFILE_BYTES = 20_959_000
 LEVELS = (0, 2, 3, 4, 8, 16)
 
 
