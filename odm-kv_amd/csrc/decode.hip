@@ -1,31 +1,31 @@
 // Fused LUT decode attention over the packed mixed-width KV store (one query token per sequence).
 //
-// Three launches per call:
-//   1. prep:  q16 = the query rounded to fp16 (what a model in fp16/bf16 hands over anyway);
-//             q' = Pi_k q16 in fp32, stored as fp16 high + low halves (queries in the rotated basis of
-//             the quantised keys); q16 itself for the exact tokens.
-//   2. main:  one workgroup per work item = a run of 64-token tiles of one (sequence, kv-head,
-//             level).  The packed bytes are read once from HBM; nothing else is.
-//   3. merge: log-sum-exp merge of a kv-head's items per query head, rotation of the quantised
+// Two launches per call:
+//   1. main:  one workgroup (8 or 16 wavefronts) per work item = a run of 64-token tiles of one (sequence,
+//             kv-head, level).  It rounds the group's queries to fp16 (what a model in fp16/bf16 hands over
+//             anyway), rotates them into the basis of the quantised keys (q' = Pi_k q16 in fp32, kept as fp16
+//             high + low halves), and streams the item's packed bytes once from HBM; nothing else is read from there.
+//   2. merge: log-sum-exp merge of a kv-head's items per query head, rotation of the quantised
 //             part back to the model basis (acc . Pi_v), addition of the exact part, normalise.
 // (Merging inside the main kernel, by the workgroup that finishes last among a kv-head's items, was built
 // and measured: the count and the other workgroups' results have to cross the device at agent scope, two
-// to three dependent trips to memory of 2-3 us each under the streaming load, against one launch of 4 us.)
+// to three dependent trips to memory of 2-3 us each under the streaming load, against one launch of 4-5 us.
+// A separate query-preparation launch was measured too: the same time per call, one launch more.)
 //
-// Main kernel, per wavefront and tile, on v_mfma_f32_16x16x32_f16 (D[16x16] += A[16x32] B[32x16];
-// lane l supplies A[l%16][8(l/16)+e] and B[8(l/16)+e][l%16], e = 0..7, and holds D[4(l/16)+r][l%16]):
+// Main kernel, per wavefront and unit of 32 tokens (half a tile), on v_mfma_f32_16x16x32_f16 (D[16x16] += A[16x32]
+// B[32x16]; lane l supplies A[l%16][8(l/16)+e] and B[8(l/16)+e][l%16], e = 0..7, and holds D[4(l/16)+r][l%16]):
 //   keys    A = the queries: row 2h = high half of head h, row 2h+1 = low half (up to 8 heads of the
-//           GQA group, 16 bytes per lane and step, loaded once per work item).  B = the centroids of
+//           GQA group, 16 bytes per lane and step, read from LDS once per work item).  B = the centroids of
 //           16 tokens x 32 dims, fetched from an LDS table by the code bytes; the packed layout puts
-//           the codes of (4 tokens x 32 dims) into each lane's 16*W bytes.  4 token blocks x 4 dim
-//           blocks = 16 matrix instructions; lane (n, j) then holds the logits of tokens 4n..4n+3
+//           the codes of (2 tokens x 32 dims) per unit into each lane's bytes.  2 token blocks x 4 dim
+//           blocks = 8 matrix instructions; lane (n, j) then holds the logits of its two slots
 //           (one per block) for heads 2j and 2j+1.
-//   softmax two heads per lane, maximum over the 16 lanes of a row by DPP row rotations, base-2
-//           exponentials, running (m, l) per head; p |v| is rounded to fp16 and handed to the value
-//           product through a per-wave LDS buffer (the product needs tokens along the contraction).
-//   values  A = p |v| (row = head), B = the centroids of 32 tokens x 16 dims; 2 token blocks x 8 dim
-//           blocks = 16 matrix instructions accumulate sum_t p_t |v_t| c[code] for 8 heads x 128 dims
-//           in the rotated basis.
+//   softmax two heads per lane, base-2 exponentials, running (m, l) per head, m a reference point that moves
+//           (DPP row reduction, rescale of the accumulators) only when a logit exceeds it by more than a slack;
+//           p |v| is rounded to fp16 and handed to the value product through a per-wave LDS buffer (the product
+//           needs tokens along the contraction).
+//   values  A = p |v| (row = head), B = the centroids of 32 tokens x 16 dims; 8 matrix instructions accumulate
+//           sum_t p_t |v_t| c[code] for 8 heads x 128 dims in the rotated basis.
 // The LDS table is replicated over 32 slots (slot = lane % 32) so that lanes never share a bank.
 // All softmax state is kept in base-2 logarithms.
 #include "decode.h"
