@@ -218,8 +218,8 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  *   out[b,q] = sum_t softmax_t( scaling * q[b,q] . Khat[b,q/G,t] ) Vhat[b,q/G,t]
  * over the stored (non-evicted) tokens.  Evicted tokens are simply absent.
  *
- * q: device [B, Hq, 128] of q_dtype (ODMKV_F16 / ODMKV_BF16 / ODMKV_F32), contiguous: the model's
- * query states are passed as they are.  work: the work list (below), built by the caller once per
+ * q: device [B, Hq, 128] of q_dtype (ODMKV_F16 / ODMKV_BF16 / ODMKV_F32), contiguous and 16-byte
+ * aligned: the model's query states are passed as they are.  work: the work list (below), built by the caller once per
  * change of the store.
  * out: device [B, Hq, 128] of out_dtype (accumulated in fp32, rounded once on the store);
  * lse: device fp32 [B, Hq] or NULL (log-sum-exp of the scaled logits).
@@ -242,7 +242,8 @@ int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v
  * items in the order the workgroups should take them (longest first, when there are more items than
  * compute units).
  * wavefronts: wavefronts of the workgroup that runs an item: 8 (0 means 8) or 16.  Eight start and finish
- * faster and suit items of up to about thirty tiles; sixteen stream long items about 1.7 times faster.
+ * faster and suit items of fewer than sixteen tiles; sixteen stream long items about 1.1 times faster.
+ * Two launches per call (main kernel, merge); the workspace holds the per-item partial results.
  */
 typedef struct odmkv_worklist {
     const int32_t* items;            /* device [n_items, 8] */
@@ -262,7 +263,7 @@ int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
 
 /* The same call without a workspace, for callers that cannot allocate device memory and have none
  * to hand over (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
- * No counterpart in the reference.  The prepared queries and the per-item partial results live in
+ * No counterpart in the reference.  The per-item partial results live in
  * a fixed array of ODMKV_STATIC_SCRATCH_BYTES inside the library's device image (held by every GPU
  * the library runs on until the process ends); a call whose odmkv_decode_workspace_bytes(B, Hq,
  * n_items) exceeds it fails with ODMKV_ENOSPACE and launches nothing.  The call allocates and
