@@ -60,6 +60,17 @@ int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int T,
                 const float* mu, int Hq, const float* attn, int n_sink, float eps,
                 float* scores, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same score as a model of 16-bit dtype computes it in the reference: the mean-query logits are rounded
+ * to round_dtype (ODMKV_F16 / ODMKV_BF16) after the product and again after the division by sqrt(d), every
+ * query head's softmax and the mean over the GQA group are rounded to it (kvquant/scorer.py:309-315, where
+ * these tensors have the module's dtype), and so are eps, p + eps and its square (kvquant/scorer.py:403); the
+ * rest is fp32 as in odmkv_score.  round_dtype = -1 is odmkv_score.  mu holds values of that dtype, widened to fp32. */
+int odmkv_score_model_dtype(const void* K, const void* V, int dtype, int Hkv, int T,
+                            int64_t stride_h, int64_t stride_t,
+                            const float* mu, int Hq, const float* attn, int n_sink, float eps,
+                            int round_dtype, float* scores, void* workspace, size_t workspace_bytes,
+                            void* stream);
+
 /* Expected-attention score.  Replaces ExpectedAttentionScorer.score_prefill after the query
  * statistics are known (kvquant/scorer.py:204-257):
  *

@@ -20,6 +20,7 @@ struct ScoreArgs {
     const float* mu;      // [Hq, 128]
     const float* attn;    // [Hkv, T] or null
     const float* cov;     // [Hq, 128, 128] query covariance (expected-attention score only) or null
+    int round_dt;         // -1, or ODMKV_F16 / ODMKV_BF16: round logits, softmax and group mean like a model of that dtype
     int use_vnorm;        // expected-attention score: multiply (p + eps) by |v|
     int ea_cpw;           // expected-attention score: 256-token chunks a workgroup walks
     int nstat;            // softmax statistics entries per query head (one per chunk, or one per wave and chunk)
@@ -97,6 +98,12 @@ __device__ static inline float group16_sum(float v) {
 #define SC_UNROLL_V 4          // the same for the two passes over V
 
 // merge two online-softmax states
+// x as a model of 16-bit dtype `dt` would hold it (-1: unchanged)
+__device__ static inline float round_model(float x, int dt) {
+    return dt == ODMKV_F16 ? __half2float(__float2half_rn(x))
+         : dt == ODMKV_BF16 ? Elem<ODMKV_BF16>::to_f32(Elem<ODMKV_BF16>::from_f32(x)) : x;
+}
+
 __device__ static inline void ms_merge(float& m, float& s, float m2, float s2) {
     const float mn = fmaxf(m, m2);
     if (mn == -INFINITY) { m = mn; s = 0.0f; return; }
@@ -163,7 +170,9 @@ __global__ __launch_bounds__(256) void score_logits_kernel(ScoreArgs a) {
                     float d = 0.0f;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) d = __fmaf_rn(x[e], mu_r[g][e], d);
-                    d = group16_sum(d) * inv_sqrt_d;
+                    d = group16_sum(d);
+                    // a 16-bit model rounds the product and, again, the division by sqrt(d) (kvquant/scorer.py:309-310)
+                    d = a.round_dt < 0 ? d * inv_sqrt_d : round_model(round_model(d, a.round_dt) / 11.313708498984761f, a.round_dt);
                     d_own[g] = part == u ? d : d_own[g];
                 }
             }
@@ -262,10 +271,19 @@ __global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
                     pt = lg[u][0];
                 } else {
                     float acc = 0.0f;
+                    if (a.round_dt < 0) {
 #pragma unroll
-                    for (int g = 0; g < GMAX; ++g)
-                        if (g < a.G) acc = __fmaf_rn(__expf(lg[u][g] - Mg[g]), Zg[g], acc);
-                    pt = acc * inv_g;
+                        for (int g = 0; g < GMAX; ++g)
+                            if (g < a.G) acc = __fmaf_rn(__expf(lg[u][g] - Mg[g]), Zg[g], acc);
+                        pt = acc * inv_g;
+                    } else {
+                        // the softmax of every query head and the mean over the group, each rounded to the model's
+                        // dtype (kvquant/scorer.py:314-315)
+#pragma unroll
+                        for (int g = 0; g < GMAX; ++g)
+                            if (g < a.G) acc += round_model(expf(lg[u][g] - Mg[g]) * Zg[g], a.round_dt);
+                        pt = round_model(acc * inv_g, a.round_dt);
+                    }
                 }
                 if (part == 0) { a.p[(size_t)h * a.Tc + t] = pt; ps += pt; }
 #pragma unroll
@@ -350,9 +368,11 @@ __global__ __launch_bounds__(256) void score_final_kernel(ScoreArgs a) {
             vn = group16_sum(vn);
             ir = group16_sum(ir);
             if (ok && part == 0) {
-                const float pe = pin[u] + a.eps;
+                // (p + eps)^2 is formed on the tensor of the model's dtype in the reference (kvquant/scorer.py:403):
+                // eps becomes a scalar of that dtype, the sum and the square are rounded to it
+                const float pe = round_model(pin[u] + round_model(a.eps, a.round_dt), a.round_dt);
                 const float kterm = (knin[u] * (1.0f / (float)HD)) * ir;      // 1/128: exact
-                const float sc = (pe * pe) * (vn + kterm);
+                const float sc = round_model(pe * pe, a.round_dt) * (vn + kterm);
                 a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
                 best = fmaxf(best, sc);
             }
@@ -784,7 +804,18 @@ extern "C" int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int
                            int64_t stride_h, int64_t stride_t,
                            const float* mu, int Hq, const float* attn, int n_sink, float eps,
                            float* scores, void* workspace, size_t workspace_bytes, void* stream) {
+    return odmkv_score_model_dtype(K, V, dtype, Hkv, T, stride_h, stride_t, mu, Hq, attn, n_sink, eps, -1,
+                                   scores, workspace, workspace_bytes, stream);
+}
+
+extern "C" int odmkv_score_model_dtype(const void* K, const void* V, int dtype, int Hkv, int T,
+                                       int64_t stride_h, int64_t stride_t,
+                                       const float* mu, int Hq, const float* attn, int n_sink, float eps,
+                                       int round_dtype, float* scores, void* workspace, size_t workspace_bytes,
+                                       void* stream) {
     ODMKV_CHECK_ARG(K && V && scores && workspace, "score: null pointer");
+    ODMKV_CHECK_ARG(round_dtype == -1 || round_dtype == ODMKV_F16 || round_dtype == ODMKV_BF16,
+                    "score: rounding dtype %d (-1, fp16 or bf16)", round_dtype);
     ODMKV_CHECK_ARG(mu || attn, "score: need the mean query or attention weights");
     ODMKV_CHECK_ARG(dtype == ODMKV_F16 || dtype == ODMKV_BF16 || dtype == ODMKV_F32, "score: bad dtype %d", dtype);
     ODMKV_CHECK_ARG(Hkv > 0 && Hq > 0 && Hq % Hkv == 0 && Hq / Hkv <= ODMKV_MAX_GROUP,
@@ -802,7 +833,7 @@ extern "C" int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int
     a.K = K; a.V = V; a.sH = stride_h; a.sT = stride_t;
     a.Hkv = Hkv; a.Hq = Hq; a.G = Hq / Hkv; a.Gl = attn ? 0 : Hq / Hkv; a.T = T; a.Tc = T - n_sink; a.n_sink = n_sink;
     a.nchunks = n_chunks(a.Tc); a.eps = eps; a.mu = mu; a.attn = attn; a.scores = scores;
-    a.cov = nullptr; a.use_vnorm = 0; a.ea_cpw = 1; a.nstat = a.nchunks;
+    a.cov = nullptr; a.use_vnorm = 0; a.ea_cpw = 1; a.nstat = a.nchunks; a.round_dt = round_dtype;
     a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
     a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
     a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);
@@ -886,7 +917,7 @@ extern "C" int odmkv_score_expected(const void* K, const void* V, int dtype, int
     a.K = K; a.V = V; a.sH = stride_h; a.sT = stride_t;
     a.Hkv = Hkv; a.Hq = Hq; a.G = Hq / Hkv; a.Gl = a.G; a.T = T; a.Tc = T - n_sink; a.n_sink = n_sink;
     a.nchunks = n_chunks(a.Tc); a.eps = eps; a.mu = mu; a.attn = nullptr; a.scores = scores;
-    a.cov = cov; a.use_vnorm = use_vnorm ? 1 : 0; a.ea_cpw = 1; a.nstat = a.nchunks;
+    a.cov = cov; a.use_vnorm = use_vnorm ? 1 : 0; a.ea_cpw = 1; a.nstat = a.nchunks; a.round_dt = -1;
     a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
     a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
     a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);

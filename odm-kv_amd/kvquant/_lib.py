@@ -56,6 +56,7 @@ def _load() -> C.CDLL:
         "odmkv_last_error": (C.c_char_p, []),
         "odmkv_score_workspace_bytes": (sz, [i32, i32, i32]),
         "odmkv_score": (C.c_int, [vp, vp, i32, i32, i32, i64, i64, vp, i32, vp, i32, f32, vp, vp, sz, vp]),
+        "odmkv_score_model_dtype": (C.c_int, [vp, vp, i32, i32, i32, i64, i64, vp, i32, vp, i32, f32, i32, vp, vp, sz, vp]),
         "odmkv_score_expected": (C.c_int, [vp, vp, i32, i32, i32, i64, i64, vp, vp, i32, i32, f32, i32, vp, vp, sz, vp]),
         "odmkv_window_attention_workspace_bytes": (sz, [i32, i32, i32, i32]),
         "odmkv_window_attention": (C.c_int, [vp, i32, i32, i32, i64, i64, vp, i32, i32, i32, i32, f32, vp, vp, sz, vp]),
@@ -84,7 +85,7 @@ def _load() -> C.CDLL:
 
 
 lib = _load()
-EXPORTS = ("odmkv_version", "odmkv_last_error", "odmkv_score_workspace_bytes", "odmkv_score", "odmkv_score_expected",
+EXPORTS = ("odmkv_version", "odmkv_last_error", "odmkv_score_workspace_bytes", "odmkv_score", "odmkv_score_model_dtype", "odmkv_score_expected",
            "odmkv_window_attention_workspace_bytes", "odmkv_window_attention",
            "odmkv_allocate_workspace_bytes", "odmkv_allocate", "odmkv_level_counts",
            "odmkv_pack_workspace_bytes", "odmkv_quant_pack", "odmkv_quantize_rows",

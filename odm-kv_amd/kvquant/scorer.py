@@ -170,7 +170,10 @@ def _launch_score_expected(keys: torch.Tensor, values: torch.Tensor, mu: torch.T
 
 
 def _launch_score(keys: torch.Tensor, values: torch.Tensor, mu: Optional[torch.Tensor],
-                  attn: Optional[torch.Tensor], n_q_heads: int, n_sink: int, eps: float) -> torch.Tensor:
+                  attn: Optional[torch.Tensor], n_q_heads: int, n_sink: int, eps: float,
+                  round_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """round_dtype (float16 / bfloat16): round the logits, the softmax and the group mean as a model of that
+    dtype does in the reference (kvquant/scorer.py:309-315, 403); None: fp32 throughout."""
     keys, values = _kv_operands(keys, values)
     H, T, D = keys.shape
     dev = keys.device
@@ -179,9 +182,10 @@ def _launch_score(keys: torch.Tensor, values: torch.Tensor, mu: Optional[torch.T
     ws = _lib.workspace(dev, ws_bytes, "score")
     mu32 = None if mu is None else mu.reshape(n_q_heads, D).float().contiguous()
     a32 = None if attn is None else attn.float().contiguous()
-    _lib.check(lib.odmkv_score(
+    rd = -1 if round_dtype is None else {torch.float16: 0, torch.bfloat16: 1}[round_dtype]
+    _lib.check(lib.odmkv_score_model_dtype(
         keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys), H, T, keys.stride(0), keys.stride(1),
-        _lib.ptr(mu32), n_q_heads, _lib.ptr(a32), n_sink, float(eps), scores.data_ptr(),
+        _lib.ptr(mu32), n_q_heads, _lib.ptr(a32), n_sink, float(eps), rd, scores.data_ptr(),
         ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
     return scores
 
@@ -190,9 +194,14 @@ class RiskScorer(ExpectedAttentionScorer):
     """s = (p + eps)^2 * [ |v|^2 + (|k|^2 / d) * |v - o|^2 ]: first-order joint error of the
     attention output under independent key and value quantisation noise."""
 
-    def __init__(self, **kw):
+    def __init__(self, *, model_dtype_rounding: bool = False, **kw):
+        """model_dtype_rounding (not in the reference's constructor; off by default): with keys in fp16 / bf16, round
+        the attention estimate where the reference's tensors have the model's dtype (logits, softmax, group mean,
+        (p + eps)^2: kvquant/scorer.py:309-315, 403), so that the scores are the ones the reference computes on such a model, not
+        the fp32 ones."""
         kw["use_covariance"] = False
         super().__init__(**kw)
+        self.model_dtype_rounding = bool(model_dtype_rounding)
 
     def score_prefill(self, keys, values, layer_idx, *, module=None, hidden_states=None):
         if module is None or hidden_states is None:
@@ -206,7 +215,8 @@ class RiskScorer(ExpectedAttentionScorer):
         except (AttributeError, NotImplementedError, ValueError):
             return self._fallback.score_prefill(keys, values, layer_idx)
         n_q = mu.shape[1]
-        scores = _launch_score(keys, values, mu[0], None, n_q, self.n_sink, self.epsilon)
+        rd = keys.dtype if self.model_dtype_rounding and keys.dtype in (torch.float16, torch.bfloat16) else None
+        scores = _launch_score(keys, values, mu[0], None, n_q, self.n_sink, self.epsilon, round_dtype=rd)
         return self._maybe_normalize(scores)
 
     def score_with_attn(self, keys, values, attn_weights, *, module=None):

@@ -62,6 +62,35 @@ def test_score_prefill_matches_oracle(hkv, hq, T, dtype, rotary):
     assert torch.all(got[:, :4] == got[:, 4:].max())
 
 
+@pytest.mark.parametrize("name", ["f16", "bf16"])
+def test_model_dtype_rounding_matches_reference_vectors(name):
+    """The score with the roundings of a 16-bit model (kvquant/scorer.py:309-315: logits, softmax and group mean
+    in the model's dtype) against what the reference returned for the same tensors, from the reference's own mean
+    query (the query statistics are torch code on both sides; on the GPU their 16-bit matrix products round
+    differently from the CPU's, which is not the kernel's doing).  Most scores agree to fp32 rounding; where an fp32
+    sum lands on the other side of a 16-bit rounding boundary than the reference's CPU sum did, p moves by one unit
+    of that dtype and the score by about twice that, relatively."""
+    from kvquant.scorer import RiskScorer, _launch_score
+    from test_oracle_scorer import MODEL_DTYPE_CASES, model_dtype_case
+    k, v, h, mod, mu_ref, out_ref = model_dtype_case(name)
+    dt, hq = MODEL_DTYPE_CASES[name]
+    sc = RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2, model_dtype_rounding=True)
+    sc.normalize_grain = "global"
+    mu = torch.from_numpy(mu_ref)[0].to(DEV)
+    got = sc._maybe_normalize(_launch_score(k.to(DEV), v.to(DEV), mu, None, hq, 4, 1e-2, round_dtype=dt)).cpu().numpy()
+    rel = np.abs(got - out_ref) / np.abs(out_ref)
+    ulp = 2.0 ** -10 if name == "f16" else 2.0 ** -7
+    assert rel.max() < 4 * ulp, rel.max()
+    assert np.median(rel) < 1e-5 and (rel < 1e-4).mean() > 0.9, (np.median(rel), (rel < 1e-4).mean())
+    # fp32 arithmetic on the same inputs is measurably further from the 16-bit reference
+    far = sc._maybe_normalize(_launch_score(k.to(DEV), v.to(DEV), mu, None, hq, 4, 1e-2)).cpu().numpy()
+    assert np.median(np.abs(far - out_ref) / np.abs(out_ref)) > 10 * np.median(rel) + 1e-5
+    # the host class passes the flag on: same module on the GPU, scores within a few units of the dtype
+    with torch.no_grad():
+        e2e = sc.score_prefill(k.to(DEV), v.to(DEV), 0, module=mod.to(DEV), hidden_states=h.to(DEV)).float().cpu().numpy()
+    assert (np.abs(e2e - out_ref) / np.abs(out_ref)).max() < 8 * ulp
+
+
 def test_score_special_cases():
     from kvquant.scorer import RiskScorer
     sc = RiskScorer(n_future_positions=512, n_sink=4, use_vnorm=True, epsilon=1e-2)

@@ -65,6 +65,37 @@ def test_fp16_model_dtype_matches_reference(golden):
     np.testing.assert_allclose(got.float().numpy(), golden["score_f16_out"], rtol=5e-3)
 
 
+MODEL_DTYPE_CASES = {"f16": (torch.float16, 8), "bf16": (torch.bfloat16, 4)}
+
+
+def model_dtype_case(name):
+    """(keys, values, hidden states, module, the reference's mean query and scores) of one case of
+    tests/golden/score_model_dtype_d128.npz (written by tests/golden/make_score_model_dtype_vectors.py)."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "score_model_dtype_d128.npz"))
+    dt, hq = MODEL_DTYPE_CASES[name]
+    k = torch.from_numpy(g[f"{name}_k_bits"]).view(dt)
+    v = torch.from_numpy(g[f"{name}_v_bits"]).view(dt)
+    h = torch.from_numpy(g[f"{name}_h"]).to(dt)
+    mod = Stub(g[f"{name}_w"], g[f"{name}_b"], hq, 128).to(dt)
+    return k, v, h, mod, g[f"{name}_mu"], g[f"{name}_out"]
+
+
+@pytest.mark.parametrize("name", ["f16", "bf16"])
+def test_model_dtype_scores_at_head_dim_128_match_reference(name):
+    """The scorer on a 16-bit module at the head size the kernels take: the oracle rounds where the reference's
+    tensors have the model's dtype, and an fp32 evaluation of the same inputs is measurably elsewhere."""
+    k, v, h, mod, mu_ref, out_ref = model_dtype_case(name)
+    with torch.no_grad():
+        mu = sc.mean_query(mod, h, 4, 512)
+        got = sc.risk_score_prefill(k, v, module=mod, hidden_states=h)
+    np.testing.assert_array_equal(mu.float().numpy(), mu_ref)
+    np.testing.assert_allclose(got.float().numpy(), out_ref, rtol=1e-6)
+    fp32 = sc.risk_score_from_mu(k.float(), v.float(), mu.float(), mu.shape[1]).numpy()
+    far = np.abs(fp32 - out_ref) / np.abs(out_ref)
+    assert far.max() > (1e-3 if name == "f16" else 5e-3)
+
+
 def test_with_attn_and_fallback_match_reference(golden):
     k, v, a = (torch.from_numpy(golden[f"swa_{x}"]) for x in "kva")
     np.testing.assert_allclose(sc.risk_score_with_attn(k, v, a).numpy(), golden["swa_out"], rtol=1e-5)
