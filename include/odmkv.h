@@ -144,10 +144,11 @@ int odmkv_allocate(const float* scores, int rows, int n,
  * l = 0..63 (C = w for codes of width w, C = 16 for exact rows), chunk c of lane l at byte
  * (c*64 + l)*16 of the tile, and with l = 16*j + n the lane's 16*C bytes hold
  *   K codes:  128 codes as one little-endian bit stream (code i at bits [i*w, i*w + w));
- *             code 32*b + i  is dim 32*j + i  of slot 4*n + b          (b = 0..3, i = 0..31)
+ *             code 32*b + i  is dim 32*j + i  of slot key_slot(n, b)    (b = 0..3, i = 0..31),
+ *             key_slot(n, b) = 32*(b>>1) + 8*(n>>2) + 2*(n&3) + (b&1): the bytes of blocks 0, 1 hold slots 0..31
  *   V codes:  128 codes likewise; code 64*k + 8*m + e  is slot 32*k + 8*j + e  of dim 16*m + n
  *                                                                        (k = 0..1, m = 0..7, e = 0..7)
- *   exact K:  chunk 4*b + k  = the 8 elements  dims 32*j + 8*k .. + 7  of slot 4*n + b
+ *   exact K:  chunk 4*b + k  = the 8 elements  dims 32*j + 8*k .. + 7  of slot key_slot(n, b)
  *   exact V:  chunk 8*k + m  = the 8 elements  slots 32*k + 8*j .. + 7 of dim 16*m + n
  *   norms fp32 [64], pos int32 [64] per tile, in slot order.
  */
@@ -212,6 +213,14 @@ int odmkv_dequant(const odmkv_packed_t* store, void* K, void* V, int dtype, int 
                   int64_t stride_b, int64_t stride_h, int64_t stride_t,
                   const float* pi_k, const float* pi_v, const float* codebooks,
                   int include_exact, void* stream);
+/* The same for the quantised tokens at positions t_min <= t < T only (include_exact must be 0 when t_min > 0):
+ * after a decode-time flush only the re-stored tokens have new values in the dense copy
+ * (materialize_quantized_into, kvquant/tq_adaptive_backend.py:452-464, restricted to what changed). */
+int odmkv_dequant_from(const odmkv_packed_t* store, void* K, void* V, int dtype, int t_min, int T,
+                       int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                       const float* pi_k, const float* pi_v, const float* codebooks,
+                       int include_exact, void* stream);
+
 
 /* Append one fp16/bf16 token per (b, h) to the exact segments (append_all_exact,
  * kvquant/tq_adaptive_backend.py:380-425, for one decode step).  k, v: [B, Hkv, 128] of the
@@ -221,6 +230,35 @@ int odmkv_dequant(const odmkv_packed_t* store, void* K, void* V, int dtype, int 
  * untouched when a segment is full; the caller sizes segments. */
 int odmkv_append_exact(const odmkv_packed_t* store, const void* k, const void* v, int64_t stride_b,
                        int64_t stride_h, int pos, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Decode-time flush of the exact token buffer on the device.  Stands where the reference scores the
+ * buffered tokens with the current query and ranks them with a chain of torch operations
+ * (kvquant/adaptive_backend_press.py:464-665).
+ *
+ * odmkv_exact_tail: the newest n_tail tokens of every exact segment as dense rows K, V [B*Hkv, n_tail, 128]
+ * of the store's exact type, oldest first (get_buffer_tokens, kvquant/tq_adaptive_backend.py:466-497, when
+ * every head buffers the same positions).  A segment holding fewer tokens yields zero rows in front.
+ *
+ * odmkv_flush_score: per (sequence, kv-head) bh, with its n buffered rows K, V [BH, n, 128] of `dtype` and one
+ * query q fp32 [BH, 128] (the GQA group's mean query at the last position, post-RoPE):
+ *   a_t = softmax_t(q . k_t * scaling)                                  (_flush_attention, :602-665)
+ *   mode 0: s_t = (a_t + eps)^2 * (|v_t|^2 + |k_t|^2/128 * |v_t - o|^2), o = sum_t a_t v_t / max(sum a, 1e-8)
+ *           (RiskScorer.score_with_attn, kvquant/scorer.py:406-416);  mode 1: s_t = a_t^2 |v_t|^2 (no scorer).
+ * attn (fp32 [BH, n], may be NULL), scores fp32 [BH, n], minmax fp32 [BH, 2] (min and max score of each bh).
+ * n <= 2048.  Arithmetic in fp32 on the 16-bit inputs.
+ *
+ * odmkv_flush_rank: scores [B, H, n] are min-max normalised over the whole flush as the press does
+ * ((x - lo) / max(hi - lo, 1e-30); 0.5 everywhere when hi - lo <= 1e-8; lo, hi from minmax), then each
+ * kv-head's B*n tokens (sequence after sequence) are sorted ascending, equal values in index order, and the token
+ * of rank r gets by_rank[h][r] (device int32 [H, B*n]: the head's level shares cached at prefill, expanded to
+ * levels by rank on the host, _allocate_bits_via_cached_ratios :198-241).  bits: device int32 [B, H, n] out.
+ * B*n <= 4096. */
+int odmkv_exact_tail(const odmkv_packed_t* store, int n_tail, void* K, void* V, void* stream);
+int odmkv_flush_score(const void* K, const void* V, int dtype, int BH, int n, const float* q, float scaling,
+                      float eps, int mode, float* attn, float* scores, float* minmax, void* stream);
+int odmkv_flush_rank(const float* scores, const float* minmax, int B, int H, int n, const int32_t* by_rank,
+                     int32_t* bits, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Fused LUT decode attention over the packed store: one query token per sequence.

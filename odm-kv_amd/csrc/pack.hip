@@ -936,7 +936,7 @@ struct DequantArgs {
     void* K;
     void* V;
     int64_t sB, sH, sT;
-    int Hkv, nseg, T;
+    int Hkv, nseg, T, t_min;           // positions t_min <= t < T are written
     const float* pi_k;
     const float* pi_v;
     const float* cb;
@@ -982,11 +982,13 @@ __global__ __launch_bounds__(DQ_NW * 64) void dequant_kernel(DequantArgs a, int 
         const int ts = (tile - a.seg_tile[bh]) * TILE;
         const int hi = min(a.seg_count[bh] - ts, TILE);
         if (hi <= 0) continue;                                       // wave-uniform
+        // positions ascend inside a segment: a tile whose last token lies before t_min has nothing to write
+        if (a.t_min > 0 && a.pos[(size_t)tile * TILE + hi - 1] < a.t_min) continue;
         const size_t slot = (size_t)tile * TILE + lane;
         const bool valid = lane < hi;
         {
             const int t = valid ? a.pos[slot] : -1;
-            const bool write = valid && t >= 0 && t < a.T;
+            const bool write = valid && t >= a.t_min && t < a.T;
             offs[lane] = write ? (long long)((size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH + (size_t)t * a.sT) : -1ll;
             norms[lane] = valid ? (is_v ? a.vnorm[slot] : a.knorm[slot]) : 0.0f;
         }
@@ -1131,7 +1133,15 @@ extern "C" int odmkv_dequant(const odmkv_packed_t* store, void* K, void* V, int 
                              int64_t stride_b, int64_t stride_h, int64_t stride_t,
                              const float* pi_k, const float* pi_v, const float* codebooks,
                              int include_exact, void* stream) {
+    return odmkv_dequant_from(store, K, V, dtype, 0, T, stride_b, stride_h, stride_t, pi_k, pi_v, codebooks, include_exact, stream);
+}
+
+extern "C" int odmkv_dequant_from(const odmkv_packed_t* store, void* K, void* V, int dtype, int t_min, int T,
+                                  int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                                  const float* pi_k, const float* pi_v, const float* codebooks,
+                                  int include_exact, void* stream) {
     ODMKV_CHECK_ARG(K && V && pi_k && pi_v && codebooks, "dequant: null pointer");
+    ODMKV_CHECK_ARG(t_min >= 0 && !(t_min > 0 && include_exact), "dequant: t_min=%d (>= 0; quantised tokens only when > 0)", t_min);
     ODMKV_CHECK_ARG(dtype == ODMKV_F16 || dtype == ODMKV_BF16 || dtype == ODMKV_F32, "dequant: bad dtype %d", dtype);
     if (int rc = check_store(store, "dequant")) return rc;
     const int align = dtype == ODMKV_F32 ? 4 : 8;
@@ -1144,7 +1154,7 @@ extern "C" int odmkv_dequant(const odmkv_packed_t* store, void* K, void* V, int 
         if (store->n_tiles[li] == 0) continue;
         DequantArgs da;
         da.K = K; da.V = V; da.sB = stride_b; da.sH = stride_h; da.sT = stride_t;
-        da.Hkv = store->Hkv; da.nseg = nseg; da.T = T;
+        da.Hkv = store->Hkv; da.nseg = nseg; da.T = T; da.t_min = t_min;
         da.pi_k = pi_k; da.pi_v = pi_v; da.cb = codebooks + codebook_offset(li);
         da.pos = store->pos[li]; da.seg_tile = store->seg_tile[li]; da.seg_count = store->seg_count[li];
         da.kcodes = store->kcodes[li]; da.vcodes = store->vcodes[li];

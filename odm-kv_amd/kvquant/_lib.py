@@ -70,12 +70,16 @@ def _load() -> C.CDLL:
         "odmkv_quantize_rows": (C.c_int, [vp, i32, i64, i64, i32, vp, vp, vp, vp, vp]),
         "odmkv_dequantize_rows": (C.c_int, [vp, vp, i64, i32, vp, vp, vp, vp]),
         "odmkv_dequant": (C.c_int, [C.POINTER(Packed), vp, vp, i32, i32, i64, i64, i64, vp, vp, vp, i32, vp]),
+        "odmkv_dequant_from": (C.c_int, [C.POINTER(Packed), vp, vp, i32, i32, i32, i64, i64, i64, vp, vp, vp, i32, vp]),
         "odmkv_append_exact": (C.c_int, [C.POINTER(Packed), vp, vp, i64, i64, i32, vp]),
         "odmkv_decode_workspace_bytes": (sz, [i32, i32, i32]),
         "odmkv_decode_attn": (C.c_int, [vp, i32, i32, i32, f32, C.POINTER(Packed), C.POINTER(Worklist), vp, vp, vp,
                                         C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp, sz, vp]),
         "odmkv_decode_attn_static": (C.c_int, [vp, i32, i32, i32, f32, C.POINTER(Packed), C.POINTER(Worklist), vp, vp, vp,
                                                C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp]),
+        "odmkv_exact_tail": (C.c_int, [C.POINTER(Packed), i32, vp, vp, vp]),
+        "odmkv_flush_score": (C.c_int, [vp, vp, i32, i32, i32, vp, f32, f32, i32, vp, vp, vp, vp]),
+        "odmkv_flush_rank": (C.c_int, [vp, vp, i32, i32, i32, vp, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -89,8 +93,9 @@ EXPORTS = ("odmkv_version", "odmkv_last_error", "odmkv_score_workspace_bytes", "
            "odmkv_window_attention_workspace_bytes", "odmkv_window_attention",
            "odmkv_allocate_workspace_bytes", "odmkv_allocate", "odmkv_level_counts",
            "odmkv_pack_workspace_bytes", "odmkv_quant_pack", "odmkv_quantize_rows",
-           "odmkv_dequantize_rows", "odmkv_dequant", "odmkv_append_exact",
-           "odmkv_decode_workspace_bytes", "odmkv_decode_attn", "odmkv_decode_attn_static")
+           "odmkv_dequantize_rows", "odmkv_dequant", "odmkv_dequant_from", "odmkv_append_exact",
+           "odmkv_decode_workspace_bytes", "odmkv_decode_attn", "odmkv_decode_attn_static",
+           "odmkv_exact_tail", "odmkv_flush_score", "odmkv_flush_rank")
 
 
 def check(rc: int) -> None:

@@ -23,6 +23,7 @@ from typing import Optional
 import torch
 from torch import nn
 
+from kvquant import _lib
 from kvquant.allocator import optimal_scores_to_bits, ratio_scores_to_bits, scores_to_bits
 from kvquant.attention_patch import fused_decode_enabled
 from kvquant.attention_utils import _aligned_rotary_outputs, _apply_rotary_pos_emb_q, _get_query_states
@@ -122,13 +123,15 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         if hasattr(cache, "layers"):
             cache.layers[layer_idx]._tq_backend_state = state
 
-    def _sync_cache_from_state(self, cache, layer_idx: int, module: nn.Module, state, *, prefill_fast: bool = False) -> None:
+    def _sync_cache_from_state(self, cache, layer_idx: int, module: nn.Module, state, *, prefill_fast: bool = False,
+                               start: int = 0) -> None:
+        """`start`: only positions >= start have changed in the store (a flush re-stores the buffered tokens)."""
         if self._packed_layer(cache, layer_idx) is not None:
             self._attach(cache, layer_idx, module, state)            # no dense copy to bring up to date
             return
         if prefill_fast:
             keys, values = self._get_cache_tensors(cache, layer_idx)
-            state.materialize_quantized_into(keys, values)
+            state.materialize_quantized_into(keys, values, start=start)
         else:
             keys, values = state.materialize()
             self._set_cache_tensors(cache, layer_idx, keys, values)
@@ -292,6 +295,8 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         if buffer_start is None:
             self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True)
             return
+        if self._flush_on_device(state, layer_idx, cache, module, hidden_states, int(buffer_start)):
+            return
         positions, buf_keys, buf_values = state.get_buffer_tokens(buffer_start)
         if positions.shape[0] == 0:
             self._buffer_start_seqs[layer_idx] = state.seq_len
@@ -343,15 +348,101 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         state.flush_buffer(buffer_start, bits)
         self._buffer_start_seqs[layer_idx] = state.seq_len
         self._buffer_counts[layer_idx] = 0
-        self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True)
+        self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True, start=int(buffer_start))
 
     @torch.no_grad()
-    def _flush_attention(self, module: nn.Module, hidden_states, buf_keys: torch.Tensor,
-                         positions: torch.Tensor, state) -> Optional[torch.Tensor]:
-        """Attention weights [N_buf] of the current query (GQA mean, RoPE at the last position) over
-        the buffered keys, softmax within each (batch, head); None if the query cannot be formed."""
+    def _flush_on_device(self, state, layer_idx: int, cache, module: nn.Module, hidden_states, buffer_start: int) -> bool:
+        """The flush in a handful of launches and without reading anything back, where its inputs allow it: the
+        budget is a target (levels by the per-head shares cached at prefill), the scorer is the risk scorer (or
+        none), every head buffers the same positions and the buffer is small enough for the kernels
+        (odmkv_exact_tail, odmkv_flush_score, odmkv_flush_rank).  False: nothing was done, the caller goes the
+        general way (as it does when `device_flush` is set to False on the press).  With `record_flush` set on the
+        press the attention weights, scores and levels of the last flush are kept in `last_flush` (for tests)."""
+        from .scorer import RiskScorer
+        if not getattr(self, "device_flush", True):
+            return False
+        if self.ratios is not None or self.target_avg_bits is None or hidden_states is None:
+            return False
+        if self.scorer is not None and type(self.scorer).score_with_attn is not RiskScorer.score_with_attn:
+            return False
+        B, H = state.batch_size, state.num_heads
+        n_buf = state.seq_len - buffer_start
+        if n_buf <= 0 or n_buf > 2048 or B * n_buf > 4096:
+            return False
+        table = self._by_rank_table(layer_idx, H, B * n_buf, state.device)
+        if table is None:
+            return False
+        q_kv = self._flush_query(module, hidden_states, state)
+        if q_kv is None:
+            return False
+        rows = state.exact_tail(n_buf)
+        if rows is None:
+            return False
+        k, v = rows
+        by_rank, counts = table
+        dev = state.device
+        q32 = q_kv.reshape(B * H, -1).float().contiguous()
+        record = bool(getattr(self, "record_flush", False))
+        attn = torch.empty(B * H, n_buf, dtype=torch.float32, device=dev) if record else None
+        scores = torch.empty(B * H, n_buf, dtype=torch.float32, device=dev)
+        minmax = torch.empty(B * H, 2, dtype=torch.float32, device=dev)
+        bits = torch.empty(B, H, n_buf, dtype=torch.int32, device=dev)
+        st = _lib.stream_ptr(dev)
+        eps = float(self.scorer.epsilon) if self.scorer is not None else 0.0
+        _lib.check(_lib.lib.odmkv_flush_score(
+            k.data_ptr(), v.data_ptr(), _lib.dtype_code(k), B * H, n_buf, q32.data_ptr(), 1.0 / math.sqrt(k.shape[-1]),
+            eps, 0 if self.scorer is not None else 1, _lib.ptr(attn), scores.data_ptr(), minmax.data_ptr(), st))
+        _lib.check(_lib.lib.odmkv_flush_rank(scores.data_ptr(), minmax.data_ptr(), B, H, n_buf, by_rank.data_ptr(),
+                                             bits.data_ptr(), st))
+        if record:
+            self.last_flush = {"layer": layer_idx, "start": buffer_start, "q_kv": q_kv, "keys": k, "values": v,
+                               "attn": attn.reshape(B, H, n_buf), "scores": scores.reshape(B, H, n_buf), "bits": bits}
+        # with one sequence the level counts of every head are those of its table: no read-back in the append
+        state.flush_buffer(buffer_start, bits, rows=rows, known_counts=counts if B == 1 else None)
+        self._buffer_start_seqs[layer_idx] = state.seq_len
+        self._buffer_counts[layer_idx] = 0
+        self._sync_cache_from_state(cache, layer_idx, module, state, prefill_fast=True, start=buffer_start)
+        return True
+
+    def _by_rank_table(self, layer_idx: int, num_heads: int, n_tok: int, device):
+        """(device int32 [H, n_tok]: level of every rank per kv-head, host int64 [H, 6]: tokens per level 0, 2, 3, 4, 8,
+        16) from the shares cached at prefill, as `_allocate_bits_via_cached_ratios` forms them; None when a head
+        has no usable shares.  Kept per (layer, n_tok)."""
+        import numpy as np
+        cache = self.__dict__.setdefault("_by_rank_cache", {})
+        key = (layer_idx, num_heads, n_tok, str(device))
+        if key in cache:
+            return cache[key]
+        allowed = set(self._decode_bit_levels)
+        rows = []
+        for h in range(num_heads):
+            got = self._observed_ratios.get((layer_idx, h))
+            kept = [(b, r) for b, r in (got or ()) if b in allowed and r > 0]
+            if not kept:
+                return None
+            total = sum(r for _, r in kept)
+            levels, ratios = zip(*[(b, r / total) for b, r in kept])
+            rows.append(_levels_by_rank(levels, ratios, n_tok))
+        by_rank = np.stack(rows)
+        counts = np.stack([(by_rank == b).sum(axis=1) for b in _lib.LEVEL_ORDER], axis=1).astype(np.int64)
+        cache[key] = (torch.from_numpy(by_rank).to(device), counts)
+        return cache[key]
+
+    @torch.no_grad()
+    def _flush_query(self, module: nn.Module, hidden_states, state) -> Optional[torch.Tensor]:
+        """[B, H, d]: the current query at the last position (RoPE applied), averaged over each GQA group; None if
+        it cannot be formed."""
         if hidden_states is None or not hasattr(module, "layer_idx"):
             return None
+        H = state.num_heads
+        # the attention call of this very step left the token's query (post-RoPE) on the module: what the
+        # reference recomputes from the hidden state (q_proj, RoPE at the last position) is that tensor
+        q = getattr(module, "_odmkv_last_query", None)
+        module._odmkv_last_query = None
+        if (q is not None and q.dim() == 4 and q.shape[0] == hidden_states.shape[0] == state.batch_size and q.shape[2] == 1
+                and q.shape[1] % H == 0 and q.shape[3] == state.head_dim and hidden_states.shape[1] == 1):
+            B, Hq, _, d = q.shape
+            return q[:, :, 0, :].reshape(B, H, Hq // H, d).mean(dim=2)
         try:
             q = _get_query_states(module, hidden_states)                    # [B, Hq, q, d]
         except (AttributeError, NotImplementedError, ValueError):
@@ -362,8 +453,17 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
             cos, sin = _aligned_rotary_outputs(rotary_emb, q, pos_ids)
             q = _apply_rotary_pos_emb_q(q, cos, sin)
         B, Hq, _, d = q.shape
-        H = state.num_heads
-        q_kv = q[:, :, -1, :].reshape(B, H, Hq // H, d).mean(dim=2)          # [B, H, d]
+        return q[:, :, -1, :].reshape(B, H, Hq // H, d).mean(dim=2)
+
+    @torch.no_grad()
+    def _flush_attention(self, module: nn.Module, hidden_states, buf_keys: torch.Tensor,
+                         positions: torch.Tensor, state) -> Optional[torch.Tensor]:
+        """Attention weights [N_buf] of the current query (GQA mean, RoPE at the last position) over
+        the buffered keys, softmax within each (batch, head); None if the query cannot be formed."""
+        q_kv = self._flush_query(module, hidden_states, state)
+        if q_kv is None:
+            return None
+        B, H, d = q_kv.shape
         n_buf = positions.shape[0] // (B * H)
         if n_buf * B * H != positions.shape[0]:
             return None

@@ -89,6 +89,10 @@ def _attention_patch(func):
             module.masked_key_indices = None
             module._odmkv_state = None
         else:
+            if query.shape[2] == 1:
+                # the newest token's query, after RoPE: the press's flush scores its buffer with it and need not
+                # project and rotate the hidden state a second time
+                module._odmkv_last_query = query
             fused = _fused_decode(module, query, key, value, attention_mask, dropout, kwargs)
             if fused is not None:
                 call_counts["fused"] += 1

@@ -43,6 +43,14 @@ def _exact_index_tables():
 
 
 _EXACT_K_IDX, _EXACT_V_IDX = _exact_index_tables()
+_CU_COUNT: dict = {}
+
+
+def _compute_units(device) -> int:
+    key = str(device)
+    if key not in _CU_COUNT:
+        _CU_COUNT[key] = torch.cuda.get_device_properties(device).multi_processor_count
+    return _CU_COUNT[key]
 _TILE_BYTES = [TILE * 16 * w + 2 * TILE * 4 for w in WIDTHS] + [2 * TILE * HEAD_DIM * 2]
 # what one compute unit was measured to need per 64-token tile of each level (nanoseconds; 2, 3, 4, 8 bits, exact rows)
 # and per work item (microseconds: start, table, query rotation, combining the wavefronts)
@@ -312,7 +320,9 @@ class TurboQuantAdaptiveKVCacheState:
         self.append(keys, values, bits)
 
     def append(self, keys: torch.Tensor, values: torch.Tensor, bits: torch.Tensor,
-               _pos_offset: Optional[int] = None) -> None:
+               _pos_offset: Optional[int] = None, _known_counts: Optional[np.ndarray] = None) -> None:
+        """_known_counts (int [B*H, 6], levels 0, 2, 3, 4, 8, 16): what odmkv_level_counts would return for `bits`,
+        when the caller knows it without looking (levels assigned by rank with fixed shares): no read-back."""
         self._validate_shapes(keys, values, bits)
         B, H, T, D = keys.shape
         if T == 0:
@@ -325,9 +335,12 @@ class TurboQuantAdaptiveKVCacheState:
             values = values.contiguous()
             keys = keys.contiguous()
         st = _lib.stream_ptr(dev)
-        counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
-        _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
-        counts = counts_dev.cpu().numpy().astype(np.int64)            # the one synchronisation
+        if _known_counts is not None:
+            counts = np.asarray(_known_counts, np.int64).reshape(self._nseg, 6)
+        else:
+            counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
+            _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
+            counts = counts_dev.cpu().numpy().astype(np.int64)        # the one synchronisation
         if int(counts.sum()) != self._nseg * T:
             raise ValueError("bits must take values in (0, 2, 3, 4, 8, 16)")
         present = {lvl for lvl, c in zip(_lib.LEVEL_ORDER, counts.sum(axis=0)) if c > 0}
@@ -415,14 +428,14 @@ class TurboQuantAdaptiveKVCacheState:
         self._items = None
 
     # ------------------------------------------------------------------ reads
-    def _dequant_into(self, keys: torch.Tensor, values: torch.Tensor, include_exact: bool) -> None:
+    def _dequant_into(self, keys: torch.Tensor, values: torch.Tensor, include_exact: bool, start: int = 0) -> None:
         if self._bufs is None:
             return
         if not (self._rows_ok(keys) and self._rows_ok(values) and keys.stride() == values.stride()):
             raise ValueError("materialisation targets must be row-contiguous [B, H, T, D] tensors with equal strides")
-        _lib.check(lib.odmkv_dequant(
+        _lib.check(lib.odmkv_dequant_from(
             C.byref(self._packed), keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys),
-            int(keys.shape[2]), keys.stride(0), keys.stride(1), keys.stride(2),
+            int(start), int(keys.shape[2]), keys.stride(0), keys.stride(1), keys.stride(2),
             self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
             1 if include_exact else 0, _lib.stream_ptr(self.device)))
 
@@ -435,10 +448,10 @@ class TurboQuantAdaptiveKVCacheState:
         self._dequant_into(keys, values, True)
         return keys, values
 
-    def materialize_quantized_into(self, keys: torch.Tensor, values: torch.Tensor) -> None:
+    def materialize_quantized_into(self, keys: torch.Tensor, values: torch.Tensor, start: int = 0) -> None:
         """Overwrite the quantised positions of existing dense tensors; exact and evicted
-        positions are left as they are."""
-        self._dequant_into(keys, values, False)
+        positions are left as they are.  `start` (an addition): only positions >= start."""
+        self._dequant_into(keys, values, False, start)
 
     def masked_key_indices(self):
         """Indices (b, h, t) of the evicted positions, or None when there are none.  The answer is
@@ -501,26 +514,45 @@ class TurboQuantAdaptiveKVCacheState:
             return _empty_positions(self.device), empty, empty.clone()
         return got
 
-    def flush_buffer(self, buffer_start_seq: int, new_bits: torch.Tensor) -> None:
+    def exact_tail(self, n_tail: int):
+        """(keys, values) [B, H, n_tail, D] of the store's exact dtype: the newest n_tail tokens of every exact
+        segment, oldest first, in one launch and without reading anything back (the host's own mirror of the
+        segment lengths says whether every segment holds that many); None otherwise."""
+        n_tail = int(n_tail)
+        if self._bufs is None or n_tail <= 0 or int(self._counts[4].min()) < n_tail:
+            return None
+        k = torch.empty(self.batch_size, self.num_heads, n_tail, self.head_dim, dtype=self._exact_torch_dtype, device=self.device)
+        v = torch.empty_like(k)
+        _lib.check(lib.odmkv_exact_tail(C.byref(self._packed), n_tail, k.data_ptr(), v.data_ptr(), _lib.stream_ptr(self.device)))
+        return k, v
+
+    def flush_buffer(self, buffer_start_seq: int, new_bits: torch.Tensor, rows=None, known_counts=None) -> None:
         """Re-quantise the exact tokens at positions >= buffer_start_seq to `new_bits` (one entry
-        per token, in the order `get_buffer_tokens` returns them)."""
+        per token, in the order `get_buffer_tokens` returns them).  `rows` = (keys, values) [B, H, n, D] as
+        `exact_tail` returned them for the same tokens and `known_counts` (see `append`) spare the gather and the
+        read-back."""
         start = int(buffer_start_seq)
-        got = self._exact_rows(start)
-        if got is None:
-            return
-        pos3, krows, vrows = got
         n_buf = self.seq_len - start
-        if pos3.shape[0] != self._nseg * n_buf:
-            raise ValueError("flush_buffer expects every position >= buffer_start_seq to be exact in every head")
         B, H = self.batch_size, self.num_heads
-        k = krows.reshape(B, H, n_buf, self.head_dim).contiguous()
-        v = vrows.reshape(B, H, n_buf, self.head_dim).contiguous()
+        if rows is not None:
+            k, v = rows
+            if tuple(k.shape) != (B, H, n_buf, self.head_dim):
+                raise ValueError("flush_buffer: rows do not cover the positions >= buffer_start_seq")
+        else:
+            got = self._exact_rows(start)
+            if got is None:
+                return
+            pos3, krows, vrows = got
+            if pos3.shape[0] != self._nseg * n_buf:
+                raise ValueError("flush_buffer expects every position >= buffer_start_seq to be exact in every head")
+            k = krows.reshape(B, H, n_buf, self.head_dim).contiguous()
+            v = vrows.reshape(B, H, n_buf, self.head_dim).contiguous()
         bits = new_bits.to(device=self.device, dtype=torch.int32).reshape(B, H, n_buf)
         # drop the buffered tokens from the exact segments, then append them at their new levels
         self._counts[4] -= n_buf
         self._exact_room = None
         self._bufs["seg_count"][4].copy_(torch.from_numpy(self._counts[4].astype(np.int32)))
-        self.append(k, v, bits, _pos_offset=start)
+        self.append(k, v, bits, _pos_offset=start, _known_counts=known_counts)
 
     # ------------------------------------------------------------------ fused attention
     def _build_items(self, target_items: Optional[int] = None, min_item_bytes: Optional[int] = None) -> None:
@@ -535,7 +567,7 @@ class TurboQuantAdaptiveKVCacheState:
         the workgroups take the items (longest first) is handed to the kernel as well.  Items of sixteen
         tiles and more on average are run by sixteen wavefronts, shorter ones by eight."""
         import os
-        n_cu = torch.cuda.get_device_properties(self.device).multi_processor_count
+        n_cu = _compute_units(self.device)
         env_target = int(os.environ.get("ODMKV_DECODE_ITEMS", 0))
         min_item_bytes = int(os.environ.get("ODMKV_DECODE_MIN_ITEM_BYTES", 16384)) if min_item_bytes is None else min_item_bytes
         used = (self._counts + TILE - 1) // TILE
@@ -543,13 +575,19 @@ class TurboQuantAdaptiveKVCacheState:
         total_bytes = sum(int(used[li].sum()) * _TILE_BYTES[li] for li in range(5))
         total = sum(int(used[li].sum()) * _TILE_COST[li] for li in range(5))      # cost units: nanoseconds of one compute unit
         min_item_bytes = min_item_bytes * _TILE_COST[0] // _TILE_BYTES[0]          # the same floor, as a cost
-        runs = [(s, li, int(used[li, s])) for s in range(self._nseg) for li in range(5) if used[li, s] > 0]
+        # the runs of tiles, segment by segment (the merge finds a segment's items next to each other), as arrays
+        run_li, run_s = np.nonzero(used.T > 0)[1], np.nonzero(used.T > 0)[0]
+        run_nt = used[run_li, run_s].astype(np.int64)
+        run_t0 = self._seg_tile[run_li, run_s].astype(np.int64)
+        run_cnt = self._counts[run_li, run_s].astype(np.int64)
+        tile_cost = np.asarray(_TILE_COST, np.float64)
 
-        def step_of(per_item: int, li: int) -> int:
-            return max(1, int(round(per_item / _TILE_COST[li])))
+        def steps_of(per_item: int) -> np.ndarray:                     # tiles per item, by level
+            return np.maximum(1, np.rint(per_item / tile_cost).astype(np.int64))
 
         def n_pieces(per_item: int) -> int:
-            return sum(-(-nt // step_of(per_item, li)) for _, li, nt in runs)
+            step = steps_of(per_item)[run_li]
+            return int((-(-run_nt // step)).sum())
 
         def fit(target: int) -> int:
             # the coarsest cut with at most `target` items (a run's last piece may be short)
@@ -558,24 +596,25 @@ class TurboQuantAdaptiveKVCacheState:
                 per_item += max(per_item // 64, 1)
             return per_item
 
-        def cut(per_item: int):
-            items = []
-            for s, li, nt in runs:
-                step = step_of(per_item, li)
-                t0, cnt = int(self._seg_tile[li, s]), int(self._counts[li, s])
-                for a0 in range(0, nt, step):
-                    n = min(step, nt - a0)
-                    # (segment, level, first tile, tiles, tokens in those tiles, segment's first tile, -, -)
-                    items.append((s, li, t0 + a0, n, min(cnt - a0 * TILE, n * TILE), t0, 0, 0))
-            return items
+        def cut(per_item: int) -> np.ndarray:
+            # rows (segment, level, first tile, tiles, tokens in those tiles, segment's first tile, -, -)
+            step = steps_of(per_item)[run_li]
+            pieces = -(-run_nt // step)
+            run = np.repeat(np.arange(run_nt.size), pieces)
+            a0 = (np.arange(run.size) - np.repeat(np.cumsum(pieces) - pieces, pieces)) * step[run]
+            n = np.minimum(step[run], run_nt[run] - a0)
+            out = np.zeros((run.size, 8), np.int64)
+            out[:, 0], out[:, 1], out[:, 2], out[:, 3] = run_s[run], run_li[run], run_t0[run] + a0, n
+            out[:, 4], out[:, 5] = np.minimum(run_cnt[run] - a0 * TILE, n * TILE), run_t0[run]
+            return out
 
-        def cost(item) -> float:                     # microseconds of one workgroup, roughly
-            return _ITEM_FIXED_US + item[3] * _TILE_COST[item[1]] * 1e-3
+        def cost(items: np.ndarray) -> np.ndarray:                       # microseconds of one workgroup, roughly
+            return _ITEM_FIXED_US + items[:, 3] * tile_cost[items[:, 1]] * 1e-3
 
-        def makespan(items) -> float:
+        def makespan(items: np.ndarray) -> float:
             import heapq
             free = [0.0] * n_cu
-            for c in sorted((cost(it) for it in items), reverse=True):
+            for c in sorted(cost(items).tolist(), reverse=True):
                 heapq.heappush(free, heapq.heappop(free) + c)
             return max(free)
 
@@ -597,15 +636,22 @@ class TurboQuantAdaptiveKVCacheState:
                         best = (t, cand, mult)
                 items = best[1]
                 self._items_choice = (best[2], total_bytes)
-        arr = np.asarray(items, np.int32).reshape(-1, 8)
+        arr = items.astype(np.int32).reshape(-1, 8)
         per_seg = np.bincount(arr[:, 0], minlength=self._nseg) if len(items) else np.zeros(self._nseg, np.int64)
         ranges = np.concatenate([[0], np.cumsum(per_seg)])          # items are generated in segment order
         order = None
         if len(items) > n_cu:
-            order = np.argsort(-np.asarray([cost(it) for it in items]), kind="stable").astype(np.int32)
-        self._item_order = None if order is None else torch.from_numpy(order).to(self.device)
-        self._items = (torch.from_numpy(arr).to(self.device),
-                       torch.from_numpy(ranges.astype(np.int32)).to(self.device), len(items))
+            order = np.argsort(-cost(items), kind="stable").astype(np.int32)
+        # one upload for the item table, the ranges and the order (the parts start at multiples of 4 integers)
+        n_arr, n_rng = arr.size, (ranges.size + 3) & ~3
+        blob = np.zeros(n_arr + n_rng + (0 if order is None else order.size), np.int32)
+        blob[:n_arr] = arr.reshape(-1)
+        blob[n_arr:n_arr + ranges.size] = ranges
+        if order is not None:
+            blob[n_arr + n_rng:] = order
+        dev_blob = torch.from_numpy(blob).to(self.device)
+        self._item_order = None if order is None else dev_blob[n_arr + n_rng:]
+        self._items = (dev_blob[:n_arr].view(-1, 8), dev_blob[n_arr:n_arr + ranges.size], len(items))
         w = _lib.Worklist()
         w.items, w.item_range = self._items[0].data_ptr(), self._items[1].data_ptr()
         w.dispatch_order = _lib.ptr(self._item_order)

@@ -341,10 +341,12 @@ def test_press_with_other_scorers(kind):
 
 
 @torch.inference_mode()
-def test_flush_levels_match_the_oracle():
+@pytest.mark.parametrize("path", ["device", "host"])
+def test_flush_levels_match_the_oracle(path):
     """Decode-time flush (reference: kvquant/adaptive_backend_press.py:464-665, 198-241) against
     oracle.flush on the same buffered tokens: attention weights of the current query, normalised risk
-    scores, and the levels from the level shares recorded at prefill."""
+    scores, and the levels from the level shares recorded at prefill.  Both ways the press can take: the
+    device kernels (odmkv_exact_tail / odmkv_flush_score / odmkv_flush_rank) and the general torch path."""
     from transformers import DynamicCache
     from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
     from oracle import flush as ofl
@@ -353,6 +355,8 @@ def test_flush_levels_match_the_oracle():
     ids = _ids(T, 61)
     forced = torch.randint(0, 1000, (n_buf + 3,), generator=torch.Generator().manual_seed(62)).to(DEV)
     press = _press(target=2.5)
+    press.device_flush = path == "device"
+    press.record_flush = True
     rec = {}
     orig_flush, orig_attn, orig_alloc = press._flush_decode_buffer, press._flush_attention, press._allocate_bits_via_cached_ratios
 
@@ -362,8 +366,19 @@ def test_flush_levels_match_the_oracle():
         r.update(pos=pos.cpu().numpy(), k=k.float().cpu(), v=v.float().cpu(), hidden=hidden_states.clone(),
                  seq_len=state.seq_len, module=module, observed={h: press._observed_ratios[(layer_idx, h)] for h in range(state.num_heads)})
         press._cur = r
+        press.last_flush = None
         orig_flush(state, layer_idx, cache, module, hidden_states)
         r["levels"] = state._level_map[0].cpu().numpy().copy()
+        if path == "device":
+            lf = press.last_flush
+            assert lf is not None and lf["layer"] == layer_idx, "the device path was not taken"
+            # the kernels' rows are the buffered tokens in (batch, head, position) order
+            assert torch.equal(lf["keys"].reshape(-1, 128).float().cpu(), r["k"]) and torch.equal(lf["values"].reshape(-1, 128).float().cpu(), r["v"])
+            raw = lf["scores"].reshape(-1).float()
+            lo, hi = raw.min(), raw.max()
+            r["attn"] = lf["attn"].reshape(-1).float().cpu()
+            r["scores"] = ((raw - lo) / (hi - lo).clamp_min(1e-30)).cpu()      # the normalisation the rank kernel applies
+            r["bits"] = lf["bits"].reshape(-1).cpu()
 
     def spy_attn(*a, **kw):
         out = orig_attn(*a, **kw)
