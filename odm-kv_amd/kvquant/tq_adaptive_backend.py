@@ -364,7 +364,8 @@ class TurboQuantAdaptiveKVCacheState:
             self.seq_len += T
         else:
             self._level_store[:, :, pos_offset:pos_offset + T] = lm
-        self._masked = None
+        if not (_known_counts is not None and _pos_offset is not None and int(counts[:, 0].sum()) == 0):
+            self._masked = None           # (a re-store without evictions leaves the evicted set as it was)
         self._items = None
 
     def append_all_exact(self, keys: torch.Tensor, values: torch.Tensor) -> None:
