@@ -274,7 +274,8 @@ int odmkv_flush_rank(const float* scores, const float* minmax, int B, int H, int
  * lse: device fp32 [B, Hq] or NULL (log-sum-exp of the scaled logits).
  * pi_k_t is the key rotation TRANSPOSED (row-major [128,128] of Pi_k^T), pi_v the value rotation as is.
  * The query is rounded to fp16 on entry (the attention being replaced receives it in the model's
- * fp16/bf16).  The centroid tables live in LDS as fp16; to keep their rounding out of the result,
+ * fp16/bf16); bf16 and fp32 values beyond fp16's range saturate at +-65504.  The centroid tables live in
+ * LDS as fp16; to keep their rounding out of the result,
  * `codebooks` here holds the centroids of each width times a per-width scale chosen on the host
  * so that the scaled values are (nearly) exact in fp16, codebooks_host a host copy of the same 284
  * floats (the small tables travel as kernel arguments), and inv_scales (host, 4 floats) the

@@ -286,16 +286,18 @@ __device__ static inline RawQ8 request_q8(const void* q, int dt, size_t elem) {
     }
     return r;
 }
+// (fp32 and bf16 queries beyond fp16's range saturate at +-65504 instead of becoming infinite)
+__device__ static inline float to_q16(float x) { return __half2float(__float2half_rn(fminf(fmaxf(x, -65504.0f), 65504.0f))); }
 __device__ static inline void convert_q8(const RawQ8& r, int dt, float* out) {
     const uint32_t w[8] = {r.x.x, r.x.y, r.x.z, r.x.w, r.y.x, r.y.y, r.y.z, r.y.w};
     if (dt == ODMKV_F32) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) out[e] = __half2float(__float2half_rn(__uint_as_float(w[e])));
+        for (int e = 0; e < 8; ++e) out[e] = to_q16(__uint_as_float(w[e]));
     } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const uint16_t bits = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
-            out[e] = dt == ODMKV_F16 ? Elem<ODMKV_F16>::to_f32(bits) : __half2float(__float2half_rn(Elem<ODMKV_BF16>::to_f32(bits)));
+            out[e] = dt == ODMKV_F16 ? Elem<ODMKV_F16>::to_f32(bits) : to_q16(Elem<ODMKV_BF16>::to_f32(bits));
         }
     }
 }
