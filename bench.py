@@ -293,10 +293,12 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--read-ceiling", action="store_true",
                     help="time a plain streaming read kernel at the decode kernel's launch sizes (cold buffers) and exit")
-    ap.add_argument("--decode-shape", choices=["c3", "c4"],
+    ap.add_argument("--decode-shape", choices=["c3", "c4", "w2", "w3", "w4", "w8", "exact"],
                     help="time the fused decode call on six stores of configuration c3's (16 sequences x 8192 tokens, "
                          "cycling budgets) or c4's (131072 tokens, heavy eviction) shape, compressed by the real pipeline, "
-                         "rotating over the stores so that every call reads HBM; prints main-kernel and whole-call times and exits")
+                         "or on single-level stores (w2..w8: every token of a 131072-token layer at that width; exact: 32768 "
+                         "fp16 tokens), rotating over the stores so that every call reads HBM; prints main-kernel and "
+                         "whole-call times and exits")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for counter runs under rocprofv3 --pmc: a few eager decode steps and one plain 256 MiB "
                          "device copy (the calibration kernel), nothing else timed")
@@ -449,19 +451,26 @@ def main() -> int:
         name, n_stores = args.decode_shape, 6
         sts, sqs = [], []
         for li in range(n_stores):
+            single = {"w2": 2, "w3": 3, "w4": 4, "w8": 8, "exact": 16}.get(name)
             if name == "c3":
                 Ls = [synthetic.gaussian_layer(3003 + 100 * li + s, 8, 32, 8192) for s in range(16)]
                 targets = [synthetic.C3_TARGETS[s % 3] for s in range(16)]
-            else:
+            elif name == "c4":
                 Ls = [synthetic.lognormal_norm_layer(4004 + li, 8, 32, 131072)]
                 targets = [2.0]
+            else:
+                Ls = [synthetic.gaussian_layer(6006 + li, 8, 32, 32768 if single == 16 else 131072)]
             Bs, Ts = len(Ls), Ls[0].keys.shape[1]
             k = torch.stack([L.keys for L in Ls]).to(dev)
             v = torch.stack([L.values for L in Ls]).to(dev)
-            sc = torch.stack([_launch_score(k[b], v[b], Ls[b].mu.to(dev), None, 32, 4, 1e-2) for b in range(Bs)])
-            bits = optimal_scores_to_bits_batched(sc.reshape(Bs, -1), LEVELS, targets, eps, n_sink=4, period=Ts,
-                                                  eviction_cost=0.5).reshape(Bs, 8, Ts)
-            bits[..., -128:] = 16
+            if single is None:
+                sc = torch.stack([_launch_score(k[b], v[b], Ls[b].mu.to(dev), None, 32, 4, 1e-2) for b in range(Bs)])
+                bits = optimal_scores_to_bits_batched(sc.reshape(Bs, -1), LEVELS, targets, eps, n_sink=4, period=Ts,
+                                                      eviction_cost=0.5).reshape(Bs, 8, Ts)
+                bits[..., -128:] = 16
+            else:
+                sc = None
+                bits = torch.full((Bs, 8, Ts), single, dtype=torch.int32, device=dev)
             st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=dev, dtype=torch.float16, key_quantizer="mse",
                                                 value_quantizer="mse", seed=42 + li)
             st.prefill(k, v, bits)
