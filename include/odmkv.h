@@ -291,8 +291,9 @@ int odmkv_flush_rank(const float* scores, const float* minmax, int B, int H, int
  * dispatch_order: NULL (workgroup k takes item k), or device int32 [n_items], a permutation of the
  * items in the order the workgroups should take them (longest first, when there are more items than
  * compute units).
- * wavefronts: wavefronts of the workgroup that runs an item: 8 (0 means 8) or 16.  Eight start and finish
- * faster and suit items of fewer than sixteen tiles; sixteen stream long items about 1.1 times faster.
+ * wavefronts: wavefronts of the workgroup that runs an item: 8 (0 means 8), 12 or 16.  Eight start and finish
+ * faster and suit items of fewer than sixteen tiles; sixteen stream long 2- and 3-bit items about 1.1 times
+ * faster; twelve (three units in flight per wavefront) are 5 % ahead where 4- and 8-bit tokens carry the bytes.
  * Two launches per call (main kernel, merge); the workspace holds the per-item partial results.
  */
 typedef struct odmkv_worklist {
@@ -300,7 +301,7 @@ typedef struct odmkv_worklist {
     const int32_t* item_range;       /* device [B*Hkv + 1] */
     const int32_t* dispatch_order;   /* device [n_items] or NULL */
     int32_t n_items;
-    int32_t wavefronts;              /* 0, 8 or 16 */
+    int32_t wavefronts;              /* 0, 8, 12 or 16 */
 } odmkv_worklist_t;
 
 size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);

@@ -59,7 +59,7 @@ struct Lds {
     static constexpr int SCALARS = LDS_PBUFS + NW * 2 * PBUF;
     static constexpr int TOTAL = SCALARS + NW * 4 * 8 * 4 + 8 * 4;
     static_assert(NW * ODMKV_MAX_GROUP * HD * 4 <= LUT_BYTES, "combine area must fit the table's space");
-    static_assert((256 / NW) % 4 == 0 && NW <= 16 && NW * 64 >= ROT_THREADS, "wave count");
+    static_assert(NW >= 4 && NW <= 16 && NW * 64 >= ROT_THREADS, "wave count");
     static_assert(TOTAL <= 160 * 1024, "LDS of one workgroup");
 };
 static_assert(ROT_TERMS == 8, "rotation slices");
@@ -169,10 +169,11 @@ __device__ static inline void build_lut(uint8_t* lut, const DecodeArgs& a, int t
         for (int k = 0; k < 4; ++k) h[k] = half_bits(a.cbs[k]);
         const auto sel = [&](int k) { return k == 0 ? h[0] : k == 1 ? h[1] : k == 2 ? h[2] : h[3]; };
         const uint32_t own = sel(lane >> 4);
-        constexpr int ROWS = 256 / NW;             // rows of this wavefront
+        // groups of four rows go round the wavefronts
 #pragma unroll
-        for (int i = 0; i < ROWS / 4; ++i) {
-            const int base = wave * ROWS + i * 4;            // wave-uniform; the row is base + (lane >> 4)
+        for (int i = 0; i < (64 + NW - 1) / NW; ++i) {
+            const int base = (i * NW + wave) * 4;            // wave-uniform; the row is base + (lane >> 4)
+            if (base >= 256) break;
             const uint32_t x = own | (sel((base >> 2) & 3) << 16), y = sel((base >> 4) & 3) | (sel(base >> 6) << 16);
             *reinterpret_cast<uint4*>(lut + (base + (lane >> 4)) * 256 + (lane & 15) * 16) = make_uint4(x, y, x, y);
         }
@@ -533,58 +534,109 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     RawQ8 qraw;
     const bool stages_q = tid < 16 * a.G;
     if (stages_q) qraw = request_q8(a.q, a.q_dt, (size_t)bq_first * HD + 8 * tid);
-    Unit<W> cur;
-    int u = wave;
-    int nvalid = tokens_of(u);
-    if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
-    f4 pk_late[ROT_TERMS];
-    if constexpr (NW != 8) {
-#pragma unroll
-        for (int t = 0; t < ROT_TERMS; ++t)
-            if (tid < ROT_THREADS) pk_late[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
-    }
-    build_lut<W, NW>(lut, a, tid);
-    float* qsh = reinterpret_cast<float*>(smem + LDS_QROWS);       // [G][128] floats; the rotated rows take this place later
-    if (stages_q) {
-        float qv[8];
-        convert_q8(qraw, a.q_dt, qv);
-        *reinterpret_cast<f4*>(qsh + 8 * tid) = (f4){qv[0], qv[1], qv[2], qv[3]};
-        *reinterpret_cast<f4*>(qsh + 8 * tid + 4) = (f4){qv[4], qv[5], qv[6], qv[7]};
-    }
-    lds_barrier();
-    rotate_partial<GP>(a, qsh, NW == 8 ? pk : pk_late, reinterpret_cast<float*>(smem + LDS_ROT), tid);
-    lds_barrier();
-    rotate_finish<GP, NW>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
-    lds_barrier();
-    // second buffer (not for the widest rows), requested before the first unit is used
-    Unit<W> nxt;
-    int nv1 = 0;
-    if constexpr (W != 8) {
-        nv1 = tokens_of(u + NW);
-        if (nv1 > 0) load_unit<W>(nxt, a, li, unit0 + u + NW, lane);
-    }
-    if (nvalid <= 0) return;
-    h8 qa[4];
-    load_queries(smem + LDS_QROWS, lane, 2 * GP, qa);
-    if constexpr (W == 8) {
-        while (true) {
-            compute_unit<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
-            u += NW;
-            nvalid = tokens_of(u);
-            if (nvalid <= 0) break;
-            load_unit<W>(cur, a, li, unit0 + u, lane);
+    // DEPTH units of this wavefront are under way at any time: two (one for the widest rows: registers); twelve
+    // wavefronts have the registers for a third 2-bit unit.  (Six units in flight with eight wavefronts were measured:
+    // no gain, the eight are bound by their arithmetic.)
+    constexpr int DEPTH = W == 8 ? 1 : (NW == 12 && W == 2) ? 3 : 2;
+    if constexpr (DEPTH <= 2) {
+        // two buffers, written out: the compiler schedules this form a microsecond per item better than the ring
+        Unit<W> cur;
+        int u = wave;
+        int nvalid = tokens_of(u);
+        if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
+        f4 pk_late[ROT_TERMS];
+        if constexpr (NW != 8) {
+    #pragma unroll
+            for (int t = 0; t < ROT_TERMS; ++t)
+                if (tid < ROT_THREADS) pk_late[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
         }
-    } else {
-        while (true) {
-            compute_unit<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
-            if (nv1 <= 0) break;
-            u += 2 * NW;
-            nvalid = tokens_of(u);
-            if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
-            compute_unit<W>(nxt, nv1, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
-            if (nvalid <= 0) break;
+        build_lut<W, NW>(lut, a, tid);
+        float* qsh = reinterpret_cast<float*>(smem + LDS_QROWS);       // [G][128] floats; the rotated rows take this place later
+        if (stages_q) {
+            float qv[8];
+            convert_q8(qraw, a.q_dt, qv);
+            *reinterpret_cast<f4*>(qsh + 8 * tid) = (f4){qv[0], qv[1], qv[2], qv[3]};
+            *reinterpret_cast<f4*>(qsh + 8 * tid + 4) = (f4){qv[4], qv[5], qv[6], qv[7]};
+        }
+        lds_barrier();
+        rotate_partial<GP>(a, qsh, NW == 8 ? pk : pk_late, reinterpret_cast<float*>(smem + LDS_ROT), tid);
+        lds_barrier();
+        rotate_finish<GP, NW>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
+        lds_barrier();
+        // second buffer (not for the widest rows), requested before the first unit is used
+        Unit<W> nxt;
+        int nv1 = 0;
+        if constexpr (W != 8) {
             nv1 = tokens_of(u + NW);
             if (nv1 > 0) load_unit<W>(nxt, a, li, unit0 + u + NW, lane);
+        }
+        if (nvalid <= 0) return;
+        h8 qa[4];
+        load_queries(smem + LDS_QROWS, lane, 2 * GP, qa);
+        if constexpr (W == 8) {
+            while (true) {
+                compute_unit<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
+                u += NW;
+                nvalid = tokens_of(u);
+                if (nvalid <= 0) break;
+                load_unit<W>(cur, a, li, unit0 + u, lane);
+            }
+        } else {
+            while (true) {
+                compute_unit<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
+                if (nv1 <= 0) break;
+                u += 2 * NW;
+                nvalid = tokens_of(u);
+                if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
+                compute_unit<W>(nxt, nv1, lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
+                if (nvalid <= 0) break;
+                nv1 = tokens_of(u + NW);
+                if (nv1 > 0) load_unit<W>(nxt, a, li, unit0 + u + NW, lane);
+            }
+        }
+    } else {
+        Unit<W> buf[DEPTH];
+        int nv[DEPTH];
+        nv[0] = tokens_of(wave);
+        if (nv[0] > 0) load_unit<W>(buf[0], a, li, unit0 + wave, lane);
+        f4 pk_late[ROT_TERMS];
+        if constexpr (NW != 8) {
+    #pragma unroll
+            for (int t = 0; t < ROT_TERMS; ++t)
+                if (tid < ROT_THREADS) pk_late[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
+        }
+        build_lut<W, NW>(lut, a, tid);
+        float* qsh = reinterpret_cast<float*>(smem + LDS_QROWS);       // [G][128] floats; the rotated rows take this place later
+        if (stages_q) {
+            float qv[8];
+            convert_q8(qraw, a.q_dt, qv);
+            *reinterpret_cast<f4*>(qsh + 8 * tid) = (f4){qv[0], qv[1], qv[2], qv[3]};
+            *reinterpret_cast<f4*>(qsh + 8 * tid + 4) = (f4){qv[4], qv[5], qv[6], qv[7]};
+        }
+        lds_barrier();
+        rotate_partial<GP>(a, qsh, NW == 8 ? pk : pk_late, reinterpret_cast<float*>(smem + LDS_ROT), tid);
+        lds_barrier();
+        rotate_finish<GP, NW>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
+        lds_barrier();
+        // the rest of the ring, requested before the first unit is used
+    #pragma unroll
+        for (int d = 1; d < DEPTH; ++d) {
+            nv[d] = tokens_of(wave + d * NW);
+            if (nv[d] > 0) load_unit<W>(buf[d], a, li, unit0 + wave + d * NW, lane);
+        }
+        if (nv[0] <= 0) return;
+        h8 qa[4];
+        load_queries(smem + LDS_QROWS, lane, 2 * GP, qa);
+        // units wave, wave + NW, ...: a unit's buffer is requested again as soon as it has been used
+        for (int u = wave;; u += DEPTH * NW) {
+    #pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                if (nv[d] <= 0) return;                         // the units of a wavefront run out in order
+                compute_unit<W>(buf[d], nv[d], lane, lut, slot4, qa, ksc, vsc, pbuf, alpha_sh, st);
+                const int nu = u + (d + DEPTH) * NW;
+                nv[d] = tokens_of(nu);
+                if (nv[d] > 0) load_unit<W>(buf[d], a, li, unit0 + nu, lane);
+            }
         }
     }
 }
@@ -943,8 +995,8 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     ODMKV_CHECK_ARG(((uintptr_t)q & 15) == 0, "decode_attn: the query must be 16-byte aligned");
     const int n_items = work->n_items;
     ODMKV_CHECK_ARG(n_items >= 0, "decode_attn: negative item count");
-    ODMKV_CHECK_ARG(work->wavefronts == 0 || work->wavefronts == 8 || work->wavefronts == 16,
-                    "decode_attn: %d wavefronts per work item (0, 8 or 16)", work->wavefronts);
+    ODMKV_CHECK_ARG(work->wavefronts == 0 || work->wavefronts == 8 || work->wavefronts == 12 || work->wavefronts == 16,
+                    "decode_attn: %d wavefronts per work item (0, 8, 12 or 16)", work->wavefronts);
     ODMKV_CHECK_ARG(work->item_range, "decode_attn: null item ranges");
     ODMKV_CHECK_ARG(n_items == 0 || work->items, "decode_attn: null work list");
     ODMKV_CHECK_ARG(B > 0 && Hq > 0 && store->B == B && store->Hkv > 0 && Hq % store->Hkv == 0,
@@ -971,12 +1023,16 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
         // when measuring, the events are attached to the dispatch itself: they carry the kernel's own
         // start and end timestamps, not those of separate marker packets
         hipEvent_t e0 = (hipEvent_t)ev_start, e1 = (hipEvent_t)ev_stop;
-        const bool wide = work->wavefronts == 16;
+        const int nw = work->wavefronts == 0 ? 8 : work->wavefronts;
         int rc;
-        if (GP == 4 && !a.order) rc = wide ? launch_main<4, false, 16>(a, n_items, e0, e1, st) : launch_main<4, false, 8>(a, n_items, e0, e1, st);
-        else if (GP == 4) rc = wide ? launch_main<4, true, 16>(a, n_items, e0, e1, st) : launch_main<4, true, 8>(a, n_items, e0, e1, st);
-        else if (!a.order) rc = wide ? launch_main<8, false, 16>(a, n_items, e0, e1, st) : launch_main<8, false, 8>(a, n_items, e0, e1, st);
-        else rc = wide ? launch_main<8, true, 16>(a, n_items, e0, e1, st) : launch_main<8, true, 8>(a, n_items, e0, e1, st);
+#define ODMKV_LAUNCH_MAIN(GPV, ORD) \
+        (nw == 16 ? launch_main<GPV, ORD, 16>(a, n_items, e0, e1, st) : nw == 12 ? launch_main<GPV, ORD, 12>(a, n_items, e0, e1, st) \
+                                                                     : launch_main<GPV, ORD, 8>(a, n_items, e0, e1, st))
+        if (GP == 4 && !a.order) rc = ODMKV_LAUNCH_MAIN(4, false);
+        else if (GP == 4) rc = ODMKV_LAUNCH_MAIN(4, true);
+        else if (!a.order) rc = ODMKV_LAUNCH_MAIN(8, false);
+        else rc = ODMKV_LAUNCH_MAIN(8, true);
+#undef ODMKV_LAUNCH_MAIN
         if (rc) return rc;
     }
     if (stage_mask & 4) {

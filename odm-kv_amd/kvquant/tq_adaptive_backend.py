@@ -566,7 +566,7 @@ class TurboQuantAdaptiveKVCacheState:
         are compared by the time a longest-first assignment of their items to the compute units
         would take, and the best is kept; when it has more items than compute units, the order in which
         the workgroups take the items (longest first) is handed to the kernel as well.  Items of sixteen
-        tiles and more on average are run by sixteen wavefronts, shorter ones by eight."""
+        tiles and more on average are run by sixteen (or twelve) wavefronts, shorter ones by eight."""
         import os
         n_cu = _compute_units(self.device)
         env_target = int(os.environ.get("ODMKV_DECODE_ITEMS", 0))
@@ -657,8 +657,14 @@ class TurboQuantAdaptiveKVCacheState:
         w.items, w.item_range = self._items[0].data_ptr(), self._items[1].data_ptr()
         w.dispatch_order = _lib.ptr(self._item_order)
         w.n_items = len(items)
+        # wavefronts per item: eight for short items (less set-up, a lighter combine); for long ones sixteen where
+        # the narrow levels carry the bytes (their loop wants four wavefronts per SIMD) and twelve where 4- and 8-bit
+        # tokens do (memory-bound: a third unit in flight per wavefront pays more than the fourth wavefront)
         quant = arr[arr[:, 1] < 4, 3] if len(items) else arr[:0, 3]
-        w.wavefronts = int(os.environ.get("ODMKV_DECODE_WAVES", 0)) or (16 if quant.size and quant.mean() >= 16 else 8)
+        q_bytes = [int(used[li].sum()) * _TILE_BYTES[li] for li in range(4)]
+        wide = (q_bytes[2] + q_bytes[3]) >= 0.4 * max(sum(q_bytes), 1)
+        auto = 8 if not (quant.size and quant.mean() >= 16) else (12 if wide else 16)
+        w.wavefronts = int(os.environ.get("ODMKV_DECODE_WAVES", 0)) or auto
         self._worklist = w
 
     def decode_attention(self, query: torch.Tensor, scaling: Optional[float] = None,
