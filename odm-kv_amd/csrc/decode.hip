@@ -831,120 +831,81 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
 // ------------------------------------------------------------------------------------------------
 #define MERGE_THREADS 512
 #define MERGE_SLICES (MERGE_THREADS / HD)
-#define MERGE_CHUNK 1024          // items whose weights are held in LDS at a time
+#define MERGE_CHUNK 64            // items merged per round: one per lane of a wavefront
 
 // MERGE_SPLIT: workgroups per query head (4 when there are few heads, so that the launch still covers the device;
 // 1 for large batches, where every further workgroup only repeats the reading)
 template <int GP, int MERGE_SPLIT>
 __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs a) {
-    __shared__ float wts[MERGE_CHUNK];               // exp2(m_item - M); the sign bit marks exact items
-    __shared__ float red[MERGE_THREADS / 64];
     __shared__ float part[2][MERGE_SLICES][HD];      // [rotated | exact][slice][dim]
-    __shared__ float rot[HD];
-    __shared__ float Lsh;
-    // MERGE_SPLIT workgroups per query head: each merges the head's partial results in full (they are small and
-    // shared through the caches) and rotates back a quarter of the output dims, so that no workgroup has to pull
-    // the whole 64 KB rotation through one compute unit
-    const int bq = blockIdx.x / MERGE_SPLIT, quarter = blockIdx.x % MERGE_SPLIT;
-    const int tid = threadIdx.x, j = tid & (HD - 1), slice = tid >> 7;
-    const int b = bq / a.Hq, hq = bq % a.Hq;
-    const int bh = b * a.s.Hkv + hq / a.G, g = hq % a.G;
-    const int i0 = a.item_range[bh], n = a.item_range[bh + 1] - i0;
-    // Everything that does not depend on the weights is requested now, in one round trip: this thread's
-    // share of the value rotation, the first MERGE_PRE accumulator values of its slice, its item's (m, l, level)
     constexpr int QD = HD / MERGE_SPLIT;                 // output dims of this workgroup
     constexpr int RS = MERGE_THREADS / QD;                // row slices of the rotation
     constexpr int IN = HD / RS;                           // rows per slice
+    __shared__ float part2[RS * QD];
+    // MERGE_SPLIT workgroups per query head: each merges the head's partial results in full (they are small and
+    // shared through the caches) and rotates back its share of the output dims, so that no workgroup has to pull
+    // the whole 64 KB rotation through one compute unit
+    const int bq = blockIdx.x / MERGE_SPLIT, quarter = blockIdx.x % MERGE_SPLIT;
+    const int tid = threadIdx.x, lane = tid & 63, j = tid & (HD - 1);
+    const int slice = __builtin_amdgcn_readfirstlane(tid >> 7);
+    const int b = bq / a.Hq, hq = bq % a.Hq;
+    const int bh = b * a.s.Hkv + hq / a.G, g = hq % a.G;
+    const int i0 = a.item_range[bh], n = a.item_range[bh + 1] - i0;
+    // this thread's share of the value rotation: requested first, it does not depend on the items
     const int jj = tid % QD, rs = tid / QD;
     float pv[IN];
 #pragma unroll
     for (int ii = 0; ii < IN; ++ii) pv[ii] = a.pi_v[(size_t)(rs * IN + ii) * HD + quarter * QD + jj];
-    constexpr int MERGE_PRE = 16;
-    float pre[MERGE_PRE];
-#pragma unroll
-    for (int k = 0; k < MERGE_PRE; ++k) {
-        const int it = slice + k * MERGE_SLICES;
-        pre[k] = it < n ? a.partial[((size_t)(i0 + it) * GP + g) * PSTRIDE + j] : 0.0f;
-    }
-    float my_m = -INFINITY, my_l = 0.0f;
-    int my_level = 0;
-    if (tid < n) {
-        const float* p = a.partial + ((size_t)(i0 + tid) * GP + g) * PSTRIDE;
-        my_m = p[HD]; my_l = p[HD + 1];
-        my_level = a.items[8 * (i0 + tid) + 1];
-    }
-    // maximum over all the items
-    float mx = my_m;
-    for (int it = tid + MERGE_THREADS; it < n; it += MERGE_THREADS)
-        mx = fmaxf(mx, a.partial[((size_t)(i0 + it) * GP + g) * PSTRIDE + HD]);
-    mx = wave_max(mx);
-    if ((tid & 63) == 0) red[tid >> 6] = mx;
-    __syncthreads();
-    float M = red[0];
-#pragma unroll
-    for (int w = 1; w < MERGE_THREADS / 64; ++w) M = fmaxf(M, red[w]);
-    __syncthreads();
-    // weights, the normaliser and the weighted sums, MERGE_CHUNK items at a time (one round for the usual work list)
-    float lpart = 0.0f, arot = 0.0f, aex = 0.0f;
+    // The items are merged MERGE_CHUNK at a time with a running maximum, like an online softmax.  Inside a round
+    // nothing crosses wavefronts: lane i of every wavefront holds item i's (m, l, level), the maximum and the
+    // normaliser come from wave reductions, and the weight of the item a wavefront is adding (the same item for the
+    // whole wavefront) is read from its lane.  Every wavefront thus repeats the few scalars and no barrier is needed.
+    float M = -INFINITY, L = 0.0f, arot = 0.0f, aex = 0.0f;
     for (int c0 = 0; c0 < n; c0 += MERGE_CHUNK) {
         const int nc = min(n - c0, MERGE_CHUNK);
-        if (c0 == 0 && tid < nc) {
-            const float f = M > -INFINITY ? __builtin_amdgcn_exp2f(my_m - M) : 0.0f;
-            lpart = my_l * f;
-            wts[tid] = my_level == 4 ? -f : f;
+        float m_i = -INFINITY, l_i = 0.0f;
+        int level = 0;
+        if (lane < nc) {
+            const float* p = a.partial + ((size_t)(i0 + c0 + lane) * GP + g) * PSTRIDE;
+            m_i = p[HD]; l_i = p[HD + 1];
+            level = a.items[8 * (i0 + c0 + lane) + 1];
         }
-        for (int it = tid + (c0 == 0 ? MERGE_THREADS : 0); it < nc; it += MERGE_THREADS) {
-            const float* p = a.partial + ((size_t)(i0 + c0 + it) * GP + g) * PSTRIDE;
-            const float f = M > -INFINITY ? __builtin_amdgcn_exp2f(p[HD] - M) : 0.0f;
-            lpart = __fmaf_rn(p[HD + 1], f, lpart);
-            wts[it] = a.items[8 * (i0 + c0 + it) + 1] == 4 ? -f : f;
-        }
-        __syncthreads();                                   // weights written
-        int first = slice;
-        if (c0 == 0) {
+        float vals[MERGE_CHUNK / MERGE_SLICES];
 #pragma unroll
-            for (int k = 0; k < MERGE_PRE; ++k) {
-                const int it = slice + k * MERGE_SLICES;
-                if (it < nc) {
-                    const float w = wts[it];
-                    if (__float_as_uint(w) >> 31) aex = __fmaf_rn(pre[k], -w, aex);
-                    else arot = __fmaf_rn(pre[k], w, arot);
-                }
+        for (int k = 0; k < MERGE_CHUNK / MERGE_SLICES; ++k) {
+            const int it = slice + k * MERGE_SLICES;
+            vals[k] = it < nc ? a.partial[((size_t)(i0 + c0 + it) * GP + g) * PSTRIDE + j] : 0.0f;
+        }
+        const float Mc = fmaxf(M, wave_max(m_i));
+        const float f_old = M > -INFINITY ? __builtin_amdgcn_exp2f(M - Mc) : 0.0f;
+        const float w = m_i > -INFINITY ? __builtin_amdgcn_exp2f(m_i - Mc) : 0.0f;
+        L = __fmaf_rn(L, f_old, wave_sum(l_i * w));
+        arot *= f_old; aex *= f_old;
+        const int wsgn = __float_as_int(level == 4 ? -w : w);          // the sign bit marks exact items
+#pragma unroll
+        for (int k = 0; k < MERGE_CHUNK / MERGE_SLICES; ++k) {
+            const int it = slice + k * MERGE_SLICES;                     // wave-uniform
+            if (it < nc) {
+                const float ww = __int_as_float(__builtin_amdgcn_readlane(wsgn, it));
+                if (__float_as_uint(ww) >> 31) aex = __fmaf_rn(vals[k], -ww, aex);
+                else arot = __fmaf_rn(vals[k], ww, arot);
             }
-            first = slice + MERGE_PRE * MERGE_SLICES;
         }
-#pragma unroll 4
-        for (int it = first; it < nc; it += MERGE_SLICES) {
-            const float w = wts[it];
-            const float v = a.partial[((size_t)(i0 + c0 + it) * GP + g) * PSTRIDE + j];
-            if (__float_as_uint(w) >> 31) aex = __fmaf_rn(v, -w, aex);
-            else arot = __fmaf_rn(v, w, arot);
-        }
-        __syncthreads();                                   // the weights are overwritten by the next round
+        M = Mc;
     }
-    lpart = wave_sum(lpart);
-    if ((tid & 63) == 0) red[tid >> 6] = lpart;
     part[0][slice][j] = arot;
     part[1][slice][j] = aex;
-    __syncthreads();
-    if (tid == 0) {
-        float L = 0.0f;
-        for (int w = 0; w < MERGE_THREADS / 64; ++w) L += red[w];
-        Lsh = L;
-    }
-    if (tid < HD) {
-        float r = 0.0f;
-#pragma unroll
-        for (int s = 0; s < MERGE_SLICES; ++s) r += part[0][s][tid];
-        rot[tid] = r;
-    }
     __syncthreads();
     // rotate the quantised part back: out_j = sum_i rot_i Pi_v[i][j] for this workgroup's dims; the slices split the i range
     float o = 0.0f;
 #pragma unroll
-    for (int ii = 0; ii < IN; ++ii) o = __fmaf_rn(rot[rs * IN + ii], pv[ii], o);
-    __syncthreads();
-    float* part2 = &part[0][0][0];                        // [RS][QD], the first half of `part` is free again
+    for (int ii = 0; ii < IN; ++ii) {
+        const int i = rs * IN + ii;
+        float r = part[0][0][i];
+#pragma unroll
+        for (int sl = 1; sl < MERGE_SLICES; ++sl) r += part[0][sl][i];
+        o = __fmaf_rn(r, pv[ii], o);
+    }
     part2[rs * QD + jj] = o;
     __syncthreads();
     if (tid < QD) {
@@ -953,8 +914,7 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
 #pragma unroll
         for (int r = 0; r < RS; ++r) tot += part2[r * QD + tid];
 #pragma unroll
-        for (int s = 0; s < MERGE_SLICES; ++s) tot += part[1][s][dim];
-        const float L = Lsh;
+        for (int sl = 0; sl < MERGE_SLICES; ++sl) tot += part[1][sl][dim];
         const float o32 = L > 0.0f ? tot / L : 0.0f;
         const size_t oi = (size_t)bq * HD + dim;
         if (a.out_dt == ODMKV_F32) reinterpret_cast<float*>(a.out)[oi] = o32;
