@@ -79,3 +79,11 @@ extern "C" int odmkv_bench_probe_read(const void* buf, size_t bytes, int grid, v
     ODMKV_CHECK_LAUNCH("probe_read_kernel");
     return 0;
 }
+
+extern "C" int odmkv_bench_pack_handed_over(const void* workspace, int B, int Hkv, int T, int32_t* counts, void* stream) {
+    ODMKV_CHECK_ARG(workspace && counts && B > 0 && Hkv > 0 && T > 0, "bench_pack_handed_over: bad arguments");
+    const char* p = (const char*)workspace + pack_redo_offset(B * Hkv, T);
+    ODMKV_CHECK_HIP(hipMemcpyAsync(counts, p, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    ODMKV_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}

@@ -44,6 +44,8 @@ void odmkv_set_error(const char* fmt, ...);
     } while (0)
 
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+// pack.hip: byte offset, inside the pack workspace, of the list of tiles the fp16 quantiser hands to the exact one
+size_t pack_redo_offset(int nseg, int T);
 
 // level index of a bit width: 0 -> evicted, 2,3,4,8 -> 1..4, 16 -> 5; anything else -> -1
 __host__ __device__ static inline int level_slot(int bits) {

@@ -11,7 +11,8 @@
 // ------------------------------------------------------------------------------------------------
 // level counts
 // ------------------------------------------------------------------------------------------------
-#define LC_THREADS 1024
+#define LC_THREADS 256
+#define LC_CHUNK 4096           // tokens per workgroup
 
 __device__ static inline int wave_sum_i32(int v) {
 #pragma unroll
@@ -19,46 +20,68 @@ __device__ static inline int wave_sum_i32(int v) {
     return v;
 }
 
+// 6-bit counters of the six levels in one 64-bit word; a value that is no level adds nothing.
+// nibble b of the table = level index + 1 of bit width b (0: none); 16 is handled apart.
+__device__ static inline unsigned long long level_increment(int bits) {
+    const unsigned long long table = 0x0000000500043201ull;      // widths 0, 2, 3, 4, 8 -> 1, 2, 3, 4, 5
+    const unsigned int ub = (unsigned int)bits;
+    const unsigned int code = ub == 16u ? 6u : ub < 16u ? (unsigned int)(table >> (4 * ub)) & 15u : 0u;
+    return code ? 1ull << (6 * (code - 1)) : 0ull;
+}
+
+// grid (chunks, rows): every workgroup adds its chunk's counts to the row's six counters (cleared by the
+// launch before this one)
 __global__ __launch_bounds__(LC_THREADS) void level_counts_kernel(const int32_t* __restrict__ bits, int T,
                                                                   int32_t* __restrict__ counts) {
     __shared__ int c[6];
-    const int bh = blockIdx.x, tid = threadIdx.x;
+    const int bh = blockIdx.y, tid = threadIdx.x;
     if (tid < 6) c[tid] = 0;
     __syncthreads();
-    int local[6] = {0, 0, 0, 0, 0, 0};
     const int32_t* row = bits + (size_t)bh * T;
-    const bool vec = (T % 4 == 0) && ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
+    const int t0 = blockIdx.x * LC_CHUNK;
+    const int n = min(T - t0, LC_CHUNK);
+    unsigned long long acc = 0ull;                       // at most 16 per thread and field
+    const bool vec = ((reinterpret_cast<uintptr_t>(row + t0) & 15) == 0);
     if (vec) {
-        const int4* row4 = reinterpret_cast<const int4*>(row);
-        for (int q = tid; q < T / 4; q += LC_THREADS) {
-            const int4 v = row4[q];
-            const int s4[4] = {level_slot(v.x), level_slot(v.y), level_slot(v.z), level_slot(v.w)};
+        const int4* p = reinterpret_cast<const int4*>(row + t0);
+        int4 v[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-#pragma unroll
-                for (int k = 0; k < 6; ++k) local[k] += (s4[e] == k);
+        for (int u = 0; u < 4; ++u) {
+            const int q = u * LC_THREADS + tid;
+            v[u] = 4 * q + 3 < n ? p[q] : make_int4(-1, -1, -1, -1);
         }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            acc += level_increment(v[u].x) + level_increment(v[u].y) + level_increment(v[u].z) + level_increment(v[u].w);
+        for (int t = (n & ~3) + tid; t < n; t += LC_THREADS) acc += level_increment(row[t0 + t]);
     } else {
-        for (int t = tid; t < T; t += LC_THREADS) {
-            const int sl = level_slot(row[t]);
-#pragma unroll
-            for (int k = 0; k < 6; ++k) local[k] += (sl == k);
-        }
+        for (int t = tid; t < n; t += LC_THREADS) acc += level_increment(row[t0 + t]);
     }
 #pragma unroll
     for (int k = 0; k < 6; ++k) {
-        const int w = wave_sum_i32(local[k]);
+        const int w = wave_sum_i32((int)((acc >> (6 * k)) & 63ull));
         if ((tid & 63) == 0 && w) atomicAdd(&c[k], w);
     }
     __syncthreads();
-    if (tid < 6) counts[bh * 6 + tid] = c[tid];
+    if (tid < 6 && c[tid]) atomicAdd(&counts[bh * 6 + tid], c[tid]);
+}
+
+__global__ void level_counts_clear_kernel(int32_t* __restrict__ counts, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) counts[i] = 0;
 }
 
 extern "C" int odmkv_level_counts(const int32_t* bits, int B, int Hkv, int T, int32_t* counts,
                                   void* stream) {
     ODMKV_CHECK_ARG(bits && counts, "level_counts: null pointer");
     ODMKV_CHECK_ARG(B > 0 && Hkv > 0 && T >= 0, "level_counts: bad shape B=%d Hkv=%d T=%d", B, Hkv, T);
-    hipLaunchKernelGGL(level_counts_kernel, dim3(B * Hkv), dim3(LC_THREADS), 0, (hipStream_t)stream, bits, T, counts);
+    ODMKV_CHECK_ARG(B * Hkv <= 65535, "level_counts: at most 65535 (sequence, head) pairs per call");
+    // a fill kernel, not a memset: callers may capture this call in a graph
+    hipLaunchKernelGGL(level_counts_clear_kernel, dim3((B * Hkv * 6 + 255) / 256), dim3(256), 0, (hipStream_t)stream, counts, B * Hkv * 6);
+    ODMKV_CHECK_LAUNCH("level_counts_clear_kernel");
+    if (T == 0) return 0;
+    hipLaunchKernelGGL(level_counts_kernel, dim3((T + LC_CHUNK - 1) / LC_CHUNK, B * Hkv), dim3(LC_THREADS), 0, (hipStream_t)stream,
+                       bits, T, counts);
     ODMKV_CHECK_LAUNCH("level_counts_kernel");
     return 0;
 }
@@ -80,6 +103,7 @@ struct CompactArgs {
     int32_t* seg_count[5];
     int32_t* old_count;     // [5][nseg]
     int32_t* chunk_count;   // [nseg][n_chunks][5]
+    int32_t* redo;          // two counters the quantise kernels use, cleared here (may be null)
 };
 
 // levels (1..5, 0 = evicted, -1 = past the end) of the 8 consecutive tokens this thread owns
@@ -102,6 +126,7 @@ __global__ __launch_bounds__(CP_THREADS) void chunk_count_kernel(CompactArgs a) 
     const int bh = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     if (tid < 5) c[tid] = 0;
     if (chunk == 0 && tid < 5) a.old_count[tid * a.nseg + bh] = a.seg_count[tid][bh];
+    if (a.redo && chunk == 0 && bh == 0 && tid < 2) a.redo[tid] = 0;
     __syncthreads();
     int sl[CP_TPT];
     load_slots(a, bh, chunk * CP_TOKENS + tid * CP_TPT, sl);
@@ -196,6 +221,11 @@ struct QuantArgs {
     const float* cb;             // centroids of widths 2, 3, 4, 8 back to back
     const int32_t* old_count;    // [5][nseg]
     int tile_base[ODMKV_NQ + 1]; // running sum of the levels' tile counts
+    // Tiles handed from the fp16 kernel to this one: redo[0] / redo[1] = number of key / value tiles,
+    // then redo_cap key tile numbers and redo_cap value tile numbers.  The fp16 kernel appends; with
+    // from_list set the exact kernel walks the lists instead of all tiles.
+    int32_t* redo;
+    int redo_cap, from_list;
     odmkv_packed_t s;
 };
 
@@ -508,6 +538,9 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);          // wave-uniform: keep it in a scalar register
     uint8_t* stage = smem + QP_PI_BYTES + wave * QP_STAGE;
     const bool is_v = (blockIdx.x & 1) != 0;
+    const int32_t* tile_list = a.from_list ? a.redo + 2 + (is_v ? a.redo_cap : 0) : nullptr;
+    const int n_work = a.from_list ? min(a.redo[is_v ? 1 : 0], a.redo_cap) : a.tile_base[ODMKV_NQ];
+    if (n_work == 0) return;                                            // nothing handed over: the usual case
 
     // rotation -> LDS, transposed.  Keys: slot = output index.  Values: slot 4c+g holds output
     // g*32+c, so that a lane's four accumulators are 32 outputs apart and its registers hold four
@@ -527,9 +560,9 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
     }
     __syncthreads();
 
-    const int total_tiles = a.tile_base[ODMKV_NQ];
     const int wg = blockIdx.x >> 1, n_wg = gridDim.x >> 1;
-    for (int gt = wg * NW + wave; gt < total_tiles; gt += n_wg * NW) {
+    for (int wi = wg * NW + wave; wi < n_work; wi += n_wg * NW) {
+        const int gt = tile_list ? tile_list[wi] : wi;
         int li = 0;
 #pragma unroll
         for (int k = 1; k < ODMKV_NQ; ++k) li += (gt >= a.tile_base[k]);
@@ -720,6 +753,462 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// quantise + pack, fp16 inputs: rotation on the fp16 matrix cores, exact codes through a guard band
+//
+// A code is the number of decision thresholds at or below y = sum_j u_j Pi[i][j] (summed in the
+// sequential fp32 order of the definition).  The chain of 128 dependent fp32 steps is what the exact
+// kernel above spends its time on, yet the chain's last bits matter only when y lies next to a
+// threshold.  So y is first computed fast: the fp16 row as it is, against Pi split into two fp16
+// terms (hi + lo, 22 bits), on v_mfma_f32_16x16x32_f16, then scaled by 1 / (|x| + 1e-10).  That
+// estimate differs from the chain's result by rounding alone: at most about 2.5e-5 on the scale
+// |y| <= 1 under the most pessimistic model of the matrix unit's adder (every one of the 128 terms
+// truncated at the scale of the largest partial sum), and about 1e-6 in practice.  Values farther
+// than QF_BAND from every threshold therefore have the chain's code already; the few within the band
+// (two to eight in a thousand) are listed, and whenever a wave has 64 of them it recomputes them by
+// the chain itself, one lane per value, and replaces their codes in the packed tiles it has already
+// written.  Rows of zeros are exact either way.
+// Tiles the scheme does not cover go to the exact kernel through a list: 8-bit tiles (a tenth of
+// their values lie inside the band), tiles with a row whose squared norm is not finite, and tiles
+// with more listed values than the list has room for.
+//
+// Operands: for keys D = Pi (rows) x tokens (columns), so a lane ends with four consecutive outputs
+// of one token; for values the same registers with the operands swapped give D = tokens x outputs
+// and four consecutive tokens of one output: in both cases the 4*W bits that are neighbours in the
+// packed stream, as the staging formats of the exact kernel expect them.
+// ------------------------------------------------------------------------------------------------
+typedef _Float16 qf_h8 __attribute__((ext_vector_type(8)));
+typedef float qf_f4 __attribute__((ext_vector_type(4)));
+
+#define QF_BAND 1.0e-4f
+#define QF_LIST 256                     // listed values a wave can hold (it works them off 64 at a time)
+#define QF_GT_BITS 19                   // tile numbers in a list entry
+#define QF_NW 8
+#define QF_PI_BYTES (2 * HD * HD * 2)   // Pi as fp16 hi and lo, in matrix-operand order
+#define QF_THR_BYTES 1152               // QP_THR_FLOATS floats, padded to a multiple of 16
+
+struct QfWave {                          // per-wave scratch in LDS
+    unsigned long long off[TILE];        // element offset of the token's row (~0: no row, zeros)
+    float den[TILE], rinv[TILE], band[TILE];
+    uint32_t list[QF_LIST];              // slot in the tile | output << 6 | tile number << 13
+    int count, pad[3];
+};
+
+template <int W> struct GuardCoder {
+    static constexpr int K = 1 << W;
+    float t[(W <= 3) ? K - 1 : 1];
+    const float* thr;
+    __device__ inline GuardCoder(const float* thr_li) : thr(thr_li) {
+        if constexpr (W <= 3) {
+#pragma unroll
+            for (int k = 0; k < K - 1; ++k) t[k] = thr_li[k];
+        }
+    }
+    // r * 2^W + code(y), and m = distance from y to the nearest threshold: the binary search meets
+    // both neighbours of y on its way, so the minimum over the thresholds it compares with is exact
+    __device__ __forceinline__ uint32_t push(uint32_t r, float y, float& m) const {
+        if constexpr (W == 2) {
+            const bool b1 = y >= t[1];
+            r = r + r + (b1 ? 1u : 0u);
+            const float ts = b1 ? t[2] : t[0];
+            const bool b0 = y >= ts;
+            m = fminf(fabsf(y - t[1]), fabsf(y - ts));
+            return r + r + (b0 ? 1u : 0u);
+        } else if constexpr (W == 3) {
+            const bool b2 = y >= t[3];
+            r = r + r + (b2 ? 1u : 0u);
+            const float ta = b2 ? t[5] : t[1];
+            const bool b1 = y >= ta;
+            r = r + r + (b1 ? 1u : 0u);
+            const float lo_pair = b1 ? t[2] : t[0], hi_pair = b1 ? t[6] : t[4];
+            const float tb = b2 ? hi_pair : lo_pair;
+            const bool b0 = y >= tb;
+            m = fminf(fminf(fabsf(y - t[3]), fabsf(y - ta)), fabsf(y - tb));
+            return r + r + (b0 ? 1u : 0u);
+        } else {
+            int pos = 0;
+            m = INFINITY;
+#pragma unroll
+            for (int s = K / 2; s >= 1; s >>= 1) {
+                const float tv = thr[pos + s - 1];
+                m = fminf(m, fabsf(y - tv));
+                if (y >= tv) pos += s;
+            }
+            return (r << W) | (uint32_t)pos;
+        }
+    }
+};
+
+// rotation estimate -> codes into the staging area; values inside the band -> the wave's list
+template <int W, bool IS_V, bool DIRECT>
+__device__ static __forceinline__ void qf_code_tile(const void* base, const uint4* piA, const float* thr, QfWave& w,
+                                                    uint8_t* stage, int lane, int gt) {
+    const int r16 = lane & 15, q = lane >> 4;
+    const GuardCoder<W> code(thr);
+    constexpr int NT = IS_V ? 16 : 4;
+    float rinv[NT], band[NT];
+    uint4 xb[4][4];
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+        if constexpr (IS_V) {
+            const float4 ri = *reinterpret_cast<const float4*>(&w.rinv[16 * tb + 4 * q]);
+            const float4 bd = *reinterpret_cast<const float4*>(&w.band[16 * tb + 4 * q]);
+            rinv[4 * tb] = ri.x; rinv[4 * tb + 1] = ri.y; rinv[4 * tb + 2] = ri.z; rinv[4 * tb + 3] = ri.w;
+            band[4 * tb] = bd.x; band[4 * tb + 1] = bd.y; band[4 * tb + 2] = bd.z; band[4 * tb + 3] = bd.w;
+        } else {
+            rinv[tb] = w.rinv[16 * tb + r16];
+            band[tb] = w.band[16 * tb + r16];
+        }
+        const unsigned long long o = w.off[16 * tb + r16];
+        const uint4* row = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) + (o == ~0ull ? 0ull : o)) + q;
+#pragma unroll
+        for (int ch = 0; ch < 4; ++ch) xb[tb][ch] = (o == ~0ull) ? make_uint4(0u, 0u, 0u, 0u) : row[4 * ch];
+    }
+#pragma unroll 1
+    for (int k = 0; k < 4; ++k) {
+        uint32_t f = 0u;                                        // band flags of this pair of output blocks, first value on top
+#pragma unroll
+        for (int o2 = 0; o2 < 2; ++o2) {
+            const int ob = 2 * k + o2;
+            qf_f4 acc[4];
+#pragma unroll
+            for (int tb = 0; tb < 4; ++tb) acc[tb] = (qf_f4){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int ch = 0; ch < 4; ++ch) {
+                const qf_h8 ah = __builtin_bit_cast(qf_h8, piA[(ob * 4 + ch) * 64 + lane]);
+                const qf_h8 al = __builtin_bit_cast(qf_h8, piA[HD * HD / 8 + (ob * 4 + ch) * 64 + lane]);
+#pragma unroll
+                for (int tb = 0; tb < 4; ++tb) {
+                    const qf_h8 xh = __builtin_bit_cast(qf_h8, xb[tb][ch]);
+                    if constexpr (IS_V) {
+                        acc[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, ah, acc[tb], 0, 0, 0);
+                        acc[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, al, acc[tb], 0, 0, 0);
+                    } else {
+                        acc[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, xh, acc[tb], 0, 0, 0);
+                        acc[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, xh, acc[tb], 0, 0, 0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int tb = 0; tb < 4; ++tb) {
+                uint32_t g = 0u;
+#pragma unroll
+                for (int r = 3; r >= 0; --r) {
+                    const float y = acc[tb][r] * (IS_V ? rinv[4 * tb + r] : rinv[tb]);
+                    float m;
+                    if constexpr (DIRECT) g = code.push(g, y, m);
+                    else g = (g << 8) | code.push(0u, y, m);
+                    const bool near = m < (IS_V ? band[4 * tb + r] : band[tb]);
+                    f = f + f + (near ? 1u : 0u);
+                }
+                if constexpr (!IS_V) {
+                    const int token = 16 * tb + r16, grp = 4 * ob + q;
+                    if constexpr (DIRECT) put_group<W>(stage + token * Direct<W>::ROW_K + grp * Direct<W>::GROUP_BYTES, g);
+                    else *reinterpret_cast<uint32_t*>(stage + token * CODE_ROW + 4 * grp) = g;
+                } else {
+                    const int dim = 16 * ob + r16, tg = 4 * tb + q;
+                    if constexpr (DIRECT) put_group<W>(stage + dim * Direct<W>::ROW_V + tg * Direct<W>::GROUP_BYTES, g);
+                    else *reinterpret_cast<uint32_t*>(stage + dim * CODE_ROW_T + 4 * tg) = g;
+                }
+            }
+        }
+        while (f) {                                             // rare: a few values per lane and tile
+            const int b = 31 - __clz(f);
+            f &= ~(1u << b);
+            const int v = 31 - b;                               // v = o2*16 + tb*4 + (3 - r)
+            const int ob = 2 * k + (v >> 4), tb = (v >> 2) & 3, r = 3 - (v & 3);
+            const int token = IS_V ? 16 * tb + 4 * q + r : 16 * tb + r16;
+            const int out = IS_V ? 16 * ob + r16 : 16 * ob + 4 * q + r;
+            const int idx = atomicAdd(&w.count, 1);
+            if (idx < QF_LIST) w.list[idx] = (uint32_t)token | ((uint32_t)out << 6) | ((uint32_t)gt << 13);
+        }
+    }
+}
+
+// Entries first .. first + n - 1 of the wave's list (n <= 64), a lane each: the value by the definition's
+// own chain, its code, and that code in place of the estimate's in the packed tile.  The tile's codes,
+// positions and norms were written by this wave: the caller has waited for those stores.
+template <bool IS_V>
+__device__ static void qf_fix_listed(const QuantArgs& a, const float* thrs, const QfWave& w, int lane, int first, int n) {
+    const bool on = lane < n;
+    const uint32_t e = w.list[first + (on ? lane : 0)];
+    const int token = e & 63, out = (e >> 6) & 127, gt = (int)(e >> 13);
+    int li = 0;
+#pragma unroll
+    for (int k = 1; k < ODMKV_NQ; ++k) li += (gt >= a.tile_base[k]);
+    const int tile = gt - a.tile_base[li];
+    const int bh = find_segment(a.s.seg_tile[li], a.nseg, tile);
+    const size_t slot = (size_t)tile * TILE + token;
+    const size_t off = (size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH +
+                       (size_t)(a.s.pos[li][slot] - a.pos_offset) * a.sT;
+    // written by this wave a moment ago: read past the vector cache
+    const float den = __hip_atomic_load((IS_V ? a.s.vnorm[li] : a.s.knorm[li]) + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1e-10f;
+    RowRegs<ODMKV_F16> x;
+    x.load(IS_V ? a.V : a.K, off);
+    const float4* __restrict__ prow = reinterpret_cast<const float4*>((IS_V ? a.pi_v : a.pi_k) + out * HD);
+    float y = 0.0f;
+    const bool row_plain = !(den >= 9.094947017729282e-13f && den <= 1.152921504606847e18f);
+    if (!__any(row_plain)) {                                    // same quotient sequence as the exact kernel
+        const float r0 = __builtin_amdgcn_rcpf(den);
+        const float rr = __fmaf_rn(__fmaf_rn(-den, r0, 1.0f), r0, r0);
+        const float nden = -den;
+#pragma unroll
+        for (int c = 0; c < HD / 4; ++c) {
+            const float4 p = prow[c];
+            const float pv[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const float nv = x.get(4 * c + e4);
+                const float q0 = __fmul_rn(nv, rr);
+                const float q1 = __fmaf_rn(__fmaf_rn(nden, q0, nv), rr, q0);
+                const float u = __fmaf_rn(__fmaf_rn(nden, q1, nv), rr, q1);
+                y = __fmaf_rn(u, pv[e4], y);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < HD / 4; ++c) {
+            const float4 p = prow[c];
+            const float pv[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) y = __fmaf_rn(x.get(4 * c + e4) / den, pv[e4], y);
+        }
+    }
+    // code = number of thresholds at or below y; the entries of a pass may be of different widths
+    const int W = width_of(li);
+    const float* thr = thrs + thr_offset(li);
+    int code = 0;
+#pragma unroll
+    for (int st = 8; st >= 1; st >>= 1)
+        if (st < (1 << W) && y >= thr[code + st - 1]) code += st;
+    if (!on) return;
+    // where the code lives (quant.h: tile layouts): lane l of the tile, code number ci of its stream
+    int l, ci;
+    if constexpr (!IS_V) {
+        const int b = 2 * (token >> 5) + (token & 1), nn = 4 * ((token >> 3) & 3) + ((token >> 1) & 3);   // token = key_slot(nn, b)
+        l = 16 * (out >> 5) + nn;
+        ci = 32 * b + (out & 31);
+    } else {
+        l = 16 * ((token >> 3) & 3) + (out & 15);
+        ci = 64 * (token >> 5) + 8 * (out >> 4) + (token & 7);
+    }
+    uint8_t* tile_codes = (IS_V ? a.s.vcodes[li] : a.s.kcodes[li]) + (size_t)tile * (TILE * 16 * W);
+    const int bit = ci * W, k = bit >> 5, sh = bit & 31;
+    uint32_t* word = reinterpret_cast<uint32_t*>(tile_codes + ((size_t)(k >> 2) * TILE + l) * 16) + (k & 3);
+    const uint32_t mask = (1u << W) - 1u;
+    uint32_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> sh;
+    uint32_t* word2 = nullptr;
+    if (sh + W > 32) {                                          // a 3-bit code across two words of the stream
+        const int k2 = k + 1;
+        word2 = reinterpret_cast<uint32_t*>(tile_codes + ((size_t)(k2 >> 2) * TILE + l) * 16) + (k2 & 3);
+        old |= __hip_atomic_load(word2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) << (32 - sh);
+    }
+    const uint32_t diff = (old & mask) ^ (uint32_t)code;
+    if (diff) {
+        atomicXor(word, diff << sh);                            // other lanes may change other codes of the same word
+        if (word2) atomicXor(word2, diff >> (32 - sh));
+    }
+}
+
+// the staged codes packed into the store
+template <int W, bool IS_V, bool DIRECT>
+__device__ static __forceinline__ void qf_store_tile(const QuantArgs& a, const uint8_t* stage, int lane, int li, int tile, int lo) {
+    uint8_t* codes = IS_V ? a.s.vcodes[li] : a.s.kcodes[li];
+    if constexpr (!IS_V) {
+        if constexpr (DIRECT) store_direct_k<W>(stage, codes, tile, lane);
+        else if (lo > 0) pack_store_k<W, true>(stage, codes, tile, lane, lo);
+        else pack_store_k<W, false>(stage, codes, tile, lane, 0);
+    } else {
+        if constexpr (DIRECT) store_direct_v<W>(stage, codes, tile, lane);
+        else if (lo > 0) pack_store_v<W, true>(stage, codes, tile, lane, lo);
+        else pack_store_v<W, false>(stage, codes, tile, lane, 0);
+    }
+}
+
+struct QfTile { int gt, li, tile, bh, lo, hi; };
+
+// Per wave the tiles form a pipeline: while tile n is coded, the token positions of tile n + 1 are on
+// their way; its rows are asked for before tile n's listed values are recomputed and its codes packed,
+// and are there when the next round starts.  Only the reads that depend on the tile's own results
+// (the matrix-layout reload, which hits the cache, and the rows of the listed values) are waited for.
+template <bool IS_V>
+__device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float* thrs, QfWave& w, uint8_t* stage,
+                               int lane, int wave) {
+    const int total_tiles = a.tile_base[ODMKV_NQ];
+    const int stride = (gridDim.x >> 1) * QF_NW;
+    int32_t* redo_count = a.redo + (IS_V ? 1 : 0);
+    int32_t* redo_list = a.redo + 2 + (IS_V ? a.redo_cap : 0);
+    const void* base = IS_V ? a.V : a.K;
+    const auto hand_over = [&](int gt) {
+        if (lane == 0) {
+            const int k = atomicAdd(redo_count, 1);
+            if (k < a.redo_cap) redo_list[k] = gt;
+        }
+    };
+    // the next tile at or behind gt with new tokens of widths 2, 3, 4; 8-bit tiles on the way are handed over
+    const auto next_tile = [&](int gt, QfTile& d) -> bool {
+        for (; gt < total_tiles; gt += stride) {
+            int li = 0;
+#pragma unroll
+            for (int k = 1; k < ODMKV_NQ; ++k) li += (gt >= a.tile_base[k]);
+            const int tile = gt - a.tile_base[li];
+            const int32_t* seg_tile = a.s.seg_tile[li];
+            const int bh = find_segment(seg_tile, a.nseg, tile);
+            const int ts = (tile - seg_tile[bh]) * TILE;
+            const int lo = max(a.old_count[li * a.nseg + bh] - ts, 0);
+            const int hi = min(a.s.seg_count[li][bh] - ts, TILE);
+            if (lo >= hi) continue;                             // nothing new in this tile (wave-uniform)
+            if (li == 3) { hand_over(gt); continue; }
+            d.gt = gt; d.li = li; d.tile = tile; d.bh = bh; d.lo = lo; d.hi = hi;
+            return true;
+        }
+        return false;
+    };
+    const auto row_offset = [&](const QfTile& d, int pos) {
+        return (size_t)(d.bh / a.Hkv) * a.sB + (size_t)(d.bh % a.Hkv) * a.sH + (size_t)(pos - a.pos_offset) * a.sT;
+    };
+
+    QfTile cur;
+    if (!next_tile((blockIdx.x >> 1) * QF_NW + wave, cur)) return;
+    int n_listed = 0;                                           // == w.count between tiles
+    if (lane == 0) w.count = 0;
+    bool valid = lane >= cur.lo && lane < cur.hi;
+    size_t off = 0;
+    RowRegs<ODMKV_F16> x;
+    if (valid) {
+        off = row_offset(cur, a.s.pos[cur.li][(size_t)cur.tile * TILE + lane]);
+        x.load(base, off);
+    } else {
+        x.zero();
+    }
+    while (true) {
+        QfTile nxt;
+        const bool more = next_tile(cur.gt + stride, nxt);
+        const bool valid_n = more && lane >= nxt.lo && lane < nxt.hi;
+        int pos_n = 0;
+        if (valid_n) pos_n = a.s.pos[nxt.li][(size_t)nxt.tile * TILE + lane];
+
+        // a token per lane: the norm in the definition's order, and what the matrix layout needs per token
+        float ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < HD; ++j) {
+            const float xj = x.get(j);
+            ss = __fmaf_rn(xj, xj, ss);
+        }
+        const float norm = sqrtf(ss);
+        const bool ok = !__any(!(ss <= 3.4028234663852886e38f));    // a row with an infinite or NaN norm: exact kernel
+        const float* thr = thrs + thr_offset(cur.li);
+        const bool direct = cur.li != 1 && cur.lo == 0 && (!IS_V || cur.hi == TILE);
+        const int variant = cur.li == 0 ? (direct ? 0 : 1) : cur.li == 1 ? 2 : (direct ? 3 : 4);
+        const int n_before = n_listed;
+        int n = 0;
+        if (ok) {
+            const float den = norm + 1e-10f;
+            w.off[lane] = valid ? (unsigned long long)off : ~0ull;
+            w.den[lane] = den;
+            w.rinv[lane] = 1.0f / den;
+            w.band[lane] = (valid && ss > 0.0f) ? QF_BAND : -1.0f;  // rows of zeros: the estimate is the exact 0
+            wave_lds_fence();
+            switch (variant) {
+                case 0: qf_code_tile<2, IS_V, true>(base, piA, thr, w, stage, lane, cur.gt); break;
+                case 1: qf_code_tile<2, IS_V, false>(base, piA, thr, w, stage, lane, cur.gt); break;
+                case 2: qf_code_tile<3, IS_V, false>(base, piA, thr, w, stage, lane, cur.gt); break;
+                case 3: qf_code_tile<4, IS_V, true>(base, piA, thr, w, stage, lane, cur.gt); break;
+                default: qf_code_tile<4, IS_V, false>(base, piA, thr, w, stage, lane, cur.gt); break;
+            }
+            wave_lds_fence();
+            n = w.count;
+        }
+        // the next tile's rows: asked for now, used in the next round
+        RowRegs<ODMKV_F16> xn;
+        size_t off_n = 0;
+        if (valid_n) {
+            off_n = row_offset(nxt, pos_n);
+            xn.load(base, off_n);
+        } else {
+            xn.zero();
+        }
+        if (ok && n <= QF_LIST) {
+            switch (variant) {
+                case 0: qf_store_tile<2, IS_V, true>(a, stage, lane, cur.li, cur.tile, cur.lo); break;
+                case 1: qf_store_tile<2, IS_V, false>(a, stage, lane, cur.li, cur.tile, cur.lo); break;
+                case 2: qf_store_tile<3, IS_V, false>(a, stage, lane, cur.li, cur.tile, cur.lo); break;
+                case 3: qf_store_tile<4, IS_V, true>(a, stage, lane, cur.li, cur.tile, cur.lo); break;
+                default: qf_store_tile<4, IS_V, false>(a, stage, lane, cur.li, cur.tile, cur.lo); break;
+            }
+            if (valid) (IS_V ? a.s.vnorm[cur.li] : a.s.knorm[cur.li])[(size_t)cur.tile * TILE + lane] = norm;
+            n_listed = n;
+        } else {
+            // a row the estimate does not cover, or more listed values than there was room for: the exact
+            // kernel does the whole tile (what the list got of it is dropped)
+            hand_over(cur.gt);
+            n_listed = n_before;
+            if (ok && lane == 0) w.count = n_before;
+        }
+        wave_lds_fence();                                       // staging area and scratch free for the next tile
+        if (n_listed >= WAVE || (!more && n_listed > 0)) {
+            __builtin_amdgcn_s_waitcnt(0);                      // this wave's codes, positions and norms are in memory
+            while (n_listed >= WAVE) {
+                n_listed -= WAVE;
+                qf_fix_listed<IS_V>(a, thrs, w, lane, n_listed, WAVE);
+            }
+            if (!more && n_listed > 0) { qf_fix_listed<IS_V>(a, thrs, w, lane, 0, n_listed); n_listed = 0; }
+            if (lane == 0) w.count = n_listed;
+            wave_lds_fence();
+        }
+        if (!more) break;
+        cur = nxt; valid = valid_n; off = off_n; x = xn;
+    }
+}
+
+__global__ __launch_bounds__(QF_NW * 64) void quant_pack_f16_kernel(QuantArgs a) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    _Float16* pih = reinterpret_cast<_Float16*>(smem);
+    float* thrs = reinterpret_cast<float*>(smem + QF_PI_BYTES + QF_NW * QP_STAGE);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint8_t* stage = smem + QF_PI_BYTES + wave * QP_STAGE;
+    QfWave& w = reinterpret_cast<QfWave*>(smem + QF_PI_BYTES + QF_NW * QP_STAGE + QF_THR_BYTES)[wave];
+    const bool is_v = (blockIdx.x & 1) != 0;
+    {
+        // Pi -> hi + lo in fp16, in the order the matrix instruction reads a 16-output x 32-step block:
+        // lane 16q + r of block (ob, ch) holds Pi[16 ob + r][32 ch + 8 q .. + 7]
+        // (all of a thread's reads are asked for at once: eight round trips to memory would cost more
+        // than the tiles of a short call)
+        const float4* __restrict__ pi4 = reinterpret_cast<const float4*>(is_v ? a.pi_v : a.pi_k);
+        constexpr int PER_THREAD = HD * HD / 4 / (QF_NW * 64);
+        float4 p[PER_THREAD];
+#pragma unroll
+        for (int k = 0; k < PER_THREAD; ++k) p[k] = pi4[tid + k * (QF_NW * 64)];
+#pragma unroll
+        for (int k = 0; k < PER_THREAD; ++k) {
+            const int c = tid + k * (QF_NW * 64);               // four consecutive j of row i
+            const int i = c >> 5, j = (c & 31) * 4;
+            const int ob = i >> 4, r = i & 15, ch = j >> 5, q = (j >> 3) & 3, e = j & 7;
+            const int dst = (((ob * 4 + ch) * 64) + 16 * q + r) * 8 + e;
+            const float pv[4] = {p[k].x, p[k].y, p[k].z, p[k].w};
+            typedef _Float16 qf_h4 __attribute__((ext_vector_type(4)));
+            qf_h4 h, l;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                h[t] = (_Float16)pv[t];
+                l[t] = (_Float16)(pv[t] - (float)h[t]);
+            }
+            *reinterpret_cast<qf_h4*>(pih + dst) = h;
+            *reinterpret_cast<qf_h4*>(pih + HD * HD + dst) = l;
+        }
+        for (int i = tid; i < QP_THR_FLOATS; i += QF_NW * 64) {
+            const int li = i < 3 ? 0 : i < 10 ? 1 : i < 25 ? 2 : 3;
+            const int k = i - thr_offset(li);
+            thrs[i] = decision_threshold(a.cb[codebook_offset(li) + k], a.cb[codebook_offset(li) + k + 1]);
+        }
+    }
+    __syncthreads();
+    const uint4* piA = reinterpret_cast<const uint4*>(smem);
+    if (is_v) qf_walk<true>(a, piA, thrs, w, stage, lane, wave);
+    else qf_walk<false>(a, piA, thrs, w, stage, lane, wave);
+}
+
+// ------------------------------------------------------------------------------------------------
 // exact rows: gather into the tiled fp16/bf16 layout
 // ------------------------------------------------------------------------------------------------
 struct ExactArgs {
@@ -827,11 +1316,39 @@ static int check_store(const odmkv_packed_t* s, const char* who) {
 }
 
 static inline int compact_chunks(int T) { return (T + CP_TOKENS - 1) / CP_TOKENS; }
+// tiles one call can touch, per tensor: a level that receives n tokens of a segment touches at most
+// n / 64 + 2 tiles, and the four quantised levels share the segment's T tokens
+static inline int redo_capacity(int nseg, int T) { return nseg * (T / TILE + 2 * ODMKV_NQ); }
+
+// byte offset, inside the pack workspace, of the hand-over list (two counters, then the tile numbers)
+size_t pack_redo_offset(int nseg, int T) {
+    return align_up((size_t)5 * nseg * sizeof(int32_t), 256) +
+           align_up((size_t)5 * nseg * compact_chunks(T) * sizeof(int32_t), 256);
+}
 
 extern "C" size_t odmkv_pack_workspace_bytes(int B, int Hkv, int T) {
     if (B <= 0 || Hkv <= 0 || T <= 0) return 0;
-    return align_up((size_t)5 * B * Hkv * sizeof(int32_t), 256) +
-           align_up((size_t)5 * B * Hkv * compact_chunks(T) * sizeof(int32_t), 256);
+    return pack_redo_offset(B * Hkv, T) + align_up((size_t)(2 + 2 * redo_capacity(B * Hkv, T)) * sizeof(int32_t), 256);
+}
+
+static int launch_quant_f16(const QuantArgs& qa, hipStream_t st) {
+    const size_t lds = QF_PI_BYTES + (size_t)QF_NW * QP_STAGE + QF_THR_BYTES + QF_NW * sizeof(QfWave);
+    static bool attr_set = false;
+    if (!attr_set) {
+        ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&quant_pack_f16_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        attr_set = true;
+    }
+    const int total = qa.tile_base[ODMKV_NQ];
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+    }
+    const int per_tensor = std::max(1, std::min((total + QF_NW - 1) / QF_NW, std::max(cus / 2, 1)));
+    hipLaunchKernelGGL(quant_pack_f16_kernel, dim3(2 * per_tensor), dim3(QF_NW * 64), lds, st, qa);
+    ODMKV_CHECK_LAUNCH("quant_pack_f16_kernel");
+    return 0;
 }
 
 template <int DT>
@@ -892,6 +1409,9 @@ extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, 
     ca.bits = bits; ca.T = T; ca.pos_offset = pos_offset; ca.nseg = nseg; ca.old_count = old_count;
     ca.n_chunks = compact_chunks(T);
     ca.chunk_count = (int32_t*)((char*)workspace + align_up((size_t)5 * nseg * sizeof(int32_t), 256));
+    // fp16 rows take the matrix-core estimate first; what it leaves over reaches the exact kernel through this list
+    int32_t* redo = (int32_t*)((char*)workspace + pack_redo_offset(nseg, T));
+    ca.redo = redo;
     for (int li = 0; li < 5; ++li) { ca.pos[li] = store->pos[li]; ca.seg_tile[li] = store->seg_tile[li]; ca.seg_count[li] = store->seg_count[li]; }
     ODMKV_CHECK_ARG(nseg <= 65535, "quant_pack: at most 65535 (sequence, head) pairs per call");
     hipLaunchKernelGGL(chunk_count_kernel, dim3(ca.n_chunks, nseg), dim3(CP_THREADS), 0, st, ca);
@@ -907,10 +1427,16 @@ extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, 
         qa.s = *store;
         qa.tile_base[0] = 0;
         for (int li = 0; li < ODMKV_NQ; ++li) qa.tile_base[li + 1] = qa.tile_base[li] + store->n_tiles[li];
+        qa.redo = redo; qa.redo_cap = redo_capacity(nseg, T); qa.from_list = 0;
         if (qa.tile_base[ODMKV_NQ] > 0) {
-            int rc = dtype == ODMKV_F16 ? launch_quant<ODMKV_F16>(qa, st)
-                   : dtype == ODMKV_BF16 ? launch_quant<ODMKV_BF16>(qa, st)
-                                         : launch_quant<ODMKV_F32>(qa, st);
+            int rc;
+            if (dtype == ODMKV_F16 && qa.tile_base[ODMKV_NQ] < (1 << QF_GT_BITS)) {
+                rc = launch_quant_f16(qa, st);
+                qa.from_list = 1;
+                if (!rc) rc = launch_quant<ODMKV_F16>(qa, st);
+            } else {
+                rc = dtype == ODMKV_BF16 ? launch_quant<ODMKV_BF16>(qa, st) : launch_quant<ODMKV_F32>(qa, st);
+            }
             if (rc) return rc;
         }
     }

@@ -213,11 +213,21 @@ class TurboQuantAdaptiveKVCacheState:
                 spare = torch.empty(off + off // 8, dtype=torch.uint8, device=dev)
             arena, self._arena_spare = spare, arena
         self._arena = arena
-        table = np.zeros(tables_end // 4, np.int32)
+        # the tables go up through page-locked memory, without waiting; the buffer is rewritten only once
+        # the copy before has been done
+        host = getattr(self, "_table_host", None)
+        if host is None or host.numel() < tables_end // 4:
+            host = self._table_host = torch.zeros(tables_end // 4 + 64, dtype=torch.int32, pin_memory=True)
+            self._table_sent = torch.cuda.Event()
+        else:
+            self._table_sent.synchronize()
+        table = host.numpy()
+        table[:tables_end // 4] = 0
         for li in range(5):
             o = plan[("seg_tile", li)][0] // 4
             table[o:o + nseg + 1] = seg_tile[li]
-        arena[:tables_end].view(torch.int32).copy_(torch.from_numpy(table))
+        arena[:tables_end].view(torch.int32).copy_(host[:tables_end // 4], non_blocking=True)
+        self._table_sent.record(torch.cuda.current_stream(dev))
         arena[tables_end:zero_end].zero_()
         arena[zero_end:pos_end].view(torch.int32).fill_(-1)
         return _Buffers(arena, plan)
@@ -340,7 +350,12 @@ class TurboQuantAdaptiveKVCacheState:
         else:
             counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
             _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
-            counts = counts_dev.cpu().numpy().astype(np.int64)        # the one synchronisation
+            host = getattr(self, "_counts_host", None)
+            if host is None or host.shape[0] != self._nseg:
+                host = self._counts_host = torch.empty(self._nseg, 6, dtype=torch.int32, pin_memory=True)
+            host.copy_(counts_dev, non_blocking=True)
+            torch.cuda.current_stream(dev).synchronize()              # the one synchronisation
+            counts = host.numpy().astype(np.int64)
         if int(counts.sum()) != self._nseg * T:
             raise ValueError("bits must take values in (0, 2, 3, 4, 8, 16)")
         present = {lvl for lvl, c in zip(_lib.LEVEL_ORDER, counts.sum(axis=0)) if c > 0}

@@ -235,3 +235,122 @@ def test_edge_cases_and_errors():
         TurboQuantAdaptiveKVCacheState(128, (0, 2, 4), device=DEV)      # defaults are prod / minmax
     with pytest.raises(ValueError):
         TurboQuantAdaptiveKVCacheState(64, (0, 2, 4), device=DEV, key_quantizer="mse", value_quantizer="mse")
+
+
+# ---- fp16 tensors: the matrix-core estimate with exact codes next to the decision thresholds ----------
+# fp16 rows are quantised by a kernel that estimates the rotation on the fp16 matrix cores and recomputes,
+# by the definition's own chain, only the values within a guard band of a threshold; fp32 rows (and what
+# that kernel hands over) go through the exact kernel alone.  The same numbers given in either type must
+# therefore come out as the same bytes.
+def _handed_over(state, B, H, T):
+    import ctypes as C
+    import os
+    from kvquant import _lib
+    blib = C.CDLL(os.path.join(os.path.dirname(_lib.__file__), "..", "lib", "libodmkv_bench.so"))
+    ws = _lib.workspace(state.device, _lib.lib.odmkv_pack_workspace_bytes(B, H, T), "pack")     # the buffer the state's call used
+    out = (C.c_int32 * 2)()
+    blib.odmkv_bench_pack_handed_over.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int32), C.c_void_p]
+    rc = blib.odmkv_bench_pack_handed_over(ws.data_ptr(), B, H, T, out, _lib.stream_ptr(state.device))
+    assert rc == 0
+    return int(out[0]), int(out[1])
+
+
+def _same_bytes_in_both_types(k16, v16, bits):
+    """Prefill the fp16 tensors and their fp32 copies; compare every quantised level's buffers bit for bit.
+    Returns the tiles the fp16 call handed to the exact kernel (keys, values)."""
+    B, H, T, _ = k16.shape
+    s16, s32 = _state(), _state()
+    s16.prefill(k16, v16, bits)
+    handed = _handed_over(s16, B, H, T)
+    s32.prefill(k16.float(), v16.float(), bits)
+    assert np.array_equal(s16._seg_tile, s32._seg_tile) and np.array_equal(s16._counts, s32._counts)
+    for li in range(4):
+        nt = int(s16._seg_tile[li, -1])
+        if nt == 0:
+            continue
+        for name, per_tile in (("kcodes", 64 * 16 * (2, 3, 4, 8)[li]), ("vcodes", 64 * 16 * (2, 3, 4, 8)[li]),
+                               ("knorm", 64), ("vnorm", 64), ("pos", 64)):
+            a, b = s16._bufs[name][li].view(-1), s32._bufs[name][li].view(-1)
+            n = nt * per_tile
+            if a.dtype == torch.float32:
+                a, b = a.view(torch.int32), b.view(torch.int32)
+            bad = (a[:n] != b[:n]).nonzero()
+            assert bad.numel() == 0, f"level index {li}, {name}: {bad.numel()} of {n} differ, first at {int(bad[0])}"
+    return handed
+
+
+def _rows_on_thresholds(state, pi, n_rows, per_row, width, g):
+    """fp16 rows whose rotated unit vectors have `per_row` entries on decision thresholds of `width` bits
+    (up to fp16 rounding of the row: a few 1e-5, well inside the guard band)."""
+    cb = state.codebooks.cpu()
+    off = {2: 0, 3: 4, 4: 12}[width]
+    c = cb[off:off + (1 << width)].double()
+    thr = (c[:-1] + c[1:]) / 2
+    if per_row > 20:
+        thr = thr[thr.abs() < 0.09]                                        # many entries: inner thresholds, so that the row stays a unit vector
+    y = torch.randn(n_rows, 128, generator=g, dtype=torch.float64) / 128 ** 0.5
+    for r in range(n_rows):
+        idx = torch.randperm(128, generator=g)[:per_row]
+        y[r, idx] = thr[torch.randint(len(thr), (per_row,), generator=g)]
+        rest = torch.ones(128, dtype=torch.bool); rest[idx] = False
+        left = 1.0 - float((y[r, idx] ** 2).sum())
+        assert left > 0
+        y[r, rest] *= (left / float((y[r, rest] ** 2).sum())) ** 0.5       # unit norm keeps the chosen entries where they are
+    x = y @ pi.cpu().double()                                              # y = Pi x
+    scale = torch.rand(n_rows, 1, generator=g, dtype=torch.float64) * 20 + 0.05
+    return (x * scale).half()
+
+
+@pytest.mark.parametrize("per_row", [2, 100])
+def test_fp16_rows_next_to_thresholds_get_the_exact_codes(per_row):
+    g = torch.Generator().manual_seed(per_row)
+    B, H, T = 1, 2, 1024
+    probe = _state()
+    bits = torch.tensor([2, 3, 4], dtype=torch.int32)[torch.randint(3, (B, H, T), generator=g)]
+    k = torch.empty(B, H, T, 128, dtype=torch.float16)
+    v = torch.empty(B, H, T, 128, dtype=torch.float16)
+    for w in (2, 3, 4):
+        m = bits == w
+        n = int(m.sum())
+        k[m] = _rows_on_thresholds(probe, probe.pi_k, n, per_row, w, g)
+        v[m] = _rows_on_thresholds(probe, probe.pi_v, n, per_row, w, g)
+    hk, hv = _same_bytes_in_both_types(k.to(DEV), v.to(DEV), bits.to(DEV))
+    if per_row == 2:
+        assert (hk, hv) == (0, 0)          # a couple of hundred listed values per tile: worked off in the kernel
+    else:
+        assert hk > 0 and hv > 0           # thousands per tile: the tiles go to the exact kernel
+    # and the oracle agrees on a sample of the rows
+    ref = KVState(128, (0, 2, 3, 4, 8, 16), seed=42, order="canonical")
+    ref.prefill(k[:, :, :192], v[:, :, :192], bits[:, :, :192])
+    st = _state()
+    st.prefill(k[:, :, :192].to(DEV), v[:, :, :192].to(DEV), bits[:, :, :192].to(DEV))
+    _check_store_against_oracle(st, ref)
+
+
+def test_fp16_special_rows_and_ordinary_ones():
+    g = torch.Generator().manual_seed(11)
+    B, H, T = 2, 2, 1500
+    k = torch.randn(B, H, T, 128, generator=g).half()
+    v = (torch.randn(B, H, T, 128, generator=g) * 3).half()
+    bits = _rand_bits(g, (B, H, T), levels=(0, 2, 3, 4, 16), probs=(0.1, 0.45, 0.25, 0.15, 0.05))
+    hk, hv = _same_bytes_in_both_types(k.to(DEV), v.to(DEV), bits.to(DEV))
+    assert (hk, hv) == (0, 0)              # no 8-bit tiles, ordinary rows: nothing for the exact kernel
+    # rows of zeros, the largest and the smallest fp16 numbers, a huge outlier, infinities and NaNs
+    k2, v2 = k.clone(), v.clone()
+    k2[0, 0, 5] = 0; v2[0, 0, 5] = 0
+    k2[0, 1, 70:80] = 65504.0; v2[0, 1, 70:80] = -65504.0
+    k2[1, 0, 200:210] = 6e-8; v2[1, 0, 200:210] *= 1e-4
+    k2[1, 1, 300, 7] = 30000.0; v2[1, 1, 300, 90] = -30000.0
+    k2[0, 0, 900, 3] = float("inf"); v2[0, 0, 901, 4] = float("nan")
+    k2[1, 1, 1400, 0] = float("-inf"); v2[1, 1, 1400, 127] = float("inf")
+    hk, hv = _same_bytes_in_both_types(k2.to(DEV), v2.to(DEV), bits.to(DEV))
+    lvl = bits.numpy()
+    expect_k = int(lvl[0, 0, 900] in (2, 3, 4)) + int(lvl[1, 1, 1400] in (2, 3, 4))
+    expect_v = int(lvl[0, 0, 901] in (2, 3, 4)) + int(lvl[1, 1, 1400] in (2, 3, 4))
+    assert hk <= expect_k and hv <= expect_v       # (two such rows can share a tile)
+    assert (hk > 0) == (expect_k > 0) and (hv > 0) == (expect_v > 0)
+    # 8-bit tiles always go to the exact kernel
+    bits8 = _rand_bits(g, (B, H, T))
+    hk, hv = _same_bytes_in_both_types(k.to(DEV), v.to(DEV), bits8.to(DEV))
+    n8 = sum(-(-int((bits8[b, h] == 8).sum()) // 64) for b in range(B) for h in range(H))
+    assert (hk, hv) == (n8, n8)
