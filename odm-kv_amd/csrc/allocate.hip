@@ -11,13 +11,13 @@
 // The costs use lambda rounded to fp32, so once the bracket's ends are neighbouring fp32 numbers
 // (after about 32 halvings on typical scores) the rest of the search is decided by rounding alone:
 // it is walked on the spot and the remaining halving launches return immediately.
-// Every workgroup writes its partial bit sums; the workgroup that finishes last (found by an
-// atomic ticket) adds them up, walks the bracket and prepares the next launch's candidates.
-// Nothing ever waits on another workgroup and the host is never consulted.  All sums are
-// integers, so the result does not depend on the order in which workgroups run.
-// The partial sums travel as device-scope atomic stores and loads (they go to the memory side of
-// the per-XCD L2s), ordered before the ticket by waiting for the stores to complete; a device-scope
-// fence instead would write back the whole L2 from every workgroup.
+// Every workgroup writes its partial bit sums with plain stores and is done.  The next launch begins,
+// in every workgroup, by adding up the row's partial sums of the launch before (a few hundred
+// numbers) and walking the bracket with them; the row's first workgroup also writes the new state
+// down for the launch after.  Nothing waits on another workgroup, no atomics cross workgroups, and
+// the host is never consulted.  All sums are integers, so the result does not depend on the order
+// in which workgroups run.  Partial sums and states are double-buffered by launch parity: a workgroup
+// that finishes early must not overwrite what a late one of the same launch still reads.
 //
 // Arithmetic is kept exactly as the host formulation it replaces: fp32 products rounded
 // separately and then added (no fused multiply-add), lambda rounded to fp32 before use, the
@@ -34,7 +34,7 @@
 #define SLOTS 16                              // partial sums per workgroup
 #define EV_THREADS 512
 #ifndef EV_TPT
-#define EV_TPT 4                              // tokens per thread in an evaluation
+#define EV_TPT 2                              // tokens per thread in an evaluation
 #endif
 #define EV_TOKENS (EV_THREADS * EV_TPT)
 #define CAND_MAX 16                           // repair moves of at most this many tokens take the short path
@@ -58,10 +58,10 @@ struct AllocArgs {
     int nominal[NLV];
     const double* target;          // device, [rows]
     uint8_t* chosen;               // [rows, n]
-    unsigned int* partial;         // [rows, n_chunks, SLOTS]
-    unsigned int* tickets;         // [rows, N_LAUNCH]
+    unsigned int* partial;         // [2][rows, n_chunks, SLOTS]: launch L writes half L & 1
     unsigned long long* cand;      // [rows, n_chunks, CAND_MAX]
-    RowState* state;               // [rows]
+    RowState* state;               // [3][rows]: launch L >= 1 leaves the state it starts from in third L & 1 (launch 0 starts
+                                   // from third 0, which the set-up kernels fill); third 2 is the final one
     int32_t* bits_out;
     int32_t* level_counts;
     double* lambda_out;
@@ -97,7 +97,6 @@ __device__ static inline int wave_sum_int(int v) {
 // ---- clear counters, set up the bracket ----
 __global__ void alloc_init_kernel(AllocArgs a) {
     const int row = blockIdx.x;
-    for (int e = threadIdx.x; e < N_LAUNCH; e += blockDim.x) a.tickets[(size_t)row * N_LAUNCH + e] = 0u;
     if (a.level_counts && threadIdx.x < a.K) a.level_counts[row * a.K + threadIdx.x] = 0;
     if (threadIdx.x == 0) {
         RowState& st = a.state[row];
@@ -112,7 +111,7 @@ __global__ void alloc_init_kernel(AllocArgs a) {
 }
 
 // ---- what the sanitiser needs to know about a row ----
-#define SC_THREADS 1024
+#define SC_THREADS 512
 #define SC_TPT 8
 #define SC_TOKENS (SC_THREADS * SC_TPT)
 __global__ __launch_bounds__(SC_THREADS) void alloc_scan_kernel(AllocArgs a) {
@@ -124,11 +123,19 @@ __global__ __launch_bounds__(SC_THREADS) void alloc_scan_kernel(AllocArgs a) {
     unsigned int mx = 0u;
     int fin = 0, non = 0, act = 0;
     const int base = blockIdx.x * SC_TOKENS;
-    for (int e = 0; e < SC_TPT; ++e) {
+    float raw[SC_TPT];
+    bool on[SC_TPT];
+#pragma unroll
+    for (int e = 0; e < SC_TPT; ++e) {                       // all reads first: one round trip, not SC_TPT
         const int i = base + e * SC_THREADS + threadIdx.x;
-        if (i < a.n && !is_sink(a, row, i)) {
+        on[e] = i < a.n && !is_sink(a, row, i);
+        raw[e] = on[e] ? a.scores[(size_t)row * a.n + i] : 0.0f;
+    }
+#pragma unroll
+    for (int e = 0; e < SC_TPT; ++e) {
+        if (on[e]) {
             ++act;
-            float v = a.scores[(size_t)row * a.n + i];
+            float v = raw[e];
             if (!(v != v)) v = fmaxf(v, 0.0f);
             if (isfinite(v)) { fin = 1; mx = max(mx, __float_as_uint(v)); }
             else non = 1;
@@ -159,9 +166,8 @@ __device__ static inline float tree_candidate(double lo, double hi, int node) {
     return (float)((lo + hi) * 0.5);
 }
 
-// the last workgroup of launch L: sums[] holds the row's totals; advance the search
-__device__ static void advance(const AllocArgs& a, int row, int L, const unsigned int* sums) {
-    RowState& st = a.state[row];
+// sums[] holds the row's totals of launch L, st the state that launch started from: advance the search
+__device__ static void advance(const AllocArgs& a, RowState& st, int L, const unsigned int* sums) {
     const float nf = (float)st.n_active;
     if (L == 0) {
         double hi = 1.0;
@@ -204,7 +210,6 @@ __device__ static void advance(const AllocArgs& a, int row, int L, const unsigne
         }
         const double avg = (double)((float)S / nf);
         st.gap = (avg - st.target) * (double)st.n_active;
-        if (a.lambda_out) a.lambda_out[row] = st.lam;
         return;
     }
     if (L + 1 == L_FINAL) st.lam = (st.lo + st.hi) * 0.5;
@@ -219,6 +224,41 @@ __device__ static inline float candidate(const RowState& st, int L, int c) {
     }
     if (L == L_FINAL) return (float)((st.lo + st.hi) * 0.5);
     return c >= 1 ? tree_candidate(st.lo, st.hi, c) : 0.0f;
+}
+
+// did launch L pass over the scores, given the state it started from?
+__device__ static inline bool launch_evaluates(const RowState& st, int L) {
+    return st.n_active != 0 && !(L > 0 && L < L_FINAL && st.collapsed);
+}
+
+// Start of launch L >= 1 (the candidate kernel calls it as launch L_FINAL + 1): the state launch L - 1
+// started from plus that launch's partial sums give the state this launch starts from, left in `cur`
+// (shared memory) for the whole workgroup; the row's first workgroup writes it to `out` as well.
+// Ends with a barrier.
+__device__ static void carry_state(const AllocArgs& a, int row, int L, RowState* out, RowState* cur, unsigned int* tot) {
+    const int tid = threadIdx.x;
+    const RowState* in = a.state + (size_t)((L - 1) & 1) * a.rows + row;
+    if (tid < SLOTS) tot[tid] = 0u;
+    __syncthreads();
+    const bool evaluated = launch_evaluates(*in, L - 1);
+    if (evaluated) {
+        const unsigned int* p = a.partial + ((size_t)((L - 1) & 1) * a.rows + row) * a.n_chunks * SLOTS;
+        for (int idx = tid; idx < a.n_chunks * SLOTS; idx += blockDim.x) {
+            const unsigned int v = p[idx];
+            if (v) atomicAdd(&tot[idx & (SLOTS - 1)], v);
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        RowState st = *in;
+        if (evaluated) advance(a, st, L - 1, tot);
+        *cur = st;
+        if (blockIdx.x == 0) {
+            *out = st;
+            if (L - 1 == L_FINAL && evaluated && a.lambda_out) a.lambda_out[row] = st.lam;
+        }
+    }
+    __syncthreads();
 }
 
 // sums of 16-bit fields over the wave: on return, lanes with (lane & 7) == 0 hold packed pair
@@ -244,11 +284,26 @@ __global__ __launch_bounds__(EV_THREADS) void alloc_eval_kernel(AllocArgs a, int
     __shared__ __align__(16) float lamb[SLOTS][NLV];     // fl32(lambda_c * b_k)
     __shared__ int lsum[SLOTS];
     __shared__ unsigned int tot[SLOTS];
-    __shared__ int is_last;
+    __shared__ RowState cur;
     const int row = blockIdx.y, tid = threadIdx.x;
-    const RowState& st = a.state[row];
-    if (st.n_active == 0) return;
-    if (L > 0 && L < L_FINAL && st.collapsed) return;       // this launch's halvings are already decided
+    // the scores are asked for first: they do not depend on the state, which takes a round trip of its own
+    const int base = blockIdx.x * EV_TOKENS;
+    float raw[EV_TPT];
+    bool active[EV_TPT];
+#pragma unroll
+    for (int e = 0; e < EV_TPT; ++e) {
+        const int i = base + e * EV_THREADS + tid;
+        active[e] = i < a.n && !is_sink(a, row, i);
+        raw[e] = active[e] ? a.scores[(size_t)row * a.n + i] : 0.0f;
+    }
+    if (L == 0) {
+        if (tid == 0) cur = a.state[row];
+        __syncthreads();
+    } else {
+        carry_state(a, row, L, a.state + (size_t)(L & 1) * a.rows + row, &cur, tot);
+    }
+    const RowState& st = cur;
+    if (!launch_evaluates(st, L)) return;                   // an empty row, or this launch's halvings are already decided
     if (tid < SLOTS * NLV) {
         const int c = tid / NLV, k = tid % NLV;
         lamb[c][k] = __fmul_rn(candidate(st, L, c), a.bitsf[k]);
@@ -258,13 +313,9 @@ __global__ __launch_bounds__(EV_THREADS) void alloc_eval_kernel(AllocArgs a, int
 
     const Cleaner clean(st);
     float se[EV_TPT][K];
-    bool active[EV_TPT];
-    const int base = blockIdx.x * EV_TOKENS;
 #pragma unroll
     for (int e = 0; e < EV_TPT; ++e) {
-        const int i = base + e * EV_THREADS + tid;
-        active[e] = i < a.n && !is_sink(a, row, i);
-        const float s = active[e] ? clean(a.scores[(size_t)row * a.n + i]) : 0.0f;
+        const float s = active[e] ? clean(raw[e]) : 0.0f;
 #pragma unroll
         for (int k = 0; k < K; ++k) se[e][k] = __fmul_rn(s, a.eps[k]);
     }
@@ -324,32 +375,8 @@ __global__ __launch_bounds__(EV_THREADS) void alloc_eval_kernel(AllocArgs a, int
         }
     }
     __syncthreads();
-    unsigned int* mine = a.partial + ((size_t)row * a.n_chunks + blockIdx.x) * SLOTS;
-    if (tid < SLOTS) {
-        __hip_atomic_store(mine + tid, (unsigned int)lsum[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_s_waitcnt(0);            // the stores have reached the memory side
-    }
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned int t = __hip_atomic_fetch_add(&a.tickets[(size_t)row * N_LAUNCH + L], 1u, __ATOMIC_RELAXED,
-                                                      __HIP_MEMORY_SCOPE_AGENT);
-        is_last = (t == gridDim.x - 1);
-    }
-    __syncthreads();
-    if (!is_last) return;
-    if (tid < SLOTS) tot[tid] = 0u;
-    __syncthreads();
-    {
-        // 16 threads per slot walk the chunks
-        const int slot = tid & (SLOTS - 1), part = tid / SLOTS;
-        unsigned int s = 0u;
-        const unsigned int* p = a.partial + (size_t)row * a.n_chunks * SLOTS;
-        for (int w = part; w < a.n_chunks; w += EV_THREADS / SLOTS)
-            s += __hip_atomic_load(p + (size_t)w * SLOTS + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (s) atomicAdd(&tot[slot], s);
-    }
-    __syncthreads();
-    if (tid == 0) advance(a, row, L, tot);
+    unsigned int* mine = a.partial + (((size_t)(L & 1) * a.rows + row) * a.n_chunks + blockIdx.x) * SLOTS;
+    if (tid < SLOTS) mine[tid] = (unsigned int)lsum[tid];
 }
 
 // ---- budget repair -------------------------------------------------------------------------------
@@ -419,8 +446,11 @@ __device__ static inline void select_smallest(unsigned long long (&keys)[NK], in
 // per chunk: the candidates for the first move when it is small
 __global__ __launch_bounds__(EV_THREADS) void alloc_cand_kernel(AllocArgs a) {
     __shared__ unsigned long long wbest[EV_THREADS / 64];
+    __shared__ unsigned int tot[SLOTS];
+    __shared__ RowState cur;
     const int row = blockIdx.y, tid = threadIdx.x;
-    const RowState& st = a.state[row];
+    carry_state(a, row, L_FINAL + 1, a.state + (size_t)2 * a.rows + row, &cur, tot);     // the final state: gap, histogram, lambda
+    const RowState& st = cur;
     if (st.n_active == 0 || fabs(st.gap) <= 0.5) return;
     const bool over = st.gap > 0;
     Move m;
@@ -530,7 +560,7 @@ __global__ __launch_bounds__(RB) void alloc_repair_kernel(AllocArgs a) {
     __shared__ int scratch[32];
     __shared__ unsigned long long wbest[RB / 64];
     const int row = blockIdx.x, tid = threadIdx.x;
-    const RowState& st = a.state[row];
+    const RowState& st = a.state[(size_t)2 * a.rows + row];
     if (st.n_active == 0) return;
     double gap = st.gap;
     if (fabs(gap) <= 0.5) return;
@@ -593,17 +623,16 @@ __global__ __launch_bounds__(EV_THREADS) void alloc_write_kernel(AllocArgs a, in
         atomicAdd(&a.level_counts[row * a.K + threadIdx.x], lh[threadIdx.x]);
 }
 
-struct AllocLayout { size_t chosen, partial, tickets, cand, state, total; };
+struct AllocLayout { size_t chosen, partial, cand, state, total; };
 static AllocLayout alloc_layout(int rows, int n) {
     AllocLayout L;
     const size_t chunks = ((size_t)n + EV_TOKENS - 1) / EV_TOKENS;
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes, 256); return o; };
     L.chosen = take((size_t)rows * n);
-    L.partial = take((size_t)rows * chunks * SLOTS * sizeof(unsigned int));
-    L.tickets = take((size_t)rows * N_LAUNCH * sizeof(unsigned int));
+    L.partial = take((size_t)2 * rows * chunks * SLOTS * sizeof(unsigned int));
     L.cand = take((size_t)rows * chunks * CAND_MAX * sizeof(unsigned long long));
-    L.state = take((size_t)rows * sizeof(RowState));
+    L.state = take((size_t)3 * rows * sizeof(RowState));
     L.total = off;
     return L;
 }
@@ -646,7 +675,7 @@ extern "C" int odmkv_allocate(const float* scores, int rows, int n,
     }
     a.target = target;
     a.chosen = (uint8_t*)(ws + L.chosen);
-    a.partial = (unsigned int*)(ws + L.partial); a.tickets = (unsigned int*)(ws + L.tickets);
+    a.partial = (unsigned int*)(ws + L.partial);
     a.cand = (unsigned long long*)(ws + L.cand);
     a.state = (RowState*)(ws + L.state);
     a.bits_out = bits_out; a.level_counts = level_counts; a.lambda_out = lambda_out;

@@ -762,8 +762,8 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
 // terms (hi + lo, 22 bits), on v_mfma_f32_16x16x32_f16, then scaled by 1 / (|x| + 1e-10).  That
 // estimate differs from the chain's result by rounding alone: at most about 2.5e-5 on the scale
 // |y| <= 1 under the most pessimistic model of the matrix unit's adder (every one of the 128 terms
-// truncated at the scale of the largest partial sum), and about 1e-6 in practice.  Values farther
-// than QF_BAND from every threshold therefore have the chain's code already; the few within the band
+// truncated at the scale of the largest partial sum); measured, a band of 1e-7 already leaves no code
+// different over 1e8 values.  Values farther than QF_BAND (twice that bound) from every threshold therefore have the chain's code already; the few within the band
 // (two to eight in a thousand) are listed, and whenever a wave has 64 of them it recomputes them by
 // the chain itself, one lane per value, and replaces their codes in the packed tiles it has already
 // written.  Rows of zeros are exact either way.
@@ -779,7 +779,9 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
 typedef _Float16 qf_h8 __attribute__((ext_vector_type(8)));
 typedef float qf_f4 __attribute__((ext_vector_type(4)));
 
-#define QF_BAND 1.0e-4f
+#ifndef QF_BAND
+#define QF_BAND 5.0e-5f
+#endif
 #define QF_LIST 256                     // listed values a wave can hold (it works them off 64 at a time)
 #define QF_GT_BITS 19                   // tile numbers in a list entry
 #define QF_NW 8
