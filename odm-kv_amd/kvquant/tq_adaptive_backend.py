@@ -80,21 +80,6 @@ class _Buffers:
         return [self.view(name, li) for li in range(n)]
 
 
-_PAGE_LOCKED: dict = {}
-
-
-def _page_locked(name: str, numel: int):
-    """(int32 host tensor of at least `numel` elements in page-locked memory, event) shared by all states of the
-    process: allocating such memory costs as much as packing a layer, so it is done once.  The event is
-    recorded behind the last asynchronous copy out of the tensor; wait for it before writing the tensor again."""
-    got = _PAGE_LOCKED.get(name)
-    if got is None or got[0].numel() < numel:
-        if got is not None:
-            got[1].synchronize()
-        got = _PAGE_LOCKED[name] = (torch.zeros(max(2 * numel, 1024), dtype=torch.int32, pin_memory=True), torch.cuda.Event())
-    return got
-
-
 def _empty_positions(device) -> torch.Tensor:
     return torch.empty((0, 3), dtype=torch.long, device=device)
 
@@ -228,17 +213,11 @@ class TurboQuantAdaptiveKVCacheState:
                 spare = torch.empty(off + off // 8, dtype=torch.uint8, device=dev)
             arena, self._arena_spare = spare, arena
         self._arena = arena
-        # the tables go up through page-locked memory, without waiting; the buffer is rewritten only once
-        # the copy before has been done
-        host, sent = _page_locked("tables", tables_end // 4)
-        sent.synchronize()
-        table = host.numpy()
-        table[:tables_end // 4] = 0
+        table = np.zeros(tables_end // 4, np.int32)
         for li in range(5):
             o = plan[("seg_tile", li)][0] // 4
             table[o:o + nseg + 1] = seg_tile[li]
-        arena[:tables_end].view(torch.int32).copy_(host[:tables_end // 4], non_blocking=True)
-        sent.record(torch.cuda.current_stream(dev))
+        arena[:tables_end].view(torch.int32).copy_(torch.from_numpy(table))
         arena[tables_end:zero_end].zero_()
         arena[zero_end:pos_end].view(torch.int32).fill_(-1)
         return _Buffers(arena, plan)
@@ -361,10 +340,7 @@ class TurboQuantAdaptiveKVCacheState:
         else:
             counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
             _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
-            host = _page_locked("counts", self._nseg * 6)[0][:self._nseg * 6].view(self._nseg, 6)
-            host.copy_(counts_dev, non_blocking=True)
-            torch.cuda.current_stream(dev).synchronize()              # the one synchronisation
-            counts = host.numpy().astype(np.int64)
+            counts = counts_dev.cpu().numpy().astype(np.int64)        # the one synchronisation
         if int(counts.sum()) != self._nseg * T:
             raise ValueError("bits must take values in (0, 2, 3, 4, 8, 16)")
         present = {lvl for lvl, c in zip(_lib.LEVEL_ORDER, counts.sum(axis=0)) if c > 0}
