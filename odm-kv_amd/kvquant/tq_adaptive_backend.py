@@ -80,6 +80,9 @@ class _Buffers:
         return [self.view(name, li) for li in range(n)]
 
 
+_ARENA_HINT: dict = {}     # (device, segments, tokens) -> bytes of the last store first filled with that shape
+
+
 def _empty_positions(device) -> torch.Tensor:
     return torch.empty((0, 3), dtype=torch.long, device=device)
 
@@ -335,11 +338,19 @@ class TurboQuantAdaptiveKVCacheState:
             values = values.contiguous()
             keys = keys.contiguous()
         st = _lib.stream_ptr(dev)
+        fresh = self._bufs is None and getattr(self, "_arena", None) is None       # the store's first tokens
+        hint_key = (str(dev), self._nseg, T)
         if _known_counts is not None:
             counts = np.asarray(_known_counts, np.int64).reshape(self._nseg, 6)
         else:
             counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
             _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
+            if fresh and hint_key in _ARENA_HINT:
+                # while the counts are on their way: room for a store the size of the last one of this shape (a
+                # layer's store is about as large as its neighbour's).  A new device allocation costs as much as
+                # packing the layer; here it runs beside the kernels still in the queue.  Too small a guess is
+                # replaced in _alloc.
+                self._arena = torch.empty(_ARENA_HINT[hint_key], dtype=torch.uint8, device=dev)
             counts = counts_dev.cpu().numpy().astype(np.int64)        # the one synchronisation
         if int(counts.sum()) != self._nseg * T:
             raise ValueError("bits must take values in (0, 2, 3, 4, 8, 16)")
@@ -348,6 +359,8 @@ class TurboQuantAdaptiveKVCacheState:
             raise ValueError(f"bits use levels {sorted(present - set(self.bit_levels))} outside bit_levels={self.bit_levels}")
         new_counts = self._counts + counts[:, 1:].T
         self._ensure_capacity(new_counts)
+        if fresh:
+            _ARENA_HINT[hint_key] = self._arena.numel()
         pos_offset = self.seq_len if _pos_offset is None else int(_pos_offset)
         ws_bytes = lib.odmkv_pack_workspace_bytes(B, H, T)
         ws = _lib.workspace(dev, ws_bytes, "pack")
