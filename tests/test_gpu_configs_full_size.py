@@ -157,3 +157,30 @@ def test_c2_one_layer_score_matches_oracle_at_full_size():
     got = _launch_score(L.keys.to(DEV), L.values.to(DEV), L.mu.to(DEV), None, 32, 4, 1e-2).cpu()
     want = osc.risk_score_from_mu(L.keys.float(), L.values.float(), L.mu.unsqueeze(0), 32)
     np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=1e-3, atol=0)
+
+
+def test_c2_one_layer_fp16_store_equals_the_exact_quantisers_at_full_size():
+    """fp16 tensors are quantised through the matrix-core estimate plus exact codes next to the thresholds, fp32
+    tensors by the exact kernel alone: on a whole 32k-token layer (2.7e8 rotated values, levels
+    drawn at random over widths 2, 3 and 4) both must leave the same bytes."""
+    from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+    L = synthetic.config("c2", layer=9)
+    g = torch.Generator().manual_seed(9)
+    pick = torch.multinomial(torch.tensor([0.02, 0.45, 0.3, 0.2, 0.0, 0.03]), 8 * 32768, replacement=True, generator=g)
+    stored = torch.tensor(LEVELS, dtype=torch.int32)[pick].reshape(1, 8, 32768).to(DEV)
+    st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=DEV, dtype=torch.float16, key_quantizer="mse",
+                                        value_quantizer="mse", seed=42)
+    st.prefill(L.keys[None].to(DEV), L.values[None].to(DEV), stored)
+    counts = st.level_counts()
+    assert min(counts[2], counts[3], counts[4]) > 10000 and counts[8] == 0
+    ref = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=DEV, dtype=torch.float16, key_quantizer="mse",
+                                         value_quantizer="mse", seed=42)
+    ref.prefill(L.keys[None].to(DEV).float(), L.values[None].to(DEV).float(), stored)
+    assert np.array_equal(st._seg_tile, ref._seg_tile)
+    for li in range(4):
+        nt = int(st._seg_tile[li, -1])
+        for name, per_tile in (("kcodes", 1024 * (2, 3, 4, 8)[li]), ("vcodes", 1024 * (2, 3, 4, 8)[li]), ("knorm", 64), ("vnorm", 64)):
+            a, b = st._bufs[name][li].view(-1)[:nt * per_tile], ref._bufs[name][li].view(-1)[:nt * per_tile]
+            if a.dtype == torch.float32:
+                a, b = a.view(torch.int32), b.view(torch.int32)
+            assert torch.equal(a, b), f"level index {li}, {name}"
