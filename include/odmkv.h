@@ -182,7 +182,10 @@ int odmkv_level_counts(const int32_t* bits, int B, int Hkv, int T, int32_t* coun
  * The arithmetic per token is, in this order and in fp32:
  *   ss = fma(x_j, x_j, ss) j=0..127; norm = sqrt(ss); u_j = x_j / (norm + 1e-10);
  *   y_i = fma(u_j, Pi[i][j], y_i) j=0..127; code_i = nearer of the two centroids bracketing y_i
- *   (lower index on a tie). */
+ *   (lower index on a tie).
+ * fp16 tensors take a shorter route to the same bytes (widths 2, 3, 4): y_i is first estimated on the
+ * fp16 matrix cores, and only values next to a decision threshold are recomputed by the chain above.
+ * The workspace (odmkv_pack_workspace_bytes(B, Hkv, T) bytes, device) holds per-call scratch only. */
 size_t odmkv_pack_workspace_bytes(int B, int Hkv, int T);
 int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, int Hkv, int T,
                      int64_t stride_b, int64_t stride_h, int64_t stride_t,
