@@ -1437,7 +1437,9 @@ extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, 
                 qa.from_list = 1;
                 if (!rc) rc = launch_quant<ODMKV_F16>(qa, st);
             } else {
-                rc = dtype == ODMKV_BF16 ? launch_quant<ODMKV_BF16>(qa, st) : launch_quant<ODMKV_F32>(qa, st);
+                // (fp16 stores of 2^19 tiles and more: the list entries of the fp16 kernel have no room for their numbers)
+                rc = dtype == ODMKV_F16 ? launch_quant<ODMKV_F16>(qa, st)
+                   : dtype == ODMKV_BF16 ? launch_quant<ODMKV_BF16>(qa, st) : launch_quant<ODMKV_F32>(qa, st);
             }
             if (rc) return rc;
         }
