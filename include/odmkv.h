@@ -172,6 +172,16 @@ typedef struct odmkv_packed {
  * (The per-level mask / nonzero of tq_adaptive_backend.py:355-361.) */
 int odmkv_level_counts(const int32_t* bits, int B, int Hkv, int T, int32_t* counts, void* stream);
 
+/* Prepare a store's buffers, laid out by the caller inside one device allocation `arena` (16-byte
+ * aligned), in one launch: the five seg_tile tables (tables_host: host int32 [5][words_per_table], table
+ * li written at byte table_offsets[li] of the arena), bytes [zero_begin, zero_end) cleared (segment
+ * counts, norms, exact rows) and bytes [zero_end, fill_end) set to 0xff (positions: int32 -1).  Offsets
+ * are multiples of 16.  It stands for the empty banks the reference starts from (ExactBank / QuantizedBank
+ * __post_init__, kvquant/tq_adaptive_backend.py:39-40, 97-98), for the packed layout. */
+int odmkv_store_init(void* arena, const int32_t* tables_host, int n_tables, int words_per_table,
+                     const uint32_t* table_offsets, uint64_t zero_begin, uint64_t zero_end, uint64_t fill_end,
+                     void* stream);
+
 /* Quantise and pack T new tokens per (b, h) into a store whose seg_tile tables are filled in
  * and whose seg_count hold the tokens already present (0 after a reset); new tokens are
  * appended behind them and seg_count is advanced.  K, V: [B, Hkv, T, 128] of `dtype` with

@@ -87,6 +87,63 @@ extern "C" int odmkv_level_counts(const int32_t* bits, int B, int Hkv, int T, in
 }
 
 // ------------------------------------------------------------------------------------------------
+// a store's buffers before their first use: segment tables written, counters / norms / exact rows
+// cleared, positions set to -1: one launch
+// ------------------------------------------------------------------------------------------------
+#define SI_MAX_TABLE 640                 // int32 words of tables that travel as kernel arguments
+
+struct StoreInitArgs {
+    uint8_t* arena;
+    unsigned long long zero_begin, zero_end, fill_end;      // [zero_begin, zero_end) = 0, [zero_end, fill_end) = 0xff
+    int n_words;                                            // words of `table`
+    unsigned int table_off[5];                              // byte offset of each level's table in the arena
+    int words_per_table;
+    int32_t table[SI_MAX_TABLE];
+};
+
+__global__ __launch_bounds__(256) void store_init_kernel(StoreInitArgs a) {
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x, nthreads = (size_t)gridDim.x * 256;
+    if (tid < (size_t)a.n_words) {
+        const int li = (int)tid / a.words_per_table, e = (int)tid % a.words_per_table;
+        reinterpret_cast<int32_t*>(a.arena + a.table_off[li])[e] = a.table[tid];
+    }
+    // both regions start and end on multiples of 16 bytes
+    uint4* p = reinterpret_cast<uint4*>(a.arena);
+    const size_t z0 = a.zero_begin / 16, z1 = a.zero_end / 16, f1 = a.fill_end / 16;
+    for (size_t i = z0 + tid; i < z1; i += nthreads) p[i] = make_uint4(0u, 0u, 0u, 0u);
+    for (size_t i = z1 + tid; i < f1; i += nthreads) p[i] = make_uint4(~0u, ~0u, ~0u, ~0u);
+}
+
+extern "C" int odmkv_store_init(void* arena, const int32_t* tables_host, int n_tables, int words_per_table,
+                                const uint32_t* table_offsets, uint64_t zero_begin, uint64_t zero_end, uint64_t fill_end,
+                                void* stream) {
+    ODMKV_CHECK_ARG(arena && tables_host && table_offsets, "store_init: null pointer");
+    ODMKV_CHECK_ARG(n_tables == 5 && words_per_table > 0, "store_init: five tables expected");
+    ODMKV_CHECK_ARG(((uintptr_t)arena & 15) == 0 && zero_begin % 16 == 0 && zero_end % 16 == 0 && fill_end % 16 == 0 &&
+                    zero_begin <= zero_end && zero_end <= fill_end, "store_init: regions must be ordered and 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    StoreInitArgs a;
+    a.arena = (uint8_t*)arena; a.zero_begin = zero_begin; a.zero_end = zero_end; a.fill_end = fill_end;
+    a.words_per_table = words_per_table;
+    for (int li = 0; li < 5; ++li) a.table_off[li] = table_offsets[li];
+    const int n_words = 5 * words_per_table;
+    if (n_words <= SI_MAX_TABLE) {
+        a.n_words = n_words;
+        for (int i = 0; i < n_words; ++i) a.table[i] = tables_host[i];
+    } else {
+        a.n_words = 0;                   // too many segments for the argument block: plain copies
+        for (int li = 0; li < 5; ++li)
+            ODMKV_CHECK_HIP(hipMemcpyAsync((uint8_t*)arena + table_offsets[li], tables_host + (size_t)li * words_per_table,
+                                           (size_t)words_per_table * sizeof(int32_t), hipMemcpyHostToDevice, st));
+    }
+    const size_t chunks = (fill_end - zero_begin) / 16;
+    const int grid = (int)std::min<size_t>(std::max<size_t>((chunks + 255) / 256, 1), 2048);
+    hipLaunchKernelGGL(store_init_kernel, dim3(grid), dim3(256), 0, st, a);
+    ODMKV_CHECK_LAUNCH("store_init_kernel");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
 // compaction: ascending token positions per (bh, level), appended behind what is stored.
 // Two launches over chunks of 2048 tokens: count per (bh, chunk, level), then every chunk places
 // its tokens behind the chunks before it.

@@ -216,13 +216,11 @@ class TurboQuantAdaptiveKVCacheState:
                 spare = torch.empty(off + off // 8, dtype=torch.uint8, device=dev)
             arena, self._arena_spare = spare, arena
         self._arena = arena
-        table = np.zeros(tables_end // 4, np.int32)
-        for li in range(5):
-            o = plan[("seg_tile", li)][0] // 4
-            table[o:o + nseg + 1] = seg_tile[li]
-        arena[:tables_end].view(torch.int32).copy_(torch.from_numpy(table))
-        arena[tables_end:zero_end].zero_()
-        arena[zero_end:pos_end].view(torch.int32).fill_(-1)
+        # tables written, counters / norms / exact rows cleared, positions -1: one launch, the tables in its arguments
+        tables = np.ascontiguousarray(seg_tile, dtype=np.int32)
+        offs = np.array([plan[("seg_tile", li)][0] for li in range(5)], np.uint32)
+        _lib.check(lib.odmkv_store_init(arena.data_ptr(), tables.ctypes.data, 5, nseg + 1, offs.ctypes.data,
+                                        tables_end, zero_end, pos_end, _lib.stream_ptr(dev)))
         return _Buffers(arena, plan)
 
     def _make_struct(self) -> None:
