@@ -193,8 +193,8 @@ int odmkv_store_init(void* arena, const int32_t* tables_host, int n_tables, int 
  *   ss = fma(x_j, x_j, ss) j=0..127; norm = sqrt(ss); u_j = x_j / (norm + 1e-10);
  *   y_i = fma(u_j, Pi[i][j], y_i) j=0..127; code_i = nearer of the two centroids bracketing y_i
  *   (lower index on a tie).
- * fp16 tensors take a shorter route to the same bytes (widths 2, 3, 4): y_i is first estimated on the
- * fp16 matrix cores, and only values next to a decision threshold are recomputed by the chain above.
+ * fp16 and bf16 tensors take a shorter route to the same bytes (widths 2, 3, 4): y_i is first estimated on
+ * the 16-bit matrix cores, and only values next to a decision threshold are recomputed by the chain above.
  * The workspace (odmkv_pack_workspace_bytes(B, Hkv, T) bytes, device) holds per-call scratch only. */
 size_t odmkv_pack_workspace_bytes(int B, int Hkv, int T);
 int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, int Hkv, int T,

@@ -38,7 +38,7 @@ int odmkv_bench_decode_attn(const void* q, int q_dtype, int B, int Hq, float sca
  * one launch of that size can reach on the machine. */
 int odmkv_bench_probe_read(const void* buf, size_t bytes, int grid, void* sink, void* stream);
 
-/* After odmkv_quant_pack(B, Hkv, T, ..., workspace) with fp16 tensors: how many key tiles (counts[0]) and
+/* After odmkv_quant_pack(B, Hkv, T, ..., workspace) with fp16 or bf16 tensors: how many key tiles (counts[0]) and
  * value tiles (counts[1]) of that call the matrix-core quantiser handed to the exact one (8-bit tiles,
  * tiles with a row whose norm is not finite, tiles with more values next to a decision threshold than
  * its list holds).  counts: host int32[2].  Waits for the stream. */

@@ -810,7 +810,7 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// quantise + pack, fp16 inputs: rotation on the fp16 matrix cores, exact codes through a guard band
+// quantise + pack, fp16 and bf16 inputs: rotation on the 16-bit matrix cores, exact codes through a guard band
 //
 // A code is the number of decision thresholds at or below y = sum_j u_j Pi[i][j] (summed in the
 // sequential fp32 order of the definition).  The chain of 128 dependent fp32 steps is what the exact
@@ -834,11 +834,23 @@ __global__ __launch_bounds__(NW * 64) void quant_pack_kernel(QuantArgs a) {
 // packed stream, as the staging formats of the exact kernel expect them.
 // ------------------------------------------------------------------------------------------------
 typedef _Float16 qf_h8 __attribute__((ext_vector_type(8)));
+typedef __bf16 qf_b8 __attribute__((ext_vector_type(8)));
 typedef float qf_f4 __attribute__((ext_vector_type(4)));
 
 #ifndef QF_BAND
 #define QF_BAND 5.0e-5f
 #endif
+// bf16 rows meet Pi as two bf16 terms (16 bits: up to 7.6e-6 more on the estimate, by Cauchy-Schwarz over the row)
+#define QF_BAND_BF16 7.0e-5f
+
+// D += A x B on the matrix cores of the rows' own 16-bit type (operands as they sit in four 32-bit registers)
+template <int DT>
+__device__ static __forceinline__ qf_f4 qf_mfma(const uint4& a, const uint4& b, const qf_f4& c) {
+    if constexpr (DT == ODMKV_F16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(qf_h8, a), __builtin_bit_cast(qf_h8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(qf_b8, a), __builtin_bit_cast(qf_b8, b), c, 0, 0, 0);
+}
 #define QF_LIST 256                     // listed values a wave can hold (it works them off 64 at a time)
 #define QF_GT_BITS 19                   // tile numbers in a list entry
 #define QF_NW 8
@@ -898,7 +910,7 @@ template <int W> struct GuardCoder {
 };
 
 // rotation estimate -> codes into the staging area; values inside the band -> the wave's list
-template <int W, bool IS_V, bool DIRECT>
+template <int DT, int W, bool IS_V, bool DIRECT>
 __device__ static __forceinline__ void qf_code_tile(const void* base, const uint4* piA, const float* thr, QfWave& w,
                                                     uint8_t* stage, int lane, int gt) {
     const int r16 = lane & 15, q = lane >> 4;
@@ -933,17 +945,16 @@ __device__ static __forceinline__ void qf_code_tile(const void* base, const uint
             for (int tb = 0; tb < 4; ++tb) acc[tb] = (qf_f4){0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int ch = 0; ch < 4; ++ch) {
-                const qf_h8 ah = __builtin_bit_cast(qf_h8, piA[(ob * 4 + ch) * 64 + lane]);
-                const qf_h8 al = __builtin_bit_cast(qf_h8, piA[HD * HD / 8 + (ob * 4 + ch) * 64 + lane]);
+                const uint4 ah = piA[(ob * 4 + ch) * 64 + lane];
+                const uint4 al = piA[HD * HD / 8 + (ob * 4 + ch) * 64 + lane];
 #pragma unroll
                 for (int tb = 0; tb < 4; ++tb) {
-                    const qf_h8 xh = __builtin_bit_cast(qf_h8, xb[tb][ch]);
                     if constexpr (IS_V) {
-                        acc[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, ah, acc[tb], 0, 0, 0);
-                        acc[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xh, al, acc[tb], 0, 0, 0);
+                        acc[tb] = qf_mfma<DT>(xb[tb][ch], ah, acc[tb]);
+                        acc[tb] = qf_mfma<DT>(xb[tb][ch], al, acc[tb]);
                     } else {
-                        acc[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, xh, acc[tb], 0, 0, 0);
-                        acc[tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, xh, acc[tb], 0, 0, 0);
+                        acc[tb] = qf_mfma<DT>(ah, xb[tb][ch], acc[tb]);
+                        acc[tb] = qf_mfma<DT>(al, xb[tb][ch], acc[tb]);
                     }
                 }
             }
@@ -986,7 +997,7 @@ __device__ static __forceinline__ void qf_code_tile(const void* base, const uint
 // Entries first .. first + n - 1 of the wave's list (n <= 64), a lane each: the value by the definition's
 // own chain, its code, and that code in place of the estimate's in the packed tile.  The tile's codes,
 // positions and norms were written by this wave: the caller has waited for those stores.
-template <bool IS_V>
+template <int DT, bool IS_V>
 __device__ static void qf_fix_listed(const QuantArgs& a, const float* thrs, const QfWave& w, int lane, int first, int n) {
     const bool on = lane < n;
     const uint32_t e = w.list[first + (on ? lane : 0)];
@@ -1001,11 +1012,20 @@ __device__ static void qf_fix_listed(const QuantArgs& a, const float* thrs, cons
                        (size_t)(a.s.pos[li][slot] - a.pos_offset) * a.sT;
     // written by this wave a moment ago: read past the vector cache
     const float den = __hip_atomic_load((IS_V ? a.s.vnorm[li] : a.s.knorm[li]) + slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1e-10f;
-    RowRegs<ODMKV_F16> x;
+    RowRegs<DT> x;
     x.load(IS_V ? a.V : a.K, off);
     const float4* __restrict__ prow = reinterpret_cast<const float4*>((IS_V ? a.pi_v : a.pi_k) + out * HD);
     float y = 0.0f;
-    const bool row_plain = !(den >= 9.094947017729282e-13f && den <= 1.152921504606847e18f);
+    bool row_plain = !(den >= 9.094947017729282e-13f && den <= 1.152921504606847e18f);
+    if constexpr (DT != ODMKV_F16) {                            // fp16 elements cannot get that small against their norm
+        float amin = INFINITY;
+#pragma unroll
+        for (int j = 0; j < HD; ++j) {
+            const float ax = fabsf(x.get(j));
+            amin = fminf(amin, ax == 0.0f ? INFINITY : ax);
+        }
+        row_plain = row_plain || !(amin >= den * 8.673617379884035e-19f);
+    }
     if (!__any(row_plain)) {                                    // same quotient sequence as the exact kernel
         const float r0 = __builtin_amdgcn_rcpf(den);
         const float rr = __fmaf_rn(__fmaf_rn(-den, r0, 1.0f), r0, r0);
@@ -1089,7 +1109,7 @@ struct QfTile { int gt, li, tile, bh, lo, hi; };
 // their way; its rows are asked for before tile n's listed values are recomputed and its codes packed,
 // and are there when the next round starts.  Only the reads that depend on the tile's own results
 // (the matrix-layout reload, which hits the cache, and the rows of the listed values) are waited for.
-template <bool IS_V>
+template <int DT, bool IS_V>
 __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float* thrs, QfWave& w, uint8_t* stage,
                                int lane, int wave) {
     const int total_tiles = a.tile_base[ODMKV_NQ];
@@ -1132,7 +1152,7 @@ __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float
     if (lane == 0) w.count = 0;
     bool valid = lane >= cur.lo && lane < cur.hi;
     size_t off = 0;
-    RowRegs<ODMKV_F16> x;
+    RowRegs<DT> x;
     if (valid) {
         off = row_offset(cur, a.s.pos[cur.li][(size_t)cur.tile * TILE + lane]);
         x.load(base, off);
@@ -1154,7 +1174,15 @@ __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float
             ss = __fmaf_rn(xj, xj, ss);
         }
         const float norm = sqrtf(ss);
-        const bool ok = !__any(!(ss <= 3.4028234663852886e38f));    // a row with an infinite or NaN norm: exact kernel
+        bool odd = !(ss <= 3.4028234663852886e38f);              // a row with an infinite or NaN norm: exact kernel
+        if constexpr (DT != ODMKV_F16) {
+            // bf16 reaches down to 1e-38: a row whose squares vanish or nearly do (but which is not all zeros) also goes there
+            uint32_t any = 0u;
+#pragma unroll
+            for (int i = 0; i < RowRegs<DT>::N; ++i) any |= x.w[i];
+            odd = odd || ((any & 0x7fff7fffu) != 0u && ss < 1e-30f);
+        }
+        const bool ok = !__any(odd);
         const float* thr = thrs + thr_offset(cur.li);
         const bool direct = cur.li != 1 && cur.lo == 0 && (!IS_V || cur.hi == TILE);
         const int variant = cur.li == 0 ? (direct ? 0 : 1) : cur.li == 1 ? 2 : (direct ? 3 : 4);
@@ -1165,20 +1193,20 @@ __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float
             w.off[lane] = valid ? (unsigned long long)off : ~0ull;
             w.den[lane] = den;
             w.rinv[lane] = 1.0f / den;
-            w.band[lane] = (valid && ss > 0.0f) ? QF_BAND : -1.0f;  // rows of zeros: the estimate is the exact 0
+            w.band[lane] = (valid && ss > 0.0f) ? (DT == ODMKV_F16 ? QF_BAND : QF_BAND_BF16) : -1.0f;  // rows of zeros: the estimate is the exact 0
             wave_lds_fence();
             switch (variant) {
-                case 0: qf_code_tile<2, IS_V, true>(base, piA, thr, w, stage, lane, cur.gt); break;
-                case 1: qf_code_tile<2, IS_V, false>(base, piA, thr, w, stage, lane, cur.gt); break;
-                case 2: qf_code_tile<3, IS_V, false>(base, piA, thr, w, stage, lane, cur.gt); break;
-                case 3: qf_code_tile<4, IS_V, true>(base, piA, thr, w, stage, lane, cur.gt); break;
-                default: qf_code_tile<4, IS_V, false>(base, piA, thr, w, stage, lane, cur.gt); break;
+                case 0: qf_code_tile<DT, 2, IS_V, true>(base, piA, thr, w, stage, lane, cur.gt); break;
+                case 1: qf_code_tile<DT, 2, IS_V, false>(base, piA, thr, w, stage, lane, cur.gt); break;
+                case 2: qf_code_tile<DT, 3, IS_V, false>(base, piA, thr, w, stage, lane, cur.gt); break;
+                case 3: qf_code_tile<DT, 4, IS_V, true>(base, piA, thr, w, stage, lane, cur.gt); break;
+                default: qf_code_tile<DT, 4, IS_V, false>(base, piA, thr, w, stage, lane, cur.gt); break;
             }
             wave_lds_fence();
             n = w.count;
         }
         // the next tile's rows: asked for now, used in the next round
-        RowRegs<ODMKV_F16> xn;
+        RowRegs<DT> xn;
         size_t off_n = 0;
         if (valid_n) {
             off_n = row_offset(nxt, pos_n);
@@ -1208,9 +1236,9 @@ __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float
             __builtin_amdgcn_s_waitcnt(0);                      // this wave's codes, positions and norms are in memory
             while (n_listed >= WAVE) {
                 n_listed -= WAVE;
-                qf_fix_listed<IS_V>(a, thrs, w, lane, n_listed, WAVE);
+                qf_fix_listed<DT, IS_V>(a, thrs, w, lane, n_listed, WAVE);
             }
-            if (!more && n_listed > 0) { qf_fix_listed<IS_V>(a, thrs, w, lane, 0, n_listed); n_listed = 0; }
+            if (!more && n_listed > 0) { qf_fix_listed<DT, IS_V>(a, thrs, w, lane, 0, n_listed); n_listed = 0; }
             if (lane == 0) w.count = n_listed;
             wave_lds_fence();
         }
@@ -1219,9 +1247,10 @@ __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float
     }
 }
 
+template <int DT>
 __global__ __launch_bounds__(QF_NW * 64) void quant_pack_f16_kernel(QuantArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
-    _Float16* pih = reinterpret_cast<_Float16*>(smem);
+    uint16_t* pih = reinterpret_cast<uint16_t*>(smem);
     float* thrs = reinterpret_cast<float*>(smem + QF_PI_BYTES + QF_NW * QP_STAGE);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1229,7 +1258,7 @@ __global__ __launch_bounds__(QF_NW * 64) void quant_pack_f16_kernel(QuantArgs a)
     QfWave& w = reinterpret_cast<QfWave*>(smem + QF_PI_BYTES + QF_NW * QP_STAGE + QF_THR_BYTES)[wave];
     const bool is_v = (blockIdx.x & 1) != 0;
     {
-        // Pi -> hi + lo in fp16, in the order the matrix instruction reads a 16-output x 32-step block:
+        // Pi -> hi + lo in the rows' 16-bit type, in the order the matrix instruction reads a 16-output x 32-step block:
         // lane 16q + r of block (ob, ch) holds Pi[16 ob + r][32 ch + 8 q .. + 7]
         // (all of a thread's reads are asked for at once: eight round trips to memory would cost more
         // than the tiles of a short call)
@@ -1245,15 +1274,14 @@ __global__ __launch_bounds__(QF_NW * 64) void quant_pack_f16_kernel(QuantArgs a)
             const int ob = i >> 4, r = i & 15, ch = j >> 5, q = (j >> 3) & 3, e = j & 7;
             const int dst = (((ob * 4 + ch) * 64) + 16 * q + r) * 8 + e;
             const float pv[4] = {p[k].x, p[k].y, p[k].z, p[k].w};
-            typedef _Float16 qf_h4 __attribute__((ext_vector_type(4)));
-            qf_h4 h, l;
+            uint16_t h[4], l[4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                h[t] = (_Float16)pv[t];
-                l[t] = (_Float16)(pv[t] - (float)h[t]);
+                h[t] = Elem<DT>::from_f32(pv[t]);
+                l[t] = Elem<DT>::from_f32(pv[t] - Elem<DT>::to_f32(h[t]));
             }
-            *reinterpret_cast<qf_h4*>(pih + dst) = h;
-            *reinterpret_cast<qf_h4*>(pih + HD * HD + dst) = l;
+            *reinterpret_cast<uint2*>(pih + dst) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+            *reinterpret_cast<uint2*>(pih + HD * HD + dst) = make_uint2(l[0] | ((uint32_t)l[1] << 16), l[2] | ((uint32_t)l[3] << 16));
         }
         for (int i = tid; i < QP_THR_FLOATS; i += QF_NW * 64) {
             const int li = i < 3 ? 0 : i < 10 ? 1 : i < 25 ? 2 : 3;
@@ -1263,8 +1291,8 @@ __global__ __launch_bounds__(QF_NW * 64) void quant_pack_f16_kernel(QuantArgs a)
     }
     __syncthreads();
     const uint4* piA = reinterpret_cast<const uint4*>(smem);
-    if (is_v) qf_walk<true>(a, piA, thrs, w, stage, lane, wave);
-    else qf_walk<false>(a, piA, thrs, w, stage, lane, wave);
+    if (is_v) qf_walk<DT, true>(a, piA, thrs, w, stage, lane, wave);
+    else qf_walk<DT, false>(a, piA, thrs, w, stage, lane, wave);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1390,11 +1418,12 @@ extern "C" size_t odmkv_pack_workspace_bytes(int B, int Hkv, int T) {
     return pack_redo_offset(B * Hkv, T) + align_up((size_t)(2 + 2 * redo_capacity(B * Hkv, T)) * sizeof(int32_t), 256);
 }
 
+template <int DT>
 static int launch_quant_f16(const QuantArgs& qa, hipStream_t st) {
     const size_t lds = QF_PI_BYTES + (size_t)QF_NW * QP_STAGE + QF_THR_BYTES + QF_NW * sizeof(QfWave);
     static bool attr_set = false;
     if (!attr_set) {
-        ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&quant_pack_f16_kernel),
+        ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&quant_pack_f16_kernel<DT>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_set = true;
     }
@@ -1405,7 +1434,7 @@ static int launch_quant_f16(const QuantArgs& qa, hipStream_t st) {
         if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
     }
     const int per_tensor = std::max(1, std::min((total + QF_NW - 1) / QF_NW, std::max(cus / 2, 1)));
-    hipLaunchKernelGGL(quant_pack_f16_kernel, dim3(2 * per_tensor), dim3(QF_NW * 64), lds, st, qa);
+    hipLaunchKernelGGL(quant_pack_f16_kernel<DT>, dim3(2 * per_tensor), dim3(QF_NW * 64), lds, st, qa);
     ODMKV_CHECK_LAUNCH("quant_pack_f16_kernel");
     return 0;
 }
@@ -1489,12 +1518,12 @@ extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, 
         qa.redo = redo; qa.redo_cap = redo_capacity(nseg, T); qa.from_list = 0;
         if (qa.tile_base[ODMKV_NQ] > 0) {
             int rc;
-            if (dtype == ODMKV_F16 && qa.tile_base[ODMKV_NQ] < (1 << QF_GT_BITS)) {
-                rc = launch_quant_f16(qa, st);
+            if (dtype != ODMKV_F32 && qa.tile_base[ODMKV_NQ] < (1 << QF_GT_BITS)) {
+                rc = dtype == ODMKV_F16 ? launch_quant_f16<ODMKV_F16>(qa, st) : launch_quant_f16<ODMKV_BF16>(qa, st);
                 qa.from_list = 1;
-                if (!rc) rc = launch_quant<ODMKV_F16>(qa, st);
+                if (!rc) rc = dtype == ODMKV_F16 ? launch_quant<ODMKV_F16>(qa, st) : launch_quant<ODMKV_BF16>(qa, st);
             } else {
-                // (fp16 stores of 2^19 tiles and more: the list entries of the fp16 kernel have no room for their numbers)
+                // (16-bit stores of 2^19 tiles and more: the list entries of the matrix-core kernel have no room for their numbers)
                 rc = dtype == ODMKV_F16 ? launch_quant<ODMKV_F16>(qa, st)
                    : dtype == ODMKV_BF16 ? launch_quant<ODMKV_BF16>(qa, st) : launch_quant<ODMKV_F32>(qa, st);
             }

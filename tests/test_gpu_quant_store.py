@@ -237,11 +237,11 @@ def test_edge_cases_and_errors():
         TurboQuantAdaptiveKVCacheState(64, (0, 2, 4), device=DEV, key_quantizer="mse", value_quantizer="mse")
 
 
-# ---- fp16 tensors: the matrix-core estimate with exact codes next to the decision thresholds ----------
-# fp16 rows are quantised by a kernel that estimates the rotation on the fp16 matrix cores and recomputes,
-# by the definition's own chain, only the values within a guard band of a threshold; fp32 rows (and what
-# that kernel hands over) go through the exact kernel alone.  The same numbers given in either type must
-# therefore come out as the same bytes.
+# ---- 16-bit tensors: the matrix-core estimate with exact codes next to the decision thresholds ----------
+# fp16 and bf16 rows are quantised by a kernel that estimates the rotation on the 16-bit matrix cores and
+# recomputes, by the definition's own chain, only the values within a guard band of a threshold; fp32 rows
+# (and what that kernel hands over) go through the exact kernel alone.  The same numbers given in either
+# type must therefore come out as the same bytes.
 def _handed_over(state, B, H, T):
     import ctypes as C
     import os
@@ -256,10 +256,10 @@ def _handed_over(state, B, H, T):
 
 
 def _same_bytes_in_both_types(k16, v16, bits):
-    """Prefill the fp16 tensors and their fp32 copies; compare every quantised level's buffers bit for bit.
-    Returns the tiles the fp16 call handed to the exact kernel (keys, values)."""
+    """Prefill the 16-bit tensors and their fp32 copies; compare every quantised level's buffers bit for bit.
+    Returns the tiles the 16-bit call handed to the exact kernel (keys, values)."""
     B, H, T, _ = k16.shape
-    s16, s32 = _state(), _state()
+    s16, s32 = _state(dtype=k16.dtype), _state(dtype=k16.dtype)
     s16.prefill(k16, v16, bits)
     handed = _handed_over(s16, B, H, T)
     s32.prefill(k16.float(), v16.float(), bits)
@@ -279,8 +279,8 @@ def _same_bytes_in_both_types(k16, v16, bits):
     return handed
 
 
-def _rows_on_thresholds(state, pi, n_rows, per_row, width, g):
-    """fp16 rows whose rotated unit vectors have `per_row` entries on decision thresholds of `width` bits
+def _rows_on_thresholds(state, pi, n_rows, per_row, width, g, dtype=torch.float16):
+    """16-bit rows whose rotated unit vectors have `per_row` entries on decision thresholds of `width` bits
     (up to fp16 rounding of the row: a few 1e-5, well inside the guard band)."""
     cb = state.codebooks.cpu()
     off = {2: 0, 3: 4, 4: 12}[width]
@@ -298,55 +298,63 @@ def _rows_on_thresholds(state, pi, n_rows, per_row, width, g):
         y[r, rest] *= (left / float((y[r, rest] ** 2).sum())) ** 0.5       # unit norm keeps the chosen entries where they are
     x = y @ pi.cpu().double()                                              # y = Pi x
     scale = torch.rand(n_rows, 1, generator=g, dtype=torch.float64) * 20 + 0.05
-    return (x * scale).half()
+    return (x * scale).to(dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("per_row", [2, 100])
-def test_fp16_rows_next_to_thresholds_get_the_exact_codes(per_row):
+def test_fp16_rows_next_to_thresholds_get_the_exact_codes(per_row, dtype):
     g = torch.Generator().manual_seed(per_row)
     B, H, T = 1, 2, 1024
     probe = _state()
     bits = torch.tensor([2, 3, 4], dtype=torch.int32)[torch.randint(3, (B, H, T), generator=g)]
-    k = torch.empty(B, H, T, 128, dtype=torch.float16)
-    v = torch.empty(B, H, T, 128, dtype=torch.float16)
+    k = torch.empty(B, H, T, 128, dtype=dtype)
+    v = torch.empty(B, H, T, 128, dtype=dtype)
     for w in (2, 3, 4):
         m = bits == w
         n = int(m.sum())
-        k[m] = _rows_on_thresholds(probe, probe.pi_k, n, per_row, w, g)
-        v[m] = _rows_on_thresholds(probe, probe.pi_v, n, per_row, w, g)
+        k[m] = _rows_on_thresholds(probe, probe.pi_k, n, per_row, w, g, dtype)
+        v[m] = _rows_on_thresholds(probe, probe.pi_v, n, per_row, w, g, dtype)
     hk, hv = _same_bytes_in_both_types(k.to(DEV), v.to(DEV), bits.to(DEV))
     if per_row == 2:
         assert (hk, hv) == (0, 0)          # a couple of hundred listed values per tile: worked off in the kernel
-    else:
+    elif dtype == torch.float16:
         assert hk > 0 and hv > 0           # thousands per tile: the tiles go to the exact kernel
+    # (bf16 rounds the rows a hundred times more coarsely than the guard band is wide: few entries stay inside it)
     # and the oracle agrees on a sample of the rows
-    ref = KVState(128, (0, 2, 3, 4, 8, 16), seed=42, order="canonical")
+    ref = KVState(128, (0, 2, 3, 4, 8, 16), dtype=dtype, seed=42, order="canonical")
     ref.prefill(k[:, :, :192], v[:, :, :192], bits[:, :, :192])
-    st = _state()
+    st = _state(dtype=dtype)
     st.prefill(k[:, :, :192].to(DEV), v[:, :, :192].to(DEV), bits[:, :, :192].to(DEV))
     _check_store_against_oracle(st, ref)
 
 
-def test_fp16_special_rows_and_ordinary_ones():
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fp16_special_rows_and_ordinary_ones(dtype):
     g = torch.Generator().manual_seed(11)
     B, H, T = 2, 2, 1500
-    k = torch.randn(B, H, T, 128, generator=g).half()
-    v = (torch.randn(B, H, T, 128, generator=g) * 3).half()
+    big, small = (65504.0, 6e-8) if dtype == torch.float16 else (1e18, 1e-10)
+    k = torch.randn(B, H, T, 128, generator=g).to(dtype)
+    v = (torch.randn(B, H, T, 128, generator=g) * 3).to(dtype)
     bits = _rand_bits(g, (B, H, T), levels=(0, 2, 3, 4, 16), probs=(0.1, 0.45, 0.25, 0.15, 0.05))
     hk, hv = _same_bytes_in_both_types(k.to(DEV), v.to(DEV), bits.to(DEV))
     assert (hk, hv) == (0, 0)              # no 8-bit tiles, ordinary rows: nothing for the exact kernel
     # rows of zeros, the largest and the smallest fp16 numbers, a huge outlier, infinities and NaNs
     k2, v2 = k.clone(), v.clone()
     k2[0, 0, 5] = 0; v2[0, 0, 5] = 0
-    k2[0, 1, 70:80] = 65504.0; v2[0, 1, 70:80] = -65504.0
-    k2[1, 0, 200:210] = 6e-8; v2[1, 0, 200:210] *= 1e-4
+    k2[0, 1, 70:80] = big; v2[0, 1, 70:80] = -big
+    k2[1, 0, 200:210] = small; v2[1, 0, 200:210] *= 1e-4
     k2[1, 1, 300, 7] = 30000.0; v2[1, 1, 300, 90] = -30000.0
     k2[0, 0, 900, 3] = float("inf"); v2[0, 0, 901, 4] = float("nan")
     k2[1, 1, 1400, 0] = float("-inf"); v2[1, 1, 1400, 127] = float("inf")
+    odd_k, odd_v = [(0, 0, 900), (1, 1, 1400)], [(0, 0, 901), (1, 1, 1400)]
+    if dtype == torch.bfloat16:            # rows whose squares vanish in fp32 although the row is not zero
+        k2[0, 1, 1000] = 1e-20; v2[0, 1, 1001] = -3e-21
+        odd_k.append((0, 1, 1000)); odd_v.append((0, 1, 1001))
     hk, hv = _same_bytes_in_both_types(k2.to(DEV), v2.to(DEV), bits.to(DEV))
     lvl = bits.numpy()
-    expect_k = int(lvl[0, 0, 900] in (2, 3, 4)) + int(lvl[1, 1, 1400] in (2, 3, 4))
-    expect_v = int(lvl[0, 0, 901] in (2, 3, 4)) + int(lvl[1, 1, 1400] in (2, 3, 4))
+    expect_k = sum(int(lvl[i] in (2, 3, 4)) for i in odd_k)
+    expect_v = sum(int(lvl[i] in (2, 3, 4)) for i in odd_v)
     assert hk <= expect_k and hv <= expect_v       # (two such rows can share a tile)
     assert (hk > 0) == (expect_k > 0) and (hv > 0) == (expect_v > 0)
     # 8-bit tiles always go to the exact kernel
