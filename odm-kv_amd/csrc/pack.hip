@@ -1565,34 +1565,58 @@ struct DequantArgs {
     const float* vnorm;
 };
 
-// x_hat[token][j] = |x| * sum_i c[code_i] * Pi[i][j] on the fp32 matrix cores, like the rotation of the
-// quantiser: operand A = the centroid of the token's code i (lane = token), operand B = row i of Pi
-// from LDS (four outputs per lane), 128 steps of K = 1.  Persistent workgroups of DQ_NW waves keep Pi in
-// LDS (even workgroups keys, odd ones values) and walk the level's tiles, a wave per tile.  A lane
-// ends up with outputs 4c..4c+3 of 32 tokens: 8 (16) bytes of a row per store, the 32 lanes of a half
-// wave covering the row.
+// x_hat[token][j] = |x| * sum_i c[code_i] * Pi[i][j] on the fp16 matrix cores (v_mfma_f32_16x16x32_f16): operand
+// A = Pi^T (rows = outputs j, steps = i), B = the centroids of 16 tokens' codes, both as fp16 high + low terms
+// (three products: hi*hi, lo*hi, hi*lo; the fourth is below 2^-22), accumulated in fp32.  The result differs from
+// the fp32 sum by about 1e-6 of the row's norm: less than the rounding of a 16-bit cache by two orders of magnitude.
+// Persistent workgroups of DQ_NW waves keep Pi^T in LDS in operand order (even workgroups keys, odd ones values) and
+// walk the level's tiles, a wave per tile.  A lane ends up with four consecutive outputs of one token: 8 (16) bytes
+// of a row per store.
 #define DQ_NW 8
-#define DQ_GROUP 16                       // centroid lookups are done in blocks, ahead of their matrix instructions
 template <int W, int DT>
 __global__ __launch_bounds__(DQ_NW * 64) void dequant_kernel(DequantArgs a, int n_tiles) {
     extern __shared__ __align__(16) uint8_t smem[];
-    float* pis = reinterpret_cast<float*>(smem);                                  // Pi [i][j], as stored
+    uint16_t* pih = reinterpret_cast<uint16_t*>(smem);                             // Pi^T hi, then lo, in operand order
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     uint8_t* codes = smem + QP_PI_BYTES + wave * QP_STAGE;                         // this wave's [token][dim] codes (values)
-    float* cb = reinterpret_cast<float*>(smem + QP_PI_BYTES + DQ_NW * QP_STAGE);   // [256] centroids
-    float* norms = cb + 256 + wave * TILE;                                         // [DQ_NW][64] norm of the wave's tokens
+    uint32_t* cb = reinterpret_cast<uint32_t*>(smem + QP_PI_BYTES + DQ_NW * QP_STAGE);   // [256] centroids: fp16 hi | lo << 16
+    float* norms = reinterpret_cast<float*>(cb + 256) + wave * TILE;              // [DQ_NW][64] norm of the wave's tokens
     long long* offs = reinterpret_cast<long long*>(cb + 256 + DQ_NW * TILE) + wave * TILE;   // element offset of the row, -1: none
     const bool is_v = (blockIdx.x & 1) != 0;
     {
+        // lane 16q + r of block (jb, ch) holds Pi[32 ch + 8 q .. + 7][16 jb + r]
         const float4* __restrict__ src = reinterpret_cast<const float4*>(is_v ? a.pi_v : a.pi_k);
-        for (int i = tid; i < HD * HD / 4; i += DQ_NW * 64) reinterpret_cast<float4*>(pis)[i] = src[i];
-        for (int i = tid; i < (1 << W); i += DQ_NW * 64) cb[i] = a.cb[i];
+        constexpr int PER_THREAD = HD * HD / 4 / (DQ_NW * 64);
+        float4 p[PER_THREAD];
+#pragma unroll
+        for (int k = 0; k < PER_THREAD; ++k) p[k] = src[tid + k * (DQ_NW * 64)];
+#pragma unroll
+        for (int k = 0; k < PER_THREAD; ++k) {
+            const int c = tid + k * (DQ_NW * 64);                // four consecutive j of row i
+            const int i = c >> 5, j0 = (c & 31) * 4;
+            const int ch = i >> 5, q = (i >> 3) & 3, e = i & 7;
+            const float pv[4] = {p[k].x, p[k].y, p[k].z, p[k].w};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int j = j0 + t, jb = j >> 4, r = j & 15;
+                const int dst = (((jb * 4 + ch) * 64) + 16 * q + r) * 8 + e;
+                const uint16_t h = Elem<ODMKV_F16>::from_f32(pv[t]);
+                pih[dst] = h;
+                pih[HD * HD + dst] = Elem<ODMKV_F16>::from_f32(pv[t] - Elem<ODMKV_F16>::to_f32(h));
+            }
+        }
+        for (int i = tid; i < (1 << W); i += DQ_NW * 64) {
+            const float c = a.cb[i];
+            const uint16_t h = Elem<ODMKV_F16>::from_f32(c);
+            cb[i] = (uint32_t)h | ((uint32_t)Elem<ODMKV_F16>::from_f32(c - Elem<ODMKV_F16>::to_f32(h)) << 16);
+        }
     }
     __syncthreads();
+    const uint4* piA = reinterpret_cast<const uint4*>(smem);
     void* out = is_v ? a.V : a.K;
     const int wg = blockIdx.x >> 1, n_wg = gridDim.x >> 1;
-    const float4* __restrict__ brow = reinterpret_cast<const float4*>(pis) + (lane & 31);
+    const int r16 = lane & 15, q = lane >> 4;
     for (int tile = wg * DQ_NW + wave; tile < n_tiles; tile += n_wg * DQ_NW) {
         const int bh = find_segment(a.seg_tile, a.nseg, tile);
         const int ts = (tile - a.seg_tile[bh]) * TILE;
@@ -1608,8 +1632,8 @@ __global__ __launch_bounds__(DQ_NW * 64) void dequant_kernel(DequantArgs a, int 
             offs[lane] = write ? (long long)((size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH + (size_t)t * a.sT) : -1ll;
             norms[lane] = valid ? (is_v ? a.vnorm[slot] : a.knorm[slot]) : 0.0f;
         }
-        // the lane's 128 codes -> one byte each in LDS, [token][dim]: the matrix instructions below want a
-        // token per lane, the tile keeps (4 tokens x 32 dims) of keys or (16 tokens x 8 dims) of values per lane
+        // the lane's 128 codes -> one byte each in LDS, [token][dim]: the matrix operand below wants eight consecutive
+        // dims of a token per lane, the tile keeps (4 tokens x 32 dims) of keys or (16 tokens x 8 dims) of values per lane
         {
             const int n = lane & 15, j = lane >> 4;
             const uint8_t* src = (is_v ? a.vcodes : a.kcodes) + (size_t)tile * (TILE * 16 * W);
@@ -1639,47 +1663,50 @@ __global__ __launch_bounds__(DQ_NW * 64) void dequant_kernel(DequantArgs a, int 
             }
         }
         wave_lds_fence();
-        f32x32 acc0, acc1, acc2, acc3;
-#pragma unroll
-        for (int i = 0; i < 32; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; acc2[i] = 0.0f; acc3[i] = 0.0f; }
-        float4 b = brow[0];
-#pragma unroll
-        for (int i0 = 0; i0 < HD; i0 += DQ_GROUP) {
-            float y[DQ_GROUP];
-            {
-                const uint4 v = *reinterpret_cast<const uint4*>(&codes[lane * CODE_ROW + i0]);
-                const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                for (int g = 0; g < DQ_GROUP; ++g) y[g] = cb[(w4[g >> 2] >> (8 * (g & 3))) & 0xffu];
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int g = 0; g < DQ_GROUP; ++g) {
-                const int in = i0 + g + 1 < HD ? i0 + g + 1 : i0 + g;
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(y[g], b.x, acc0, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(y[g], b.y, acc1, 0, 0, 0);
-                acc2 = __builtin_amdgcn_mfma_f32_32x32x1f32(y[g], b.z, acc2, 0, 0, 0);
-                acc3 = __builtin_amdgcn_mfma_f32_32x32x1f32(y[g], b.w, acc3, 0, 0, 0);
-                b = brow[in * (HD / 4)];
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        int ln = lane;
-        asm volatile("" : "+v"(ln));                                 // keeps the store addresses out of the loop above
-        const int c4 = (ln & 31) * 4;
-#pragma unroll
-        for (int vv = 0; vv < 32; ++vv) {
-            const int token = mfma_token(vv, ln);
+#pragma unroll 1
+        for (int tb = 0; tb < 4; ++tb) {
+            // (the lane index is made opaque per round: Pi^T's 64 operand reads do not depend on the round, and hoisted
+            // out of it they would take every register there is)
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const int token = 16 * tb + r16;
             const long long off = offs[token];
-            const float n = norms[token];
-            if (off >= 0) {
-                const float r[4] = {acc0[vv] * n, acc1[vv] * n, acc2[vv] * n, acc3[vv] * n};
-                if constexpr (DT == ODMKV_F32) {
-                    *reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + off + c4) = make_float4(r[0], r[1], r[2], r[3]);
-                } else {
-                    const uint32_t lo = (uint32_t)Elem<DT>::from_f32(r[0]) | ((uint32_t)Elem<DT>::from_f32(r[1]) << 16);
-                    const uint32_t hi2 = (uint32_t)Elem<DT>::from_f32(r[2]) | ((uint32_t)Elem<DT>::from_f32(r[3]) << 16);
-                    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(out) + off + c4) = make_uint2(lo, hi2);
+            const float nrm = norms[token];
+            // operand B: the centroids of the token's codes 32 ch + 8 q .. + 7, high and low halves
+            uint4 bh4[4], bl4[4];
+#pragma unroll
+            for (int ch = 0; ch < 4; ++ch) {
+                const uint2 cw = *reinterpret_cast<const uint2*>(&codes[token * CODE_ROW + 32 * ch + 8 * q]);
+                const uint32_t w2[2] = {cw.x, cw.y};
+                uint32_t t[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) t[e] = cb[(w2[e >> 2] >> (8 * (e & 3))) & 0xffu];
+                bh4[ch] = make_uint4(__builtin_amdgcn_perm(t[1], t[0], 0x05040100u), __builtin_amdgcn_perm(t[3], t[2], 0x05040100u),
+                                     __builtin_amdgcn_perm(t[5], t[4], 0x05040100u), __builtin_amdgcn_perm(t[7], t[6], 0x05040100u));
+                bl4[ch] = make_uint4(__builtin_amdgcn_perm(t[1], t[0], 0x07060302u), __builtin_amdgcn_perm(t[3], t[2], 0x07060302u),
+                                     __builtin_amdgcn_perm(t[5], t[4], 0x07060302u), __builtin_amdgcn_perm(t[7], t[6], 0x07060302u));
+            }
+#pragma unroll
+            for (int jb = 0; jb < 8; ++jb) {
+                qf_f4 acc = (qf_f4){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int ch = 0; ch < 4; ++ch) {
+                    const uint4 ah = piA[(jb * 4 + ch) * 64 + ln];
+                    const uint4 al = piA[HD * HD / 8 + (jb * 4 + ch) * 64 + ln];
+                    acc = qf_mfma<ODMKV_F16>(ah, bh4[ch], acc);
+                    acc = qf_mfma<ODMKV_F16>(al, bh4[ch], acc);
+                    acc = qf_mfma<ODMKV_F16>(ah, bl4[ch], acc);
+                }
+                if (off >= 0) {                                     // outputs 16 jb + 4 q .. + 3 of the token
+                    const float r[4] = {acc[0] * nrm, acc[1] * nrm, acc[2] * nrm, acc[3] * nrm};
+                    const int c4 = 16 * jb + 4 * q;
+                    if constexpr (DT == ODMKV_F32) {
+                        *reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + off + c4) = make_float4(r[0], r[1], r[2], r[3]);
+                    } else {
+                        const uint32_t lo = (uint32_t)Elem<DT>::from_f32(r[0]) | ((uint32_t)Elem<DT>::from_f32(r[1]) << 16);
+                        const uint32_t hi2 = (uint32_t)Elem<DT>::from_f32(r[2]) | ((uint32_t)Elem<DT>::from_f32(r[3]) << 16);
+                        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(out) + off + c4) = make_uint2(lo, hi2);
+                    }
                 }
             }
         }

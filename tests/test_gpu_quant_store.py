@@ -94,12 +94,16 @@ def _check_store_against_oracle(state, ref: KVState):
         np.testing.assert_array_equal(ex["v"][o_got], ref.exact.v.view(torch.int16).numpy()[o_ref])
 
 
-def _ulp_close_fp16(a: torch.Tensor, b: torch.Tensor, max_ulp=1, max_frac=0.02):
+def _ulp_close_fp16(a: torch.Tensor, b: torch.Tensor, max_ulp=1, max_frac=0.02, sum_noise=1e-6):
+    """a equals b up to how an fp32 sum of 128 terms depends on its order (the oracle sums in the canonical
+    order, the kernel on the matrix cores): `sum_noise` of the row's norm before the rounding to fp16, hence at
+    most one fp16 step, or that noise where it is larger than a step (elements near zero), and few such."""
     ai, bi = a.view(torch.int16).int(), b.view(torch.int16).int()
     ai = torch.where(ai < 0, -32768 - ai, ai)          # map sign-magnitude to a monotone scale
     bi = torch.where(bi < 0, -32768 - bi, bi)
     d = (ai - bi).abs()
-    assert int(d.max()) <= max_ulp, f"max fp16 ulp distance {int(d.max())}"
+    small = (a.float() - b.float()).abs() <= sum_noise * b.float().norm(dim=-1, keepdim=True)
+    assert int(d[~small].max() if (~small).any() else 0) <= max_ulp, f"max fp16 ulp distance {int(d[~small].max())}"
     assert float((d > 0).float().mean()) <= max_frac
 
 
