@@ -182,6 +182,14 @@ int odmkv_store_init(void* arena, const int32_t* tables_host, int n_tables, int 
                      const uint32_t* table_offsets, uint64_t zero_begin, uint64_t zero_end, uint64_t fill_end,
                      void* stream);
 
+/* Move what a staging store holds into `store`: for every level and segment the tiles that hold tokens
+ * (codes, norms, positions, exact rows), and the segment counts.  A staging store is a store whose
+ * segments are laid out for the worst case (every token of a call at every level), so that
+ * odmkv_quant_pack can fill it before the host has read the level counts back; `store` is laid out for
+ * the counts, prepared by odmkv_store_init and still empty.  No counterpart in the reference, whose
+ * banks grow by torch.cat (kvquant/tq_adaptive_backend.py:46-52, 149-174). */
+int odmkv_store_gather(const odmkv_packed_t* staging, const odmkv_packed_t* store, void* stream);
+
 /* Quantise and pack T new tokens per (b, h) into a store whose seg_tile tables are filled in
  * and whose seg_count hold the tokens already present (0 after a reset); new tokens are
  * appended behind them and seg_count is advanced.  K, V: [B, Hkv, T, 128] of `dtype` with

@@ -1103,16 +1103,20 @@ __device__ static __forceinline__ void qf_store_tile(const QuantArgs& a, const u
     }
 }
 
-struct QfTile { int gt, li, tile, bh, lo, hi; };
+struct QfTile { int wi, gt, li, tile, bh, lo, hi; };
+#define QF_MAX_RUNS 1024                // (level, segment) pairs whose tile counts fit the walk table
 
-// Per wave the tiles form a pipeline: while tile n is coded, the token positions of tile n + 1 are on
-// their way; its rows are asked for before tile n's listed values are recomputed and its codes packed,
-// and are there when the next round starts.  Only the reads that depend on the tile's own results
-// (the matrix-layout reload, which hits the cache, and the rows of the listed values) are waited for.
+// Per wave: the next tile and the positions of its tokens are looked up while the current tile's rows are on
+// their way.  (Requesting the next tile's rows a whole tile ahead was measured: no faster, and its 64 registers
+// per lane are the ones the kernel does not have.)
 template <int DT, bool IS_V>
 __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float* thrs, QfWave& w, uint8_t* stage,
-                               int lane, int wave) {
-    const int total_tiles = a.tile_base[ODMKV_NQ];
+                               int lane, int wave, const int* wbase) {
+    // wbase (LDS, or null): running count, over the (level, segment) pairs, of the tiles that receive tokens in this
+    // call.  The waves then share out those tiles alone; a store laid out for the worst case, or one that already
+    // holds a long context, has many times more tiles than that.  Without the table every tile is looked at.
+    const int n_runs = ODMKV_NQ * a.nseg;
+    const int total_tiles = wbase ? wbase[n_runs] : a.tile_base[ODMKV_NQ];
     const int stride = (gridDim.x >> 1) * QF_NW;
     int32_t* redo_count = a.redo + (IS_V ? 1 : 0);
     int32_t* redo_list = a.redo + 2 + (IS_V ? a.redo_cap : 0);
@@ -1124,20 +1128,34 @@ __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float
         }
     };
     // the next tile at or behind gt with new tokens of widths 2, 3, 4; 8-bit tiles on the way are handed over
-    const auto next_tile = [&](int gt, QfTile& d) -> bool {
-        for (; gt < total_tiles; gt += stride) {
-            int li = 0;
+    const auto next_tile = [&](int wi, QfTile& d) -> bool {
+        for (; wi < total_tiles; wi += stride) {
+            int li, bh, tile, lo, hi;
+            if (wbase) {
+                int e = 0;                                       // the largest pair with wbase[e] <= wi
+                for (int step = QF_MAX_RUNS / 2; step >= 1; step >>= 1)
+                    if (e + step < n_runs && wbase[e + step] <= wi) e += step;
+                li = e / a.nseg; bh = e - li * a.nseg;
+                const int old = a.old_count[e];
+                const int local = old / TILE + (wi - wbase[e]);
+                tile = a.s.seg_tile[li][bh] + local;
+                lo = max(old - local * TILE, 0);
+                hi = min(a.s.seg_count[li][bh] - local * TILE, TILE);
+            } else {
+                li = 0;
 #pragma unroll
-            for (int k = 1; k < ODMKV_NQ; ++k) li += (gt >= a.tile_base[k]);
-            const int tile = gt - a.tile_base[li];
-            const int32_t* seg_tile = a.s.seg_tile[li];
-            const int bh = find_segment(seg_tile, a.nseg, tile);
-            const int ts = (tile - seg_tile[bh]) * TILE;
-            const int lo = max(a.old_count[li * a.nseg + bh] - ts, 0);
-            const int hi = min(a.s.seg_count[li][bh] - ts, TILE);
-            if (lo >= hi) continue;                             // nothing new in this tile (wave-uniform)
+                for (int k = 1; k < ODMKV_NQ; ++k) li += (wi >= a.tile_base[k]);
+                tile = wi - a.tile_base[li];
+                const int32_t* seg_tile = a.s.seg_tile[li];
+                bh = find_segment(seg_tile, a.nseg, tile);
+                const int ts = (tile - seg_tile[bh]) * TILE;
+                lo = max(a.old_count[li * a.nseg + bh] - ts, 0);
+                hi = min(a.s.seg_count[li][bh] - ts, TILE);
+                if (lo >= hi) continue;                         // nothing new in this tile (wave-uniform)
+            }
+            const int gt = a.tile_base[li] + tile;
             if (li == 3) { hand_over(gt); continue; }
-            d.gt = gt; d.li = li; d.tile = tile; d.bh = bh; d.lo = lo; d.hi = hi;
+            d.wi = wi; d.gt = gt; d.li = li; d.tile = tile; d.bh = bh; d.lo = lo; d.hi = hi;
             return true;
         }
         return false;
@@ -1147,24 +1165,26 @@ __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float
     };
 
     QfTile cur;
-    if (!next_tile((blockIdx.x >> 1) * QF_NW + wave, cur)) return;
+    bool more = next_tile((blockIdx.x >> 1) * QF_NW + wave, cur);
+    if (!more) return;
     int n_listed = 0;                                           // == w.count between tiles
     if (lane == 0) w.count = 0;
-    bool valid = lane >= cur.lo && lane < cur.hi;
-    size_t off = 0;
-    RowRegs<DT> x;
-    if (valid) {
-        off = row_offset(cur, a.s.pos[cur.li][(size_t)cur.tile * TILE + lane]);
-        x.load(base, off);
-    } else {
-        x.zero();
-    }
+    int pos = 0;
+    if (lane >= cur.lo && lane < cur.hi) pos = a.s.pos[cur.li][(size_t)cur.tile * TILE + lane];
     while (true) {
+        const bool valid = lane >= cur.lo && lane < cur.hi;
+        size_t off = 0;
+        RowRegs<DT> x;
+        if (valid) {
+            off = row_offset(cur, pos);
+            x.load(base, off);
+        } else {
+            x.zero();
+        }
+        // the next tile and its positions are found while this tile's rows are on their way
         QfTile nxt;
-        const bool more = next_tile(cur.gt + stride, nxt);
-        const bool valid_n = more && lane >= nxt.lo && lane < nxt.hi;
-        int pos_n = 0;
-        if (valid_n) pos_n = a.s.pos[nxt.li][(size_t)nxt.tile * TILE + lane];
+        more = next_tile(cur.wi + stride, nxt);
+        if (more && lane >= nxt.lo && lane < nxt.hi) pos = a.s.pos[nxt.li][(size_t)nxt.tile * TILE + lane];
 
         // a token per lane: the norm in the definition's order, and what the matrix layout needs per token
         float ss = 0.0f;
@@ -1205,15 +1225,6 @@ __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float
             wave_lds_fence();
             n = w.count;
         }
-        // the next tile's rows: asked for now, used in the next round
-        RowRegs<DT> xn;
-        size_t off_n = 0;
-        if (valid_n) {
-            off_n = row_offset(nxt, pos_n);
-            xn.load(base, off_n);
-        } else {
-            xn.zero();
-        }
         if (ok && n <= QF_LIST) {
             switch (variant) {
                 case 0: qf_store_tile<2, IS_V, true>(a, stage, lane, cur.li, cur.tile, cur.lo); break;
@@ -1243,7 +1254,7 @@ __device__ static void qf_walk(const QuantArgs& a, const uint4* piA, const float
             wave_lds_fence();
         }
         if (!more) break;
-        cur = nxt; valid = valid_n; off = off_n; x = xn;
+        cur = nxt;
     }
 }
 
@@ -1256,7 +1267,21 @@ __global__ __launch_bounds__(QF_NW * 64) void quant_pack_f16_kernel(QuantArgs a)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     uint8_t* stage = smem + QF_PI_BYTES + wave * QP_STAGE;
     QfWave& w = reinterpret_cast<QfWave*>(smem + QF_PI_BYTES + QF_NW * QP_STAGE + QF_THR_BYTES)[wave];
+    int* wbase = reinterpret_cast<int*>(smem + QF_PI_BYTES + QF_NW * QP_STAGE + QF_THR_BYTES + QF_NW * sizeof(QfWave));
     const bool is_v = (blockIdx.x & 1) != 0;
+    const int n_runs = ODMKV_NQ * a.nseg;
+    const bool walk_table = n_runs <= QF_MAX_RUNS;
+    if (walk_table) {
+        // tiles of every (level, segment) pair that receive tokens: behind the tiles filled before, up to the new count
+        for (int e = tid; e < QF_MAX_RUNS; e += QF_NW * 64) {
+            int n = 0;
+            if (e < n_runs) {
+                const int old = a.old_count[e], cnt = a.s.seg_count[e / a.nseg][e % a.nseg];
+                n = cnt > old ? (cnt + TILE - 1) / TILE - old / TILE : 0;
+            }
+            wbase[e + 1] = n;
+        }
+    }
     {
         // Pi -> hi + lo in the rows' 16-bit type, in the order the matrix instruction reads a 16-output x 32-step block:
         // lane 16q + r of block (ob, ch) holds Pi[16 ob + r][32 ch + 8 q .. + 7]
@@ -1290,9 +1315,26 @@ __global__ __launch_bounds__(QF_NW * 64) void quant_pack_f16_kernel(QuantArgs a)
         }
     }
     __syncthreads();
+    if (walk_table && wave == 0) {
+        // running sum by one wave: 16 entries per lane, a scan over the lanes' totals, the entries again
+        int mine[QF_MAX_RUNS / 64], tot = 0;
+#pragma unroll
+        for (int i = 0; i < QF_MAX_RUNS / 64; ++i) { mine[i] = wbase[lane * (QF_MAX_RUNS / 64) + i + 1]; tot += mine[i]; }
+        int incl = tot;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int up = __shfl_up(incl, o, WAVE);
+            if (lane >= o) incl += up;
+        }
+        int run = incl - tot;
+#pragma unroll
+        for (int i = 0; i < QF_MAX_RUNS / 64; ++i) { run += mine[i]; wbase[lane * (QF_MAX_RUNS / 64) + i + 1] = run; }
+        if (lane == 0) wbase[0] = 0;
+    }
+    __syncthreads();
     const uint4* piA = reinterpret_cast<const uint4*>(smem);
-    if (is_v) qf_walk<DT, true>(a, piA, thrs, w, stage, lane, wave);
-    else qf_walk<DT, false>(a, piA, thrs, w, stage, lane, wave);
+    if (is_v) qf_walk<DT, true>(a, piA, thrs, w, stage, lane, wave, walk_table ? wbase : nullptr);
+    else qf_walk<DT, false>(a, piA, thrs, w, stage, lane, wave, walk_table ? wbase : nullptr);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1319,12 +1361,16 @@ __device__ static inline uint16_t to_store16(typename Elem<DT>::raw v) {
 
 template <int DT, int ODT>
 __global__ __launch_bounds__(64) void exact_gather_kernel(ExactArgs a) {
-    const int lane = threadIdx.x, tile = blockIdx.x;
-    const int bh = find_segment(a.seg_tile, a.nseg, tile);
-    const int ts = (tile - a.seg_tile[bh]) * TILE;
-    const int lo = max(a.old_count[bh] - ts, 0);
-    const int hi = min(a.seg_count[bh] - ts, TILE);
-    if (lane < lo || lane >= hi) return;
+    // grid (slices, segments): the workgroups of a segment share out its tiles that receive tokens (a store laid
+    // out for the worst case has thousands of tiles and a handful of them in use)
+    const int lane = threadIdx.x, bh = blockIdx.y;
+    const int old = a.old_count[bh], cnt = a.seg_count[bh], first = a.seg_tile[bh];
+    for (int local = old / TILE + blockIdx.x; local * TILE < cnt; local += gridDim.x) {
+    const int tile = first + local;
+    const int ts = local * TILE;
+    const int lo = max(old - ts, 0);
+    const int hi = min(cnt - ts, TILE);
+    if (lane < lo || lane >= hi) continue;
     const size_t slot = (size_t)tile * TILE + lane;
     const int t = a.pos[slot] - a.pos_offset;
     const size_t off = (size_t)(bh / a.Hkv) * a.sB + (size_t)(bh % a.Hkv) * a.sH + (size_t)t * a.sT;
@@ -1344,6 +1390,7 @@ __global__ __launch_bounds__(64) void exact_gather_kernel(ExactArgs a) {
     load_row<DT>(a.V, off, x);
 #pragma unroll
     for (int j = 0; j < HD; ++j) vd[exact_v_index(lane, j)] = Elem<ODT>::from_f32(x[j]);
+    }
 }
 
 // one new token per (b, h) behind the stored exact tokens
@@ -1420,7 +1467,7 @@ extern "C" size_t odmkv_pack_workspace_bytes(int B, int Hkv, int T) {
 
 template <int DT>
 static int launch_quant_f16(const QuantArgs& qa, hipStream_t st) {
-    const size_t lds = QF_PI_BYTES + (size_t)QF_NW * QP_STAGE + QF_THR_BYTES + QF_NW * sizeof(QfWave);
+    const size_t lds = QF_PI_BYTES + (size_t)QF_NW * QP_STAGE + QF_THR_BYTES + QF_NW * sizeof(QfWave) + (QF_MAX_RUNS + 1) * sizeof(int);
     static bool attr_set = false;
     if (!attr_set) {
         ODMKV_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&quant_pack_f16_kernel<DT>),
@@ -1464,10 +1511,11 @@ static int launch_quant(const QuantArgs& qa, hipStream_t st) {
 
 template <int DT>
 static int launch_exact(const ExactArgs& ea, int out_dt, int n_tiles, hipStream_t st) {
+    const dim3 grid(std::max(1, std::min(64, n_tiles / std::max(ea.nseg, 1))), ea.nseg);
     if (out_dt == ODMKV_F16)
-        hipLaunchKernelGGL((exact_gather_kernel<DT, ODMKV_F16>), dim3(n_tiles), dim3(64), 0, st, ea);
+        hipLaunchKernelGGL((exact_gather_kernel<DT, ODMKV_F16>), grid, dim3(64), 0, st, ea);
     else
-        hipLaunchKernelGGL((exact_gather_kernel<DT, ODMKV_BF16>), dim3(n_tiles), dim3(64), 0, st, ea);
+        hipLaunchKernelGGL((exact_gather_kernel<DT, ODMKV_BF16>), grid, dim3(64), 0, st, ea);
     ODMKV_CHECK_LAUNCH("exact_gather_kernel");
     return 0;
 }
@@ -1542,6 +1590,85 @@ extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, 
                                      : launch_exact<ODMKV_F32>(ea, store->exact_dtype, store->n_tiles[4], st);
         if (rc) return rc;
     }
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// the tiles of a staging store (every segment laid out for the worst case, so that it can be filled
+// before anybody knows the level counts) moved into a store laid out for the counts
+// ------------------------------------------------------------------------------------------------
+struct GatherArgs {
+    odmkv_packed_t src, dst;
+    int nseg;
+};
+
+__global__ __launch_bounds__(256) void store_gather_kernel(GatherArgs a) {
+    // grid (slices, segments, levels): the wavefronts of a (level, segment)'s workgroups share out its tiles that hold
+    // tokens, a tile per wavefront at a time
+    const int tid = threadIdx.x & 63, wave = threadIdx.x >> 6, bh = blockIdx.y, li = blockIdx.z;
+    const int count = a.src.seg_count[li][bh];
+    if (blockIdx.x == 0 && threadIdx.x == 0) a.dst.seg_count[li][bh] = count;
+    const int src0 = a.src.seg_tile[li][bh], dst0 = a.dst.seg_tile[li][bh];
+    for (int local = blockIdx.x * 4 + wave; local * TILE < count; local += gridDim.x * 4) {
+    const int tile = dst0 + local;
+    const int hi = min(count - local * TILE, TILE);
+    const size_t st = (size_t)src0 + local;                      // the tile in the staging store
+    // lanes behind the count keep what the destination was prepared with (position -1, norm 0, zero rows)
+    if (tid < hi) a.dst.pos[li][(size_t)tile * TILE + tid] = a.src.pos[li][st * TILE + tid];
+    if (li < ODMKV_NQ) {
+        const int W = width_of(li);
+        if (tid < hi) {
+            a.dst.knorm[li][(size_t)tile * TILE + tid] = a.src.knorm[li][st * TILE + tid];
+            a.dst.vnorm[li][(size_t)tile * TILE + tid] = a.src.vnorm[li][st * TILE + tid];
+        }
+        const int n16 = TILE * W;                                // 16-byte pieces per tensor and tile
+        const uint4* sk = reinterpret_cast<const uint4*>(a.src.kcodes[li]) + st * n16;
+        const uint4* sv = reinterpret_cast<const uint4*>(a.src.vcodes[li]) + st * n16;
+        uint4* dk = reinterpret_cast<uint4*>(a.dst.kcodes[li]) + (size_t)tile * n16;
+        uint4* dv = reinterpret_cast<uint4*>(a.dst.vcodes[li]) + (size_t)tile * n16;
+        for (int i = tid; i < n16; i += 64) { dk[i] = sk[i]; dv[i] = sv[i]; }
+    } else {
+        // exact rows (quant.h: tile layouts): key piece 4b + k of lane (n, j) belongs to slot key_slot(n, b); value
+        // piece 8k + m of the lane holds slots 32k + 8j .. + 7 of one dim.  Rows behind the count are not copied.
+        constexpr int n16 = TILE * HD * 2 / 16;
+        const uint4* sk = reinterpret_cast<const uint4*>(a.src.kexact) + st * n16;
+        const uint4* sv = reinterpret_cast<const uint4*>(a.src.vexact) + st * n16;
+        uint4* dk = reinterpret_cast<uint4*>(a.dst.kexact) + (size_t)tile * n16;
+        uint4* dv = reinterpret_cast<uint4*>(a.dst.vexact) + (size_t)tile * n16;
+        for (int i = tid; i < n16; i += 64) {
+            const int c = i >> 6, l = i & 63, n = l & 15, j = l >> 4;
+            if (key_slot(n, c >> 2) < hi) dk[i] = sk[i];
+            const int s0 = 32 * (c >> 3) + 8 * j;                // first of the piece's eight slots
+            if (s0 < hi) {
+                uint4 v = sv[i];
+                const int keep = hi - s0;                        // slots s0 .. s0 + keep - 1 are stored
+                if (keep < 8) {
+                    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (e >= keep) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+                    v = make_uint4(w[0], w[1], w[2], w[3]);
+                }
+                dv[i] = v;
+            }
+        }
+    }
+    }
+}
+
+extern "C" int odmkv_store_gather(const odmkv_packed_t* staging, const odmkv_packed_t* store, void* stream) {
+    if (int rc = check_store(staging, "store_gather")) return rc;
+    if (int rc = check_store(store, "store_gather")) return rc;
+    ODMKV_CHECK_ARG(staging->B == store->B && staging->Hkv == store->Hkv && staging->exact_dtype == store->exact_dtype,
+                    "store_gather: the two stores differ in shape or exact dtype");
+    GatherArgs a;
+    a.src = *staging; a.dst = *store; a.nseg = store->B * store->Hkv;
+    ODMKV_CHECK_ARG(a.nseg <= 65535, "store_gather: at most 65535 (sequence, head) pairs");
+    int most = 1;
+    for (int li = 0; li <= ODMKV_NQ; ++li) most = std::max(most, store->n_tiles[li]);
+    const dim3 grid(std::max(1, std::min(128, (most / a.nseg + 4) / 4)), a.nseg, ODMKV_NQ + 1);
+    hipLaunchKernelGGL(store_gather_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);
+    ODMKV_CHECK_LAUNCH("store_gather_kernel");
     return 0;
 }
 

@@ -81,6 +81,52 @@ class _Buffers:
 
 
 _ARENA_HINT: dict = {}     # (device, segments, tokens) -> bytes of the last store first filled with that shape
+_STAGING_LIMIT = 1 << 30   # bytes a staging store may take (larger first fills wait for the counts instead)
+_STAGING: dict = {}        # (device, stream) -> _Staging: one per stream, rebuilt when the shape changes
+_MAILBOX: dict = {}        # device -> (page-locked int32 tensor, event): where the level counts arrive
+
+
+class _Staging:
+    """A store whose every segment has room for all T tokens of a call at every level: it can be filled before the
+    level counts are known.  The first fill of a store quantises into it while the host still waits for the counts
+    and lays out the store proper; odmkv_store_gather then moves the tiles that hold tokens."""
+
+    def __init__(self, dev, B: int, H: int, T: int, exact_dtype: torch.dtype):
+        nseg = B * H
+        self.key = (B, H, T, exact_dtype)
+        per_seg = (T + TILE - 1) // TILE
+        self.seg_tile = np.tile(np.arange(nseg + 1, dtype=np.int64) * per_seg, (5, 1))
+        plan, self.tables_end, self.counts_end, _, _, total = TurboQuantAdaptiveKVCacheState._plan(self.seg_tile, nseg, exact_dtype)
+        self.bufs = _Buffers(torch.empty(total, dtype=torch.uint8, device=dev), plan)
+        self.packed = TurboQuantAdaptiveKVCacheState._struct_of(self.bufs, self.seg_tile, B, H, exact_dtype)
+        self._tables = np.ascontiguousarray(self.seg_tile, dtype=np.int32)
+        self._offs = np.array([plan[("seg_tile", li)][0] for li in range(5)], np.uint32)
+        self._nseg = nseg
+
+    @staticmethod
+    def bytes_needed(nseg: int, T: int) -> int:
+        tiles = nseg * ((T + TILE - 1) // TILE)
+        return tiles * (sum(2 * TILE * 16 * w + 2 * TILE * 4 for w in WIDTHS) + 2 * TILE * HEAD_DIM * 2 + 5 * TILE * 4)
+
+    def reset(self, stream: int) -> None:
+        """Tables in place, segment counts zero; everything else is written before it is read."""
+        _lib.check(lib.odmkv_store_init(self.bufs.arena.data_ptr(), self._tables.ctypes.data, 5, self._nseg + 1,
+                                        self._offs.ctypes.data, self.tables_end, self.counts_end, self.counts_end, stream))
+
+
+def _staging_for(dev, stream: int, B: int, H: int, T: int, exact_dtype: torch.dtype) -> "_Staging":
+    got = _STAGING.get((str(dev), stream))
+    if got is None or got.key != (B, H, T, exact_dtype):
+        _STAGING.pop((str(dev), stream), None)          # the old one is released before the new one is requested
+        got = _STAGING[(str(dev), stream)] = _Staging(dev, B, H, T, exact_dtype)
+    return got
+
+
+def _mailbox(dev, numel: int):
+    got = _MAILBOX.get(str(dev))
+    if got is None or got[0].numel() < numel:
+        got = _MAILBOX[str(dev)] = (torch.zeros(max(numel, 4096), dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+    return got
 
 
 def _empty_positions(device) -> torch.Tensor:
@@ -171,12 +217,11 @@ class TurboQuantAdaptiveKVCacheState:
             self._level_store = grown
         self._level_store[:, :, self.seq_len:need] = lm
 
-    def _alloc(self, seg_tile: np.ndarray) -> "_Buffers":
-        """All buffers of the store as views into one allocation: the segment tables (one upload),
-        the counters, norms and exact rows (zeroed), the positions (-1), then the codes (left as they
-        come: every code the kernels read is written first or is a padding lane masked by count)."""
-        dev = self.device
-        nseg = self._nseg
+    @staticmethod
+    def _plan(seg_tile: np.ndarray, nseg: int, exact_dtype: torch.dtype):
+        """Byte offsets of all buffers of a store inside one allocation: the segment tables, the counters, norms and
+        exact rows (to be cleared), the positions (to be set to -1), then the codes.
+        -> (plan, end of the tables, end of the counters, end of the cleared part, end of the positions, total)."""
         n_tiles = [max(int(t), 1) for t in seg_tile[:, -1]]
         plan, off = {}, 0
 
@@ -190,12 +235,13 @@ class TurboQuantAdaptiveKVCacheState:
         tables_end = off
         for li in range(5):
             take("seg_count", li, nseg * 4, torch.int32)
+        counts_end = off
         for li in range(4):
             take("knorm", li, n_tiles[li] * TILE * 4, torch.float32)
             take("vnorm", li, n_tiles[li] * TILE * 4, torch.float32)
         # exact rows take part in the products as they are (a zero weight does not silence a NaN)
-        take("kexact", None, n_tiles[4] * TILE * HEAD_DIM * 2, self._exact_torch_dtype)
-        take("vexact", None, n_tiles[4] * TILE * HEAD_DIM * 2, self._exact_torch_dtype)
+        take("kexact", None, n_tiles[4] * TILE * HEAD_DIM * 2, exact_dtype)
+        take("vexact", None, n_tiles[4] * TILE * HEAD_DIM * 2, exact_dtype)
         zero_end = off
         for li in range(5):
             take("pos", li, n_tiles[li] * TILE * 4, torch.int32)
@@ -204,6 +250,15 @@ class TurboQuantAdaptiveKVCacheState:
             w = WIDTHS[li]
             take("kcodes", li, n_tiles[li] * TILE * 16 * w, torch.uint8)
             take("vcodes", li, n_tiles[li] * HEAD_DIM * 8 * w, torch.uint8)
+        return plan, tables_end, counts_end, zero_end, pos_end, off
+
+    def _alloc(self, seg_tile: np.ndarray) -> "_Buffers":
+        """All buffers of the store as views into one allocation: the segment tables (one upload),
+        the counters, norms and exact rows (zeroed), the positions (-1), then the codes (left as they
+        come: every code the kernels read is written first or is a padding lane masked by count)."""
+        dev = self.device
+        nseg = self._nseg
+        plan, tables_end, _, zero_end, pos_end, off = self._plan(seg_tile, nseg, self._exact_torch_dtype)
 
         arena = getattr(self, "_arena", None)
         if arena is None or arena.numel() < off or arena.device != dev:
@@ -224,12 +279,15 @@ class TurboQuantAdaptiveKVCacheState:
         return _Buffers(arena, plan)
 
     def _make_struct(self) -> None:
+        self._packed = self._struct_of(self._bufs, self._seg_tile, self.batch_size, self.num_heads, self._exact_torch_dtype)
+
+    @staticmethod
+    def _struct_of(b: "_Buffers", seg_tile: np.ndarray, B: int, H: int, exact_dtype: torch.dtype) -> Packed:
         p = Packed()
-        p.B, p.Hkv = self.batch_size, self.num_heads
-        p.exact_dtype = _lib.BF16 if self._exact_torch_dtype == torch.bfloat16 else _lib.F16
-        b = self._bufs
+        p.B, p.Hkv = B, H
+        p.exact_dtype = _lib.BF16 if exact_dtype == torch.bfloat16 else _lib.F16
         for li in range(5):
-            p.n_tiles[li] = int(self._seg_tile[li, -1])
+            p.n_tiles[li] = int(seg_tile[li, -1])
             p.pos[li] = b.ptr("pos", li)
             p.seg_tile[li] = b.ptr("seg_tile", li)
             p.seg_count[li] = b.ptr("seg_count", li)
@@ -240,7 +298,7 @@ class TurboQuantAdaptiveKVCacheState:
                 p.vnorm[li] = b.ptr("vnorm", li)
         p.kexact = b.ptr("kexact", None)
         p.vexact = b.ptr("vexact", None)
-        self._packed = p
+        return p
 
     def _capacity_tiles(self, counts: np.ndarray) -> np.ndarray:
         """Tiles per (level, segment) for `counts` tokens; exact segments get room to grow."""
@@ -338,8 +396,34 @@ class TurboQuantAdaptiveKVCacheState:
         st = _lib.stream_ptr(dev)
         fresh = self._bufs is None and getattr(self, "_arena", None) is None       # the store's first tokens
         hint_key = (str(dev), self._nseg, T)
+        pos_offset = self.seq_len if _pos_offset is None else int(_pos_offset)
+        ws_bytes = lib.odmkv_pack_workspace_bytes(B, H, T)
+        # The first fill of a store does not wait for the level counts: the tokens are quantised into a staging store
+        # laid out for the worst case while the counts travel and the host lays the store out; the tiles are moved after.
+        staged = (self._bufs is None and _known_counts is None and _pos_offset is None and T >= 4 * TILE
+                  and _Staging.bytes_needed(self._nseg, T) <= _STAGING_LIMIT)
+        stg = None
         if _known_counts is not None:
             counts = np.asarray(_known_counts, np.int64).reshape(self._nseg, 6)
+        elif staged:
+            counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
+            _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
+            box, arrived = _mailbox(dev, self._nseg * 6)
+            arrived.synchronize()                                     # (the last reader of the box is long done)
+            box[:self._nseg * 6].copy_(counts_dev.view(-1), non_blocking=True)
+            arrived.record(torch.cuda.current_stream(dev))
+            stg = _staging_for(dev, st, B, H, T, self._exact_torch_dtype)
+            stg.reset(st)
+            ws = _lib.workspace(dev, ws_bytes, "pack")
+            _lib.check(lib.odmkv_quant_pack(
+                keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys), B, H, T,
+                keys.stride(0), keys.stride(1), keys.stride(2), bits.data_ptr(), pos_offset,
+                self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
+                C.byref(stg.packed), ws.data_ptr(), ws_bytes, st))
+            if fresh and hint_key in _ARENA_HINT:
+                self._arena = torch.empty(_ARENA_HINT[hint_key], dtype=torch.uint8, device=dev)
+            arrived.synchronize()                                     # the one wait: for the counts alone
+            counts = box[:self._nseg * 6].numpy().reshape(self._nseg, 6).astype(np.int64)
         else:
             counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
             _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
@@ -359,14 +443,15 @@ class TurboQuantAdaptiveKVCacheState:
         self._ensure_capacity(new_counts)
         if fresh:
             _ARENA_HINT[hint_key] = self._arena.numel()
-        pos_offset = self.seq_len if _pos_offset is None else int(_pos_offset)
-        ws_bytes = lib.odmkv_pack_workspace_bytes(B, H, T)
-        ws = _lib.workspace(dev, ws_bytes, "pack")
-        _lib.check(lib.odmkv_quant_pack(
-            keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys), B, H, T,
-            keys.stride(0), keys.stride(1), keys.stride(2), bits.data_ptr(), pos_offset,
-            self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
-            C.byref(self._packed), ws.data_ptr(), ws_bytes, st))
+        if stg is not None:
+            _lib.check(lib.odmkv_store_gather(C.byref(stg.packed), C.byref(self._packed), st))
+        else:
+            ws = _lib.workspace(dev, ws_bytes, "pack")
+            _lib.check(lib.odmkv_quant_pack(
+                keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys), B, H, T,
+                keys.stride(0), keys.stride(1), keys.stride(2), bits.data_ptr(), pos_offset,
+                self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
+                C.byref(self._packed), ws.data_ptr(), ws_bytes, st))
         self._counts = new_counts
         self._exact_room = None
         lm = bits.to(torch.uint8)
