@@ -29,6 +29,13 @@ import statistics
 import sys
 import time
 
+# The CPU generator of the synthetic layers runs on all cores right before every timed compression.  Worker threads
+# that spin after a parallel region would share the cores with the one thread that launches the kernels; let them
+# sleep instead (the thread count is left as it is).  Must be set before the OpenMP runtimes are loaded.
+os.environ.setdefault("OMP_WAIT_POLICY", "passive")
+os.environ.setdefault("KMP_BLOCKTIME", "0")
+os.environ.setdefault("GOMP_SPINCOUNT", "0")
+
 ROOT = os.path.dirname(os.path.abspath(__file__))
 for p in (ROOT, os.path.join(ROOT, "odm-kv_amd")):
     if p not in sys.path:
