@@ -238,12 +238,16 @@ __device__ static inline bool launch_evaluates(const RowState& st, int L) {
 __device__ static void carry_state(const AllocArgs& a, int row, int L, RowState* out, RowState* cur, unsigned int* tot) {
     const int tid = threadIdx.x;
     const RowState* in = a.state + (size_t)((L - 1) & 1) * a.rows + row;
+    // a thread's first partial sum is asked for together with the state (it is discarded if that launch did not evaluate)
+    const unsigned int* p = a.partial + ((size_t)((L - 1) & 1) * a.rows + row) * a.n_chunks * SLOTS;
+    const int n_part = a.n_chunks * SLOTS;
+    const unsigned int v0 = tid < n_part ? p[tid] : 0u;
     if (tid < SLOTS) tot[tid] = 0u;
     __syncthreads();
     const bool evaluated = launch_evaluates(*in, L - 1);
     if (evaluated) {
-        const unsigned int* p = a.partial + ((size_t)((L - 1) & 1) * a.rows + row) * a.n_chunks * SLOTS;
-        for (int idx = tid; idx < a.n_chunks * SLOTS; idx += blockDim.x) {
+        if (v0) atomicAdd(&tot[tid & (SLOTS - 1)], v0);
+        for (int idx = tid + blockDim.x; idx < n_part; idx += blockDim.x) {
             const unsigned int v = p[idx];
             if (v) atomicAdd(&tot[idx & (SLOTS - 1)], v);
         }
