@@ -172,6 +172,17 @@ typedef struct odmkv_packed {
  * (The per-level mask / nonzero of tq_adaptive_backend.py:355-361.) */
 int odmkv_level_counts(const int32_t* bits, int B, int Hkv, int T, int32_t* counts, void* stream);
 
+/* Host arithmetic for callers that keep a store in ONE device allocation: where its 33 buffers lie, given the
+ * segments' first tiles (seg_tile: host int32 [5][nseg + 1], the last entry of a row = tiles of the level).
+ * Order: seg_tile[5], seg_count[5], (knorm, vnorm)[4], kexact, vexact, pos[5], (kcodes, vcodes)[4]; offsets and
+ * sizes in bytes (host uint64 [33] each), every buffer on a multiple of 256; marks (host uint64 [5]): end of the
+ * tables, of the counts, of what odmkv_store_init clears, of the positions, and the bytes in all.
+ * odmkv_store_bind fills the descriptor over such an allocation.  (The reference keeps a Python object per
+ * bank with a tensor per field: kvquant/tq_adaptive_backend.py:31-44, 75-98.) */
+int odmkv_store_layout(const int32_t* seg_tile, int nseg, uint64_t* offsets, uint64_t* sizes, uint64_t* marks);
+int odmkv_store_bind(void* arena, const uint64_t* offsets, const int32_t* seg_tile, int nseg, int B, int Hkv,
+                     int exact_dtype, odmkv_packed_t* out);
+
 /* Prepare a store's buffers, laid out by the caller inside one device allocation `arena` (16-byte
  * aligned), in one launch: the five seg_tile tables (tables_host: host int32 [5][words_per_table], table
  * li written at byte table_offsets[li] of the arena), bytes [zero_begin, zero_end) cleared (segment
@@ -179,7 +190,7 @@ int odmkv_level_counts(const int32_t* bits, int B, int Hkv, int T, int32_t* coun
  * are multiples of 16.  It stands for the empty banks the reference starts from (ExactBank / QuantizedBank
  * __post_init__, kvquant/tq_adaptive_backend.py:39-40, 97-98), for the packed layout. */
 int odmkv_store_init(void* arena, const int32_t* tables_host, int n_tables, int words_per_table,
-                     const uint32_t* table_offsets, uint64_t zero_begin, uint64_t zero_end, uint64_t fill_end,
+                     const uint64_t* table_offsets, uint64_t zero_begin, uint64_t zero_end, uint64_t fill_end,
                      void* stream);
 
 /* Move what a staging store holds into `store`: for every level and segment the tiles that hold tokens

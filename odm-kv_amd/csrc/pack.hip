@@ -87,6 +87,63 @@ extern "C" int odmkv_level_counts(const int32_t* bits, int B, int Hkv, int T, in
 }
 
 // ------------------------------------------------------------------------------------------------
+// where a store's buffers lie inside one allocation (host arithmetic only), and the descriptor over them.
+// Order of the 33 buffers: seg_tile[5], seg_count[5], (knorm, vnorm)[4], kexact, vexact, pos[5], (kcodes, vcodes)[4];
+// every buffer starts on a multiple of 256 bytes.  What is cleared lies between marks[0] and marks[2], the
+// positions end at marks[3].
+// ------------------------------------------------------------------------------------------------
+#define SL_BUFFERS 33
+
+extern "C" int odmkv_store_layout(const int32_t* seg_tile, int nseg, uint64_t* offsets, uint64_t* sizes, uint64_t* marks) {
+    ODMKV_CHECK_ARG(seg_tile && offsets && sizes && marks && nseg > 0, "store_layout: bad arguments");
+    uint64_t nt[5];
+    for (int li = 0; li < 5; ++li) {
+        const int32_t last = seg_tile[(size_t)li * (nseg + 1) + nseg];
+        ODMKV_CHECK_ARG(last >= 0, "store_layout: negative tile count");
+        nt[li] = last > 0 ? (uint64_t)last : 1;                 // an unused level keeps one tile of room: no null pointers
+    }
+    uint64_t off = 0;
+    int n = 0;
+    auto take = [&](uint64_t bytes) { offsets[n] = off; sizes[n] = bytes; ++n; off += align_up(bytes, 256); };
+    for (int li = 0; li < 5; ++li) take((uint64_t)(nseg + 1) * 4);
+    marks[0] = off;                                              // end of the tables
+    for (int li = 0; li < 5; ++li) take((uint64_t)nseg * 4);
+    marks[1] = off;                                              // end of the segment counts
+    for (int li = 0; li < 4; ++li) { take(nt[li] * TILE * 4); take(nt[li] * TILE * 4); }
+    take(nt[4] * TILE * HD * 2);
+    take(nt[4] * TILE * HD * 2);
+    marks[2] = off;                                              // end of what is cleared
+    for (int li = 0; li < 5; ++li) take(nt[li] * TILE * 4);
+    marks[3] = off;                                              // end of the positions
+    for (int li = 0; li < 4; ++li) { take(nt[li] * TILE * 16 * width_of(li)); take(nt[li] * TILE * 16 * width_of(li)); }
+    marks[4] = off;                                              // bytes in all
+    return 0;
+}
+
+extern "C" int odmkv_store_bind(void* arena, const uint64_t* offsets, const int32_t* seg_tile, int nseg, int B, int Hkv,
+                                int exact_dtype, odmkv_packed_t* out) {
+    ODMKV_CHECK_ARG(arena && offsets && seg_tile && out && nseg == B * Hkv && nseg > 0, "store_bind: bad arguments");
+    ODMKV_CHECK_ARG(exact_dtype == ODMKV_F16 || exact_dtype == ODMKV_BF16, "store_bind: exact dtype must be fp16 or bf16");
+    uint8_t* base = (uint8_t*)arena;
+    out->B = B; out->Hkv = Hkv; out->exact_dtype = exact_dtype;
+    for (int li = 0; li < 5; ++li) {
+        out->n_tiles[li] = seg_tile[(size_t)li * (nseg + 1) + nseg];
+        out->seg_tile[li] = (int32_t*)(base + offsets[li]);
+        out->seg_count[li] = (int32_t*)(base + offsets[5 + li]);
+        out->pos[li] = (int32_t*)(base + offsets[20 + li]);
+        if (li < 4) {
+            out->knorm[li] = (float*)(base + offsets[10 + 2 * li]);
+            out->vnorm[li] = (float*)(base + offsets[11 + 2 * li]);
+            out->kcodes[li] = base + offsets[25 + 2 * li];
+            out->vcodes[li] = base + offsets[26 + 2 * li];
+        }
+    }
+    out->kexact = (uint16_t*)(base + offsets[18]);
+    out->vexact = (uint16_t*)(base + offsets[19]);
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
 // a store's buffers before their first use: segment tables written, counters / norms / exact rows
 // cleared, positions set to -1: one launch
 // ------------------------------------------------------------------------------------------------
@@ -115,7 +172,7 @@ __global__ __launch_bounds__(256) void store_init_kernel(StoreInitArgs a) {
 }
 
 extern "C" int odmkv_store_init(void* arena, const int32_t* tables_host, int n_tables, int words_per_table,
-                                const uint32_t* table_offsets, uint64_t zero_begin, uint64_t zero_end, uint64_t fill_end,
+                                const uint64_t* table_offsets, uint64_t zero_begin, uint64_t zero_end, uint64_t fill_end,
                                 void* stream) {
     ODMKV_CHECK_ARG(arena && tables_host && table_offsets, "store_init: null pointer");
     ODMKV_CHECK_ARG(n_tables == 5 && words_per_table > 0, "store_init: five tables expected");
@@ -125,7 +182,10 @@ extern "C" int odmkv_store_init(void* arena, const int32_t* tables_host, int n_t
     StoreInitArgs a;
     a.arena = (uint8_t*)arena; a.zero_begin = zero_begin; a.zero_end = zero_end; a.fill_end = fill_end;
     a.words_per_table = words_per_table;
-    for (int li = 0; li < 5; ++li) a.table_off[li] = table_offsets[li];
+    for (int li = 0; li < 5; ++li) {
+        ODMKV_CHECK_ARG(table_offsets[li] < (1ull << 32), "store_init: the tables must lie in the first 4 GiB of the allocation");
+        a.table_off[li] = (unsigned int)table_offsets[li];
+    }
     const int n_words = 5 * words_per_table;
     if (n_words <= SI_MAX_TABLE) {
         a.n_words = n_words;

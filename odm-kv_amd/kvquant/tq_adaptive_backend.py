@@ -58,23 +58,57 @@ _TILE_COST = [300, 420, 450, 890, 1310]
 _ITEM_FIXED_US = 4.0
 
 
+_U64x33 = C.c_uint64 * 33
+_U64x5 = C.c_uint64 * 5
+# index of a buffer in the layout of odmkv_store_layout: name -> (first index, step per level)
+_SLOT = {"seg_tile": (0, 1), "seg_count": (5, 1), "knorm": (10, 2), "vnorm": (11, 2), "kexact": (18, 0), "vexact": (19, 0),
+         "pos": (20, 1), "kcodes": (25, 2), "vcodes": (26, 2)}
+
+
+class _Layout:
+    """Where the buffers of a store lie inside one allocation (odmkv_store_layout) for given segment tables."""
+
+    def __init__(self, seg_tile: np.ndarray, nseg: int):
+        self.tables = np.ascontiguousarray(seg_tile, dtype=np.int32)     # [5, nseg + 1]
+        self.tables_ptr = self.tables.ctypes.data
+        self.nseg = nseg
+        self.offsets, self.sizes, marks = _U64x33(), _U64x33(), _U64x5()
+        _lib.check(lib.odmkv_store_layout(self.tables_ptr, nseg, self.offsets, self.sizes, marks))
+        self.tables_end, self.counts_end, self.zero_end, self.pos_end, self.total = (int(m) for m in marks)
+
+    def init(self, arena: torch.Tensor, stream: int, counts_only: bool = False) -> None:
+        """Tables written, counters / norms / exact rows cleared, positions -1 (counts_only: just the tables and
+        the segment counts): one launch, the tables in its arguments."""
+        zero_end = self.counts_end if counts_only else self.zero_end
+        fill_end = self.counts_end if counts_only else self.pos_end
+        _lib.check(lib.odmkv_store_init(arena.data_ptr(), self.tables_ptr, 5, self.nseg + 1, C.addressof(self.offsets),
+                                        self.tables_end, zero_end, fill_end, stream))
+
+    def struct(self, arena: torch.Tensor, B: int, H: int, exact_dtype: torch.dtype) -> Packed:
+        p = Packed()
+        _lib.check(lib.odmkv_store_bind(arena.data_ptr(), self.offsets, self.tables_ptr, self.nseg, B, H,
+                                        _lib.BF16 if exact_dtype == torch.bfloat16 else _lib.F16, C.byref(p)))
+        return p
+
+
 class _Buffers:
     """The store's buffers inside one allocation; tensor views are made when somebody asks."""
 
-    def __init__(self, arena: torch.Tensor, plan: dict):
+    def __init__(self, arena: torch.Tensor, layout: _Layout, exact_dtype: torch.dtype):
         self.arena = arena
-        self.plan = plan
-        self._base = arena.data_ptr()
-
-    def ptr(self, name: str, li) -> int:
-        return self._base + self.plan[(name, li)][0]
+        self.layout = layout
+        self._exact_dtype = exact_dtype
 
     def view(self, name: str, li=None) -> torch.Tensor:
-        off, nbytes, dtype = self.plan[(name, li)]
+        first, step = _SLOT[name]
+        i = first + step * (li or 0)
+        off, nbytes = int(self.layout.offsets[i]), int(self.layout.sizes[i])
+        dtype = (torch.int32 if name in ("seg_tile", "seg_count", "pos") else torch.float32 if name in ("knorm", "vnorm")
+                 else self._exact_dtype if name in ("kexact", "vexact") else torch.uint8)
         return self.arena[off:off + nbytes].view(dtype)
 
     def __getitem__(self, name: str):
-        if (name, None) in self.plan:
+        if name in ("kexact", "vexact"):
             return self.view(name)
         n = 5 if name in ("pos", "seg_tile", "seg_count") else 4
         return [self.view(name, li) for li in range(n)]
@@ -96,12 +130,9 @@ class _Staging:
         self.key = (B, H, T, exact_dtype)
         per_seg = (T + TILE - 1) // TILE
         self.seg_tile = np.tile(np.arange(nseg + 1, dtype=np.int64) * per_seg, (5, 1))
-        plan, self.tables_end, self.counts_end, _, _, total = TurboQuantAdaptiveKVCacheState._plan(self.seg_tile, nseg, exact_dtype)
-        self.bufs = _Buffers(torch.empty(total, dtype=torch.uint8, device=dev), plan)
-        self.packed = TurboQuantAdaptiveKVCacheState._struct_of(self.bufs, self.seg_tile, B, H, exact_dtype)
-        self._tables = np.ascontiguousarray(self.seg_tile, dtype=np.int32)
-        self._offs = np.array([plan[("seg_tile", li)][0] for li in range(5)], np.uint32)
-        self._nseg = nseg
+        self.layout = _Layout(self.seg_tile, nseg)
+        self.bufs = _Buffers(torch.empty(self.layout.total, dtype=torch.uint8, device=dev), self.layout, exact_dtype)
+        self.packed = self.layout.struct(self.bufs.arena, B, H, exact_dtype)
 
     @staticmethod
     def bytes_needed(nseg: int, T: int) -> int:
@@ -110,8 +141,7 @@ class _Staging:
 
     def reset(self, stream: int) -> None:
         """Tables in place, segment counts zero; everything else is written before it is read."""
-        _lib.check(lib.odmkv_store_init(self.bufs.arena.data_ptr(), self._tables.ctypes.data, 5, self._nseg + 1,
-                                        self._offs.ctypes.data, self.tables_end, self.counts_end, self.counts_end, stream))
+        self.layout.init(self.bufs.arena, stream, counts_only=True)
 
 
 def _staging_for(dev, stream: int, B: int, H: int, T: int, exact_dtype: torch.dtype) -> "_Staging":
@@ -217,49 +247,14 @@ class TurboQuantAdaptiveKVCacheState:
             self._level_store = grown
         self._level_store[:, :, self.seq_len:need] = lm
 
-    @staticmethod
-    def _plan(seg_tile: np.ndarray, nseg: int, exact_dtype: torch.dtype):
-        """Byte offsets of all buffers of a store inside one allocation: the segment tables, the counters, norms and
-        exact rows (to be cleared), the positions (to be set to -1), then the codes.
-        -> (plan, end of the tables, end of the counters, end of the cleared part, end of the positions, total)."""
-        n_tiles = [max(int(t), 1) for t in seg_tile[:, -1]]
-        plan, off = {}, 0
-
-        def take(name, li, nbytes, dtype):
-            nonlocal off
-            plan[(name, li)] = (off, nbytes, dtype)
-            off += (nbytes + 255) // 256 * 256
-
-        for li in range(5):
-            take("seg_tile", li, (nseg + 1) * 4, torch.int32)
-        tables_end = off
-        for li in range(5):
-            take("seg_count", li, nseg * 4, torch.int32)
-        counts_end = off
-        for li in range(4):
-            take("knorm", li, n_tiles[li] * TILE * 4, torch.float32)
-            take("vnorm", li, n_tiles[li] * TILE * 4, torch.float32)
-        # exact rows take part in the products as they are (a zero weight does not silence a NaN)
-        take("kexact", None, n_tiles[4] * TILE * HEAD_DIM * 2, exact_dtype)
-        take("vexact", None, n_tiles[4] * TILE * HEAD_DIM * 2, exact_dtype)
-        zero_end = off
-        for li in range(5):
-            take("pos", li, n_tiles[li] * TILE * 4, torch.int32)
-        pos_end = off
-        for li in range(4):
-            w = WIDTHS[li]
-            take("kcodes", li, n_tiles[li] * TILE * 16 * w, torch.uint8)
-            take("vcodes", li, n_tiles[li] * HEAD_DIM * 8 * w, torch.uint8)
-        return plan, tables_end, counts_end, zero_end, pos_end, off
-
     def _alloc(self, seg_tile: np.ndarray) -> "_Buffers":
-        """All buffers of the store as views into one allocation: the segment tables (one upload),
-        the counters, norms and exact rows (zeroed), the positions (-1), then the codes (left as they
-        come: every code the kernels read is written first or is a padding lane masked by count)."""
+        """All buffers of the store as views into one allocation: the segment tables, the counters, norms and
+        exact rows (zeroed; exact rows take part in the products as they are: a zero weight does not silence a
+        NaN), the positions (-1), then the codes (left as they come: every code the kernels read is written
+        first or is a padding lane masked by count)."""
         dev = self.device
-        nseg = self._nseg
-        plan, tables_end, _, zero_end, pos_end, off = self._plan(seg_tile, nseg, self._exact_torch_dtype)
-
+        layout = _Layout(seg_tile, self._nseg)
+        off = layout.total
         arena = getattr(self, "_arena", None)
         if arena is None or arena.numel() < off or arena.device != dev:
             arena = torch.empty(off + off // 8, dtype=torch.uint8, device=dev)
@@ -271,34 +266,11 @@ class TurboQuantAdaptiveKVCacheState:
                 spare = torch.empty(off + off // 8, dtype=torch.uint8, device=dev)
             arena, self._arena_spare = spare, arena
         self._arena = arena
-        # tables written, counters / norms / exact rows cleared, positions -1: one launch, the tables in its arguments
-        tables = np.ascontiguousarray(seg_tile, dtype=np.int32)
-        offs = np.array([plan[("seg_tile", li)][0] for li in range(5)], np.uint32)
-        _lib.check(lib.odmkv_store_init(arena.data_ptr(), tables.ctypes.data, 5, nseg + 1, offs.ctypes.data,
-                                        tables_end, zero_end, pos_end, _lib.stream_ptr(dev)))
-        return _Buffers(arena, plan)
+        layout.init(arena, _lib.stream_ptr(dev))
+        return _Buffers(arena, layout, self._exact_torch_dtype)
 
     def _make_struct(self) -> None:
-        self._packed = self._struct_of(self._bufs, self._seg_tile, self.batch_size, self.num_heads, self._exact_torch_dtype)
-
-    @staticmethod
-    def _struct_of(b: "_Buffers", seg_tile: np.ndarray, B: int, H: int, exact_dtype: torch.dtype) -> Packed:
-        p = Packed()
-        p.B, p.Hkv = B, H
-        p.exact_dtype = _lib.BF16 if exact_dtype == torch.bfloat16 else _lib.F16
-        for li in range(5):
-            p.n_tiles[li] = int(seg_tile[li, -1])
-            p.pos[li] = b.ptr("pos", li)
-            p.seg_tile[li] = b.ptr("seg_tile", li)
-            p.seg_count[li] = b.ptr("seg_count", li)
-            if li < 4:
-                p.kcodes[li] = b.ptr("kcodes", li)
-                p.vcodes[li] = b.ptr("vcodes", li)
-                p.knorm[li] = b.ptr("knorm", li)
-                p.vnorm[li] = b.ptr("vnorm", li)
-        p.kexact = b.ptr("kexact", None)
-        p.vexact = b.ptr("vexact", None)
-        return p
+        self._packed = self._bufs.layout.struct(self._bufs.arena, self.batch_size, self.num_heads, self._exact_torch_dtype)
 
     def _capacity_tiles(self, counts: np.ndarray) -> np.ndarray:
         """Tiles per (level, segment) for `counts` tokens; exact segments get room to grow."""
