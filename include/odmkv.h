@@ -201,6 +201,20 @@ int odmkv_store_init(void* arena, const int32_t* tables_host, int n_tables, int 
  * banks grow by torch.cat (kvquant/tq_adaptive_backend.py:46-52, 149-174). */
 int odmkv_store_gather(const odmkv_packed_t* staging, const odmkv_packed_t* store, void* stream);
 
+/* The part of a store's first fill that does not depend on the level counts, in one call: odmkv_level_counts into
+ * counts_dev, an asynchronous copy of the counts to counts_host (page-locked host memory, int32 [B*Hkv, 6]) with
+ * counts_event (a hipEvent_t) recorded behind it, the staging store emptied (its tables as odmkv_store_layout gave
+ * them: staging_tables_host, staging_offsets, tables_end, counts_end) and odmkv_quant_pack into it.  The caller
+ * waits for the event alone, lays out the store proper and calls odmkv_store_gather.  No counterpart in the reference. */
+int odmkv_quant_pack_staged(const void* K, const void* V, int dtype, int B, int Hkv, int T,
+                            int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                            const int32_t* bits, int pos_offset,
+                            const float* pi_k, const float* pi_v, const float* codebooks,
+                            const odmkv_packed_t* staging, void* staging_arena, const int32_t* staging_tables_host,
+                            const uint64_t* staging_offsets, uint64_t tables_end, uint64_t counts_end,
+                            int32_t* counts_dev, int32_t* counts_host, void* counts_event,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 /* Quantise and pack T new tokens per (b, h) into a store whose seg_tile tables are filled in
  * and whose seg_count hold the tokens already present (0 after a reset); new tokens are
  * appended behind them and seg_count is advanced.  K, V: [B, Hkv, T, 128] of `dtype` with

@@ -1653,6 +1653,27 @@ extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, 
     return 0;
 }
 
+// The first fill of a store, everything that does not depend on the level counts in one call: count the levels, send the
+// counts to the host (page-locked memory, an event behind the copy), empty the staging store and quantise into it.
+extern "C" int odmkv_quant_pack_staged(const void* K, const void* V, int dtype, int B, int Hkv, int T,
+                                       int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                                       const int32_t* bits, int pos_offset,
+                                       const float* pi_k, const float* pi_v, const float* codebooks,
+                                       const odmkv_packed_t* staging, void* staging_arena, const int32_t* staging_tables_host,
+                                       const uint64_t* staging_offsets, uint64_t tables_end, uint64_t counts_end,
+                                       int32_t* counts_dev, int32_t* counts_host, void* counts_event,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+    ODMKV_CHECK_ARG(staging && staging_arena && staging_tables_host && staging_offsets && counts_dev && counts_host && counts_event,
+                    "quant_pack_staged: null pointer");
+    if (int rc = odmkv_level_counts(bits, B, Hkv, T, counts_dev, stream)) return rc;
+    ODMKV_CHECK_HIP(hipMemcpyAsync(counts_host, counts_dev, (size_t)B * Hkv * 6 * sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    ODMKV_CHECK_HIP(hipEventRecord((hipEvent_t)counts_event, (hipStream_t)stream));
+    if (int rc = odmkv_store_init(staging_arena, staging_tables_host, 5, B * Hkv + 1, staging_offsets, tables_end, counts_end, counts_end, stream))
+        return rc;
+    return odmkv_quant_pack(K, V, dtype, B, Hkv, T, stride_b, stride_h, stride_t, bits, pos_offset, pi_k, pi_v, codebooks,
+                            staging, workspace, workspace_bytes, stream);
+}
+
 // ------------------------------------------------------------------------------------------------
 // the tiles of a staging store (every segment laid out for the worst case, so that it can be filled
 // before anybody knows the level counts) moved into a store laid out for the counts

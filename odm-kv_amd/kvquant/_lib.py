@@ -66,6 +66,8 @@ def _load() -> C.CDLL:
         "odmkv_level_counts": (C.c_int, [vp, i32, i32, i32, vp, vp]),
         "odmkv_store_init": (C.c_int, [vp, vp, i32, i32, vp, C.c_uint64, C.c_uint64, C.c_uint64, vp]),
         "odmkv_store_gather": (C.c_int, [C.POINTER(Packed), C.POINTER(Packed), vp]),
+        "odmkv_quant_pack_staged": (C.c_int, [vp, vp, i32, i32, i32, i32, i64, i64, i64, vp, i32, vp, vp, vp,
+                                              C.POINTER(Packed), vp, vp, vp, C.c_uint64, C.c_uint64, vp, vp, vp, vp, sz, vp]),
         "odmkv_store_layout": (C.c_int, [vp, i32, vp, vp, vp]),
         "odmkv_store_bind": (C.c_int, [vp, vp, vp, i32, i32, i32, i32, C.POINTER(Packed)]),
         "odmkv_pack_workspace_bytes": (sz, [i32, i32, i32]),
@@ -96,7 +98,7 @@ lib = _load()
 EXPORTS = ("odmkv_version", "odmkv_last_error", "odmkv_score_workspace_bytes", "odmkv_score", "odmkv_score_model_dtype", "odmkv_score_expected",
            "odmkv_window_attention_workspace_bytes", "odmkv_window_attention",
            "odmkv_allocate_workspace_bytes", "odmkv_allocate", "odmkv_level_counts",
-           "odmkv_store_init", "odmkv_store_gather", "odmkv_store_layout", "odmkv_store_bind", "odmkv_pack_workspace_bytes", "odmkv_quant_pack", "odmkv_quantize_rows",
+           "odmkv_store_init", "odmkv_store_gather", "odmkv_quant_pack_staged", "odmkv_store_layout", "odmkv_store_bind", "odmkv_pack_workspace_bytes", "odmkv_quant_pack", "odmkv_quantize_rows",
            "odmkv_dequantize_rows", "odmkv_dequant", "odmkv_dequant_from", "odmkv_append_exact",
            "odmkv_decode_workspace_bytes", "odmkv_decode_attn", "odmkv_decode_attn_static",
            "odmkv_exact_tail", "odmkv_flush_score", "odmkv_flush_rank")

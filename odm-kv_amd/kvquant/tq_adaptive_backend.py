@@ -153,9 +153,15 @@ def _staging_for(dev, stream: int, B: int, H: int, T: int, exact_dtype: torch.dt
 
 
 def _mailbox(dev, numel: int):
+    """(page-locked int32 tensor, device int32 tensor, event, the event's handle): where the level counts arrive."""
     got = _MAILBOX.get(str(dev))
     if got is None or got[0].numel() < numel:
-        got = _MAILBOX[str(dev)] = (torch.zeros(max(numel, 4096), dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(dev))          # (the handle exists once the event has been recorded)
+        ev.synchronize()
+        n = max(numel, 4096)
+        got = _MAILBOX[str(dev)] = (torch.zeros(n, dtype=torch.int32, pin_memory=True),
+                                    torch.empty(n, dtype=torch.int32, device=dev), ev, int(ev.cuda_event))
     return got
 
 
@@ -378,20 +384,18 @@ class TurboQuantAdaptiveKVCacheState:
         if _known_counts is not None:
             counts = np.asarray(_known_counts, np.int64).reshape(self._nseg, 6)
         elif staged:
-            counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
-            _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
-            box, arrived = _mailbox(dev, self._nseg * 6)
+            box, box_dev, arrived, arrived_handle = _mailbox(dev, self._nseg * 6)
             arrived.synchronize()                                     # (the last reader of the box is long done)
-            box[:self._nseg * 6].copy_(counts_dev.view(-1), non_blocking=True)
-            arrived.record(torch.cuda.current_stream(dev))
             stg = _staging_for(dev, st, B, H, T, self._exact_torch_dtype)
-            stg.reset(st)
             ws = _lib.workspace(dev, ws_bytes, "pack")
-            _lib.check(lib.odmkv_quant_pack(
+            lay = stg.layout
+            _lib.check(lib.odmkv_quant_pack_staged(
                 keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys), B, H, T,
                 keys.stride(0), keys.stride(1), keys.stride(2), bits.data_ptr(), pos_offset,
                 self.pi_k.data_ptr(), self.pi_v.data_ptr(), self.codebooks.data_ptr(),
-                C.byref(stg.packed), ws.data_ptr(), ws_bytes, st))
+                C.byref(stg.packed), stg.bufs.arena.data_ptr(), lay.tables_ptr, C.addressof(lay.offsets),
+                lay.tables_end, lay.counts_end, box_dev.data_ptr(), box.data_ptr(), arrived_handle,
+                ws.data_ptr(), ws_bytes, st))
             if fresh and hint_key in _ARENA_HINT:
                 self._arena = torch.empty(_ARENA_HINT[hint_key], dtype=torch.uint8, device=dev)
             arrived.synchronize()                                     # the one wait: for the counts alone
