@@ -118,3 +118,44 @@ def test_product_rotation_is_the_reference_matrix(golden):
     assert (cached_rotation(128, "cpu", 42).numpy() == golden["pi_seed42"]).all()
     # another seed is another matrix; the value rotation of a state is seed + 2000
     assert not (random_rotation(128, "cpu", torch.float32, seed=2042).numpy() == golden["pi_seed42"]).all()
+
+
+def test_store_layout_and_bind_are_host_arithmetic(lib):
+    """odmkv_store_layout / odmkv_store_bind touch no GPU: 33 buffers in the documented order, each on a multiple
+    of 256 bytes and as large as its level's tiles need, the marks between the groups, and a descriptor whose
+    pointers are the allocation's base plus those offsets."""
+    import numpy as np
+    from kvquant._lib import Packed
+    nseg, B, H = 6, 2, 3
+    rng = np.random.default_rng(5)
+    cap = rng.integers(0, 9, size=(5, nseg))
+    cap[1] = 0                                             # a level nobody uses keeps one tile of room
+    seg_tile = np.zeros((5, nseg + 1), np.int32)
+    seg_tile[:, 1:] = np.cumsum(cap, axis=1)
+    off, size, marks = (C.c_uint64 * 33)(), (C.c_uint64 * 33)(), (C.c_uint64 * 5)()
+    lib.odmkv_store_layout.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+    assert lib.odmkv_store_layout(seg_tile.ctypes.data, nseg, off, size, marks) == 0
+    off, size, marks = list(off), list(size), list(marks)
+    nt = [max(int(t), 1) for t in seg_tile[:, -1]]
+    widths = (2, 3, 4, 8)
+    want = ([(nseg + 1) * 4] * 5 + [nseg * 4] * 5 + [nt[li] * 64 * 4 for li in range(4) for _ in (0, 1)]
+            + [nt[4] * 64 * 128 * 2] * 2 + [nt[li] * 64 * 4 for li in range(5)]
+            + [nt[li] * 64 * 16 * widths[li] for li in range(4) for _ in (0, 1)])
+    assert size == want
+    assert off[0] == 0 and all(o % 256 == 0 for o in off)
+    assert all(off[i + 1] == off[i] + -(-size[i] // 256) * 256 for i in range(32))
+    assert marks == [off[5], off[10], off[20], off[25], off[32] + -(-size[32] // 256) * 256]
+    p = Packed()
+    base = 0x7000_0000_0000
+    lib.odmkv_store_bind.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(Packed)]
+    assert lib.odmkv_store_bind(base, (C.c_uint64 * 33)(*off), seg_tile.ctypes.data, nseg, B, H, 0, C.byref(p)) == 0
+    assert (p.B, p.Hkv, p.exact_dtype) == (B, H, 0) and list(p.n_tiles) == [int(t) for t in seg_tile[:, -1]]
+    for li in range(5):
+        assert p.seg_tile[li] == base + off[li] and p.seg_count[li] == base + off[5 + li] and p.pos[li] == base + off[20 + li]
+    for li in range(4):
+        assert (p.knorm[li], p.vnorm[li]) == (base + off[10 + 2 * li], base + off[11 + 2 * li])
+        assert (p.kcodes[li], p.vcodes[li]) == (base + off[25 + 2 * li], base + off[26 + 2 * li])
+    assert (p.kexact, p.vexact) == (base + off[18], base + off[19])
+    lib.odmkv_last_error.restype = C.c_char_p
+    assert lib.odmkv_store_bind(base, (C.c_uint64 * 33)(*off), seg_tile.ctypes.data, nseg, B, H + 1, 0, C.byref(p)) == -1
+    assert b"store_bind" in lib.odmkv_last_error()
