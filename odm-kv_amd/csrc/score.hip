@@ -33,7 +33,6 @@ struct ScoreArgs {
     float* opart;         // [Hkv, nchunks, 128]
     float* psum;          // [Hkv, nchunks]
     float* obar;          // [Hkv, 128]
-    unsigned int* gmax;   // bit pattern of the running maximum score (scores are >= 0)
 };
 
 template <int DT>
@@ -212,11 +211,139 @@ __global__ __launch_bounds__(256) void score_logits_kernel(ScoreArgs a) {
     }
 }
 
-// ---- merge chunk statistics into (max, sum) per query head; also clears the running maximum ----
+// ---- pass 1 over 16-bit K on the matrix cores ----
+// v_mfma_f32_16x16x32_{f16,bf16}: D[16x16] += A[16x32] . B[32x16]; lane (n = lane % 16, j = lane / 16) supplies
+// A[n][8j+e] and B[8j+e][n] and holds D[4j+r][n].  B = 16 tokens x 32 dims of K exactly as they lie in memory (a
+// lane's 16 bytes), A = the mean queries of four heads, head (row % 4) in every row, as 16-bit pieces whose sum
+// is the fp32 value (fp16: high + low of the vector scaled by a power of two into fp16's range; bf16: three
+// pieces).  A wave takes 64 tokens as four groups of 16; after the products lane (j, n) keeps group j's
+// accumulator: the logits of four heads for token 16j + n.  |k|^2 is the diagonal of K_g . K_g^T, the same
+// registers as both operands.  All of a workgroup's rows are requested before anything is computed.
+typedef _Float16 sc_h8 __attribute__((ext_vector_type(8)));
+typedef __bf16 sc_b8 __attribute__((ext_vector_type(8)));
+typedef float sc_f4 __attribute__((ext_vector_type(4)));
+template <int DT>
+__device__ static __forceinline__ sc_f4 sc_mfma(const uint4& a, const uint4& b, const sc_f4& c) {
+    if constexpr (DT == ODMKV_F16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(sc_h8, a), __builtin_bit_cast(sc_h8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sc_b8, a), __builtin_bit_cast(sc_b8, b), c, 0, 0, 0);
+}
+
+template <int DT, int GMAX>
+__global__ __launch_bounds__(256) void score_logits16_kernel(ScoreArgs a) {
+    static_assert(DT == ODMKV_F16 || DT == ODMKV_BF16, "16-bit keys");
+    static_assert(ROWS_PER_WG == 256, "four waves of 64 tokens");
+    constexpr int NP = DT == ODMKV_F16 ? 2 : 3;     // 16-bit pieces of a mean query
+    constexpr int HB = GMAX / 4;                    // blocks of four heads
+    __shared__ uint4 mu_op[HB][4][NP][16];          // [head block][32-dim block][piece][4 j + head % 4]: 8 elements
+    __shared__ float unscale[GMAX];                 // 2^exponent / sqrt(d) per head
+    __shared__ float red_m[4][GMAX], red_s[4][GMAX];
+    const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, n = lane & 15, j = lane >> 4;
+    const int t0 = chunk * ROWS_PER_WG + wave * 64;
+    // the keys: group q's token n, dims 32 i + 8 j .. + 7 (rows past the end repeat the last row, never stored)
+    uint4 kx[4][4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint16_t* row = reinterpret_cast<const uint16_t*>(a.K) + (size_t)h * a.sH
+                              + (size_t)(a.n_sink + min(t0 + 16 * q + n, a.Tc - 1)) * a.sT + 8 * j;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) kx[q][i] = *reinterpret_cast<const uint4*>(row + 32 * i);
+    }
+    // per head: the power of two that brings the largest entry below 1 (fp16 pieces; bf16 has fp32's range)
+    {
+        const int g = tid >> 5, sub = tid & 31;     // 8 heads x 32 threads x 4 dims
+        float mx = 0.0f;
+        if (g < a.Gl) {
+            const float4 v = *reinterpret_cast<const float4*>(a.mu + ((size_t)h * a.G + g) * HD + 4 * sub);
+            mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        }
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, WAVE));
+        if (sub == 0 && g < GMAX) {
+            int ex = 0;
+            if (DT == ODMKV_F16 && mx > 0.0f && mx < INFINITY) { (void)frexpf(mx, &ex); ex = max(-100, min(112, ex)); }
+            unscale[g] = ldexpf(0.08838834764831845f, ex);     // 1 / sqrt(128) times the scale taken out below
+            red_m[0][g] = ldexpf(1.0f, -ex);                   // (borrowed until the barrier after the split)
+        }
+    }
+    __syncthreads();
+    if (tid < HB * 64) {
+        const int hb = tid >> 6, i = (tid >> 4) & 3, jj = (tid >> 2) & 3, g = 4 * hb + (tid & 3);
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = 0.0f;
+        if (g < a.Gl) {
+            const float* src = a.mu + ((size_t)h * a.G + g) * HD + 32 * i + 8 * jj;
+            const float4 v0 = *reinterpret_cast<const float4*>(src), v1 = *reinterpret_cast<const float4*>(src + 4);
+            const float sc = red_m[0][g];
+            x[0] = v0.x * sc; x[1] = v0.y * sc; x[2] = v0.z * sc; x[3] = v0.w * sc;
+            x[4] = v1.x * sc; x[5] = v1.y * sc; x[6] = v1.z * sc; x[7] = v1.w * sc;
+        }
+#pragma unroll
+        for (int pc = 0; pc < NP; ++pc) {
+            uint32_t w[4];
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                const uint16_t b0 = Elem<DT>::from_f32(x[e]), b1 = Elem<DT>::from_f32(x[e + 1]);
+                x[e] -= Elem<DT>::to_f32(b0); x[e + 1] -= Elem<DT>::to_f32(b1);       // exact: what the piece left over
+                w[e >> 1] = (uint32_t)b0 | ((uint32_t)b1 << 16);
+            }
+            mu_op[hb][i][pc][tid & 15] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+    __syncthreads();
+    // |k|^2: lane (n / 4, n) holds the diagonal element of token n in component n % 4
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        sc_f4 gr = (sc_f4){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) gr = sc_mfma<DT>(kx[q][i], kx[q][i], gr);
+        const int r = n & 3, t = t0 + 16 * q + n;
+        const float kn = r == 0 ? gr[0] : r == 1 ? gr[1] : r == 2 ? gr[2] : gr[3];
+        if (j == (n >> 2) && t < a.Tc) a.kn2[(size_t)h * a.Tc + t] = kn;
+    }
+    const int t = t0 + lane;                      // this lane's token: group j, column n
+#pragma unroll
+    for (int hb = 0; hb < HB; ++hb) {
+        if (4 * hb >= a.Gl) break;
+        sc_f4 acc[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q] = (sc_f4){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int pc = NP - 1; pc >= 0; --pc) {           // small pieces first
+                const uint4 mu8 = mu_op[hb][i][pc][4 * j + (n & 3)];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc[q] = sc_mfma<DT>(mu8, kx[q][i], acc[q]);
+            }
+        const sc_f4 mine = j == 0 ? acc[0] : j == 1 ? acc[1] : j == 2 ? acc[2] : acc[3];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int g = 4 * hb + r;
+            if (g < a.Gl) {
+                const float d = t < a.Tc ? mine[r] * unscale[g] : -INFINITY;
+                if (t < a.Tc) a.logits[((size_t)h * a.G + g) * a.Tc + t] = d;
+                const float m = wave_max(d);
+                const float s = wave_sum(d == -INFINITY ? 0.0f : __expf(d - m));
+                if (lane == 0) { red_m[wave][g] = m; red_s[wave][g] = s; }
+            }
+        }
+    }
+    __syncthreads();
+    if (tid < a.Gl) {
+        float mm = red_m[0][tid], ss = red_s[0][tid];
+        for (int w = 1; w < 4; ++w) ms_merge(mm, ss, red_m[w][tid], red_s[w][tid]);
+        float* st = a.stats + (((size_t)h * a.G + tid) * a.nchunks + chunk) * 2;
+        st[0] = mm; st[1] = ss;
+    }
+}
+
+// ---- merge chunk statistics into (max, sum) per query head ----
 __global__ __launch_bounds__(64) void score_stats_kernel(ScoreArgs a) {
     const int hq = blockIdx.x, lane = threadIdx.x;
-    if (hq == 0 && lane == 0) *a.gmax = 0u;
-    if (a.Gl == 0) return;                    // attention weights were supplied: nothing to merge
     float m = -INFINITY, s = 0.0f;
     for (int c = lane; c < a.nstat; c += WAVE) {
         const float* st = a.stats + ((size_t)hq * a.nstat + c) * 2;
@@ -231,81 +358,110 @@ __global__ __launch_bounds__(64) void score_stats_kernel(ScoreArgs a) {
 }
 
 // ---- pass 1 over V: p, sum p, partial sums of p * v ----
+// The two passes over V share one shape: a group of 16 lanes takes 16 consecutive rows (4 KB of a dense cache),
+// lane `part` of the group owns row `part` (it reads and writes that row's scalars: 64 consecutive floats per
+// wave), and all rows of a trip are requested before any is used.  16-bit rows: one trip of 16; fp32: two of 8.
+template <int DT> struct VTrip { static constexpr int ROWS = DT == ODMKV_F32 ? 8 : 16; };
+
+// lane `src` of this lane's group of 16 (a row of the data-parallel-primitive network)
+__device__ static inline float group16_bcast(float v, int src) {
+    return __shfl(v, (int)((threadIdx.x & 48u) | (unsigned)src), WAVE);
+}
+
 template <int DT, int GMAX>
 __global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
+    constexpr int U = VTrip<DT>::ROWS;
     __shared__ float osum[16][HD];
-    __shared__ float psum_s[16];
+    __shared__ float psum_s[4];
+    __shared__ float mz_s[2 * GMAX];
     const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, part = lane & 15, rsub = lane >> 4;
-    float Mg[GMAX], Zg[GMAX];
+    const int wave = tid >> 6, lane = tid & 63, part = lane & 15, grp = tid >> 4;
+    const int tb = chunk * ROWS_PER_WG + grp * 16;
+    Raw8<DT> raw[U];
+    auto request = [&](int u0) {
 #pragma unroll
-    for (int g = 0; g < GMAX; ++g) {
-        Mg[g] = (a.attn == nullptr && g < a.G) ? a.mz[2 * (h * a.G + g)] : 0.0f;
-        Zg[g] = (a.attn == nullptr && g < a.G) ? 1.0f / a.mz[2 * (h * a.G + g) + 1] : 1.0f;   // reciprocal of the sum
+        for (int u = 0; u < U; ++u)
+            load8_raw<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + min(tb + u0 + u, a.Tc - 1)) * a.sT + part * 8, raw[u]);
+    };
+    request(0);
+    const int t = tb + part;                       // the lane's own row
+    float lg[GMAX];
+    if (a.attn == nullptr && t < a.Tc) {
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g)
+            if (g < a.G) lg[g] = a.logits[((size_t)h * a.G + g) * a.Tc + t];
     }
-    const float inv_g = 1.0f / (float)a.G;
+    // (max, sum) of every query head of the group over all chunks: each workgroup merges the chunk statistics
+    // again (a kilobyte per head out of the L2, under the loads above) instead of waiting for a launch that does
+    if (a.attn == nullptr) {
+        for (int g = wave; g < a.G; g += 4) {
+            float m = -INFINITY, sm = 0.0f;
+            for (int c = lane; c < a.nstat; c += WAVE) {
+                const float2 e = *reinterpret_cast<const float2*>(a.stats + ((size_t)(h * a.G + g) * a.nstat + c) * 2);
+                ms_merge(m, sm, e.x, e.y);
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float m2 = __shfl_xor(m, o, WAVE), s2 = __shfl_xor(sm, o, WAVE);
+                ms_merge(m, sm, m2, s2);
+            }
+            if (lane == 0) { mz_s[2 * g] = m; mz_s[2 * g + 1] = 1.0f / sm; }     // reciprocal of the sum
+        }
+        __syncthreads();
+    }
+    // the weight of the lane's own row
+    float pt = 0.0f;
+    if (t < a.Tc) {
+        if (a.attn != nullptr) {
+            pt = a.attn[(size_t)h * a.T + a.n_sink + t];
+        } else {
+            float Mg[GMAX], Zg[GMAX];
+#pragma unroll
+            for (int g = 0; g < GMAX; ++g) {
+                if (g < a.G) { Mg[g] = mz_s[2 * g]; Zg[g] = mz_s[2 * g + 1]; }
+            }
+            const float inv_g = 1.0f / (float)a.G;
+            float acc = 0.0f;
+            if (a.round_dt < 0) {
+#pragma unroll
+                for (int g = 0; g < GMAX; ++g)
+                    if (g < a.G) acc = __fmaf_rn(__expf(lg[g] - Mg[g]), Zg[g], acc);
+                pt = acc * inv_g;
+            } else {
+                // the softmax of every query head and the mean over the group, each rounded to the model's
+                // dtype (kvquant/scorer.py:314-315)
+#pragma unroll
+                for (int g = 0; g < GMAX; ++g)
+                    if (g < a.G) acc += round_model(expf(lg[g] - Mg[g]) * Zg[g], a.round_dt);
+                pt = round_model(acc * inv_g, a.round_dt);
+            }
+        }
+        a.p[(size_t)h * a.Tc + t] = pt;
+    }
     float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    float ps = 0.0f;
-    const int t0 = chunk * ROWS_PER_WG;
-    for (int it0 = 0; it0 < ROWS_PER_WG / 16; it0 += SC_UNROLL_V) {
-        float xs[SC_UNROLL_V][8], lg[SC_UNROLL_V][GMAX];
 #pragma unroll
-        for (int u = 0; u < SC_UNROLL_V; ++u) {
-            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
-            if (t < a.Tc) {
-                load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, xs[u]);
-                if (a.attn != nullptr) lg[u][0] = a.attn[(size_t)h * a.T + a.n_sink + t];
-                else {
+    for (int u0 = 0; u0 < 16; u0 += U) {
+        if (u0 > 0) request(u0);
 #pragma unroll
-                    for (int g = 0; g < GMAX; ++g)
-                        if (g < a.G) lg[u][g] = a.logits[((size_t)h * a.G + g) * a.Tc + t];
-                }
-            }
-        }
+        for (int u = 0; u < U; ++u) {
+            const float pu = group16_bcast(pt, u0 + u);       // 0 for rows past the end
+            float x[8];
+            cvt8<DT>(raw[u], x);
 #pragma unroll
-        for (int u = 0; u < SC_UNROLL_V; ++u) {
-            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
-            if (t < a.Tc) {
-                float pt;
-                if (a.attn != nullptr) {
-                    pt = lg[u][0];
-                } else {
-                    float acc = 0.0f;
-                    if (a.round_dt < 0) {
-#pragma unroll
-                        for (int g = 0; g < GMAX; ++g)
-                            if (g < a.G) acc = __fmaf_rn(__expf(lg[u][g] - Mg[g]), Zg[g], acc);
-                        pt = acc * inv_g;
-                    } else {
-                        // the softmax of every query head and the mean over the group, each rounded to the model's
-                        // dtype (kvquant/scorer.py:314-315)
-#pragma unroll
-                        for (int g = 0; g < GMAX; ++g)
-                            if (g < a.G) acc += round_model(expf(lg[u][g] - Mg[g]) * Zg[g], a.round_dt);
-                        pt = round_model(acc * inv_g, a.round_dt);
-                    }
-                }
-                if (part == 0) { a.p[(size_t)h * a.Tc + t] = pt; ps += pt; }
-#pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = __fmaf_rn(pt, xs[u][e], o[e]);
-            }
+            for (int e = 0; e < 8; ++e) o[e] = __fmaf_rn(pu, x[e], o[e]);
         }
     }
-    const int grp = wave * 4 + rsub;
 #pragma unroll
     for (int e = 0; e < 8; ++e) osum[grp][part * 8 + e] = o[e];
-    if (part == 0) psum_s[grp] = ps;
+    const float ps = wave_sum(pt);
+    if (lane == 0) psum_s[wave] = ps;
     __syncthreads();
     if (tid < HD) {
         float acc = 0.0f;
         for (int g = 0; g < 16; ++g) acc += osum[g][tid];
         a.opart[((size_t)h * a.nchunks + chunk) * HD + tid] = acc;
     }
-    if (tid == 0) {
-        float acc = 0.0f;
-        for (int g = 0; g < 16; ++g) acc += psum_s[g];
-        a.psum[(size_t)h * a.nchunks + chunk] = acc;
-    }
+    if (tid == 0) a.psum[(size_t)h * a.nchunks + chunk] = (psum_s[0] + psum_s[1]) + (psum_s[2] + psum_s[3]);
 }
 
 __global__ __launch_bounds__(1024) void score_obar_kernel(ScoreArgs a) {
@@ -314,6 +470,7 @@ __global__ __launch_bounds__(1024) void score_obar_kernel(ScoreArgs a) {
     __shared__ float part_p[8];
     const int h = blockIdx.x, j = threadIdx.x & (HD - 1), grp = threadIdx.x >> 7;
     float acc = 0.0f, P = 0.0f;
+#pragma unroll 8
     for (int c = grp; c < a.nchunks; c += 8) {
         acc += a.opart[((size_t)h * a.nchunks + c) * HD + j];
         P += a.psum[(size_t)h * a.nchunks + c];
@@ -332,64 +489,74 @@ __global__ __launch_bounds__(1024) void score_obar_kernel(ScoreArgs a) {
 // ---- pass 2 over V: |v|^2, |v - obar|^2, the score, and its global maximum ----
 template <int DT>
 __global__ __launch_bounds__(256) void score_final_kernel(ScoreArgs a) {
+    constexpr int U = VTrip<DT>::ROWS;
     __shared__ unsigned int wmax[4];
     const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, part = lane & 15, rsub = lane >> 4;
+    const int wave = tid >> 6, lane = tid & 63, part = lane & 15, grp = tid >> 4;
+    const int tb = chunk * ROWS_PER_WG + grp * 16;
+    Raw8<DT> raw[U];
+    auto request = [&](int u0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            load8_raw<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + min(tb + u0 + u, a.Tc - 1)) * a.sT + part * 8, raw[u]);
+    };
+    request(0);
+    const int t = tb + part;                       // the lane's own row
+    const bool ok = t < a.Tc;
+    const float pin = ok ? a.p[(size_t)h * a.Tc + t] : 0.0f;
+    const float knin = ok ? a.kn2[(size_t)h * a.Tc + t] : 0.0f;
     float ob[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) ob[e] = a.obar[h * HD + part * 8 + e];
-    float best = 0.0f;
-    const int t0 = chunk * ROWS_PER_WG;
-    for (int it0 = 0; it0 < ROWS_PER_WG / 16; it0 += SC_UNROLL_V) {
-        float xs[SC_UNROLL_V][8], pin[SC_UNROLL_V], knin[SC_UNROLL_V];
+    float vn_own = 0.0f, ir_own = 0.0f;
 #pragma unroll
-        for (int u = 0; u < SC_UNROLL_V; ++u) {
-            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
-            pin[u] = 0.0f; knin[u] = 0.0f;
-            if (t < a.Tc) {
-                load8<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + t) * a.sT + part * 8, xs[u]);
-                if (part == 0) { pin[u] = a.p[(size_t)h * a.Tc + t]; knin[u] = a.kn2[(size_t)h * a.Tc + t]; }
-            } else {
+    for (int u0 = 0; u0 < 16; u0 += U) {
+        if (u0 > 0) request(u0);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) xs[u][e] = 0.0f;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < SC_UNROLL_V; ++u) {
-            const int t = t0 + (it0 + u) * 16 + wave * 4 + rsub;
-            const bool ok = t < a.Tc;
+        for (int u = 0; u < U; ++u) {
+            float x[8];
+            cvt8<DT>(raw[u], x);
             float vn = 0.0f, ir = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                vn = __fmaf_rn(xs[u][e], xs[u][e], vn);
-                const float dlt = xs[u][e] - ob[e];
+                vn = __fmaf_rn(x[e], x[e], vn);
+                const float dlt = x[e] - ob[e];
                 ir = __fmaf_rn(dlt, dlt, ir);
             }
             vn = group16_sum(vn);
             ir = group16_sum(ir);
-            if (ok && part == 0) {
-                // (p + eps)^2 is formed on the tensor of the model's dtype in the reference (kvquant/scorer.py:403):
-                // eps becomes a scalar of that dtype, the sum and the square are rounded to it
-                const float pe = round_model(pin[u] + round_model(a.eps, a.round_dt), a.round_dt);
-                const float kterm = (knin[u] * (1.0f / (float)HD)) * ir;      // 1/128: exact
-                const float sc = round_model(pe * pe, a.round_dt) * (vn + kterm);
-                a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
-                best = fmaxf(best, sc);
-            }
+            vn_own = part == u0 + u ? vn : vn_own;
+            ir_own = part == u0 + u ? ir : ir_own;
         }
+    }
+    float best = 0.0f;
+    if (ok) {
+        // (p + eps)^2 is formed on the tensor of the model's dtype in the reference (kvquant/scorer.py:403):
+        // eps becomes a scalar of that dtype, the sum and the square are rounded to it
+        const float pe = round_model(pin + round_model(a.eps, a.round_dt), a.round_dt);
+        const float kterm = (knin * (1.0f / (float)HD)) * ir_own;      // 1/128: exact
+        const float sc = round_model(pe * pe, a.round_dt) * (vn_own + kterm);
+        a.scores[(size_t)h * a.T + a.n_sink + t] = sc;
+        best = sc;
     }
     best = wave_max(best);
     if (lane == 0) wmax[wave] = __float_as_uint(best);
     __syncthreads();
-    if (tid == 0) {
-        unsigned int mx = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
-        atomicMax(a.gmax, mx);        // non-negative floats order like their bit patterns
-    }
+    if (tid == 0)       // non-negative floats order like their bit patterns; the partial sums of p have been consumed
+        reinterpret_cast<unsigned int*>(a.psum)[(size_t)h * a.nchunks + chunk] = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
 }
 
-__global__ void score_pad_kernel(ScoreArgs a) {
+// the sinks take the largest score of the layer: every workgroup of the last pass left its own maximum (one
+// store each; a single word updated atomically by a thousand workgroups kept that pass waiting on the updates)
+__global__ __launch_bounds__(64) void score_pad_kernel(ScoreArgs a) {
     const int h = blockIdx.x, i = threadIdx.x;
-    if (i < a.n_sink) a.scores[(size_t)h * a.T + i] = __uint_as_float(*a.gmax);
+    const unsigned int* part = reinterpret_cast<const unsigned int*>(a.psum);
+    unsigned int mx = 0u;
+#pragma unroll 8
+    for (int c = i; c < a.Hkv * a.nchunks; c += WAVE) mx = max(mx, part[c]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = max(mx, (unsigned int)__shfl_xor((int)mx, o, WAVE));
+    if (i < a.n_sink) a.scores[(size_t)h * a.T + i] = __uint_as_float(mx);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -749,12 +916,13 @@ __global__ __launch_bounds__(256) void ea_final_kernel(ScoreArgs a) {
     best = wave_max(best);
     if (lane == 0) wmax[wave] = __float_as_uint(best);
     __syncthreads();
-    if (tid == 0) atomicMax(a.gmax, max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
+    if (tid == 0)
+        reinterpret_cast<unsigned int*>(a.psum)[(size_t)h * a.nchunks + chunk] = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
 }
 
 static inline int n_chunks(int Tc) { return (Tc + ROWS_PER_WG - 1) / ROWS_PER_WG; }
 
-struct ScoreLayout { size_t logits, kn2, p, stats, mz, opart, psum, obar, gmax, total; };
+struct ScoreLayout { size_t logits, kn2, p, stats, mz, opart, psum, obar, total; };
 static ScoreLayout score_layout(int Hkv, int Hq, int T) {
     ScoreLayout L;
     const size_t Tc = T, nc = n_chunks(T);
@@ -768,7 +936,6 @@ static ScoreLayout score_layout(int Hkv, int Hq, int T) {
     L.opart = take((size_t)Hkv * nc * HD * 4);
     L.psum = take((size_t)Hkv * nc * 4);
     L.obar = take((size_t)Hkv * HD * 4);
-    L.gmax = take(4);
     L.total = off;
     return L;
 }
@@ -781,11 +948,17 @@ extern "C" size_t odmkv_score_workspace_bytes(int Hkv, int Hq, int T) {
 template <int DT>
 static int run_score(ScoreArgs& a, hipStream_t st) {
     dim3 grid(a.nchunks, a.Hkv), block(256);
-    if (a.G <= 4) hipLaunchKernelGGL((score_logits_kernel<DT, 4>), grid, block, 0, st, a);
+    if constexpr (DT != ODMKV_F32) {
+        // 16-bit keys feed the matrix cores as they lie in memory; the mode that rounds like a 16-bit model and
+        // the call that brings its own attention weights keep the kernel that forms every product in fp32
+        if (a.round_dt < 0 && a.Gl > 0) {
+            if (a.G <= 4) hipLaunchKernelGGL((score_logits16_kernel<DT, 4>), grid, block, 0, st, a);
+            else hipLaunchKernelGGL((score_logits16_kernel<DT, 8>), grid, block, 0, st, a);
+        } else if (a.G <= 4) hipLaunchKernelGGL((score_logits_kernel<DT, 4>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((score_logits_kernel<DT, 8>), grid, block, 0, st, a);
+    } else if (a.G <= 4) hipLaunchKernelGGL((score_logits_kernel<DT, 4>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((score_logits_kernel<DT, 8>), grid, block, 0, st, a);
     ODMKV_CHECK_LAUNCH("score_logits_kernel");
-    hipLaunchKernelGGL(score_stats_kernel, dim3(a.attn ? 1 : a.Hq), dim3(64), 0, st, a);
-    ODMKV_CHECK_LAUNCH("score_stats_kernel");
     if (a.G <= 4) hipLaunchKernelGGL((score_pv_kernel<DT, 4>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((score_pv_kernel<DT, 8>), grid, block, 0, st, a);
     ODMKV_CHECK_LAUNCH("score_pv_kernel");
@@ -836,7 +1009,7 @@ extern "C" int odmkv_score_model_dtype(const void* K, const void* V, int dtype, 
     a.cov = nullptr; a.use_vnorm = 0; a.ea_cpw = 1; a.nstat = a.nchunks; a.round_dt = round_dtype;
     a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
     a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
-    a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);
+    a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar);
     hipStream_t st = (hipStream_t)stream;
     if (dtype == ODMKV_F16) return run_score<ODMKV_F16>(a, st);
     if (dtype == ODMKV_BF16) return run_score<ODMKV_BF16>(a, st);
@@ -920,7 +1093,7 @@ extern "C" int odmkv_score_expected(const void* K, const void* V, int dtype, int
     a.cov = cov; a.use_vnorm = use_vnorm ? 1 : 0; a.ea_cpw = 1; a.nstat = a.nchunks; a.round_dt = -1;
     a.logits = (float*)(ws + L.logits); a.kn2 = (float*)(ws + L.kn2); a.p = (float*)(ws + L.p);
     a.stats = (float*)(ws + L.stats); a.mz = (float*)(ws + L.mz); a.opart = (float*)(ws + L.opart);
-    a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar); a.gmax = (unsigned int*)(ws + L.gmax);
+    a.psum = (float*)(ws + L.psum); a.obar = (float*)(ws + L.obar);
     hipStream_t st = (hipStream_t)stream;
     if (dtype == ODMKV_F16) return run_expected<ODMKV_F16>(a, st);
     if (dtype == ODMKV_BF16) return run_expected<ODMKV_BF16>(a, st);

@@ -62,6 +62,24 @@ def test_score_prefill_matches_oracle(hkv, hq, T, dtype, rotary):
     assert torch.all(got[:, :4] == got[:, 4:].max())
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mu_scale", [2.0 ** -14, 1.0, 3.0e3])
+def test_score_with_mean_queries_far_from_one(dtype, mu_scale):
+    """16-bit keys meet the mean query on the matrix cores as 16-bit pieces of it: mean queries thousands of times
+    larger or smaller than one (keys scaled the other way, so that the logits are ordinary), heads of different
+    magnitude inside one group, one head all zero, a token count that ends inside a block of 16."""
+    from kvquant.scorer import _launch_score
+    hkv, hq, T = 2, 14, 1003
+    g = torch.Generator().manual_seed(int(mu_scale * 7) + 11)
+    k = (torch.randn(hkv, T, 128, generator=g) / mu_scale).clamp(-6e4, 6e4).to(dtype)
+    v = torch.randn(hkv, T, 128, generator=g).to(dtype)
+    mu = torch.randn(hq, 128, generator=g) * mu_scale * 0.3
+    mu[1] *= 50.0; mu[2] *= 0.01; mu[5] = 0.0
+    want = osc.risk_score_from_mu(k.float(), v.float(), mu.unsqueeze(0), hq)
+    got = _launch_score(k.to(DEV), v.to(DEV), mu.to(DEV), None, hq, 4, 1e-2).cpu()
+    np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=SCORE_RTOL)
+
+
 @pytest.mark.parametrize("name", ["f16", "bf16"])
 def test_model_dtype_rounding_matches_reference_vectors(name):
     """The score with the roundings of a 16-bit model (kvquant/scorer.py:309-315: logits, softmax and group mean
