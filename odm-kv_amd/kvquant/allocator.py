@@ -137,6 +137,23 @@ def _eps_table(levels, target_avg_bits, epsilon, eviction_cost, above_target_alp
     return eps_raw
 
 
+_TARGETS: dict = {}        # (device, budgets) -> the budgets as an fp64 device tensor
+
+
+def _targets_on(dev: torch.device, tgt: torch.Tensor) -> torch.Tensor:
+    """The per-row budgets on the device.  A model asks for the same few budgets layer after layer; uploading eight
+    bytes from pageable memory costs a staging copy and a small kernel every call, so the uploaded tensors are kept
+    (they are never written again; the upload is waited for once, so that any stream may read them)."""
+    key = (dev.type, dev.index if dev.index is not None else torch.cuda.current_device(), tuple(tgt.tolist()))
+    hit = _TARGETS.get(key)
+    if hit is None:
+        if len(_TARGETS) >= 256:
+            _TARGETS.clear()
+        hit = _TARGETS[key] = tgt.to(dev)
+        torch.cuda.current_stream(dev).synchronize()
+    return hit
+
+
 def optimal_scores_to_bits_batched(scores: torch.Tensor, bit_levels, targets, epsilon: dict,
                                    *, n_sink: int = 0, period: Optional[int] = None,
                                    sink_mask: Optional[torch.Tensor] = None, sink_bits: int = 16,
@@ -169,7 +186,7 @@ def optimal_scores_to_bits_batched(scores: torch.Tensor, bit_levels, targets, ep
     ws = _lib.workspace(dev, ws_bytes, "allocate")
     lv = (C.c_int32 * len(levels))(*levels)
     ep = (C.c_double * len(levels))(*eps_raw)
-    tgt_dev = tgt.to(dev)
+    tgt_dev = _targets_on(dev, tgt)
     _lib.check(lib.odmkv_allocate(
         s.data_ptr(), rows, n, _lib.ptr(mask), int(period or n), int(n_sink), int(sink_bits),
         lv, len(levels), ep, tgt_dev.data_ptr(), bits.data_ptr(), _lib.ptr(counts), _lib.ptr(lam),

@@ -240,10 +240,14 @@ class TurboQuantAdaptiveKVCacheState:
         """uint8 [B, H, seq_len]: bit level of every position (a view of the growing store)."""
         return None if self._level_store is None else self._level_store[:, :, :self.seq_len]
 
-    def _extend_levels(self, lm: torch.Tensor) -> None:
-        """Write the levels of T new positions behind the current ones (before seq_len is advanced)."""
+    def _extend_levels(self, lm: torch.Tensor, owned: bool = False) -> None:
+        """Write the levels of T new positions behind the current ones (before seq_len is advanced).  owned: lm is
+        a tensor nobody else holds; the first fill of a store keeps it as the level store instead of copying it."""
         B, H, T = lm.shape
         need = self.seq_len + T
+        if owned and self._level_store is None and self.seq_len == 0 and T >= 256 and lm.is_contiguous():
+            self._level_store = lm
+            return
         if self._level_store is None or self._level_store.shape[2] < need:
             cap = max(need, 2 * (0 if self._level_store is None else self._level_store.shape[2]), 256)
             # positions behind seq_len read 16, so that a single exact token needs no write
@@ -432,7 +436,7 @@ class TurboQuantAdaptiveKVCacheState:
         self._exact_room = None
         lm = bits.to(torch.uint8)
         if _pos_offset is None:
-            self._extend_levels(lm)
+            self._extend_levels(lm, owned=lm is not bits)
             self.seq_len += T
         else:
             self._level_store[:, :, pos_offset:pos_offset + T] = lm
