@@ -1681,16 +1681,22 @@ extern "C" int odmkv_quant_pack_staged(const void* K, const void* V, int dtype, 
 struct GatherArgs {
     odmkv_packed_t src, dst;
     int nseg;
+    int slice_begin[ODMKV_NQ + 2];      // workgroups along x: level li owns slice_begin[li] .. slice_begin[li + 1] - 1
 };
 
 __global__ __launch_bounds__(256) void store_gather_kernel(GatherArgs a) {
-    // grid (slices, segments, levels): the wavefronts of a (level, segment)'s workgroups share out its tiles that hold
-    // tokens, a tile per wavefront at a time
-    const int tid = threadIdx.x & 63, wave = threadIdx.x >> 6, bh = blockIdx.y, li = blockIdx.z;
+    // grid (slices of all levels, segments): the wavefronts of a (level, segment)'s workgroups share out its tiles that
+    // hold tokens, a tile per wavefront at a time.  A level gets slices for the tiles the destination has of it (a level
+    // nobody uses: one, which copies the zero counts), so that the launch is not mostly workgroups with nothing to do.
+    const int tid = threadIdx.x & 63, wave = threadIdx.x >> 6, bh = blockIdx.y;
+    int li = 0;
+#pragma unroll
+    for (int k = 1; k <= ODMKV_NQ; ++k) li += ((int)blockIdx.x >= a.slice_begin[k]);
+    const int slice = blockIdx.x - a.slice_begin[li], nslice = a.slice_begin[li + 1] - a.slice_begin[li];
     const int count = a.src.seg_count[li][bh];
-    if (blockIdx.x == 0 && threadIdx.x == 0) a.dst.seg_count[li][bh] = count;
+    if (slice == 0 && threadIdx.x == 0) a.dst.seg_count[li][bh] = count;
     const int src0 = a.src.seg_tile[li][bh], dst0 = a.dst.seg_tile[li][bh];
-    for (int local = blockIdx.x * 4 + wave; local * TILE < count; local += gridDim.x * 4) {
+    for (int local = slice * 4 + wave; local * TILE < count; local += nslice * 4) {
     const int tile = dst0 + local;
     const int hi = min(count - local * TILE, TILE);
     const size_t st = (size_t)src0 + local;                      // the tile in the staging store
@@ -1745,9 +1751,10 @@ extern "C" int odmkv_store_gather(const odmkv_packed_t* staging, const odmkv_pac
     GatherArgs a;
     a.src = *staging; a.dst = *store; a.nseg = store->B * store->Hkv;
     ODMKV_CHECK_ARG(a.nseg <= 65535, "store_gather: at most 65535 (sequence, head) pairs");
-    int most = 1;
-    for (int li = 0; li <= ODMKV_NQ; ++li) most = std::max(most, store->n_tiles[li]);
-    const dim3 grid(std::max(1, std::min(128, (most / a.nseg + 4) / 4)), a.nseg, ODMKV_NQ + 1);
+    a.slice_begin[0] = 0;
+    for (int li = 0; li <= ODMKV_NQ; ++li)        // four tiles (one per wavefront) per workgroup and trip
+        a.slice_begin[li + 1] = a.slice_begin[li] + std::max(1, std::min(128, (store->n_tiles[li] / a.nseg + 4) / 4));
+    const dim3 grid(a.slice_begin[ODMKV_NQ + 1], a.nseg);
     hipLaunchKernelGGL(store_gather_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);
     ODMKV_CHECK_LAUNCH("store_gather_kernel");
     return 0;
