@@ -93,6 +93,9 @@ __device__ static inline float group16_sum(float v) {
     v += dpp_move<0x128>(v);    // row_ror 8
     return v;
 }
+// workgroup barrier that orders LDS traffic only: global loads requested before it stay in flight
+// (__syncthreads would first wait for every outstanding load of the wavefront, the rows from memory included)
+__device__ static inline void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 #define SC_UNROLL 4            // rows in flight per lane group: their loads are issued before any is used
 #define SC_UNROLL_V 4          // the same for the two passes over V
 
@@ -242,6 +245,18 @@ __global__ __launch_bounds__(256) void score_logits16_kernel(ScoreArgs a) {
     const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, n = lane & 15, j = lane >> 4;
     const int t0 = chunk * ROWS_PER_WG + wave * 64;
+    // The mean queries first: loads return in the order of their requests, and these few kilobytes come out of the
+    // L2 while the keys come from memory; requested behind the keys they would arrive no earlier than the keys, and
+    // the two barriers of the split below would start only then.
+    const int mg = tid >> 5, msub = tid & 31;       // 8 heads x 32 threads x 4 dims: the largest entry per head
+    float4 mu_max = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (mg < a.Gl) mu_max = *reinterpret_cast<const float4*>(a.mu + ((size_t)h * a.G + mg) * HD + 4 * msub);
+    const int shb = tid >> 6, si = (tid >> 4) & 3, sjj = (tid >> 2) & 3, sg = 4 * shb + (tid & 3);   // the split's share
+    float4 mu_a = make_float4(0.0f, 0.0f, 0.0f, 0.0f), mu_b = mu_a;
+    if (tid < HB * 64 && sg < a.Gl) {
+        const float* src = a.mu + ((size_t)h * a.G + sg) * HD + 32 * si + 8 * sjj;
+        mu_a = *reinterpret_cast<const float4*>(src); mu_b = *reinterpret_cast<const float4*>(src + 4);
+    }
     // the keys: group q's token n, dims 32 i + 8 j .. + 7 (rows past the end repeat the last row, never stored)
     uint4 kx[4][4];
 #pragma unroll
@@ -253,12 +268,8 @@ __global__ __launch_bounds__(256) void score_logits16_kernel(ScoreArgs a) {
     }
     // per head: the power of two that brings the largest entry below 1 (fp16 pieces; bf16 has fp32's range)
     {
-        const int g = tid >> 5, sub = tid & 31;     // 8 heads x 32 threads x 4 dims
-        float mx = 0.0f;
-        if (g < a.Gl) {
-            const float4 v = *reinterpret_cast<const float4*>(a.mu + ((size_t)h * a.G + g) * HD + 4 * sub);
-            mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        }
+        const int g = mg, sub = msub;
+        float mx = fmaxf(fmaxf(fabsf(mu_max.x), fabsf(mu_max.y)), fmaxf(fabsf(mu_max.z), fabsf(mu_max.w)));
 #pragma unroll
         for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, WAVE));
         if (sub == 0 && g < GMAX) {
@@ -268,19 +279,11 @@ __global__ __launch_bounds__(256) void score_logits16_kernel(ScoreArgs a) {
             red_m[0][g] = ldexpf(1.0f, -ex);                   // (borrowed until the barrier after the split)
         }
     }
-    __syncthreads();
+    lds_barrier();
     if (tid < HB * 64) {
-        const int hb = tid >> 6, i = (tid >> 4) & 3, jj = (tid >> 2) & 3, g = 4 * hb + (tid & 3);
-        float x[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = 0.0f;
-        if (g < a.Gl) {
-            const float* src = a.mu + ((size_t)h * a.G + g) * HD + 32 * i + 8 * jj;
-            const float4 v0 = *reinterpret_cast<const float4*>(src), v1 = *reinterpret_cast<const float4*>(src + 4);
-            const float sc = red_m[0][g];
-            x[0] = v0.x * sc; x[1] = v0.y * sc; x[2] = v0.z * sc; x[3] = v0.w * sc;
-            x[4] = v1.x * sc; x[5] = v1.y * sc; x[6] = v1.z * sc; x[7] = v1.w * sc;
-        }
+        const int hb = shb, i = si, g = sg;
+        const float sc = g < a.Gl ? red_m[0][g] : 0.0f;
+        float x[8] = {mu_a.x * sc, mu_a.y * sc, mu_a.z * sc, mu_a.w * sc, mu_b.x * sc, mu_b.y * sc, mu_b.z * sc, mu_b.w * sc};
 #pragma unroll
         for (int pc = 0; pc < NP; ++pc) {
             uint32_t w[4];
@@ -293,7 +296,7 @@ __global__ __launch_bounds__(256) void score_logits16_kernel(ScoreArgs a) {
             mu_op[hb][i][pc][tid & 15] = make_uint4(w[0], w[1], w[2], w[3]);
         }
     }
-    __syncthreads();
+    lds_barrier();
     // |k|^2: lane (n / 4, n) holds the diagonal element of token n in component n % 4
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -383,7 +386,9 @@ __global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
         for (int u = 0; u < U; ++u)
             load8_raw<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + min(tb + u0 + u, a.Tc - 1)) * a.sT + part * 8, raw[u]);
     };
-    request(0);
+    // The small operands first (the row's logits, the block statistics): loads return in the order of their
+    // requests, these come out of the L2 and the rows of V from memory; behind V they would arrive with V, and the
+    // merge of the statistics, a barrier and the weights would start only then.
     const int t = tb + part;                       // the lane's own row
     float lg[GMAX];
     if (a.attn == nullptr && t < a.Tc) {
@@ -391,12 +396,29 @@ __global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
         for (int g = 0; g < GMAX; ++g)
             if (g < a.G) lg[g] = a.logits[((size_t)h * a.G + g) * a.Tc + t];
     }
+    constexpr int NPRE = 4;                        // statistics entries per lane and head requested ahead (256 blocks)
+    float2 pre[GMAX / 4][NPRE];
+#pragma unroll
+    for (int gi = 0; gi < GMAX / 4; ++gi)
+#pragma unroll
+        for (int k = 0; k < NPRE; ++k) {
+            const int g = wave + 4 * gi, c = lane + WAVE * k;
+            pre[gi][k] = make_float2(-INFINITY, 0.0f);
+            if (a.attn == nullptr && g < a.G && c < a.nstat)
+                pre[gi][k] = *reinterpret_cast<const float2*>(a.stats + ((size_t)(h * a.G + g) * a.nstat + c) * 2);
+        }
+    request(0);
     // (max, sum) of every query head of the group over all chunks: each workgroup merges the chunk statistics
-    // again (a kilobyte per head out of the L2, under the loads above) instead of waiting for a launch that does
+    // again (a kilobyte per head out of the L2) instead of waiting for a launch that does
     if (a.attn == nullptr) {
-        for (int g = wave; g < a.G; g += 4) {
+#pragma unroll
+        for (int gi = 0; gi < GMAX / 4; ++gi) {
+            const int g = wave + 4 * gi;
+            if (g >= a.G) break;
             float m = -INFINITY, sm = 0.0f;
-            for (int c = lane; c < a.nstat; c += WAVE) {
+#pragma unroll
+            for (int k = 0; k < NPRE; ++k) ms_merge(m, sm, pre[gi][k].x, pre[gi][k].y);
+            for (int c = lane + WAVE * NPRE; c < a.nstat; c += WAVE) {
                 const float2 e = *reinterpret_cast<const float2*>(a.stats + ((size_t)(h * a.G + g) * a.nstat + c) * 2);
                 ms_merge(m, sm, e.x, e.y);
             }
@@ -407,7 +429,7 @@ __global__ __launch_bounds__(256) void score_pv_kernel(ScoreArgs a) {
             }
             if (lane == 0) { mz_s[2 * g] = m; mz_s[2 * g + 1] = 1.0f / sm; }     // reciprocal of the sum
         }
-        __syncthreads();
+        lds_barrier();
     }
     // the weight of the lane's own row
     float pt = 0.0f;
@@ -500,14 +522,19 @@ __global__ __launch_bounds__(256) void score_final_kernel(ScoreArgs a) {
         for (int u = 0; u < U; ++u)
             load8_raw<DT>(a.V, (size_t)h * a.sH + (size_t)(a.n_sink + min(tb + u0 + u, a.Tc - 1)) * a.sT + part * 8, raw[u]);
     };
-    request(0);
+    // the row's scalars and the mean output first (loads return in the order of their requests: behind the rows,
+    // the first row could not be used before the last had arrived)
     const int t = tb + part;                       // the lane's own row
     const bool ok = t < a.Tc;
     const float pin = ok ? a.p[(size_t)h * a.Tc + t] : 0.0f;
     const float knin = ok ? a.kn2[(size_t)h * a.Tc + t] : 0.0f;
     float ob[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) ob[e] = a.obar[h * HD + part * 8 + e];
+    {
+        const float4 o0 = *reinterpret_cast<const float4*>(a.obar + h * HD + part * 8);
+        const float4 o1 = *reinterpret_cast<const float4*>(a.obar + h * HD + part * 8 + 4);
+        ob[0] = o0.x; ob[1] = o0.y; ob[2] = o0.z; ob[3] = o0.w; ob[4] = o1.x; ob[5] = o1.y; ob[6] = o1.z; ob[7] = o1.w;
+    }
+    request(0);
     float vn_own = 0.0f, ir_own = 0.0f;
 #pragma unroll
     for (int u0 = 0; u0 < 16; u0 += U) {
