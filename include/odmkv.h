@@ -53,6 +53,9 @@ const char* odmkv_last_error(void);
  * attn: NULL, or device fp32 [Hkv, T] attention weights to use instead of computing p from mu
  *       (then n_sink must be 0 and no sink padding happens: score_with_attn).
  * scores: device fp32 [Hkv, T] out.
+ * Arithmetic: every sum is accumulated in fp32 in a fixed order.  With fp16 / bf16 keys the products mu . k run on
+ * the matrix cores: the keys as they are, mu as 16-bit pieces whose sum is the fp32 vector (fp16: high + low of the
+ * vector scaled by a power of two; bf16: three pieces), so that no bit of mu is dropped; fp32 keys take fp32 products.
  */
 size_t odmkv_score_workspace_bytes(int Hkv, int Hq, int T);
 int odmkv_score(const void* K, const void* V, int dtype, int Hkv, int T,
