@@ -42,7 +42,8 @@ class Stub(torch.nn.Module):
 
 @pytest.mark.parametrize("hkv,hq,T,dtype,rotary", [
     (2, 8, 700, torch.float32, False), (8, 32, 4096, torch.float16, False), (4, 28, 1500, torch.bfloat16, False),
-    (2, 4, 300, torch.float32, True), (3, 3, 261, torch.float16, False), (1, 1, 5, torch.float32, False)])
+    (2, 4, 300, torch.float32, True), (3, 3, 261, torch.float16, False), (1, 1, 5, torch.float32, False),
+    (2, 8, 7, torch.float16, False), (1, 4, 70, torch.bfloat16, False), (2, 16, 5, torch.bfloat16, False)])
 def test_score_prefill_matches_oracle(hkv, hq, T, dtype, rotary):
     from kvquant.scorer import RiskScorer
     g = torch.Generator().manual_seed(T)
