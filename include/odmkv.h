@@ -240,6 +240,15 @@ int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, int Hkv, in
                      const odmkv_packed_t* store, void* workspace, size_t workspace_bytes,
                      void* stream);
 
+/* Lloyd-Max codebook of 2 <= k <= 256 levels for the coordinate density of a randomly rotated unit vector in
+ * d >= 100 dimensions, N(0, 1/d): the reference's offline routine (codebook.py:75-113 compute_codebook with
+ * :36-72 lloyd_max_iteration: 10 000 grid points over +-x_range / sqrt(d), at most n_iter rounds, stop when no
+ * centroid moves by tol) run by one workgroup in fp64.  centroids: device fp64 [k], ascending; rounds: device
+ * int (rounds run) or NULL.  Agrees with the host routine to about 1e-16 relative (only the order inside a
+ * cell's sums differs), i.e. gives the same fp32 tables. */
+int odmkv_lloyd_max(int k, int d, int n_iter, double tol, double x_range, double* centroids, int* rounds,
+                    void* stream);
+
 /* Row-wise quantiser without the packed store: x [N, 128] of `dtype` with element stride
  * `stride_n` -> codes uint8 [N, 128] (one code per byte) and norms fp32 [N], same arithmetic as
  * odmkv_quant_pack.  `bits` is 2, 3, 4 or 8; cb the 2^bits centroids (device).  This is

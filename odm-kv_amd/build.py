@@ -21,7 +21,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libodmkv.so")
 BENCH_LIB = os.path.join(LIBDIR, "libodmkv_bench.so")
-SOURCES = ["error.hip", "score.hip", "window.hip", "allocate.hip", "pack.hip", "rows.hip", "decode.hip", "flush.hip"]
+SOURCES = ["error.hip", "score.hip", "window.hip", "allocate.hip", "pack.hip", "rows.hip", "decode.hip", "flush.hip", "codebook.hip"]
 BENCH_SOURCES = ["bench_hooks.hip"]
 FLAGS = [
     "-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-ffp-contract=off",

@@ -54,11 +54,28 @@ def cached_rotation(dim: int, device, seed: int) -> torch.Tensor:
     return pi
 
 
+def lloyd_max_on_device(k: int, dim: int, device, n_iter: int = 500, tol: float = 1e-10,
+                        x_range: float = 5.0) -> np.ndarray:
+    """compute_codebook(k, dim) run by the GPU (odmkv_lloyd_max): fp64 centroids, ascending."""
+    dev = torch.device(device)
+    out = torch.empty(k, dtype=torch.float64, device=dev)
+    _lib.check(lib.odmkv_lloyd_max(int(k), int(dim), int(n_iter), float(tol), float(x_range), out.data_ptr(), None,
+                                   _lib.stream_ptr(dev)))
+    return out.cpu().numpy()
+
+
 def _load_or_compute_codebook(bits: int, dim: int, device, dtype: torch.dtype) -> torch.Tensor:
+    """The 2^bits centroids as a tensor on `device` (kvquant/tq_backend.py:39-46).  Built once per (bits, dim): by
+    the GPU when `device` is one and the density is the normal one (dim >= 100; 0.6 s of host time for the 8-bit
+    table otherwise), by codebook.compute_codebook on the host else.  The two give the same fp32 numbers."""
     key = (bits, dim)
     cached = _CODEBOOK_CACHE.get(key)
     if cached is None:
-        cached = torch.from_numpy(compute_codebook(2 ** bits, dim).astype(np.float32))
+        if torch.device(device).type == "cuda" and dim >= 100 and bits <= 8:
+            c64 = lloyd_max_on_device(2 ** bits, dim, device)
+        else:
+            c64 = compute_codebook(2 ** bits, dim)
+        cached = torch.from_numpy(c64.astype(np.float32))
         _CODEBOOK_CACHE[key] = cached
     return cached.to(device=device, dtype=dtype)
 
@@ -68,8 +85,8 @@ def codebook_table(dim: int, device) -> torch.Tensor:
     key = (dim, str(device))
     tab = _TABLE_CACHE.get(key)
     if tab is None:
-        parts = [_load_or_compute_codebook(b, dim, "cpu", torch.float32) for b in SUPPORTED_WIDTHS]
-        tab = torch.cat(parts).to(device).contiguous()
+        parts = [_load_or_compute_codebook(b, dim, device, torch.float32) for b in SUPPORTED_WIDTHS]
+        tab = torch.cat(parts).contiguous()
         _TABLE_CACHE[key] = tab
     return tab
 
@@ -100,7 +117,7 @@ def decode_tables(dim: int, device) -> tuple[torch.Tensor, list[float]]:
     if got is None:
         parts, inv = [], []
         for b in SUPPORTED_WIDTHS:
-            c = _load_or_compute_codebook(b, dim, "cpu", torch.float32).numpy()
+            c = _load_or_compute_codebook(b, dim, device, torch.float32).cpu().numpy()
             s = _fp16_friendly_scale(c)
             parts.append(torch.from_numpy((c.astype(np.float64) * s).astype(np.float32)))
             inv.append(float(np.float32(1.0 / s)))

@@ -366,3 +366,25 @@ def test_fp16_special_rows_and_ordinary_ones(dtype):
     hk, hv = _same_bytes_in_both_types(k.to(DEV), v.to(DEV), bits8.to(DEV))
     n8 = sum(-(-int((bits8[b, h] == 8).sum()) // 64) for b in range(B) for h in range(H))
     assert (hk, hv) == (n8, n8)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 8])
+def test_lloyd_max_on_the_device_gives_the_reference_tables(golden, bits):
+    """odmkv_lloyd_max against the fp64 centroids the reference's compute_codebook returned (fixture) and against the
+    host routine of the product: the same numbers to 1e-13 relative to the table's scale, and the same fp32 tables
+    bit for bit (only the order of the additions inside a cell differs)."""
+    from codebook import compute_codebook
+    from kvquant.tq_backend import lloyd_max_on_device
+    got = lloyd_max_on_device(2 ** bits, 128, DEV)
+    ref = golden[f"codebook_d128_b{bits}"]
+    host = compute_codebook(2 ** bits, 128)
+    assert got.dtype == np.float64 and got.shape == ref.shape and np.all(np.diff(got) > 0)
+    scale = np.abs(ref).max()
+    assert np.abs(got - ref).max() <= 1e-13 * scale, np.abs(got - ref).max() / scale
+    assert np.array_equal(got.astype(np.float32), ref.astype(np.float32))
+    assert np.array_equal(got.astype(np.float32), host.astype(np.float32))
+    # the argument checks: too many levels, a dimension whose density is not the normal one
+    from kvquant import _lib
+    out = torch.empty(512, dtype=torch.float64, device=DEV)
+    assert _lib.lib.odmkv_lloyd_max(512, 128, 500, 1e-10, 5.0, out.data_ptr(), None, None) == -1
+    assert _lib.lib.odmkv_lloyd_max(4, 64, 500, 1e-10, 5.0, out.data_ptr(), None, None) == -1
