@@ -81,6 +81,24 @@ def test_score_with_mean_queries_far_from_one(dtype, mu_scale):
     np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=SCORE_RTOL)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_score_reads_keys_where_they_lie(dtype):
+    """Keys and values that are views (token-major storage seen as [H, T, d]; the upper half of 256-wide rows; a
+    window of a longer cache) are read through their strides, not copied: same scores as for contiguous copies."""
+    from kvquant.scorer import _launch_score
+    hkv, hq, T = 3, 12, 777
+    g = torch.Generator().manual_seed(5)
+    mu = torch.randn(hq, 128, generator=g)
+    base_k = torch.randn(T + 9, hkv, 256, generator=g).to(dtype)
+    base_v = torch.randn(T + 9, hkv, 256, generator=g).to(dtype)
+    views = lambda t: t.to(DEV)[5:5 + T, :, 128:].transpose(0, 1)          # noqa: E731
+    k, v = views(base_k), views(base_v)
+    assert not k.is_contiguous() and k.stride(-1) == 1
+    got = _launch_score(k, v, mu.to(DEV), None, hq, 4, 1e-2).cpu()
+    want = osc.risk_score_from_mu(k.cpu().float().contiguous(), v.cpu().float().contiguous(), mu.unsqueeze(0), hq)
+    np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=SCORE_RTOL)
+
+
 @pytest.mark.parametrize("name", ["f16", "bf16"])
 def test_model_dtype_rounding_matches_reference_vectors(name):
     """The score with the roundings of a 16-bit model (kvquant/scorer.py:309-315: logits, softmax and group mean
