@@ -227,9 +227,10 @@ __device__ static inline float candidate(const RowState& st, int L, int c) {
 }
 
 // did launch L pass over the scores, given the state it started from?
-__device__ static inline bool launch_evaluates(const RowState& st, int L) {
-    return st.n_active != 0 && !(L > 0 && L < L_FINAL && st.collapsed);
+__device__ static inline bool launch_evaluates(int n_active, int collapsed, int L) {
+    return n_active != 0 && !(L > 0 && L < L_FINAL && collapsed);
 }
+__device__ static inline bool launch_evaluates(const RowState& st, int L) { return launch_evaluates(st.n_active, st.collapsed, L); }
 
 // Start of launch L >= 1 (the candidate kernel calls it as launch L_FINAL + 1): the state launch L - 1
 // started from plus that launch's partial sums give the state this launch starts from, left in `cur`
@@ -238,13 +239,18 @@ __device__ static inline bool launch_evaluates(const RowState& st, int L) {
 __device__ static void carry_state(const AllocArgs& a, int row, int L, RowState* out, RowState* cur, unsigned int* tot) {
     const int tid = threadIdx.x;
     const RowState* in = a.state + (size_t)((L - 1) & 1) * a.rows + row;
-    // a thread's first partial sum is asked for together with the state (it is discarded if that launch did not evaluate)
+    // Everything the launch needs of the last one is asked for here, at once: the two fields that say whether that
+    // launch evaluated, a thread's first partial sum (discarded if it did not), and the whole state, which thread 0
+    // copies into shared memory and advances there (a private copy lived in scratch memory, behind the barriers, and
+    // every access to it was a round trip of its own).
+    const int in_active = in->n_active, in_collapsed = in->collapsed;
     const unsigned int* p = a.partial + ((size_t)((L - 1) & 1) * a.rows + row) * a.n_chunks * SLOTS;
     const int n_part = a.n_chunks * SLOTS;
     const unsigned int v0 = tid < n_part ? p[tid] : 0u;
+    if (tid == 0) *cur = *in;
     if (tid < SLOTS) tot[tid] = 0u;
     __syncthreads();
-    const bool evaluated = launch_evaluates(*in, L - 1);
+    const bool evaluated = launch_evaluates(in_active, in_collapsed, L - 1);
     if (evaluated) {
         if (v0) atomicAdd(&tot[tid & (SLOTS - 1)], v0);
         for (int idx = tid + blockDim.x; idx < n_part; idx += blockDim.x) {
@@ -254,12 +260,10 @@ __device__ static void carry_state(const AllocArgs& a, int row, int L, RowState*
     }
     __syncthreads();
     if (tid == 0) {
-        RowState st = *in;
-        if (evaluated) advance(a, st, L - 1, tot);
-        *cur = st;
+        if (evaluated) advance(a, *cur, L - 1, tot);
         if (blockIdx.x == 0) {
-            *out = st;
-            if (L - 1 == L_FINAL && evaluated && a.lambda_out) a.lambda_out[row] = st.lam;
+            *out = *cur;
+            if (L - 1 == L_FINAL && evaluated && a.lambda_out) a.lambda_out[row] = cur->lam;
         }
     }
     __syncthreads();
