@@ -141,10 +141,21 @@ __global__ __launch_bounds__(SC_THREADS) void alloc_scan_kernel(AllocArgs a) {
             else non = 1;
         }
     }
-    if (mx) atomicMax(&smax, mx);
-    if (fin) atomicOr(&sfin, 1);
-    if (non) atomicOr(&snon, 1);
-    if (act) atomicAdd(&sact, act);
+    // a wavefront first combines its own lanes: 512 threads updating the same four words one after the other took
+    // longer than reading the scores
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        mx = max(mx, (unsigned int)__shfl_xor((int)mx, o, WAVE));
+        act += __shfl_xor(act, o, WAVE);
+    }
+    fin = __any(fin);
+    non = __any(non);
+    if ((threadIdx.x & 63) == 0) {
+        if (mx) atomicMax(&smax, mx);
+        if (fin) atomicOr(&sfin, 1);
+        if (non) atomicOr(&snon, 1);
+        if (act) atomicAdd(&sact, act);
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
         RowState& st = a.state[row];
@@ -252,11 +263,15 @@ __device__ static void carry_state(const AllocArgs& a, int row, int L, RowState*
     __syncthreads();
     const bool evaluated = launch_evaluates(in_active, in_collapsed, L - 1);
     if (evaluated) {
-        if (v0) atomicAdd(&tot[tid & (SLOTS - 1)], v0);
-        for (int idx = tid + blockDim.x; idx < n_part; idx += blockDim.x) {
-            const unsigned int v = p[idx];
-            if (v) atomicAdd(&tot[idx & (SLOTS - 1)], v);
-        }
+        // thread tid holds slot tid % SLOTS of chunk tid / SLOTS (the block size is a multiple of SLOTS, so every
+        // further element of the thread is the same slot); the four chunks of a wavefront are added across its
+        // 16-lane rows before one lane per slot updates the total
+        static_assert(SLOTS == 16 && EV_THREADS % SLOTS == 0, "a slot per lane of a 16-lane row");
+        unsigned int v = v0;
+        for (int idx = tid + blockDim.x; idx < n_part; idx += blockDim.x) v += p[idx];
+        v += (unsigned int)__shfl_xor((int)v, 16, WAVE);
+        v += (unsigned int)__shfl_xor((int)v, 32, WAVE);
+        if ((tid & 63) < SLOTS && v) atomicAdd(&tot[tid & (SLOTS - 1)], v);
     }
     __syncthreads();
     if (tid == 0) {
