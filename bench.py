@@ -729,6 +729,7 @@ def main() -> int:
         "level_counts": counts,
         "score_alloc_pack_ms_per_layer": round(statistics.median(t_stage["total"]) * 1e3, 3),
         "stage_ms": {k: round(statistics.median(v) * 1e3, 3) for k, v in t_stage.items()},
+        "stage_ms_min_max": {k: [round(min(v) * 1e3, 3), round(max(v) * 1e3, 3)] for k, v in t_stage.items()},
         "parity": {"gate_attn_rel_err": gate_err, "full_size_fused_vs_dense_rel_err": full_err},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
