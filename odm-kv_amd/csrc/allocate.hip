@@ -628,17 +628,26 @@ __global__ __launch_bounds__(EV_THREADS) void alloc_write_kernel(AllocArgs a, in
     if (threadIdx.x < NLV) lh[threadIdx.x] = 0;
     __syncthreads();
     const int base = blockIdx.x * EV_TOKENS;
+    const bool count = a.level_counts != nullptr;          // the histogram is optional
     for (int e = 0; e < EV_TPT; ++e) {
         const int i = base + e * EV_THREADS + threadIdx.x;
+        int k = -1;
         if (i < a.n) {
             int out;
             if (is_sink(a, row, i)) out = a.sink_bits;
             else {
-                const int k = single_level ? 0 : a.chosen[(size_t)row * a.n + i];
+                k = single_level ? 0 : a.chosen[(size_t)row * a.n + i];
                 out = a.nominal[k];
-                atomicAdd(&lh[k], 1);
             }
             a.bits_out[(size_t)row * a.n + i] = out;
+        }
+        if (count) {
+            // a wavefront counts its lanes per level by ballot: a thousand threads adding 1 to the same word, one
+            // after the other, took longer than writing the bits
+            for (int lv = 0; lv < a.K; ++lv) {
+                const int n = __popcll(__ballot(k == lv));
+                if ((threadIdx.x & 63) == 0 && n) atomicAdd(&lh[lv], n);
+            }
         }
     }
     __syncthreads();
