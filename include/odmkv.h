@@ -204,11 +204,14 @@ int odmkv_store_init(void* arena, const int32_t* tables_host, int n_tables, int 
  * banks grow by torch.cat (kvquant/tq_adaptive_backend.py:46-52, 149-174). */
 int odmkv_store_gather(const odmkv_packed_t* staging, const odmkv_packed_t* store, void* stream);
 
-/* The part of a store's first fill that does not depend on the level counts, in one call: odmkv_level_counts into
- * counts_dev, an asynchronous copy of the counts to counts_host (page-locked host memory, int32 [B*Hkv, 6]) with
- * counts_event (a hipEvent_t) recorded behind it, the staging store emptied (its tables as odmkv_store_layout gave
- * them: staging_tables_host, staging_offsets, tables_end, counts_end) and odmkv_quant_pack into it.  The caller
- * waits for the event alone, lays out the store proper and calls odmkv_store_gather.  No counterpart in the reference. */
+/* The part of a store's first fill that does not depend on the level counts, in one call: the staging store emptied
+ * (its tables as odmkv_store_layout gave them: staging_tables_host, staging_offsets, tables_end, counts_end), then
+ * odmkv_quant_pack into it, whose first kernel counts the levels of every 2048-token chunk anyway: those counts go to
+ * counts_dev (device int32 [B*Hkv, odmkv_pack_count_chunks(T), 6]: evicted, then 2, 3, 4, 8, 16 bits; a value that is
+ * no level is counted nowhere) and from there, asynchronously, to counts_host (page-locked host memory of the same
+ * size), with counts_event (a hipEvent_t) recorded behind the copy.  The caller waits for the event alone, adds up the
+ * chunks, lays out the store proper and calls odmkv_store_gather.  No counterpart in the reference. */
+int odmkv_pack_count_chunks(int T);
 int odmkv_quant_pack_staged(const void* K, const void* V, int dtype, int B, int Hkv, int T,
                             int64_t stride_b, int64_t stride_h, int64_t stride_t,
                             const int32_t* bits, int pos_offset,

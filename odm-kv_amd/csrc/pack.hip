@@ -221,6 +221,7 @@ struct CompactArgs {
     int32_t* old_count;     // [5][nseg]
     int32_t* chunk_count;   // [nseg][n_chunks][5]
     int32_t* redo;          // two counters the quantise kernels use, cleared here (may be null)
+    int32_t* totals;        // [nseg][n_chunks][6] tokens per chunk that are evicted / at each of the five levels, or null
 };
 
 // levels (1..5, 0 = evicted, -1 = past the end) of the 8 consecutive tokens this thread owns
@@ -240,8 +241,10 @@ __device__ static inline void load_slots(const CompactArgs& a, int bh, int t0, i
 
 __global__ __launch_bounds__(CP_THREADS) void chunk_count_kernel(CompactArgs a) {
     __shared__ int c[5];
+    __shared__ int c_evicted;
     const int bh = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
     if (tid < 5) c[tid] = 0;
+    if (tid == 5) c_evicted = 0;
     if (chunk == 0 && tid < 5) a.old_count[tid * a.nseg + bh] = a.seg_count[tid][bh];
     if (a.redo && chunk == 0 && bh == 0 && tid < 2) a.redo[tid] = 0;
     __syncthreads();
@@ -255,8 +258,16 @@ __global__ __launch_bounds__(CP_THREADS) void chunk_count_kernel(CompactArgs a) 
         n = wave_sum_i32(n);
         if ((tid & 63) == 0 && n) atomicAdd(&c[L], n);
     }
+    if (a.totals) {                                       // wave-uniform
+        int n = 0;
+#pragma unroll
+        for (int e = 0; e < CP_TPT; ++e) n += (sl[e] == 0);
+        n = wave_sum_i32(n);
+        if ((tid & 63) == 0 && n) atomicAdd(&c_evicted, n);
+    }
     __syncthreads();
     if (tid < 5) a.chunk_count[((size_t)bh * a.n_chunks + chunk) * 5 + tid] = c[tid];
+    if (a.totals && tid < 6) a.totals[((size_t)bh * a.n_chunks + chunk) * 6 + tid] = tid == 0 ? c_evicted : c[tid - 1];
 }
 
 __global__ __launch_bounds__(CP_THREADS) void compact_kernel(CompactArgs a) {
@@ -1580,12 +1591,14 @@ static int launch_exact(const ExactArgs& ea, int out_dt, int n_tiles, hipStream_
     return 0;
 }
 
-extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, int Hkv, int T,
-                                int64_t stride_b, int64_t stride_h, int64_t stride_t,
-                                const int32_t* bits, int pos_offset,
-                                const float* pi_k, const float* pi_v, const float* codebooks,
-                                const odmkv_packed_t* store, void* workspace, size_t workspace_bytes,
-                                void* stream) {
+// totals_dev / totals_host / totals_event: null, or where the per-chunk level counts go as soon as they are known
+// (device buffer, page-locked host copy, event recorded behind the copy)
+static int quant_pack_impl(const void* K, const void* V, int dtype, int B, int Hkv, int T,
+                           int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                           const int32_t* bits, int pos_offset,
+                           const float* pi_k, const float* pi_v, const float* codebooks,
+                           const odmkv_packed_t* store, void* workspace, size_t workspace_bytes,
+                           void* stream, int32_t* totals_dev, int32_t* totals_host, void* totals_event) {
     ODMKV_CHECK_ARG(K && V && bits && pi_k && pi_v && codebooks && workspace, "quant_pack: null pointer");
     ODMKV_CHECK_ARG(dtype == ODMKV_F16 || dtype == ODMKV_BF16 || dtype == ODMKV_F32, "quant_pack: bad dtype %d", dtype);
     ODMKV_CHECK_ARG(B > 0 && Hkv > 0 && T > 0, "quant_pack: bad shape B=%d Hkv=%d T=%d", B, Hkv, T);
@@ -1608,10 +1621,15 @@ extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, 
     // fp16 rows take the matrix-core estimate first; what it leaves over reaches the exact kernel through this list
     int32_t* redo = (int32_t*)((char*)workspace + pack_redo_offset(nseg, T));
     ca.redo = redo;
+    ca.totals = totals_dev;
     for (int li = 0; li < 5; ++li) { ca.pos[li] = store->pos[li]; ca.seg_tile[li] = store->seg_tile[li]; ca.seg_count[li] = store->seg_count[li]; }
     ODMKV_CHECK_ARG(nseg <= 65535, "quant_pack: at most 65535 (sequence, head) pairs per call");
     hipLaunchKernelGGL(chunk_count_kernel, dim3(ca.n_chunks, nseg), dim3(CP_THREADS), 0, st, ca);
     ODMKV_CHECK_LAUNCH("chunk_count_kernel");
+    if (totals_dev) {
+        ODMKV_CHECK_HIP(hipMemcpyAsync(totals_host, totals_dev, (size_t)nseg * ca.n_chunks * 6 * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        ODMKV_CHECK_HIP(hipEventRecord((hipEvent_t)totals_event, st));
+    }
     hipLaunchKernelGGL(compact_kernel, dim3(ca.n_chunks, nseg), dim3(CP_THREADS), 0, st, ca);
     ODMKV_CHECK_LAUNCH("compact_kernel");
 
@@ -1653,8 +1671,21 @@ extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, 
     return 0;
 }
 
-// The first fill of a store, everything that does not depend on the level counts in one call: count the levels, send the
-// counts to the host (page-locked memory, an event behind the copy), empty the staging store and quantise into it.
+extern "C" int odmkv_quant_pack(const void* K, const void* V, int dtype, int B, int Hkv, int T,
+                                int64_t stride_b, int64_t stride_h, int64_t stride_t,
+                                const int32_t* bits, int pos_offset,
+                                const float* pi_k, const float* pi_v, const float* codebooks,
+                                const odmkv_packed_t* store, void* workspace, size_t workspace_bytes,
+                                void* stream) {
+    return quant_pack_impl(K, V, dtype, B, Hkv, T, stride_b, stride_h, stride_t, bits, pos_offset, pi_k, pi_v, codebooks,
+                           store, workspace, workspace_bytes, stream, nullptr, nullptr, nullptr);
+}
+
+extern "C" int odmkv_pack_count_chunks(int T) { return T > 0 ? compact_chunks(T) : 0; }
+
+// The first fill of a store, everything that does not depend on the level counts in one call: empty the staging store,
+// count the levels chunk by chunk (the compaction needs those counts anyway), send the counts to the host (page-locked
+// memory, an event behind the copy) and quantise into the staging store.
 extern "C" int odmkv_quant_pack_staged(const void* K, const void* V, int dtype, int B, int Hkv, int T,
                                        int64_t stride_b, int64_t stride_h, int64_t stride_t,
                                        const int32_t* bits, int pos_offset,
@@ -1665,13 +1696,11 @@ extern "C" int odmkv_quant_pack_staged(const void* K, const void* V, int dtype, 
                                        void* workspace, size_t workspace_bytes, void* stream) {
     ODMKV_CHECK_ARG(staging && staging_arena && staging_tables_host && staging_offsets && counts_dev && counts_host && counts_event,
                     "quant_pack_staged: null pointer");
-    if (int rc = odmkv_level_counts(bits, B, Hkv, T, counts_dev, stream)) return rc;
-    ODMKV_CHECK_HIP(hipMemcpyAsync(counts_host, counts_dev, (size_t)B * Hkv * 6 * sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream));
-    ODMKV_CHECK_HIP(hipEventRecord((hipEvent_t)counts_event, (hipStream_t)stream));
+    ODMKV_CHECK_ARG(B > 0 && Hkv > 0 && T > 0, "quant_pack_staged: bad shape B=%d Hkv=%d T=%d", B, Hkv, T);
     if (int rc = odmkv_store_init(staging_arena, staging_tables_host, 5, B * Hkv + 1, staging_offsets, tables_end, counts_end, counts_end, stream))
         return rc;
-    return odmkv_quant_pack(K, V, dtype, B, Hkv, T, stride_b, stride_h, stride_t, bits, pos_offset, pi_k, pi_v, codebooks,
-                            staging, workspace, workspace_bytes, stream);
+    return quant_pack_impl(K, V, dtype, B, Hkv, T, stride_b, stride_h, stride_t, bits, pos_offset, pi_k, pi_v, codebooks,
+                           staging, workspace, workspace_bytes, stream, counts_dev, counts_host, counts_event);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -388,7 +388,8 @@ class TurboQuantAdaptiveKVCacheState:
         if _known_counts is not None:
             counts = np.asarray(_known_counts, np.int64).reshape(self._nseg, 6)
         elif staged:
-            box, box_dev, arrived, arrived_handle = _mailbox(dev, self._nseg * 6)
+            n_chunks = lib.odmkv_pack_count_chunks(T)                 # the counts arrive chunk by chunk
+            box, box_dev, arrived, arrived_handle = _mailbox(dev, self._nseg * n_chunks * 6)
             arrived.synchronize()                                     # (the last reader of the box is long done)
             stg = _staging_for(dev, st, B, H, T, self._exact_torch_dtype)
             ws = _lib.workspace(dev, ws_bytes, "pack")
@@ -403,7 +404,7 @@ class TurboQuantAdaptiveKVCacheState:
             if fresh and hint_key in _ARENA_HINT:
                 self._arena = torch.empty(_ARENA_HINT[hint_key], dtype=torch.uint8, device=dev)
             arrived.synchronize()                                     # the one wait: for the counts alone
-            counts = box[:self._nseg * 6].numpy().reshape(self._nseg, 6).astype(np.int64)
+            counts = box[:self._nseg * n_chunks * 6].numpy().reshape(self._nseg, n_chunks, 6).astype(np.int64).sum(axis=1)
         else:
             counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
             _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
