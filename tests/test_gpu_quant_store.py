@@ -233,6 +233,20 @@ def test_edge_cases_and_errors():
         st.prefill(k, k, torch.zeros(1, 2, 63, dtype=torch.int32, device=DEV))
     with pytest.raises(ValueError):
         st.prefill(k, k, torch.full((1, 2, 64), 5, dtype=torch.int32, device=DEV))
+    # the same on a first fill long enough to go through the staging store (its level counts come from the compaction's
+    # chunk counts): a value that is no level, a level the store was not built for; the store stays usable afterwards
+    k2 = torch.randn(1, 2, 2048 + 70, 128, generator=g).half().to(DEV)
+    good = torch.full((1, 2, 2048 + 70), 2, dtype=torch.int32, device=DEV)
+    good[0, 0, 100:300] = 4; good[0, 1, 2048:] = 16; good[0, 1, :9] = 0
+    for bad_value, levels in ((5, (0, 2, 3, 4, 8, 16)), (3, (0, 2, 4, 16))):
+        st = TurboQuantAdaptiveKVCacheState(128, levels, device=DEV, dtype=torch.float16, key_quantizer="mse", value_quantizer="mse", seed=42)
+        bad = good.clone(); bad[0, 1, 2050] = bad_value
+        with pytest.raises(ValueError):
+            st.prefill(k2, k2, bad)
+        st.prefill(k2, k2, good)
+        assert st.level_counts() == {0: 9, 2: 2 * 2118 - 200 - 70 - 9, 3: 0, 4: 200, 8: 0, 16: 70}
+        km, _ = st.materialize()
+        assert torch.equal(km[0, 1, 2048:], k2[0, 1, 2048:]) and torch.all(km[0, 1, :9] == 0)
     with pytest.raises(ValueError):
         TurboQuantAdaptiveKVCacheState(128, (0, 1, 4), device=DEV, key_quantizer="prod", value_quantizer="mse")
     with pytest.raises(NotImplementedError):
