@@ -204,6 +204,20 @@ int odmkv_store_init(void* arena, const int32_t* tables_host, int n_tables, int 
  * banks grow by torch.cat (kvquant/tq_adaptive_backend.py:46-52, 149-174). */
 int odmkv_store_gather(const odmkv_packed_t* staging, const odmkv_packed_t* store, void* stream);
 
+/* The other half of a staged first fill, in one call, once counts_event has arrived: the chunk counts (host memory,
+ * as odmkv_quant_pack_staged delivered them) are added up into counts (host int32 [B*Hkv, 6]); every segment gets a
+ * tile per 64 tokens, the exact segments `exact_slack` tokens of room to grow (seg_tile: host int32 [5][B*Hkv + 1],
+ * written); the store is laid out in `arena` (offsets, sizes, marks as odmkv_store_layout gives them), prepared
+ * (odmkv_store_init), described (odmkv_store_bind into `store`) and filled from the staging store
+ * (odmkv_store_gather).  need_bytes receives the size of the layout; if `arena` is NULL or smaller, nothing is
+ * launched and ODMKV_ENOSPACE returned: allocate and call again.  Counts that do not add up to B*Hkv*T (a value that
+ * is no level) give ODMKV_EINVAL.  No counterpart in the reference. */
+int odmkv_store_finish_staged(const int32_t* chunk_counts, int n_chunks, int B, int Hkv, int T,
+                              int exact_slack, int exact_dtype, void* arena, uint64_t arena_bytes,
+                              const odmkv_packed_t* staging, int32_t* counts, int32_t* seg_tile,
+                              uint64_t* offsets, uint64_t* sizes, uint64_t* marks,
+                              odmkv_packed_t* store, uint64_t* need_bytes, void* stream);
+
 /* The part of a store's first fill that does not depend on the level counts, in one call: the staging store emptied
  * (its tables as odmkv_store_layout gave them: staging_tables_host, staging_offsets, tables_end, counts_end), then
  * odmkv_quant_pack into it, whose first kernel counts the levels of every 2048-token chunk anyway: those counts go to

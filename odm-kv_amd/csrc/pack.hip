@@ -1789,6 +1789,49 @@ extern "C" int odmkv_store_gather(const odmkv_packed_t* staging, const odmkv_pac
     return 0;
 }
 
+// The second half of a staged first fill, in one call, for the moment the level counts have arrived: add up the chunks,
+// size every segment (a tile per 64 tokens; the exact segments with `exact_slack` tokens of room to grow), lay the store
+// out in `arena`, prepare it (odmkv_store_init), fill the descriptor and move the staging store's tiles over
+// (odmkv_store_gather).  What the host does between the arrival of the counts and the launch of the gather decides
+// whether the GPU runs dry behind the quantiser; here that is a few microseconds of arithmetic and two launches.
+extern "C" int odmkv_store_finish_staged(const int32_t* chunk_counts, int n_chunks, int B, int Hkv, int T,
+                                         int exact_slack, int exact_dtype, void* arena, uint64_t arena_bytes,
+                                         const odmkv_packed_t* staging, int32_t* counts, int32_t* seg_tile,
+                                         uint64_t* offsets, uint64_t* sizes, uint64_t* marks,
+                                         odmkv_packed_t* store, uint64_t* need_bytes, void* stream) {
+    ODMKV_CHECK_ARG(chunk_counts && staging && counts && seg_tile && offsets && sizes && marks && store && need_bytes,
+                    "store_finish_staged: null pointer");
+    ODMKV_CHECK_ARG(B > 0 && Hkv > 0 && T > 0 && n_chunks > 0 && exact_slack >= 0, "store_finish_staged: bad shape");
+    const int nseg = B * Hkv;
+    long long all = 0;
+    for (int s = 0; s < nseg; ++s)
+        for (int k = 0; k < 6; ++k) {
+            long long v = 0;
+            for (int c = 0; c < n_chunks; ++c) v += chunk_counts[((size_t)s * n_chunks + c) * 6 + k];
+            counts[s * 6 + k] = (int32_t)v;
+            all += v;
+        }
+    ODMKV_CHECK_ARG(all == (long long)nseg * T, "store_finish_staged: bits must take values in (0, 2, 3, 4, 8, 16)");
+    for (int li = 0; li < 5; ++li) {
+        int32_t* row = seg_tile + (size_t)li * (nseg + 1);
+        row[0] = 0;
+        for (int s = 0; s < nseg; ++s) {
+            const long long n = (long long)counts[s * 6 + li + 1] + (li == 4 ? exact_slack : 0);
+            row[s + 1] = row[s] + (int32_t)((n + TILE - 1) / TILE);
+        }
+    }
+    if (int rc = odmkv_store_layout(seg_tile, nseg, offsets, sizes, marks)) return rc;
+    *need_bytes = marks[4];
+    if (arena == nullptr || arena_bytes < marks[4]) {
+        odmkv_set_error("store_finish_staged: the store needs %llu bytes, the allocation has %llu",
+                        (unsigned long long)marks[4], (unsigned long long)arena_bytes);
+        return ODMKV_ENOSPACE;
+    }
+    if (int rc = odmkv_store_init(arena, seg_tile, 5, nseg + 1, offsets, marks[0], marks[2], marks[3], stream)) return rc;
+    if (int rc = odmkv_store_bind(arena, offsets, seg_tile, nseg, B, Hkv, exact_dtype, store)) return rc;
+    return odmkv_store_gather(staging, store, stream);
+}
+
 // ------------------------------------------------------------------------------------------------
 // dequantise to dense tensors
 // ------------------------------------------------------------------------------------------------

@@ -76,6 +76,20 @@ class _Layout:
         _lib.check(lib.odmkv_store_layout(self.tables_ptr, nseg, self.offsets, self.sizes, marks))
         self.tables_end, self.counts_end, self.zero_end, self.pos_end, self.total = (int(m) for m in marks)
 
+    @classmethod
+    def blank(cls, nseg: int) -> "_Layout":
+        """Arrays for odmkv_store_finish_staged to fill; `adopt` reads the marks afterwards."""
+        self = cls.__new__(cls)
+        self.tables = np.zeros((5, nseg + 1), np.int32)
+        self.tables_ptr = self.tables.ctypes.data
+        self.nseg = nseg
+        self.offsets, self.sizes, self.marks = _U64x33(), _U64x33(), _U64x5()
+        return self
+
+    def adopt(self) -> "_Layout":
+        self.tables_end, self.counts_end, self.zero_end, self.pos_end, self.total = (int(m) for m in self.marks)
+        return self
+
     def init(self, arena: torch.Tensor, stream: int, counts_only: bool = False) -> None:
         """Tables written, counters / norms / exact rows cleared, positions -1 (counts_only: just the tables and
         the segment counts): one launch, the tables in its arguments."""
@@ -404,7 +418,23 @@ class TurboQuantAdaptiveKVCacheState:
             if fresh and hint_key in _ARENA_HINT:
                 self._arena = torch.empty(_ARENA_HINT[hint_key], dtype=torch.uint8, device=dev)
             arrived.synchronize()                                     # the one wait: for the counts alone
-            counts = box[:self._nseg * n_chunks * 6].numpy().reshape(self._nseg, n_chunks, 6).astype(np.int64).sum(axis=1)
+            # what remains up to the launch of the gather is one call (the GPU has the quantiser's run to wait for it)
+            new_lay, new_packed, counts32 = _Layout.blank(self._nseg), Packed(), np.zeros((self._nseg, 6), np.int32)
+            need = C.c_uint64(0)
+            for attempt in (0, 1):
+                arena = getattr(self, "_arena", None)
+                rc = lib.odmkv_store_finish_staged(
+                    box.data_ptr(), n_chunks, B, H, T, int(self.exact_slack),
+                    _lib.BF16 if self._exact_torch_dtype == torch.bfloat16 else _lib.F16,
+                    None if arena is None else arena.data_ptr(), 0 if arena is None else arena.numel(),
+                    C.byref(stg.packed), counts32.ctypes.data, new_lay.tables_ptr, new_lay.offsets, new_lay.sizes,
+                    new_lay.marks, C.byref(new_packed), C.byref(need), st)
+                if rc != -2 or attempt == 1:
+                    break
+                self._arena = torch.empty(int(need.value) + int(need.value) // 8, dtype=torch.uint8, device=dev)
+                self._arena_spare = None
+            _lib.check(rc)
+            counts = counts32.astype(np.int64)
         else:
             counts_dev = torch.empty(self._nseg, 6, dtype=torch.int32, device=dev)
             _lib.check(lib.odmkv_level_counts(bits.data_ptr(), B, H, T, counts_dev.data_ptr(), st))
@@ -421,12 +451,16 @@ class TurboQuantAdaptiveKVCacheState:
         if not present <= set(self.bit_levels):
             raise ValueError(f"bits use levels {sorted(present - set(self.bit_levels))} outside bit_levels={self.bit_levels}")
         new_counts = self._counts + counts[:, 1:].T
-        self._ensure_capacity(new_counts)
+        if stg is not None:
+            # laid out, prepared and filled by odmkv_store_finish_staged above
+            self._bufs = _Buffers(self._arena, new_lay.adopt(), self._exact_torch_dtype)
+            self._seg_tile = new_lay.tables.astype(np.int64)
+            self._packed = new_packed
+        else:
+            self._ensure_capacity(new_counts)
         if fresh:
             _ARENA_HINT[hint_key] = self._arena.numel()
-        if stg is not None:
-            _lib.check(lib.odmkv_store_gather(C.byref(stg.packed), C.byref(self._packed), st))
-        else:
+        if stg is None:
             ws = _lib.workspace(dev, ws_bytes, "pack")
             _lib.check(lib.odmkv_quant_pack(
                 keys.data_ptr(), values.data_ptr(), _lib.dtype_code(keys), B, H, T,
