@@ -159,3 +159,43 @@ def test_store_layout_and_bind_are_host_arithmetic(lib):
     lib.odmkv_last_error.restype = C.c_char_p
     assert lib.odmkv_store_bind(base, (C.c_uint64 * 33)(*off), seg_tile.ctypes.data, nseg, B, H + 1, 0, C.byref(p)) == -1
     assert b"store_bind" in lib.odmkv_last_error()
+
+
+def test_store_finish_staged_sizes_the_store_without_a_gpu(lib):
+    """With no allocation to lay the store out in, odmkv_store_finish_staged launches nothing: it adds up the chunk
+    counts, sizes the segments (a tile per 64 tokens, the exact segments with room to grow), reports the bytes the
+    layout needs and returns ODMKV_ENOSPACE; counts that do not add up to every token are refused."""
+    import numpy as np
+    from kvquant._lib import Packed
+    B, H, T, n_chunks, slack = 1, 3, 5000, 3, 256
+    nseg = B * H
+    rng = np.random.default_rng(9)
+    per_seg = np.zeros((nseg, 6), np.int64)
+    for s in range(nseg):
+        cut = np.sort(rng.integers(0, T + 1, size=5))
+        per_seg[s] = np.diff(np.concatenate([[0], cut, [T]]))
+    per_seg[1, 2] += per_seg[1, 3]; per_seg[1, 3] = 0                 # a level nobody uses in one segment
+    chunks = np.zeros((nseg, n_chunks, 6), np.int32)
+    for s in range(nseg):
+        for k in range(6):
+            parts = rng.multinomial(per_seg[s, k], [1 / n_chunks] * n_chunks)
+            chunks[s, :, k] = parts
+    counts = np.zeros((nseg, 6), np.int32)
+    seg_tile = np.zeros((5, nseg + 1), np.int32)
+    off, size, marks = (C.c_uint64 * 33)(), (C.c_uint64 * 33)(), (C.c_uint64 * 5)()
+    staging, store, need = Packed(), Packed(), C.c_uint64(0)
+    f = lib.odmkv_store_finish_staged
+    f.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_uint64, C.POINTER(Packed),
+                  C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Packed), C.c_void_p, C.c_void_p]
+    rc = f(chunks.ctypes.data, n_chunks, B, H, T, slack, 0, None, 0, C.byref(staging), counts.ctypes.data,
+           seg_tile.ctypes.data, off, size, marks, C.byref(store), C.byref(need), None)
+    assert rc == -2 and b"needs" in lib.odmkv_last_error()
+    assert np.array_equal(counts, per_seg)
+    want = (per_seg[:, 1:].T + 63) // 64
+    want[4] = (per_seg[:, 5] + slack + 63) // 64
+    assert np.array_equal(np.diff(seg_tile, axis=1), want) and np.all(seg_tile[:, 0] == 0)
+    assert need.value == marks[4] > 0
+    chunks[2, 1, 4] += 1                                               # one token too many
+    rc = f(chunks.ctypes.data, n_chunks, B, H, T, slack, 0, None, 0, C.byref(staging), counts.ctypes.data,
+           seg_tile.ctypes.data, off, size, marks, C.byref(store), C.byref(need), None)
+    assert rc == -1 and b"must take values" in lib.odmkv_last_error()
