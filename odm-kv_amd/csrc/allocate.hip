@@ -97,7 +97,7 @@ __device__ static inline int wave_sum_int(int v) {
 // ---- clear counters, set up the bracket ----
 __global__ void alloc_init_kernel(AllocArgs a) {
     const int row = blockIdx.x;
-    if (a.level_counts && threadIdx.x < a.K) a.level_counts[row * a.K + threadIdx.x] = 0;
+    if (a.level_counts && (int)threadIdx.x < a.K) a.level_counts[row * a.K + threadIdx.x] = 0;
     if (threadIdx.x == 0) {
         RowState& st = a.state[row];
         double t = a.target[row];                    // clamp the budget into the level range
@@ -651,7 +651,7 @@ __global__ __launch_bounds__(EV_THREADS) void alloc_write_kernel(AllocArgs a, in
         }
     }
     __syncthreads();
-    if (a.level_counts && threadIdx.x < a.K && lh[threadIdx.x])
+    if (a.level_counts && (int)threadIdx.x < a.K && lh[threadIdx.x])
         atomicAdd(&a.level_counts[row * a.K + threadIdx.x], lh[threadIdx.x]);
 }
 
