@@ -49,7 +49,7 @@ const char* odmkv_last_error(void);
  *   s[h, 0..n_sink) = max over all (h, t >= n_sink) of s
  *
  * K, V: [Hkv, T, 128] of `dtype`, element strides (stride_h, stride_t), innermost contiguous.
- * mu: device fp32 [Hq, 128] (the RoPE-averaged mean query; Hq = G * Hkv).
+ * mu: device fp32 [Hq, 128], 16-byte aligned (the RoPE-averaged mean query; Hq = G * Hkv).
  * attn: NULL, or device fp32 [Hkv, T] attention weights to use instead of computing p from mu
  *       (then n_sink must be 0 and no sink padding happens: score_with_attn).
  * scores: device fp32 [Hkv, T] out.

@@ -1026,6 +1026,7 @@ extern "C" int odmkv_score_model_dtype(const void* K, const void* V, int dtype, 
     ODMKV_CHECK_ARG(stride_h % align == 0 && stride_t % align == 0 && stride_t >= HD,
                     "score: strides must keep rows 16-byte aligned");
     ODMKV_CHECK_ARG(((uintptr_t)K & 15) == 0 && ((uintptr_t)V & 15) == 0, "score: K/V must be 16-byte aligned");
+    ODMKV_CHECK_ARG(((uintptr_t)mu & 15) == 0, "score: the mean queries must be 16-byte aligned");
     ODMKV_CHECK_ARG(workspace_bytes >= odmkv_score_workspace_bytes(Hkv, Hq, T), "score: workspace too small");
     const ScoreLayout L = score_layout(Hkv, Hq, T);
     char* ws = (char*)workspace;
