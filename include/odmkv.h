@@ -368,7 +368,8 @@ int odmkv_flush_rank(const float* scores, const float* minmax, int B, int H, int
  * compute units).
  * wavefronts: wavefronts of the workgroup that runs an item: 8 (0 means 8), 12 or 16.  Eight start and finish
  * faster and suit items of fewer than sixteen tiles; sixteen stream long 2- and 3-bit items about 1.1 times
- * faster; twelve (three units in flight per wavefront) are 5 % ahead where 4- and 8-bit tokens carry the bytes.
+ * faster; twelve (three units in flight per wavefront) are 5 % ahead where 4- and 8-bit tokens carry the bytes, and
+ * 2 % ahead of eight on items of 6 to 15 tiles of 3 bits and wider.
  * Two launches per call (main kernel, merge); the workspace holds the per-item partial results.
  */
 typedef struct odmkv_worklist {
