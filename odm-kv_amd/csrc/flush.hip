@@ -122,6 +122,7 @@ __global__ __launch_bounds__(FLUSH_THREADS) void flush_score_kernel(FlushScoreAr
     __syncthreads();
     const float inv_p = 1.0f / fmaxf((red[0] + red[1]) + (red[2] + red[3]), 1e-8f);
     float lo = INFINITY, hi = -INFINITY;
+    bool nan_seen = false;          // a NaN score makes the whole flush's range NaN, as torch's min() / max() do
     if (a.mode == 0) {
         // pass 2: o = sum_t p_hat_t v_t
         float o[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -157,6 +158,7 @@ __global__ __launch_bounds__(FLUSH_THREADS) void flush_score_kernel(FlushScoreAr
                 const float sc = (pe * pe) * (vn2[t] + (kn2[t] * (1.0f / (float)HD)) * ir);
                 a.scores[(size_t)bh * a.n + t] = sc;
                 lo = fminf(lo, sc); hi = fmaxf(hi, sc);
+                nan_seen |= sc != sc;
             }
         }
     } else {
@@ -164,15 +166,18 @@ __global__ __launch_bounds__(FLUSH_THREADS) void flush_score_kernel(FlushScoreAr
             const float sc = (lg[t] * lg[t]) * vn2[t];
             a.scores[(size_t)bh * a.n + t] = sc;
             lo = fminf(lo, sc); hi = fmaxf(hi, sc);
+            nan_seen |= sc != sc;
         }
     }
     lo = -wave_max(-lo); hi = wave_max(hi);
+    if (__builtin_amdgcn_ballot_w64(nan_seen) != 0) { lo = NAN; hi = NAN; }       // (fminf / fmaxf drop NaN operands)
     __syncthreads();
     if (lane == 0) { red[wave] = lo; red2[wave] = hi; }
     __syncthreads();
     if (tid == 0) {
-        a.minmax[2 * bh] = fminf(fminf(red[0], red[1]), fminf(red[2], red[3]));
-        a.minmax[2 * bh + 1] = fmaxf(fmaxf(red2[0], red2[1]), fmaxf(red2[2], red2[3]));
+        const bool bad = red[0] != red[0] || red[1] != red[1] || red[2] != red[2] || red[3] != red[3];
+        a.minmax[2 * bh] = bad ? NAN : fminf(fminf(red[0], red[1]), fminf(red[2], red[3]));
+        a.minmax[2 * bh + 1] = bad ? NAN : fmaxf(fmaxf(red2[0], red2[1]), fmaxf(red2[2], red2[3]));
     }
 }
 
@@ -198,21 +203,32 @@ extern "C" int odmkv_flush_score(const void* K, const void* V, int dtype, int BH
 // sequences, row after row) are sorted ascending, equal scores in index order, and the token of rank r gets
 // by_rank[h][r] (adaptive_backend_press.py:198-241 with the shares cached at prefill).
 // One workgroup per kv-head, a bitonic sort of (score, index) pairs in LDS.
+// Scores that are not finite follow torch: a NaN anywhere in the flush makes the range NaN and every key 0.5 (ranks in
+// index order); an infinite score makes the spread infinite, its own key NaN and every finite key 0; NaN keys sort
+// behind every number, among themselves in index order.  The keys are compared as integers whose order is that of the
+// floats with NaN on top and the sort's padding above NaN, so the comparison is a total order whatever the scores.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(FLUSH_THREADS) void flush_rank_kernel(const float* scores, const float* minmax, int B, int H,
                                                                    int n, const int32_t* by_rank, int32_t* bits) {
-    __shared__ float key[RANK_MAX_TOKENS];
+    __shared__ uint32_t key[RANK_MAX_TOKENS];
     __shared__ uint32_t idx[RANK_MAX_TOKENS];
     __shared__ float red[FLUSH_THREADS / 64], red2[FLUSH_THREADS / 64];
     const int h = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     float lo = INFINITY, hi = -INFINITY;
-    for (int i = tid; i < B * H; i += FLUSH_THREADS) { lo = fminf(lo, minmax[2 * i]); hi = fmaxf(hi, minmax[2 * i + 1]); }
+    bool nan_seen = false;
+    for (int i = tid; i < B * H; i += FLUSH_THREADS) {
+        const float l = minmax[2 * i], u = minmax[2 * i + 1];
+        nan_seen |= l != l || u != u;
+        lo = fminf(lo, l); hi = fmaxf(hi, u);
+    }
     lo = -wave_max(-lo); hi = wave_max(hi);
+    if (__builtin_amdgcn_ballot_w64(nan_seen) != 0) { lo = NAN; hi = NAN; }
     if (lane == 0) { red[wave] = lo; red2[wave] = hi; }
     __syncthreads();
+    const bool bad = red[0] != red[0] || red[1] != red[1] || red[2] != red[2] || red[3] != red[3];
     lo = fminf(fminf(red[0], red[1]), fminf(red[2], red[3]));
     hi = fmaxf(fmaxf(red2[0], red2[1]), fmaxf(red2[2], red2[3]));
-    const float spread = hi - lo;
+    const float spread = bad ? NAN : hi - lo;               // NaN: the comparison below fails and every key is 0.5
     const int N = B * n;
     int P = 1;
     while (P < N) P <<= 1;
@@ -220,9 +236,11 @@ __global__ __launch_bounds__(FLUSH_THREADS) void flush_rank_kernel(const float* 
         if (i < N) {
             const int b = i / n, t = i % n;
             const float x = scores[((size_t)b * H + h) * n + t];
-            key[i] = spread > 1e-8f ? (x - lo) / fmaxf(spread, 1e-30f) : 0.5f;
+            const float y = (spread > 1e-8f ? (x - lo) / fmaxf(spread, 1e-30f) : 0.5f) + 0.0f;      // (-0 -> +0)
+            const uint32_t u = __float_as_uint(y);
+            key[i] = y != y ? 0xfffffffeu : (u & 0x80000000u) ? ~u : (u | 0x80000000u);
         } else {
-            key[i] = INFINITY;
+            key[i] = 0xffffffffu;                          // padding: above every token, NaN keys included
         }
         idx[i] = (uint32_t)i;
     }
@@ -233,7 +251,7 @@ __global__ __launch_bounds__(FLUSH_THREADS) void flush_rank_kernel(const float* 
                 const int l = i ^ j;
                 if (l > i) {
                     const bool up = (i & k) == 0;
-                    const float a0 = key[i], a1 = key[l];
+                    const uint32_t a0 = key[i], a1 = key[l];
                     const uint32_t i0 = idx[i], i1 = idx[l];
                     const bool gt = a0 > a1 || (a0 == a1 && i0 > i1);       // (score, index) pairs: a total order, so the sort is stable
                     if (gt == up) { key[i] = a1; key[l] = a0; idx[i] = i1; idx[l] = i0; }
@@ -244,7 +262,7 @@ __global__ __launch_bounds__(FLUSH_THREADS) void flush_rank_kernel(const float* 
     }
     for (int r = tid; r < N; r += FLUSH_THREADS) {
         const int i = (int)idx[r], b = i / n, t = i % n;
-        bits[((size_t)b * H + h) * n + t] = by_rank[(size_t)h * N + r];
+        if (i < N) bits[((size_t)b * H + h) * n + t] = by_rank[(size_t)h * N + r];      // (always: the padding sorts last)
     }
 }
 

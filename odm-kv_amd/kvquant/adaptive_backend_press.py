@@ -407,26 +407,31 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
     def _by_rank_table(self, layer_idx: int, num_heads: int, n_tok: int, device):
         """(device int32 [H, n_tok]: level of every rank per kv-head, host int64 [H, 6]: tokens per level 0, 2, 3, 4, 8,
         16) from the shares cached at prefill, as `_allocate_bits_via_cached_ratios` forms them; None when a head
-        has no usable shares.  Kept per (layer, n_tok)."""
+        has no usable shares.  Kept per layer; the entry is keyed by the shares it was expanded from, so a press
+        that sees another prompt (whose prefill overwrites the shares) never flushes with the old prompt's table."""
         import numpy as np
-        cache = self.__dict__.setdefault("_by_rank_cache", {})
-        key = (layer_idx, num_heads, n_tok, str(device))
-        if key in cache:
-            return cache[key]
         allowed = set(self._decode_bit_levels)
-        rows = []
+        shares = []
         for h in range(num_heads):
             got = self._observed_ratios.get((layer_idx, h))
-            kept = [(b, r) for b, r in (got or ()) if b in allowed and r > 0]
+            kept = tuple((b, r) for b, r in (got or ()) if b in allowed and r > 0)
             if not kept:
                 return None
+            shares.append(kept)
+        cache = self.__dict__.setdefault("_by_rank_cache", {})
+        slot, key = (layer_idx, str(device)), (num_heads, n_tok, tuple(shares))
+        hit = cache.get(slot)
+        if hit is not None and hit[0] == key:
+            return hit[1]
+        rows = []
+        for kept in shares:
             total = sum(r for _, r in kept)
             levels, ratios = zip(*[(b, r / total) for b, r in kept])
             rows.append(_levels_by_rank(levels, ratios, n_tok))
         by_rank = np.stack(rows)
         counts = np.stack([(by_rank == b).sum(axis=1) for b in _lib.LEVEL_ORDER], axis=1).astype(np.int64)
-        cache[key] = (torch.from_numpy(by_rank).to(device), counts)
-        return cache[key]
+        cache[slot] = (key, (torch.from_numpy(by_rank).to(device), counts))      # one entry per layer: the old table goes
+        return cache[slot][1]
 
     @torch.no_grad()
     def _flush_query(self, module: nn.Module, hidden_states, state) -> Optional[torch.Tensor]:

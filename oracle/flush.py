@@ -76,7 +76,9 @@ def flush_scores(buf_keys: torch.Tensor, buf_values: torch.Tensor, attn: Optiona
 
 
 def minmax(scores: torch.Tensor) -> torch.Tensor:
-    """adaptive_backend_press.py:531-536."""
+    """adaptive_backend_press.py:531-536.  Scores that are not finite go through torch's own rules: a NaN makes
+    min() and max() NaN, the comparison below fails and every score becomes 0.5; an infinite score makes the range
+    infinite, itself NaN and every finite score 0.  The stable sort of the ranking puts NaN behind every number."""
     lo, hi = scores.min(), scores.max()
     if hi - lo > 1e-8:
         return (scores - lo) / (hi - lo)

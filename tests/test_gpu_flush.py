@@ -58,6 +58,28 @@ def test_flush_score_matches_oracle(B, H, n, dtype):
     np.testing.assert_allclose(plain.reshape(-1).cpu().numpy(), want_plain.numpy(), rtol=1e-4, atol=1e-12)
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+def test_flush_score_range_carries_a_nan(mode):
+    """A NaN among the buffered values gives NaN scores; the range the kernel reports for that head must say so
+    (torch's min() / max() in the reference's normalisation return NaN then), and the ranking that follows must
+    still give every token a level: the whole chain on one poisoned buffer."""
+    g = torch.Generator().manual_seed(31)
+    B, H, n = 1, 2, 64
+    k = torch.randn(B, H, n, 128, generator=g).half()
+    v = torch.randn(B, H, n, 128, generator=g).half()
+    v[0, 1, 7, 3] = float("nan")
+    q = torch.randn(B, H, 128, generator=g).half()
+    _, scores, minmax = _score(k.to(DEV), v.to(DEV), q.to(DEV), 1e-2, mode)
+    mm = minmax.cpu()
+    assert torch.isnan(scores.reshape(B, H, n)[0, 1]).any()
+    assert torch.isnan(mm[1]).all() and torch.isfinite(mm[0]).all()
+    observed = {h: ((2, 0.5), (4, 0.5)) for h in range(H)}
+    got = _rank(scores, minmax, B, H, n, observed, {2, 4, 16}).cpu()
+    want = ofl.cached_ratio_bits(ofl.minmax(scores.reshape(-1).cpu()), _positions(B, H, n), H, observed, (2, 4, 16))
+    assert torch.equal(got.reshape(-1), want)                # all keys 0.5: index order, the first half 2 bits
+    assert got[0, 0].tolist() == [2] * 32 + [4] * 32
+
+
 def _rank(scores, minmax, B, H, n, observed, allowed):
     from kvquant import _lib
     from kvquant.adaptive_backend_press import _levels_by_rank
@@ -75,7 +97,8 @@ def _rank(scores, minmax, B, H, n, observed, allowed):
 
 
 @pytest.mark.parametrize("B,H,n,kind", [(1, 8, 128, "random"), (4, 3, 100, "random"), (2, 2, 64, "ties"), (1, 2, 33, "flat"),
-                                        (8, 1, 512, "random"), (1, 1, 1, "random")])
+                                        (8, 1, 512, "random"), (1, 1, 1, "random"), (2, 2, 37, "nan"), (1, 3, 100, "inf"),
+                                        (2, 2, 37, "neginf"), (1, 2, 3, "inf")])
 def test_flush_rank_matches_oracle_bit_for_bit(B, H, n, kind):
     g = torch.Generator().manual_seed(B * 77 + n)
     scores = torch.rand(B, H, n, generator=g) * 3.0 + 0.5
@@ -83,6 +106,18 @@ def test_flush_rank_matches_oracle_bit_for_bit(B, H, n, kind):
         scores = (scores * 4).round() / 4                                       # many equal scores across sequences
     if kind == "flat":
         scores = torch.full((B, H, n), 2.0) + torch.rand(B, H, n, generator=g) * 1e-9      # range below the 1e-8 floor
+    # scores that are not finite (a NaN or inf in the buffered rows or the query): torch's min / max / sort set the rule
+    # (a NaN makes every normalised score 0.5, an inf makes its own NaN and the finite ones 0, NaN sorts last), and
+    # every token still gets a level of its head's table
+    if kind == "nan":
+        scores[0, 1, 5] = float("nan")
+        scores[-1, 0, n - 1] = float("nan")
+    if kind == "inf":
+        scores[0, 0, 1] = float("inf")
+        scores[0, H - 1, 0] = float("inf")
+        scores[0, H - 1, n - 1] = float("inf")
+    if kind == "neginf":
+        scores[0, 0, 3] = float("-inf")
     observed = {h: ((0, 0.3), (2, 0.4), (3, 0.1 + 0.01 * h), (4, 0.15), (8, 0.05)) for h in range(H)}
     allowed = (2, 3, 4, 8, 16)
     s_dev = scores.to(DEV).contiguous()

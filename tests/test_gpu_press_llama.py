@@ -423,3 +423,46 @@ def test_flush_levels_match_the_oracle(path):
         lm = r["levels"]
         assert (lm[r["pos"][:, 1], r["pos"][:, 2]] == r["bits"].numpy()).all()
         assert not (r["bits"] == 0).any()                 # no decode-time eviction
+
+
+@torch.inference_mode()
+def test_second_prompt_through_one_press_flushes_with_its_own_shares():
+    """One press object, two prompts with different budgets: the device flush of the second prompt must rank
+    with the level shares of the second prefill (the expanded rank table is cached per layer), exactly as
+    the oracle does on the same scores and as the general torch path does."""
+    from transformers import DynamicCache
+    from oracle import flush as ofl
+    model = _model(9)
+    T, n_buf = 500, 128
+    forced = torch.randint(0, 1000, (n_buf + 2,), generator=torch.Generator().manual_seed(72)).to(DEV)
+    press = _press(target=2.2)
+    press.record_flush = True
+    seen = []
+    orig_flush = press._flush_decode_buffer
+
+    def spy_flush(state, layer_idx, cache, module, hidden_states=None):
+        pos = state.get_buffer_tokens(press._buffer_start_seqs[layer_idx])[0].cpu().numpy()
+        observed = {h: press._observed_ratios[(layer_idx, h)] for h in range(state.num_heads)}
+        press.last_flush = None
+        orig_flush(state, layer_idx, cache, module, hidden_states)
+        lf = press.last_flush
+        assert lf is not None and lf["layer"] == layer_idx, "the device path was not taken"
+        raw = lf["scores"].reshape(-1).float()
+        scores = ((raw - raw.min()) / (raw.max() - raw.min()).clamp_min(1e-30)).cpu()
+        want = ofl.cached_ratio_bits(scores, pos, 2, observed, (2, 3, 4, 8, 16))
+        assert torch.equal(lf["bits"].reshape(-1).cpu(), want), f"layer {layer_idx}, prompt {len(seen) // 2}"
+        seen.append((layer_idx, observed, lf["bits"].reshape(-1).cpu()))
+
+    press._flush_decode_buffer = spy_flush
+    for prompt, target in enumerate((2.2, 5.0)):
+        press.target_avg_bits = target
+        cache = DynamicCache()
+        with press(model):
+            model.model(input_ids=_ids(T, 70 + prompt), past_key_values=cache)
+            for step in range(forced.shape[0]):
+                model(input_ids=forced[step].view(1, 1), past_key_values=cache, position_ids=torch.tensor([[T + step]], device=DEV))
+    assert [s[0] for s in seen] == [0, 1, 0, 1]
+    for layer in (0, 1):
+        first, second = seen[layer], seen[2 + layer]
+        assert first[1] != second[1]                              # the two prefills left different shares ...
+        assert sorted(first[2].tolist()) != sorted(second[2].tolist())       # ... and the flushes different tier sizes

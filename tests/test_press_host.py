@@ -103,6 +103,31 @@ def test_observed_ratios_and_cached_allocation():
         assert torch.equal(p._allocate_bits_via_cached_ratios(scores, pos, H, 3, allowed, batch_size=B), loop)
 
 
+def test_rank_table_follows_the_shares_of_the_latest_prefill():
+    """A press object that is used for a second prompt must flush with the second prompt's level shares:
+    the expanded rank table is cached, and the cache has to notice that the shares changed."""
+    from kvquant import TurboQuantPerTokenBackendPress
+    p = TurboQuantPerTokenBackendPress(scorer=_scorer(), bit_levels=(0, 2, 4, 16), key_quantizer="mse",
+                                       value_quantizer="mse", target_avg_bits=2.0, sink_tokens=4, buffer_size=8)
+    p._decode_bit_levels = {2, 4, 16}
+    T = 4 + 40 + 8
+
+    def prompt(n2):
+        bits = torch.full((1, 1, T), 16, dtype=torch.int32)
+        bits[0, 0, 4:44] = torch.tensor([2] * n2 + [4] * (40 - n2))
+        p._record_observed_ratios(0, bits)
+
+    prompt(30)
+    table, counts = p._by_rank_table(0, 1, 16, "cpu")
+    assert table[0].tolist() == [2] * 12 + [4] * 4 and counts[0].tolist() == [0, 12, 0, 4, 0, 0]
+    assert p._by_rank_table(0, 1, 16, "cpu")[0] is table            # same shares: the cached table
+    prompt(10)                                                      # the next prompt: 25 % / 75 %
+    table2, counts2 = p._by_rank_table(0, 1, 16, "cpu")
+    assert table2[0].tolist() == [2] * 4 + [4] * 12 and counts2[0].tolist() == [0, 4, 0, 12, 0, 0]
+    p._decode_bit_levels = {4, 16}                                  # and another set of allowed levels
+    assert p._by_rank_table(0, 1, 16, "cpu")[0][0].tolist() == [4] * 16
+
+
 def test_backend_press_rejects_unbuilt_quantisers():
     from kvquant import TurboQuantBackendPress
     with pytest.raises(NotImplementedError):
