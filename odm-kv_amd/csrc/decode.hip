@@ -29,6 +29,7 @@
 // The LDS table is replicated over 32 slots (slot = lane % 32) so that lanes never share a bank.
 // All softmax state is kept in base-2 logarithms.
 #include "decode.h"
+#include <stdlib.h>
 
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
@@ -469,6 +470,131 @@ __device__ static inline void compute_unit(const Unit<W>& t, int nvalid, int lan
     wave_lds_fence();                                      // the p buffer is free for the next unit
 }
 
+// ---- groups of up to four query heads, long work items (decode_main_kernel<4, ., 16, true>) -----------------------
+// Four heads need 8 of the 16 matrix rows.  The general form leaves rows 8..15 empty and every lane of wave rows 2, 3
+// (lanes 32..63) then runs the softmax step on heads that do not exist.  Here rows 8..15 repeat rows 0..7
+// (load_queries_g4) and the two token blocks of a unit share the lanes out between them: after the key products lane
+// (n, j) of rows j < 2 keeps block 0's logits of slot pair_slot(n) for heads 2j, 2j+1, and a lane of rows j >= 2 keeps
+// block 1's logits of slot pair_slot(n) + 1 for heads 2(j-2), 2(j-2)+1: one slot and two heads per lane, every lane with
+// work of its own, half the softmax instructions.  The value product reads p of head (n & 3) for every row n, so all
+// four row groups accumulate the same 4 heads x 128 dims (acc[m][r] = head r, dim 16m + n).
+// While a work item runs, st.mA / st.mB hold the reference points minus P_SHIFT (the form the loop subtracts) and
+// st.lA / st.lB this lane's own share of the normalisers; g4_finish puts them into the form the combine expects.
+#define G4_PROW 80          // bytes per head row of the p buffer: 32 x 16 bit + 16 (rows on different banks)
+template <int W>
+struct Unit4 {
+    uint32_t kw[2 * W];
+    uint32_t vw[2 * W];
+    float kn, vn;           // of the lane's one slot
+};
+template <int W>
+__device__ static inline void load_unit4(Unit4<W>& t, const DecodeArgs& a, int li, int unit, int lane) {
+    const int tile = unit >> 1, h = unit & 1;               // wave-uniform
+    load_half_stream<W>(t.kw, a.s.kcodes[li] + (size_t)tile * (TILE * 16 * W), h, lane);
+    load_half_stream<W>(t.vw, a.s.vcodes[li] + (size_t)tile * (TILE * 16 * W), h, lane);
+    const size_t slot = (size_t)unit * UNIT + pair_slot(lane & 15) + (lane >> 5);
+    t.kn = __builtin_nontemporal_load(a.s.knorm[li] + slot);
+    t.vn = __builtin_nontemporal_load(a.s.vnorm[li] + slot);
+}
+template <int W>
+__device__ static inline void compute_unit_g4(const Unit4<W>& t, int nvalid, int lane, const uint8_t* lut,
+                                              uint32_t slot4, const h8* qa, float ksc, float vsc,
+                                              uint8_t* pbuf, WaveState& st) {
+    const int n = lane & 15, j = lane >> 4;
+    f4 dk[2];
+    dk[0] = (f4){0.f, 0.f, 0.f, 0.f};
+    dk[1] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            if constexpr (W == 8) {
+                h8 chi, clo;
+                lut8_split(t.kw, 4 * b + kb, lut, slot4, chi, clo);
+                dk[b] = MFMA_F16(qa[kb], chi, dk[b]);
+                dk[b] = MFMA_F16(qa[kb], clo, dk[b]);
+            } else {
+                dk[b] = MFMA_F16(qa[kb], lut8<W>(t.kw, 4 * b + kb, lut, slot4), dk[b]);
+            }
+        }
+    // high + low row sums; rows 2, 3 of the wave take block 1's (a DPP move that writes those rows only)
+    const float kn = t.kn * ksc;
+    float tA = dk[0][0] + dk[0][1], tB = dk[0][2] + dk[0][3];
+    {
+        const float uA = dk[1][0] + dk[1][1], uB = dk[1][2] + dk[1][3];
+        tA = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(tA), __float_as_int(uA), 0xe4, 0xc, 0xf, false));
+        tB = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(tB), __float_as_int(uB), 0xe4, 0xc, 0xf, false));
+    }
+    tA *= kn; tB *= kn;
+    const int slot = pair_slot(n) + (j >> 1);
+    if (nvalid < UNIT) {                                   // the last unit of a run (wave-uniform)
+        const bool ok = slot < nvalid;
+        tA = ok ? tA : -INFINITY;
+        tB = ok ? tB : -INFINITY;
+    }
+    float xA = tA - st.mA, xB = tB - st.mB;
+    if (__builtin_amdgcn_ballot_w64(fmaxf(xA, xB) > SOFTMAX_SLACK + P_SHIFT) != 0) {      // wave-uniform; always on the first unit
+        float mxA = tA, mxB = tB;
+        row_max2(mxA, mxB);
+        mxA = fmaxf(mxA, __shfl_xor(mxA, 32, WAVE));       // the same heads live in rows j and j ^ 2
+        mxB = fmaxf(mxB, __shfl_xor(mxB, 32, WAVE));
+        const float nA = fmaxf(st.mA, mxA - P_SHIFT), nB = fmaxf(st.mB, mxB - P_SHIFT);
+        if (__builtin_amdgcn_ballot_w64(st.mA > -INFINITY || st.mB > -INFINITY) != 0) {     // not the wave's first unit
+            const float aA = st.mA > -INFINITY ? __builtin_amdgcn_exp2f(st.mA - nA) : 0.0f;
+            const float aB = st.mB > -INFINITY ? __builtin_amdgcn_exp2f(st.mB - nB) : 0.0f;
+            st.lA *= aA; st.lB *= aB;
+            f4 al;                                          // heads 0, 1 sit in row 0 of the wave, heads 2, 3 in row 1
+            al[0] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(aA), 0));
+            al[1] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(aB), 0));
+            al[2] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(aA), 16));
+            al[3] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(aB), 16));
+#pragma unroll
+            for (int nb = 0; nb < 8; ++nb) st.acc[nb] *= al;
+        }
+        st.mA = nA; st.mB = nB;
+        xA = tA - nA; xB = tB - nB;
+    }
+    const float pA = __builtin_amdgcn_exp2f(xA), pB = __builtin_amdgcn_exp2f(xB);      // padded slots: -inf -> 0
+    st.lA += pA; st.lB += pB;
+    {
+        // p |v| as fp16 into this lane's slot of head rows 2(j & 1) and 2(j & 1) + 1
+        // (the clamp only matters for value norms thousands of times the table's scale: no infinities)
+        const float vn = t.vn * vsc;
+        const uint32_t pk = pack_h2(fminf(pA * vn, FP16_MAX), fminf(pB * vn, FP16_MAX));
+        uint8_t* dst = pbuf + (2 * (j & 1)) * G4_PROW + 2 * slot;
+        *reinterpret_cast<uint16_t*>(dst) = (uint16_t)pk;
+        *reinterpret_cast<uint16_t*>(dst + G4_PROW) = (uint16_t)(pk >> 16);
+    }
+    wave_lds_fence();
+    const h8 pa = as_h8(*reinterpret_cast<const uint4*>(pbuf + (n & 3) * G4_PROW + 16 * j));
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        if constexpr (W == 8) {
+            h8 chi, clo;
+            lut8_split(t.vw, m, lut, slot4, chi, clo);
+            st.acc[m] = MFMA_F16(pa, chi, st.acc[m]);
+            st.acc[m] = MFMA_F16(pa, clo, st.acc[m]);
+        } else {
+            st.acc[m] = MFMA_F16(pa, lut8<W>(t.vw, m, lut, slot4), st.acc[m]);
+        }
+    }
+    wave_lds_fence();                                      // the p buffer is free for the next unit
+}
+// the state of compute_unit_g4 in the form of the general one: reference points without the shift, and rows 0, 1 of the
+// wave (the lanes whose heads the combine reads) with the whole wave's normaliser shares once summed over their 16 lanes
+__device__ static inline void g4_finish(WaveState& st) {
+    st.mA += P_SHIFT; st.mB += P_SHIFT;                     // (-inf stays -inf)
+    st.lA += __shfl_xor(st.lA, 32, WAVE);
+    st.lB += __shfl_xor(st.lB, 32, WAVE);
+}
+// rows 8..15 of the A operand repeat rows 0..7
+__device__ static inline void load_queries_g4(const uint8_t* qrows, int lane, h8* qa) {
+    const int n = lane & 7, j = lane >> 4;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+        qa[kb] = as_h8(*reinterpret_cast<const uint4*>(qrows + n * QROW_LDS + (32 * j + 8 * kb) * 2));
+}
+
 // the A operand of the key products: rows 2h, 2h+1 = high, low half of head h; row `n` of this lane,
 // dims 32j + 8kb .. + 7 for step kb, from the query rows in LDS.  Rows behind the group's slots are zero.
 __device__ static inline void load_queries(const uint8_t* qrows, int lane, int nrows, h8* qa) {
@@ -645,6 +771,77 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     }
 }
 
+// The same walk for groups of up to four heads with compute_unit_g4 (sixteen wavefronts, two unit buffers).
+template <int W, int NW>
+__device__ static inline void run_quant_level_g4(const DecodeArgs& a, int li, int bq_first, int tile0, int ntiles, int ntok,
+                                              int tid, const f4* pk, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
+    uint8_t* lut = smem;
+    const int wave = tid >> 6, lane = tid & 63;
+    const uint32_t slot4 = (lane & 31) * 4;
+    const float vsc = a.inv_s[li], ksc = a.inv_s[li] * a.scaling * LOG2E;
+    const int unit0 = 2 * tile0;
+    const auto tokens_of = [&](int u) { return min(ntok - u * UNIT, UNIT); };    // <= 0 behind the item's last token
+    // (the order of the requests, the table and the rotation is run_quant_level's)
+    RawQ8 qraw;
+    const bool stages_q = tid < 16 * a.G;
+    if (stages_q) qraw = request_q8(a.q, a.q_dt, (size_t)bq_first * HD + 8 * tid);
+    f4 pk_late[ROT_TERMS];
+    if constexpr (NW != 8) {
+#pragma unroll
+        for (int t = 0; t < ROT_TERMS; ++t)
+            if (tid < ROT_THREADS) pk_late[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
+    }
+    Unit4<W> cur;
+    int u = wave;
+    int nvalid = tokens_of(u);
+    if (nvalid > 0) load_unit4<W>(cur, a, li, unit0 + u, lane);
+    build_lut<W, NW>(lut, a, tid);
+    float* qsh = reinterpret_cast<float*>(smem + LDS_QROWS);       // [G][128] floats; the rotated rows take this place later
+    if (stages_q) {
+        float qv[8];
+        convert_q8(qraw, a.q_dt, qv);
+        *reinterpret_cast<f4*>(qsh + 8 * tid) = (f4){qv[0], qv[1], qv[2], qv[3]};
+        *reinterpret_cast<f4*>(qsh + 8 * tid + 4) = (f4){qv[4], qv[5], qv[6], qv[7]};
+    }
+    lds_barrier();
+    rotate_partial<4>(a, qsh, NW == 8 ? pk : pk_late, reinterpret_cast<float*>(smem + LDS_ROT), tid);
+    lds_barrier();
+    rotate_finish<4, NW>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
+    lds_barrier();
+    // second buffer (not for the widest rows)
+    Unit4<W> nxt;
+    int nv1 = 0;
+    if constexpr (W != 8) {
+        nv1 = tokens_of(u + NW);
+        if (nv1 > 0) load_unit4<W>(nxt, a, li, unit0 + u + NW, lane);
+    }
+    if (nvalid <= 0) return;                               // (the untouched state needs no g4_finish)
+    h8 qa[4];
+    load_queries_g4(smem + LDS_QROWS, lane, qa);
+    if constexpr (W == 8) {
+        while (true) {
+            compute_unit_g4<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, st);
+            u += NW;
+            nvalid = tokens_of(u);
+            if (nvalid <= 0) break;
+            load_unit4<W>(cur, a, li, unit0 + u, lane);
+        }
+    } else {
+        while (true) {
+            compute_unit_g4<W>(cur, nvalid, lane, lut, slot4, qa, ksc, vsc, pbuf, st);
+            if (nv1 <= 0) break;
+            u += 2 * NW;
+            nvalid = tokens_of(u);
+            if (nvalid > 0) load_unit4<W>(cur, a, li, unit0 + u, lane);
+            compute_unit_g4<W>(nxt, nv1, lane, lut, slot4, qa, ksc, vsc, pbuf, st);
+            if (nvalid <= 0) break;
+            nv1 = tokens_of(u + NW);
+            if (nv1 > 0) load_unit4<W>(nxt, a, li, unit0 + u + NW, lane);
+        }
+    }
+    g4_finish(st);
+}
+
 // ---- exact (fp16 / bf16) units ---------------------------------------------------------------------
 // Unit h of a tile is chunks 8h .. 8h+7 of every lane.  Keys: chunk 8h + 4b + kb of lane (n, j) = dims
 // 32j+8kb..+7 of slot 32h + pair_slot(n) + b.  Values: chunk 8h + m = slots 32h+8j..+7 of dim 16m+n.
@@ -741,8 +938,10 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
 // ------------------------------------------------------------------------------------------------
 // main kernel
 // ------------------------------------------------------------------------------------------------
-template <int GP, bool ORDERED, int NW>
+// G4: the quantised levels run compute_unit_g4 (GP = 4 and sixteen wavefronts only; chosen for long work items)
+template <int GP, bool ORDERED, int NW, bool G4 = false>
 __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
+    static_assert(!G4 || (GP == 4 && NW == 16), "the shared-lane form is built for four heads and sixteen wavefronts");
     // one static LDS block: the table sits at LDS address 0 and that is known when the kernel is compiled, so a
     // lookup address needs no base added
     __shared__ __align__(16) uint8_t smem[Lds<NW>::TOTAL];
@@ -777,10 +976,22 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
     uint8_t* pbuf = smem + LDS_PBUFS + wave * 2 * PBUF;
     float* alpha_sh = alphas + wave * 8;
     switch (li) {
-        case 0: run_quant_level<2, GP, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
-        case 1: run_quant_level<3, GP, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
-        case 2: run_quant_level<4, GP, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
-        case 3: run_quant_level<8, GP, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st); break;
+        case 0:
+            if constexpr (G4) run_quant_level_g4<2, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            else run_quant_level<2, GP, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            break;
+        case 1:
+            if constexpr (G4) run_quant_level_g4<3, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            else run_quant_level<3, GP, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            break;
+        case 2:
+            if constexpr (G4) run_quant_level_g4<4, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            else run_quant_level<4, GP, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            break;
+        case 3:
+            if constexpr (G4) run_quant_level_g4<8, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            else run_quant_level<8, GP, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            break;
         default:
             if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
             else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
@@ -932,15 +1143,16 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
 // host side
 // ------------------------------------------------------------------------------------------------
 static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
+#define G4_MIN_TILES_PER_ITEM 24      // quantised tiles per work item, on average, from which compute_unit_g4 is ahead
 
 extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     if (B <= 0 || Hq <= 0 || n_items < 0) return 0;
     return align_up((size_t)(n_items > 0 ? n_items : 1) * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
 }
 
-template <int GP, bool ORDERED, int NW>
+template <int GP, bool ORDERED, int NW, bool G4 = false>
 static int launch_main(const DecodeArgs& a, int grid, hipEvent_t e0, hipEvent_t e1, hipStream_t st) {
-    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED, NW>), dim3(grid), dim3(NW * 64), 0, st, e0, e1, 0, a);
+    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED, NW, G4>), dim3(grid), dim3(NW * 64), 0, st, e0, e1, 0, a);
     ODMKV_CHECK_LAUNCH("decode_main_kernel");
     return 0;
 }
@@ -992,7 +1204,16 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
 #define ODMKV_LAUNCH_MAIN(GPV, ORD) \
         (nw == 16 ? launch_main<GPV, ORD, 16>(a, n_items, e0, e1, st) : nw == 12 ? launch_main<GPV, ORD, 12>(a, n_items, e0, e1, st) \
                                                                      : launch_main<GPV, ORD, 8>(a, n_items, e0, e1, st))
-        if (GP == 4 && !a.order) rc = ODMKV_LAUNCH_MAIN(4, false);
+        // groups of up to four heads, sixteen wavefronts, long items: the form that shares the lanes out between a unit's
+        // two token blocks (its softmax step costs half the instructions; on short items the general form's
+        // schedule is a few hundred nanoseconds ahead, measured)
+        long long tiles = 0;
+        for (int li = 0; li < 4; ++li) tiles += store->n_tiles[li];
+        static const int g4_forced = [] { const char* e = getenv("ODMKV_DECODE_G4"); return e ? atoi(e) : -1; }();      // 0 / 1: measurements
+        const bool g4 = GP == 4 && nw == 16 && (g4_forced >= 0 ? g4_forced != 0 : tiles >= (long long)G4_MIN_TILES_PER_ITEM * n_items);
+        if (g4 && !a.order) rc = launch_main<4, false, 16, true>(a, n_items, e0, e1, st);
+        else if (g4) rc = launch_main<4, true, 16, true>(a, n_items, e0, e1, st);
+        else if (GP == 4 && !a.order) rc = ODMKV_LAUNCH_MAIN(4, false);
         else if (GP == 4) rc = ODMKV_LAUNCH_MAIN(4, true);
         else if (!a.order) rc = ODMKV_LAUNCH_MAIN(8, false);
         else rc = ODMKV_LAUNCH_MAIN(8, true);

@@ -118,6 +118,30 @@ def test_one_segment_cut_into_more_than_a_thousand_items():
     assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
 
 
+@pytest.mark.parametrize("G", [1, 3, 4])
+def test_long_items_of_a_small_group_take_the_shared_lane_form(G):
+    """Groups of up to four query heads on long work items (sixteen wavefronts, 24 tiles per item and more) run the
+    form of the main kernel that shares a unit's two token blocks out between the lanes.  Mixed levels, a ragged
+    last unit in every run, and key norms that grow along the sequence, so that the softmax reference point moves
+    many times and the accumulators are rescaled."""
+    g = torch.Generator().manual_seed(40 + G)
+    T, Hkv = 30000 + 37, 2
+    k = torch.randn(1, Hkv, T, 128, generator=g)
+    v = torch.randn(1, Hkv, T, 128, generator=g)
+    k *= torch.linspace(0.4, 1.3, T).view(1, 1, T, 1)             # later tokens: larger logits
+    k, v = k.half(), v.half()
+    bits = _rand_bits(g, (1, Hkv, T), (0.1, 0.6, 0.2, 0.06, 0.02, 0.02))     # (mostly narrow levels: sixteen wavefronts)
+    bits[..., :4] = 16
+    st, ref = _pair(k, v, bits)
+    q = torch.randn(1, Hkv * G, 128, generator=g).half().float()
+    want = decode_attention_state(q, ref)
+    st._build_items(16, 1 << 30)                      # a handful of long items: every quantised run in one or two pieces
+    items = st._items[0].cpu().numpy()
+    quant = items[items[:, 1] < 4]
+    assert st._worklist.wavefronts == 16 and quant[:, 3].sum() >= 24 * len(items), (st._worklist.wavefronts, quant[:, 3])
+    assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
+
+
 def test_decode_replayed_from_a_graph_matches_eager():
     """The three launches of a decode call captured in a HIP graph and replayed with new queries in the
     captured buffer, with eager work and synchronisations between the replays: every replay must give
