@@ -90,7 +90,7 @@ def bench_decode(blib, st, q, out, ws, stage_mask=7, timer=None):
     B, Hq, _ = q.shape
     rc = blib.odmkv_bench_decode_attn(
         q.data_ptr(), _lib.dtype_code(q), B, Hq, 128 ** -0.5, C.byref(st._packed), C.byref(st._worklist),
-        st._pi_k_t.data_ptr(), st.pi_v.data_ptr(), st._decode_cb.data_ptr(),
+        st._pi_k_ops.data_ptr(), st.pi_v.data_ptr(), st._decode_cb.data_ptr(),
         st._decode_cb_host, st._decode_inv, out.data_ptr(), _lib.dtype_code(out), None, ws.data_ptr(), ws.numel(),
         _lib.stream_ptr(q.device), stage_mask, timer)
     if rc != 0:

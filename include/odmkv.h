@@ -347,7 +347,8 @@ int odmkv_flush_rank(const float* scores, const float* minmax, int B, int H, int
  * change of the store.
  * out: device [B, Hq, 128] of out_dtype (accumulated in fp32, rounded once on the store);
  * lse: device fp32 [B, Hq] or NULL (log-sum-exp of the scaled logits).
- * pi_k_t is the key rotation TRANSPOSED (row-major [128,128] of Pi_k^T), pi_v the value rotation as is.
+ * pi_k_ops is the key rotation as the operand table odmkv_rotation_operands writes (the kernel rotates the query on the
+ * matrix cores: q' = Pi_k q, keys are never un-rotated), pi_v the value rotation as is (row-major fp32 [128,128]).
  * The query is rounded to fp16 on entry (the attention being replaced receives it in the model's
  * fp16/bf16); bf16 and fp32 values beyond fp16's range saturate at +-65504.  The centroid tables live in
  * LDS as fp16; to keep their rounding out of the result,
@@ -381,9 +382,15 @@ typedef struct odmkv_worklist {
 } odmkv_worklist_t;
 
 size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);
+/* The key rotation (random_rotation, kvquant/tq_backend.py:25-36, as TurboQuantMSE.dequantize applies it,
+ * tq_backend.py:199-203) in the form the decode kernel multiplies the query by: pi_k device fp32 row-major [128,128];
+ * ops device uint16 [32768] (64 KB): block (rb, kk, part), rb < 8, kk < 4, part < 2, at ((rb*4 + kk)*2 + part) * 512
+ * elements, holds for lane l = 16 j + n its 8 fp16 values e < 8 of row 16 rb + n, columns 32 kk + 8 j + e: part 0 = the
+ * entries rounded to fp16, part 1 = 4096 times what the rounding left, as fp16.  Once per rotation (per layer). */
+int odmkv_rotation_operands(const float* pi_k, uint16_t* ops, void* stream);
 int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
                       const odmkv_packed_t* store, const odmkv_worklist_t* work,
-                      const float* pi_k_t, const float* pi_v, const float* codebooks,
+                      const uint16_t* pi_k_ops, const float* pi_v, const float* codebooks,
                       const float* codebooks_host, const float* inv_scales,
                       void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                       void* stream);
@@ -401,7 +408,7 @@ int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
 #define ODMKV_STATIC_SCRATCH_BYTES (8u << 20)
 int odmkv_decode_attn_static(const void* q, int q_dtype, int B, int Hq, float scaling,
                              const odmkv_packed_t* store, const odmkv_worklist_t* work,
-                             const float* pi_k_t, const float* pi_v, const float* codebooks,
+                             const uint16_t* pi_k_ops, const float* pi_v, const float* codebooks,
                              const float* codebooks_host, const float* inv_scales,
                              void* out, int out_dtype, float* lse, void* stream);
 

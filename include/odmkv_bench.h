@@ -27,7 +27,7 @@ int odmkv_bench_timer_destroy(void* timer);
  * timer whose next event pair is attached to the main kernel. */
 int odmkv_bench_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
                             const odmkv_packed_t* store, const odmkv_worklist_t* work,
-                            const float* pi_k_t, const float* pi_v, const float* codebooks,
+                            const uint16_t* pi_k_ops, const float* pi_v, const float* codebooks,
                             const float* codebooks_host, const float* inv_scales,
                             void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                             void* stream, int stage_mask, void* timer);

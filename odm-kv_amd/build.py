@@ -8,6 +8,7 @@ hipcc cross-compiles without a GPU.  Flags that matter:
   -ffp-contract=off   nothing is fused unless the source says fma: the allocator's cost and the
                       quantiser's rotation are bit-exact contracts with their CPU statements;
   packed-fp32-ops off the compiler must not form packed fp32 instructions.
+Both libraries are linked with csrc/exports.map: only the C entry points (odmkv_*) are dynamic symbols.
 """
 from __future__ import annotations
 
@@ -36,7 +37,7 @@ def _newest(paths):
 
 def build(force: bool = False, verbose: bool = True) -> str:
     srcs = [os.path.join(CSRC, s) for s in SOURCES + BENCH_SOURCES]
-    deps = srcs + [os.path.join(CSRC, h) for h in ("common.h", "quant.h", "decode.h")] + [
+    deps = srcs + [os.path.join(CSRC, h) for h in ("common.h", "quant.h", "decode.h", "exports.map")] + [
         os.path.join(HERE, "..", "include", "odmkv.h"), os.path.join(HERE, "..", "include", "odmkv_bench.h"), __file__]
     if (not force and os.path.exists(LIB) and os.path.exists(BENCH_LIB)
             and min(os.path.getmtime(LIB), os.path.getmtime(BENCH_LIB)) >= _newest(deps)):
@@ -62,7 +63,8 @@ def build(force: bool = False, verbose: bool = True) -> str:
         objs = list(ex.map(compile_one, srcs))
     product = objs[:len(SOURCES)]
     for lib, parts in ((LIB, product), (BENCH_LIB, objs)):
-        cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib, *parts]
+        cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", f"-Wl,--version-script={os.path.join(CSRC, 'exports.map')}",
+               "-o", lib, *parts]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)

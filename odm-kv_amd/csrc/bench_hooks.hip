@@ -48,14 +48,14 @@ extern "C" int odmkv_bench_timer_destroy(void* timer) {
 
 extern "C" int odmkv_bench_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
                                        const odmkv_packed_t* store, const odmkv_worklist_t* work,
-                                       const float* pi_k_t, const float* pi_v, const float* codebooks,
+                                       const uint16_t* pi_k_ops, const float* pi_v, const float* codebooks,
                                        const float* codebooks_host, const float* inv_scales,
                                        void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                                        void* stream, int stage_mask, void* timer) {
     BenchTimer* t = (BenchTimer*)timer;
     const bool rec = t && work && (size_t)(2 * t->used + 1) < t->events.size() && work->n_items > 0 && (stage_mask & 2);
     hipEvent_t e0 = rec ? t->events[2 * t->used] : nullptr, e1 = rec ? t->events[2 * t->used + 1] : nullptr;
-    const int rc = odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, work, pi_k_t,
+    const int rc = odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, work, pi_k_ops,
                                        pi_v, codebooks, codebooks_host, inv_scales, out, out_dtype, lse, workspace,
                                        workspace_bytes, stream, stage_mask & 7, e0, e1);
     if (rc == 0 && rec) ++t->used;

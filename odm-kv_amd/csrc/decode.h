@@ -15,7 +15,7 @@ struct DecodeArgs {
     const int32_t* items;
     const int32_t* item_range;
     const int32_t* order;      // order[k] = item that workgroup k takes (long items first), or null: item k
-    const float* pi_k_t;   // Pi_k transposed
+    const uint16_t* pi_k_ops;   // Pi_k as the A operands of the query rotation (odmkv_rotation_operands)
     const float* pi_v;
     const float* cb;
     float inv_s[4];   // 1 / table scale per width
@@ -30,7 +30,7 @@ struct DecodeArgs {
 // call; bit 0 is unused).  ev_start / ev_stop: hipEvent_t attached to the main kernel's dispatch, or null.
 int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling,
                         const odmkv_packed_t* store, const odmkv_worklist_t* work,
-                        const float* pi_k_t, const float* pi_v, const float* codebooks,
+                        const uint16_t* pi_k_ops, const float* pi_v, const float* codebooks,
                         const float* codebooks_host, const float* inv_scales,
                         void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                         void* stream, int stage_mask, void* ev_start, void* ev_stop);

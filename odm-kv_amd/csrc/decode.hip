@@ -44,26 +44,20 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 #define PROW 96             // bytes per head row of a wave's p buffer: 32 x 16 bit + padding (bank spread)
 #define PBUF (8 * PROW)     // one p buffer: 8 head rows
 
-// LDS of the main kernel: [table, later the combine area] [partial sums of the query rotation] [rotated query rows]
+// LDS of the main kernel: [table, later the combine area] [rotated query rows]
 // [p buffers] [per-wave scalars].  NW = wavefronts of the workgroup: 8 (short items: less set-up and a lighter combine)
 // or 16 (long items: four wavefronts per SIMD keep its issue slots full).
-#define ROT_THREADS 512                          // threads that rotate the queries (the first 512 of the workgroup)
-#define ROT_SLICES (ROT_THREADS / 32)            // slices of the rotation's sum: a thread covers 4 dims x HD / ROT_SLICES terms
-#define ROT_TERMS (HD / ROT_SLICES)
 #define QROW_LDS 272                             // bytes of a query row in LDS: 128 x 16 bit + 16 (bank spread)
-#define LDS_ROT LUT_BYTES
-#define LDS_QROWS (LDS_ROT + ROT_SLICES * ODMKV_MAX_GROUP * HD * 4)
+#define LDS_QROWS LUT_BYTES
 #define LDS_PBUFS (LDS_QROWS + 16 * QROW_LDS)
-static_assert(ODMKV_MAX_GROUP * HD * 4 <= 16 * QROW_LDS, "the staged query shares the rotated rows' space");
 template <int NW>
 struct Lds {
     static constexpr int SCALARS = LDS_PBUFS + NW * 2 * PBUF;
     static constexpr int TOTAL = SCALARS + NW * 4 * 8 * 4 + 8 * 4;
     static_assert(NW * ODMKV_MAX_GROUP * HD * 4 <= LUT_BYTES, "combine area must fit the table's space");
-    static_assert(NW >= 4 && NW <= 16 && NW * 64 >= ROT_THREADS, "wave count");
+    static_assert(NW >= 8 && NW <= 16, "wave count (the first eight rotate the queries)");
     static_assert(TOTAL <= 160 * 1024, "LDS of one workgroup");
 };
-static_assert(ROT_TERMS == 8, "rotation slices");
 
 __device__ static inline uint32_t half_bits(float f) { return (uint32_t)__half_as_ushort(__float2half_rn(f)); }
 
@@ -470,7 +464,7 @@ __device__ static inline void compute_unit(const Unit<W>& t, int nvalid, int lan
     wave_lds_fence();                                      // the p buffer is free for the next unit
 }
 
-// ---- groups of up to four query heads, long work items (decode_main_kernel<4, ., 16, true>) -----------------------
+// ---- groups of up to four query heads on sixteen wavefronts (decode_main_kernel<4, ., 16, true>) ------------------
 // Four heads need 8 of the 16 matrix rows.  The general form leaves rows 8..15 empty and every lane of wave rows 2, 3
 // (lanes 32..63) then runs the softmax step on heads that do not exist.  Here rows 8..15 repeat rows 0..7
 // (load_queries_g4) and the two token blocks of a unit share the lanes out between them: after the key products lane
@@ -605,92 +599,106 @@ __device__ static inline void load_queries(const uint8_t* qrows, int lane, int n
         qa[kb] = as_h8(on ? *reinterpret_cast<const uint4*>(qrows + n * QROW_LDS + (32 * j + 8 * kb) * 2) : make_uint4(0u, 0u, 0u, 0u));
 }
 
-// The queries in the rotated basis of the quantised keys, q' = Pi_k q16, as fp16 high + low halves.  Thread
-// (i4 = tid % 32, slice = tid / 32) holds Pi_k^T[8 slice .. + 7][4 i4 .. + 3] (requested when the kernel starts, before
-// the work item is known) and sums its eight terms for every head of the group, in order; the slices are added in
-// order by the thread that owns (head, dim).  Every workgroup of a KV head repeats this: the matrix comes out of the
-// L2 cache, and the work hides behind the first unit's way from memory.
-// The query of the group's heads goes through LDS: thread t < 16 G requests eight elements (request_q8), and
-// stages them as floats once they are there; after a barrier every rotating thread reads the eight terms of its slice.
-template <int GP>
-__device__ static inline void rotate_partial(const DecodeArgs& a, const float* qsh, const f4* pk, float* rot, int tid) {
-    const int i4 = tid & 31, slice = tid >> 5;
-    if (tid >= ROT_THREADS) return;
+// The queries in the rotated basis of the quantised keys, q' = Pi_k q16, as fp16 high + low halves, on the matrix cores.
+// Pi_k arrives as a table of A operands (odmkv_rotation_operands): block (rb, kk, part) = rows 16 rb .. + 15 of Pi_k, columns
+// 32 kk .. + 31, part 0 = the entries rounded to fp16, part 1 = 2^12 times what the rounding left (fp16 again): 64 lanes x
+// 16 bytes in operand order, 64 KB in all.  Wavefront w < 8 requests the eight blocks of its 16 rows (8 KB, out of the L2
+// for all but the first workgroup to ask) together with the queries, ahead of its first unit, and forms output dims
+// 16 w .. + 15 of all heads of the group: D[dim][head] = sum over 4 column blocks of A . B, B = the group's queries rounded
+// to fp16 (columns = heads), products exact, sums fp32, the two parts in accumulators of their own.  Lane (n, j) ends with
+// dims 16 w + 4j .. + 3 of head n and writes their fp16 high and low halves into rows 2n, 2n + 1 of the A operand of
+// the key products: one barrier, no LDS staging.  (Copying the table into LDS with LDS-direct loads when the kernel
+// starts, before the item is known, measured the same; the vector-ALU rotation it replaces cost 0.9 us more per item on
+// 28-head stores and long items, and the same on the 32-head 32k-token store.)
+// the rotation's operands of a rotating wavefront: a[2 kk + part] = its block (kk, part) of the table; r[kk] = the group's
+// queries as B operands, lane (n, j) = elements 32 kk + 8j .. + 7 of head n (head 0 for the columns behind the group,
+// zeroed later).  fp32 queries (no model hands them over) would take twice the registers: they are fetched when the
+// rotation runs.
+struct RotQuery { uint4 r[4]; uint4 a[8]; };
+__device__ static inline void request_rot_query(RotQuery& rq, const DecodeArgs& a, int bq_first, int tid) {
+    const int lane = tid & 63, n = lane & 15, j = lane >> 4;
+    const size_t elem = (size_t)(bq_first + (n < a.G ? n : 0)) * HD + 8 * j;
+    if ((tid >> 6) >= 8) return;                         // wave-uniform
+    {
 #pragma unroll
-    for (int g = 0; g < GP; ++g) {
-        f4 acc = (f4){0.f, 0.f, 0.f, 0.f};
-        if (g < a.G) {                                     // wave-uniform
-            const f4 q0 = *reinterpret_cast<const f4*>(qsh + g * HD + slice * ROT_TERMS);
-            const f4 q1 = *reinterpret_cast<const f4*>(qsh + g * HD + slice * ROT_TERMS + 4);
+        for (int i = 0; i < 8; ++i) rq.a[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.pi_k_ops) + (size_t)(((tid >> 6) * 8 + i) * 64 + lane) * 16);
+    }
+    if (a.q_dt != ODMKV_F32) {
 #pragma unroll
-            for (int t = 0; t < ROT_TERMS; ++t)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[e] = __fmaf_rn(pk[t][e], t < 4 ? q0[t] : q1[t - 4], acc[e]);
-        }
-        *reinterpret_cast<f4*>(rot + ((size_t)(slice * GP + g) * HD) + 4 * i4) = acc;
+        for (int kk = 0; kk < 4; ++kk) rq.r[kk] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(a.q) + elem + 32 * kk);
     }
 }
-template <int GP, int NW>
-__device__ static inline void rotate_finish(const float* rot, uint8_t* qrows, int tid) {
-    for (int o = tid; o < GP * HD; o += NW * 64) {
-        const int g = o / HD, dim = o % HD;
-        float tot = rot[(size_t)g * HD + dim];
+// The low part of the table is kept 2^12 times larger (odmkv_rotation_operands): as it is it would lie in fp16's subnormal
+// range, which the matrix instruction does not read; its products are summed apart and scaled back.
+#define ROT_LOW_SCALE 4096.0f
+template <int GP>
+__device__ static inline void rotate_queries(const DecodeArgs& a, uint8_t* smem, int tid, int bq_first, const RotQuery& rq) {
+    const int wave = tid >> 6, lane = tid & 63, n = lane & 15, j = lane >> 4;
+    if (wave >= 8) return;                               // wave-uniform
+    f4 dh = (f4){0.f, 0.f, 0.f, 0.f}, dl = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int sl = 1; sl < ROT_SLICES; ++sl) tot += rot[((size_t)sl * GP + g) * HD + dim];
-        const __half hi = __float2half_rn(tot);
-        *reinterpret_cast<uint16_t*>(qrows + (2 * g) * QROW_LDS + dim * 2) = __half_as_ushort(hi);
-        *reinterpret_cast<uint16_t*>(qrows + (2 * g + 1) * QROW_LDS + dim * 2) = (uint16_t)half_bits(tot - __half2float(hi));
+    for (int kk = 0; kk < 4; ++kk) {
+        uint4 b;
+        if (a.q_dt == ODMKV_F16) {
+            b = rq.r[kk];
+        } else {
+            float qv[8];
+            if (a.q_dt == ODMKV_F32) {
+                load_q8(a.q, ODMKV_F32, (size_t)(bq_first + (n < a.G ? n : 0)) * HD + 32 * kk + 8 * j, qv);
+            } else {
+                RawQ8 raw;
+                raw.x = rq.r[kk]; raw.y = make_uint4(0u, 0u, 0u, 0u);
+                convert_q8(raw, ODMKV_BF16, qv);
+            }
+            b = make_uint4(pack_h2(qv[0], qv[1]), pack_h2(qv[2], qv[3]), pack_h2(qv[4], qv[5]), pack_h2(qv[6], qv[7]));
+        }
+        if (n >= a.G) b = make_uint4(0u, 0u, 0u, 0u);
+        dh = MFMA_F16(as_h8(rq.a[2 * kk]), as_h8(b), dh);
+        dl = MFMA_F16(as_h8(rq.a[2 * kk + 1]), as_h8(b), dl);
+    }
+    if (n < GP) {
+        uint32_t hi[2], lo[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const float x0 = __fmaf_rn(dl[2 * e], 1.0f / ROT_LOW_SCALE, dh[2 * e]), x1 = __fmaf_rn(dl[2 * e + 1], 1.0f / ROT_LOW_SCALE, dh[2 * e + 1]);
+            const __half h0 = __float2half_rn(x0), h1 = __float2half_rn(x1);
+            hi[e] = (uint32_t)__half_as_ushort(h0) | ((uint32_t)__half_as_ushort(h1) << 16);
+            lo[e] = half_bits(x0 - __half2float(h0)) | (half_bits(x1 - __half2float(h1)) << 16);
+        }
+        uint8_t* row = smem + LDS_QROWS + (2 * n) * QROW_LDS + (16 * wave + 4 * j) * 2;
+        *reinterpret_cast<uint2*>(row) = make_uint2(hi[0], hi[1]);
+        *reinterpret_cast<uint2*>(row + QROW_LDS) = make_uint2(lo[0], lo[1]);
     }
 }
 
 // One work item of a quantised level: the workgroup's wavefronts walk the item's units.
 template <int W, int GP, int NW>
 __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq_first, int tile0, int ntiles, int ntok,
-                                              int tid, const f4* pk, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
+                                              int tid, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
     uint8_t* lut = smem;
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
     const float vsc = a.inv_s[li], ksc = a.inv_s[li] * a.scaling * LOG2E;
     const int unit0 = 2 * tile0;
     const auto tokens_of = [&](int u) { return min(ntok - u * UNIT, UNIT); };    // <= 0 behind the item's last token
-    // Each wavefront requests the rotation and its first unit, then rotates the queries and builds its share of the
-    // table while memory answers; the second unit is requested after that (LDS stores behind a long queue of requests wait until the
-    // memory pipeline has accepted them: with both units requested first the table was ready a microsecond later).
-    // Loads return in issue order: the (small) query goes first.
-    RawQ8 qraw;
-    const bool stages_q = tid < 16 * a.G;
-    if (stages_q) qraw = request_q8(a.q, a.q_dt, (size_t)bq_first * HD + 8 * tid);
+    // Each wavefront requests the queries and its first unit, builds its share of the centroid table while memory answers,
+    // and the first eight rotate the queries; the second unit is requested after that (LDS stores behind a long queue of
+    // requests wait until the memory pipeline has accepted them: with both units requested first the table was ready a
+    // microsecond later).  Loads return in issue order: the (small) query goes first.
+    RotQuery rq;
+    request_rot_query(rq, a, bq_first, tid);
     // DEPTH units of this wavefront are under way at any time: two (one for the widest rows: registers); twelve
     // wavefronts have the registers for a third 2-bit unit.  (Six units in flight with eight wavefronts were measured:
     // no gain, the eight are bound by their arithmetic.)
     constexpr int DEPTH = W == 8 ? 1 : (NW == 12 && W == 2) ? 3 : 2;
     if constexpr (DEPTH <= 2) {
         // two buffers, written out: the compiler schedules this form a microsecond per item better than the ring.
-        // The rotation is requested before the unit: loads return in the order of their requests, and the rotation's
-        // comes out of the L2 while the unit's comes from memory; behind the unit it arrives no earlier than the unit,
-        // and the rotation's arithmetic then starts that much later (0.7 us per item, measured).
-        f4 pk_late[ROT_TERMS];
-        if constexpr (NW != 8) {
-    #pragma unroll
-            for (int t = 0; t < ROT_TERMS; ++t)
-                if (tid < ROT_THREADS) pk_late[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
-        }
         Unit<W> cur;
         int u = wave;
         int nvalid = tokens_of(u);
         if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
         build_lut<W, NW>(lut, a, tid);
-        float* qsh = reinterpret_cast<float*>(smem + LDS_QROWS);       // [G][128] floats; the rotated rows take this place later
-        if (stages_q) {
-            float qv[8];
-            convert_q8(qraw, a.q_dt, qv);
-            *reinterpret_cast<f4*>(qsh + 8 * tid) = (f4){qv[0], qv[1], qv[2], qv[3]};
-            *reinterpret_cast<f4*>(qsh + 8 * tid + 4) = (f4){qv[4], qv[5], qv[6], qv[7]};
-        }
-        lds_barrier();
-        rotate_partial<GP>(a, qsh, NW == 8 ? pk : pk_late, reinterpret_cast<float*>(smem + LDS_ROT), tid);
-        lds_barrier();
-        rotate_finish<GP, NW>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
+        rotate_queries<GP>(a, smem, tid, bq_first, rq);
         lds_barrier();
         // second buffer (not for the widest rows), requested before the first unit is used (requested before the
         // rotation instead, it delays the table's LDS stores behind its queue of requests: 0.9 us per item slower)
@@ -729,24 +737,8 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
         int nv[DEPTH];
         nv[0] = tokens_of(wave);
         if (nv[0] > 0) load_unit<W>(buf[0], a, li, unit0 + wave, lane);
-        f4 pk_late[ROT_TERMS];                                  // (long items: the order of the two requests made no difference)
-        if constexpr (NW != 8) {
-    #pragma unroll
-            for (int t = 0; t < ROT_TERMS; ++t)
-                if (tid < ROT_THREADS) pk_late[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
-        }
         build_lut<W, NW>(lut, a, tid);
-        float* qsh = reinterpret_cast<float*>(smem + LDS_QROWS);       // [G][128] floats; the rotated rows take this place later
-        if (stages_q) {
-            float qv[8];
-            convert_q8(qraw, a.q_dt, qv);
-            *reinterpret_cast<f4*>(qsh + 8 * tid) = (f4){qv[0], qv[1], qv[2], qv[3]};
-            *reinterpret_cast<f4*>(qsh + 8 * tid + 4) = (f4){qv[4], qv[5], qv[6], qv[7]};
-        }
-        lds_barrier();
-        rotate_partial<GP>(a, qsh, NW == 8 ? pk : pk_late, reinterpret_cast<float*>(smem + LDS_ROT), tid);
-        lds_barrier();
-        rotate_finish<GP, NW>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
+        rotate_queries<GP>(a, smem, tid, bq_first, rq);
         lds_barrier();
         // the rest of the ring, requested before the first unit is used
     #pragma unroll
@@ -771,10 +763,11 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     }
 }
 
-// The same walk for groups of up to four heads with compute_unit_g4 (sixteen wavefronts, two unit buffers).
+// The same walk for groups of up to four heads with compute_unit_g4 (sixteen wavefronts, two unit buffers; an
+// eight-wavefront ring of five buffers, every unit of a short item requested at once, measured no faster).
 template <int W, int NW>
 __device__ static inline void run_quant_level_g4(const DecodeArgs& a, int li, int bq_first, int tile0, int ntiles, int ntok,
-                                              int tid, const f4* pk, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
+                                              int tid, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
     uint8_t* lut = smem;
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
@@ -782,31 +775,14 @@ __device__ static inline void run_quant_level_g4(const DecodeArgs& a, int li, in
     const int unit0 = 2 * tile0;
     const auto tokens_of = [&](int u) { return min(ntok - u * UNIT, UNIT); };    // <= 0 behind the item's last token
     // (the order of the requests, the table and the rotation is run_quant_level's)
-    RawQ8 qraw;
-    const bool stages_q = tid < 16 * a.G;
-    if (stages_q) qraw = request_q8(a.q, a.q_dt, (size_t)bq_first * HD + 8 * tid);
-    f4 pk_late[ROT_TERMS];
-    if constexpr (NW != 8) {
-#pragma unroll
-        for (int t = 0; t < ROT_TERMS; ++t)
-            if (tid < ROT_THREADS) pk_late[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
-    }
+    RotQuery rq;
+    request_rot_query(rq, a, bq_first, tid);
     Unit4<W> cur;
     int u = wave;
     int nvalid = tokens_of(u);
     if (nvalid > 0) load_unit4<W>(cur, a, li, unit0 + u, lane);
     build_lut<W, NW>(lut, a, tid);
-    float* qsh = reinterpret_cast<float*>(smem + LDS_QROWS);       // [G][128] floats; the rotated rows take this place later
-    if (stages_q) {
-        float qv[8];
-        convert_q8(qraw, a.q_dt, qv);
-        *reinterpret_cast<f4*>(qsh + 8 * tid) = (f4){qv[0], qv[1], qv[2], qv[3]};
-        *reinterpret_cast<f4*>(qsh + 8 * tid + 4) = (f4){qv[4], qv[5], qv[6], qv[7]};
-    }
-    lds_barrier();
-    rotate_partial<4>(a, qsh, NW == 8 ? pk : pk_late, reinterpret_cast<float*>(smem + LDS_ROT), tid);
-    lds_barrier();
-    rotate_finish<4, NW>(reinterpret_cast<const float*>(smem + LDS_ROT), smem + LDS_QROWS, tid);
+    rotate_queries<4>(a, smem, tid, bq_first, rq);
     lds_barrier();
     // second buffer (not for the widest rows)
     Unit4<W> nxt;
@@ -938,7 +914,7 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
 // ------------------------------------------------------------------------------------------------
 // main kernel
 // ------------------------------------------------------------------------------------------------
-// G4: the quantised levels run compute_unit_g4 (GP = 4 and sixteen wavefronts only; chosen for long work items)
+// G4: the quantised levels run compute_unit_g4 (GP = 4 and sixteen wavefronts only)
 template <int GP, bool ORDERED, int NW, bool G4 = false>
 __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
     static_assert(!G4 || (GP == 4 && NW == 16), "the shared-lane form is built for four heads and sixteen wavefronts");
@@ -953,21 +929,15 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
     float* wM = wf + NW * 8;                                // [8]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    // this thread's share of Pi_k^T for the query rotation: the same for every item, requested first
-    // (eight wavefronts only: sixteen have half the registers, and their long items do not feel the wait)
-    f4 pk[ROT_TERMS];
-#pragma unroll
-    for (int t = 0; t < ROT_TERMS; ++t)
-        if (NW == 8 && tid < ROT_THREADS) pk[t] = *reinterpret_cast<const f4*>(a.pi_k_t + (size_t)((tid >> 5) * ROT_TERMS + t) * HD + 4 * (tid & 31));
     const int item = ORDERED ? a.order[blockIdx.x] : (int)blockIdx.x;
     const int4 d0 = reinterpret_cast<const int4*>(a.items)[2 * item];       // bh, level, first tile, tiles
     const int4 d1 = reinterpret_cast<const int4*>(a.items)[2 * item + 1];   // tokens, first tile of the segment
+    // the rotation's operand table on its way into LDS right behind the request for the work item (loads return in the
+    // order of their requests: asked for first, the table would hold the item back; it does not depend on the item)
     const int bh = d0.x, li = d0.y, tile0 = d0.z, ntiles = d0.w;
     const int bq_first = (bh / a.s.Hkv) * a.Hq + (bh % a.s.Hkv) * a.G;      // first query head of the group
 
-    // where this item's result goes: fetched now, not when the workgroup is about to finish
-    float* dst = a.partial + (size_t)item * GP * PSTRIDE;
-    asm volatile("" : "+s"(dst));
+    float* dst = a.partial + (size_t)item * GP * PSTRIDE;      // where this item's result goes
 
     WaveState st;
     st.mA = -INFINITY; st.mB = -INFINITY; st.lA = 0.0f; st.lB = 0.0f;
@@ -977,20 +947,20 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
     float* alpha_sh = alphas + wave * 8;
     switch (li) {
         case 0:
-            if constexpr (G4) run_quant_level_g4<2, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
-            else run_quant_level<2, GP, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            if constexpr (G4) run_quant_level_g4<2, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
+            else run_quant_level<2, GP, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
             break;
         case 1:
-            if constexpr (G4) run_quant_level_g4<3, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
-            else run_quant_level<3, GP, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            if constexpr (G4) run_quant_level_g4<3, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
+            else run_quant_level<3, GP, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
             break;
         case 2:
-            if constexpr (G4) run_quant_level_g4<4, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
-            else run_quant_level<4, GP, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            if constexpr (G4) run_quant_level_g4<4, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
+            else run_quant_level<4, GP, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
             break;
         case 3:
-            if constexpr (G4) run_quant_level_g4<8, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
-            else run_quant_level<8, GP, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, pk, smem, pbuf, alpha_sh, st);
+            if constexpr (G4) run_quant_level_g4<8, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
+            else run_quant_level<8, GP, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
             break;
         default:
             if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
@@ -1143,7 +1113,37 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
 // host side
 // ------------------------------------------------------------------------------------------------
 static inline int group_pad(int G) { return G <= 4 ? 4 : 8; }
-#define G4_MIN_TILES_PER_ITEM 24      // quantised tiles per work item, on average, from which compute_unit_g4 is ahead
+
+// Pi_k -> the operand table of rotate_queries: thread t of block (rb, kk) writes lane t's eight values of both parts
+__global__ __launch_bounds__(64) void rotation_operands_kernel(const float* __restrict__ pi_k, uint16_t* __restrict__ ops) {
+    const int rb = blockIdx.x >> 2, kk = blockIdx.x & 3, lane = threadIdx.x, n = lane & 15, j = lane >> 4;
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+        float x[2];
+        uint32_t h[2], l[2];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            x[k] = pi_k[(size_t)(16 * rb + n) * HD + 32 * kk + 8 * j + e + k];
+            const __half hv = __float2half_rn(x[k]);
+            h[k] = (uint32_t)__half_as_ushort(hv);
+            l[k] = half_bits((x[k] - __half2float(hv)) * ROT_LOW_SCALE);
+        }
+        hi[e >> 1] = h[0] | (h[1] << 16);
+        lo[e >> 1] = l[0] | (l[1] << 16);
+    }
+    uint4* dst = reinterpret_cast<uint4*>(ops) + (size_t)(blockIdx.x * 2) * 64 + lane;
+    dst[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    dst[64] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+}
+
+extern "C" int odmkv_rotation_operands(const float* pi_k, uint16_t* ops, void* stream) {
+    ODMKV_CHECK_ARG(pi_k && ops, "rotation_operands: null pointer");
+    ODMKV_CHECK_ARG(((uintptr_t)ops & 15) == 0, "rotation_operands: the table must be 16-byte aligned");
+    hipLaunchKernelGGL(rotation_operands_kernel, dim3(32), dim3(64), 0, (hipStream_t)stream, pi_k, ops);
+    ODMKV_CHECK_LAUNCH("rotation_operands_kernel");
+    return 0;
+}
 
 extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     if (B <= 0 || Hq <= 0 || n_items < 0) return 0;
@@ -1159,7 +1159,7 @@ static int launch_main(const DecodeArgs& a, int grid, hipEvent_t e0, hipEvent_t 
 
 int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling,
                         const odmkv_packed_t* store, const odmkv_worklist_t* work,
-                        const float* pi_k_t, const float* pi_v, const float* codebooks,
+                        const uint16_t* pi_k_ops, const float* pi_v, const float* codebooks,
                         const float* codebooks_host, const float* inv_scales,
                         void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                         void* stream, int stage_mask, void* ev_start, void* ev_stop) {
@@ -1167,8 +1167,9 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     ODMKV_CHECK_ARG(out_dtype == ODMKV_F16 || out_dtype == ODMKV_BF16 || out_dtype == ODMKV_F32, "decode_attn: bad output dtype %d", out_dtype);
     ODMKV_CHECK_ARG(codebooks_host != nullptr, "decode_attn: null host copy of the centroid tables");
     ODMKV_CHECK_ARG(inv_scales != nullptr, "decode_attn: null table scales");
-    ODMKV_CHECK_ARG(q && store && work && pi_k_t && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
+    ODMKV_CHECK_ARG(q && store && work && pi_k_ops && pi_v && codebooks && out && workspace, "decode_attn: null pointer");
     ODMKV_CHECK_ARG(((uintptr_t)q & 15) == 0, "decode_attn: the query must be 16-byte aligned");
+    ODMKV_CHECK_ARG(((uintptr_t)pi_k_ops & 15) == 0, "decode_attn: the rotation's operand table must be 16-byte aligned");
     const int n_items = work->n_items;
     ODMKV_CHECK_ARG(n_items >= 0, "decode_attn: negative item count");
     ODMKV_CHECK_ARG(work->wavefronts == 0 || work->wavefronts == 8 || work->wavefronts == 12 || work->wavefronts == 16,
@@ -1188,7 +1189,7 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     DecodeArgs a;
     a.s = *store; a.q = q; a.q_dt = q_dtype; a.out_dt = out_dtype; a.Hq = Hq; a.G = G; a.B = B; a.scaling = scaling;
     a.items = work->items; a.item_range = work->item_range; a.order = work->dispatch_order;
-    a.pi_k_t = pi_k_t; a.pi_v = pi_v; a.cb = codebooks;
+    a.pi_k_ops = pi_k_ops; a.pi_v = pi_v; a.cb = codebooks;
     for (int w = 0; w < 4; ++w) a.inv_s[w] = inv_scales[w];
     for (int k = 0; k < 28; ++k) a.cbs[k] = codebooks_host[k];
     a.partial = (float*)workspace;
@@ -1204,13 +1205,10 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
 #define ODMKV_LAUNCH_MAIN(GPV, ORD) \
         (nw == 16 ? launch_main<GPV, ORD, 16>(a, n_items, e0, e1, st) : nw == 12 ? launch_main<GPV, ORD, 12>(a, n_items, e0, e1, st) \
                                                                      : launch_main<GPV, ORD, 8>(a, n_items, e0, e1, st))
-        // groups of up to four heads, sixteen wavefronts, long items: the form that shares the lanes out between a unit's
-        // two token blocks (its softmax step costs half the instructions; on short items the general form's
-        // schedule is a few hundred nanoseconds ahead, measured)
-        long long tiles = 0;
-        for (int li = 0; li < 4; ++li) tiles += store->n_tiles[li];
-        static const int g4_forced = [] { const char* e = getenv("ODMKV_DECODE_G4"); return e ? atoi(e) : -1; }();      // 0 / 1: measurements
-        const bool g4 = GP == 4 && nw == 16 && (g4_forced >= 0 ? g4_forced != 0 : tiles >= (long long)G4_MIN_TILES_PER_ITEM * n_items);
+        // groups of up to four heads on sixteen wavefronts: the form that shares the lanes out between a unit's two token
+        // blocks (its softmax step costs half the instructions); ODMKV_DECODE_G4=0 selects the general form, for measurements
+        static const int g4_forced = [] { const char* e = getenv("ODMKV_DECODE_G4"); return e ? atoi(e) : -1; }();
+        const bool g4 = GP == 4 && nw == 16 && g4_forced != 0;
         if (g4 && !a.order) rc = launch_main<4, false, 16, true>(a, n_items, e0, e1, st);
         else if (g4) rc = launch_main<4, true, 16, true>(a, n_items, e0, e1, st);
         else if (GP == 4 && !a.order) rc = ODMKV_LAUNCH_MAIN(4, false);
@@ -1239,11 +1237,11 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
 
 extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
                                  const odmkv_packed_t* store, const odmkv_worklist_t* work,
-                                 const float* pi_k_t, const float* pi_v, const float* codebooks,
+                                 const uint16_t* pi_k_ops, const float* pi_v, const float* codebooks,
                                  const float* codebooks_host, const float* inv_scales,
                                  void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                                  void* stream) {
-    return odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, work, pi_k_t, pi_v, codebooks, codebooks_host, inv_scales,
+    return odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, work, pi_k_ops, pi_v, codebooks, codebooks_host, inv_scales,
                                out, out_dtype, lse, workspace, workspace_bytes, stream, 7, nullptr, nullptr);
 }
 
@@ -1275,7 +1273,7 @@ static int static_scratch(void** ptr) {
 
 extern "C" int odmkv_decode_attn_static(const void* q, int q_dtype, int B, int Hq, float scaling,
                                         const odmkv_packed_t* store, const odmkv_worklist_t* work,
-                                        const float* pi_k_t, const float* pi_v, const float* codebooks,
+                                        const uint16_t* pi_k_ops, const float* pi_v, const float* codebooks,
                                         const float* codebooks_host, const float* inv_scales,
                                         void* out, int out_dtype, float* lse, void* stream) {
     ODMKV_CHECK_ARG(work != nullptr, "decode_attn_static: null work list");
@@ -1288,6 +1286,6 @@ extern "C" int odmkv_decode_attn_static(const void* q, int q_dtype, int B, int H
     }
     void* ws = nullptr;
     if (int rc = static_scratch(&ws)) return rc;
-    return odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, work, pi_k_t, pi_v, codebooks, codebooks_host, inv_scales,
+    return odmkv_decode_launch(q, q_dtype, B, Hq, scaling, store, work, pi_k_ops, pi_v, codebooks, codebooks_host, inv_scales,
                                out, out_dtype, lse, ws, (size_t)ODMKV_STATIC_SCRATCH_BYTES, stream, 7, nullptr, nullptr);
 }

@@ -76,6 +76,7 @@ def _load() -> C.CDLL:
         "odmkv_quantize_rows": (C.c_int, [vp, i32, i64, i64, i32, vp, vp, vp, vp, vp]),
         "odmkv_dequantize_rows": (C.c_int, [vp, vp, i64, i32, vp, vp, vp, vp]),
         "odmkv_lloyd_max": (C.c_int, [i32, i32, i32, C.c_double, C.c_double, vp, vp, vp]),
+        "odmkv_rotation_operands": (C.c_int, [vp, vp, vp]),
         "odmkv_pack_count_chunks": (C.c_int, [i32]),
         "odmkv_store_finish_staged": (C.c_int, [vp, i32, i32, i32, i32, i32, i32, vp, C.c_uint64, C.POINTER(Packed), vp, vp,
                                                 vp, vp, vp, C.POINTER(Packed), vp, vp]),
@@ -104,7 +105,7 @@ EXPORTS = ("odmkv_version", "odmkv_last_error", "odmkv_score_workspace_bytes", "
            "odmkv_allocate_workspace_bytes", "odmkv_allocate", "odmkv_level_counts",
            "odmkv_store_init", "odmkv_store_gather", "odmkv_quant_pack_staged", "odmkv_store_layout", "odmkv_store_bind", "odmkv_pack_workspace_bytes", "odmkv_pack_count_chunks", "odmkv_store_finish_staged", "odmkv_quant_pack", "odmkv_quantize_rows",
            "odmkv_dequantize_rows", "odmkv_lloyd_max", "odmkv_dequant", "odmkv_dequant_from", "odmkv_append_exact",
-           "odmkv_decode_workspace_bytes", "odmkv_decode_attn", "odmkv_decode_attn_static",
+           "odmkv_decode_workspace_bytes", "odmkv_rotation_operands", "odmkv_decode_attn", "odmkv_decode_attn_static",
            "odmkv_exact_tail", "odmkv_flush_score", "odmkv_flush_rank")
 
 

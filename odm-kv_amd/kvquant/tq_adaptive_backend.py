@@ -179,6 +179,23 @@ def _mailbox(dev, numel: int):
     return got
 
 
+HEAD_DIM_OPS = 128 * 128      # elements of one part of the operand table
+_ROT_OPS_CACHE: dict = {}
+
+
+def _rotation_operands(pi_k: torch.Tensor) -> torch.Tensor:
+    """The key rotation as the matrix operands of the decode kernel's query rotation (odmkv_rotation_operands):
+    int16 [32768] on pi_k's device, built once per rotation tensor (rotations are cached per (dim, seed, device), so
+    every layer's state that shares a seed shares the table)."""
+    key = (pi_k.data_ptr(), str(pi_k.device))
+    hit = _ROT_OPS_CACHE.get(key)
+    if hit is None or hit[0] is not pi_k:
+        ops = torch.empty(2 * HEAD_DIM_OPS, dtype=torch.int16, device=pi_k.device)
+        _lib.check(lib.odmkv_rotation_operands(pi_k.data_ptr(), ops.data_ptr(), _lib.stream_ptr(pi_k.device)))
+        hit = _ROT_OPS_CACHE[key] = (pi_k, ops)
+    return hit[1]
+
+
 def _empty_positions(device) -> torch.Tensor:
     return torch.empty((0, 3), dtype=torch.long, device=device)
 
@@ -223,7 +240,8 @@ class TurboQuantAdaptiveKVCacheState:
             raise RuntimeError("the packed KV store lives on the GPU; there is no CPU path")
         self.pi_k = cached_rotation(head_dim, self.device, seed)
         self.pi_v = cached_rotation(head_dim, self.device, seed + 2000)
-        self._pi_k_t = self.pi_k.t().contiguous()
+        # the key rotation as the decode kernel's matrix operands (fp16 high + low parts in operand order)
+        self._pi_k_ops = _rotation_operands(self.pi_k)
         self.codebooks = codebook_table(head_dim, self.device)
         self._decode_cb, inv = decode_tables(head_dim, self.device)
         self._decode_inv = (C.c_float * 4)(*inv)
@@ -807,7 +825,7 @@ class TurboQuantAdaptiveKVCacheState:
         ws = _lib.workspace(self.device, ws_bytes, "decode")
         _lib.check(lib.odmkv_decode_attn(
             q.data_ptr(), _lib.dtype_code(q), B, Hq, scale, C.byref(self._packed), C.byref(self._worklist),
-            self._pi_k_t.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
+            self._pi_k_ops.data_ptr(), self.pi_v.data_ptr(), self._decode_cb.data_ptr(),
             self._decode_cb_host, self._decode_inv, out.data_ptr(), _lib.dtype_code(out), _lib.ptr(lse), ws.data_ptr(), ws_bytes,
             _lib.stream_ptr(self.device)))
         return (out, lse) if return_lse else out

@@ -34,6 +34,11 @@ def test_exports_every_declared_symbol(lib):
         assert hasattr(blib, name) and not hasattr(lib, name)
     for name in declared:
         assert hasattr(blib, name)
+    # and nothing else is a dynamic symbol of the product library: no C++ helper, no kernel stub, no measurement door
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", LIB], capture_output=True, text=True, check=True).stdout
+    exported = {ln.split()[-1] for ln in out.splitlines() if len(ln.split()) == 3 and ln.split()[1] in "TDBRW"}
+    assert exported == declared, sorted(exported ^ declared)
 
 
 def test_version_and_error_slot(lib):

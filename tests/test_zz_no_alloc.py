@@ -36,7 +36,7 @@ def _call(st, q, static):
     out = torch.full((B, Hq, 128), float("nan"), dtype=torch.float32, device=DEV)
     lse = torch.full((B, Hq), float("nan"), dtype=torch.float32, device=DEV)
     common = (q.data_ptr(), _lib.dtype_code(q), B, Hq, 128 ** -0.5, C.byref(st._packed), C.byref(st._worklist),
-              st._pi_k_t.data_ptr(), st.pi_v.data_ptr(), st._decode_cb.data_ptr(), st._decode_cb_host, st._decode_inv, out.data_ptr(), _lib.F32, lse.data_ptr())
+              st._pi_k_ops.data_ptr(), st.pi_v.data_ptr(), st._decode_cb.data_ptr(), st._decode_cb_host, st._decode_inv, out.data_ptr(), _lib.F32, lse.data_ptr())
     stream = _lib.stream_ptr(torch.device(DEV, torch.cuda.current_device()))
     if static:
         rc = lib.odmkv_decode_attn_static(*common, stream)
@@ -74,7 +74,7 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     work.items, work.item_range, work.n_items = big._items[0].data_ptr(), big._items[1].data_ptr(), n_items
     out = torch.zeros(2, 14, 128, device=DEV)
     rc = lib.odmkv_decode_attn_static(q_big.data_ptr(), _lib.F16, 2, 14, 0.1, C.byref(big._packed), C.byref(work),
-                                      big._pi_k_t.data_ptr(), big.pi_v.data_ptr(), big._decode_cb.data_ptr(), big._decode_cb_host, big._decode_inv, out.data_ptr(),
+                                      big._pi_k_ops.data_ptr(), big.pi_v.data_ptr(), big._decode_cb.data_ptr(), big._decode_cb_host, big._decode_inv, out.data_ptr(),
                                       _lib.F32, None, None)
     assert rc == -2 and b"fixed array" in lib.odmkv_last_error()
     torch.cuda.synchronize()
