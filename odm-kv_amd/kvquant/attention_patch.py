@@ -2,12 +2,13 @@
 
 Stands where the reference's kvquant/attention_patch.py:13-62 stands.  Two behaviours:
 
-* decode (one query token) on a module whose layer has a packed store attached
-  (``module._odmkv_state``): the attention output comes from the fused LUT kernel over the packed
-  cache (``TurboQuantAdaptiveKVCacheState.decode_attention``); the dense ``key``/``value`` tensors
-  handed in by the model are not read, except for the newest token, which the store does not hold
-  yet when the attention function runs (the press appends it in its forward hook, afterwards).
-  Evicted tokens are absent from the store, so no fake keys are needed.
+* decode (one query token, or a block of new tokens such as the question after a prefill) on a module
+  whose layer has a packed store attached (``module._odmkv_state``): the attention output comes from
+  the fused LUT kernel over the packed cache (``TurboQuantAdaptiveKVCacheState.decode_attention`` /
+  ``decode_attention_block``); the dense ``key``/``value`` tensors handed in by the model are not read,
+  except for the new tokens, which the store does not hold yet when the attention function runs (the
+  press appends them in its forward hook, afterwards).  Evicted tokens are absent from the store, so
+  no fake keys are needed.
 * everything else goes to the wrapped attention function as in the reference, with evicted keys
   replaced by a fake key whose weight underflows to zero (``search_hyperplane``).
 """
@@ -42,23 +43,44 @@ def fused_decode_enabled() -> bool:
     return os.environ.get("ODMKV_FUSED_DECODE", "1") != "0"
 
 
+_causal_checked: dict = {}
+
+
+def _store_part_is_open(attention_mask: torch.Tensor, store_len: int) -> bool:
+    """True when the boolean / additive mask of a multi-token step lets every query see every stored token (what a
+    causal mask without padding does).  The same mask object goes to every layer of a forward: checked once."""
+    hit = _causal_checked.get("last")
+    if hit is not None and hit[0] is attention_mask and hit[1] == store_len:      # (the entry keeps the tensor alive)
+        return hit[2]
+    part = attention_mask[..., :store_len]
+    ok = bool(part.all()) if attention_mask.dtype == torch.bool else bool((part == 0).all())
+    _causal_checked["last"] = (attention_mask, store_len, ok)
+    return ok
+
+
 def _fused_decode(module, query, key, value, attention_mask, dropout, kwargs):
-    """Attention output [B, 1, Hq, D] from the packed store, or None when this call is not a plain
-    single-token decode over a store that is in step with the dense cache."""
+    """Attention output [B, L, Hq, D] from the packed store, or None when this call is not a decode step (one token, or
+    a block of tokens that all see the whole store) over a store that is in step with the dense cache."""
     state = getattr(module, "_odmkv_state", None)
     if state is None or not fused_decode_enabled():
         return None
-    if query.shape[2] != 1 or attention_mask is not None or dropout:
+    B, Hq, L, D = query.shape
+    if dropout or (L == 1 and attention_mask is not None):
         return None
     if kwargs.get("sliding_window") is not None or kwargs.get("softcap") is not None or kwargs.get("s_aux") is not None:
         return None
-    k_len = key.shape[2]
-    if state.seq_len not in (k_len - 1, k_len) or state.batch_size != query.shape[0]:
+    # a cache layer without a dense copy hands over the new tokens only, tagged with the store's length
+    store_len = getattr(key, "_odmkv_store_len", None)
+    k_len = key.shape[2] if store_len is None else store_len + key.shape[2]
+    if state.batch_size != B:
         return None
     scaling = kwargs.get("scaling")
     if scaling is None:
-        scaling = query.shape[-1] ** -0.5
-    B, Hq, _, D = query.shape
+        scaling = D ** -0.5
+    if L > 1:
+        return _fused_block(state, query, key, value, attention_mask, scaling, k_len)
+    if state.seq_len not in (k_len - 1, k_len):
+        return None
     if state.seq_len == k_len - 1 and getattr(state, "exact_decode_append", False):
         # the press keeps new tokens exact until its buffer flushes: store the token now, the
         # press's hook sees the store already in step and does not append it again
@@ -79,13 +101,48 @@ def _fused_decode(module, query, key, value, attention_mask, dropout, kwargs):
     return out.to(query.dtype).view(B, 1, Hq, D)
 
 
+def _fused_block(state, query, key, value, attention_mask, scaling, k_len):
+    """A block of L new tokens after the prefill (the reference runner feeds every question this way,
+    benchmark/core/pipeline.py:170-185; the reference's wrapper treats any q_len != k_len alike,
+    attention_patch.py:38-48): every new token sees the whole store, through the fused kernel, and the new tokens at or
+    before its own position, through a small dense product over the L tokens the model handed over; the two parts
+    are merged by their log-sum-exps.  The store must not hold the new tokens yet (the press appends them in its
+    hook, afterwards), and the mask, if there is one, must leave the stored tokens open."""
+    B, Hq, L, D = query.shape
+    if state.seq_len != k_len - L:
+        return None
+    if attention_mask is not None:
+        if attention_mask.dim() != 4 or attention_mask.shape[-2] != L or attention_mask.shape[-1] != k_len:
+            return None
+        if not _store_part_is_open(attention_mask, k_len - L):
+            return None
+    out_s, lse_s = state.decode_attention_block(query, scaling=scaling)          # [B, Hq, L, D], [B, Hq, L]
+    G = Hq // key.shape[1]
+    k_new = key[:, :, -L:, :].float().repeat_interleave(G, dim=1)                # [B, Hq, L, D]
+    v_new = value[:, :, -L:, :].float().repeat_interleave(G, dim=1)
+    logits = torch.matmul(query.float(), k_new.transpose(-1, -2)) * scaling      # [B, Hq, L, L]
+    if attention_mask is None:
+        keep = torch.ones(L, L, dtype=torch.bool, device=query.device).tril()
+        logits = logits.masked_fill(~keep, float("-inf"))
+    elif attention_mask.dtype == torch.bool:
+        logits = logits.masked_fill(~attention_mask[..., -L:], float("-inf"))
+    else:
+        logits = logits + attention_mask[..., -L:].float()
+    lse_n = torch.logsumexp(logits, dim=-1)                                      # every token sees itself: finite
+    out_n = torch.matmul(torch.exp(logits - lse_n.unsqueeze(-1)), v_new)
+    m = torch.maximum(lse_s, lse_n)
+    w_s, w_n = torch.exp(lse_s - m).unsqueeze(-1), torch.exp(lse_n - m).unsqueeze(-1)
+    out = (out_s * w_s + out_n * w_n) / (w_s + w_n)
+    return out.to(query.dtype).transpose(1, 2).contiguous()                      # [B, L, Hq, D]
+
+
 def _attention_patch(func):
     if getattr(func, _PATCH_ATTR, False):
         return func
 
     @functools.wraps(func)
     def wrapper(module, query, key, value, attention_mask, dropout=0.0, **kwargs):
-        if query.shape[2] == key.shape[2]:
+        if query.shape[2] == key.shape[2] and not hasattr(key, "_odmkv_store_len"):      # a prefill (no cached tokens)
             module.masked_key_indices = None
             module._odmkv_state = None
         else:
@@ -97,7 +154,7 @@ def _attention_patch(func):
             if fused is not None:
                 call_counts["fused"] += 1
                 return fused, None
-            if key.dim() == 4 and key.shape[2] > 1 and key.stride(2) == 0:
+            if (key.dim() == 4 and key.shape[2] > 1 and key.stride(2) == 0) or hasattr(key, "_odmkv_store_len"):
                 raise RuntimeError(
                     "this layer's dense cache was released (release_dense_cache=True) and the call cannot take the "
                     "fused decode path (padding mask, dropout, sliding window, soft cap or a batch the store was "

@@ -11,8 +11,8 @@ prefill has been packed:
   are stride-0 views of the newest token: no memory, no concatenation;
 * a single-token ``update`` re-aliases the views; the attention function takes the token from
   them and everything older from the store;
-* an ``update`` with several tokens (prompt text after the prefill) dequantises the store once,
-  returns real dense tensors for that call and drops them again;
+* an ``update`` with several tokens (prompt text after the prefill) returns the new tokens alone, tagged
+  with the store's length: the attention patch runs the block through the fused kernel as well;
 * ``crop`` truncates the store; a harness that rewinds the cache the reference's way
   (benchmark/core/pipeline.py:211-228: ``layer._tq_backend_state.truncate`` and a slice of
   ``layer.keys``) works on it unchanged.
@@ -54,12 +54,13 @@ class PackedCacheLayer(DynamicLayer):
         if self.state.seq_len != before:
             raise RuntimeError(f"the packed store holds {self.state.seq_len} tokens, the cache layer {before}: "
                                "a multi-token step needs the two in step")
-        dense_k, dense_v = self.state.materialize()
-        keys = torch.cat([dense_k.to(key_states.dtype), key_states], dim=-2)
-        values = torch.cat([dense_v.to(value_states.dtype), value_states], dim=-2)
+        # the new tokens alone, tagged with the number of tokens the store holds: the attention patch takes the
+        # stored part from the fused kernel and the block's own attention from these (nothing is dequantised)
+        key_states._odmkv_store_len = before
+        value_states._odmkv_store_len = before
         self.recent = (key_states, value_states)
         self._alias(before + q_len)
-        return keys, values
+        return key_states, value_states
 
     def crop(self, tokens_to_remove: int) -> None:
         current = self.keys.shape[-2]

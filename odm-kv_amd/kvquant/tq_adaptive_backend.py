@@ -799,6 +799,35 @@ class TurboQuantAdaptiveKVCacheState:
         w.wavefronts = int(os.environ.get("ODMKV_DECODE_WAVES", 0)) or auto
         self._worklist = w
 
+    def decode_attention_block(self, query: torch.Tensor, scaling: Optional[float] = None):
+        """The same for a block of L query tokens per sequence that all see the whole store (the question after a
+        prefill, a draft to verify): query [B, Hq, L, D] -> (out fp32 [B, Hq, L, D], lse fp32 [B, Hq, L]).
+
+        The kernel's GQA sharing carries the block: the L tokens of a kv-head's G query heads are handed over as G * L
+        heads of that kv-head, up to 8 per call, so the packed bytes are streamed once per 8 // G tokens instead of
+        once per token (attention among the L tokens themselves is the caller's: see attention_patch)."""
+        _lib.require_gpu(query, "query")
+        if query.dim() != 4:
+            raise ValueError(f"query must be [B, Hq, L, D], got {tuple(query.shape)}")
+        B, Hq, L, D = query.shape
+        H = self.num_heads
+        if Hq % H:
+            raise ValueError(f"{Hq} query heads do not divide over {H} kv heads")
+        G = Hq // H
+        if G > 8:
+            raise ValueError(f"GQA group {G} exceeds 8")
+        per = max(1, 8 // G)
+        out = torch.empty(B, Hq, L, D, dtype=torch.float32, device=self.device)
+        lse = torch.empty(B, Hq, L, dtype=torch.float32, device=self.device)
+        q5 = query.reshape(B, H, G, L, D)
+        for l0 in range(0, L, per):
+            lc = min(per, L - l0)
+            qv = q5[:, :, :, l0:l0 + lc].permute(0, 1, 3, 2, 4).reshape(B, H * lc * G, D).contiguous()
+            o, s = self.decode_attention(qv, scaling=scaling, return_lse=True)
+            out.view(B, H, G, L, D)[:, :, :, l0:l0 + lc] = o.view(B, H, lc, G, D).permute(0, 1, 3, 2, 4)
+            lse.view(B, H, G, L)[:, :, :, l0:l0 + lc] = s.view(B, H, lc, G).permute(0, 1, 3, 2)
+        return out, lse
+
     def decode_attention(self, query: torch.Tensor, scaling: Optional[float] = None,
                          return_lse: bool = False, out_dtype: torch.dtype = torch.float32):
         """softmax(scaling * q K^T) V over the stored tokens, for one query token per sequence.

@@ -142,6 +142,30 @@ def test_long_items_of_a_small_group_take_the_shared_lane_form(G):
     assert rel_err(st.decode_attention(q.to(DEV)).cpu(), want) < ATTN_RTOL
 
 
+@pytest.mark.parametrize("L,G,Hkv,T", [(2, 4, 2, 900), (7, 4, 2, 1500), (32, 4, 1, 700), (5, 7, 1, 400), (9, 1, 2, 300), (3, 8, 1, 260)])
+def test_block_of_query_tokens_matches_oracle(L, G, Hkv, T):
+    """decode_attention_block: L query tokens per sequence that all see the whole store (the question after a
+    prefill, which the reference feeds as one multi-token forward, benchmark/core/pipeline.py:170-185): every
+    token's output and log-sum-exp against the oracle, token by token, on a mixed-level store."""
+    g = torch.Generator().manual_seed(100 * L + G)
+    B = 2 if T < 500 else 1
+    k = torch.randn(B, Hkv, T, 128, generator=g).half(); v = torch.randn(B, Hkv, T, 128, generator=g).half()
+    bits = _rand_bits(g, (B, Hkv, T), (0.2, 0.4, 0.15, 0.1, 0.1, 0.05)); bits[..., :4] = 16; bits[..., -8:] = 16
+    st, ref = _pair(k, v, bits)
+    q = torch.randn(B, Hkv * G, L, 128, generator=g).half()
+    out, lse = st.decode_attention_block(q.to(DEV))
+    assert out.shape == (B, Hkv * G, L, 128) and lse.shape == (B, Hkv * G, L)
+    kk, vv = ref.materialize()
+    alive = ref.visible_mask()
+    for l in range(L):
+        ql = q[:, :, l].float()
+        want = decode_attention_state(ql, ref)
+        assert rel_err(out[:, :, l].cpu(), want) < ATTN_RTOL, l
+        logits = torch.einsum("bhd,bhtd->bht", ql.double(), kk.double().repeat_interleave(G, dim=1)) * 128 ** -0.5
+        logits = logits.masked_fill(~alive.repeat_interleave(G, dim=1), float("-inf"))
+        np.testing.assert_allclose(lse[:, :, l].cpu().numpy(), torch.logsumexp(logits, -1).numpy(), rtol=2e-3, atol=2e-3)
+
+
 def test_decode_replayed_from_a_graph_matches_eager():
     """The three launches of a decode call captured in a HIP graph and replayed with new queries in the
     captured buffer, with eager work and synchronisations between the replays: every replay must give

@@ -466,3 +466,54 @@ def test_second_prompt_through_one_press_flushes_with_its_own_shares():
         first, second = seen[layer], seen[2 + layer]
         assert first[1] != second[1]                              # the two prefills left different shares ...
         assert sorted(first[2].tolist()) != sorted(second[2].tolist())       # ... and the flushes different tier sizes
+
+
+@torch.inference_mode()
+@pytest.mark.parametrize("release", [False, True])
+def test_question_block_takes_the_fused_path(release):
+    """The reference's runner feeds every question as ONE multi-token forward over the compressed cache
+    (benchmark/core/pipeline.py:170-185).  That forward must run on the fused kernel too (stored tokens through
+    decode_attention_block, the question's own causal part densely over its few tokens), give the logits of the dense
+    path at every question position, and, with the dense copy released, dequantise nothing."""
+    from transformers import DynamicCache
+    from kvquant import attention_patch
+    from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+    model = _model(12)
+    T, n_q = 700, 9
+    ids = _ids(T, 81)
+    question = torch.randint(0, 1000, (1, n_q), generator=torch.Generator().manual_seed(82)).to(DEV)
+    pos = torch.arange(T, T + n_q, device=DEV).view(1, -1)
+    n_layers = len(model.model.layers)
+
+    def run(fused, released):
+        os.environ["ODMKV_FUSED_DECODE"] = "1" if fused else "0"
+        try:
+            press = _press(release_dense_cache=released)
+            cache = DynamicCache()
+            with press(model):
+                model.model(input_ids=ids, past_key_values=cache)
+                before = dict(attention_patch.call_counts)
+                out = model(input_ids=question, past_key_values=cache, position_ids=pos)
+                took = {k: attention_patch.call_counts[k] - before[k] for k in before}
+                # and one ordinary step after the block: the store took the question's tokens
+                nxt = model(input_ids=question[:, :1], past_key_values=cache, position_ids=torch.tensor([[T + n_q]], device=DEV))
+                assert all(st.seq_len == T + n_q + 1 for st in press._states.values())
+            return out.logits[0].float(), nxt.logits[0, -1].float(), took
+        finally:
+            os.environ.pop("ODMKV_FUSED_DECODE", None)
+
+    dense, dense_next, took_d = run(False, False)
+    assert took_d == {"fused": 0, "dense": n_layers}
+    orig = TurboQuantAdaptiveKVCacheState.materialize
+    if release:
+        def refuse(self, *a, **kw):
+            raise AssertionError("the store was dequantised for a multi-token step")
+        TurboQuantAdaptiveKVCacheState.materialize = refuse
+    try:
+        fused, fused_next, took_f = run(True, release)
+    finally:
+        TurboQuantAdaptiveKVCacheState.materialize = orig
+    assert took_f == {"fused": n_layers, "dense": 0}
+    assert fused.shape == (n_q, 1000)
+    assert (fused - dense).abs().max().item() < LOGIT_ATOL
+    assert (fused_next - dense_next).abs().max().item() < LOGIT_ATOL
