@@ -9,6 +9,8 @@ under the press at 2.0 average bits, then 256 greedy tokens over the packed cach
   dense re-materialised cache with the model's own attention (what the reference executes), under teacher forcing,
   across a flush of the 128-token decode buffer.
 """
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -35,9 +37,13 @@ def _c2_model(layers=2):
         torch.set_default_dtype(default)
 
 
-def test_c2_stack_prefill_32k_then_256_greedy_tokens():
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+def test_c2_stack_prefill_32k_then_256_greedy_tokens(dtype):
+    """bf16 (what Llama-3 checkpoints ship in): exact tokens are stored as bf16 and the model rounds every logit to
+    bf16's eight significant bits, so the two attention paths may differ by a few of those steps (three, at the
+    largest logit of the run)."""
     from kvquant.allocator import calibrate_epsilon
-    model = _c2_model()
+    model = _c2_model().to(dtype)
     ids = _ids(T, 21)
     # the reference's path first: dense re-materialised cache, the model's own attention
     tok_d, log_d, _, _ = _generate(model, _press(target=2.0), ids, N_NEW, fused=False)
@@ -54,13 +60,17 @@ def test_c2_stack_prefill_32k_then_256_greedy_tokens():
     press._score_prefill = spy
     tok_f, log_f, cache, states = _generate(model, press, ids, N_NEW, forced=tok_d, fused=True)
     err = (log_f - log_d).abs().max().item()
-    assert err < LOGIT_ATOL, err
+    top = log_d.abs().max().item()
+    bf16_step = 2.0 ** (math.floor(math.log2(top)) - 7)
+    logit_atol, min_agree = (LOGIT_ATOL, 0.97) if dtype == torch.float16 else (3 * bf16_step, 0.95)
+    assert err <= logit_atol, (err, top)
     agree = (log_f.argmax(-1) == tok_d).float().mean().item()
-    assert agree >= 0.97, agree
+    assert agree >= min_agree, agree
 
     eps = calibrate_epsilon(128, LEVELS, seed=42, device=DEV, value_quantizer="mse")
     assert sorted(states) == [0, 1]
     for layer_idx, st in states.items():
+        assert st._exact_torch_dtype == dtype
         assert st.seq_len == T + N_NEW - 1
         lm = st._level_map[0].cpu().numpy()
         # the prefill's part of the store: the oracle allocator on the same scores, window and sinks exact

@@ -3,6 +3,11 @@ CPU oracle to run at that size (it would take minutes): the allocation against t
 the GPU's own scores (bit exact; the oracle allocator is fast), budget and sink/window invariants,
 the partition of every position over the levels, and the fused decode attention against dense
 attention over the store's own dequantised tensors (<= 1e-3 relative, the stated tolerance).
+
+One kv-head of each configuration is small enough for the oracle (a hundred thousand tokens quantise in seconds in
+its fixed-order C restatement): for that head the attention of its query group is compared with the oracle's own
+store, built from the same keys, values and stored levels, so the full-size result does not rest on the GPU's own
+dequantiser alone.
 """
 import numpy as np
 import pytest
@@ -65,6 +70,27 @@ def _check_attention(st, layers, G):
     return err
 
 
+def _check_attention_against_oracle(st, layers, stored, G, b=0, h=0):
+    """The query group of kv-head (b, h): fused attention over the whole store against the oracle's attention over its
+    own store of that head alone (fixed-order quantiser, keys and values dequantised in fp32 and then, as the
+    reference does, in fp16).  Tokens appended after the prefill are not covered: call before any append."""
+    from oracle.attention import decode_attention_state
+    from oracle.kvstate import KVState
+    L = layers[b]
+    k, v = L.keys[None, h:h + 1], L.values[None, h:h + 1]
+    bits = stored[b:b + 1, h:h + 1].cpu()
+    q = L.query[None, h * G:(h + 1) * G].float()
+    fused = st.decode_attention(torch.stack([x.query for x in layers]).to(DEV))[b, h * G:(h + 1) * G].cpu().double()
+    errs = {}
+    for name, dt in (("fp32", torch.float32), ("fp16", torch.float16)):
+        ref = KVState(128, LEVELS, dtype=dt, seed=42, order="canonical")
+        ref.prefill(k.to(dt), v.to(dt), bits)
+        want = decode_attention_state(q, ref)[0]
+        errs[name] = ((fused - want).norm(dim=-1) / want.norm(dim=-1)).max().item()
+    assert errs["fp32"] < ATTN_RTOL, errs
+    return errs
+
+
 def _check_levels(st, stored):
     lm = st._level_map
     assert torch.equal(lm.to(torch.int32), stored)
@@ -91,6 +117,7 @@ def test_c3_sixteen_sequences_with_cycling_budgets():
         assert (bits[s, :, :4] == 16).all()
     _check_levels(st, stored)
     _check_attention(st, layers, 4)
+    _check_attention_against_oracle(st, layers, stored, 4, b=7, h=3)
 
 
 def test_c4_long_context_heavy_eviction():
@@ -108,6 +135,7 @@ def test_c4_long_context_heavy_eviction():
     masked = st.masked_key_indices()
     assert masked[0].numel() == int((stored == 0).sum())
     _check_attention(st, [L], 4)
+    _check_attention_against_oracle(st, [L], stored, 4, h=5)
     # 128 decode steps keep new tokens exact and visible
     g = torch.Generator().manual_seed(9)
     new_k = torch.randn(128, 1, 8, 1, 128, generator=g).half().to(DEV)
@@ -134,6 +162,7 @@ def test_c5_group_of_seven_heavy_tailed_values():
     assert len(used) >= 4, used                          # a 3-bit budget on heavy tails spreads over the levels
     _check_levels(st, stored)
     _check_attention(st, [L], 7)
+    _check_attention_against_oracle(st, [L], stored, 7, h=2)
 
 
 def test_c2_one_layer_pack_and_decode_at_full_size():
@@ -148,6 +177,7 @@ def test_c2_one_layer_pack_and_decode_at_full_size():
     assert torch.equal(bits[0].cpu(), want)
     _check_levels(st, stored)
     _check_attention(st, [L], 4)
+    _check_attention_against_oracle(st, [L], stored, 4, h=6)
 
 
 def test_c2_one_layer_score_matches_oracle_at_full_size():
@@ -159,21 +189,24 @@ def test_c2_one_layer_score_matches_oracle_at_full_size():
     np.testing.assert_allclose(got.numpy(), want.numpy(), rtol=1e-3, atol=0)
 
 
-def test_c2_one_layer_fp16_store_equals_the_exact_quantisers_at_full_size():
-    """fp16 tensors are quantised through the matrix-core estimate plus exact codes next to the thresholds, fp32
-    tensors by the exact kernel alone: on a whole 32k-token layer (2.7e8 rotated values, levels
-    drawn at random over widths 2, 3 and 4) both must leave the same bytes."""
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+def test_c2_one_layer_16bit_store_equals_the_exact_quantisers_at_full_size(dtype):
+    """fp16 and bf16 tensors are quantised through the matrix-core estimate plus exact codes next to the thresholds,
+    fp32 tensors by the exact kernel alone: on a whole 32k-token layer (2.7e8 rotated values, levels
+    drawn at random over widths 2, 3 and 4) both must leave the same bytes.  (bf16 rows meet the rotation as two
+    bf16 terms: a wider guard band, the same exact codes.)"""
     from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
     L = synthetic.config("c2", layer=9)
+    L.keys, L.values = L.keys.to(dtype), L.values.to(dtype)
     g = torch.Generator().manual_seed(9)
     pick = torch.multinomial(torch.tensor([0.02, 0.45, 0.3, 0.2, 0.0, 0.03]), 8 * 32768, replacement=True, generator=g)
     stored = torch.tensor(LEVELS, dtype=torch.int32)[pick].reshape(1, 8, 32768).to(DEV)
-    st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=DEV, dtype=torch.float16, key_quantizer="mse",
+    st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=DEV, dtype=dtype, key_quantizer="mse",
                                         value_quantizer="mse", seed=42)
     st.prefill(L.keys[None].to(DEV), L.values[None].to(DEV), stored)
     counts = st.level_counts()
     assert min(counts[2], counts[3], counts[4]) > 10000 and counts[8] == 0
-    ref = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=DEV, dtype=torch.float16, key_quantizer="mse",
+    ref = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=DEV, dtype=dtype, key_quantizer="mse",
                                          value_quantizer="mse", seed=42)
     ref.prefill(L.keys[None].to(DEV).float(), L.values[None].to(DEV).float(), stored)
     assert np.array_equal(st._seg_tile, ref._seg_tile)
