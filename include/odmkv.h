@@ -395,6 +395,31 @@ int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, float scaling,
                       void* out, int out_dtype, float* lse, void* workspace, size_t workspace_bytes,
                       void* stream);
 
+/* One decode step of a layer in one call, for a serving loop whose host time per layer matters: the step's new token
+ * of every (sequence, kv-head) is stored exact behind the others (odmkv_append_exact: k_new, v_new, strides, pos as
+ * there; both NULL = the store already holds it), then odmkv_decode_attn runs for the step's query over the store, the
+ * new token included.  Stands where the reference's forward hook appends the token to its state and the model then
+ * attends over the re-materialised cache (kvquant/adaptive_backend_press.py:221-262; append_all_exact,
+ * kvquant/tq_adaptive_backend.py:412-440).  What does not change from step to step sits in a block the caller fills
+ * once per store and work list (the pointers in it are those of odmkv_decode_attn and must stay valid); q, out and lse
+ * as in odmkv_decode_attn.  Three launches on `stream`. */
+typedef struct odmkv_step {
+    const odmkv_packed_t* store;
+    const odmkv_worklist_t* work;
+    const uint16_t* pi_k_ops;
+    const float* pi_v;
+    const float* codebooks;
+    const float* codebooks_host;
+    const float* inv_scales;
+    void* workspace;
+    size_t workspace_bytes;
+    int32_t B, Hq;
+    int32_t q_dtype, out_dtype;
+    float scaling;
+} odmkv_step_t;
+int odmkv_decode_step(const odmkv_step_t* step, const void* q, const void* k_new, const void* v_new,
+                      int64_t stride_b, int64_t stride_h, int pos, void* out, float* lse, void* stream);
+
 /* The same call without a workspace, for callers that cannot allocate device memory and have none
  * to hand over (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
  * No counterpart in the reference.  The per-item partial results live in

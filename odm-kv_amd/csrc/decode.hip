@@ -1245,6 +1245,20 @@ extern "C" int odmkv_decode_attn(const void* q, int q_dtype, int B, int Hq, floa
                                out, out_dtype, lse, workspace, workspace_bytes, stream, 7, nullptr, nullptr);
 }
 
+// One decode step of a layer in a single call: the new token of every (sequence, kv-head) goes behind the stored
+// exact tokens, then the attention of the step's query runs over the store, the new token included.
+extern "C" int odmkv_decode_step(const odmkv_step_t* step, const void* q, const void* k_new, const void* v_new,
+                                 int64_t stride_b, int64_t stride_h, int pos, void* out, float* lse, void* stream) {
+    ODMKV_CHECK_ARG(step != nullptr, "decode_step: null step block");
+    if (k_new || v_new) {
+        ODMKV_CHECK_ARG(step->store != nullptr, "decode_step: null store");
+        if (int rc = odmkv_append_exact(step->store, k_new, v_new, stride_b, stride_h, pos, stream)) return rc;
+    }
+    return odmkv_decode_launch(q, step->q_dtype, step->B, step->Hq, step->scaling, step->store, step->work, step->pi_k_ops,
+                               step->pi_v, step->codebooks, step->codebooks_host, step->inv_scales, out, step->out_dtype, lse,
+                               step->workspace, step->workspace_bytes, stream, 7, nullptr, nullptr);
+}
+
 // ------------------------------------------------------------------------------------------------
 // The same call for callers that cannot allocate and have no workspace to hand over: the prepared
 // queries and the partial results live in a fixed array of the library's own device image.

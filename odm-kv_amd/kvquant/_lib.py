@@ -44,6 +44,16 @@ class Worklist(C.Structure):
     ]
 
 
+class Step(C.Structure):
+    """struct odmkv_step of include/odmkv.h."""
+    _fields_ = [
+        ("store", C.POINTER(Packed)), ("work", C.POINTER(Worklist)), ("pi_k_ops", C.c_void_p), ("pi_v", C.c_void_p),
+        ("codebooks", C.c_void_p), ("codebooks_host", C.POINTER(C.c_float)), ("inv_scales", C.POINTER(C.c_float)),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("B", C.c_int32), ("Hq", C.c_int32),
+        ("q_dtype", C.c_int32), ("out_dtype", C.c_int32), ("scaling", C.c_float),
+    ]
+
+
 def _load() -> C.CDLL:
     if not os.path.exists(LIB_PATH):
         raise ImportError(
@@ -88,6 +98,7 @@ def _load() -> C.CDLL:
                                         C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp, sz, vp]),
         "odmkv_decode_attn_static": (C.c_int, [vp, i32, i32, i32, f32, C.POINTER(Packed), C.POINTER(Worklist), vp, vp, vp,
                                                C.POINTER(C.c_float), C.POINTER(C.c_float), vp, i32, vp, vp]),
+        "odmkv_decode_step": (C.c_int, [C.POINTER(Step), vp, vp, vp, i64, i64, i32, vp, vp, vp]),
         "odmkv_exact_tail": (C.c_int, [C.POINTER(Packed), i32, vp, vp, vp]),
         "odmkv_flush_score": (C.c_int, [vp, vp, i32, i32, i32, vp, f32, f32, i32, vp, vp, vp, vp]),
         "odmkv_flush_rank": (C.c_int, [vp, vp, i32, i32, i32, vp, vp, vp]),
@@ -106,7 +117,7 @@ EXPORTS = ("odmkv_version", "odmkv_last_error", "odmkv_score_workspace_bytes", "
            "odmkv_store_init", "odmkv_store_gather", "odmkv_quant_pack_staged", "odmkv_store_layout", "odmkv_store_bind", "odmkv_pack_workspace_bytes", "odmkv_pack_count_chunks", "odmkv_store_finish_staged", "odmkv_quant_pack", "odmkv_quantize_rows",
            "odmkv_dequantize_rows", "odmkv_lloyd_max", "odmkv_dequant", "odmkv_dequant_from", "odmkv_append_exact",
            "odmkv_decode_workspace_bytes", "odmkv_rotation_operands", "odmkv_decode_attn", "odmkv_decode_attn_static",
-           "odmkv_exact_tail", "odmkv_flush_score", "odmkv_flush_rank")
+           "odmkv_decode_step", "odmkv_exact_tail", "odmkv_flush_score", "odmkv_flush_rank")
 
 
 def check(rc: int) -> None:

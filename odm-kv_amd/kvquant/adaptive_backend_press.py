@@ -118,10 +118,20 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         cache.layers[layer_idx] = PackedCacheLayer(state, keys, values)
 
     def _attach(self, cache, layer_idx: int, module: nn.Module, state) -> None:
-        module.masked_key_indices = state.masked_key_indices()
-        module._odmkv_state = state
+        # plain attributes, set past nn.Module's own __setattr__ (its checks for parameters, buffers and submodules cost
+        # more than the rest of the hook on a decode step)
+        object.__setattr__(module, "masked_key_indices", state.masked_key_indices())
+        object.__setattr__(module, "_odmkv_state", state)
         if hasattr(cache, "layers"):
             cache.layers[layer_idx]._tq_backend_state = state
+
+    @staticmethod
+    def _attached(cache, layer_idx: int, module: nn.Module, state) -> bool:
+        """Whether _attach(state) has run for this module and cache layer (an exact append changes nothing it sets)."""
+        if module.__dict__.get("_odmkv_state") is not state:
+            return False
+        layers = getattr(cache, "layers", None)
+        return layers is None or getattr(layers[layer_idx], "_tq_backend_state", None) is state
 
     def _sync_cache_from_state(self, cache, layer_idx: int, module: nn.Module, state, *, prefill_fast: bool = False,
                                start: int = 0) -> None:
@@ -250,6 +260,15 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
                 self._buffer_counts[layer_idx] = 0
 
         already_stored = state.seq_len == cache_len       # the fused attention path stored the token
+        if already_stored and q_len == 1 and self.buffer_size > 0:
+            # the usual decode step: nothing to store, the buffer grows by one token
+            count = self._buffer_counts.get(layer_idx, 0) + 1
+            self._buffer_counts[layer_idx] = count
+            if count >= self.buffer_size:
+                self._flush_decode_buffer(state, layer_idx, cache, module, hidden_states)
+            elif not self._attached(cache, layer_idx, module, state):
+                self._attach(cache, layer_idx, module, state)
+            return output
         packed_layer = self._packed_layer(cache, layer_idx)
         if packed_layer is not None:
             new_k, new_v = packed_layer.recent            # the layer's tensors alias one token

@@ -82,9 +82,10 @@ def _fused_decode(module, query, key, value, attention_mask, dropout, kwargs):
     if state.seq_len not in (k_len - 1, k_len):
         return None
     if state.seq_len == k_len - 1 and getattr(state, "exact_decode_append", False):
-        # the press keeps new tokens exact until its buffer flushes: store the token now, the
-        # press's hook sees the store already in step and does not append it again
-        state.append_all_exact(key[:, :, -1:, :], value[:, :, -1:, :])
+        # the press keeps new tokens exact until its buffer flushes: store the token now (the press's hook sees
+        # the store already in step and does not append it again) and attend, in one library call
+        return state.decode_step(query, key[:, :, -1:, :], value[:, :, -1:, :], scaling=scaling,
+                                 out_dtype=query.dtype).view(B, 1, Hq, D)
     if state.seq_len == k_len:
         return state.decode_attention(query, scaling=scaling, out_dtype=query.dtype).view(B, 1, Hq, D)
     else:
@@ -149,7 +150,7 @@ def _attention_patch(func):
             if query.shape[2] == 1:
                 # the newest token's query, after RoPE: the press's flush scores its buffer with it and need not
                 # project and rotate the hidden state a second time
-                module._odmkv_last_query = query
+                object.__setattr__(module, "_odmkv_last_query", query)         # (past nn.Module's slower __setattr__)
             fused = _fused_decode(module, query, key, value, attention_mask, dropout, kwargs)
             if fused is not None:
                 call_counts["fused"] += 1

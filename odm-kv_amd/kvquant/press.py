@@ -161,10 +161,10 @@ class TurboQuantPerTokenPress:
 
     @staticmethod
     def _get_cache_tensors(cache, layer_idx: int):
-        if hasattr(cache, "key_cache") and isinstance(cache.key_cache, list):
+        layers = getattr(cache, "layers", None)
+        if layers is None:                                   # caches of older transformers: two lists of tensors
             return cache.key_cache[layer_idx], cache.value_cache[layer_idx]
-        layer = cache.layers[layer_idx]
-        return layer.keys, layer.values
+        return layers[layer_idx].keys, layers[layer_idx].values
 
     @staticmethod
     def _set_cache_tensors(cache, layer_idx: int, keys: torch.Tensor, values: torch.Tensor) -> None:

@@ -264,6 +264,7 @@ class TurboQuantAdaptiveKVCacheState:
         self._items = None
         self._item_order = None
         self._worklist = None         # ctypes twin of odmkv_worklist_t over the tensors above
+        self._step = None             # decode_step's odmkv_step_t with what it was built for and what it points to
         self._items_choice = None     # (winning items-per-compute-unit multiple, packed bytes it was chosen at)
         self._packed = None
 
@@ -858,3 +859,44 @@ class TurboQuantAdaptiveKVCacheState:
             self._decode_cb_host, self._decode_inv, out.data_ptr(), _lib.dtype_code(out), _lib.ptr(lse), ws.data_ptr(), ws_bytes,
             _lib.stream_ptr(self.device)))
         return (out, lse) if return_lse else out
+
+    def decode_step(self, query: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, scaling: Optional[float] = None,
+                    out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """``append_all_exact(keys, values)`` (one new token, [B, Hkv, 1, D]) followed by ``decode_attention(query)``:
+        what one layer does in one decode step under a press that buffers new tokens exact.  When the exact segments
+        have room for the token (every step but the one in 64 that opens a tile) both run in one library call whose
+        constant arguments are kept in a block per store and work list."""
+        room = self._exact_room
+        if (room is None or room <= 0 or self._bufs is None or keys.shape[2] != 1 or keys.dtype != self._exact_torch_dtype
+                or self._level_store.shape[2] < self.seq_len + 1 or not query.is_contiguous()
+                or query.dtype not in (torch.float16, torch.bfloat16, torch.float32)):
+            self.append_all_exact(keys, values)
+            return self.decode_attention(query, scaling=scaling, out_dtype=out_dtype)
+        _lib.require_gpu(query, "query")
+        self._validate_shapes(keys, values, None)
+        B, Hq = query.shape[0], query.shape[1]
+        if self._items is None:
+            self._build_items()
+        scale = 1.0 / math.sqrt(self.head_dim) if scaling is None else float(scaling)
+        stream = _lib.stream_ptr(self.device)
+        key = (Hq, query.dtype, out_dtype, scale, stream)
+        blk = self._step
+        if blk is None or blk[4] is not self._packed or blk[5] is not self._worklist or blk[0] != key:
+            if B != self.batch_size or Hq % self.num_heads != 0 or query.numel() != B * Hq * self.head_dim:
+                raise ValueError(f"query {tuple(query.shape)} does not match the store (B={self.batch_size}, Hkv={self.num_heads})")
+            ws_bytes = lib.odmkv_decode_workspace_bytes(B, Hq, self._items[2])
+            ws = _lib.workspace(self.device, ws_bytes, "decode")
+            st = _lib.Step(C.pointer(self._packed), C.pointer(self._worklist), self._pi_k_ops.data_ptr(), self.pi_v.data_ptr(),
+                           self._decode_cb.data_ptr(), self._decode_cb_host, self._decode_inv, ws.data_ptr(), ws_bytes, B, Hq,
+                           _lib.dtype_code(query), _lib._DT[out_dtype], scale)
+            blk = self._step = (key, st, C.byref(st), ws, self._packed, self._worklist)
+        k, v = keys[:, :, 0, :], values[:, :, 0, :]
+        if k.stride(2) != 1 or v.stride() != k.stride():
+            k, v = k.contiguous(), v.contiguous()
+        out = torch.empty(B, Hq, self.head_dim, dtype=out_dtype, device=self.device)
+        _lib.check(lib.odmkv_decode_step(blk[2], query.data_ptr(), k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1),
+                                         self.seq_len, out.data_ptr(), None, stream))
+        self._counts[4] += 1
+        self._exact_room = room - 1
+        self.seq_len += 1
+        return out

@@ -219,6 +219,45 @@ def test_decode_after_appends_and_flush():
     assert rel_err(st.decode_attention(q.to(DEV)).cpu(), decode_attention_state(q, ref)) < ATTN_RTOL
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+def test_step_in_one_call_equals_append_then_attention(dtype):
+    """decode_step = append_all_exact + decode_attention: bit for bit the two separate calls on a twin store, over 140
+    steps (the exact segments open new tiles on the way, which takes the step through the separate calls), and the
+    oracle's attention at a few of them; the new token is read where the model's cache holds it (a strided row)."""
+    g = torch.Generator().manual_seed(31)
+    B, H, G, T = 2, 2, 4, 300
+    k = torch.randn(B, H, T, 128, generator=g).to(dtype); v = torch.randn(B, H, T, 128, generator=g).to(dtype)
+    bits = _rand_bits(g, (B, H, T), (0.2, 0.4, 0.15, 0.1, 0.05, 0.1)); bits[..., -20:] = 16
+    one, ref = _pair(k, v, bits, dtype=dtype)
+    two, _ = _pair(k, v, bits, dtype=dtype)
+    if dtype == torch.bfloat16:
+        # an oracle that materialises in bf16 rounds every dequantised key to eight bits (2.6e-3 on the output, its own
+        # error, not the kernel's): the fp32-materialising oracle over the same bf16 tokens is the yardstick
+        ref = KVState(128, (0, 2, 3, 4, 8, 16), dtype=torch.float32, seed=42, order="canonical")
+        ref.prefill(k.float(), v.float(), bits)
+    cache_k = torch.zeros(B, H, 140, 128, dtype=dtype, device=DEV); cache_v = torch.zeros_like(cache_k)
+    fast = 0
+    for step in range(140):
+        kn = torch.randn(B, H, 1, 128, generator=g).to(dtype); vn = torch.randn(B, H, 1, 128, generator=g).to(dtype)
+        cache_k[:, :, step:step + 1] = kn.to(DEV); cache_v[:, :, step:step + 1] = vn.to(DEV)
+        q = torch.randn(B, H * G, 1, 128, generator=g).to(dtype).to(DEV)
+        room = one._exact_room
+        got = one.decode_step(q, cache_k[:, :, step:step + 1], cache_v[:, :, step:step + 1], out_dtype=dtype)
+        fast += int(room is not None and room > 0)
+        two.append_all_exact(kn.to(DEV), vn.to(DEV))
+        want = two.decode_attention(q, out_dtype=dtype)
+        assert got.dtype == dtype and torch.equal(got, want), step
+        assert one.seq_len == two.seq_len == T + step + 1
+        ref.append_all_exact(kn.to(ref.dtype), vn.to(ref.dtype))
+        if step in (0, 70, 139):
+            got32 = one.decode_attention(q.float())
+            assert rel_err(got32.cpu(), decode_attention_state(q[:, :, 0].float().cpu(), ref)) < ATTN_RTOL
+    assert fast >= 120                                      # all but the steps that opened a tile took the single call
+    assert torch.equal(one._level_map, two._level_map) and one.level_counts() == two.level_counts()
+    ka, va = one.materialize(); kb, vb = two.materialize()
+    assert torch.equal(ka, kb) and torch.equal(va, vb)
+
+
 def test_config1_end_to_end():
     """Benchmark config 1: score -> allocate (2.0 bits) -> pack -> one-token decode, all on the GPU,
     each stage compared with the oracle fed the previous stage's GPU output."""
