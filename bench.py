@@ -42,11 +42,7 @@ for p in (ROOT, os.path.join(ROOT, "odm-kv_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the main decode kernel on the default workload, NOT measured by this run: from
-# the L2 counters of two rocprofv3 --pmc runs of `python bench.py --traffic-probe` (FETCH_SIZE, WRITE_SIZE),
-# each scaled by what the same counter reads for a 256 MiB device copy; the figures and the commands are in
-# profiles/decode_main_c2_32k_hbm_traffic.txt.  Applies to --layers 32 --ctx 32768 --target 2.0 only.
-TRAFFIC_FROM_PROFILE_BYTES = 20_959_000
+TRAFFIC_LAYERS = 6      # layers of the counter runs: the bytes per launch do not depend on how many layers take turns
 LEVELS = (0, 2, 3, 4, 8, 16)
 
 
@@ -60,7 +56,8 @@ def make_layer(li, n_kv, n_q, T, dev):
         L = synthetic.config("c5", layer=li, T=T)
     else:
         L = synthetic.gaussian_layer(2002 + li, n_kv, n_q, T)
-    return L.keys.to(dev), L.values.to(dev), L.mu.to(dev), L.query[None].to(dev)
+    # the decode query in the model's dtype, as a model hands it over (the generator keeps fp16 values in an fp32 tensor)
+    return L.keys.to(dev), L.values.to(dev), L.mu.to(dev), L.query[None].to(L.keys.dtype).to(dev)
 
 
 def load_bench_lib():
@@ -129,6 +126,60 @@ def parity_gate(dev):
     err = ((got - exp).norm(dim=-1) / exp.norm(dim=-1)).max().item()
     assert err < 1e-3, err
     return eps, err
+
+
+def measure_traffic(args):
+    """HBM bytes per launch of the main decode kernel, from the L2 counters, measured by this invocation: two child runs
+    of this file's --traffic-probe (the same workload, TRAFFIC_LAYERS layers) under ``rocprofv3 --pmc``, one counter
+    each (FETCH_SIZE, WRITE_SIZE; KiB per dispatch), each scaled by what the same counter reads for the probe's plain
+    256 MiB device copy.  Runs BEFORE this process touches the GPU (a child must not be started from a process that
+    holds the device), one child at a time, each under a hard time limit.  Returns (dict, None) or (None, reason)."""
+    import csv
+    import shutil
+    import subprocess
+    import tempfile
+    if shutil.which("rocprofv3") is None:
+        return None, "rocprofv3 not on PATH"
+    if any(k.startswith("ROCPROF") for k in os.environ) or "rocprof" in os.environ.get("LD_PRELOAD", ""):
+        return None, "this run is itself under a profiler"
+    tmp = tempfile.mkdtemp(prefix="odmkv_pmc_", dir="/tmp")
+    env = dict(os.environ, TMPDIR="/tmp")
+    res = {}
+    try:
+        for ctr in ("FETCH_SIZE", "WRITE_SIZE"):
+            cmd = ["timeout", "-s", "KILL", "240", "rocprofv3", "--pmc", ctr, "--output-format", "csv", "-d", tmp, "-o", ctr, "--",
+                   sys.executable, os.path.abspath(__file__), "--traffic-probe", "--layers", str(TRAFFIC_LAYERS), "--ctx", str(args.ctx),
+                   "--target", str(args.target), "--kv-heads", str(args.kv_heads), "--q-heads", str(args.q_heads)]
+            print(f"[traffic] {ctr}: counter run of {TRAFFIC_LAYERS} layers", file=sys.stderr, flush=True)
+            r = subprocess.run(cmd, cwd=tmp, env=env, stdin=subprocess.DEVNULL, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+            if r.returncode != 0:
+                return None, f"counter run for {ctr} ended with status {r.returncode}: {r.stderr[-300:]!r}"
+            probe = [json.loads(ln) for ln in r.stdout.splitlines() if ln.startswith("{") and "traffic_probe" in ln]
+            found = [os.path.join(d, f) for d, _, fs in os.walk(tmp) for f in fs if f == f"{ctr}_counter_collection.csv"]
+            if not probe or not found:
+                return None, f"counter run for {ctr} left no output"
+            main, copy = [], []
+            with open(found[0], newline="") as fh:
+                for row in csv.DictReader(fh):
+                    if row["Counter_Name"] != ctr:
+                        continue
+                    if "decode_main_kernel" in row["Kernel_Name"]:
+                        main.append(float(row["Counter_Value"]))
+                    elif "copyBuffer" in row["Kernel_Name"]:
+                        copy.append(float(row["Counter_Value"]))
+            if len(main) < 3 or not copy or max(copy) <= 0:
+                return None, f"{ctr}: {len(main)} main-kernel dispatches and {len(copy)} copies in the counter file"
+            copy_kib = probe[-1]["copy_bytes"] / 1024.0
+            factor = copy_kib / max(copy)                 # the largest copy is the probe's 256 MiB one
+            res[ctr] = {"kib_per_dispatch_median": round(statistics.median(main), 1), "copy_reads_kib": round(max(copy), 1),
+                        "factor": round(factor, 4), "dispatches": len(main)}
+            res["packed_bytes_per_layer"] = probe[-1]["packed_bytes_per_layer"]
+    except Exception as exc:                                               # noqa: BLE001
+        return None, f"{type(exc).__name__}: {exc}"
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    res["bytes"] = int(1024 * sum(res[c]["kib_per_dispatch_median"] * res[c]["factor"] for c in ("FETCH_SIZE", "WRITE_SIZE")))
+    return res, None
 
 
 def press_e2e(dev, T, target, n_new, n_layers=2, vocab=32000):
@@ -319,6 +370,12 @@ def main() -> int:
                     help="instead of the kernel benchmark: a random-init Llama-3-8B-shaped model (--e2e-layers) under the "
                          "press, prefill of --ctx tokens, then greedy decode with the fused kernel and with the dense "
                          "re-materialised cache (the reference's path); prints per-token times")
+    ap.add_argument("--traffic", choices=["live", "none"], default="live",
+                    help="live: before the benchmark, two short counter runs of --traffic-probe under rocprofv3 --pmc give "
+                         "roofline.traffic (about 25 s each); none: roofline.traffic is null")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="leave out the e2e record (a 2-layer Llama-3-8B-shaped model under the press: ms per decode step "
+                         "with the fused kernel, with the reference's dense path and of the model alone; about 20 s)")
     ap.add_argument("--e2e-tokens", type=int, default=48)
     ap.add_argument("--e2e-layers", type=int, default=2, help="layers of the --press-e2e model (32 = Llama-3-8B)")
     ap.add_argument("--e2e-vocab", type=int, default=32000, help="vocabulary of the --press-e2e model (Llama-3: 128256)")
@@ -327,6 +384,14 @@ def main() -> int:
         print("bench.py measures one GPU's share of the path: every box in this build has one GPU and "
               "nothing here shards across devices; run with --gpus 1", file=sys.stderr)
         return 2
+
+    headline = not (args.press_e2e or args.score_expected or args.score_window or args.read_ceiling or args.decode_shape
+                    or args.traffic_probe)
+    traffic, traffic_note = None, "not measured (--traffic none)"
+    if headline and args.traffic == "live":
+        traffic, traffic_note = measure_traffic(args)       # child processes: before this one touches the GPU
+        if traffic is None:
+            print(f"[traffic] not measured: {traffic_note}", file=sys.stderr, flush=True)
 
     import torch
     from kvquant import _lib
@@ -483,7 +548,7 @@ def main() -> int:
             st.prefill(k, v, bits)
             st._build_items()
             sts.append(st)
-            sqs.append(torch.stack([L.query for L in Ls]).to(dev))
+            sqs.append(torch.stack([L.query for L in Ls]).half().to(dev))        # the model's dtype
             del k, v, sc, bits
         Bs = sqs[0].shape[0]
         ws_bytes = max(blib.odmkv_decode_workspace_bytes(Bs, 32, st._items[2]) for st in sts)
@@ -733,8 +798,13 @@ def main() -> int:
         "parity": {"gate_attn_rel_err": gate_err, "full_size_fused_vs_dense_rel_err": full_err},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": TRAFFIC_FROM_PROFILE_BYTES if (NL, T, args.target) == (32, 32768, 2.0) else None,
-                     "traffic_source": "profiles/decode_main_c2_32k_hbm_traffic.txt (rocprofv3 --pmc runs, not this run)",
+                     "traffic": None if traffic is None else traffic["bytes"],
+                     "traffic_source": (traffic_note if traffic is None else
+                                        {"how": f"this invocation: rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, over bench.py --traffic-probe "
+                                                f"--layers {TRAFFIC_LAYERS} (child runs before the timed part), KiB per dispatch (median) x the "
+                                                "factor the same counter gives for a plain 256 MiB copy",
+                                         "FETCH_SIZE": traffic["FETCH_SIZE"], "WRITE_SIZE": traffic["WRITE_SIZE"],
+                                         "over_algorithmic": round(traffic["bytes"] / traffic["packed_bytes_per_layer"], 4)}),
                      "kernel": "decode_main_kernel", "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
                      "kernel_avg_method": ("the step's main-kernel launches alone (no merge) as one graph, replayed between two "
                                            "HIP events on the launch stream: elapsed / launches, launch gaps included"
@@ -759,6 +829,23 @@ def main() -> int:
             "score_ms": round(cb["t_score"] * 1e3, 1), "alloc_ms": round(cb["t_alloc"] * 1e3, 1),
             "pack_ms": round(cb["t_pack"] * 1e3, 1), "cpu_model": _cpu_model(),
         }
+    if not args.no_e2e and (n_kv, n_q) == (8, 32):
+        # outside every timed region above: what the kernels buy a whole decode step (host side of the press included)
+        torch.cuda.empty_cache()
+        try:
+            e = press_e2e(dev, T, args.target, 24, n_layers=2, vocab=32000)
+            out["e2e"] = {
+                "model": e["model"], "prefill_tokens": T, "decode_tokens": 24, "note": "wall ms per decode step, device-synchronised, median",
+                "fused_ms_per_step": e["fused"]["decode_step_ms_median"],
+                "fused_dense_cache_released_ms_per_step": e["fused_released"]["decode_step_ms_median"],
+                "dense_reference_path_ms_per_step": e["dense"]["decode_step_ms_median"],
+                "model_alone_short_context_ms_per_step": e["decode_step_ms_model_alone_short_context"],
+                "dense_over_fused": e["dense_over_fused"],
+                "cache_bytes_after_prefill": {m: e[m]["cache_bytes_after_prefill"] for m in ("fused", "fused_released", "dense")},
+                "attention_calls": {m: e[m]["attention_calls"] for m in ("fused", "fused_released", "dense")},
+            }
+        except Exception as exc:                                           # noqa: BLE001
+            out["e2e"] = {"error": f"{type(exc).__name__}: {exc}"}
     print(json.dumps(out))
     return 0
 
