@@ -80,7 +80,7 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         # (layer, head) -> ((level, fraction), ...) observed in the prefill allocation
         self._observed_ratios: dict[tuple[int, int], tuple[tuple[int, float], ...]] = {}
 
-    def _prewarm_quantizers(self, model) -> None:
+    def _build_tables(self, model) -> None:
         return          # the state builds its rotations and tables when it is created
 
     def _get_or_create_state(self, layer_idx: int, keys: torch.Tensor) -> TurboQuantAdaptiveKVCacheState:

@@ -14,7 +14,7 @@ from typing import Any, Optional
 import torch
 from torch import nn
 
-from kvquant.press import _backbone
+from kvquant.press import hooked_attention
 from kvquant.tq_backend import TurboQuantMSE, normalize_key_quantizer, normalize_value_quantizer
 
 
@@ -83,19 +83,9 @@ class TurboQuantBackendPress:
 
     @contextlib.contextmanager
     def __call__(self, model):
-        lm = _backbone(model)
         self._done = {}
-        hooks = []
         try:
-            for i, layer in enumerate(lm.layers):
-                attn = getattr(layer, "self_attn", None)
-                if attn is None or getattr(attn, "is_sliding", False):
-                    continue
-                if not hasattr(attn, "layer_idx"):
-                    attn.layer_idx = i
-                hooks.append(attn.register_forward_hook(self.forward_hook, with_kwargs=True))
-            yield
+            with hooked_attention(model, self.forward_hook):
+                yield
         finally:
-            for h in hooks:
-                h.remove()
             self._done = {}

@@ -53,12 +53,68 @@ def _qd_values_group(x: torch.Tensor, b: int, group_size: int = 32) -> torch.Ten
 
 
 def _backbone(model):
-    lm = model
-    if hasattr(lm, "model"):
-        lm = lm.model
-    if hasattr(lm, "language_model"):
-        lm = lm.language_model
-    return lm
+    """The module that owns the decoder layers (a causal LM wraps it once, a multimodal model twice)."""
+    for name in ("model", "language_model"):
+        model = getattr(model, name, model)
+    return model
+
+
+def full_attention_modules(model):
+    """(layer index, attention module) of every decoder layer with full (not sliding-window) attention."""
+    layers = getattr(_backbone(model), "layers", None)
+    if layers is None:
+        raise ValueError(f"Cannot find transformer layers in {type(model)}")
+    found = []
+    for index, layer in enumerate(layers):
+        attn = getattr(layer, "self_attn", None)
+        if attn is not None and not getattr(attn, "is_sliding", False):
+            found.append((index, attn))
+    return found
+
+
+@contextlib.contextmanager
+def hooked_attention(model, hook, adopt=None):
+    """Every full-attention module of `model` calls `hook(module, args, kwargs, output)` after its forward for the
+    duration of the block; yields the hooked layer indices.  A module without a ``layer_idx`` gets its position in
+    the stack; `adopt(module)`, if given, runs once per module before its hook is registered.  Shared by all presses
+    (the reference registers its hooks in each press's ``__call__``: kvquant/press.py:638-692)."""
+    handles, indices = [], []
+    try:
+        for index, attn in full_attention_modules(model):
+            if not hasattr(attn, "layer_idx"):
+                attn.layer_idx = index
+            if adopt is not None:
+                adopt(attn)
+            handles.append(attn.register_forward_hook(hook, with_kwargs=True))
+            indices.append(index)
+        yield indices
+    finally:
+        for handle in handles:
+            handle.remove()
+
+
+class _QuantizerPool:
+    """The press's TurboQuantMSE instances, one per (role, head_dim, width, device, dtype), built on first use.
+    Keys rotate with the press's seed, values with seed + 1000 (kvquant/press.py:202-212)."""
+    _SEED_OFFSET = {"key": 0, "value": 1000}
+
+    def __init__(self, seed: int):
+        self._seed = seed
+        self._made: dict = {}
+
+    def get(self, role: str, head_dim: int, width: int, device, dtype) -> TurboQuantMSE:
+        slot = (role, head_dim, width, device, dtype)
+        q = self._made.get(slot)
+        if q is None:
+            q = self._made[slot] = TurboQuantMSE(head_dim, width, device=device, dtype=dtype,
+                                                 seed=self._seed + self._SEED_OFFSET[role])
+        return q
+
+    def build(self, roles, head_dim: int, widths, devices, dtype) -> None:
+        for role in roles:
+            for width in widths:
+                for device in devices:
+                    self.get(role, head_dim, width, device, dtype)
 
 
 class TurboQuantPerTokenPress:
@@ -92,8 +148,8 @@ class TurboQuantPerTokenPress:
             self._decode_bit_levels = tuple(b for b in bit_levels if b != 0) or (16,)
         self._epsilon: Optional[dict[int, float]] = None
         self._head_dim: Optional[int] = None
-        self._key_qs: dict = {}
-        self._value_qs: dict = {}
+        self._quantizers = _QuantizerPool(seed)
+        self._model = None
         self._prefill_hooks_fired = 0
         self._score_prefill_supports_kwargs = self._supports_kwargs(self.scorer.score_prefill)
         self._score_decode_supports_kwargs = self._supports_kwargs(self.scorer.score_decode)
@@ -101,19 +157,6 @@ class TurboQuantPerTokenPress:
         self._last_hooked_layer_idx: Optional[int] = None
         self._layer_modules: dict[int, nn.Module] = {}
         self._reset_prefill_state()
-
-    # ------------------------------------------------------------------ quantiser cache
-    def _key_q(self, d: int, b: int, device, dtype) -> TurboQuantMSE:
-        k = (d, b, device, dtype)
-        if k not in self._key_qs:
-            self._key_qs[k] = TurboQuantMSE(d, b, device=device, dtype=dtype, seed=self.seed)
-        return self._key_qs[k]
-
-    def _value_q(self, d: int, b: int, device, dtype) -> TurboQuantMSE:
-        k = (d, b, device, dtype)
-        if k not in self._value_qs:
-            self._value_qs[k] = TurboQuantMSE(d, b, device=device, dtype=dtype, seed=self.seed + 1000)
-        return self._value_qs[k]
 
     # ------------------------------------------------------------------ scores -> bits
     def _build_sink_mask(self, H: int, T: int, device) -> Optional[torch.Tensor]:
@@ -268,9 +311,9 @@ class TurboQuantPerTokenPress:
                 keys[h_idx, t_idx] = _qd_scalar(keys[h_idx, t_idx].float(), b).to(dtype)
                 values[h_idx, t_idx] = _qd_scalar(values[h_idx, t_idx].float(), b).to(dtype)
                 continue
-            keys[h_idx, t_idx] = _qd_keys(self._key_q(d, b, device, dtype), keys[h_idx, t_idx]).to(dtype)
+            keys[h_idx, t_idx] = _qd_keys(self._quantizers.get("key", d, b, device, dtype), keys[h_idx, t_idx]).to(dtype)
             if self.value_quantizer == "mse":
-                values[h_idx, t_idx] = _qd_values_mse(self._value_q(d, b, device, dtype), values[h_idx, t_idx]).to(dtype)
+                values[h_idx, t_idx] = _qd_values_mse(self._quantizers.get("value", d, b, device, dtype), values[h_idx, t_idx]).to(dtype)
             else:
                 values[h_idx, t_idx] = _qd_values_group(values[h_idx, t_idx].float(), b, self.value_group_size).to(dtype)
 
@@ -335,65 +378,49 @@ class TurboQuantPerTokenPress:
                 self._apply_bits(k_new, v_new, scores_to_bits(scores, self._decode_bit_levels))
         return output
 
-    def _prewarm_quantizers(self, model) -> None:
-        """Build every codebook / rotation before the first hook fires."""
+    def _build_tables(self, model) -> None:
+        """Rotations and codebooks for every quantised width, on every device that holds an attention module, before
+        the first hook fires (built lazily they would sit in the first prefill's time; kvquant/press.py:594-620)."""
         if self.quantizer == "scalar":
             return
         cfg = model.config
         head_dim = getattr(cfg, "head_dim", None) or cfg.hidden_size // cfg.num_attention_heads
-        dtype = next(model.parameters()).dtype
-        devices = set()
-        for layer in _backbone(model).layers:
-            attn = getattr(layer, "self_attn", None)
-            p = next(attn.parameters(), None) if attn is not None else None
-            if p is not None:
-                devices.add(p.device)
-        if not devices:
-            devices = {next(model.parameters()).device}
-        for b in sorted(set(self.bit_levels)):
-            if b in (0, 16):
-                continue
-            for device in devices:
-                self._key_q(head_dim, b, device, dtype)
-                if self.value_quantizer == "mse":
-                    self._value_q(head_dim, b, device, dtype)
+        first = next(model.parameters())
+        devices = {p.device for _, attn in full_attention_modules(model) for p in list(attn.parameters())[:1]} or {first.device}
+        widths = sorted(set(self.bit_levels) - {0, 16})
+        roles = ("key", "value") if self.value_quantizer == "mse" else ("key",)
+        self._quantizers.build(roles, head_dim, widths, devices, first.dtype)
 
-    @contextlib.contextmanager
-    def __call__(self, model):
-        """Register one forward hook per (non-sliding) attention module for the duration of the block."""
-        lm = _backbone(model)
-        if not hasattr(lm, "layers"):
-            raise ValueError(f"Cannot find transformer layers in {type(model)}")
-        self._prewarm_quantizers(model)
-        patch_attention_functions()
-        self._reset_prefill_state()
+    def _adopt_module(self, attn: nn.Module) -> None:
+        attn.masked_key_indices = None
+        rotary = getattr(_backbone(self._model), "rotary_emb", None)
+        if rotary is not None:
+            try:
+                attn.rotary_emb = rotary               # scorers that rebuild queries read it from the module
+            except Exception:                          # a module that refuses the attribute keeps working without it
+                pass
+
+    def _forget_run(self) -> None:
         self._hooked_layer_indices = []
         self._last_hooked_layer_idx = None
         self._layer_modules = {}
-        hooks = []
+        self._reset_prefill_state()
+
+    @contextlib.contextmanager
+    def __call__(self, model):
+        """For the duration of the block the press sees every full-attention module's forward."""
+        full_attention_modules(model)                      # raises for a model without decoder layers
+        self._build_tables(model)
+        patch_attention_functions()
+        self._forget_run()
+        self._model = model
         try:
-            for i, layer in enumerate(lm.layers):
-                attn = getattr(layer, "self_attn", None)
-                if attn is None or getattr(attn, "is_sliding", False):
-                    continue
-                if not hasattr(attn, "layer_idx"):
-                    attn.layer_idx = i
-                attn.masked_key_indices = None
-                if hasattr(lm, "rotary_emb"):
-                    try:
-                        attn.rotary_emb = lm.rotary_emb
-                    except Exception:
-                        pass
-                self._hooked_layer_indices.append(i)
-                hooks.append(attn.register_forward_hook(self._forward_hook, with_kwargs=True))
-            self._last_hooked_layer_idx = self._hooked_layer_indices[-1] if self._hooked_layer_indices else None
-            yield
+            with hooked_attention(model, self._forward_hook, adopt=self._adopt_module) as indices:
+                self._hooked_layer_indices = indices
+                self._last_hooked_layer_idx = indices[-1] if indices else None
+                yield
         finally:
-            for h in hooks:
-                h.remove()
-            # the eviction masks stay on the modules: decode outside the block must keep honouring them;
-            # the attention patch clears them at the next fresh prefill
-            self._hooked_layer_indices = []
-            self._last_hooked_layer_idx = None
-            self._layer_modules = {}
-            self._reset_prefill_state()
+            # the eviction masks stay on the modules: decode outside the block must keep honouring them; the attention
+            # patch clears them at the next fresh prefill
+            self._model = None
+            self._forget_run()
