@@ -23,6 +23,7 @@ from __future__ import annotations
 
 import argparse
 import ctypes as C
+import gc
 import json
 import os
 import statistics
@@ -613,6 +614,10 @@ def main() -> int:
             ev[3].record()
         return st, bits
 
+    # what a press does when it is attached to a model: the allocator's small-block pool takes the stores' tables now,
+    # not by a device allocation every few layers in the middle of a compression
+    from kvquant.tq_adaptive_backend import reserve_state_memory
+    reserve_state_memory(dev, 2 * NL)
     warm = None
     for li in range(NL):
         k, v, mu, q = make_layer(li, n_kv, n_q, T, dev)        # about a second of CPU work: the GPU idles meanwhile
@@ -622,8 +627,10 @@ def main() -> int:
         compress(*(warm if warm is not None else (k, v, mu)), seed=41)
         ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
         torch.cuda.synchronize()
+        gc.disable()                     # as timeit does: the interpreter's cyclic collector (0.1-0.3 ms a run) stays out
         st, bits = compress(k, v, mu, 42 + 7 * li, ev)
         torch.cuda.synchronize()
+        gc.enable()
         warm = (k, v, mu)
         # device events on the launch stream, no host synchronisation between the stages (the pack
         # stage's own read-back of the level counts is inside its interval)
@@ -637,6 +644,9 @@ def main() -> int:
             dense0 = (k, v, bits)
     packed_bytes = sum(s.packed_bytes() for s in states)
     counts = {b: sum(s.level_counts()[b] for s in states) for b in LEVELS}
+    print("[stages] ms per layer (score, alloc, pack): " + " ".join(
+        f"{a * 1e3:.3f}/{b * 1e3:.3f}/{c * 1e3:.3f}" for a, b, c in zip(t_stage["score"], t_stage["alloc"], t_stage["pack"])),
+        file=sys.stderr, flush=True)
 
     # ---- full-size self-consistency: fused attention == dense attention over the dequantised cache ----
     # (dequantised without rounding to the model dtype and summed in fp64: next to logits of 20 to 100, as the

@@ -28,8 +28,8 @@ from kvquant.allocator import optimal_scores_to_bits, ratio_scores_to_bits, scor
 from kvquant.attention_patch import fused_decode_enabled
 from kvquant.attention_utils import _aligned_rotary_outputs, _apply_rotary_pos_emb_q, _get_query_states
 from kvquant.hf_cache import PackedCacheLayer
-from kvquant.press import TurboQuantPerTokenPress
-from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+from kvquant.press import TurboQuantPerTokenPress, full_attention_modules
+from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState, release_staging, reserve_state_memory
 
 
 def _levels_by_rank(levels, ratios, n: int):
@@ -233,6 +233,8 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
             if self.buffer_size > 0:
                 self._buffer_start_seqs[layer_idx] = int(keys.shape[2])
                 self._buffer_counts[layer_idx] = 0
+            if self._last_hooked_layer_idx is None or layer_idx == self._last_hooked_layer_idx:
+                release_staging(keys.device)             # the prompt is stored: the worst-case staging store can go
         self._reset_prefill_state()
 
     # ------------------------------------------------------------------ hook
@@ -500,6 +502,10 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
         self._states, self._buffer_counts, self._buffer_start_seqs = {}, {}, {}
         try:
             with super().__call__(model):
+                devices = [p.device for _, attn in full_attention_modules(model) for p in list(attn.parameters())[:1]]
+                for device in set(devices):
+                    if device.type == "cuda":
+                        reserve_state_memory(device, devices.count(device))
                 yield
         finally:
             self._states, self._buffer_counts, self._buffer_start_seqs = {}, {}, {}

@@ -129,9 +129,34 @@ class _Buffers:
 
 
 _ARENA_HINT: dict = {}     # (device, segments, tokens) -> bytes of the last store first filled with that shape
-_STAGING_LIMIT = 1 << 30   # bytes a staging store may take (larger first fills wait for the counts instead)
+_STAGING_LIMIT = 4 << 30   # bytes a staging store may take (1.4 % of the device's memory; a 131072-token layer of 8 KV
+#                            heads takes 1.2 GB); larger first fills wait for the counts instead
 _STAGING: dict = {}        # (device, stream) -> _Staging: one per stream, rebuilt when the shape changes
-_MAILBOX: dict = {}        # device -> (page-locked int32 tensor, event): where the level counts arrive
+_MAILBOX: dict = {}        # (device, stream) -> (page-locked int32 tensor, ..., event): where the level counts arrive
+
+
+def _dev_key(dev) -> str:
+    d = torch.device(dev)
+    return f"{d.type}:{torch.cuda.current_device() if d.index is None else d.index}"
+
+
+def reserve_state_memory(device, n_states: int) -> None:
+    """Grow the allocator's small-block pool, in one go, by what `n_states` stores will keep in it (rotations, operand
+    and centroid tables, work lists: about a third of a megabyte each).  Otherwise the pool grows by one 2 MB device
+    allocation every few layers of a first prefill, 0.2 ms of host time each, at whatever small request comes next:
+    between the kernels of a layer's compression.  The blocks go back to the pool at once; a process that has served a
+    prompt before has them anyway."""
+    hold = [torch.empty(384 << 10, dtype=torch.uint8, device=device) for _ in range(int(n_states))]
+    del hold
+
+
+def release_staging(device=None) -> None:
+    """Hand the staging stores (of one device, or of all) back to the allocator: a press does so when the last layer
+    of a prefill is stored, so that the decode steps which follow do not hold a worst-case store they never use.
+    (Work already queued on the staging store's stream keeps its memory until it has run: the allocator returns a
+    block to the stream it was requested on.)"""
+    for key in [k for k in _STAGING if device is None or k[0] == _dev_key(device)]:
+        del _STAGING[key]
 
 
 class _Staging:
@@ -159,22 +184,23 @@ class _Staging:
 
 
 def _staging_for(dev, stream: int, B: int, H: int, T: int, exact_dtype: torch.dtype) -> "_Staging":
-    got = _STAGING.get((str(dev), stream))
+    got = _STAGING.get((_dev_key(dev), stream))
     if got is None or got.key != (B, H, T, exact_dtype):
-        _STAGING.pop((str(dev), stream), None)          # the old one is released before the new one is requested
-        got = _STAGING[(str(dev), stream)] = _Staging(dev, B, H, T, exact_dtype)
+        _STAGING.pop((_dev_key(dev), stream), None)          # the old one is released before the new one is requested
+        got = _STAGING[(_dev_key(dev), stream)] = _Staging(dev, B, H, T, exact_dtype)
     return got
 
 
-def _mailbox(dev, numel: int):
-    """(page-locked int32 tensor, device int32 tensor, event, the event's handle): where the level counts arrive."""
-    got = _MAILBOX.get(str(dev))
+def _mailbox(dev, stream: int, numel: int):
+    """(page-locked int32 tensor, device int32 tensor, event, the event's handle): where the level counts of the fills
+    queued on `stream` arrive (one box per stream: fills on two streams of a device do not share it)."""
+    got = _MAILBOX.get((_dev_key(dev), stream))
     if got is None or got[0].numel() < numel:
         ev = torch.cuda.Event()
         ev.record(torch.cuda.current_stream(dev))          # (the handle exists once the event has been recorded)
         ev.synchronize()
         n = max(numel, 4096)
-        got = _MAILBOX[str(dev)] = (torch.zeros(n, dtype=torch.int32, pin_memory=True),
+        got = _MAILBOX[(_dev_key(dev), stream)] = (torch.zeros(n, dtype=torch.int32, pin_memory=True),
                                     torch.empty(n, dtype=torch.int32, device=dev), ev, int(ev.cuda_event))
     return got
 
@@ -299,6 +325,9 @@ class TurboQuantAdaptiveKVCacheState:
         layout = _Layout(seg_tile, self._nseg)
         off = layout.total
         arena = getattr(self, "_arena", None)
+        if arena is not None and self._level_store is not None and (self._level_store.untyped_storage().data_ptr()
+                                                                    == arena.untyped_storage().data_ptr()):
+            self._level_store = self._level_store.clone()    # the level map of a staged first fill lies behind the old store
         if arena is None or arena.numel() < off or arena.device != dev:
             arena = torch.empty(off + off // 8, dtype=torch.uint8, device=dev)
             self._arena_spare = None
@@ -417,12 +446,16 @@ class TurboQuantAdaptiveKVCacheState:
         # laid out for the worst case while the counts travel and the host lays the store out; the tiles are moved after.
         staged = (self._bufs is None and _known_counts is None and _pos_offset is None and T >= 4 * TILE
                   and _Staging.bytes_needed(self._nseg, T) <= _STAGING_LIMIT)
+        # A staged first fill keeps its level map (one byte per token) behind the store, in the same allocation: a tensor
+        # of its own would now and then make the allocator open a new segment (a device allocation, 0.2 ms of host time)
+        # between this call's kernels.
+        lm_bytes = (B * H * T + 255) & ~255 if staged else 0
         stg = None
         if _known_counts is not None:
             counts = np.asarray(_known_counts, np.int64).reshape(self._nseg, 6)
         elif staged:
             n_chunks = lib.odmkv_pack_count_chunks(T)                 # the counts arrive chunk by chunk
-            box, box_dev, arrived, arrived_handle = _mailbox(dev, self._nseg * n_chunks * 6)
+            box, box_dev, arrived, arrived_handle = _mailbox(dev, st, self._nseg * n_chunks * 6)
             arrived.synchronize()                                     # (the last reader of the box is long done)
             stg = _staging_for(dev, st, B, H, T, self._exact_torch_dtype)
             ws = _lib.workspace(dev, ws_bytes, "pack")
@@ -445,12 +478,12 @@ class TurboQuantAdaptiveKVCacheState:
                 rc = lib.odmkv_store_finish_staged(
                     box.data_ptr(), n_chunks, B, H, T, int(self.exact_slack),
                     _lib.BF16 if self._exact_torch_dtype == torch.bfloat16 else _lib.F16,
-                    None if arena is None else arena.data_ptr(), 0 if arena is None else arena.numel(),
+                    None if arena is None else arena.data_ptr(), 0 if arena is None else max(arena.numel() - lm_bytes, 0),
                     C.byref(stg.packed), counts32.ctypes.data, new_lay.tables_ptr, new_lay.offsets, new_lay.sizes,
                     new_lay.marks, C.byref(new_packed), C.byref(need), st)
                 if rc != -2 or attempt == 1:
                     break
-                self._arena = torch.empty(int(need.value) + int(need.value) // 8, dtype=torch.uint8, device=dev)
+                self._arena = torch.empty(int(need.value) + int(need.value) // 8 + lm_bytes, dtype=torch.uint8, device=dev)
                 self._arena_spare = None
             _lib.check(rc)
             counts = counts32.astype(np.int64)
@@ -488,9 +521,13 @@ class TurboQuantAdaptiveKVCacheState:
                 C.byref(self._packed), ws.data_ptr(), ws_bytes, st))
         self._counts = new_counts
         self._exact_room = None
-        lm = bits.to(torch.uint8)
+        if stg is not None:
+            lm = self._arena[self._arena.numel() - lm_bytes:][:B * H * T].view(B, H, T)
+            lm.copy_(bits)
+        else:
+            lm = bits.to(torch.uint8)
         if _pos_offset is None:
-            self._extend_levels(lm, owned=lm is not bits)
+            self._extend_levels(lm, owned=True)
             self.seq_len += T
         else:
             self._level_store[:, :, pos_offset:pos_offset + T] = lm

@@ -121,8 +121,16 @@ def test_c3_sixteen_sequences_with_cycling_budgets():
 
 
 def test_c4_long_context_heavy_eviction():
+    from kvquant import tq_adaptive_backend as tqa
     L = synthetic.config("c4")
+    tqa.release_staging()
     st, bits, stored, scores = _compress([L], [2.0])
+    # the first fill of this store went through the staging store (1.2 GB for 8 x 131072 tokens), which a caller can
+    # hand back once the prompt is stored
+    assert [s.key[:3] for s in tqa._STAGING.values()] == [(1, 8, 131072)]
+    held = torch.cuda.memory_allocated()
+    tqa.release_staging(DEV)
+    assert not tqa._STAGING and held - torch.cuda.memory_allocated() > 1.1e9
     evicted = (bits == 0).float().mean().item()
     assert 0.30 <= evicted <= 0.50, evicted              # the configuration is built to evict about 40 %
     n_active = 8 * (131072 - 4)

@@ -459,6 +459,9 @@ def test_second_prompt_through_one_press_flushes_with_its_own_shares():
         cache = DynamicCache()
         with press(model):
             model.model(input_ids=_ids(T, 70 + prompt), past_key_values=cache)
+            # the prompt is stored: the press has handed the worst-case staging store of the first fills back
+            from kvquant import tq_adaptive_backend as tqa
+            assert not tqa._STAGING
             for step in range(forced.shape[0]):
                 model(input_ids=forced[step].view(1, 1), past_key_values=cache, position_ids=torch.tensor([[T + step]], device=DEV))
     assert [s[0] for s in seen] == [0, 1, 0, 1]

@@ -79,3 +79,56 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     assert rc == -2 and b"fixed array" in lib.odmkv_last_error()
     torch.cuda.synchronize()
     assert (out == 0).all()
+
+
+def test_static_call_leaves_device_memory_as_it_is_and_replays_from_a_graph():
+    """No allocation: the device's free memory and torch's allocated bytes are the same before and after a
+    run of calls (outputs are allocated beforehand); and the call can be captured into a HIP graph, whose
+    replays (with eager work and synchronisations between them) give the eager call's bits."""
+    from kvquant import _lib
+    lib = _lib.lib
+    st = _store(81, 1, 4, 2500, (0.15, 0.45, 0.15, 0.1, 0.05, 0.1))
+    g = torch.Generator().manual_seed(82)
+    qs = [torch.randn(1, 16, 128, generator=g).half().to(DEV) for _ in range(4)]
+    q = qs[0].clone()
+    out = torch.zeros(1, 16, 128, dtype=torch.float32, device=DEV)
+    lse = torch.zeros(1, 16, dtype=torch.float32, device=DEV)
+
+    def call(stream):
+        _lib.check(lib.odmkv_decode_attn_static(
+            q.data_ptr(), _lib.F16, 1, 16, 128 ** -0.5, C.byref(st._packed), C.byref(st._worklist), st._pi_k_ops.data_ptr(),
+            st.pi_v.data_ptr(), st._decode_cb.data_ptr(), st._decode_cb_host, st._decode_inv, out.data_ptr(), _lib.F32,
+            lse.data_ptr(), stream))
+
+    dev = torch.device(DEV, torch.cuda.current_device())
+    call(_lib.stream_ptr(dev))                                  # the first call on a device looks the array up
+    torch.cuda.synchronize()
+    free0, allocated0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(20):
+        call(_lib.stream_ptr(dev))
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.cuda.memory_allocated() == allocated0 and torch.cuda.memory_reserved() == reserved0
+
+    want = []
+    for x in qs:                                                # eager results for four queries
+        q.copy_(x)
+        call(_lib.stream_ptr(dev))
+        torch.cuda.synchronize()
+        want.append((out.clone(), lse.clone()))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(_lib.stream_ptr(dev))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(_lib.stream_ptr(dev))
+    for x, (w_out, w_lse) in zip(qs, want):
+        q.copy_(x)
+        out.zero_(); lse.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, w_out) and torch.equal(lse, w_lse)
+        (out * 2).sum().item()                                  # the program's own eager work between replays
