@@ -359,7 +359,8 @@ int odmkv_flush_rank(const float* scores, const float* minmax, int B, int H, int
  * query and the softmax weights split into two bf16 pieces each): nothing is narrowed.
  *
  * Work list.  items: device int32 [n_items, 8], sorted by bh: (bh, level index 0..4, first tile,
- * tile count, tokens held by those tiles, first tile of the segment, 0, 0); for the exact level
+ * tile count, tokens held by those tiles, first tile of the segment, items that follow in the same workgroup,
+ * 1 if the item belongs to an earlier item's workgroup: 0 and 0 without n_workgroups); for the exact level
  * (index 4) the token count is read from seg_count instead, so that tokens appended since the list
  * was built are seen.  item_range: device int32 [B*Hkv + 1] first item of each bh (any number of
  * items per bh; one item per compute unit is what performs best; a bh without items gets zeros and
@@ -379,6 +380,10 @@ typedef struct odmkv_worklist {
     const int32_t* dispatch_order;   /* device [n_items] or NULL */
     int32_t n_items;
     int32_t wavefronts;              /* 0, 8, 12 or 16 */
+    int32_t n_workgroups;            /* 0 or n_items: a workgroup per item.  Fewer: workgroup k starts at item
+                                      * dispatch_order[k] and also takes the items[.][6] items behind it (further quantised
+                                      * levels of the same (sequence, kv-head): one query rotation, one result); those
+                                      * items carry items[.][7] = 1 */
 } odmkv_worklist_t;
 
 size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);

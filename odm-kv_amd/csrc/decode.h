@@ -13,6 +13,7 @@ struct DecodeArgs {
     int Hq, G, B;
     float scaling;
     const int32_t* items;
+    int n_items;
     const int32_t* item_range;
     const int32_t* order;      // order[k] = item that workgroup k takes (long items first), or null: item k
     const uint16_t* pi_k_ops;   // Pi_k as the A operands of the query rotation (odmkv_rotation_operands)

@@ -672,9 +672,11 @@ __device__ static inline void rotate_queries(const DecodeArgs& a, uint8_t* smem,
 }
 
 // One work item of a quantised level: the workgroup's wavefronts walk the item's units.
+// first: the workgroup's first item (the queries are rotated now); a further item of a chain (another level of the same
+// (sequence, kv-head), same queries, same accumulators) only waits until every wavefront has left the previous table.
 template <int W, int GP, int NW>
 __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int bq_first, int tile0, int ntiles, int ntok,
-                                              int tid, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
+                                              int tid, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st, bool first) {
     uint8_t* lut = smem;
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
@@ -686,7 +688,8 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     // requests wait until the memory pipeline has accepted them: with both units requested first the table was ready a
     // microsecond later).  Loads return in issue order: the (small) query goes first.
     RotQuery rq;
-    request_rot_query(rq, a, bq_first, tid);
+    if (first) request_rot_query(rq, a, bq_first, tid);
+    else __syncthreads();
     // DEPTH units of this wavefront are under way at any time: two (one for the widest rows: registers); twelve
     // wavefronts have the registers for a third 2-bit unit.  (Six units in flight with eight wavefronts were measured:
     // no gain, the eight are bound by their arithmetic.)
@@ -698,7 +701,7 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
         int nvalid = tokens_of(u);
         if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
         build_lut<W, NW>(lut, a, tid);
-        rotate_queries<GP>(a, smem, tid, bq_first, rq);
+        if (first) rotate_queries<GP>(a, smem, tid, bq_first, rq);
         lds_barrier();
         // second buffer (not for the widest rows), requested before the first unit is used (requested before the
         // rotation instead, it delays the table's LDS stores behind its queue of requests: 0.9 us per item slower)
@@ -738,7 +741,7 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
         nv[0] = tokens_of(wave);
         if (nv[0] > 0) load_unit<W>(buf[0], a, li, unit0 + wave, lane);
         build_lut<W, NW>(lut, a, tid);
-        rotate_queries<GP>(a, smem, tid, bq_first, rq);
+        if (first) rotate_queries<GP>(a, smem, tid, bq_first, rq);
         lds_barrier();
         // the rest of the ring, requested before the first unit is used
     #pragma unroll
@@ -767,7 +770,7 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
 // eight-wavefront ring of five buffers, every unit of a short item requested at once, measured no faster).
 template <int W, int NW>
 __device__ static inline void run_quant_level_g4(const DecodeArgs& a, int li, int bq_first, int tile0, int ntiles, int ntok,
-                                              int tid, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
+                                              int tid, uint8_t* smem, uint8_t* pbuf, float* alpha_sh, WaveState& st, bool first) {
     uint8_t* lut = smem;
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t slot4 = (lane & 31) * 4;
@@ -776,13 +779,14 @@ __device__ static inline void run_quant_level_g4(const DecodeArgs& a, int li, in
     const auto tokens_of = [&](int u) { return min(ntok - u * UNIT, UNIT); };    // <= 0 behind the item's last token
     // (the order of the requests, the table and the rotation is run_quant_level's)
     RotQuery rq;
-    request_rot_query(rq, a, bq_first, tid);
+    if (first) request_rot_query(rq, a, bq_first, tid);
+    else __syncthreads();
     Unit4<W> cur;
     int u = wave;
     int nvalid = tokens_of(u);
     if (nvalid > 0) load_unit4<W>(cur, a, li, unit0 + u, lane);
     build_lut<W, NW>(lut, a, tid);
-    rotate_queries<4>(a, smem, tid, bq_first, rq);
+    if (first) rotate_queries<4>(a, smem, tid, bq_first, rq);
     lds_barrier();
     // second buffer (not for the widest rows)
     Unit4<W> nxt;
@@ -791,7 +795,7 @@ __device__ static inline void run_quant_level_g4(const DecodeArgs& a, int li, in
         nv1 = tokens_of(u + NW);
         if (nv1 > 0) load_unit4<W>(nxt, a, li, unit0 + u + NW, lane);
     }
-    if (nvalid <= 0) return;                               // (the untouched state needs no g4_finish)
+    if (nvalid <= 0) return;
     h8 qa[4];
     load_queries_g4(smem + LDS_QROWS, lane, qa);
     if constexpr (W == 8) {
@@ -815,7 +819,6 @@ __device__ static inline void run_quant_level_g4(const DecodeArgs& a, int li, in
             if (nv1 > 0) load_unit4<W>(nxt, a, li, unit0 + u + NW, lane);
         }
     }
-    g4_finish(st);
 }
 
 // ---- exact (fp16 / bf16) units ---------------------------------------------------------------------
@@ -915,9 +918,13 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
 // main kernel
 // ------------------------------------------------------------------------------------------------
 // G4: the quantised levels run compute_unit_g4 (GP = 4 and sixteen wavefronts only)
-template <int GP, bool ORDERED, int NW, bool G4 = false>
+// CHAIN: a workgroup may take several consecutive items, the quantised levels of one (sequence, kv-head) one after the
+// other (item word 6 = how many follow): the queries are rotated once, the accumulators run through, the table is rebuilt
+// between the levels, one result is written at the first item's place and empty results at the others'.
+template <int GP, bool ORDERED, int NW, bool G4 = false, bool CHAIN = false>
 __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
     static_assert(!G4 || (GP == 4 && NW == 16), "the shared-lane form is built for four heads and sixteen wavefronts");
+    static_assert(!CHAIN || ORDERED, "chains come with a dispatch order (fewer workgroups than items)");
     // one static LDS block: the table sits at LDS address 0 and that is known when the kernel is compiled, so a
     // lookup address needs no base added
     __shared__ __align__(16) uint8_t smem[Lds<NW>::TOTAL];
@@ -934,7 +941,8 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
     const int4 d1 = reinterpret_cast<const int4*>(a.items)[2 * item + 1];   // tokens, first tile of the segment
     // the rotation's operand table on its way into LDS right behind the request for the work item (loads return in the
     // order of their requests: asked for first, the table would hold the item back; it does not depend on the item)
-    const int bh = d0.x, li = d0.y, tile0 = d0.z, ntiles = d0.w;
+    const int bh = d0.x;
+    int li = d0.y, tile0 = d0.z, ntiles = d0.w, ntok = d1.x;
     const int bq_first = (bh / a.s.Hkv) * a.Hq + (bh % a.s.Hkv) * a.G;      // first query head of the group
 
     float* dst = a.partial + (size_t)item * GP * PSTRIDE;      // where this item's result goes
@@ -945,27 +953,60 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
     for (int nb = 0; nb < 8; ++nb) st.acc[nb] = (f4){0.f, 0.f, 0.f, 0.f};
     uint8_t* pbuf = smem + LDS_PBUFS + wave * 2 * PBUF;
     float* alpha_sh = alphas + wave * 8;
-    switch (li) {
-        case 0:
-            if constexpr (G4) run_quant_level_g4<2, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
-            else run_quant_level<2, GP, NW>(a, 0, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
-            break;
-        case 1:
-            if constexpr (G4) run_quant_level_g4<3, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
-            else run_quant_level<3, GP, NW>(a, 1, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
-            break;
-        case 2:
-            if constexpr (G4) run_quant_level_g4<4, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
-            else run_quant_level<4, GP, NW>(a, 2, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
-            break;
-        case 3:
-            if constexpr (G4) run_quant_level_g4<8, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
-            else run_quant_level<8, GP, NW>(a, 3, bq_first, tile0, ntiles, d1.x, tid, smem, pbuf, alpha_sh, st);
-            break;
-        default:
-            if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
-            else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
-            break;
+#define ODMKV_RUN_LEVEL(W, L, FIRST) \
+    do { if constexpr (G4) run_quant_level_g4<W, NW>(a, L, bq_first, tile0, ntiles, ntok, tid, smem, pbuf, alpha_sh, st, FIRST); \
+         else run_quant_level<W, GP, NW>(a, L, bq_first, tile0, ntiles, ntok, tid, smem, pbuf, alpha_sh, st, FIRST); } while (0)
+    if constexpr (!CHAIN) {
+        switch (li) {
+            case 0: ODMKV_RUN_LEVEL(2, 0, true); break;
+            case 1: ODMKV_RUN_LEVEL(3, 1, true); break;
+            case 2: ODMKV_RUN_LEVEL(4, 2, true); break;
+            case 3: ODMKV_RUN_LEVEL(8, 3, true); break;
+            default:
+                if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
+                else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
+                break;
+        }
+    } else if (li == 4) {
+        if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
+        else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
+    } else {
+        // The levels of a chain ascend: the four walkers stand one behind the other, each taken if the current item is of
+        // its level.  The queries are rotated before the first of them (its barrier is the walker's own).
+        {
+            RotQuery rq;
+            request_rot_query(rq, a, bq_first, tid);
+            rotate_queries<GP>(a, smem, tid, bq_first, rq);
+        }
+        // the (up to three) items behind the first one, asked for together (the list is padded: reading past a chain's
+        // end reads other items, which are then not used)
+        const int follow = d1.z;
+        int4 r0[3], r1[3];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const int idx = min(item + 1 + k, a.n_items - 1);
+            r0[k] = reinterpret_cast<const int4*>(a.items)[2 * idx];
+            r1[k] = reinterpret_cast<const int4*>(a.items)[2 * idx + 1];
+        }
+        // the places of the items this workgroup takes along get an empty result (no visible token), now, while the first
+        // bytes are on their way: the merge reads them like any other item's
+        for (int e = tid; e < follow * GP * PSTRIDE; e += NW * 64) dst[GP * PSTRIDE + e] = (e % PSTRIDE) == HD ? -INFINITY : 0.0f;
+        const int first_li = li, first_tile0 = tile0, first_ntiles = ntiles, first_ntok = ntok;
+#define ODMKV_PICK_LEVEL(L) \
+        bool has = first_li == L; \
+        tile0 = first_tile0; ntiles = first_ntiles; ntok = first_ntok; \
+        _Pragma("unroll") for (int k = 0; k < 3; ++k) \
+            if (k < follow && r0[k].y == L) { has = true; tile0 = r0[k].z; ntiles = r0[k].w; ntok = r1[k].x; }
+        { ODMKV_PICK_LEVEL(0) if (has) ODMKV_RUN_LEVEL(2, 0, false); }
+        { ODMKV_PICK_LEVEL(1) if (has) ODMKV_RUN_LEVEL(3, 1, false); }
+        { ODMKV_PICK_LEVEL(2) if (has) ODMKV_RUN_LEVEL(4, 2, false); }
+        { ODMKV_PICK_LEVEL(3) if (has) ODMKV_RUN_LEVEL(8, 3, false); }
+#undef ODMKV_PICK_LEVEL
+        li = 0;                                                // (a quantised item: the shared-lane state is finished below)
+    }
+#undef ODMKV_RUN_LEVEL
+    if constexpr (G4) {
+        if (li < 4) g4_finish(st);                             // (wave-uniform; exact items keep the general form)
     }
 
     // ---- combine the wavefronts (the table is no longer needed) ----
@@ -1150,9 +1191,9 @@ extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     return align_up((size_t)(n_items > 0 ? n_items : 1) * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
 }
 
-template <int GP, bool ORDERED, int NW, bool G4 = false>
+template <int GP, bool ORDERED, int NW, bool G4 = false, bool CHAIN = false>
 static int launch_main(const DecodeArgs& a, int grid, hipEvent_t e0, hipEvent_t e1, hipStream_t st) {
-    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED, NW, G4>), dim3(grid), dim3(NW * 64), 0, st, e0, e1, 0, a);
+    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED, NW, G4, CHAIN>), dim3(grid), dim3(NW * 64), 0, st, e0, e1, 0, a);
     ODMKV_CHECK_LAUNCH("decode_main_kernel");
     return 0;
 }
@@ -1176,6 +1217,9 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
                     "decode_attn: %d wavefronts per work item (0, 8, 12 or 16)", work->wavefronts);
     ODMKV_CHECK_ARG(work->item_range, "decode_attn: null item ranges");
     ODMKV_CHECK_ARG(n_items == 0 || work->items, "decode_attn: null work list");
+    ODMKV_CHECK_ARG(work->n_workgroups >= 0 && work->n_workgroups <= n_items, "decode_attn: %d workgroups for %d items", work->n_workgroups, n_items);
+    ODMKV_CHECK_ARG(work->n_workgroups == 0 || work->n_workgroups == n_items || work->dispatch_order,
+                    "decode_attn: workgroups that take several items need the dispatch order (their first items)");
     ODMKV_CHECK_ARG(B > 0 && Hq > 0 && store->B == B && store->Hkv > 0 && Hq % store->Hkv == 0,
                     "decode_attn: bad head counts B=%d Hq=%d store(B=%d,Hkv=%d)", B, Hq, store->B, store->Hkv);
     ODMKV_CHECK_ARG(store->exact_dtype == ODMKV_F16 || store->exact_dtype == ODMKV_BF16, "decode_attn: exact dtype must be fp16 or bf16");
@@ -1189,6 +1233,7 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     DecodeArgs a;
     a.s = *store; a.q = q; a.q_dt = q_dtype; a.out_dt = out_dtype; a.Hq = Hq; a.G = G; a.B = B; a.scaling = scaling;
     a.items = work->items; a.item_range = work->item_range; a.order = work->dispatch_order;
+    a.n_items = n_items;
     a.pi_k_ops = pi_k_ops; a.pi_v = pi_v; a.cb = codebooks;
     for (int w = 0; w < 4; ++w) a.inv_s[w] = inv_scales[w];
     for (int k = 0; k < 28; ++k) a.cbs[k] = codebooks_host[k];
@@ -1202,19 +1247,24 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
         hipEvent_t e0 = (hipEvent_t)ev_start, e1 = (hipEvent_t)ev_stop;
         const int nw = work->wavefronts == 0 ? 8 : work->wavefronts;
         int rc;
-#define ODMKV_LAUNCH_MAIN(GPV, ORD) \
-        (nw == 16 ? launch_main<GPV, ORD, 16>(a, n_items, e0, e1, st) : nw == 12 ? launch_main<GPV, ORD, 12>(a, n_items, e0, e1, st) \
-                                                                     : launch_main<GPV, ORD, 8>(a, n_items, e0, e1, st))
+#define ODMKV_LAUNCH_MAIN(GPV, ORD, CH) \
+        (nw == 16 ? launch_main<GPV, ORD, 16, false, CH>(a, grid, e0, e1, st) : nw == 12 ? launch_main<GPV, ORD, 12, false, CH>(a, grid, e0, e1, st) \
+                                                                               : launch_main<GPV, ORD, 8, false, CH>(a, grid, e0, e1, st))
         // groups of up to four heads on sixteen wavefronts: the form that shares the lanes out between a unit's two token
         // blocks (its softmax step costs half the instructions); ODMKV_DECODE_G4=0 selects the general form, for measurements
         static const int g4_forced = [] { const char* e = getenv("ODMKV_DECODE_G4"); return e ? atoi(e) : -1; }();
         const bool g4 = GP == 4 && nw == 16 && g4_forced != 0;
-        if (g4 && !a.order) rc = launch_main<4, false, 16, true>(a, n_items, e0, e1, st);
-        else if (g4) rc = launch_main<4, true, 16, true>(a, n_items, e0, e1, st);
-        else if (GP == 4 && !a.order) rc = ODMKV_LAUNCH_MAIN(4, false);
-        else if (GP == 4) rc = ODMKV_LAUNCH_MAIN(4, true);
-        else if (!a.order) rc = ODMKV_LAUNCH_MAIN(8, false);
-        else rc = ODMKV_LAUNCH_MAIN(8, true);
+        const bool chain = work->n_workgroups > 0 && work->n_workgroups != n_items;      // workgroups that take several items
+        const int grid = chain ? work->n_workgroups : n_items;
+        if (chain && g4) rc = launch_main<4, true, 16, true, true>(a, grid, e0, e1, st);
+        else if (chain && GP == 4) rc = ODMKV_LAUNCH_MAIN(4, true, true);
+        else if (chain) rc = ODMKV_LAUNCH_MAIN(8, true, true);
+        else if (g4 && !a.order) rc = launch_main<4, false, 16, true>(a, grid, e0, e1, st);
+        else if (g4) rc = launch_main<4, true, 16, true>(a, grid, e0, e1, st);
+        else if (GP == 4 && !a.order) rc = ODMKV_LAUNCH_MAIN(4, false, false);
+        else if (GP == 4) rc = ODMKV_LAUNCH_MAIN(4, true, false);
+        else if (!a.order) rc = ODMKV_LAUNCH_MAIN(8, false, false);
+        else rc = ODMKV_LAUNCH_MAIN(8, true, false);
 #undef ODMKV_LAUNCH_MAIN
         if (rc) return rc;
     }

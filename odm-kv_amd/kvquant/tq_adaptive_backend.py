@@ -55,7 +55,17 @@ _TILE_BYTES = [TILE * 16 * w + 2 * TILE * 4 for w in WIDTHS] + [2 * TILE * HEAD_
 # what one compute unit was measured to need per 64-token tile of each level (nanoseconds; 2, 3, 4, 8 bits, exact rows)
 # and per work item (microseconds: start, table, query rotation, combining the wavefronts)
 _TILE_COST = [300, 420, 450, 890, 1310]
-_ITEM_FIXED_US = 4.0
+_ITEM_FIXED_US = 4.0           # what the cuts without chains are compared with (its choices were measured shape by shape)
+# Chains (a workgroup that walks several levels of a pair) are weighed against the best cut without them with constants
+# fitted to whole-call times of lists of 256 to 3000 items (64 sequences of 2048 tokens, mixed levels: 90 us without
+# chains, 69 us with, both reproduced to a microsecond): a workgroup 6 us beside its tiles, a further level 2.1 us (a
+# barrier, the new table, its first bytes from memory), 1 us because a chained workgroup rotates its queries before it asks
+# for the first unit.  They are taken when the model promises 15 % (16 sequences of 8192 tokens: 4 %, measured the same
+# or slower: not taken).
+_CHAIN_ITEM_FIXED_US = 6.0
+_CHAIN_LINK_US = 2.1
+_CHAIN_ROTATE_US = 1.0
+_CHAIN_MIN_GAIN = 0.15
 
 
 _U64x33 = C.c_uint64 * 33
@@ -776,40 +786,132 @@ class TurboQuantAdaptiveKVCacheState:
             out[:, 4], out[:, 5] = np.minimum(run_cnt[run] - a0 * TILE, n * TILE), run_t0[run]
             return out
 
-        def cost(items: np.ndarray) -> np.ndarray:                       # microseconds of one workgroup, roughly
-            return _ITEM_FIXED_US + items[:, 3] * tile_cost[items[:, 1]] * 1e-3
+        # -- chains: the quantised levels of a segment as ONE run of work, cut into pieces of equal cost; a piece that
+        # crosses a level boundary becomes consecutive items of one workgroup (one query rotation, one result)
+        qr = run_li < 4
+        q_s, q_li, q_nt, q_t0, q_cnt = run_s[qr], run_li[qr], run_nt[qr], run_t0[qr], run_cnt[qr]
+        q_cost = q_nt * tile_cost[q_li]
+        q_end = np.cumsum(q_cost)
+        q_start = q_end - q_cost
+        seg_cost = np.bincount(q_s, q_cost, minlength=self._nseg) if q_s.size else np.zeros(self._nseg)
+        seg_start = np.cumsum(seg_cost) - seg_cost
+        q_first = np.ones(q_s.size, bool)
+        q_first[1:] = q_s[1:] != q_s[:-1]                               # a segment's first quantised run
 
-        def makespan(items: np.ndarray) -> float:
+        def chain_pieces(per_item: int) -> np.ndarray:                  # workgroups per segment
+            return np.ceil(seg_cost / max(per_item, 1)).astype(np.int64)
+
+        def cut_exact(per_item: int) -> np.ndarray:
+            keep = run_li == 4
+            step = steps_of(per_item)[4]
+            nt, t0 = run_nt[keep], run_t0[keep]
+            pieces = -(-nt // step)
+            run = np.repeat(np.arange(nt.size), pieces)
+            a0 = (np.arange(run.size) - np.repeat(np.cumsum(pieces) - pieces, pieces)) * step
+            n = np.minimum(step, nt[run] - a0)
+            out = np.zeros((run.size, 8), np.int64)
+            out[:, 0], out[:, 1], out[:, 2], out[:, 3] = run_s[keep][run], 4, t0[run] + a0, n
+            out[:, 4], out[:, 5] = np.minimum(run_cnt[keep][run] - a0 * TILE, n * TILE), t0[run]
+            return out
+
+        def cut_chained(per_item: int) -> np.ndarray:
+            # rows as in cut(), word 6 = items that follow in the same workgroup, word 7 = 1 for those items
+            k = chain_pieces(per_item)
+            nb = np.maximum(k - 1, 0)
+            b_s = np.repeat(np.arange(self._nseg), nb)                  # one row per inner piece boundary
+            b_j = np.arange(b_s.size) - np.repeat(np.cumsum(nb) - nb, nb) + 1
+            x = seg_start[b_s] + b_j * seg_cost[b_s] / k[b_s]           # where the boundary lies on the line of all runs' cost
+            run = np.minimum(np.searchsorted(q_end, x, side="right"), q_s.size - 1)
+            off = np.clip(np.rint((x - q_start[run]) / tile_cost[q_li[run]]).astype(np.int64), 0, q_nt[run])
+            at_end = off == q_nt[run]                                   # a boundary on a run's end belongs to the next run's start
+            run, off = np.where(at_end, np.minimum(run + 1, q_s.size - 1), run), np.where(at_end, 0, off)
+            # the items' starts: every run's first tile, and the boundaries inside runs
+            st_run = np.concatenate([np.arange(q_s.size), run])
+            st_off = np.concatenate([np.zeros(q_s.size, np.int64), off])
+            st_head = np.concatenate([q_first, np.ones(run.size, bool)])  # starts a workgroup's chain
+            order_ = np.lexsort((~st_head, st_off, st_run))             # duplicates: the one that starts a chain first
+            st_run, st_off, st_head = st_run[order_], st_off[order_], st_head[order_]
+            uniq = np.ones(st_run.size, bool)
+            uniq[1:] = (st_run[1:] != st_run[:-1]) | (st_off[1:] != st_off[:-1])
+            st_run, st_off, st_head = st_run[uniq], st_off[uniq], st_head[uniq]
+            nxt = np.append(st_off[1:], 0)
+            last_of_run = np.append(st_run[1:] != st_run[:-1], True)
+            n = np.where(last_of_run, q_nt[st_run], nxt) - st_off
+            out = np.zeros((st_run.size, 8), np.int64)
+            out[:, 0], out[:, 1], out[:, 2], out[:, 3] = q_s[st_run], q_li[st_run], q_t0[st_run] + st_off, n
+            out[:, 4], out[:, 5] = np.minimum(q_cnt[st_run] - st_off * TILE, n * TILE), q_t0[st_run]
+            head_idx = np.flatnonzero(st_head)
+            follow = np.diff(np.append(head_idx, st_run.size)) - 1
+            out[head_idx, 6] = follow
+            out[:, 7] = ~st_head
+            both = np.concatenate([out, cut_exact(per_item)])
+            return both[np.lexsort((both[:, 2], both[:, 1] & 7, both[:, 0]))]
+
+        def fit_chained(target: int) -> int:
+            per_item = max(total // max(target, 1), min_item_bytes)
+            n_exact = lambda p: int((-(-run_nt[run_li == 4] // steps_of(p)[4])).sum())
+            while int(chain_pieces(per_item).sum()) + n_exact(per_item) > target and per_item < total:
+                per_item += max(per_item // 64, 1)
+            return per_item
+
+        def cost(items: np.ndarray, fixed: float = _ITEM_FIXED_US) -> np.ndarray:
+            # microseconds of one workgroup, roughly: per workgroup (an item with word 7 set adds to the one before it)
+            own = items[:, 3] * tile_cost[items[:, 1] & 7] * 1e-3
+            head = items[:, 7] == 0
+            group = np.cumsum(head) - 1
+            return (fixed + np.bincount(group, own, minlength=int(head.sum()))
+                    + _CHAIN_LINK_US * items[head, 6] + np.where(items[head, 6] > 0, _CHAIN_ROTATE_US, 0.0))
+
+        def makespan(items: np.ndarray, fixed: float = _ITEM_FIXED_US) -> float:
             import heapq
             free = [0.0] * n_cu
-            for c in sorted(cost(items).tolist(), reverse=True):
+            for c in sorted(cost(items, fixed).tolist(), reverse=True):
                 heapq.heappush(free, heapq.heappop(free) + c)
             return max(free)
 
+        chain_env = os.environ.get("ODMKV_DECODE_CHAINS")                # "0": never, "1": always (measurements)
+        may_chain = q_s.size > 0 and bool((~q_first).any()) and chain_env != "0"
         explicit = target_items if target_items is not None else (env_target or None)
         if explicit is not None:
-            items = cut(fit(int(explicit)))
+            items = cut_chained(fit_chained(int(explicit))) if (may_chain and chain_env == "1") else cut(fit(int(explicit)))
         else:
             # the comparison is repeated only when the store has grown by more than 5 % since the
             # last one (a decode-time flush adds a fraction of a percent): until then its winner is re-cut
             chosen = self._items_choice
             if chosen is not None and abs(total_bytes - chosen[1]) <= 0.05 * chosen[1]:
-                items = cut(fit(int(n_cu * chosen[0])))
+                items = (cut_chained(fit_chained(int(n_cu * chosen[0]))) if chosen[2] and may_chain
+                         else cut(fit(int(n_cu * chosen[0]))))
             else:
                 best = None
-                for mult in (1.0, 1.5, 2.0, 3.0, 4.0):
-                    cand = cut(fit(int(n_cu * mult)))
-                    t = makespan(cand)
-                    if best is None or t < best[0] - 1e-9:
-                        best = (t, cand, mult)
+                if chain_env != "1" or not may_chain:
+                    for mult in (1.0, 1.5, 2.0, 3.0, 4.0):
+                        cand = cut(fit(int(n_cu * mult)))
+                        t = makespan(cand)
+                        if best is None or t < best[0] - 1e-9:
+                            best = (t, cand, mult, False)
+                if may_chain:
+                    # only lists with more runs than compute units can gain: a chain saves the fixed part of a workgroup
+                    plain_t = None if best is None else makespan(best[1], _CHAIN_ITEM_FIXED_US)
+                    if plain_t is None or len(best[1]) > n_cu:
+                        link = None
+                        for mult in (1.0, 1.5, 2.0, 3.0, 4.0):
+                            cand = cut_chained(fit_chained(int(n_cu * mult)))
+                            t = makespan(cand, _CHAIN_ITEM_FIXED_US)
+                            if link is None or t < link[0] - 1e-9:
+                                link = (t, cand, mult, True)
+                        if plain_t is None or link[0] < (1.0 - _CHAIN_MIN_GAIN) * plain_t:
+                            best = link
                 items = best[1]
-                self._items_choice = (best[2], total_bytes)
+                self._items_choice = (best[2], total_bytes, best[3])
         arr = items.astype(np.int32).reshape(-1, 8)
         per_seg = np.bincount(arr[:, 0], minlength=self._nseg) if len(items) else np.zeros(self._nseg, np.int64)
         ranges = np.concatenate([[0], np.cumsum(per_seg)])          # items are generated in segment order
         order = None
-        if len(items) > n_cu:
-            order = np.argsort(-cost(items), kind="stable").astype(np.int32)
+        heads = np.flatnonzero(arr[:, 7] == 0) if len(items) else np.zeros(0, np.int64)
+        chained = len(items) > 0 and heads.size != len(items)
+        if len(items) > n_cu or chained:
+            # the workgroups' first items, longest workgroup first
+            order = heads[np.argsort(-cost(items), kind="stable")].astype(np.int32)
         # one upload for the item table, the ranges and the order (the parts start at multiples of 4 integers)
         n_arr, n_rng = arr.size, (ranges.size + 3) & ~3
         blob = np.zeros(n_arr + n_rng + (0 if order is None else order.size), np.int32)
@@ -824,10 +926,16 @@ class TurboQuantAdaptiveKVCacheState:
         w.items, w.item_range = self._items[0].data_ptr(), self._items[1].data_ptr()
         w.dispatch_order = _lib.ptr(self._item_order)
         w.n_items = len(items)
+        w.n_workgroups = int(heads.size) if chained else 0
         # wavefronts per item: eight for short items (less set-up, a lighter combine); for long ones sixteen where
         # the narrow levels carry the bytes (their loop wants four wavefronts per SIMD) and twelve where 4- and 8-bit
         # tokens do (memory-bound: a third unit in flight per wavefront pays more than the fourth wavefront)
-        quant = arr[arr[:, 1] < 4, 3] if len(items) else arr[:0, 3]
+        if chained:                                                     # quantised tiles per workgroup
+            qi = (arr[:, 1] & 7) < 4
+            quant = np.bincount((np.cumsum(arr[:, 7] == 0) - 1)[qi], arr[qi, 3])
+            quant = quant[quant > 0]
+        else:
+            quant = arr[arr[:, 1] < 4, 3] if len(items) else arr[:0, 3]
         q_bytes = [int(used[li].sum()) * _TILE_BYTES[li] for li in range(4)]
         wide = (q_bytes[2] + q_bytes[3]) >= 0.4 * max(sum(q_bytes), 1)
         # (items of 6 to 15 tiles that are mostly 3 bits and wider: twelve as well, 2-3 % ahead of eight, measured on

@@ -258,6 +258,62 @@ def test_step_in_one_call_equals_append_then_attention(dtype):
     assert torch.equal(ka, kb) and torch.equal(va, vb)
 
 
+@pytest.mark.parametrize("G,waves", [(4, 16), (4, 8), (2, 12), (7, 16), (8, 8)])
+def test_workgroups_that_take_several_levels_of_a_pair(G, waves, monkeypatch):
+    """A batch of short sequences has more (sequence, kv-head, level) runs than the device has compute units: the work
+    list then lets one workgroup walk several quantised levels of a pair one after the other (one query rotation, one
+    result).  Forced here on a small store, for every kernel form: the result is the oracle's, and the unchained work
+    list's up to what a different cut changes (the reference points of the softmax, hence the fp16 rounding of the weights)."""
+    g = torch.Generator().manual_seed(90 + G)
+    B, H, T = 3, 2, 2600
+    k = torch.randn(B, H, T, 128, generator=g).half(); v = torch.randn(B, H, T, 128, generator=g).half()
+    bits = _rand_bits(g, (B, H, T), (0.1, 0.35, 0.25, 0.15, 0.1, 0.05))
+    bits[..., :4] = 16; bits[..., -16:] = 16
+    bits[1, 0][bits[1, 0] == 3] = 2                           # a pair without 3-bit tokens: its chain skips a level
+    bits[2, 1][(bits[2, 1] != 8) & (bits[2, 1] != 16)] = 8    # a pair with one quantised level only
+    st, ref = _pair(k, v, bits)
+    q = torch.randn(B, H * G, 128, generator=g).half()
+    want = decode_attention_state(q.float(), ref)
+    monkeypatch.setenv("ODMKV_DECODE_WAVES", str(waves))
+    monkeypatch.setenv("ODMKV_DECODE_CHAINS", "0")
+    st._build_items(24, 1)
+    assert st._worklist.n_workgroups == 0
+    plain = st.decode_attention(q.to(DEV))
+    monkeypatch.setenv("ODMKV_DECODE_CHAINS", "1")
+    for target in (8, 24):
+        st._build_items(target, 1)
+        items = st._items[0].cpu().numpy()
+        assert (items[:, 6] > 0).any() and 0 < st._worklist.n_workgroups < len(items)
+        heads = items[:, 7] == 0
+        assert int(heads.sum()) == st._worklist.n_workgroups and (items[~heads, 6] == 0).all()
+        # a chain stays inside one pair, its levels ascend, and every tile of the store is covered once
+        for i in np.flatnonzero(items[:, 6] > 0):
+            chain = items[i:i + items[i, 6] + 1]
+            assert (chain[:, 0] == chain[0, 0]).all() and (np.diff(chain[:, 1] & 7) > 0).all() and ((chain[:, 1] & 7) < 4).all()
+            assert (chain[1:, 7] == 1).all()
+        got, lse = st.decode_attention(q.to(DEV), return_lse=True)
+        assert rel_err(got.cpu(), want) < ATTN_RTOL
+        assert rel_err(got.cpu(), plain.cpu().double()) < 5e-4
+        assert torch.isfinite(lse).all()
+
+
+def test_a_batch_of_short_sequences_gets_chained_workgroups_by_itself():
+    """48 sequences of 1024 tokens on 8 kv-heads: 384 pairs with four to five levels each, several runs per compute unit.
+    The work list chooses by itself to let a workgroup walk a pair's quantised levels one after the other; the result is
+    the oracle's."""
+    g = torch.Generator().manual_seed(123)
+    B, H, G, T = 48, 8, 4, 1024
+    k = torch.randn(B, H, T, 128, generator=g).half(); v = torch.randn(B, H, T, 128, generator=g).half()
+    bits = _rand_bits(g, (B, H, T), (0.12, 0.5, 0.18, 0.13, 0.06, 0.01))
+    bits[..., :4] = 16; bits[..., -32:] = 16
+    st, ref = _pair(k, v, bits)
+    q = torch.randn(B, H * G, 128, generator=g).half()
+    got = st.decode_attention(q.to(DEV))
+    w, items = st._worklist, st._items[0].cpu().numpy()
+    assert 0 < w.n_workgroups < w.n_items and (items[:, 6] > 0).any() and st._item_order.numel() == w.n_workgroups
+    assert rel_err(got.cpu(), decode_attention_state(q.float(), ref)) < ATTN_RTOL
+
+
 def test_config1_end_to_end():
     """Benchmark config 1: score -> allocate (2.0 bits) -> pack -> one-token decode, all on the GPU,
     each stage compared with the oracle fed the previous stage's GPU output."""
