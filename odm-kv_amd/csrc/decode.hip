@@ -689,7 +689,6 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
     // microsecond later).  Loads return in issue order: the (small) query goes first.
     RotQuery rq;
     if (first) request_rot_query(rq, a, bq_first, tid);
-    else __syncthreads();
     // DEPTH units of this wavefront are under way at any time: two (one for the widest rows: registers); twelve
     // wavefronts have the registers for a third 2-bit unit.  (Six units in flight with eight wavefronts were measured:
     // no gain, the eight are bound by their arithmetic.)
@@ -700,6 +699,7 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
         int u = wave;
         int nvalid = tokens_of(u);
         if (nvalid > 0) load_unit<W>(cur, a, li, unit0 + u, lane);
+        if (!first) __syncthreads();                       // (the level's first bytes are on their way while the others finish)
         build_lut<W, NW>(lut, a, tid);
         if (first) rotate_queries<GP>(a, smem, tid, bq_first, rq);
         lds_barrier();
@@ -740,6 +740,7 @@ __device__ static inline void run_quant_level(const DecodeArgs& a, int li, int b
         int nv[DEPTH];
         nv[0] = tokens_of(wave);
         if (nv[0] > 0) load_unit<W>(buf[0], a, li, unit0 + wave, lane);
+        if (!first) __syncthreads();
         build_lut<W, NW>(lut, a, tid);
         if (first) rotate_queries<GP>(a, smem, tid, bq_first, rq);
         lds_barrier();
@@ -780,11 +781,11 @@ __device__ static inline void run_quant_level_g4(const DecodeArgs& a, int li, in
     // (the order of the requests, the table and the rotation is run_quant_level's)
     RotQuery rq;
     if (first) request_rot_query(rq, a, bq_first, tid);
-    else __syncthreads();
     Unit4<W> cur;
     int u = wave;
     int nvalid = tokens_of(u);
     if (nvalid > 0) load_unit4<W>(cur, a, li, unit0 + u, lane);
+    if (!first) __syncthreads();                           // (the level's first bytes are on their way while the others finish)
     build_lut<W, NW>(lut, a, tid);
     if (first) rotate_queries<4>(a, smem, tid, bq_first, rq);
     lds_barrier();

@@ -56,16 +56,16 @@ _TILE_BYTES = [TILE * 16 * w + 2 * TILE * 4 for w in WIDTHS] + [2 * TILE * HEAD_
 # and per work item (microseconds: start, table, query rotation, combining the wavefronts)
 _TILE_COST = [300, 420, 450, 890, 1310]
 _ITEM_FIXED_US = 4.0           # what the cuts without chains are compared with (its choices were measured shape by shape)
-# Chains (a workgroup that walks several levels of a pair) are weighed against the best cut without them with constants
-# fitted to whole-call times of lists of 256 to 3000 items (64 sequences of 2048 tokens, mixed levels: 90 us without
-# chains, 69 us with, both reproduced to a microsecond): a workgroup 6 us beside its tiles, a further level 2.1 us (a
-# barrier, the new table, its first bytes from memory), 1 us because a chained workgroup rotates its queries before it asks
-# for the first unit.  They are taken when the model promises 15 % (16 sequences of 8192 tokens: 4 %, measured the same
-# or slower: not taken).
-_CHAIN_ITEM_FIXED_US = 6.0
-_CHAIN_LINK_US = 2.1
+# Chains (a workgroup that walks several quantised levels of a pair, _build_items) by a rule, not by the cost model, which
+# is off by a third either way on lists of several rounds: they are taken when the quantised runs number at least 1.5 per
+# compute unit and 2.5 per pair, cut so that the workgroups number 1.5 per compute unit or, with more pairs than that,
+# one per pair beside the exact items.  Measured whole calls: 64 sequences x 2048 tokens x 8 kv-heads, four levels each:
+# 90 -> 67 us; 16 x 8192 tokens with four levels: 44 -> 36 us; 16 x 8192 tokens with two levels (c3): no gain at any cut,
+# not taken by the rule.  The link and rotation costs below only rank the workgroups for the dispatch order.
+_CHAIN_LINK_US = 1.8
 _CHAIN_ROTATE_US = 1.0
-_CHAIN_MIN_GAIN = 0.15
+_CHAIN_RUNS_PER_CU = 1.5
+_CHAIN_RUNS_PER_PAIR = 2.5
 
 
 _U64x33 = C.c_uint64 * 33
@@ -889,18 +889,12 @@ class TurboQuantAdaptiveKVCacheState:
                         t = makespan(cand)
                         if best is None or t < best[0] - 1e-9:
                             best = (t, cand, mult, False)
-                if may_chain:
-                    # only lists with more runs than compute units can gain: a chain saves the fixed part of a workgroup
-                    plain_t = None if best is None else makespan(best[1], _CHAIN_ITEM_FIXED_US)
-                    if plain_t is None or len(best[1]) > n_cu:
-                        link = None
-                        for mult in (1.0, 1.5, 2.0, 3.0, 4.0):
-                            cand = cut_chained(fit_chained(int(n_cu * mult)))
-                            t = makespan(cand, _CHAIN_ITEM_FIXED_US)
-                            if link is None or t < link[0] - 1e-9:
-                                link = (t, cand, mult, True)
-                        if plain_t is None or link[0] < (1.0 - _CHAIN_MIN_GAIN) * plain_t:
-                            best = link
+                n_pairs = int(q_first.sum())
+                if may_chain and (chain_env == "1" or (q_s.size >= _CHAIN_RUNS_PER_CU * n_cu
+                                                       and q_s.size >= _CHAIN_RUNS_PER_PAIR * n_pairs)):
+                    n_exact = int((run_li == 4).sum())
+                    mult = max(1.5, (n_pairs + n_exact) / n_cu)
+                    best = (0.0, cut_chained(fit_chained(int(n_cu * mult))), mult, True)
                 items = best[1]
                 self._items_choice = (best[2], total_bytes, best[3])
         arr = items.astype(np.int32).reshape(-1, 8)
