@@ -972,9 +972,10 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
         if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
         else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
     } else {
-        // The levels of a chain ascend: the four walkers stand one behind the other, each taken if the current item is of
-        // its level.  The queries are rotated before the first of them (its barrier is the walker's own).
-        {
+        // The levels of a chain ascend: the four walkers stand one behind the other, each taken if the chain has an item of
+        // its level.  A 2-bit item is always a chain's first: its walker rotates the queries as an unchained one does (beside
+        // its first requests); chains that start higher rotate them up front.
+        if (li != 0) {
             RotQuery rq;
             request_rot_query(rq, a, bq_first, tid);
             rotate_queries<GP>(a, smem, tid, bq_first, rq);
@@ -998,7 +999,7 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
         tile0 = first_tile0; ntiles = first_ntiles; ntok = first_ntok; \
         _Pragma("unroll") for (int k = 0; k < 3; ++k) \
             if (k < follow && r0[k].y == L) { has = true; tile0 = r0[k].z; ntiles = r0[k].w; ntok = r1[k].x; }
-        { ODMKV_PICK_LEVEL(0) if (has) ODMKV_RUN_LEVEL(2, 0, false); }
+        { ODMKV_PICK_LEVEL(0) if (has) ODMKV_RUN_LEVEL(2, 0, true); }
         { ODMKV_PICK_LEVEL(1) if (has) ODMKV_RUN_LEVEL(3, 1, false); }
         { ODMKV_PICK_LEVEL(2) if (has) ODMKV_RUN_LEVEL(4, 2, false); }
         { ODMKV_PICK_LEVEL(3) if (has) ODMKV_RUN_LEVEL(8, 3, false); }
