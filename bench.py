@@ -573,23 +573,29 @@ def main() -> int:
                 sweep(mask)
             for _ in range(3):
                 gk.replay()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            e0.record()
-            for _ in range(reps):
-                gk.replay()
-            e1.record()
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) / (reps * n_stores) * 1e3
+            rounds = []
+            for _ in range(5):                      # five rounds of `reps` replays: the median, and the extremes beside it
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                e0.record()
+                for _ in range(reps):
+                    gk.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                rounds.append(e0.elapsed_time(e1) / (reps * n_stores) * 1e3)
+            rounds.sort()
+            return rounds[2], rounds[0], rounds[-1]
 
         pb = sum(st.packed_bytes() for st in sts) / n_stores
-        main_us, call_us = graph_us(2), graph_us(6)
+        (main_us, main_lo, main_hi), (call_us, call_lo, call_hi) = graph_us(2), graph_us(6)
         print(json.dumps({"decode_shape": name, "stores": n_stores, "sequences": Bs, "tokens": int(sts[0].seq_len),
                           "packed_bytes_per_store": int(pb), "work_items": int(sts[0]._items[2]),
                           "level_counts": {str(b): int(sum(st.level_counts()[b] for st in sts) / n_stores) for b in LEVELS},
-                          "main_kernel_us": round(main_us, 2), "main_kernel_GBps": round(pb / main_us / 1e3, 1),
+                          "main_kernel_us": round(main_us, 2), "main_kernel_us_min_max": [round(main_lo, 2), round(main_hi, 2)],
+                          "main_kernel_GBps": round(pb / main_us / 1e3, 1),
                           "main_kernel_frac_of_8TBps": round(pb / main_us / 1e3 / 8000.0, 4),
-                          "whole_call_us": round(call_us, 2), "whole_call_GBps": round(pb / call_us / 1e3, 1)}))
+                          "whole_call_us": round(call_us, 2), "whole_call_us_min_max": [round(call_lo, 2), round(call_hi, 2)],
+                          "whole_call_GBps": round(pb / call_us / 1e3, 1)}))
         return 0
 
     # ---- compress every layer: score -> allocate -> window -> pack (timed per layer) ----
