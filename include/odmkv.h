@@ -206,14 +206,15 @@ int odmkv_store_gather(const odmkv_packed_t* staging, const odmkv_packed_t* stor
 
 /* The other half of a staged first fill, in one call, once counts_event has arrived: the chunk counts (host memory,
  * as odmkv_quant_pack_staged delivered them) are added up into counts (host int32 [B*Hkv, 6]); every segment gets a
- * tile per 64 tokens, the exact segments `exact_slack` tokens of room to grow (seg_tile: host int32 [5][B*Hkv + 1],
- * written); the store is laid out in `arena` (offsets, sizes, marks as odmkv_store_layout gives them), prepared
+ * tile per 64 tokens, the exact segments `exact_slack` tokens of room to grow and, if `quant_headroom` is not 0, every
+ * quantised segment a sixteenth more tiles (two at least) for the tokens that decode-time flushes add, so that the
+ * first of them need not move the store (seg_tile: host int32 [5][B*Hkv + 1], written); the store is laid out in `arena` (offsets, sizes, marks as odmkv_store_layout gives them), prepared
  * (odmkv_store_init), described (odmkv_store_bind into `store`) and filled from the staging store
  * (odmkv_store_gather).  need_bytes receives the size of the layout; if `arena` is NULL or smaller, nothing is
  * launched and ODMKV_ENOSPACE returned: allocate and call again.  Counts that do not add up to B*Hkv*T (a value that
  * is no level) give ODMKV_EINVAL.  No counterpart in the reference. */
 int odmkv_store_finish_staged(const int32_t* chunk_counts, int n_chunks, int B, int Hkv, int T,
-                              int exact_slack, int exact_dtype, void* arena, uint64_t arena_bytes,
+                              int exact_slack, int quant_headroom, int exact_dtype, void* arena, uint64_t arena_bytes,
                               const odmkv_packed_t* staging, int32_t* counts, int32_t* seg_tile,
                               uint64_t* offsets, uint64_t* sizes, uint64_t* marks,
                               odmkv_packed_t* store, uint64_t* need_bytes, void* stream);

@@ -1790,12 +1790,14 @@ extern "C" int odmkv_store_gather(const odmkv_packed_t* staging, const odmkv_pac
 }
 
 // The second half of a staged first fill, in one call, for the moment the level counts have arrived: add up the chunks,
-// size every segment (a tile per 64 tokens; the exact segments with `exact_slack` tokens of room to grow), lay the store
+// size every segment (a tile per 64 tokens; the exact segments with `exact_slack` tokens of room to grow; with
+// `quant_headroom` every quantised segment a sixteenth more tiles, two at least, for the tokens later flushes add), lay the store
 // out in `arena`, prepare it (odmkv_store_init), fill the descriptor and move the staging store's tiles over
 // (odmkv_store_gather).  What the host does between the arrival of the counts and the launch of the gather decides
 // whether the GPU runs dry behind the quantiser; here that is a few microseconds of arithmetic and two launches.
 extern "C" int odmkv_store_finish_staged(const int32_t* chunk_counts, int n_chunks, int B, int Hkv, int T,
-                                         int exact_slack, int exact_dtype, void* arena, uint64_t arena_bytes,
+                                         int exact_slack, int quant_headroom, int exact_dtype, void* arena,
+                                         uint64_t arena_bytes,
                                          const odmkv_packed_t* staging, int32_t* counts, int32_t* seg_tile,
                                          uint64_t* offsets, uint64_t* sizes, uint64_t* marks,
                                          odmkv_packed_t* store, uint64_t* need_bytes, void* stream) {
@@ -1817,7 +1819,9 @@ extern "C" int odmkv_store_finish_staged(const int32_t* chunk_counts, int n_chun
         row[0] = 0;
         for (int s = 0; s < nseg; ++s) {
             const long long n = (long long)counts[s * 6 + li + 1] + (li == 4 ? exact_slack : 0);
-            row[s + 1] = row[s] + (int32_t)((n + TILE - 1) / TILE);
+            long long tiles = (n + TILE - 1) / TILE;
+            if (li < 4 && quant_headroom) tiles += std::max(tiles / 16, 2LL);
+            row[s + 1] = row[s] + (int32_t)tiles;
         }
     }
     if (int rc = odmkv_store_layout(seg_tile, nseg, offsets, sizes, marks)) return rc;

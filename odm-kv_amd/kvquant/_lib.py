@@ -88,7 +88,7 @@ def _load() -> C.CDLL:
         "odmkv_lloyd_max": (C.c_int, [i32, i32, i32, C.c_double, C.c_double, vp, vp, vp]),
         "odmkv_rotation_operands": (C.c_int, [vp, vp, vp]),
         "odmkv_pack_count_chunks": (C.c_int, [i32]),
-        "odmkv_store_finish_staged": (C.c_int, [vp, i32, i32, i32, i32, i32, i32, vp, C.c_uint64, C.POINTER(Packed), vp, vp,
+        "odmkv_store_finish_staged": (C.c_int, [vp, i32, i32, i32, i32, i32, i32, i32, vp, C.c_uint64, C.POINTER(Packed), vp, vp,
                                                 vp, vp, vp, C.POINTER(Packed), vp, vp]),
         "odmkv_dequant": (C.c_int, [C.POINTER(Packed), vp, vp, i32, i32, i64, i64, i64, vp, vp, vp, i32, vp]),
         "odmkv_dequant_from": (C.c_int, [C.POINTER(Packed), vp, vp, i32, i32, i32, i64, i64, i64, vp, vp, vp, i32, vp]),

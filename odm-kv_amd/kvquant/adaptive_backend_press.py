@@ -94,7 +94,7 @@ class TurboQuantPerTokenBackendPress(TurboQuantPerTokenPress):
             head_dim=keys.shape[-1], bit_levels=levels, key_quantizer=self.key_quantizer,
             value_quantizer=self.value_quantizer, value_group_size=self.value_group_size,
             device=keys.device, dtype=keys.dtype, seed=self.seed + layer_idx * 7,
-            outlier_min_bits=self.outlier_min_bits)
+            outlier_min_bits=self.outlier_min_bits, quant_headroom=self.buffer_size > 0 and self.decode_quant)
         state.exact_decode_append = self.buffer_size > 0 and self.decode_quant
         self._states[layer_idx] = state
         return state

@@ -240,7 +240,8 @@ class TurboQuantAdaptiveKVCacheState:
     def __init__(self, head_dim: int, bit_levels, value_group_size: int = 32, device=None,
                  dtype: torch.dtype = torch.float16, key_quantizer: str = "prod",
                  value_quantizer: str = "minmax", seed: int = 42, outlier_indices=None,
-                 regular_indices=None, outlier_min_bits: int = 4, exact_slack: int = 256):
+                 regular_indices=None, outlier_min_bits: int = 4, exact_slack: int = 256,
+                 quant_headroom: bool = False):
         levels = tuple(sorted(set(int(b) for b in bit_levels)))
         self.key_quantizer = normalize_key_quantizer(key_quantizer)
         self.value_quantizer = normalize_value_quantizer(value_quantizer)
@@ -272,6 +273,8 @@ class TurboQuantAdaptiveKVCacheState:
         self.seed = seed
         self.outlier_min_bits = outlier_min_bits
         self.exact_slack = int(exact_slack)
+        # room in the quantised segments from the first fill on, for a store that decode-time flushes will add to
+        self.quant_headroom = bool(quant_headroom)
         if self.device.type != "cuda":
             raise RuntimeError("the packed KV store lives on the GPU; there is no CPU path")
         self.pi_k = cached_rotation(head_dim, self.device, seed)
@@ -367,10 +370,11 @@ class TurboQuantAdaptiveKVCacheState:
             if np.all((new_counts + TILE - 1) // TILE <= have):
                 return
         cap = self._capacity_tiles(new_counts)
-        if self._bufs is not None:
+        if self._bufs is not None or self.quant_headroom:
             # a store that grows once will grow again (every decode-time flush adds tokens to the
             # quantised levels): leave a sixteenth of head-room so that the tiles move rarely
             cap[:4] += np.maximum(cap[:4] // 16, 2)
+        if self._bufs is not None:
             cap = np.maximum(cap, np.diff(self._seg_tile, axis=1))
         seg_tile = np.zeros((5, self._nseg + 1), np.int64)
         seg_tile[:, 1:] = np.cumsum(cap, axis=1)
@@ -486,7 +490,7 @@ class TurboQuantAdaptiveKVCacheState:
             for attempt in (0, 1):
                 arena = getattr(self, "_arena", None)
                 rc = lib.odmkv_store_finish_staged(
-                    box.data_ptr(), n_chunks, B, H, T, int(self.exact_slack),
+                    box.data_ptr(), n_chunks, B, H, T, int(self.exact_slack), int(self.quant_headroom),
                     _lib.BF16 if self._exact_torch_dtype == torch.bfloat16 else _lib.F16,
                     None if arena is None else arena.data_ptr(), 0 if arena is None else max(arena.numel() - lm_bytes, 0),
                     C.byref(stg.packed), counts32.ctypes.data, new_lay.tables_ptr, new_lay.offsets, new_lay.sizes,

@@ -190,9 +190,9 @@ def test_store_finish_staged_sizes_the_store_without_a_gpu(lib):
     off, size, marks = (C.c_uint64 * 33)(), (C.c_uint64 * 33)(), (C.c_uint64 * 5)()
     staging, store, need = Packed(), Packed(), C.c_uint64(0)
     f = lib.odmkv_store_finish_staged
-    f.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_uint64, C.POINTER(Packed),
+    f.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_uint64, C.POINTER(Packed),
                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(Packed), C.c_void_p, C.c_void_p]
-    rc = f(chunks.ctypes.data, n_chunks, B, H, T, slack, 0, None, 0, C.byref(staging), counts.ctypes.data,
+    rc = f(chunks.ctypes.data, n_chunks, B, H, T, slack, 0, 0, None, 0, C.byref(staging), counts.ctypes.data,
            seg_tile.ctypes.data, off, size, marks, C.byref(store), C.byref(need), None)
     assert rc == -2 and b"needs" in lib.odmkv_last_error()
     assert np.array_equal(counts, per_seg)
@@ -200,7 +200,15 @@ def test_store_finish_staged_sizes_the_store_without_a_gpu(lib):
     want[4] = (per_seg[:, 5] + slack + 63) // 64
     assert np.array_equal(np.diff(seg_tile, axis=1), want) and np.all(seg_tile[:, 0] == 0)
     assert need.value == marks[4] > 0
+    plain = need.value
+    # with head-room for later flushes: a sixteenth more tiles, two at least, in every quantised segment
+    rc = f(chunks.ctypes.data, n_chunks, B, H, T, slack, 1, 0, None, 0, C.byref(staging), counts.ctypes.data,
+           seg_tile.ctypes.data, off, size, marks, C.byref(store), C.byref(need), None)
+    assert rc == -2
+    roomy = want.copy()
+    roomy[:4] += np.maximum(roomy[:4] // 16, 2)
+    assert np.array_equal(np.diff(seg_tile, axis=1), roomy) and need.value > plain
     chunks[2, 1, 4] += 1                                               # one token too many
-    rc = f(chunks.ctypes.data, n_chunks, B, H, T, slack, 0, None, 0, C.byref(staging), counts.ctypes.data,
+    rc = f(chunks.ctypes.data, n_chunks, B, H, T, slack, 0, 0, None, 0, C.byref(staging), counts.ctypes.data,
            seg_tile.ctypes.data, off, size, marks, C.byref(store), C.byref(need), None)
     assert rc == -1 and b"must take values" in lib.odmkv_last_error()

@@ -213,6 +213,36 @@ def test_append_truncate_and_flush_follow_the_oracle():
     _ulp_close_fp16(km.cpu(), kr)
 
 
+def test_a_store_with_room_for_flushes_holds_the_same_tokens_and_does_not_move():
+    """quant_headroom=True (what the press asks for when it will flush decode-time tokens into the quantised levels):
+    the first fill, staged (T >= 256) or not, leaves a sixteenth more tiles (two at least) in every quantised
+    segment; the stored tokens are the oracle's, and the tokens of a flush fit without the store being laid out again."""
+    from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
+    g = torch.Generator().manual_seed(123)
+    for T in (200, 700):
+        B, H, D = 1, 3, 128
+        k = torch.randn(B, H, T, D, generator=g).half(); v = torch.randn(B, H, T, D, generator=g).half()
+        bits = _rand_bits(g, (B, H, T)); bits[..., -8:] = 16
+        state = TurboQuantAdaptiveKVCacheState(128, (0, 2, 3, 4, 8, 16), device=DEV, dtype=torch.float16, key_quantizer="mse",
+                                               value_quantizer="mse", seed=42, quant_headroom=True)
+        plain = _state()
+        ref = KVState(128, (0, 2, 3, 4, 8, 16), seed=42, order="canonical")
+        state.prefill(k.to(DEV), v.to(DEV), bits.to(DEV)); plain.prefill(k.to(DEV), v.to(DEV), bits.to(DEV)); ref.prefill(k, v, bits)
+        have, base = np.diff(state._seg_tile, axis=1), np.diff(plain._seg_tile, axis=1)
+        assert np.array_equal(have[:4], base[:4] + np.maximum(base[:4] // 16, 2)) and np.array_equal(have[4], base[4])
+        _check_store_against_oracle(state, ref)
+        assert state.packed_bytes() == ref.packed_bytes()
+        arena, tiles = state._bufs.arena.data_ptr(), state._seg_tile.copy()
+        # 100 more tokens per head at the quantised levels: inside the room left
+        k1 = torch.randn(B, H, 100, D, generator=g).half(); v1 = torch.randn(B, H, 100, D, generator=g).half()
+        bits1 = _rand_bits(g, (B, H, 100), probs=(0.0, 0.4, 0.25, 0.2, 0.15, 0.0))
+        state.append(k1.to(DEV), v1.to(DEV), bits1.to(DEV)); ref.append(k1, v1, bits1)
+        assert state._bufs.arena.data_ptr() == arena and np.array_equal(state._seg_tile, tiles)
+        _check_store_against_oracle(state, ref)
+        km, vm = state.materialize(); kr, vr = ref.materialize()
+        _ulp_close_fp16(km.cpu(), kr); _ulp_close_fp16(vm.cpu(), vr)
+
+
 def test_edge_cases_and_errors():
     from kvquant.tq_adaptive_backend import TurboQuantAdaptiveKVCacheState
     g = torch.Generator().manual_seed(5)
