@@ -385,6 +385,10 @@ typedef struct odmkv_worklist {
                                       * dispatch_order[k] and also takes the items[.][6] items behind it (further quantised
                                       * levels of the same (sequence, kv-head): one query rotation, one result); those
                                       * items carry items[.][7] = 1 */
+    int32_t two_per_cu;              /* 1: the workgroups (eight wavefronts; needs dispatch_order) are the build that keeps to
+                                      * 128 registers a wavefront and half a compute unit's LDS, so that two of them share a
+                                      * compute unit and one streams while the other starts or finishes: for lists with more
+                                      * items than compute units (a batch of sequences, many levels).  0: one per compute unit */
 } odmkv_worklist_t;
 
 size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items);

@@ -59,7 +59,7 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 #define LDS_PBUFS (LDS_QROWS + 16 * QROW_LDS)
 template <int NW>
 struct Lds {
-    static constexpr int SCALARS = LDS_PBUFS + NW * 2 * PBUF;
+    static constexpr int SCALARS = LDS_PBUFS + NW * PBUF;
     static constexpr int TOTAL = SCALARS + NW * 4 * 8 * 4 + 8 * 4;
     static_assert(NW * ODMKV_MAX_GROUP * HD * 4 <= LUT_BYTES, "combine area must fit the table's space");
     static_assert(NW >= 8 && NW <= 16, "wave count (the first eight rotate the queries)");
@@ -845,7 +845,7 @@ __device__ static inline void load_exact_unit(ExactUnit& t, const uint16_t* base
 // softmax weights (bf16 high + low piece) on the bf16 matrix instructions, products exact, sums fp32.
 template <bool BF, int NW>
 __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int bq_first, int tile0, int ntiles, int seg_first,
-                                              int tid, uint8_t* pbuf, float* alpha_sh, WaveState& st) {
+                                              int tid, uint8_t* pbuf, uint8_t* pbuf_lo, float* alpha_sh, WaveState& st) {
     const int wave = tid >> 6, lane = tid & 63, n = lane & 15, j = lane >> 4;
     const float esc = a.scaling * LOG2E;
     // the query itself (no rotation): row 2h = q16 of head h, row 2h+1 = zero for fp16 rows; for bf16 rows the two
@@ -896,11 +896,11 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
         float pA[2], pB[2];
         softmax_unit(st, tA, tB, lane, alpha_sh, pA, pB);
         if constexpr (BF) {
-            // p = hi + lo in bf16: two p buffers, two products
+            // p = hi + lo in bf16: two p buffers (the second in the table's space, which an exact item does not use), two products
             *reinterpret_cast<uint32_t*>(pbuf + (2 * j) * PROW + 4 * n) = bf16_pair(pA[0], pA[1]);
             *reinterpret_cast<uint32_t*>(pbuf + (2 * j + 1) * PROW + 4 * n) = bf16_pair(pB[0], pB[1]);
-            *reinterpret_cast<uint32_t*>(pbuf + PBUF + (2 * j) * PROW + 4 * n) = bf16_pair(bf16_rest(pA[0]), bf16_rest(pA[1]));
-            *reinterpret_cast<uint32_t*>(pbuf + PBUF + (2 * j + 1) * PROW + 4 * n) = bf16_pair(bf16_rest(pB[0]), bf16_rest(pB[1]));
+            *reinterpret_cast<uint32_t*>(pbuf_lo + (2 * j) * PROW + 4 * n) = bf16_pair(bf16_rest(pA[0]), bf16_rest(pA[1]));
+            *reinterpret_cast<uint32_t*>(pbuf_lo + (2 * j + 1) * PROW + 4 * n) = bf16_pair(bf16_rest(pB[0]), bf16_rest(pB[1]));
         } else {
             *reinterpret_cast<uint32_t*>(pbuf + (2 * j) * PROW + 4 * n) = pack_h2(pA[0], pA[1]);
             *reinterpret_cast<uint32_t*>(pbuf + (2 * j + 1) * PROW + 4 * n) = pack_h2(pB[0], pB[1]);
@@ -908,7 +908,7 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
         wave_lds_fence();
         const uint4 phi = *reinterpret_cast<const uint4*>(pbuf + (n & 7) * PROW + 16 * j);
         if constexpr (BF) {
-            const uint4 plo = *reinterpret_cast<const uint4*>(pbuf + PBUF + (n & 7) * PROW + 16 * j);
+            const uint4 plo = *reinterpret_cast<const uint4*>(pbuf_lo + (n & 7) * PROW + 16 * j);
 #pragma unroll
             for (int m = 0; m < 8; ++m) {
                 st.acc[m] = MFMA_BF16(as_bf8(phi), as_bf8(v.c[m]), st.acc[m]);
@@ -929,9 +929,13 @@ __device__ static inline void run_exact_level(const DecodeArgs& a, int bh, int b
 // CHAIN: a workgroup may take several consecutive items, the quantised levels of one (sequence, kv-head) one after the
 // other (item word 6 = how many follow): the queries are rotated once, the accumulators run through, the table is rebuilt
 // between the levels, one result is written at the first item's place and empty results at the others'.
-template <int GP, bool ORDERED, int NW, bool G4 = false, bool CHAIN = false>
-__global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
-    static_assert(!G4 || (GP == 4 && NW == 16), "the shared-lane form is built for four heads and sixteen wavefronts");
+// PAIR: eight wavefronts held to 128 registers each (four wavefronts per SIMD) and half a compute unit's LDS, so that two
+// workgroups share a compute unit: while one sets up or combines, the other streams.  For lists with more items than
+// compute units, whose workgroups would otherwise run one after the other, each paying its start and its end alone.
+template <int GP, bool ORDERED, int NW, bool G4 = false, bool CHAIN = false, bool PAIR = false>
+__global__ __launch_bounds__(NW * 64, PAIR ? 4 : 1) void decode_main_kernel(DecodeArgs a) {
+    static_assert(!G4 || (GP == 4 && (NW == 16 || PAIR)), "the shared-lane form is built for four heads and four wavefronts per SIMD");
+    static_assert(!PAIR || (NW == 8 && 2 * Lds<NW>::TOTAL <= 160 * 1024), "two workgroups of eight wavefronts share a compute unit");
     static_assert(!CHAIN || ORDERED, "chains come with a dispatch order (fewer workgroups than items)");
     // one static LDS block: the table sits at LDS address 0 and that is known when the kernel is compiled, so a
     // lookup address needs no base added
@@ -959,7 +963,8 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
     st.mA = -INFINITY; st.mB = -INFINITY; st.lA = 0.0f; st.lB = 0.0f;
 #pragma unroll
     for (int nb = 0; nb < 8; ++nb) st.acc[nb] = (f4){0.f, 0.f, 0.f, 0.f};
-    uint8_t* pbuf = smem + LDS_PBUFS + wave * 2 * PBUF;
+    uint8_t* pbuf = smem + LDS_PBUFS + wave * PBUF;
+    uint8_t* pbuf_lo = smem + wave * PBUF;                 // bf16 exact rows: the weights' low pieces (the table's space)
     float* alpha_sh = alphas + wave * 8;
 #define ODMKV_RUN_LEVEL(W, L, FIRST) \
     do { if constexpr (G4) run_quant_level_g4<W, NW>(a, L, bq_first, tile0, ntiles, ntok, tid, smem, pbuf, alpha_sh, st, FIRST); \
@@ -971,13 +976,13 @@ __global__ __launch_bounds__(NW * 64) void decode_main_kernel(DecodeArgs a) {
             case 2: ODMKV_RUN_LEVEL(4, 2, true); break;
             case 3: ODMKV_RUN_LEVEL(8, 3, true); break;
             default:
-                if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
-                else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
+                if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, pbuf_lo, alpha_sh, st);
+                else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, pbuf_lo, alpha_sh, st);
                 break;
         }
     } else if (li == 4) {
-        if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
-        else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, alpha_sh, st);
+        if (a.s.exact_dtype == ODMKV_BF16) run_exact_level<true, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, pbuf_lo, alpha_sh, st);
+        else run_exact_level<false, NW>(a, bh, bq_first, tile0, ntiles, d1.y, tid, pbuf, pbuf_lo, alpha_sh, st);
     } else {
         // The levels of a chain ascend: the four walkers stand one behind the other, each taken if the chain has an item of
         // its level.  A 2-bit item is always a chain's first: its walker rotates the queries as an unchained one does (beside
@@ -1200,9 +1205,9 @@ extern "C" size_t odmkv_decode_workspace_bytes(int B, int Hq, int n_items) {
     return align_up((size_t)(n_items > 0 ? n_items : 1) * ODMKV_MAX_GROUP * PSTRIDE * sizeof(float), 256);
 }
 
-template <int GP, bool ORDERED, int NW, bool G4 = false, bool CHAIN = false>
+template <int GP, bool ORDERED, int NW, bool G4 = false, bool CHAIN = false, bool PAIR = false>
 static int launch_main(const DecodeArgs& a, int grid, hipEvent_t e0, hipEvent_t e1, hipStream_t st) {
-    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED, NW, G4, CHAIN>), dim3(grid), dim3(NW * 64), 0, st, e0, e1, 0, a);
+    hipExtLaunchKernelGGL((decode_main_kernel<GP, ORDERED, NW, G4, CHAIN, PAIR>), dim3(grid), dim3(NW * 64), 0, st, e0, e1, 0, a);
     ODMKV_CHECK_LAUNCH("decode_main_kernel");
     return 0;
 }
@@ -1226,6 +1231,8 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
                     "decode_attn: %d wavefronts per work item (0, 8, 12 or 16)", work->wavefronts);
     ODMKV_CHECK_ARG(work->item_range, "decode_attn: null item ranges");
     ODMKV_CHECK_ARG(n_items == 0 || work->items, "decode_attn: null work list");
+    ODMKV_CHECK_ARG(work->two_per_cu == 0 || ((work->wavefronts == 0 || work->wavefronts == 8) && work->dispatch_order),
+                    "decode_attn: two workgroups per compute unit take eight wavefronts each and a dispatch order");
     ODMKV_CHECK_ARG(work->n_workgroups >= 0 && work->n_workgroups <= n_items, "decode_attn: %d workgroups for %d items", work->n_workgroups, n_items);
     ODMKV_CHECK_ARG(work->n_workgroups == 0 || work->n_workgroups == n_items || work->dispatch_order,
                     "decode_attn: workgroups that take several items need the dispatch order (their first items)");
@@ -1265,7 +1272,14 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
         const bool g4 = GP == 4 && nw == 16 && g4_forced != 0;
         const bool chain = work->n_workgroups > 0 && work->n_workgroups != n_items;      // workgroups that take several items
         const int grid = chain ? work->n_workgroups : n_items;
-        if (chain && g4) rc = launch_main<4, true, 16, true, true>(a, grid, e0, e1, st);
+        // two eight-wavefront workgroups per compute unit (always with a dispatch order: the list has more items than
+        // compute units); groups of up to four heads in the shared-lane form
+        const bool pair = work->two_per_cu != 0 && (GP == 8 || g4_forced != 0);
+        if (pair && GP == 4) rc = chain ? launch_main<4, true, 8, true, true, true>(a, grid, e0, e1, st)
+                                                          : launch_main<4, true, 8, true, false, true>(a, grid, e0, e1, st);
+        else if (pair) rc = chain ? launch_main<8, true, 8, false, true, true>(a, grid, e0, e1, st)
+                                  : launch_main<8, true, 8, false, false, true>(a, grid, e0, e1, st);
+        else if (chain && g4) rc = launch_main<4, true, 16, true, true>(a, grid, e0, e1, st);
         else if (chain && GP == 4) rc = ODMKV_LAUNCH_MAIN(4, true, true);
         else if (chain) rc = ODMKV_LAUNCH_MAIN(8, true, true);
         else if (g4 && !a.order) rc = launch_main<4, false, 16, true>(a, grid, e0, e1, st);

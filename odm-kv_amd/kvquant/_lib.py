@@ -40,7 +40,7 @@ class Worklist(C.Structure):
     """struct odmkv_worklist of include/odmkv.h."""
     _fields_ = [
         ("items", C.c_void_p), ("item_range", C.c_void_p), ("dispatch_order", C.c_void_p),
-        ("n_items", C.c_int32), ("wavefronts", C.c_int32), ("n_workgroups", C.c_int32),
+        ("n_items", C.c_int32), ("wavefronts", C.c_int32), ("n_workgroups", C.c_int32), ("two_per_cu", C.c_int32),
     ]
 
 

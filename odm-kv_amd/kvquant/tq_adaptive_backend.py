@@ -63,6 +63,7 @@ _ITEM_FIXED_US = 4.0           # what the cuts without chains are compared with 
 # 90 -> 67 us; 16 x 8192 tokens with four levels: 44 -> 36 us; 16 x 8192 tokens with two levels (c3): no gain at any cut,
 # not taken by the rule.  The link and rotation costs below only rank the workgroups for the dispatch order.
 _CHAIN_LINK_US = 1.8
+_PAIR_CHAIN_RUNS_PER_PLACE = 1.5      # two workgroups per compute unit: chains where the runs number this many per place
 _CHAIN_ROTATE_US = 1.0
 _CHAIN_RUNS_PER_CU = 1.5
 _CHAIN_RUNS_PER_PAIR = 2.5
@@ -874,8 +875,10 @@ class TurboQuantAdaptiveKVCacheState:
             return max(free)
 
         chain_env = os.environ.get("ODMKV_DECODE_CHAINS")                # "0": never, "1": always (measurements)
+        pair_env = os.environ.get("ODMKV_DECODE_PAIRS")                  # the same for two workgroups per compute unit
         may_chain = q_s.size > 0 and bool((~q_first).any()) and chain_env != "0"
         explicit = target_items if target_items is not None else (env_target or None)
+        paired = pair_env == "1"
         if explicit is not None:
             items = cut_chained(fit_chained(int(explicit))) if (may_chain and chain_env == "1") else cut(fit(int(explicit)))
         else:
@@ -885,6 +888,7 @@ class TurboQuantAdaptiveKVCacheState:
             if chosen is not None and abs(total_bytes - chosen[1]) <= 0.05 * chosen[1]:
                 items = (cut_chained(fit_chained(int(n_cu * chosen[0]))) if chosen[2] and may_chain
                          else cut(fit(int(n_cu * chosen[0]))))
+                paired = chosen[3]
             else:
                 best = None
                 if chain_env != "1" or not may_chain:
@@ -894,20 +898,34 @@ class TurboQuantAdaptiveKVCacheState:
                         if best is None or t < best[0] - 1e-9:
                             best = (t, cand, mult, False)
                 n_pairs = int(q_first.sum())
-                if may_chain and (chain_env == "1" or (q_s.size >= _CHAIN_RUNS_PER_CU * n_cu
-                                                       and q_s.size >= _CHAIN_RUNS_PER_PAIR * n_pairs)):
-                    n_exact = int((run_li == 4).sum())
+                n_exact = int((run_li == 4).sum())
+                if pair_env != "0" and (paired or (best is not None and len(best[1]) > n_cu)):
+                    # More items than compute units: the workgroups would run in rounds, each paying its start (work item,
+                    # rotation, table, first bytes: about 4 us) and its end (combine) with the compute unit to itself.
+                    # Two eight-wavefront workgroups per compute unit overlap one's start and end with the other's
+                    # stream (measured: a 16 x 8192-token batch 28.1 -> 25.9 us, 64 x 2048 tokens 52 -> 40 us; lists of
+                    # one item per compute unit lose 5-10 %, and keep the wide workgroups).  Cut for one round of the
+                    # 2 x n_cu places; where the runs alone are many more than that, chain a pair's levels instead.
+                    paired = True
+                    if may_chain and (chain_env == "1" or q_s.size + n_exact > _PAIR_CHAIN_RUNS_PER_PLACE * 2 * n_cu):
+                        mult = max(2.0, (n_pairs + n_exact) / n_cu)
+                        best = (0.0, cut_chained(fit_chained(int(n_cu * mult))), mult, True)
+                    else:
+                        best = (0.0, cut(fit(2 * n_cu)), 2.0, False)
+                elif may_chain and (chain_env == "1" or (q_s.size >= _CHAIN_RUNS_PER_CU * n_cu
+                                                         and q_s.size >= _CHAIN_RUNS_PER_PAIR * n_pairs)):
                     mult = max(1.5, (n_pairs + n_exact) / n_cu)
                     best = (0.0, cut_chained(fit_chained(int(n_cu * mult))), mult, True)
                 items = best[1]
-                self._items_choice = (best[2], total_bytes, best[3])
+                self._items_choice = (best[2], total_bytes, best[3], paired)
         arr = items.astype(np.int32).reshape(-1, 8)
         per_seg = np.bincount(arr[:, 0], minlength=self._nseg) if len(items) else np.zeros(self._nseg, np.int64)
         ranges = np.concatenate([[0], np.cumsum(per_seg)])          # items are generated in segment order
         order = None
         heads = np.flatnonzero(arr[:, 7] == 0) if len(items) else np.zeros(0, np.int64)
         chained = len(items) > 0 and heads.size != len(items)
-        if len(items) > n_cu or chained:
+        paired = paired and len(items) > 0
+        if len(items) > n_cu or chained or paired:
             # the workgroups' first items, longest workgroup first
             order = heads[np.argsort(-cost(items), kind="stable")].astype(np.int32)
         # one upload for the item table, the ranges and the order (the parts start at multiples of 4 integers)
@@ -940,7 +958,8 @@ class TurboQuantAdaptiveKVCacheState:
         # a 28-head, 3-bit store of 32k tokens: their loops wait on memory, and a third unit in flight pays)
         medium = bool(quant.size) and 6 <= quant.mean() < 16 and (sum(q_bytes) - q_bytes[0]) >= 0.5 * max(sum(q_bytes), 1)
         auto = (12 if medium else 8) if not (quant.size and quant.mean() >= 16) else (12 if wide else 16)
-        w.wavefronts = int(os.environ.get("ODMKV_DECODE_WAVES", 0)) or auto
+        w.wavefronts = 8 if paired else (int(os.environ.get("ODMKV_DECODE_WAVES", 0)) or auto)
+        w.two_per_cu = int(paired)
         self._worklist = w
 
     def decode_attention_block(self, query: torch.Tensor, scaling: Optional[float] = None):

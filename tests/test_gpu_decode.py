@@ -311,6 +311,59 @@ def test_a_batch_of_short_sequences_gets_chained_workgroups_by_itself():
     got = st.decode_attention(q.to(DEV))
     w, items = st._worklist, st._items[0].cpu().numpy()
     assert 0 < w.n_workgroups < w.n_items and (items[:, 6] > 0).any() and st._item_order.numel() == w.n_workgroups
+    assert w.two_per_cu == 1 and w.wavefronts == 8              # (and two such workgroups share a compute unit)
+    assert rel_err(got.cpu(), decode_attention_state(q.float(), ref)) < ATTN_RTOL
+
+
+@pytest.mark.parametrize("G,dtype", [(4, torch.float16), (3, torch.bfloat16), (7, torch.float16), (8, torch.bfloat16)])
+def test_two_workgroups_per_compute_unit(G, dtype, monkeypatch):
+    """Work lists with more items than compute units run on eight-wavefront workgroups built so that two share a
+    compute unit (128 registers a wavefront, half the LDS: a bf16 store's second weight buffer lies in the table's
+    space).  Forced here on a small store, with one workgroup per item and with workgroups that walk several levels:
+    the result is the oracle's and, up to what a different cut changes, the one-per-compute-unit build's."""
+    g = torch.Generator().manual_seed(70 + G)
+    B, H, T = 2, 2, 3000
+    k = torch.randn(B, H, T, 128, generator=g).to(dtype); v = torch.randn(B, H, T, 128, generator=g).to(dtype)
+    bits = _rand_bits(g, (B, H, T), (0.1, 0.35, 0.2, 0.15, 0.1, 0.1))
+    bits[..., :4] = 16; bits[..., -70:] = 16
+    st, ref = _pair(k, v, bits, dtype=dtype)
+    if dtype == torch.bfloat16:                               # (the yardstick for a bf16 store materialises in fp32)
+        ref = KVState(128, (0, 2, 3, 4, 8, 16), dtype=torch.float32, seed=42, order="canonical")
+        ref.prefill(k.float(), v.float(), bits)
+    q = torch.randn(B, H * G, 128, generator=g).to(dtype)
+    want = decode_attention_state(q.float(), ref)
+    monkeypatch.setenv("ODMKV_DECODE_PAIRS", "0")
+    monkeypatch.setenv("ODMKV_DECODE_CHAINS", "0")
+    st._build_items(20, 1)
+    assert st._worklist.two_per_cu == 0
+    one_each = st.decode_attention(q.to(DEV))
+    monkeypatch.setenv("ODMKV_DECODE_PAIRS", "1")
+    for chains, target in (("0", 20), ("0", 64), ("1", 12)):
+        monkeypatch.setenv("ODMKV_DECODE_CHAINS", chains)
+        st._build_items(target, 1)
+        w = st._worklist
+        assert w.two_per_cu == 1 and w.wavefronts == 8 and st._item_order is not None
+        assert (0 < w.n_workgroups < w.n_items) == (chains == "1")
+        got, lse = st.decode_attention(q.to(DEV), return_lse=True)
+        assert rel_err(got.cpu(), want) < ATTN_RTOL
+        assert rel_err(got.cpu(), one_each.cpu().double()) < 5e-4
+        assert torch.isfinite(lse).all()
+
+
+def test_a_batch_gets_two_workgroups_per_compute_unit_by_itself():
+    """16 sequences of 1536 tokens on 8 kv-heads, two quantised levels and the exact rows: more runs than the device
+    has compute units, few enough for one round of two workgroups per compute unit.  The work list chooses that by
+    itself (no chains: a run is an item); the result is the oracle's."""
+    g = torch.Generator().manual_seed(321)
+    B, H, G, T = 16, 8, 4, 1536
+    k = torch.randn(B, H, T, 128, generator=g).half(); v = torch.randn(B, H, T, 128, generator=g).half()
+    bits = _rand_bits(g, (B, H, T), (0.1, 0.7, 0.2, 0.0, 0.0, 0.0))
+    bits[..., :4] = 16; bits[..., -32:] = 16
+    st, ref = _pair(k, v, bits)
+    q = torch.randn(B, H * G, 128, generator=g).half()
+    got = st.decode_attention(q.to(DEV))
+    w = st._worklist
+    assert w.two_per_cu == 1 and w.wavefronts == 8 and w.n_workgroups == 0 and w.n_items > 256
     assert rel_err(got.cpu(), decode_attention_state(q.float(), ref)) < ATTN_RTOL
 
 
