@@ -7,7 +7,9 @@
 //             anyway), rotates them into the basis of the quantised keys on the matrix cores (q' = Pi_k q16 from a
 //             precomputed fp16 high + low operand table, kept as fp16 high + low rows), and streams the item's packed
 //             bytes once from HBM; nothing else is read from there.  A workgroup may take several consecutive items
-//             (the quantised levels of one (sequence, kv-head): a chain) with one rotation and one result.
+//             (the quantised levels of one (sequence, kv-head): a chain) with one rotation and one result.  For lists
+//             with more items than compute units there is a build of the eight-wavefront workgroup that two of share
+//             a compute unit (128 registers a wavefront, half the LDS): one streams while the other starts or ends.
 //   2. merge: log-sum-exp merge of a kv-head's items per query head, rotation of the quantised
 //             part back to the model basis (acc . Pi_v), addition of the exact part, normalise.
 // (Merging inside the main kernel, by the workgroup that finishes last among a kv-head's items, was built
@@ -16,8 +18,8 @@
 // A separate query-preparation launch was measured too: the same time per call, one launch more.)
 //
 // Two forms of the quantised levels: the general one (compute_unit: up to 8 heads of a group in one pass), and one for
-// groups of up to four heads on sixteen wavefronts (compute_unit_g4: the lanes are shared out between a unit's two
-// token blocks, the softmax step runs once per unit).
+// groups of up to four heads at four wavefronts per SIMD (sixteen wavefronts, or two workgroups of eight;
+// compute_unit_g4: the lanes are shared out between a unit's two token blocks, the softmax step runs once per unit).
 //
 // Main kernel, per wavefront and unit of 32 tokens (half a tile), on v_mfma_f32_16x16x32_f16 (D[16x16] += A[16x32]
 // B[32x16]; lane l supplies A[l%16][8(l/16)+e] and B[8(l/16)+e][l%16], e = 0..7, and holds D[4(l/16)+r][l%16]):
@@ -54,6 +56,8 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 // LDS of the main kernel: [table, later the combine area] [rotated query rows]
 // [p buffers] [per-wave scalars].  NW = wavefronts of the workgroup: 8 (short items: less set-up and a lighter combine),
 // 16 (long items: four wavefronts per SIMD keep its issue slots full) or 12 (three units in flight per wavefront).
+// One p buffer per wavefront (bf16 exact rows need a second one for the weights' low pieces: it lies in the table's
+// space, which an exact item does not use), so that eight wavefronts stay under half a compute unit's 160 KB.
 #define QROW_LDS 272                             // bytes of a query row in LDS: 128 x 16 bit + 16 (bank spread)
 #define LDS_QROWS LUT_BYTES
 #define LDS_PBUFS (LDS_QROWS + 16 * QROW_LDS)

@@ -748,7 +748,9 @@ class TurboQuantAdaptiveKVCacheState:
         are compared by the time a longest-first assignment of their items to the compute units
         would take, and the best is kept; when it has more items than compute units, the order in which
         the workgroups take the items (longest first) is handed to the kernel as well.  Items of sixteen
-        tiles and more on average are run by sixteen (or twelve) wavefronts, shorter ones by eight."""
+        tiles and more on average are run by sixteen (or twelve) wavefronts, shorter ones by eight.  A list
+        with more items than compute units is cut for two eight-wavefront workgroups per compute unit
+        (`two_per_cu`), as chains of a pair's levels where the runs alone are many more than those places."""
         import os
         n_cu = _compute_units(self.device)
         env_target = int(os.environ.get("ODMKV_DECODE_ITEMS", 0))
