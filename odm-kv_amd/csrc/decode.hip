@@ -11,7 +11,8 @@
 //             with more items than compute units there is a build of the eight-wavefront workgroup that two of share
 //             a compute unit (128 registers a wavefront, half the LDS): one streams while the other starts or ends.
 //   2. merge: log-sum-exp merge of a kv-head's items per query head, rotation of the quantised
-//             part back to the model basis (acc . Pi_v), addition of the exact part, normalise.
+//             part back to the model basis (acc . Pi_v), addition of the exact part, normalise (one to four workgroups
+//             per query head; from 512 heads on one workgroup per (sequence, kv-head) for all heads of the group).
 // (Merging inside the main kernel, by the workgroup that finishes last among a kv-head's items, was built
 // and measured twice: the count and the other workgroups' results have to cross the device at agent scope, two
 // to three dependent trips to memory of 2-3 us each under the streaming load, against one launch of 4-5 us.
@@ -1168,6 +1169,103 @@ __global__ __launch_bounds__(MERGE_THREADS) void decode_merge_kernel(DecodeArgs 
     }
 }
 
+// The merge for large batches: one workgroup per (sequence, kv-head) merges and rotates back all heads of the group, so
+// the 64 KB of Pi_v are pulled into a compute unit once per group, not once per query head (2048 heads: 134 MB of reads
+// out of the L2s for 1 MB of results).  The four 128-thread slices take a head each (two each for groups of five to
+// eight); a slice walks its head's items in rounds of MERGE_CHUNK with a running maximum, as above.
+template <int GP>
+__global__ __launch_bounds__(MERGE_THREADS) void decode_merge_group_kernel(DecodeArgs a) {
+    constexpr int HPS = GP / MERGE_SLICES;                // heads per slice
+    static_assert(HPS >= 1, "a slice takes whole heads");
+    constexpr int RS = MERGE_THREADS / HD;                // row slices of the rotation
+    constexpr int IN = HD / RS;                           // rows per slice
+    __shared__ __align__(16) float part[2][GP][HD];       // [rotated | exact][head][dim]
+    __shared__ float part2[GP][RS][HD];
+    __shared__ float headL[GP], headM[GP];
+    const int bh = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, j = tid & (HD - 1);
+    const int slice = __builtin_amdgcn_readfirstlane(tid >> 7);
+    const int b = bh / a.s.Hkv, hq0 = (bh % a.s.Hkv) * a.G;
+    const int i0 = a.item_range[bh], n = a.item_range[bh + 1] - i0;
+    float pv[IN];
+#pragma unroll
+    for (int ii = 0; ii < IN; ++ii) pv[ii] = a.pi_v[(size_t)(slice * IN + ii) * HD + j];
+#pragma unroll
+    for (int h = 0; h < HPS; ++h) {
+        const int g = slice * HPS + h;                    // wave-uniform
+        float M = -INFINITY, L = 0.0f, arot = 0.0f, aex = 0.0f;
+        if (g < a.G) {
+            for (int c0 = 0; c0 < n; c0 += MERGE_CHUNK) {
+                const int nc = min(n - c0, MERGE_CHUNK);
+                float m_i = -INFINITY, l_i = 0.0f;
+                int level = 0;
+                if (lane < nc) {
+                    const float* p = a.partial + ((size_t)(i0 + c0 + lane) * GP + g) * PSTRIDE;
+                    m_i = p[HD]; l_i = p[HD + 1];
+                    level = a.items[8 * (i0 + c0 + lane) + 1];
+                }
+                const float Mc = fmaxf(M, wave_max(m_i));
+                const float f_old = M > -INFINITY ? __builtin_amdgcn_exp2f(M - Mc) : 0.0f;
+                const float w = m_i > -INFINITY ? __builtin_amdgcn_exp2f(m_i - Mc) : 0.0f;
+                L = __fmaf_rn(L, f_old, wave_sum(l_i * w));
+                arot *= f_old; aex *= f_old;
+                const int wsgn = __float_as_int(level == 4 ? -w : w);      // the sign bit marks exact items
+                for (int it0 = 0; it0 < nc; it0 += 4) {                    // four items' values under way at a time
+                    float vals[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        vals[k] = it0 + k < nc ? a.partial[((size_t)(i0 + c0 + it0 + k) * GP + g) * PSTRIDE + j] : 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        if (it0 + k < nc) {
+                            const float ww = __int_as_float(__builtin_amdgcn_readlane(wsgn, it0 + k));
+                            if (__float_as_uint(ww) >> 31) aex = __fmaf_rn(vals[k], -ww, aex);
+                            else arot = __fmaf_rn(vals[k], ww, arot);
+                        }
+                    }
+                }
+                M = Mc;
+            }
+        }
+        part[0][g][j] = arot;
+        part[1][g][j] = aex;
+        if (j == 0) { headL[g] = L; headM[g] = M; }
+    }
+    __syncthreads();
+    // rotate the quantised parts back: out_g[j] = sum_i rot_g[i] Pi_v[i][j]; the slices split the i range
+    float o[GP];
+#pragma unroll
+    for (int g = 0; g < GP; ++g) o[g] = 0.0f;
+#pragma unroll
+    for (int ii = 0; ii < IN; ii += 4) {
+#pragma unroll
+        for (int g = 0; g < GP; ++g) {
+            const f4 r = *reinterpret_cast<const f4*>(&part[0][g][slice * IN + ii]);   // (one address per slice: a broadcast)
+            o[g] = __fmaf_rn(r[0], pv[ii], o[g]); o[g] = __fmaf_rn(r[1], pv[ii + 1], o[g]);
+            o[g] = __fmaf_rn(r[2], pv[ii + 2], o[g]); o[g] = __fmaf_rn(r[3], pv[ii + 3], o[g]);
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < GP; ++g) part2[g][slice][j] = o[g];
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < HPS; ++h) {
+        const int g = slice * HPS + h;
+        if (g >= a.G) continue;
+        float tot = part[1][g][j];
+#pragma unroll
+        for (int r = 0; r < RS; ++r) tot += part2[g][r][j];
+        const float L = headL[g];
+        const float o32 = L > 0.0f ? tot / L : 0.0f;
+        const size_t bq = (size_t)b * a.Hq + hq0 + g;
+        const size_t oi = bq * HD + j;
+        if (a.out_dt == ODMKV_F32) reinterpret_cast<float*>(a.out)[oi] = o32;
+        else if (a.out_dt == ODMKV_F16) reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_F16>::from_f32(o32);
+        else reinterpret_cast<uint16_t*>(a.out)[oi] = Elem<ODMKV_BF16>::from_f32(o32);
+        if (a.lse && j == 0) a.lse[bq] = L > 0.0f ? (headM[g] + __log2f(L) - P_SHIFT) * LN2 : -INFINITY;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
@@ -1297,7 +1395,13 @@ int odmkv_decode_launch(const void* q, int q_dtype, int B, int Hq, float scaling
     }
     if (stage_mask & 4) {
         const int heads = B * Hq;
-        if (heads >= 256) {
+        // from 512 query heads on, a workgroup per (sequence, kv-head) merges all heads of the group (64 x 2048 tokens, 2048
+        // heads: the merge 10.8 -> 4.8 us; 512 heads: 3.5 -> 3.2 us); ODMKV_MERGE_GROUP_FROM moves the limit, for measurements
+        static const int group_from = [] { const char* e = getenv("ODMKV_MERGE_GROUP_FROM"); return e ? atoi(e) : 512; }();
+        if (heads >= group_from) {
+            if (GP == 4) hipLaunchKernelGGL((decode_merge_group_kernel<4>), dim3(B * store->Hkv), dim3(MERGE_THREADS), 0, st, a);
+            else hipLaunchKernelGGL((decode_merge_group_kernel<8>), dim3(B * store->Hkv), dim3(MERGE_THREADS), 0, st, a);
+        } else if (heads >= 256) {
             if (GP == 4) hipLaunchKernelGGL((decode_merge_kernel<4, 1>), dim3(heads), dim3(MERGE_THREADS), 0, st, a);
             else hipLaunchKernelGGL((decode_merge_kernel<8, 1>), dim3(heads), dim3(MERGE_THREADS), 0, st, a);
         } else if (heads >= 128) {

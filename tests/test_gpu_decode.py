@@ -367,6 +367,31 @@ def test_a_batch_gets_two_workgroups_per_compute_unit_by_itself():
     assert rel_err(got.cpu(), decode_attention_state(q.float(), ref)) < ATTN_RTOL
 
 
+@pytest.mark.parametrize("B,G", [(90, 3), (40, 7), (33, 8)])
+def test_large_batches_merge_a_group_per_workgroup(B, G):
+    """From 512 query heads on, the merge runs one workgroup per (sequence, kv-head) for all heads of the group (the value
+    rotation is read once per group).  Batches of short sequences with 540 / 560 / 528 heads, one pair evicted entirely
+    (no items: zeros and lse = -inf), one pair exact only: the oracle's result and log-sum-exp."""
+    g = torch.Generator().manual_seed(400 + G)
+    H, T = 2, 150
+    k = torch.randn(B, H, T, 128, generator=g).half(); v = torch.randn(B, H, T, 128, generator=g).half()
+    bits = _rand_bits(g, (B, H, T), (0.2, 0.3, 0.2, 0.1, 0.1, 0.1))
+    bits[..., -3:] = 16
+    bits[1, 1] = 0                                            # nothing left of this pair
+    bits[2, 0] = 16                                           # exact rows only
+    st, ref = _pair(k, v, bits)
+    q = torch.randn(B, H * G, 128, generator=g).half()
+    got, lse = st.decode_attention(q.to(DEV), return_lse=True)
+    want = decode_attention_state(q.float(), ref)
+    kk, _ = ref.materialize()
+    logits = torch.einsum("bhd,bhtd->bht", q.double(), kk.double().repeat_interleave(G, dim=1)) / 128 ** 0.5
+    want_lse = torch.logsumexp(logits.masked_fill(~ref.visible_mask().repeat_interleave(G, dim=1), float("-inf")), -1)
+    empty = torch.zeros(B, H * G, dtype=torch.bool); empty[1, G:2 * G] = True
+    assert rel_err(got.cpu()[~empty], want[~empty]) < ATTN_RTOL
+    assert torch.all(got.cpu()[empty] == 0) and torch.all(torch.isinf(lse.cpu()[empty]) & (lse.cpu()[empty] < 0))
+    np.testing.assert_allclose(lse.cpu()[~empty].numpy(), want_lse[~empty].numpy(), rtol=1e-3, atol=1e-3)
+
+
 def test_config1_end_to_end():
     """Benchmark config 1: score -> allocate (2.0 bits) -> pack -> one-token decode, all on the GPU,
     each stage compared with the oracle fed the previous stage's GPU output."""
