@@ -930,6 +930,11 @@ class TurboQuantAdaptiveKVCacheState:
         if len(items) > n_cu or chained or paired:
             # the workgroups' first items, longest workgroup first
             order = heads[np.argsort(-cost(items), kind="stable")].astype(np.int32)
+            if paired and order.size > n_cu:
+                # two per compute unit: the first n_cu workgroups land one per compute unit, the next n_cu beside them in
+                # the same order of compute units; taken shortest first, the shortest joins the longest (a 16 x 8192-token
+                # batch 26.0 -> 25.5 us; long and short alternating: 32 us)
+                order = np.concatenate([order[:n_cu], order[n_cu:2 * n_cu][::-1], order[2 * n_cu:]]).astype(np.int32)
         # one upload for the item table, the ranges and the order (the parts start at multiples of 4 integers)
         n_arr, n_rng = arr.size, (ranges.size + 3) & ~3
         blob = np.zeros(n_arr + n_rng + (0 if order is None else order.size), np.int32)
