@@ -178,7 +178,6 @@ def _attention_patch(func):
 
 
 def patch_attention_functions() -> None:
-    for name, func in list(ALL_ATTENTION_FUNCTIONS.items()):
-        if getattr(func, _PATCH_ATTR, False):
-            continue
-        ALL_ATTENTION_FUNCTIONS[name] = _attention_patch(func)
+    """Wrap every registered attention function once (a wrapped one is recognised by its mark and left alone)."""
+    for name in list(ALL_ATTENTION_FUNCTIONS.keys()):
+        ALL_ATTENTION_FUNCTIONS[name] = _attention_patch(ALL_ATTENTION_FUNCTIONS[name])

@@ -60,12 +60,10 @@ class TurboQuantBackendPress:
         values[:, :, lo:hi, :] = vq.dequantize(vq.quantize(v.reshape(-1, v.shape[-1]))).reshape(v.shape).to(values.dtype)
 
     def forward_hook(self, module: nn.Module, _input: tuple, kwargs: dict, output: Any) -> Any:
-        hidden_states = kwargs.get("hidden_states")
-        if hidden_states is None and _input:
-            hidden_states = _input[0]
-        cache = kwargs.get("past_key_values")
-        layer_idx = getattr(module, "layer_idx", None)
-        if hidden_states is None or cache is None or layer_idx is None:
+        # the layer's input arrives by keyword in current transformers, positionally in older ones
+        hidden_states = kwargs["hidden_states"] if kwargs.get("hidden_states") is not None else (_input[0] if _input else None)
+        cache, layer_idx = kwargs.get("past_key_values"), getattr(module, "layer_idx", None)
+        if any(x is None for x in (hidden_states, cache, layer_idx)):
             return output
         layer_idx = int(layer_idx)
         layer = cache.layers[layer_idx]

@@ -126,27 +126,19 @@ class TurboQuantPerTokenPress:
                  value_group_size: int = 32, allow_decode_eviction: bool = False):
         if scorer is None:
             raise ValueError("TurboQuantPerTokenPress requires an explicit scorer.")
-        self.scorer = scorer
-        self.bit_levels = bit_levels
-        self.ratios = ratios
-        self.target_avg_bits = target_avg_bits
-        self.eviction_cost = eviction_cost
-        self.above_target_alpha = above_target_alpha
-        self.n_outlier_channels = n_outlier_channels
-        self.outlier_min_bits = outlier_min_bits
-        self.seed = seed
-        self.decode_quant = decode_quant
-        self.sink_tokens = sink_tokens
-        self.layerwise = layerwise
-        self.quantizer = quantizer
-        self.value_quantizer = normalize_value_quantizer(value_quantizer)
-        self.value_group_size = value_group_size
+        self.scorer, self.seed = scorer, seed
+        # the budget: fixed shares per level, or an average width met by the Lagrangian allocation
+        self.bit_levels, self.ratios, self.target_avg_bits = bit_levels, ratios, target_avg_bits
+        self.eviction_cost, self.above_target_alpha = eviction_cost, above_target_alpha
+        # the quantisers
+        self.quantizer, self.value_quantizer = quantizer, normalize_value_quantizer(value_quantizer)
+        self.value_group_size, self.n_outlier_channels, self.outlier_min_bits = value_group_size, n_outlier_channels, outlier_min_bits
+        # what happens to which tokens
+        self.sink_tokens, self.layerwise, self.decode_quant = sink_tokens, layerwise, decode_quant
         self.allow_decode_eviction = bool(allow_decode_eviction)
-        if self.allow_decode_eviction:
-            self._decode_bit_levels = tuple(bit_levels)
-        else:
-            self._decode_bit_levels = tuple(b for b in bit_levels if b != 0) or (16,)
-        self._epsilon: Optional[dict[int, float]] = None
+        kept = tuple(bit_levels) if self.allow_decode_eviction else tuple(b for b in bit_levels if b != 0)
+        self._decode_bit_levels = kept or (16,)              # levels a decode-time token may get
+        self._epsilon: Optional[dict[int, float]] = None     # distortion per width, calibrated on first use
         self._head_dim: Optional[int] = None
         self._quantizers = _QuantizerPool(seed)
         self._model = None
@@ -161,17 +153,18 @@ class TurboQuantPerTokenPress:
     # ------------------------------------------------------------------ scores -> bits
     def _build_sink_mask(self, H: int, T: int, device) -> Optional[torch.Tensor]:
         """[H, T] bool, True = sink token (kept at 16 bits, outside the budget)."""
-        if self.sink_tokens <= 0:
+        n_sink = min(self.sink_tokens, T)
+        if n_sink <= 0:
             return None
-        mask = torch.zeros(H, T, dtype=torch.bool, device=device)
-        mask[:, :min(self.sink_tokens, T)] = True
-        return mask
+        return (torch.arange(T, device=device) < n_sink).expand(H, T).contiguous()
 
     @staticmethod
     def _supports_kwargs(method) -> bool:
-        params = inspect.signature(method).parameters.values()
-        return any(p.kind == inspect.Parameter.VAR_KEYWORD for p in params) or any(
-            p.name in {"module", "hidden_states"} for p in params)
+        """Whether a scorer's method takes the module and the hidden states (by name, or through **kwargs)."""
+        for p in inspect.signature(method).parameters.values():
+            if p.kind is inspect.Parameter.VAR_KEYWORD or p.name in ("module", "hidden_states"):
+                return True
+        return False
 
     def _ensure_epsilon(self, device) -> dict[int, float]:
         if self._epsilon is None:
@@ -211,12 +204,11 @@ class TurboQuantPerTokenPress:
 
     @staticmethod
     def _set_cache_tensors(cache, layer_idx: int, keys: torch.Tensor, values: torch.Tensor) -> None:
-        if hasattr(cache, "key_cache") and isinstance(cache.key_cache, list):
-            cache.key_cache[layer_idx] = keys
-            cache.value_cache[layer_idx] = values
-            return
-        cache.layers[layer_idx].keys = keys
-        cache.layers[layer_idx].values = values
+        layers = getattr(cache, "layers", None)
+        if layers is not None:
+            layers[layer_idx].keys, layers[layer_idx].values = keys, values
+        else:                                                # caches of older transformers: two lists of tensors
+            cache.key_cache[layer_idx], cache.value_cache[layer_idx] = keys, values
 
     @staticmethod
     def _bits_to_masked_indices(bits: torch.Tensor):
