@@ -81,6 +81,20 @@ def test_argument_checks_without_a_gpu(lib):
     assert rc == -1 and b"query dtype" in lib.odmkv_last_error()
     rc = lib.odmkv_decode_attn_static(p, 0, 1, 8, C.c_float(1.0), None, None, None, None, None, None, None, p, 2, None, None)
     assert rc == -1 and b"work list" in lib.odmkv_last_error()
+    # a work list that asks for two workgroups per compute unit with sixteen wavefronts each, or without a dispatch
+    # order, or for more workgroups than items, is refused before anything is launched
+    from kvquant._lib import Packed, Worklist
+    store, cbh, inv = Packed(), (C.c_float * 284)(), (C.c_float * 4)()
+    def decode(work):
+        return lib.odmkv_decode_attn(p, 0, 1, 8, C.c_float(1.0), C.byref(store), C.byref(work), p, p, p, cbh, inv,
+                                     p, 2, None, p, C.c_size_t(1 << 20), None)
+    w = Worklist(); w.items, w.item_range, w.dispatch_order, w.n_items = 4096, 4096, 4096, 3
+    w.wavefronts, w.two_per_cu = 16, 1
+    assert decode(w) == -1 and b"two workgroups per compute unit" in lib.odmkv_last_error()
+    w.wavefronts, w.dispatch_order = 8, None
+    assert decode(w) == -1 and b"two workgroups per compute unit" in lib.odmkv_last_error()
+    w.two_per_cu, w.n_workgroups = 0, 5
+    assert decode(w) == -1 and b"workgroups for" in lib.odmkv_last_error()
 
 
 def test_host_modules_import_and_validate():
