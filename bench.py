@@ -352,12 +352,13 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--read-ceiling", action="store_true",
                     help="time a plain streaming read kernel at the decode kernel's launch sizes (cold buffers) and exit")
-    ap.add_argument("--decode-shape", choices=["c3", "c4", "w2", "w3", "w4", "w8", "exact"],
+    ap.add_argument("--decode-shape", choices=["c3", "c4", "w2", "w3", "w4", "w8", "exact", "b64", "b16"],
                     help="time the fused decode call on six stores of configuration c3's (16 sequences x 8192 tokens, "
                          "cycling budgets) or c4's (131072 tokens, heavy eviction) shape, compressed by the real pipeline, "
                          "or on single-level stores (w2..w8: every token of a 131072-token layer at that width; exact: 32768 "
-                         "fp16 tokens), rotating over the stores so that every call reads HBM; prints main-kernel and "
-                         "whole-call times and exits")
+                         "fp16 tokens), or on batches whose every (sequence, kv-head) holds four quantised levels by fixed shares "
+                         "(b64: 64 sequences x 2048 tokens, b16: 16 x 8192), rotating over the stores so that every call reads "
+                         "HBM; prints main-kernel and whole-call times and exits")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for counter runs under rocprofv3 --pmc: a few eager decode steps and one plain 256 MiB "
                          "device copy (the calibration kernel), nothing else timed")
@@ -531,6 +532,28 @@ def main() -> int:
             elif name == "c4":
                 Ls = [synthetic.lognormal_norm_layer(4004 + li, 8, 32, 131072)]
                 targets = [2.0]
+            elif name in ("b64", "b16"):
+                # batches whose (sequence, kv-head) pairs each hold four quantised levels (fixed shares, drawn per token):
+                # 64 sequences x 2048 tokens, 16 x 8192
+                nb, nt = (64, 2048) if name == "b64" else (16, 8192)
+                g = torch.Generator(device=dev).manual_seed(7007 + li)
+                Ls = None
+                Bs, Ts = nb, nt
+                k = torch.randn(nb, 8, nt, 128, generator=g, device=dev, dtype=torch.float16)
+                v = torch.randn(nb, 8, nt, 128, generator=g, device=dev, dtype=torch.float16)
+                shares = torch.tensor([0.12, 0.50, 0.18, 0.13, 0.06, 0.01], device=dev)
+                idx = torch.multinomial(shares, nb * 8 * nt, replacement=True, generator=g)
+                bits = torch.tensor(LEVELS, device=dev, dtype=torch.int32)[idx].reshape(nb, 8, nt)
+                bits[..., :4] = 16
+                bits[..., -128:] = 16
+                st = TurboQuantAdaptiveKVCacheState(128, LEVELS, device=dev, dtype=torch.float16, key_quantizer="mse",
+                                                    value_quantizer="mse", seed=42 + li)
+                st.prefill(k, v, bits)
+                st._build_items()
+                sts.append(st)
+                sqs.append((torch.randn(nb, 32, 128, generator=g, device=dev, dtype=torch.float16) * 1.5))
+                del k, v, bits
+                continue
             else:
                 Ls = [synthetic.gaussian_layer(6006 + li, 8, 32, 32768 if single == 16 else 131072)]
             Bs, Ts = len(Ls), Ls[0].keys.shape[1]
