@@ -95,6 +95,37 @@ def bench_decode(blib, st, q, out, ws, stage_mask=7, timer=None):
         raise RuntimeError(blib.odmkv_last_error().decode())
 
 
+def plain_read_us(blib, dev, pool, nbytes, grid, nbuf, stride, reps=5):
+    """Microseconds per launch of a plain streaming read of `nbytes` (odmkv_bench_probe_read), the launches of one sweep
+    over `nbuf` buffers of `pool` back to back in one graph between two events: what a launch of that size can reach."""
+    import torch
+    from kvquant import _lib
+    sink = torch.zeros(64, dtype=torch.int32, device=dev)
+
+    def sweep():
+        for it in range(nbuf):
+            rc = blib.odmkv_bench_probe_read(pool.data_ptr() + it * stride, nbytes, grid, sink.data_ptr(), _lib.stream_ptr(dev))
+            assert rc == 0, blib.odmkv_last_error()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        sweep()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        sweep()
+    g.replay()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (reps * nbuf) * 1e3
+
+
 def parity_gate(dev):
     """A small instance of the whole path against the CPU oracle, before anything is timed."""
     import numpy as np
@@ -481,38 +512,14 @@ def main() -> int:
     if args.read_ceiling:
         # what can ONE launch of a given size reach?  buffers rotate through 2 GiB so every launch reads HBM
         pool = torch.ones(2 << 30, dtype=torch.uint8, device=dev)
-        sink = torch.zeros(64, dtype=torch.int32, device=dev)
         rows = []
         for nbytes in (19336677, 80740000, 536870912):
             stride = (nbytes + (2 << 20)) & ~((2 << 20) - 1)
             nbuf = min((2 << 30) // stride, 64)
             for grid in (1024, 2048, 4096):
-                def sweep():
-                    for it in range(nbuf):
-                        rc = blib.odmkv_bench_probe_read(pool.data_ptr() + it * stride, nbytes, grid, sink.data_ptr(),
-                                                         _lib.stream_ptr(dev))
-                        assert rc == 0, blib.odmkv_last_error()
                 # the launches of one sweep over the buffers go back to back (one graph), timed between two
                 # events: event pairs around single launches would add about 2 us to each
-                side = torch.cuda.Stream()
-                side.wait_stream(torch.cuda.current_stream())
-                with torch.cuda.stream(side):
-                    sweep()
-                torch.cuda.current_stream().wait_stream(side)
-                torch.cuda.synchronize()
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    sweep()
-                g.replay()
-                reps = 5
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                torch.cuda.synchronize()
-                e0.record()
-                for _ in range(reps):
-                    g.replay()
-                e1.record()
-                torch.cuda.synchronize()
-                avg = e0.elapsed_time(e1) / (reps * nbuf)
+                avg = plain_read_us(blib, dev, pool, nbytes, grid, nbuf, stride) * 1e-3
                 rows.append({"bytes": nbytes, "grid": grid, "buffers": nbuf, "avg_us": round(avg * 1e3, 2),
                              "GBps": round(nbytes / (avg * 1e-3) / 1e9), "pct_of_8TBps": round(100 * nbytes / (avg * 1e-3) / 8e12, 1)})
         print(json.dumps({"read_ceiling": rows}))
@@ -819,6 +826,19 @@ def main() -> int:
     events_avg_ms = sum(kernel_ms) / max(len(kernel_ms), 1)
     kern_avg_ms = kern_alone_ms if kern_alone_ms is not None else events_avg_ms
     achieved = bytes_per_launch / (kern_avg_ms * 1e-3) / 1e9
+    # what a launch of this size can reach: a plain streaming read of the same number of bytes per launch, timed the same
+    # way (one graph of launches over NL buffers, so that every launch reads memory), outside the timed region
+    plain = None
+    try:
+        nb = int(bytes_per_launch)
+        stride = (nb + (2 << 20)) & ~((2 << 20) - 1)
+        pool = torch.ones(stride * NL, dtype=torch.uint8, device=dev)
+        us = plain_read_us(blib, dev, pool, nb, 4096, NL, stride)
+        plain = {"bytes_per_launch": nb, "us_per_launch": round(us, 2), "GBps": round(nb / us / 1e3, 1),
+                 "frac_of_peak": round(nb / us / 1e3 / HBM_PEAK_GBS, 4), "kernel_over_plain_read": round(us / (kern_avg_ms * 1e3), 3)}
+        del pool
+    except Exception as exc:                                       # noqa: BLE001
+        print(f"plain-read figure not available ({exc})", file=sys.stderr)
 
     out = {
         "metric": "LUT decode-attn achieved GB/s (% HBM peak); ms to score+pack a 32k-token layer",
@@ -844,6 +864,7 @@ def main() -> int:
                                                 "factor the same counter gives for a plain 256 MiB copy",
                                          "FETCH_SIZE": traffic["FETCH_SIZE"], "WRITE_SIZE": traffic["WRITE_SIZE"],
                                          "over_algorithmic": round(traffic["bytes"] / traffic["packed_bytes_per_layer"], 4)}),
+                     "plain_read_of_the_same_size": plain,
                      "kernel": "decode_main_kernel", "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
                      "kernel_avg_method": ("the step's main-kernel launches alone (no merge) as one graph, replayed between two "
                                            "HIP events on the launch stream: elapsed / launches, launch gaps included"
